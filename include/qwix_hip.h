@@ -1,0 +1,173 @@
+/*
+ * qwix_hip.h -- C ABI of libqwix_hip.so: the MI355X (gfx950) kernels behind Qwix's
+ * quantize + quantized dot_general path.
+ *
+ * Every entry point
+ *   - takes raw DEVICE pointers, sizes and a hipStream_t (passed as void*),
+ *   - only enqueues work on that stream (no hipMalloc/hipFree, no device sync),
+ *   - returns QWIX_OK or an error code; qwix_hip_last_error() gives the text of
+ *     the calling thread's last error,
+ *   - is re-entrant and keeps no mutable global state.
+ * These are exactly the symbols a jax.ffi custom-call handler (or ctypes, or a
+ * torch extension) binds; the reference functions they replace are cited per
+ * entry (paths relative to the google/qwix tree).
+ *
+ * Conventions
+ *   dtype   QWIX_F32 / QWIX_BF16                         (float arrays)
+ *   qtype   QWIX_INT8 / QWIX_INT4 / QWIX_E4M3            (quantized values)
+ *   int4    two values per byte along the physically contiguous axis; the element
+ *           with the even index sits in the LOW nibble; two's complement.
+ *   A float array of rank n that is quantized with one reduced (or tiled) axis is
+ *   described as the row-major 3-D view (outer, reduce, inner); `tile` divides
+ *   `reduce`; the scale is the row-major array (outer, reduce/tile, inner).
+ *   Per-token activations:   outer=tokens, reduce=features, inner=1, tile=reduce.
+ *   Per-channel (K,N) weight: outer=1, reduce=K, inner=N, tile=K.
+ *   Sub-channel (K,N) weight: outer=1, reduce=K, inner=N, tile=128.
+ */
+#ifndef QWIX_HIP_H_
+#define QWIX_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QWIX_API __attribute__((visibility("default")))
+
+enum { QWIX_OK = 0, QWIX_ERR_INVALID_ARGUMENT = 1, QWIX_ERR_UNSUPPORTED = 2, QWIX_ERR_LAUNCH = 3 };
+enum { QWIX_F32 = 0, QWIX_BF16 = 1, QWIX_I32 = 2 };
+enum { QWIX_INT8 = 0, QWIX_INT4 = 1, QWIX_E4M3 = 2 };
+enum { QWIX_ABSMAX = 0, QWIX_MINMAX = 1 };
+/* Quantized-value layouts for the 3-D view (outer, reduce, inner). */
+enum {
+  QWIX_LAYOUT_NATURAL = 0,      /* (outer, reduce, inner) row-major, like the input        */
+  QWIX_LAYOUT_REDUCE_MINOR = 1  /* (outer, inner, reduce) row-major: the reduced axis is    */
+                                /* contiguous, which is what the GEMM kernels consume       */
+};
+
+/* Version / diagnostics. */
+QWIX_API int qwix_hip_abi_version(void);
+QWIX_API const char* qwix_hip_last_error(void);
+
+/* ---------------------------------------------------------------------------------------
+ * Quantize: calibrate -> scale(/zero point) -> divide -> round -> saturating cast, fused.
+ * Replaces qarray.quantize (qwix/_src/core/qarray.py:638-644) = calibrate (:470-534) +
+ * compute_scale_zero_point (:537-584) + quantize_with_scale_zero_point (:594-635) +
+ * numerics.convert_to (qwix/_src/core/numerics.py:139-196).
+ *   x           (outer, reduce, inner) of `dtype`
+ *   calibration QWIX_ABSMAX or QWIX_MINMAX; calib_factor > 0 multiplies the range
+ *               ("absmax,0.9"); pass 0 for none
+ *   qvalue      out; int8/e4m3: 1 byte per element, int4: packed (see above)
+ *   scale       out, `dtype`, (outer, reduce/tile, inner)
+ *   zero_point  out for QWIX_MINMAX (int8 per scale element, also for int4), else NULL
+ *   workspace   device scratch of qwix_hip_quantize_workspace_bytes(...) bytes (may be
+ *               NULL when that is 0)
+ */
+QWIX_API size_t qwix_hip_quantize_workspace_bytes(int64_t outer, int64_t reduce, int64_t inner,
+                                         int64_t tile, int calibration);
+QWIX_API int qwix_hip_quantize(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner,
+                      int64_t tile, int qtype, int calibration, float calib_factor,
+                      int q_layout, void* qvalue, void* scale, void* zero_point,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+/* calibrate alone (qarray.py:470-534): writes absmax (QWIX_ABSMAX: out0) or min/max
+ * (QWIX_MINMAX: out0=min, out1=max), each `dtype`, shaped like the scale. */
+QWIX_API int qwix_hip_calibrate(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner,
+                       int64_t tile, int calibration, float calib_factor, void* out0,
+                       void* out1, void* workspace, size_t workspace_bytes, void* stream);
+
+/* compute_scale_zero_point (qarray.py:537-584) on n calibration values. */
+QWIX_API int qwix_hip_compute_scale_zero_point(const void* cal0, const void* cal1, int dtype, int64_t n,
+                                      int qtype, int calibration, void* scale, void* zero_point,
+                                      void* stream);
+
+/* quantize_with_scale_zero_point (qarray.py:594-635) with a given scale (static range). */
+QWIX_API int qwix_hip_quantize_with_scale(const void* x, int dtype, int64_t outer, int64_t reduce,
+                                 int64_t inner, int64_t tile, int qtype, const void* scale,
+                                 const void* zero_point, int q_layout, void* qvalue,
+                                 void* stream);
+
+/* Generic fallback for shapes the 3-D view cannot express (two tiled/reduced axes):
+ * x is the row-major 5-D view (d0, r1, d2, r3, d4); tiles t1 | r1 and t3 | r3 are reduced;
+ * scale is (d0, r1/t1, d2, r3/t3, d4).  Natural layout only.  Slow but complete. */
+QWIX_API int qwix_hip_quantize_generic(const void* x, int dtype, const int64_t dims[5], int64_t t1,
+                              int64_t t3, int qtype, int calibration, float calib_factor,
+                              void* qvalue, void* scale, void* zero_point, void* stream);
+
+/* dequantize (qarray.py:692-708): (q - zp) * scale in the scale dtype. */
+QWIX_API int qwix_hip_dequantize(const void* qvalue, int qtype, int q_layout, int64_t outer,
+                        int64_t reduce, int64_t inner, int64_t tile, const void* scale,
+                        const void* zero_point, int dtype, void* out, void* stream);
+
+/* Layout helper: (rows, cols) bytes -> (cols, rows) bytes; int4: repacks so the pairs run
+ * along the new contiguous axis.  Used to bring a NATURAL qvalue to REDUCE_MINOR. */
+QWIX_API int qwix_hip_transpose_q(const void* src, int qtype, int64_t rows, int64_t cols, void* dst,
+                         void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Quantized GEMM, dequantize-on-output.  Replaces _fast_dot_general
+ * (qwix/_src/core/dot_general.py:135-261) for a 2-D contraction:
+ *     out[m,n] = cast_R( (T(sum_k a[m,k] b[k,n]) * sa[m]) * sb[n] )
+ *   a        (M,K) row-major, lda bytes-per-row >= K (K-contiguous)
+ *   b        stored K-contiguous: b_nk[n*ldb + k]   (QWIX_LAYOUT_REDUCE_MINOR of a (K,N) weight)
+ *   qtype    QWIX_INT8 (int32 accumulate, exact) or QWIX_E4M3 (f32 accumulate)
+ *   sa, sb   per-row / per-column scales (sa_dtype / sb_dtype in {F32,BF16}); NULL = none
+ *   out      (M,N) row-major of out_dtype in {F32,BF16}; QWIX_I32 returns the raw int32
+ *            accumulators (int8 only; scales ignored)
+ * Intermediate dtypes follow the reference: int32 -> f32 -> scale dtype, one rounding per
+ * multiply, lhs scale first; e4m3: the f32 accumulator is rounded to acc_dtype first
+ * (the reference's accumulator type = result type for non-integer operands).
+ */
+QWIX_API int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M,
+                   int64_t N, int64_t K, const void* sa, int sa_dtype, const void* sb,
+                   int sb_dtype, int acc_dtype, void* out, int out_dtype, int64_t ldo,
+                   void* stream);
+
+/* Sub-channel GEMM (dot_general.py:186-203,255-260): K is split in groups of `group`
+ * (multiple of 128); per-group int32 partials are scaled and summed:
+ *     out[m,n] = cast_R( sum_g (T(acc_g[m,n]) * sa[m,g']) * sb[g,n] )
+ *   a        int8 (M,K) K-contiguous
+ *   b        int8 or int4 (b_qtype), K-contiguous rows: b_nk[n*ldb_bytes + ...]
+ *   sa       (M, ga) with ga in {1, K/group}, row-major;  sb (K/group, N) row-major
+ *   exact    1: every intermediate is rounded exactly as the reference does (bit-exact with
+ *               the CPU oracle, slower); 0: f32 throughout (within rtol 1e-2)
+ *   acc_out  optional (K/group, M, N) int32 raw partials for parity tests, else NULL
+ */
+QWIX_API int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b, int64_t ldb_bytes,
+                           int b_qtype, int64_t M, int64_t N, int64_t K, int64_t group,
+                           const void* sa, int sa_dtype, int64_t ga, const void* sb,
+                           int sb_dtype, void* out, int out_dtype, int64_t ldo, int exact,
+                           int32_t* acc_out, void* stream);
+
+/* Weight-only skinny GEMM (the reference's _slow_dot_general, dot_general.py:264-275, with
+ * the dequantize fused): out[m,n] = sum_k x[m,k] * (q[k,n] * s[k/group, n]).
+ *   x   (M,K) bf16 row-major; q int4/int8 K-contiguous rows (n*ldb_bytes); s (K/group, N)
+ *   M <= 64 is the intended range (decode); group multiple of 128 or == K.
+ */
+QWIX_API int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64_t ldb_bytes, int b_qtype,
+                     int64_t M, int64_t N, int64_t K, int64_t group, const void* s,
+                     int s_dtype, void* out, int out_dtype, int64_t ldo, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Walsh-Hadamard rotation along the last axis (qwix/contrib/hadamard_rot.py:35-117):
+ *     y[r, :] = ((x[r, :] * pre_sign) H_n) * post_sign * out_scale
+ * H_n Sylvester/natural order, n = 2^p <= 16384, unnormalised; pre/post sign vectors are
+ * +-1 arrays of `dtype` (NULL = none); out_scale is 1 for activations and 1/n for the
+ * transposed weight.  Result rounded once to `dtype` (f32 butterflies inside).
+ */
+QWIX_API int qwix_hip_fwht(const void* x, int dtype, int64_t rows, int64_t n, const void* pre_sign,
+                  const void* post_sign, float out_scale, void* y, void* stream);
+
+/* The same rotation fused with per-row (tile == n) or per-group (tile | n) absmax
+ * quantization of the rotated values; nothing but qvalue/scale is written.
+ * Equals qwix_hip_fwht followed by qwix_hip_quantize(outer=rows, reduce=n, inner=1). */
+QWIX_API int qwix_hip_fwht_quantize(const void* x, int dtype, int64_t rows, int64_t n,
+                           const void* pre_sign, const void* post_sign, float out_scale,
+                           int64_t tile, int qtype, void* qvalue, void* scale, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QWIX_HIP_H_ */

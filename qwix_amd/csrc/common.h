@@ -1,0 +1,205 @@
+// Device-side numerics shared by all kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/qwix_hip.h"
+
+namespace qwix {
+
+// ------------------------------------------------------------------ host: errors
+inline char* err_buf() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+inline int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(err_buf(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return QWIX_OK;
+}
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// ------------------------------------------------------------------ dtype tags
+struct F32 {
+  using storage = float;
+  static constexpr int kTag = QWIX_F32;
+  static constexpr int kVec = 4;  // elements per 16-byte vector
+};
+struct BF16 {
+  using storage = uint16_t;
+  static constexpr int kTag = QWIX_BF16;
+  static constexpr int kVec = 8;
+};
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) {
+  __bf16 b = static_cast<__bf16>(x);  // RNE
+  return __builtin_bit_cast(uint16_t, b);
+}
+// Round an f32 result to bf16 precision but keep it in an f32 register.
+__device__ __forceinline__ float round_bf16(float x) {
+  return bf16_bits_to_f32(f32_to_bf16_bits(x));
+}
+
+template <typename D>
+__device__ __forceinline__ float rnd(float x) {
+  if constexpr (D::kTag == QWIX_BF16) return round_bf16(x);
+  return x;
+}
+template <typename D>
+__device__ __forceinline__ float load1(const void* p, int64_t i) {
+  if constexpr (D::kTag == QWIX_BF16)
+    return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+  else
+    return reinterpret_cast<const float*>(p)[i];
+}
+template <typename D>
+__device__ __forceinline__ void store1(void* p, int64_t i, float v) {
+  if constexpr (D::kTag == QWIX_BF16)
+    reinterpret_cast<uint16_t*>(p)[i] = f32_to_bf16_bits(v);
+  else
+    reinterpret_cast<float*>(p)[i] = v;
+}
+
+// One 16-byte vector of D -> kVec floats.
+template <typename D>
+__device__ __forceinline__ void unpack16(const uint4& v, float* f) {
+  if constexpr (D::kTag == QWIX_BF16) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(w[i] << 16);
+      f[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
+    }
+  } else {
+    f[0] = __uint_as_float(v.x);
+    f[1] = __uint_as_float(v.y);
+    f[2] = __uint_as_float(v.z);
+    f[3] = __uint_as_float(v.w);
+  }
+}
+
+// ------------------------------------------------------------------ qtype traits
+template <int QT>
+struct QTraits;
+template <>
+struct QTraits<QWIX_INT8> {
+  static constexpr float kSymBound = 127.5f, kMin = -128.f, kMax = 127.f;
+};
+template <>
+struct QTraits<QWIX_INT4> {
+  static constexpr float kSymBound = 7.5f, kMin = -8.f, kMax = 7.f;
+};
+template <>
+struct QTraits<QWIX_E4M3> {
+  static constexpr float kSymBound = 448.f, kMin = -448.f, kMax = 448.f;
+};
+
+constexpr float kTinySqrt = 0x1p-63f;  // sqrt(finfo.tiny) for f32 and bf16 alike
+
+// Saturating float -> int32 of an already integral value; NaN -> 0.  The hardware convert has
+// exactly these semantics, a C cast of an out-of-range float does not.
+__device__ __forceinline__ int cvt_i32_sat(float r) {
+  int q;
+  asm("v_cvt_i32_f32 %0, %1" : "=v"(q) : "v"(r));
+  return q;
+}
+template <int QT>
+__device__ __forceinline__ int to_int_q(float v) {
+  int q = cvt_i32_sat(__builtin_rintf(v));  // rintf = round half to even
+  const int lo = static_cast<int>(QTraits<QT>::kMin), hi = static_cast<int>(QTraits<QT>::kMax);
+  return min(max(q, lo), hi);
+}
+// Two clipped floats -> two OCP e4m3 bytes in the low 16 bits (RNE, subnormals kept).
+__device__ __forceinline__ uint32_t to_e4m3x2(float a, float b) {
+  // clip propagates NaN (the comparisons are false for NaN).
+  a = a > 448.f ? 448.f : (a < -448.f ? -448.f : a);
+  b = b > 448.f ? 448.f : (b < -448.f ? -448.f : b);
+  return static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false)) & 0xFFFFu;
+}
+__device__ __forceinline__ float e4m3_to_f32(uint32_t byte) {
+  return __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(byte), 0);
+}
+
+// ------------------------------------------------------------------ scale math
+// compute_scale_zero_point, symmetric branch: scale = D(absmax / bound), tiny guard.
+template <typename D, int QT>
+__device__ __forceinline__ float sym_scale(float absmax) {
+  float s = rnd<D>(absmax / QTraits<QT>::kSymBound);
+  return (s < kTinySqrt) ? 1.0f : s;
+}
+// asymmetric branch: scale = D(D(max-min)/(qmax-qmin)); zp = convert(D(qmin - D(min/scale))).
+template <typename D, int QT>
+__device__ __forceinline__ float asym_scale_zp(float mn, float mx, int* zp) {
+  float s = rnd<D>(rnd<D>(mx - mn) / (QTraits<QT>::kMax - QTraits<QT>::kMin));
+  s = (s < kTinySqrt) ? 1.0f : s;
+  float z = rnd<D>(QTraits<QT>::kMin - rnd<D>(mn / s));
+  *zp = to_int_q<QT>(z);
+  return s;
+}
+template <typename D>
+__device__ __forceinline__ float apply_factor(float v, float factor) {
+  return factor > 0.f ? rnd<D>(v * rnd<D>(factor)) : v;
+}
+
+// x / s rounded to D.  f32: IEEE division.  bf16: both operands have 8-bit significands, so
+// the exact quotient is never closer than 2^-18 (relative) to a bf16 rounding boundary unless
+// it lies exactly on one, in which case it is representable in f32 and the residual step below
+// reproduces it exactly.  Hence one reciprocal + one Newton step gives RNE_bf16(RNE_f32(x/s)).
+// kSafe=false is for quotients known to be bounded (dynamic range: |x| <= absmax).
+template <typename D, bool kSafe = true>
+struct Divider {
+  float s, r;
+  __device__ __forceinline__ explicit Divider(float scale) : s(scale) {
+    if constexpr (D::kTag == QWIX_BF16) r = __builtin_amdgcn_rcpf(scale);
+  }
+  __device__ __forceinline__ float operator()(float x) const {
+    if constexpr (D::kTag == QWIX_BF16) {
+      float q0 = x * r;
+      float e = __builtin_fmaf(-q0, s, x);
+      float q1 = __builtin_fmaf(e, r, q0);
+      // Overflowing or non-finite quotients (static scales only): take the IEEE path.
+      if constexpr (kSafe)
+        if (!(__builtin_fabsf(q0) < 0x1p100f)) q1 = x / s;
+      return round_bf16(q1);
+    } else {
+      return x / s;
+    }
+  }
+};
+
+// ------------------------------------------------------------------ wave helpers
+__device__ __forceinline__ float wave_xor_max(float v, int width) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1)
+    if (m < width) v = fmaxf(v, __shfl_xor(v, m, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_xor_min(float v, int width) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1)
+    if (m < width) v = fminf(v, __shfl_xor(v, m, 64));
+  return v;
+}
+// NaN-propagating max of |x|: fmaxf drops NaNs, so track them separately where it matters.
+__device__ __forceinline__ float absmax_acc(float acc, float x) {
+  return fmaxf(acc, __builtin_fabsf(x));
+}
+
+// pack helpers
+__device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d) {
+  return (a & 0xFF) | ((b & 0xFF) << 8) | ((c & 0xFF) << 16) | (static_cast<uint32_t>(d) << 24);
+}
+__device__ __forceinline__ uint32_t pack2_i4(int lo, int hi) { return (lo & 0xF) | ((hi & 0xF) << 4); }
+
+}  // namespace qwix

@@ -1,0 +1,874 @@
+// Quantize / calibrate / dequantize kernels (HBM-bound) and their C entry points.
+//
+// Data model: the float array is the row-major 3-D view (outer, reduce, inner); one scale per
+// (outer, reduce/tile, inner).  Two kernel families:
+//   rows_*  inner == 1: every scale group is a contiguous segment of `tile` elements.  A group of
+//           G = 2^g threads owns a segment, keeps it in registers (up to 8 x 16-byte loads per
+//           thread), max-reduces with wave shuffles (+ LDS across waves), then divides, rounds
+//           and stores packed bytes.  One read, one write.
+//   cols_*  inner > 1: the reduced axis is strided.  Pass 1 reduces 128-row panels in registers
+//           and merges panels with a 32-bit atomic max into a caller-provided workspace; pass 2
+//           re-reads each panel, quantizes it, and writes either the natural layout or the
+//           reduce-minor (transposed) layout the GEMM kernels consume.
+#include "common.h"
+
+namespace qwix {
+namespace {
+
+enum { MODE_QUANT = 0, MODE_CALIB = 1, MODE_GIVEN = 2 };
+
+// Quantize N consecutive values (already divided / shifted) and store them packed.
+template <int QT, int N>
+__device__ __forceinline__ void store_q(const float* v, uint8_t* q, int64_t elem) {
+  if constexpr (QT == QWIX_INT8) {
+    uint32_t w[N / 4];
+#pragma unroll
+    for (int i = 0; i < N / 4; ++i)
+      w[i] = pack4_i8(to_int_q<QT>(v[4 * i]), to_int_q<QT>(v[4 * i + 1]), to_int_q<QT>(v[4 * i + 2]),
+                      to_int_q<QT>(v[4 * i + 3]));
+    if constexpr (N == 8)
+      *reinterpret_cast<uint2*>(q + elem) = make_uint2(w[0], w[1]);
+    else
+      *reinterpret_cast<uint32_t*>(q + elem) = w[0];
+  } else if constexpr (QT == QWIX_E4M3) {
+    uint32_t w[N / 4];
+#pragma unroll
+    for (int i = 0; i < N / 4; ++i)
+      w[i] = to_e4m3x2(v[4 * i], v[4 * i + 1]) | (to_e4m3x2(v[4 * i + 2], v[4 * i + 3]) << 16);
+    if constexpr (N == 8)
+      *reinterpret_cast<uint2*>(q + elem) = make_uint2(w[0], w[1]);
+    else
+      *reinterpret_cast<uint32_t*>(q + elem) = w[0];
+  } else {  // INT4: element `elem` is even; low nibble = even element.
+    uint32_t w = 0;
+#pragma unroll
+    for (int i = 0; i < N; ++i) w |= static_cast<uint32_t>(to_int_q<QT>(v[i]) & 0xF) << (4 * i);
+    if constexpr (N == 8)
+      *reinterpret_cast<uint32_t*>(q + elem / 2) = w;
+    else
+      *reinterpret_cast<uint16_t*>(q + elem / 2) = static_cast<uint16_t>(w);
+  }
+}
+
+template <int QT>
+__device__ __forceinline__ uint8_t q_byte(float v) {  // one value -> one byte (int4 unpacked)
+  if constexpr (QT == QWIX_E4M3)
+    return static_cast<uint8_t>(to_e4m3x2(v, 0.f) & 0xFF);
+  else
+    return static_cast<uint8_t>(to_int_q<QT>(v) & 0xFF);
+}
+
+// ------------------------------------------------------------------------------------ rows
+// nseg segments of L = nvec * kVec contiguous elements.  log2g: threads per segment.
+template <typename D, int QT, int CAL, int MODE>
+__global__ void __launch_bounds__(256)
+    rows_kernel(const uint8_t* __restrict__ x, int64_t nseg, int nvec, int log2g, float factor,
+                uint8_t* __restrict__ q, void* __restrict__ scale, int8_t* __restrict__ zp,
+                void* __restrict__ cal0, void* __restrict__ cal1) {
+  constexpr int EV = D::kVec;
+  constexpr bool ASYM = (CAL == QWIX_MINMAX);
+  constexpr int NL = 8;
+  __shared__ float red[2][4];
+  const int tid = threadIdx.x;
+  const int g = 1 << log2g;
+  const int64_t seg = (static_cast<int64_t>(blockIdx.x) << (8 - log2g)) + (tid >> log2g);
+  const int lane = tid & (g - 1);
+  const bool seg_ok = seg < nseg;
+  const uint4* xv = reinterpret_cast<const uint4*>(x) + seg * nvec;
+
+  float f[NL][EV];
+#pragma unroll
+  for (int j = 0; j < NL; ++j) {
+    const int v = lane + (j << log2g);
+    if (seg_ok && v < nvec) {
+      unpack16<D>(xv[v], f[j]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < EV; ++e) f[j][e] = 0.f;
+    }
+  }
+
+  float s = 1.f;
+  int z = 0;
+  if constexpr (MODE != MODE_GIVEN) {
+    float mx = 0.f, mn = 0.f;  // minmax clips to include 0; absmax >= 0
+#pragma unroll
+    for (int j = 0; j < NL; ++j)
+#pragma unroll
+      for (int e = 0; e < EV; ++e) {
+        if constexpr (ASYM) {
+          mx = fmaxf(mx, f[j][e]);
+          mn = fminf(mn, f[j][e]);
+        } else {
+          mx = absmax_acc(mx, f[j][e]);
+        }
+      }
+    mx = wave_xor_max(mx, g < 64 ? g : 64);
+    if constexpr (ASYM) mn = wave_xor_min(mn, g < 64 ? g : 64);
+    if (g > 64) {  // uniform branch: segments span 2 or 4 waves
+      const int w = tid >> 6;
+      if ((tid & 63) == 0) {
+        red[0][w] = mx;
+        red[1][w] = mn;
+      }
+      __syncthreads();
+      const int w0 = (tid >> log2g) << (log2g - 6), nw = 1 << (log2g - 6);
+      mx = red[0][w0];
+      mn = red[1][w0];
+      for (int i = 1; i < nw; ++i) {
+        mx = fmaxf(mx, red[0][w0 + i]);
+        mn = fminf(mn, red[1][w0 + i]);
+      }
+    }
+    mx = apply_factor<D>(mx, factor);
+    if constexpr (ASYM) mn = apply_factor<D>(mn, factor);
+    if constexpr (MODE == MODE_CALIB) {
+      if (seg_ok && lane == 0) {
+        if constexpr (ASYM) {
+          store1<D>(cal0, seg, mn);
+          store1<D>(cal1, seg, mx);
+        } else {
+          store1<D>(cal0, seg, mx);
+        }
+      }
+      return;
+    }
+    if constexpr (ASYM)
+      s = asym_scale_zp<D, QT>(mn, mx, &z);
+    else
+      s = sym_scale<D, QT>(mx);
+    if (seg_ok && lane == 0) {
+      store1<D>(scale, seg, s);
+      if constexpr (ASYM) zp[seg] = static_cast<int8_t>(z);
+    }
+  } else {
+    if (seg_ok) {
+      s = load1<D>(scale, seg);
+      if constexpr (ASYM) z = zp[seg];
+    }
+  }
+
+  const Divider<D, MODE == MODE_GIVEN> div(s);
+  const float zf = static_cast<float>(z);
+#pragma unroll
+  for (int j = 0; j < NL; ++j) {
+    const int v = lane + (j << log2g);
+    if (seg_ok && v < nvec) {
+      float t[EV];
+#pragma unroll
+      for (int e = 0; e < EV; ++e) {
+        t[e] = div(f[j][e]);
+        if constexpr (ASYM) t[e] = rnd<D>(t[e] + zf);
+      }
+      store_q<QT, EV>(t, q, (seg * nvec + v) * EV);
+    }
+  }
+}
+
+// Any segment length (also odd ones): one workgroup per segment, two strided scalar passes; the
+// second pass re-reads what the first left in cache.  int4 needs an even L.
+template <typename D, int QT, int CAL, int MODE>
+__global__ void __launch_bounds__(256)
+    rows_loop_kernel(const void* __restrict__ x, int64_t L, float factor, uint8_t* __restrict__ q,
+                     void* __restrict__ scale, int8_t* __restrict__ zp, void* __restrict__ cal0,
+                     void* __restrict__ cal1) {
+  constexpr bool ASYM = (CAL == QWIX_MINMAX);
+  __shared__ float red[2][4];
+  const int tid = threadIdx.x;
+  const int64_t seg = blockIdx.x;
+  const int64_t base = seg * L;
+  float s = 1.f;
+  int z = 0;
+  if constexpr (MODE != MODE_GIVEN) {
+    float mx = 0.f, mn = 0.f;
+    for (int64_t i = tid; i < L; i += 256) {
+      const float v = load1<D>(x, base + i);
+      if constexpr (ASYM) {
+        mx = fmaxf(mx, v);
+        mn = fminf(mn, v);
+      } else {
+        mx = absmax_acc(mx, v);
+      }
+    }
+    mx = wave_xor_max(mx, 64);
+    mn = wave_xor_min(mn, 64);
+    if ((tid & 63) == 0) {
+      red[0][tid >> 6] = mx;
+      red[1][tid >> 6] = mn;
+    }
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+    mn = fminf(fminf(red[1][0], red[1][1]), fminf(red[1][2], red[1][3]));
+    mx = apply_factor<D>(mx, factor);
+    if constexpr (ASYM) mn = apply_factor<D>(mn, factor);
+    if constexpr (MODE == MODE_CALIB) {
+      if (tid == 0) {
+        if constexpr (ASYM) {
+          store1<D>(cal0, seg, mn);
+          store1<D>(cal1, seg, mx);
+        } else {
+          store1<D>(cal0, seg, mx);
+        }
+      }
+      return;
+    }
+    if constexpr (ASYM)
+      s = asym_scale_zp<D, QT>(mn, mx, &z);
+    else
+      s = sym_scale<D, QT>(mx);
+    if (tid == 0) {
+      store1<D>(scale, seg, s);
+      if constexpr (ASYM) zp[seg] = static_cast<int8_t>(z);
+    }
+  } else {
+    s = load1<D>(scale, seg);
+    if constexpr (ASYM) z = zp[seg];
+  }
+  const Divider<D, true> div(s);
+  const float zf = static_cast<float>(z);
+  auto one = [&](int64_t i) {
+    float t = div(load1<D>(x, base + i));
+    if constexpr (ASYM) t = rnd<D>(t + zf);
+    return t;
+  };
+  if constexpr (QT == QWIX_INT4) {
+    for (int64_t i = tid; i < L / 2; i += 256)
+      q[(base >> 1) + i] = static_cast<uint8_t>(pack2_i4(to_int_q<QT>(one(2 * i)), to_int_q<QT>(one(2 * i + 1))));
+  } else {
+    for (int64_t i = tid; i < L; i += 256) q[base + i] = q_byte<QT>(one(i));
+  }
+}
+
+// ------------------------------------------------------------------------------------ cols
+// Panels of 128 rows x (16 * kVec) columns inside one tile.  Block index -> (outer, tile, chunk,
+// column block).  ws: [plane][outer][ntiles][inner] f32 bit patterns, plane 0 = max (or absmax),
+// plane 1 = -min.
+struct ColGeom {
+  int64_t outer, reduce, inner, tile, ntiles;
+  int chunks_per_tile, col_blocks;
+};
+
+template <typename D>
+__device__ __forceinline__ void col_decode(const ColGeom& gm, int64_t b, int64_t* o, int64_t* t,
+                                           int* chunk, int64_t* c0) {
+  const int64_t cb = b % gm.col_blocks;
+  b /= gm.col_blocks;
+  *chunk = static_cast<int>(b % gm.chunks_per_tile);
+  b /= gm.chunks_per_tile;
+  *t = b % gm.ntiles;
+  *o = b / gm.ntiles;
+  *c0 = (cb * 16 + (threadIdx.x & 15)) * D::kVec;
+}
+
+template <typename D, int CAL>
+__global__ void __launch_bounds__(256)
+    cols_absmax_kernel(const uint8_t* __restrict__ x, ColGeom gm, uint32_t* __restrict__ ws) {
+  constexpr int EV = D::kVec;
+  constexpr bool ASYM = (CAL == QWIX_MINMAX);
+  __shared__ float red[2][4][16][EV];
+  int64_t o, t, c0;
+  int chunk;
+  col_decode<D>(gm, blockIdx.x, &o, &t, &chunk, &c0);
+  const int tid = threadIdx.x, tc = tid & 15, tr = tid >> 4;
+  const bool col_ok = c0 < gm.inner;
+  const int64_t row_end = (t + 1) * gm.tile;
+  float mx[EV], mn[EV];
+#pragma unroll
+  for (int e = 0; e < EV; ++e) mx[e] = mn[e] = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int64_t r = t * gm.tile + chunk * 128 + tr + 16 * j;
+    if (col_ok && r < row_end) {
+      float f[EV];
+      unpack16<D>(*reinterpret_cast<const uint4*>(
+                      x + ((o * gm.reduce + r) * gm.inner + c0) * sizeof(typename D::storage)),
+                  f);
+#pragma unroll
+      for (int e = 0; e < EV; ++e) {
+        if constexpr (ASYM) {
+          mx[e] = fmaxf(mx[e], f[e]);
+          mn[e] = fminf(mn[e], f[e]);
+        } else {
+          mx[e] = absmax_acc(mx[e], f[e]);
+        }
+      }
+    }
+  }
+  // lanes l and l^16, l^32 hold the same columns.
+#pragma unroll
+  for (int e = 0; e < EV; ++e) {
+    mx[e] = fmaxf(mx[e], __shfl_xor(mx[e], 16, 64));
+    mx[e] = fmaxf(mx[e], __shfl_xor(mx[e], 32, 64));
+    if constexpr (ASYM) {
+      mn[e] = fminf(mn[e], __shfl_xor(mn[e], 16, 64));
+      mn[e] = fminf(mn[e], __shfl_xor(mn[e], 32, 64));
+    }
+  }
+  if ((tid & 63) < 16) {
+#pragma unroll
+    for (int e = 0; e < EV; ++e) {
+      red[0][tid >> 6][tc][e] = mx[e];
+      red[1][tid >> 6][tc][e] = mn[e];
+    }
+  }
+  __syncthreads();
+  if (tid < 16 && col_ok) {
+    const int64_t wbase = (o * gm.ntiles + t) * gm.inner + c0;
+    const int64_t plane = gm.outer * gm.ntiles * gm.inner;
+#pragma unroll
+    for (int e = 0; e < EV; ++e) {
+      float a = fmaxf(fmaxf(red[0][0][tc][e], red[0][1][tc][e]), fmaxf(red[0][2][tc][e], red[0][3][tc][e]));
+      atomicMax(ws + wbase + e, __float_as_uint(a));  // a >= 0: bit patterns order like values
+      if constexpr (ASYM) {
+        float b = fminf(fminf(red[1][0][tc][e], red[1][1][tc][e]), fminf(red[1][2][tc][e], red[1][3][tc][e]));
+        atomicMax(ws + plane + wbase + e, __float_as_uint(-b));
+      }
+    }
+  }
+}
+
+__global__ void fill_u32_kernel(uint32_t* p, int64_t n, uint32_t v) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// ws -> calibration arrays of dtype D (calibrate-only path).
+template <typename D, int CAL>
+__global__ void cols_finish_cal_kernel(const uint32_t* __restrict__ ws, int64_t n, float factor,
+                                       void* __restrict__ out0, void* __restrict__ out1) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float mx = apply_factor<D>(__uint_as_float(ws[i]), factor);
+  if constexpr (CAL == QWIX_MINMAX) {
+    const float mn = apply_factor<D>(-__uint_as_float(ws[n + i]), factor);
+    store1<D>(out0, i, mn);
+    store1<D>(out1, i, mx);
+  } else {
+    store1<D>(out0, i, mx);
+  }
+}
+
+// Pass 2.  SRC 0: scale from ws (written out by chunk 0); SRC 1: scale given.
+template <typename D, int QT, int CAL, int LAYOUT, int SRC>
+__global__ void __launch_bounds__(256)
+    cols_quantize_kernel(const uint8_t* __restrict__ x, ColGeom gm, const uint32_t* __restrict__ ws,
+                         float factor, uint8_t* __restrict__ q, void* __restrict__ scale,
+                         int8_t* __restrict__ zp) {
+  constexpr int EV = D::kVec;
+  constexpr bool ASYM = (CAL == QWIX_MINMAX);
+  int64_t o, t, c0;
+  int chunk;
+  col_decode<D>(gm, blockIdx.x, &o, &t, &chunk, &c0);
+  if (c0 >= gm.inner) return;
+  const int rb = threadIdx.x >> 4;
+  const int64_t sidx = (o * gm.ntiles + t) * gm.inner + c0;
+  float s[EV];
+  int z[EV];
+#pragma unroll
+  for (int e = 0; e < EV; ++e) {
+    z[e] = 0;
+    if constexpr (SRC == 0) {
+      const float mx = apply_factor<D>(__uint_as_float(ws[sidx + e]), factor);
+      if constexpr (ASYM) {
+        const int64_t plane = gm.outer * gm.ntiles * gm.inner;
+        const float mn = apply_factor<D>(-__uint_as_float(ws[plane + sidx + e]), factor);
+        s[e] = asym_scale_zp<D, QT>(mn, mx, &z[e]);
+      } else {
+        s[e] = sym_scale<D, QT>(mx);
+      }
+      if (chunk == 0 && rb == 0) {
+        store1<D>(scale, sidx + e, s[e]);
+        if constexpr (ASYM) zp[sidx + e] = static_cast<int8_t>(z[e]);
+      }
+    } else {
+      s[e] = load1<D>(scale, sidx + e);
+      if constexpr (ASYM) z[e] = zp[sidx + e];
+    }
+  }
+  const int64_t row_end = (t + 1) * gm.tile;
+  const int64_t r0 = t * gm.tile + chunk * 128 + rb * 8;
+  float v[8][EV];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    if (r0 + j < row_end) {
+      unpack16<D>(*reinterpret_cast<const uint4*>(
+                      x + ((o * gm.reduce + r0 + j) * gm.inner + c0) * sizeof(typename D::storage)),
+                  v[j]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < EV; ++e) v[j][e] = 0.f;
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < EV; ++e) {
+    const Divider<D, SRC == 1> div(s[e]);
+    const float zf = static_cast<float>(z[e]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      v[j][e] = div(v[j][e]);
+      if constexpr (ASYM) v[j][e] = rnd<D>(v[j][e] + zf);
+    }
+  }
+  if constexpr (LAYOUT == QWIX_LAYOUT_NATURAL) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (r0 + j < row_end) store_q<QT, EV>(v[j], q, (o * gm.reduce + r0 + j) * gm.inner + c0);
+  } else {  // (outer, inner, reduce): 8 consecutive rows of one column are 8 consecutive bytes
+    const bool full = r0 + 8 <= row_end;
+#pragma unroll
+    for (int e = 0; e < EV; ++e) {
+      const int64_t el = (o * gm.inner + c0 + e) * gm.reduce + r0;
+      if (full) {
+        float col[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) col[j] = v[j][e];
+        store_q<QT, 8>(col, q, el);
+      } else if constexpr (QT == QWIX_INT4) {
+        for (int j = 0; j + 1 < 8 && r0 + j + 1 < row_end; j += 2)
+          q[(el + j) >> 1] = static_cast<uint8_t>(pack2_i4(to_int_q<QT>(v[j][e]), to_int_q<QT>(v[j + 1][e])));
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (r0 + j < row_end) q[el + j] = q_byte<QT>(v[j][e]);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------ generic 5-D
+struct Geom5 {
+  int64_t d[5];   // d0, r1, d2, r3, d4
+  int64_t t1, t3; // tiles of r1 and r3
+};
+__device__ __forceinline__ int64_t scale_index5(const Geom5& g, int64_t i0, int64_t i1, int64_t i2,
+                                                int64_t i3, int64_t i4) {
+  const int64_t n1 = g.d[1] / g.t1, n3 = g.d[3] / g.t3;
+  return (((i0 * n1 + i1 / g.t1) * g.d[2] + i2) * n3 + i3 / g.t3) * g.d[4] + i4;
+}
+
+template <typename D, int QT, int CAL>
+__global__ void generic_scale_kernel(const void* __restrict__ x, Geom5 g, float factor,
+                                     void* __restrict__ scale, int8_t* __restrict__ zp) {
+  const int64_t n1 = g.d[1] / g.t1, n3 = g.d[3] / g.t3;
+  const int64_t ns = g.d[0] * n1 * g.d[2] * n3 * g.d[4];
+  int64_t si = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (si >= ns) return;
+  int64_t r = si;
+  const int64_t i4 = r % g.d[4]; r /= g.d[4];
+  const int64_t j3 = r % n3; r /= n3;
+  const int64_t i2 = r % g.d[2]; r /= g.d[2];
+  const int64_t j1 = r % n1;
+  const int64_t i0 = r / n1;
+  float mx = 0.f, mn = 0.f;
+  for (int64_t a = 0; a < g.t1; ++a)
+    for (int64_t b = 0; b < g.t3; ++b) {
+      const int64_t idx = ((((i0 * g.d[1]) + j1 * g.t1 + a) * g.d[2] + i2) * g.d[3] + j3 * g.t3 + b) * g.d[4] + i4;
+      const float v = load1<D>(x, idx);
+      if constexpr (CAL == QWIX_MINMAX) {
+        mx = fmaxf(mx, v);
+        mn = fminf(mn, v);
+      } else {
+        mx = absmax_acc(mx, v);
+      }
+    }
+  mx = apply_factor<D>(mx, factor);
+  if constexpr (CAL == QWIX_MINMAX) {
+    mn = apply_factor<D>(mn, factor);
+    int z;
+    const float s = asym_scale_zp<D, QT>(mn, mx, &z);
+    store1<D>(scale, si, s);
+    zp[si] = static_cast<int8_t>(z);
+  } else {
+    store1<D>(scale, si, sym_scale<D, QT>(mx));
+  }
+}
+
+// One thread per output byte (two elements for int4, along the innermost flattened axis).
+template <typename D, int QT, int CAL>
+__global__ void generic_quant_kernel(const void* __restrict__ x, Geom5 g, const void* __restrict__ scale,
+                                     const int8_t* __restrict__ zp, uint8_t* __restrict__ q) {
+  constexpr int PER = (QT == QWIX_INT4) ? 2 : 1;
+  const int64_t n = g.d[0] * g.d[1] * g.d[2] * g.d[3] * g.d[4];
+  const int64_t bi = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (bi * PER >= n) return;
+  float t[PER];
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    int64_t r = bi * PER + p;
+    const int64_t i4 = r % g.d[4]; r /= g.d[4];
+    const int64_t i3 = r % g.d[3]; r /= g.d[3];
+    const int64_t i2 = r % g.d[2]; r /= g.d[2];
+    const int64_t i1 = r % g.d[1];
+    const int64_t i0 = r / g.d[1];
+    const int64_t si = scale_index5(g, i0, i1, i2, i3, i4);
+    const Divider<D, true> div(load1<D>(scale, si));
+    t[p] = div(load1<D>(x, bi * PER + p));
+    if constexpr (CAL == QWIX_MINMAX) t[p] = rnd<D>(t[p] + static_cast<float>(zp[si]));
+  }
+  if constexpr (QT == QWIX_INT4)
+    q[bi] = static_cast<uint8_t>(pack2_i4(to_int_q<QT>(t[0]), to_int_q<QT>(t[1])));
+  else
+    q[bi] = q_byte<QT>(t[0]);
+}
+
+// ------------------------------------------------------------------------------------ misc
+template <typename D, int QT, int CAL>
+__global__ void scale_zp_kernel(const void* __restrict__ c0, const void* __restrict__ c1, int64_t n,
+                                void* __restrict__ scale, int8_t* __restrict__ zp) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  if constexpr (CAL == QWIX_MINMAX) {
+    int z;
+    const float s = asym_scale_zp<D, QT>(load1<D>(c0, i), load1<D>(c1, i), &z);
+    store1<D>(scale, i, s);
+    zp[i] = static_cast<int8_t>(z);
+  } else {
+    store1<D>(scale, i, sym_scale<D, QT>(load1<D>(c0, i)));
+  }
+}
+
+// out[(o, r, i)] = D(D(q - zp) * s).  One thread per element; layouts as documented.
+template <typename D, int QT>
+__global__ void dequant_kernel(const uint8_t* __restrict__ q, int layout, int64_t outer, int64_t reduce,
+                               int64_t inner, int64_t tile, const void* __restrict__ scale,
+                               const int8_t* __restrict__ zp, void* __restrict__ out) {
+  const int64_t n = outer * reduce * inner;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const int64_t i = idx % inner, r = (idx / inner) % reduce, o = idx / (inner * reduce);
+  const int64_t qi = layout == QWIX_LAYOUT_NATURAL ? idx : (o * inner + i) * reduce + r;
+  float v;
+  if constexpr (QT == QWIX_INT8) {
+    v = static_cast<float>(reinterpret_cast<const int8_t*>(q)[qi]);
+  } else if constexpr (QT == QWIX_E4M3) {
+    v = e4m3_to_f32(q[qi]);
+  } else {
+    const int nib = (q[qi >> 1] >> ((qi & 1) * 4)) & 0xF;
+    v = static_cast<float>((nib ^ 8) - 8);
+  }
+  const int64_t si = (o * (reduce / tile) + r / tile) * inner + i;
+  v = rnd<D>(v);
+  if (zp != nullptr) v = rnd<D>(v - rnd<D>(static_cast<float>(zp[si])));
+  store1<D>(out, idx, rnd<D>(v * load1<D>(scale, si)));
+}
+
+// (rows, cols) elements -> (cols, rows); int4 repacks along the new minor axis.
+template <int QT>
+__global__ void __launch_bounds__(256)
+    transpose_q_kernel(const uint8_t* __restrict__ src, int64_t rows, int64_t cols, uint8_t* __restrict__ dst) {
+  __shared__ uint8_t tile[64][65];
+  const int64_t r0 = static_cast<int64_t>(blockIdx.y) * 64, c0 = static_cast<int64_t>(blockIdx.x) * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+  for (int j = ty; j < 64; j += 4) {
+    const int64_t r = r0 + j, c = c0 + tx;
+    uint8_t v = 0;
+    if (r < rows && c < cols) {
+      if constexpr (QT == QWIX_INT4) {
+        const int64_t e = r * cols + c;
+        v = (src[e >> 1] >> ((e & 1) * 4)) & 0xF;
+      } else {
+        v = src[r * cols + c];
+      }
+    }
+    tile[j][tx] = v;
+  }
+  __syncthreads();
+  if constexpr (QT == QWIX_INT4) {
+    // thread -> (new row = old col, pair of old rows)
+    const int px = threadIdx.x & 31, py = threadIdx.x >> 5;  // 32 pairs x 8
+    for (int j = py; j < 64; j += 8) {
+      const int64_t nr = c0 + j, nc = r0 + 2 * px;
+      if (nr < cols && nc < rows) {
+        const uint8_t lo = tile[2 * px][j], hi = (nc + 1 < rows) ? tile[2 * px + 1][j] : 0;
+        dst[(nr * rows + nc) >> 1] = static_cast<uint8_t>(lo | (hi << 4));
+      }
+    }
+  } else {
+    for (int j = ty; j < 64; j += 4) {
+      const int64_t nr = c0 + j, nc = r0 + tx;
+      if (nr < cols && nc < rows) dst[nr * rows + nc] = tile[tx][j];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------ dispatch
+inline int log2_ceil(int64_t v) {
+  int l = 0;
+  while ((int64_t{1} << l) < v) ++l;
+  return l;
+}
+
+#define QWIX_DISPATCH_D(dtype, ...)                                         \
+  if ((dtype) == QWIX_F32) { using D = F32; __VA_ARGS__ }                   \
+  else if ((dtype) == QWIX_BF16) { using D = BF16; __VA_ARGS__ }            \
+  else return fail(QWIX_ERR_INVALID_ARGUMENT, "dtype %d is not f32/bf16", (dtype));
+
+#define QWIX_DISPATCH_QT_CAL(qtype, cal, ...)                                                   \
+  if ((qtype) == QWIX_INT8 && (cal) == QWIX_ABSMAX) { constexpr int QT = QWIX_INT8, CAL = QWIX_ABSMAX; __VA_ARGS__ } \
+  else if ((qtype) == QWIX_INT4 && (cal) == QWIX_ABSMAX) { constexpr int QT = QWIX_INT4, CAL = QWIX_ABSMAX; __VA_ARGS__ } \
+  else if ((qtype) == QWIX_E4M3 && (cal) == QWIX_ABSMAX) { constexpr int QT = QWIX_E4M3, CAL = QWIX_ABSMAX; __VA_ARGS__ } \
+  else if ((qtype) == QWIX_INT8 && (cal) == QWIX_MINMAX) { constexpr int QT = QWIX_INT8, CAL = QWIX_MINMAX; __VA_ARGS__ } \
+  else if ((qtype) == QWIX_INT4 && (cal) == QWIX_MINMAX) { constexpr int QT = QWIX_INT4, CAL = QWIX_MINMAX; __VA_ARGS__ } \
+  else return fail(QWIX_ERR_INVALID_ARGUMENT, "qtype %d / calibration %d unsupported (asymmetric needs int8/int4)", (qtype), (cal));
+
+int check_geom(int64_t outer, int64_t reduce, int64_t inner, int64_t tile) {
+  if (outer <= 0 || reduce <= 0 || inner <= 0 || tile <= 0)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "non-positive dimension (outer=%lld reduce=%lld inner=%lld tile=%lld)",
+                (long long)outer, (long long)reduce, (long long)inner, (long long)tile);
+  if (reduce % tile != 0)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "tile %lld does not divide the reduced axis %lld", (long long)tile,
+                (long long)reduce);
+  return QWIX_OK;
+}
+
+ColGeom make_col_geom(int64_t outer, int64_t reduce, int64_t inner, int64_t tile, int ev) {
+  ColGeom g;
+  g.outer = outer; g.reduce = reduce; g.inner = inner; g.tile = tile; g.ntiles = reduce / tile;
+  g.chunks_per_tile = static_cast<int>((tile + 127) / 128);
+  g.col_blocks = static_cast<int>((inner + 16 * ev - 1) / (16 * ev));
+  return g;
+}
+
+// mode: MODE_QUANT / MODE_CALIB / MODE_GIVEN.
+template <int MODE>
+int run_rows(const void* x, int dtype, int64_t nseg, int64_t L, int qtype, int cal, float factor,
+             void* q, void* scale, void* zp, void* c0, void* c1, hipStream_t st) {
+  QWIX_DISPATCH_D(dtype, {
+    QWIX_DISPATCH_QT_CAL(qtype, cal, {
+      const bool vec_ok = (L % D::kVec == 0) && aligned16(x) && (L / D::kVec <= 2048) &&
+                          (MODE == MODE_CALIB || (reinterpret_cast<uintptr_t>(q) & 7) == 0);
+      if (vec_ok) {
+        const int nvec = static_cast<int>(L / D::kVec);
+        int lg = log2_ceil((nvec + 3) / 4);  // aim at <= 4 loads per thread, 8 at most
+        if (lg > 8) lg = 8;
+        const int64_t blocks = (nseg + (256 >> lg) - 1) / (256 >> lg);
+        rows_kernel<D, QT, CAL, MODE><<<dim3(static_cast<unsigned>(blocks)), 256, 0, st>>>(
+            static_cast<const uint8_t*>(x), nseg, nvec, lg, factor, static_cast<uint8_t*>(q), scale,
+            static_cast<int8_t*>(zp), c0, c1);
+      } else {
+        if (QT == QWIX_INT4 && MODE != MODE_CALIB && (L & 1))
+          return fail(QWIX_ERR_UNSUPPORTED, "int4 needs an even contiguous length, got %lld", (long long)L);
+        rows_loop_kernel<D, QT, CAL, MODE><<<dim3(static_cast<unsigned>(nseg)), 256, 0, st>>>(
+            x, L, factor, static_cast<uint8_t*>(q), scale, static_cast<int8_t*>(zp), c0, c1);
+      }
+    })
+  })
+  return check_launch("rows quantize");
+}
+
+int run_cols_absmax(const void* x, int dtype, const ColGeom& g, int cal, uint32_t* ws, hipStream_t st) {
+  const int64_t n = g.outer * g.ntiles * g.inner * (cal == QWIX_MINMAX ? 2 : 1);
+  fill_u32_kernel<<<dim3(static_cast<unsigned>((n + 255) / 256)), 256, 0, st>>>(ws, n, 0u);
+  const int64_t blocks = g.outer * g.ntiles * g.chunks_per_tile * g.col_blocks;
+  QWIX_DISPATCH_D(dtype, {
+    if (cal == QWIX_MINMAX)
+      cols_absmax_kernel<D, QWIX_MINMAX><<<dim3(static_cast<unsigned>(blocks)), 256, 0, st>>>(
+          static_cast<const uint8_t*>(x), g, ws);
+    else
+      cols_absmax_kernel<D, QWIX_ABSMAX><<<dim3(static_cast<unsigned>(blocks)), 256, 0, st>>>(
+          static_cast<const uint8_t*>(x), g, ws);
+  })
+  return check_launch("cols absmax");
+}
+
+template <int SRC>
+int run_cols_quantize(const void* x, int dtype, const ColGeom& g, int qtype, int cal, int layout,
+                      const uint32_t* ws, float factor, void* q, void* scale, void* zp, hipStream_t st) {
+  const int64_t blocks = g.outer * g.ntiles * g.chunks_per_tile * g.col_blocks;
+  QWIX_DISPATCH_D(dtype, {
+    QWIX_DISPATCH_QT_CAL(qtype, cal, {
+      if (layout == QWIX_LAYOUT_NATURAL)
+        cols_quantize_kernel<D, QT, CAL, QWIX_LAYOUT_NATURAL, SRC><<<dim3(static_cast<unsigned>(blocks)), 256, 0, st>>>(
+            static_cast<const uint8_t*>(x), g, ws, factor, static_cast<uint8_t*>(q), scale, static_cast<int8_t*>(zp));
+      else
+        cols_quantize_kernel<D, QT, CAL, QWIX_LAYOUT_REDUCE_MINOR, SRC><<<dim3(static_cast<unsigned>(blocks)), 256, 0, st>>>(
+            static_cast<const uint8_t*>(x), g, ws, factor, static_cast<uint8_t*>(q), scale, static_cast<int8_t*>(zp));
+    })
+  })
+  return check_launch("cols quantize");
+}
+
+int check_cols(const void* x, int dtype, int64_t reduce, int64_t inner, int64_t tile, int layout,
+               const void* q) {
+  const int ev = dtype == QWIX_BF16 ? 8 : 4;
+  if (q != nullptr && !aligned16(q)) return fail(QWIX_ERR_INVALID_ARGUMENT, "qvalue must be 16-byte aligned");
+  if (inner % ev != 0 || !aligned16(x))
+    return fail(QWIX_ERR_UNSUPPORTED,
+                "strided-reduce quantize needs inner %% %d == 0 and a 16-byte aligned input (inner=%lld); "
+                "use qwix_hip_quantize_generic", ev, (long long)inner);
+  if (layout == QWIX_LAYOUT_REDUCE_MINOR && (reduce % 8 != 0 || tile % 8 != 0))
+    return fail(QWIX_ERR_UNSUPPORTED, "reduce-minor layout needs reduce and tile to be multiples of 8 (%lld, %lld)",
+                (long long)reduce, (long long)tile);
+  if (layout != QWIX_LAYOUT_NATURAL && layout != QWIX_LAYOUT_REDUCE_MINOR)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "unknown layout %d", layout);
+  return QWIX_OK;
+}
+
+}  // namespace
+}  // namespace qwix
+
+using namespace qwix;
+
+extern "C" {
+
+int qwix_hip_abi_version(void) { return 1; }
+const char* qwix_hip_last_error(void) { return err_buf(); }
+
+size_t qwix_hip_quantize_workspace_bytes(int64_t outer, int64_t reduce, int64_t inner, int64_t tile,
+                                         int calibration) {
+  if (inner <= 1 || tile <= 0 || reduce % tile != 0) return 0;
+  return static_cast<size_t>(outer * (reduce / tile) * inner) * 4u * (calibration == QWIX_MINMAX ? 2u : 1u);
+}
+
+int qwix_hip_quantize(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner, int64_t tile,
+                      int qtype, int calibration, float calib_factor, int q_layout, void* qvalue, void* scale,
+                      void* zero_point, void* workspace, size_t workspace_bytes, void* stream) {
+  if (int e = check_geom(outer, reduce, inner, tile)) return e;
+  if (!x || !qvalue || !scale) return fail(QWIX_ERR_INVALID_ARGUMENT, "null x/qvalue/scale");
+  if (calibration == QWIX_MINMAX && !zero_point)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "minmax calibration needs a zero_point output");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (inner == 1)  // both layouts coincide
+    return run_rows<MODE_QUANT>(x, dtype, outer * (reduce / tile), tile, qtype, calibration, calib_factor, qvalue,
+                                scale, zero_point, nullptr, nullptr, st);
+  if (int e = check_cols(x, dtype, reduce, inner, tile, q_layout, qvalue)) return e;
+  const size_t need = qwix_hip_quantize_workspace_bytes(outer, reduce, inner, tile, calibration);
+  if (!workspace || workspace_bytes < need)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "workspace of %zu bytes required, got %zu", need, workspace_bytes);
+  const ColGeom g = make_col_geom(outer, reduce, inner, tile, dtype == QWIX_BF16 ? 8 : 4);
+  if (int e = run_cols_absmax(x, dtype, g, calibration, static_cast<uint32_t*>(workspace), st)) return e;
+  return run_cols_quantize<0>(x, dtype, g, qtype, calibration, q_layout, static_cast<const uint32_t*>(workspace),
+                              calib_factor, qvalue, scale, zero_point, st);
+}
+
+int qwix_hip_calibrate(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner, int64_t tile,
+                       int calibration, float calib_factor, void* out0, void* out1, void* workspace,
+                       size_t workspace_bytes, void* stream) {
+  if (int e = check_geom(outer, reduce, inner, tile)) return e;
+  if (!x || !out0 || (calibration == QWIX_MINMAX && !out1))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "null input or output");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (inner == 1)
+    return run_rows<MODE_CALIB>(x, dtype, outer * (reduce / tile), tile, QWIX_INT8, calibration, calib_factor,
+                                nullptr, nullptr, nullptr, out0, out1, st);
+  if (int e = check_cols(x, dtype, reduce, inner, tile, QWIX_LAYOUT_NATURAL, nullptr)) return e;
+  const size_t need = qwix_hip_quantize_workspace_bytes(outer, reduce, inner, tile, calibration);
+  if (!workspace || workspace_bytes < need)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "workspace of %zu bytes required, got %zu", need, workspace_bytes);
+  const ColGeom g = make_col_geom(outer, reduce, inner, tile, dtype == QWIX_BF16 ? 8 : 4);
+  if (int e = run_cols_absmax(x, dtype, g, calibration, static_cast<uint32_t*>(workspace), st)) return e;
+  const int64_t n = outer * (reduce / tile) * inner;
+  QWIX_DISPATCH_D(dtype, {
+    if (calibration == QWIX_MINMAX)
+      cols_finish_cal_kernel<D, QWIX_MINMAX><<<dim3(static_cast<unsigned>((n + 255) / 256)), 256, 0, st>>>(
+          static_cast<const uint32_t*>(workspace), n, calib_factor, out0, out1);
+    else
+      cols_finish_cal_kernel<D, QWIX_ABSMAX><<<dim3(static_cast<unsigned>((n + 255) / 256)), 256, 0, st>>>(
+          static_cast<const uint32_t*>(workspace), n, calib_factor, out0, out1);
+  })
+  return check_launch("finish calibration");
+}
+
+int qwix_hip_compute_scale_zero_point(const void* cal0, const void* cal1, int dtype, int64_t n, int qtype,
+                                      int calibration, void* scale, void* zero_point, void* stream) {
+  if (n <= 0 || !cal0 || !scale || (calibration == QWIX_MINMAX && (!cal1 || !zero_point)))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad arguments to compute_scale_zero_point");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  QWIX_DISPATCH_D(dtype, {
+    QWIX_DISPATCH_QT_CAL(qtype, calibration, {
+      scale_zp_kernel<D, QT, CAL><<<dim3(static_cast<unsigned>((n + 255) / 256)), 256, 0, st>>>(
+          cal0, cal1, n, scale, static_cast<int8_t*>(zero_point));
+    })
+  })
+  return check_launch("compute_scale_zero_point");
+}
+
+int qwix_hip_quantize_with_scale(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner,
+                                 int64_t tile, int qtype, const void* scale, const void* zero_point, int q_layout,
+                                 void* qvalue, void* stream) {
+  if (int e = check_geom(outer, reduce, inner, tile)) return e;
+  if (!x || !qvalue || !scale) return fail(QWIX_ERR_INVALID_ARGUMENT, "null x/qvalue/scale");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int cal = zero_point ? QWIX_MINMAX : QWIX_ABSMAX;
+  if (inner == 1)
+    return run_rows<MODE_GIVEN>(x, dtype, outer * (reduce / tile), tile, qtype, cal, 0.f, qvalue,
+                                const_cast<void*>(scale), const_cast<void*>(zero_point), nullptr, nullptr, st);
+  if (int e = check_cols(x, dtype, reduce, inner, tile, q_layout, qvalue)) return e;
+  const ColGeom g = make_col_geom(outer, reduce, inner, tile, dtype == QWIX_BF16 ? 8 : 4);
+  return run_cols_quantize<1>(x, dtype, g, qtype, cal, q_layout, nullptr, 0.f, qvalue, const_cast<void*>(scale),
+                              const_cast<void*>(zero_point), st);
+}
+
+int qwix_hip_quantize_generic(const void* x, int dtype, const int64_t dims[5], int64_t t1, int64_t t3, int qtype,
+                              int calibration, float calib_factor, void* qvalue, void* scale, void* zero_point,
+                              void* stream) {
+  if (!x || !qvalue || !scale || !dims) return fail(QWIX_ERR_INVALID_ARGUMENT, "null argument");
+  Geom5 g;
+  int64_t n = 1;
+  for (int i = 0; i < 5; ++i) {
+    if (dims[i] <= 0) return fail(QWIX_ERR_INVALID_ARGUMENT, "dims[%d] = %lld", i, (long long)dims[i]);
+    g.d[i] = dims[i];
+    n *= dims[i];
+  }
+  if (t1 <= 0 || t3 <= 0 || dims[1] % t1 || dims[3] % t3)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "tiles (%lld, %lld) do not divide (%lld, %lld)", (long long)t1,
+                (long long)t3, (long long)dims[1], (long long)dims[3]);
+  if (qtype == QWIX_INT4 && (n & 1)) return fail(QWIX_ERR_UNSUPPORTED, "int4 needs an even element count");
+  if (calibration == QWIX_MINMAX && !zero_point) return fail(QWIX_ERR_INVALID_ARGUMENT, "minmax needs zero_point");
+  g.t1 = t1;
+  g.t3 = t3;
+  const int64_t ns = dims[0] * (dims[1] / t1) * dims[2] * (dims[3] / t3) * dims[4];
+  const int64_t nb = qtype == QWIX_INT4 ? n / 2 : n;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  QWIX_DISPATCH_D(dtype, {
+    QWIX_DISPATCH_QT_CAL(qtype, calibration, {
+      generic_scale_kernel<D, QT, CAL><<<dim3(static_cast<unsigned>((ns + 255) / 256)), 256, 0, st>>>(
+          x, g, calib_factor, scale, static_cast<int8_t*>(zero_point));
+      generic_quant_kernel<D, QT, CAL><<<dim3(static_cast<unsigned>((nb + 255) / 256)), 256, 0, st>>>(
+          x, g, scale, static_cast<const int8_t*>(zero_point), static_cast<uint8_t*>(qvalue));
+    })
+  })
+  return check_launch("generic quantize");
+}
+
+int qwix_hip_dequantize(const void* qvalue, int qtype, int q_layout, int64_t outer, int64_t reduce, int64_t inner,
+                        int64_t tile, const void* scale, const void* zero_point, int dtype, void* out,
+                        void* stream) {
+  if (int e = check_geom(outer, reduce, inner, tile)) return e;
+  if (!qvalue || !scale || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null argument");
+  if (q_layout != QWIX_LAYOUT_NATURAL && q_layout != QWIX_LAYOUT_REDUCE_MINOR)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "unknown layout %d", q_layout);
+  const int64_t n = outer * reduce * inner;
+  const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint8_t* q = static_cast<const uint8_t*>(qvalue);
+  const int8_t* zp = static_cast<const int8_t*>(zero_point);
+  QWIX_DISPATCH_D(dtype, {
+    if (qtype == QWIX_INT8)
+      dequant_kernel<D, QWIX_INT8><<<blocks, 256, 0, st>>>(q, q_layout, outer, reduce, inner, tile, scale, zp, out);
+    else if (qtype == QWIX_INT4)
+      dequant_kernel<D, QWIX_INT4><<<blocks, 256, 0, st>>>(q, q_layout, outer, reduce, inner, tile, scale, zp, out);
+    else if (qtype == QWIX_E4M3)
+      dequant_kernel<D, QWIX_E4M3><<<blocks, 256, 0, st>>>(q, q_layout, outer, reduce, inner, tile, scale, zp, out);
+    else
+      return fail(QWIX_ERR_INVALID_ARGUMENT, "unknown qtype %d", qtype);
+  })
+  return check_launch("dequantize");
+}
+
+int qwix_hip_transpose_q(const void* src, int qtype, int64_t rows, int64_t cols, void* dst, void* stream) {
+  if (!src || !dst || rows <= 0 || cols <= 0) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad transpose arguments");
+  if (qtype == QWIX_INT4 && ((rows & 1) || (cols & 1)))
+    return fail(QWIX_ERR_UNSUPPORTED, "int4 transpose needs even rows and cols");
+  const dim3 grid(static_cast<unsigned>((cols + 63) / 64), static_cast<unsigned>((rows + 63) / 64));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (qtype == QWIX_INT4)
+    transpose_q_kernel<QWIX_INT4><<<grid, 256, 0, st>>>(static_cast<const uint8_t*>(src), rows, cols,
+                                                        static_cast<uint8_t*>(dst));
+  else
+    transpose_q_kernel<QWIX_INT8><<<grid, 256, 0, st>>>(static_cast<const uint8_t*>(src), rows, cols,
+                                                        static_cast<uint8_t*>(dst));
+  return check_launch("transpose");
+}
+
+}  // extern "C"

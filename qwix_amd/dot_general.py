@@ -1,0 +1,290 @@
+"""Quantized dot_general on MI355X: the host-side operator in front of the MFMA GEMM kernels.
+
+Mirror of qwix/_src/core/dot_general.py: `get_how_to_quantize` (:28-76), the dispatcher
+`dot_general` (:407-491) with its 128 threshold (:404), `_fast_dot_general` (:135-261,
+quantized contraction + dequantize on output) and `_slow_dot_general` (:264-275, dequantize
+first).  Arguments are torch tensors / QArrays in HBM; `dimension_numbers` is
+((lhs_contracting, rhs_contracting), (lhs_batch, rhs_batch)) as in jax.lax.dot_general.
+
+What reaches a hand-written kernel:
+  int8 x int8, e4m3 x e4m3 (per-row x per-column scales)          -> qwix_hip_qgemm
+  int8 x int8/int4 with K-group scales (tile % 128 == 0)          -> qwix_hip_qgemm_grouped
+  bf16 activations x int4/int8 weight (weight-only, any group)    -> qwix_hip_gemv_wq
+Everything else on the slow path is dequantized by the HIP dequantize kernel and contracted by
+the vendor float GEMM.  Unsupported fast-path combinations raise; they never change path silently.
+"""
+from __future__ import annotations
+
+import math
+from typing import Any, Mapping, Sequence
+
+import torch
+
+from qwix_amd import _lib
+from qwix_amd import numerics
+from qwix_amd import qarray
+from qwix_amd.qarray import Int4Tensor, QArray
+
+DotDimensionNumbers = tuple[tuple[Sequence[int], Sequence[int]], tuple[Sequence[int], Sequence[int]]]
+
+
+def get_how_to_quantize(*, dimension_numbers: DotDimensionNumbers, ndims: tuple[int, int], for_lhs: bool,
+                        tile_size: Mapping[int, int | float] | int | float | None, **kwargs: Any) -> qarray.HowToQuantize:
+  """Channelwise on every non-contracting axis; sub-channel tiles on the last contracting axis
+  when tile_size is given (a mapping is used verbatim)."""
+  side = 0 if for_lhs else 1
+  ndim, contracting = ndims[side], tuple(dimension_numbers[0][side])
+  if isinstance(tile_size, Mapping):
+    tiled = dict(tile_size)
+  else:
+    tiled = {contracting[-1]: tile_size} if tile_size else {}
+  channelwise = sorted(set(range(ndim)) - set(contracting) - set(tiled))
+  return qarray.HowToQuantize(channelwise_axes=channelwise, tiled_axes=tiled, **kwargs)
+
+
+# If a contracting axis is tiled finer than this, dequantize the inputs instead (dot_general.py:404).
+MIN_TILE_SIZE_TO_DEQUANT_ON_OUTPUT = 128
+
+
+def _is_float_array(x) -> bool:
+  return isinstance(x, torch.Tensor) and numerics.should_quantize(x.dtype)
+
+
+def _use_fast_path(lhs, rhs, dimension_numbers) -> bool:
+  for operand, ca in zip((lhs, rhs), dimension_numbers[0]):
+    if not isinstance(operand, QArray):
+      if _is_float_array(operand):
+        return False
+      continue
+    qarray.validate_qarray(operand)
+    if not numerics.can_dequant_on_output(operand.qtype):
+      return False
+    for axis in ca:
+      if operand.scale.shape[axis] > 1:
+        if operand.shape[axis] // operand.scale.shape[axis] < MIN_TILE_SIZE_TO_DEQUANT_ON_OUTPUT:
+          return False
+  return True
+
+
+# ------------------------------------------------------------------------------------------
+# 2-D canonical form
+# ------------------------------------------------------------------------------------------
+
+
+class _Canon:
+  """lhs as (M, K) row-major, rhs as (N, K) K-contiguous, plus scales in kernel order."""
+
+  def __init__(self, lhs, rhs, dimension_numbers):
+    (lca, rca), (lba, rba) = dimension_numbers
+    lca, rca = [int(a) for a in lca], [int(a) for a in rca]
+    if len(lba) or len(rba):
+      raise NotImplementedError('batch dimensions are not supported by the HIP dot_general yet')
+    if len(lca) != len(rca) or not lca:
+      raise ValueError(f'bad contracting axes {lca} {rca}')
+    lshape, rshape = tuple(lhs.shape), tuple(rhs.shape)
+    for l, r in zip(lca, rca):
+      if lshape[l] != rshape[r]:
+        raise ValueError(f'contracting dimensions differ: lhs {lshape} axis {l} vs rhs {rshape} axis {r}')
+    pairs = sorted(zip(lca, rca))
+    self.lca = [p[0] for p in pairs]
+    self.rca = [p[1] for p in pairs]
+    if self.lca != list(range(len(lshape) - len(lca), len(lshape))):
+      raise NotImplementedError(
+          f'lhs contracting axes {lca} must be the trailing axes of {lshape}; transpose the activation first'
+      )
+    self.lfree = [a for a in range(len(lshape)) if a not in self.lca]
+    self.rfree = [a for a in range(len(rshape)) if a not in self.rca]
+    self.M = math.prod(lshape[a] for a in self.lfree)
+    self.N = math.prod(rshape[a] for a in self.rfree)
+    self.K = math.prod(lshape[a] for a in self.lca)
+    self.out_shape = tuple(lshape[a] for a in self.lfree) + tuple(rshape[a] for a in self.rfree)
+
+  # -- values
+  def lhs_values(self, lhs) -> torch.Tensor:
+    v = lhs.qvalue if isinstance(lhs, QArray) else lhs
+    if isinstance(v, Int4Tensor):
+      raise NotImplementedError('an int4 left operand is not supported by the HIP GEMM kernels')
+    v = v if v.is_contiguous() else v.contiguous()
+    return v.reshape(self.M, self.K)
+
+  def rhs_values(self, rhs) -> tuple[torch.Tensor, bool]:
+    """(N, K) K-contiguous storage (for int4: (N, K/2) bytes), is_int4."""
+    v = rhs.qvalue if isinstance(rhs, QArray) else rhs
+    order = self.rfree + self.rca
+    if isinstance(v, Int4Tensor):
+      p = v.permute(*order)
+      if p.packed_axis == len(order) - 1 and p.data.is_contiguous():
+        return p.data.reshape(self.N, self.K // 2), True
+      nat = v.permute(*(self.rca + self.rfree))
+      if nat.packed_axis == len(order) - 1 and nat.data.is_contiguous():
+        dst = torch.empty(self.N, self.K // 2, dtype=torch.uint8, device=v.device)
+        _lib.call('qwix_hip_transpose_q', nat.data.data_ptr(), _lib.INT4, self.K, self.N, dst.data_ptr(),
+                  _lib.stream_of(dst))
+        return dst, True
+      raise NotImplementedError(f'int4 weight layout {v} cannot be brought to K-contiguous form')
+    p = v.permute(*order)
+    if p.is_contiguous():
+      return p.reshape(self.N, self.K), False
+    nat = v.permute(*(self.rca + self.rfree))
+    if nat.is_contiguous() and v.element_size() == 1:
+      dst = torch.empty(self.N, self.K, dtype=v.dtype, device=v.device)
+      _lib.call('qwix_hip_transpose_q', nat.data_ptr(), _lib.INT8, self.K, self.N, dst.data_ptr(), _lib.stream_of(dst))
+      return dst, False
+    return p.contiguous().reshape(self.N, self.K), False
+
+  # -- scales
+  def lhs_scale(self, lhs: QArray) -> tuple[torch.Tensor | None, int]:
+    """(scale as (M, ga) contiguous, ga)."""
+    s = lhs.scale
+    for a in self.lca[:-1]:
+      if s.shape[a] != 1:
+        raise NotImplementedError('only the last contracting axis of the lhs may carry sub-channel scales')
+    ga = s.shape[self.lca[-1]]
+    if ga > 1 and len(self.lca) > 1:
+      raise NotImplementedError('sub-channel lhs scales with several contracting axes are not supported')
+    want = tuple(lhs.shape[a] for a in self.lfree)
+    got = tuple(s.shape[a] for a in self.lfree)
+    if got != want:
+      s = s.expand(*[lhs.shape[a] if a in self.lfree else s.shape[a] for a in range(s.ndim)])
+    return s.reshape(self.M, ga).contiguous(), ga
+
+  def rhs_scale(self, rhs: QArray) -> tuple[torch.Tensor | None, int]:
+    """(scale as (gb, N) contiguous, gb)."""
+    s = rhs.scale
+    for a in self.rca[:-1]:
+      if s.shape[a] != 1:
+        raise NotImplementedError('only the last contracting axis of the rhs may carry sub-channel scales')
+    gb = s.shape[self.rca[-1]]
+    if gb > 1 and len(self.rca) > 1:
+      raise NotImplementedError('sub-channel rhs scales with several contracting axes are not supported')
+    if tuple(s.shape[a] for a in self.rfree) != tuple(rhs.shape[a] for a in self.rfree):
+      s = s.expand(*[rhs.shape[a] if a in self.rfree else s.shape[a] for a in range(s.ndim)])
+    s = s.permute(*([self.rca[-1]] + self.rfree + self.rca[:-1]))
+    return s.reshape(gb, self.N).contiguous(), gb
+
+
+def _tag_of(dtype: torch.dtype) -> int:
+  if dtype == torch.int32:
+    return _lib.I32
+  return _lib.float_tag(dtype)
+
+
+def _qtype_of(x) -> str:
+  if isinstance(x, QArray):
+    return numerics.canonical_qtype(x.qtype)
+  if isinstance(x, Int4Tensor):
+    return numerics.INT4
+  return numerics.canonical_qtype(x.dtype)
+
+
+def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, *, exact: bool = False,
+                      return_accumulators: bool = False, **kwargs) -> torch.Tensor:
+  """Contract the quantized values on the matrix cores, then scale: out = ((acc * sx) * sy)."""
+  del kwargs
+  for x in (lhs, rhs):
+    if isinstance(x, QArray) and x.zero_point is not None:
+      if isinstance(lhs, QArray) and isinstance(rhs, QArray) and lhs.zero_point is not None and rhs.zero_point is not None:
+        raise ValueError('Only one operand can be asymmetric.')
+      raise NotImplementedError('zero-point operands are not supported on the fast path yet; dequantize first')
+  c = _Canon(lhs, rhs, dimension_numbers)
+  lt = qarray.get_tiled_axes(lhs) if isinstance(lhs, QArray) else {}
+  rt = qarray.get_tiled_axes(rhs) if isinstance(rhs, QArray) else {}
+  for l, r in zip(c.lca, c.rca):
+    if lt.get(l) and rt.get(r) and lt[l] != rt[r]:
+      raise ValueError(f'Contracting axes must be tiled with the same tile size. lhs_tiled_axes={lt} rhs_tiled_axes={rt} {dimension_numbers=}')
+  acc_t, res_t = qarray.get_accumulator_and_result_type(lhs, rhs, preferred_element_type=preferred_element_type)
+  lq, rq = _qtype_of(lhs), _qtype_of(rhs)
+  a = c.lhs_values(lhs)
+  b, b_is4 = c.rhs_values(rhs)
+  sa, ga = c.lhs_scale(lhs) if isinstance(lhs, QArray) else (None, 1)
+  sb, gb = c.rhs_scale(rhs) if isinstance(rhs, QArray) else (None, 1)
+  dev = a.device
+  st = _lib.stream_of(a)
+  out = torch.empty(c.M, c.N, dtype=res_t, device=dev)
+  grouped = ga > 1 or gb > 1 or b_is4
+  if not grouped:
+    if (lq, rq) == (numerics.INT8, numerics.INT8):
+      qt = _lib.INT8
+    elif (lq, rq) == (numerics.E4M3, numerics.E4M3):
+      qt = _lib.E4M3
+    else:
+      raise NotImplementedError(f'no MFMA kernel for {lq} x {rq} operands')
+    if return_accumulators:
+      acc = torch.empty(c.M, c.N, dtype=torch.int32, device=dev)
+      _lib.call('qwix_hip_qgemm', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), qt, c.M, c.N, c.K, None, 0,
+                None, 0, 0, acc.data_ptr(), _lib.I32, c.N, st)
+    _lib.call('qwix_hip_qgemm', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), qt, c.M, c.N, c.K,
+              _lib.ptr(sa), 0 if sa is None else _lib.float_tag(sa.dtype), _lib.ptr(sb),
+              0 if sb is None else _lib.float_tag(sb.dtype), _tag_of(acc_t) if acc_t != torch.int32 else 0,
+              out.data_ptr(), _tag_of(res_t), c.N, st)
+    out = out.reshape(c.out_shape)
+    return (out, acc.reshape(c.out_shape)) if return_accumulators else out
+  # sub-channel / int4 weights
+  if lq != numerics.INT8 or rq not in (numerics.INT8, numerics.INT4):
+    raise NotImplementedError(f'sub-channel MFMA kernel needs int8 x int8/int4 operands, got {lq} x {rq}')
+  ngroups = max(ga, gb)
+  if c.K % ngroups or (c.K // ngroups) % 128:
+    raise NotImplementedError(f'K-group size {c.K / ngroups} must be a multiple of 128')
+  group = c.K // ngroups
+  if sb is None:
+    raise NotImplementedError('grouped GEMM needs rhs scales')
+  if gb != ngroups:  # rhs per-channel, lhs tiled: repeat the rhs scale per group
+    sb = sb.expand(ngroups, c.N).contiguous()
+  acc = torch.empty(ngroups, c.M, c.N, dtype=torch.int32, device=dev) if return_accumulators else None
+  _lib.call('qwix_hip_qgemm_grouped', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
+            _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, group, _lib.ptr(sa),
+            0 if sa is None else _lib.float_tag(sa.dtype), ga, sb.data_ptr(), _lib.float_tag(sb.dtype), out.data_ptr(),
+            _tag_of(res_t), c.N, int(exact), _lib.ptr(acc), st)
+  out = out.reshape(c.out_shape)
+  return (out, acc.reshape((ngroups,) + c.out_shape)) if return_accumulators else out
+
+
+def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, **kwargs) -> torch.Tensor:
+  """Dequantize-first path.  A bf16 activation against an int4/int8 weight runs in one fused
+  kernel (dequantize in registers, bf16 MFMA); other combinations dequantize then use the vendor GEMM."""
+  del kwargs
+  if (_is_float_array(lhs) and lhs.dtype == torch.bfloat16 and isinstance(rhs, QArray) and rhs.zero_point is None
+      and _qtype_of(rhs) in (numerics.INT4, numerics.INT8)):
+    try:
+      c = _Canon(lhs, rhs, dimension_numbers)
+      sb, gb = c.rhs_scale(rhs)
+      group = c.K // gb
+      if c.K % 128 == 0 and (group % 128 == 0):
+        x = c.lhs_values(lhs)
+        b, b_is4 = c.rhs_values(rhs)
+        res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.scale.dtype)
+        out = torch.empty(c.M, c.N, dtype=res_t, device=x.device)
+        _lib.call('qwix_hip_gemv_wq', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0),
+                  _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, group, sb.data_ptr(), _lib.float_tag(sb.dtype),
+                  out.data_ptr(), _lib.float_tag(res_t), c.N, _lib.stream_of(x))
+        return out.reshape(c.out_shape)
+    except NotImplementedError:
+      pass
+  if isinstance(lhs, QArray):
+    lhs = qarray.dequantize(lhs)
+  if isinstance(rhs, QArray):
+    rhs = qarray.dequantize(rhs)
+  (lca, rca), (lba, rba) = dimension_numbers
+  if len(lba) or len(rba):
+    raise NotImplementedError('batch dimensions are not supported by the HIP dot_general yet')
+  res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.dtype)
+  ct = torch.promote_types(lhs.dtype, rhs.dtype)
+  out = torch.tensordot(lhs.to(ct), rhs.to(ct), dims=(list(lca), list(rca)))
+  return out.to(res_t)
+
+
+def dot_general(lhs: MaybeQ, rhs: MaybeQ, dimension_numbers: DotDimensionNumbers, precision=None,
+                preferred_element_type=None, **kwargs) -> torch.Tensor:
+  """Drop-in for lax.dot_general that accepts QArray operands.
+
+  Takes the dequantize-first path iff an operand is a raw float array, a qtype cannot be scaled
+  on output, or a contracting axis is tiled finer than 128; otherwise contracts the quantized
+  values directly.  `precision` and extra keywords (e.g. out_sharding) are accepted and ignored.
+  """
+  del precision
+  if _use_fast_path(lhs, rhs, dimension_numbers):
+    return _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type, **kwargs)
+  return _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type, **kwargs)
+
+
+MaybeQ = Any

@@ -1,0 +1,528 @@
+"""QArray and the quantize / dequantize operators, backed by the HIP kernels.
+
+Host-side mirror of qwix/_src/core/qarray.py: same names, argument meaning and errors
+(`QArray` :31-99, `HowToQuantize` :280-325, `get_scale_shape` :332-349, `calibrate` :470-534,
+`compute_scale_zero_point` :537-584, `quantize_with_scale_zero_point` :594-635, `quantize`
+:638-644, `quantize_api` :647-689, `dequantize` :692-708, `get_accumulator_and_result_type`
+:781-821).  Arrays are torch tensors living in HBM; torch only provides memory and streams,
+all arithmetic is done by libqwix_hip.so.
+
+Differences that come from the device layout, not from the numerics:
+  * int4 values are stored packed, two per byte, in an `Int4Tensor` (logical shape preserved);
+  * when the reduced axis of a weight is strided (per-channel / sub-channel (K, N) kernels) the
+    quantized values are written K-contiguous ("reduce-minor") and handed back as a strided view
+    with the logical shape, because that is the operand layout the MFMA GEMM kernels read.
+    `quantize(..., layout='natural')` keeps the input's own layout.
+"""
+from __future__ import annotations
+
+import dataclasses
+import math
+from typing import Any, Callable, Collection, Mapping, Sequence
+
+import torch
+
+from qwix_amd import _lib
+from qwix_amd import numerics
+
+# ------------------------------------------------------------------------------------------
+# Int4 storage
+# ------------------------------------------------------------------------------------------
+
+
+class Int4Tensor:
+  """Packed int4 values: `data` (uint8) has the logical shape with `packed_axis` halved.
+
+  Element 2i of the packed axis sits in the low nibble of byte i, element 2i+1 in the high nibble
+  (two's complement).  `data` may be a strided view; the packed axis is the physically contiguous
+  one for tensors produced by `quantize`.
+  """
+
+  dtype = 'int4'
+
+  def __init__(self, data: torch.Tensor, shape: Sequence[int], packed_axis: int):
+    shape = tuple(int(s) for s in shape)
+    packed_axis = packed_axis % len(shape)
+    want = tuple(s // 2 if a == packed_axis else s for a, s in enumerate(shape))
+    if data.dtype != torch.uint8 or tuple(data.shape) != want or shape[packed_axis] % 2:
+      raise ValueError(f'packed data {tuple(data.shape)} {data.dtype} does not match int4 shape {shape}')
+    self.data, self.shape, self.packed_axis = data, shape, packed_axis
+
+  ndim = property(lambda self: len(self.shape))
+  device = property(lambda self: self.data.device)
+
+  def unpack(self) -> torch.Tensor:
+    """int8 tensor of the logical shape (host-side convenience for inspection and tests)."""
+    d = self.data.movedim(self.packed_axis, -1)
+    lo = ((d & 0xF).to(torch.int8) ^ 8) - 8
+    hi = ((d >> 4).to(torch.int8) ^ 8) - 8
+    out = torch.stack([lo, hi], dim=-1).reshape(*d.shape[:-1], d.shape[-1] * 2)
+    return out.movedim(-1, self.packed_axis)
+
+  def permute(self, *axes) -> 'Int4Tensor':
+    axes = tuple(axes[0]) if len(axes) == 1 and not isinstance(axes[0], int) else tuple(axes)
+    return Int4Tensor(self.data.permute(*axes), tuple(self.shape[a] for a in axes), axes.index(self.packed_axis))
+
+  def __repr__(self):
+    return f'Int4Tensor(shape={self.shape}, packed_axis={self.packed_axis}, device={self.device})'
+
+
+def _qshape(q) -> tuple[int, ...]:
+  return tuple(q.shape)
+
+
+# ------------------------------------------------------------------------------------------
+# QArray / HowToQuantize
+# ------------------------------------------------------------------------------------------
+
+
+@dataclasses.dataclass
+class QArray:
+  """A quantized array: original ~= (qvalue - zero_point) * generic_broadcast(scale).
+
+  qvalue.shape == original.shape; scale.ndim == original.ndim and every scale dim divides the
+  array dim (sub-channel scales); zero_point is None for symmetric quantization; qtype is the
+  logical type ('int8', 'int4', 'float8_e4m3fn').
+  """
+
+  qvalue: Any  # torch.Tensor (int8 / float8_e4m3fn) or Int4Tensor
+  scale: torch.Tensor
+  zero_point: torch.Tensor | None = None
+  qtype: Any = None
+
+  def __post_init__(self):
+    if self.qtype is None:
+      self.qtype = 'int4' if isinstance(self.qvalue, Int4Tensor) else str(self.qvalue.dtype).replace('torch.', '')
+    self.qtype = numerics.canonical_qtype(self.qtype) if numerics.can_dequant_on_output(self.qtype) else self.qtype
+
+  shape = property(lambda self: _qshape(self.qvalue))
+  ndim = property(lambda self: len(self.shape))
+  dtype = property(lambda self: self.scale.dtype)
+  device = property(lambda self: self.scale.device)
+
+  @property
+  def scale_tile_shape(self) -> tuple[int, ...]:
+    return tuple(o // s for o, s in zip(self.shape, self.scale.shape))
+
+  @property
+  def zero_point_tile_shape(self) -> tuple[int, ...] | None:
+    if self.zero_point is None:
+      return None
+    return tuple(o // s for o, s in zip(self.shape, self.zero_point.shape))
+
+  def astype(self, dtype: torch.dtype) -> 'QArray':
+    """Casts the dequantized type, i.e. the scale dtype."""
+    return dataclasses.replace(self, scale=self.scale.to(dtype))
+
+  def transpose(self, *axes) -> 'QArray':
+    if not axes:
+      axes = tuple(reversed(range(self.ndim)))
+    elif len(axes) == 1 and not isinstance(axes[0], int):
+      axes = tuple(axes[0])
+    zp = None if self.zero_point is None else self.zero_point.permute(*axes)
+    return QArray(self.qvalue.permute(*axes), self.scale.permute(*axes), zp, self.qtype)
+
+  def swapaxes(self, a: int, b: int) -> 'QArray':
+    axes = list(range(self.ndim))
+    axes[a], axes[b] = axes[b], axes[a]
+    return self.transpose(*axes)
+
+  T = property(lambda self: self.transpose())
+
+
+@dataclasses.dataclass(frozen=True, kw_only=True)
+class HowToQuantize:
+  """How to quantize an array (qarray.py:280-325).
+
+  channelwise_axes get one scale per index; tiled_axes map an axis to a tile size (int) or to
+  1/tile_count (float); every other axis shares one scale.  calibration_method is
+  'absmax[,factor]' or 'minmax[,factor]'.
+  """
+
+  qtype: Any
+  channelwise_axes: Collection[int] = ()
+  tiled_axes: Mapping[int, int | float] = dataclasses.field(default_factory=dict)
+  calibration_method: str = 'absmax'
+  noise_fn: Callable | None = None
+
+
+MaybeQArray = Any
+
+
+def _resolve_tile(dim: int, tile) -> int:
+  return round(dim * tile) if isinstance(tile, float) else int(tile)
+
+
+def get_scale_shape(array_shape: Sequence[int], how: HowToQuantize) -> tuple[int, ...]:
+  if set(how.channelwise_axes) & set(how.tiled_axes.keys()):
+    raise ValueError('The same axis cannot be both channelwise and tiled.')
+  out = []
+  for axis, dim in enumerate(array_shape):
+    if axis in how.channelwise_axes:
+      out.append(dim)
+    elif axis in how.tiled_axes:
+      t = _resolve_tile(dim, how.tiled_axes[axis])
+      if t <= 0 or dim % t != 0:
+        raise ValueError(f'{tuple(array_shape)} cannot be tiled as {dict(how.tiled_axes)}.')
+      out.append(dim // t)
+    else:
+      out.append(1)
+  return tuple(out)
+
+
+def get_tiled_axes(array: QArray) -> dict[int, int]:
+  """Infers {axis: tile size} of the sub-channel axes from the shapes (qarray.py:409-422)."""
+  return {i: j // k for i, (j, k) in enumerate(zip(array.shape, array.scale.shape)) if j != k and k != 1}
+
+
+def validate_qarray(array: QArray) -> None:
+  """Internal-consistency checks of qarray.py:212-247."""
+  qs, ss = array.shape, tuple(array.scale.shape)
+  if len(qs) != len(ss):
+    raise ValueError(f'Scale {ss} should have the same rank as qvalue {qs}.')
+  if not all(a % b == 0 for a, b in zip(qs, ss)):
+    raise ValueError(f'Scale {ss} should be broadcastable to qvalue {qs}.')
+  if not numerics.should_quantize(array.scale.dtype):
+    raise ValueError(f'{array.scale.dtype} is not a valid type for scale.')
+  if array.zero_point is not None:
+    zs = tuple(array.zero_point.shape)
+    if len(zs) != len(qs):
+      raise ValueError(f'Zero point {zs} should have the same rank as qvalue {qs}.')
+    if not all(a % b == 0 for a, b in zip(qs, zs)):
+      raise ValueError(f'Zero point {zs} should be broadcastable to qvalue {qs}.')
+    if array.zero_point.dtype != torch.int8:
+      raise ValueError(f'Zero point {array.zero_point.dtype} should be int8 (the storage dtype of int8/int4).')
+
+
+# ------------------------------------------------------------------------------------------
+# Mapping an n-D quantization pattern to the kernels' (outer, reduce, inner, tile) view
+# ------------------------------------------------------------------------------------------
+
+
+@dataclasses.dataclass
+class _Plan:
+  kind: str                      # '3d' or '5d'
+  dims: tuple[int, ...]          # (outer, reduce, inner) or (d0, r1, d2, r3, d4)
+  tiles: tuple[int, ...]         # (tile,) or (t1, t3)
+  outer_axes: tuple[int, ...] = ()
+  reduce_axes: tuple[int, ...] = ()
+  inner_axes: tuple[int, ...] = ()
+
+
+def _plan(shape: Sequence[int], tiles: Sequence[int]) -> _Plan:
+  """tiles[a] = elements of axis a that share one scale (1 = channelwise, dim = fully reduced)."""
+  blocks: list[list] = []  # ['c', size, axes] or ['r', reduce, tile, axes]
+  for a, (d, t) in enumerate(zip(shape, tiles)):
+    if d == 1:
+      if blocks:
+        blocks[-1][-1].append(a)
+      else:
+        blocks.append(['c', 1, [a]])
+      continue
+    if t == 1:
+      if blocks and blocks[-1][0] == 'c':
+        blocks[-1][1] *= d
+        blocks[-1][-1].append(a)
+      else:
+        blocks.append(['c', d, [a]])
+    elif t == d and blocks and blocks[-1][0] == 'r':
+      blocks[-1][1] *= d
+      blocks[-1][2] *= d
+      blocks[-1][-1].append(a)
+    else:
+      blocks.append(['r', d, t, [a]])
+  kinds = ''.join(b[0] for b in blocks)
+  nr = kinds.count('r')
+  if nr == 0:
+    n = math.prod(shape)
+    return _Plan('3d', (n, 1, 1), (1,), tuple(range(len(shape))), (), ())
+  if nr == 1:
+    i = kinds.index('r')
+    if kinds[:i].count('c') > 1 or kinds[i + 1:].count('c') > 1:
+      raise AssertionError(kinds)
+    outer = math.prod(b[1] for b in blocks[:i])
+    inner = math.prod(b[1] for b in blocks[i + 1:])
+    flat = lambda bs: tuple(a for b in bs for a in b[-1])
+    return _Plan('3d', (outer, blocks[i][1], inner), (blocks[i][2],), flat(blocks[:i]), tuple(blocks[i][-1]), flat(blocks[i + 1:]))
+  if nr == 2 and kinds in ('rr', 'crr', 'rcr', 'rrc', 'crcr', 'crrc', 'rcrc', 'crcrc'):
+    it = iter(blocks)
+    dims, ts = [], []
+    b = next(it, None)
+    for slot in 'crcrc':
+      if b is not None and b[0] == slot:
+        dims.append(b[1])
+        if slot == 'r':
+          ts.append(b[2])
+        b = next(it, None)
+      else:
+        dims.append(1)
+        if slot == 'r':
+          ts.append(1)
+    return _Plan('5d', tuple(dims), tuple(ts))
+  raise NotImplementedError(
+      f'quantization pattern of shape {tuple(shape)} with per-axis tiles {tuple(tiles)} needs more than two '
+      'separate reduced axis groups; not supported by the HIP kernels.'
+  )
+
+
+def _tiles_from_how(shape, how: HowToQuantize) -> tuple[int, ...]:
+  ss = get_scale_shape(shape, how)
+  return tuple(d // s for d, s in zip(shape, ss))
+
+
+def _parse_calibration(method: str) -> tuple[int, float]:
+  name, *args = method.lower().split(',')
+  args = [float(a) for a in args]
+  if name not in ('absmax', 'minmax'):
+    raise ValueError(f'Unsupported calibration: {method}')
+  return (_lib.ABSMAX if name == 'absmax' else _lib.MINMAX), (args[0] if args else 0.0)
+
+
+def _check_float_input(array: torch.Tensor) -> torch.Tensor:
+  if not isinstance(array, torch.Tensor) or not numerics.should_quantize(array.dtype):
+    raise ValueError(f'Refuse to quantize: {getattr(array, "dtype", type(array))}')
+  return array if array.is_contiguous() else array.contiguous()
+
+
+def _workspace(plan: _Plan, cal: int, device) -> tuple[torch.Tensor | None, int]:
+  outer, reduce, inner = plan.dims
+  n = _lib.load().qwix_hip_quantize_workspace_bytes(outer, reduce, inner, plan.tiles[0], cal)
+  if n == 0:
+    return None, 0
+  return torch.empty(n, dtype=torch.uint8, device=device), n
+
+
+def _alloc_q(shape, qtype: str, plan: _Plan, layout: int, device):
+  """Allocates the qvalue buffer; returns (flat storage tensor, logical view)."""
+  n = math.prod(shape)
+  is4 = qtype == numerics.INT4
+  if layout == _lib.LAYOUT_NATURAL or plan.kind != '3d' or plan.dims[2] == 1:
+    if is4:
+      if shape[-1] % 2:
+        raise NotImplementedError(f'int4 needs an even last dimension, got {tuple(shape)}')
+      data = torch.empty(*shape[:-1], shape[-1] // 2, dtype=torch.uint8, device=device)
+      return data, Int4Tensor(data, shape, len(shape) - 1)
+    data = torch.empty(tuple(shape), dtype=numerics.storage_dtype(qtype), device=device)
+    return data, data
+  # reduce-minor: physical order (outer axes, inner axes, reduce axes).
+  order = plan.outer_axes + plan.inner_axes + plan.reduce_axes
+  phys_shape = [shape[a] for a in order]
+  inv = [order.index(a) for a in range(len(shape))]
+  if is4:
+    phys_shape[-1] //= 2
+    data = torch.empty(phys_shape, dtype=torch.uint8, device=device)
+    return data, Int4Tensor(data.permute(*inv), shape, order[-1])
+  data = torch.empty(phys_shape, dtype=numerics.storage_dtype(qtype), device=device)
+  return data, data.permute(*inv)
+  del n
+
+
+def _default_layout(plan: _Plan, layout: str | None) -> int:
+  if layout is None:
+    layout = 'reduce_minor' if (plan.kind == '3d' and plan.dims[2] > 1 and plan.dims[1] % 8 == 0 and plan.tiles[0] % 8 == 0) else 'natural'
+  if layout not in ('natural', 'reduce_minor'):
+    raise ValueError(f'unknown layout {layout!r}')
+  return _lib.LAYOUT_NATURAL if layout == 'natural' else _lib.LAYOUT_REDUCE_MINOR
+
+
+# ------------------------------------------------------------------------------------------
+# calibrate / compute_scale_zero_point / quantize_with_scale_zero_point / quantize
+# ------------------------------------------------------------------------------------------
+
+
+def calibrate(array: torch.Tensor, how: HowToQuantize) -> dict[str, torch.Tensor]:
+  """Returns {'absmax': ...} or {'min': ..., 'max': ...}, each shaped like the scale."""
+  array = _check_float_input(array)
+  shape = tuple(array.shape)
+  sshape = get_scale_shape(shape, how)
+  cal, factor = _parse_calibration(how.calibration_method)
+  plan = _plan(shape, _tiles_from_how(shape, how))
+  if plan.kind != '3d':
+    raise NotImplementedError('calibrate() alone supports a single reduced axis group')
+  outs = [torch.empty(sshape, dtype=array.dtype, device=array.device) for _ in range(2 if cal == _lib.MINMAX else 1)]
+  ws, nws = _workspace(plan, cal, array.device)
+  _lib.call('qwix_hip_calibrate', array.data_ptr(), _lib.float_tag(array.dtype), *plan.dims, plan.tiles[0], cal,
+            factor, outs[0].data_ptr(), _lib.ptr(outs[1] if len(outs) > 1 else None), _lib.ptr(ws), nws,
+            _lib.stream_of(array))
+  if cal == _lib.MINMAX:
+    return {'min': outs[0], 'max': outs[1]}
+  return {'absmax': outs[0]}
+
+
+def compute_scale_zero_point(calibration: Mapping[str, torch.Tensor], qtype) -> tuple[torch.Tensor, torch.Tensor | None]:
+  """scale (and zero_point for min/max calibrations) from calibration statistics."""
+  if 'min' in calibration and 'max' in calibration:
+    c0, c1, cal = calibration['min'].contiguous(), calibration['max'].contiguous(), _lib.MINMAX
+    numerics.get_asymmetric_bound(qtype)  # raises for fp8
+  elif 'absmax' in calibration:
+    c0, c1, cal = calibration['absmax'].contiguous(), None, _lib.ABSMAX
+  else:
+    raise ValueError(f'Unsupported calibration: {calibration}')
+  scale = torch.empty_like(c0)
+  zp = torch.empty(c0.shape, dtype=torch.int8, device=c0.device) if cal == _lib.MINMAX else None
+  _lib.call('qwix_hip_compute_scale_zero_point', c0.data_ptr(), _lib.ptr(c1), _lib.float_tag(c0.dtype), c0.numel(),
+            numerics.qtype_tag(qtype), cal, scale.data_ptr(), _lib.ptr(zp), _lib.stream_of(c0))
+  return scale, zp
+
+
+def quantize_with_scale_zero_point(array: torch.Tensor, qtype, scale: torch.Tensor, zero_point: torch.Tensor | None,
+                                   noise_fn=None, *, layout: str | None = None) -> QArray:
+  """Quantizes with a given (static) scale; the scale is first cast to the array dtype."""
+  if noise_fn is not None:
+    raise NotImplementedError('stochastic rounding is not part of the HIP path')
+  array = _check_float_input(array)
+  if zero_point is not None and tuple(zero_point.shape) != tuple(scale.shape):
+    raise ValueError(f'Expect zero_point shape {tuple(scale.shape)} but got {tuple(zero_point.shape)}')
+  shape = tuple(array.shape)
+  if len(shape) != scale.ndim or any(d % s for d, s in zip(shape, scale.shape)):
+    raise ValueError(f'Cannot broadcast between {shape} {tuple(scale.shape)}')
+  q = numerics.canonical_qtype(qtype)
+  scale = scale.to(array.dtype).contiguous()
+  plan = _plan(shape, tuple(d // s for d, s in zip(shape, scale.shape)))
+  if plan.kind != '3d':
+    raise NotImplementedError('static-scale quantization supports a single reduced axis group')
+  lay = _default_layout(plan, layout)
+  data, view = _alloc_q(shape, q, plan, lay, array.device)
+  zp = None if zero_point is None else zero_point.contiguous()
+  _lib.call('qwix_hip_quantize_with_scale', array.data_ptr(), _lib.float_tag(array.dtype), *plan.dims, plan.tiles[0],
+            numerics.qtype_tag(q), scale.data_ptr(), _lib.ptr(zp), lay, data.data_ptr(), _lib.stream_of(array))
+  return QArray(view, scale, zero_point, q)
+
+
+def quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = None) -> QArray:
+  """Dynamic-range quantization: calibrate, derive scale (and zero point), quantize -- one fused pass."""
+  if how.noise_fn is not None:
+    raise NotImplementedError('stochastic rounding is not part of the HIP path')
+  array = _check_float_input(array)
+  shape = tuple(array.shape)
+  q = numerics.canonical_qtype(how.qtype)
+  sshape = get_scale_shape(shape, how)
+  cal, factor = _parse_calibration(how.calibration_method)
+  if cal == _lib.MINMAX:
+    numerics.get_asymmetric_bound(q)
+  plan = _plan(shape, tuple(d // s for d, s in zip(shape, sshape)))
+  scale = torch.empty(sshape, dtype=array.dtype, device=array.device)
+  zp = torch.empty(sshape, dtype=torch.int8, device=array.device) if cal == _lib.MINMAX else None
+  tag = _lib.float_tag(array.dtype)
+  if plan.kind == '5d':
+    data, view = _alloc_q(shape, q, plan, _lib.LAYOUT_NATURAL, array.device)
+    import ctypes
+    dims = (ctypes.c_int64 * 5)(*plan.dims)
+    _lib.call('qwix_hip_quantize_generic', array.data_ptr(), tag, dims, plan.tiles[0], plan.tiles[1],
+              numerics.qtype_tag(q), cal, factor, data.data_ptr(), scale.data_ptr(), _lib.ptr(zp),
+              _lib.stream_of(array))
+    return QArray(view, scale, zp, q)
+  lay = _default_layout(plan, layout)
+  outer, reduce, inner = plan.dims
+  if inner > 1 and (inner % (8 if array.dtype == torch.bfloat16 else 4) != 0):
+    # ragged strided reduce: the complete-but-slow kernel handles it (natural layout).
+    data, view = _alloc_q(shape, q, plan, _lib.LAYOUT_NATURAL, array.device)
+    import ctypes
+    dims = (ctypes.c_int64 * 5)(outer, reduce, inner, 1, 1)
+    _lib.call('qwix_hip_quantize_generic', array.data_ptr(), tag, dims, plan.tiles[0], 1, numerics.qtype_tag(q), cal,
+              factor, data.data_ptr(), scale.data_ptr(), _lib.ptr(zp), _lib.stream_of(array))
+    return QArray(view, scale, zp, q)
+  data, view = _alloc_q(shape, q, plan, lay, array.device)
+  ws, nws = _workspace(plan, cal, array.device)
+  _lib.call('qwix_hip_quantize', array.data_ptr(), tag, outer, reduce, inner, plan.tiles[0], numerics.qtype_tag(q), cal,
+            factor, lay, data.data_ptr(), scale.data_ptr(), _lib.ptr(zp), _lib.ptr(ws), nws, _lib.stream_of(array))
+  return QArray(view, scale, zp, q)
+
+
+def quantize_api(array: torch.Tensor, qtype, *, channelwise_axes: Collection[int] = (),
+                 tiled_axes: Mapping[int, int | float] | None = None, calibration_method: str = 'absmax',
+                 scale_dtype: torch.dtype | None = None, layout: str | None = None) -> QArray:
+  """Public `qwix.quantize`: like quantize() without building a HowToQuantize; the optional
+  scale_dtype cast is applied to the already computed scale."""
+  how = HowToQuantize(qtype=qtype, channelwise_axes=channelwise_axes, tiled_axes=tiled_axes or {},
+                      calibration_method=calibration_method)
+  qa = quantize(array, how, layout=layout)
+  if scale_dtype is not None:
+    qa = dataclasses.replace(qa, scale=qa.scale.to(scale_dtype))
+  return qa
+
+
+# ------------------------------------------------------------------------------------------
+# dequantize
+# ------------------------------------------------------------------------------------------
+
+
+def physical_layout(qa: QArray) -> tuple[_Plan, int, torch.Tensor]:
+  """Finds how a QArray's values are laid out: (plan, layout tag, storage tensor)."""
+  shape = qa.shape
+  plan = _plan(shape, qa.scale_tile_shape)
+  is4 = isinstance(qa.qvalue, Int4Tensor)
+  data = qa.qvalue.data if is4 else qa.qvalue
+  if data.is_contiguous() and (not is4 or qa.qvalue.packed_axis == len(shape) - 1):
+    return plan, _lib.LAYOUT_NATURAL, data
+  if plan.kind == '3d':
+    order = plan.outer_axes + plan.inner_axes + plan.reduce_axes
+    phys = data.permute(*order)
+    if phys.is_contiguous() and (not is4 or qa.qvalue.packed_axis == order[-1]):
+      return plan, _lib.LAYOUT_REDUCE_MINOR, phys
+  raise NotImplementedError(
+      f'QArray values of shape {shape} with strides {tuple(data.stride())} are neither row-major nor '
+      'reduce-minor; make them contiguous first.'
+  )
+
+
+def dequantize(array: QArray) -> torch.Tensor:
+  """(qvalue - zero_point) * scale in the scale dtype; the reverse of quantize."""
+  validate_qarray(array)
+  plan, lay, data = physical_layout(array)
+  if plan.kind != '3d':
+    raise NotImplementedError('dequantize supports a single reduced axis group')
+  out = torch.empty(array.shape, dtype=array.scale.dtype, device=array.scale.device)
+  scale = array.scale.contiguous()
+  zp = None if array.zero_point is None else array.zero_point.contiguous()
+  _lib.call('qwix_hip_dequantize', data.data_ptr(), numerics.qtype_tag(array.qtype), lay, *plan.dims, plan.tiles[0],
+            scale.data_ptr(), _lib.ptr(zp), _lib.float_tag(scale.dtype), out.data_ptr(), _lib.stream_of(scale))
+  return out
+
+
+# ------------------------------------------------------------------------------------------
+# dtype rule
+# ------------------------------------------------------------------------------------------
+
+_INT_NAMES = ('int8', 'int4', 'uint8', 'int16', 'int32')
+
+
+def _dtype_names(x) -> tuple[str, str]:
+  """(qvalue dtype name, dequant dtype name) of an operand."""
+  name = lambda d: str(d).replace('torch.', '')
+  if isinstance(x, QArray):
+    qn = 'int4' if isinstance(x.qvalue, Int4Tensor) else name(x.qvalue.dtype)
+    return qn, name(x.scale.dtype)
+  if isinstance(x, Int4Tensor):
+    return 'int4', 'int4'
+  return name(x.dtype), name(x.dtype)
+
+
+_TORCH = {'float32': torch.float32, 'bfloat16': torch.bfloat16, 'int32': torch.int32}
+
+
+def get_accumulator_and_result_type(*args, preferred_element_type=None):
+  """(accumulator dtype, result dtype) of a quantized contraction (qarray.py:781-821).
+
+  The result type depends only on the dequantized dtypes (raw 1-byte ints count as int32, other
+  1-byte types as bf16) unless preferred_element_type is given; the accumulator is int32 iff every
+  operand's stored values are integers, otherwise it equals the result type.
+  """
+  qnames, dnames = zip(*[_dtype_names(a) for a in args])
+  result = preferred_element_type
+  if result is None:
+    ds = []
+    for n in dnames:
+      if n in ('int8', 'int4', 'uint8'):
+        ds.append(torch.int32)
+      elif n in ('bool', 'float8_e4m3fn', 'float8_e5m2'):
+        ds.append(torch.bfloat16)
+      else:
+        ds.append(_TORCH[n])
+    floats = [d for d in ds if d.is_floating_point]
+    if not floats:
+      result = torch.int32
+    else:
+      result = torch.float32 if torch.float32 in floats else torch.bfloat16
+  acc = torch.int32 if all('int' in n for n in qnames) else result
+  return acc, result

@@ -1,0 +1,108 @@
+"""GPU parity: MFMA quantized GEMM vs the CPU oracle.
+
+int8: raw int32 accumulators bit-exact; scaled outputs bit-exact (the epilogue is a deterministic
+elementwise function of the exact accumulator).  fp8: f32 accumulation order differs from the
+oracle's exact sum, so outputs are compared at rtol 1e-2 (+ atol for cancelling sums), the
+tolerance the north-star states for bf16 outputs.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import qwix_oracle as O
+from tests import util
+
+pytestmark = pytest.mark.gpu
+DN = (((1,), (0,)), ((), ()))
+
+
+def _quantized_pair(M, K, N, dtype, qtype, seed):
+  from qwix_amd import qarray
+  x_np, x_t = util.make((M, K), dtype, seed=seed)
+  w_np, w_t = util.make((K, N), dtype, seed=seed + 1, scale=0.02)
+  xq = qarray.quantize(x_t, qarray.HowToQuantize(qtype=qtype, channelwise_axes=[0]))
+  wq = qarray.quantize(w_t, qarray.HowToQuantize(qtype=qtype, channelwise_axes=[1]))
+  oxq = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(qtype=qtype, channelwise_axes=[0]))
+  owq = O.quantize(O.FArr(w_np, dtype), O.HowToQuantize(qtype=qtype, channelwise_axes=[1]))
+  return xq, wq, oxq, owq
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (128, 64, 128), (100, 272, 60), (1, 4096, 1024), (1024, 512, 1024), (1300, 1024, 1100)])
+def test_int8_gemm_bit_exact(M, K, N, dtype):
+  from qwix_amd import dot_general as dg
+  print('case int8', M, K, N, dtype, flush=True)
+  xq, wq, oxq, owq = _quantized_pair(M, K, N, dtype, 'int8', seed=M + K + N)
+  out, acc = dg._fast_dot_general(xq, wq, DN, return_accumulators=True)
+  torch.cuda.synchronize()
+  want, wacc = O.fast_dot_general(oxq, owq, DN, return_acc=True)
+  assert np.array_equal(acc.cpu().numpy(), wacc), 'int32 accumulators differ'
+  assert out.dtype == util.TORCH_DT[dtype]
+  got = util.f32np(out)
+  bad = np.flatnonzero(got.ravel() != want.v.ravel())
+  assert bad.size == 0, f'{bad.size} outputs differ: {got.ravel()[bad[:5]]} vs {want.v.ravel()[bad[:5]]}'
+
+
+@pytest.mark.parametrize('pref', [None, torch.float32, torch.bfloat16])
+def test_int8_gemm_mixed_scale_dtypes_and_preferred_type(pref):
+  """bf16 lhs scale x f32 rhs scale -> f32 (dot_general_test.py:43-54), preferred type overrides."""
+  from qwix_amd import dot_general as dg
+  xq, wq, oxq, owq = _quantized_pair(64, 256, 128, O.BF16, 'int8', seed=5)
+  wq = wq.astype(torch.float32)
+  owq = O.QArray(owq.qvalue, owq.scale.astype(O.F32), None, 'int8')
+  out = dg.dot_general(xq, wq, DN, preferred_element_type=pref)
+  want = O.dot_general(oxq, owq, DN, util.ORACLE_DT[pref] if pref else None)
+  assert out.dtype == (pref or torch.float32)
+  assert np.array_equal(util.f32np(out), want.v)
+
+
+def test_raw_int8_operand_stays_on_fast_path():
+  from qwix_amd import dot_general as dg
+  g = util.rng(9)
+  a = g.integers(-128, 128, (32, 128), dtype=np.int8)
+  xq, wq, oxq, owq = _quantized_pair(32, 128, 64, O.F32, 'int8', seed=6)
+  out = dg.dot_general(torch.from_numpy(a).to(util.DEV), wq, DN)
+  want = O.dot_general(a, owq, DN)
+  assert np.array_equal(util.f32np(out), want.v)
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (100, 320, 60), (1024, 2048, 1024)])
+def test_fp8_gemm_close(M, K, N, dtype):
+  from qwix_amd import dot_general as dg
+  print('case fp8', M, K, N, dtype, flush=True)
+  xq, wq, oxq, owq = _quantized_pair(M, K, N, dtype, 'float8_e4m3fn', seed=M + K)
+  out = dg.dot_general(xq, wq, DN)
+  torch.cuda.synchronize()
+  want = O.dot_general(oxq, owq, DN)
+  assert out.dtype == util.TORCH_DT[dtype]
+  got = util.f32np(out)
+  tol = 1e-2 if dtype == O.BF16 else 1e-5
+  scale = np.abs(want.v).mean()
+  assert np.allclose(got, want.v, rtol=tol, atol=tol * scale), np.abs(got - want.v).max()
+  # exact f32 products: with f32 outputs the only difference is summation order
+  if dtype == O.F32:
+    assert np.abs(got - want.v).max() <= 2e-6 * np.abs(want.v).max() * np.sqrt(K)
+
+
+def test_gemm_linearity_full_size_property():
+  """Size-independent check at the benchmark shape: int32 accumulators are linear in the lhs rows
+  and match a float64 product on sampled rows."""
+  from qwix_amd import dot_general as dg
+  g = util.rng(77)
+  M = N = K = 4096
+  a = torch.from_numpy(g.integers(-127, 128, (M, K), dtype=np.int8)).to(util.DEV)
+  b = torch.from_numpy(g.integers(-127, 128, (K, N), dtype=np.int8))
+  b_nk = b.t().contiguous().to(util.DEV)
+  from qwix_amd import _lib
+  acc = torch.empty(M, N, dtype=torch.int32, device=util.DEV)
+  _lib.call('qwix_hip_qgemm', a.data_ptr(), K, b_nk.data_ptr(), K, _lib.INT8, M, N, K, None, 0, None, 0, 0,
+            acc.data_ptr(), _lib.I32, N, _lib.stream_of(a))
+  torch.cuda.synchronize()
+  rows = g.choice(M, 16, replace=False)
+  want = a[rows].cpu().numpy().astype(np.float64) @ b.numpy().astype(np.float64)
+  assert np.array_equal(acc[rows].cpu().numpy(), want.astype(np.int64))
+  # checksum of checksums: sum over all outputs == (column sums of a) . (row sums of b)
+  total = acc.to(torch.float64).sum().item()
+  want_total = float(a.to(torch.float64).sum(0).cpu().numpy() @ b.numpy().astype(np.float64).sum(1))
+  assert total == want_total

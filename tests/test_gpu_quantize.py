@@ -1,0 +1,179 @@
+"""GPU parity: HIP quantize / calibrate / dequantize kernels vs the CPU oracle, bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import qwix_oracle as O
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+QTYPES = ['int8', 'int4', 'float8_e4m3fn']
+
+
+def _check(x_np, x_t, dtype, how_kwargs, layout=None, what=''):
+  import qwix_amd
+  from qwix_amd import qarray
+  print('case', what, x_np.shape, dtype, how_kwargs, layout, flush=True)
+  qa = qarray.quantize(x_t, qarray.HowToQuantize(**how_kwargs), layout=layout)
+  torch.cuda.synchronize()
+  want = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(**how_kwargs))
+  util.assert_qarray_equal(qa, want, what)
+  return qa
+
+
+@pytest.mark.parametrize('qtype', QTYPES)
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('shape', [(64, 4096), (7, 1000), (5, 130), (3, 20000), (1, 8), (300, 256), (2, 3, 512)])
+def test_per_token_rows(shape, dtype, qtype):
+  x_np, x_t = util.make(shape, dtype, seed=hash((shape, dtype, qtype)) % 1000)
+  cw = list(range(len(shape) - 1))
+  _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=cw), what='rows')
+
+
+@pytest.mark.parametrize('qtype', QTYPES)
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+def test_rows_subchannel_tiles(dtype, qtype):
+  x_np, x_t = util.make((48, 1024), dtype, seed=11)
+  for tile in (128, 32, 1 / 4):
+    _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=[0], tiled_axes={1: tile}), what=f'rows tile {tile}')
+
+
+@pytest.mark.parametrize('qtype', QTYPES)
+def test_every_bf16_value_rows(qtype):
+  """All finite bf16 bit patterns, grouped so that rows span very different magnitudes."""
+  bits = torch.arange(0, 1 << 16, dtype=torch.int32).to(torch.uint16)
+  xb = bits.view(torch.bfloat16)
+  xb = xb[torch.isfinite(xb)]
+  order = torch.argsort(xb.abs().to(torch.float32), stable=True)
+  xb = xb[order]
+  n = (xb.numel() // 512) * 512
+  for rows_of in (512, 64):
+    x = xb[:n].reshape(-1, rows_of).contiguous()
+    x_np = x.to(torch.float32).numpy()
+    _check(x_np, x.to(util.DEV), O.BF16, dict(qtype=qtype, channelwise_axes=[0]), what=f'all-bf16 rows of {rows_of}')
+  # mixed magnitudes within a row: a strided shuffle
+  x = xb[:n].reshape(512, -1).t().contiguous()
+  _check(x.to(torch.float32).numpy(), x.to(util.DEV), O.BF16, dict(qtype=qtype, channelwise_axes=[0]), what='all-bf16 mixed')
+
+
+@pytest.mark.parametrize('qtype', QTYPES)
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('layout', ['natural', 'reduce_minor'])
+@pytest.mark.parametrize('shape,tile', [((512, 256), None), ((512, 256), 128), ((1000, 64), None), ((384, 128), 64), ((256, 40), None)])
+def test_weight_columns(shape, tile, layout, dtype, qtype):
+  x_np, x_t = util.make(shape, dtype, seed=21, scale=0.02)
+  kw = dict(qtype=qtype, channelwise_axes=[1])
+  if tile:
+    kw['tiled_axes'] = {0: tile}
+  qa = _check(x_np, x_t, dtype, kw, layout=layout, what=f'cols {layout}')
+  from qwix_amd.qarray import Int4Tensor
+  data = qa.qvalue.data if isinstance(qa.qvalue, Int4Tensor) else qa.qvalue
+  if layout == 'reduce_minor':
+    assert data.stride(0) == 1, 'reduce-minor layout must be K-contiguous'
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+def test_weight_3d_einsum_kernel(dtype):
+  """(d, n, h) weight contracting d: outer=1, reduce=d, inner=n*h."""
+  x_np, x_t = util.make((256, 4, 32), dtype, seed=31, scale=0.02)
+  _check(x_np, x_t, dtype, dict(qtype='int8', channelwise_axes=[1, 2]), what='dnh')
+  _check(x_np, x_t, dtype, dict(qtype='int4', channelwise_axes=[1, 2], tiled_axes={0: 128}), what='dnh tiled')
+  # (n, h, d) contracting n, h: reduce = n*h
+  x_np, x_t = util.make((4, 64, 128), dtype, seed=32, scale=0.02)
+  _check(x_np, x_t, dtype, dict(qtype='int8', channelwise_axes=[2]), what='nhd')
+
+
+@pytest.mark.parametrize('qtype', ['int8', 'int4'])
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+def test_minmax(dtype, qtype):
+  x_np, x_t = util.make((40, 512), dtype, seed=41)
+  x_np = x_np + np.float32(0.5) if dtype == O.F32 else O.round_to_bf16(x_np + np.float32(0.5))
+  x_t = torch.from_numpy(x_np).to(util.TORCH_DT[dtype]).to(util.DEV)
+  _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=[0], calibration_method='minmax'), what='minmax rows')
+  _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=[1], calibration_method='minmax'), what='minmax cols')
+  _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=[0], calibration_method='absmax,0.8'), what='absmax factor')
+
+
+def test_reference_exact_minmax_vector():
+  """qarray_test.py:191-219 on the GPU."""
+  from qwix_amd import qarray
+  a = (np.arange(256) / 255.0).astype(np.float32)
+  qa = qarray.quantize(torch.from_numpy(a).to(util.DEV), qarray.HowToQuantize(qtype='int8', calibration_method='minmax'))
+  assert qa.zero_point.reshape(()).item() == -128
+  assert np.array_equal(util.qvalues_np(qa), np.arange(-128, 128).astype(np.int8))
+  dq = qarray.dequantize(qa)
+  assert np.allclose(util.f32np(dq), a)
+
+
+def test_2d_tiles_generic():
+  """two_dim_scales_test.py:29-50."""
+  x_np, x_t = util.make((128, 128), O.BF16, seed=51)
+  qa = _check(x_np, x_t, O.BF16, dict(qtype='int8', tiled_axes={0: 8, 1: 8}), what='2d tiles')
+  assert tuple(qa.scale.shape) == (16, 16)
+  x_np, x_t = util.make((6, 10), O.F32, seed=52)
+  _check(x_np, x_t, O.F32, dict(qtype='int8', channelwise_axes=[1]), what='ragged cols')
+  _check(x_np, x_t, O.F32, dict(qtype='int4'), what='per tensor')
+
+
+def test_zero_rows_and_reference_convert_vectors():
+  from qwix_amd import qarray
+  x = torch.zeros(4, 256, dtype=torch.bfloat16, device=util.DEV)
+  x[1] = 3.0
+  qa = qarray.quantize(x, qarray.HowToQuantize(qtype='int8', channelwise_axes=[0]))
+  assert util.f32np(qa.scale)[:, 0].tolist() == [1.0, float(torch.tensor(3.0 / 127.5).to(torch.bfloat16)), 1.0, 1.0]
+  # numerics_test.py:34-56 through the static-scale kernel with scale 1
+  v = torch.tensor([[1.2, 3.5, -127.5, 129, -1300, float('inf'), float('-inf'), 0.5]], dtype=torch.float32, device=util.DEV)
+  one = torch.ones(1, 1, device=util.DEV)
+  q8 = qarray.quantize_with_scale_zero_point(v, 'int8', one, None)
+  assert util.qvalues_np(q8)[0].tolist() == [1, 4, -128, 127, -128, 127, -128, 0]
+  q4 = qarray.quantize_with_scale_zero_point(v, 'int4', one, None)
+  assert util.qvalues_np(q4)[0].tolist() == [1, 4, -8, 7, -8, 7, -8, 0]
+  f8 = qarray.quantize_with_scale_zero_point(torch.tensor([[10.0, 500.0, -1000.0, 0.0]], device=util.DEV), 'float8_e4m3fn', one, None)
+  assert O.e4m3_to_f32(util.qvalues_np(f8))[0].tolist() == [10.0, 448.0, -448.0, 0.0]
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+def test_calibrate_scale_static_pipeline(dtype):
+  """calibrate -> compute_scale_zero_point -> quantize_with_scale_zero_point == quantize."""
+  from qwix_amd import qarray
+  for shape, kw in [((32, 512), dict(channelwise_axes=[0])), ((256, 64), dict(channelwise_axes=[1])),
+                    ((256, 64), dict(channelwise_axes=[1], tiled_axes={0: 128}))]:
+    for cal in ('absmax', 'minmax'):
+      x_np, x_t = util.make(shape, dtype, seed=61)
+      how = qarray.HowToQuantize(qtype='int8', calibration_method=cal, **kw)
+      c = qarray.calibrate(x_t, how)
+      oc = O.calibrate(O.FArr(x_np, dtype), O.HowToQuantize(qtype='int8', calibration_method=cal, **kw))
+      for k in oc:
+        assert np.array_equal(util.f32np(c[k]), oc[k].v), (shape, kw, cal, k)
+      s, zp = qarray.compute_scale_zero_point(c, 'int8')
+      qa = qarray.quantize_with_scale_zero_point(x_t, 'int8', s, zp)
+      want = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(qtype='int8', calibration_method=cal, **kw))
+      util.assert_qarray_equal(qa, want, f'pipeline {shape} {kw} {cal}')
+
+
+@pytest.mark.parametrize('qtype', QTYPES)
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+def test_dequantize(dtype, qtype):
+  from qwix_amd import qarray
+  for shape, kw, layout in [((32, 512), dict(channelwise_axes=[0]), None), ((256, 64), dict(channelwise_axes=[1], tiled_axes={0: 128}), 'natural'),
+                            ((256, 64), dict(channelwise_axes=[1], tiled_axes={0: 128}), 'reduce_minor')]:
+    x_np, x_t = util.make(shape, dtype, seed=71)
+    qa = qarray.quantize(x_t, qarray.HowToQuantize(qtype=qtype, **kw), layout=layout)
+    dq = qarray.dequantize(qa)
+    want = O.dequantize(O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(qtype=qtype, **kw)))
+    assert dq.dtype == util.TORCH_DT[dtype]
+    assert np.array_equal(util.f32np(dq), want.v), (shape, kw, layout)
+
+
+def test_errors_match_reference_behaviour():
+  from qwix_amd import qarray
+  x = torch.zeros(4, 10, device=util.DEV)
+  with pytest.raises(ValueError, match='cannot be tiled'):
+    qarray.quantize(x, qarray.HowToQuantize(qtype='int8', tiled_axes={1: 4}))
+  with pytest.raises(ValueError, match='both channelwise and tiled'):
+    qarray.quantize(x, qarray.HowToQuantize(qtype='int8', channelwise_axes=[1], tiled_axes={1: 5}))
+  with pytest.raises(ValueError, match='Refuse to quantize'):
+    qarray.quantize(x.to(torch.int32), qarray.HowToQuantize(qtype='int8'))
+  with pytest.raises(ValueError, match="doesn't support asymmetric"):
+    qarray.quantize(x, qarray.HowToQuantize(qtype='float8_e4m3fn', calibration_method='minmax'))
