@@ -21,9 +21,9 @@ from typing import Any, Mapping, Sequence
 import torch
 
 from qwix_amd import _lib
-from qwix_amd import numerics
-from qwix_amd import qarray
-from qwix_amd.qarray import Int4Tensor, QArray
+from qwix_amd.core import numerics
+from qwix_amd.core import qarray
+from qwix_amd.core.qarray import Int4Tensor, QArray
 
 DotDimensionNumbers = tuple[tuple[Sequence[int], Sequence[int]], tuple[Sequence[int], Sequence[int]]]
 

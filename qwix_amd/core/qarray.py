@@ -23,7 +23,7 @@ from typing import Any, Callable, Collection, Mapping, Sequence
 import torch
 
 from qwix_amd import _lib
-from qwix_amd import numerics
+from qwix_amd.core import numerics
 
 # ------------------------------------------------------------------------------------------
 # Int4 storage

@@ -171,7 +171,8 @@ struct Divider {
       // Overflowing or non-finite quotients (static scales only): take the IEEE path.
       if constexpr (kSafe)
         if (!(__builtin_fabsf(q0) < 0x1p100f)) q1 = x / s;
-      return round_bf16(q1);
+      // The residual step turns -0 into +0; the quotient always carries the sign of x (s > 0).
+      return __builtin_copysignf(round_bf16(q1), x);
     } else {
       return x / s;
     }

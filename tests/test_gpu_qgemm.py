@@ -3,7 +3,9 @@
 int8: raw int32 accumulators bit-exact; scaled outputs bit-exact (the epilogue is a deterministic
 elementwise function of the exact accumulator).  fp8: f32 accumulation order differs from the
 oracle's exact sum, so outputs are compared at rtol 1e-2 (+ atol for cancelling sums), the
-tolerance the north-star states for bf16 outputs.
+tolerance the north-star states for bf16 outputs.  With f32 outputs the v_mfma_f32_32x32x64_f8f6f4
+accumulation itself shows up: its 64-wide dot is summed with less than f32 alignment precision
+(measured: up to 1e-4 of the largest output), so the f32 comparison uses rtol 1e-3.
 """
 import numpy as np
 import pytest
@@ -17,7 +19,7 @@ DN = (((1,), (0,)), ((), ()))
 
 
 def _quantized_pair(M, K, N, dtype, qtype, seed):
-  from qwix_amd import qarray
+  from qwix_amd.core import qarray
   x_np, x_t = util.make((M, K), dtype, seed=seed)
   w_np, w_t = util.make((K, N), dtype, seed=seed + 1, scale=0.02)
   xq = qarray.quantize(x_t, qarray.HowToQuantize(qtype=qtype, channelwise_axes=[0]))
@@ -30,7 +32,7 @@ def _quantized_pair(M, K, N, dtype, qtype, seed):
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
 @pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (128, 64, 128), (100, 272, 60), (1, 4096, 1024), (1024, 512, 1024), (1300, 1024, 1100)])
 def test_int8_gemm_bit_exact(M, K, N, dtype):
-  from qwix_amd import dot_general as dg
+  from qwix_amd.core import dot_general as dg
   print('case int8', M, K, N, dtype, flush=True)
   xq, wq, oxq, owq = _quantized_pair(M, K, N, dtype, 'int8', seed=M + K + N)
   out, acc = dg._fast_dot_general(xq, wq, DN, return_accumulators=True)
@@ -46,7 +48,7 @@ def test_int8_gemm_bit_exact(M, K, N, dtype):
 @pytest.mark.parametrize('pref', [None, torch.float32, torch.bfloat16])
 def test_int8_gemm_mixed_scale_dtypes_and_preferred_type(pref):
   """bf16 lhs scale x f32 rhs scale -> f32 (dot_general_test.py:43-54), preferred type overrides."""
-  from qwix_amd import dot_general as dg
+  from qwix_amd.core import dot_general as dg
   xq, wq, oxq, owq = _quantized_pair(64, 256, 128, O.BF16, 'int8', seed=5)
   wq = wq.astype(torch.float32)
   owq = O.QArray(owq.qvalue, owq.scale.astype(O.F32), None, 'int8')
@@ -57,7 +59,7 @@ def test_int8_gemm_mixed_scale_dtypes_and_preferred_type(pref):
 
 
 def test_raw_int8_operand_stays_on_fast_path():
-  from qwix_amd import dot_general as dg
+  from qwix_amd.core import dot_general as dg
   g = util.rng(9)
   a = g.integers(-128, 128, (32, 128), dtype=np.int8)
   xq, wq, oxq, owq = _quantized_pair(32, 128, 64, O.F32, 'int8', seed=6)
@@ -69,7 +71,7 @@ def test_raw_int8_operand_stays_on_fast_path():
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
 @pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (100, 320, 60), (1024, 2048, 1024)])
 def test_fp8_gemm_close(M, K, N, dtype):
-  from qwix_amd import dot_general as dg
+  from qwix_amd.core import dot_general as dg
   print('case fp8', M, K, N, dtype, flush=True)
   xq, wq, oxq, owq = _quantized_pair(M, K, N, dtype, 'float8_e4m3fn', seed=M + K)
   out = dg.dot_general(xq, wq, DN)
@@ -77,18 +79,17 @@ def test_fp8_gemm_close(M, K, N, dtype):
   want = O.dot_general(oxq, owq, DN)
   assert out.dtype == util.TORCH_DT[dtype]
   got = util.f32np(out)
-  tol = 1e-2 if dtype == O.BF16 else 1e-5
+  tol = 1e-2 if dtype == O.BF16 else 1e-3
   scale = np.abs(want.v).mean()
   assert np.allclose(got, want.v, rtol=tol, atol=tol * scale), np.abs(got - want.v).max()
-  # exact f32 products: with f32 outputs the only difference is summation order
   if dtype == O.F32:
-    assert np.abs(got - want.v).max() <= 2e-6 * np.abs(want.v).max() * np.sqrt(K)
+    assert np.abs(got - want.v).max() <= 3e-4 * np.abs(want.v).max()
 
 
 def test_gemm_linearity_full_size_property():
   """Size-independent check at the benchmark shape: int32 accumulators are linear in the lhs rows
   and match a float64 product on sampled rows."""
-  from qwix_amd import dot_general as dg
+  from qwix_amd.core import dot_general as dg
   g = util.rng(77)
   M = N = K = 4096
   a = torch.from_numpy(g.integers(-127, 128, (M, K), dtype=np.int8)).to(util.DEV)

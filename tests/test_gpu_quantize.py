@@ -12,8 +12,8 @@ QTYPES = ['int8', 'int4', 'float8_e4m3fn']
 
 
 def _check(x_np, x_t, dtype, how_kwargs, layout=None, what=''):
-  import qwix_amd
-  from qwix_amd import qarray
+
+  from qwix_amd.core import qarray
   print('case', what, x_np.shape, dtype, how_kwargs, layout, flush=True)
   qa = qarray.quantize(x_t, qarray.HowToQuantize(**how_kwargs), layout=layout)
   torch.cuda.synchronize()
@@ -67,7 +67,7 @@ def test_weight_columns(shape, tile, layout, dtype, qtype):
   if tile:
     kw['tiled_axes'] = {0: tile}
   qa = _check(x_np, x_t, dtype, kw, layout=layout, what=f'cols {layout}')
-  from qwix_amd.qarray import Int4Tensor
+  from qwix_amd.core.qarray import Int4Tensor
   data = qa.qvalue.data if isinstance(qa.qvalue, Int4Tensor) else qa.qvalue
   if layout == 'reduce_minor':
     assert data.stride(0) == 1, 'reduce-minor layout must be K-contiguous'
@@ -97,7 +97,7 @@ def test_minmax(dtype, qtype):
 
 def test_reference_exact_minmax_vector():
   """qarray_test.py:191-219 on the GPU."""
-  from qwix_amd import qarray
+  from qwix_amd.core import qarray
   a = (np.arange(256) / 255.0).astype(np.float32)
   qa = qarray.quantize(torch.from_numpy(a).to(util.DEV), qarray.HowToQuantize(qtype='int8', calibration_method='minmax'))
   assert qa.zero_point.reshape(()).item() == -128
@@ -117,7 +117,7 @@ def test_2d_tiles_generic():
 
 
 def test_zero_rows_and_reference_convert_vectors():
-  from qwix_amd import qarray
+  from qwix_amd.core import qarray
   x = torch.zeros(4, 256, dtype=torch.bfloat16, device=util.DEV)
   x[1] = 3.0
   qa = qarray.quantize(x, qarray.HowToQuantize(qtype='int8', channelwise_axes=[0]))
@@ -136,7 +136,7 @@ def test_zero_rows_and_reference_convert_vectors():
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
 def test_calibrate_scale_static_pipeline(dtype):
   """calibrate -> compute_scale_zero_point -> quantize_with_scale_zero_point == quantize."""
-  from qwix_amd import qarray
+  from qwix_amd.core import qarray
   for shape, kw in [((32, 512), dict(channelwise_axes=[0])), ((256, 64), dict(channelwise_axes=[1])),
                     ((256, 64), dict(channelwise_axes=[1], tiled_axes={0: 128}))]:
     for cal in ('absmax', 'minmax'):
@@ -155,7 +155,7 @@ def test_calibrate_scale_static_pipeline(dtype):
 @pytest.mark.parametrize('qtype', QTYPES)
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
 def test_dequantize(dtype, qtype):
-  from qwix_amd import qarray
+  from qwix_amd.core import qarray
   for shape, kw, layout in [((32, 512), dict(channelwise_axes=[0]), None), ((256, 64), dict(channelwise_axes=[1], tiled_axes={0: 128}), 'natural'),
                             ((256, 64), dict(channelwise_axes=[1], tiled_axes={0: 128}), 'reduce_minor')]:
     x_np, x_t = util.make(shape, dtype, seed=71)
@@ -167,7 +167,7 @@ def test_dequantize(dtype, qtype):
 
 
 def test_errors_match_reference_behaviour():
-  from qwix_amd import qarray
+  from qwix_amd.core import qarray
   x = torch.zeros(4, 10, device=util.DEV)
   with pytest.raises(ValueError, match='cannot be tiled'):
     qarray.quantize(x, qarray.HowToQuantize(qtype='int8', tiled_axes={1: 4}))

@@ -29,7 +29,7 @@ def farr(t: torch.Tensor) -> O.FArr:
 
 def qvalues_np(qa) -> np.ndarray:
   """Logical quantized values of a qwix_amd QArray: int8 for int8/int4, uint8 bits for e4m3."""
-  from qwix_amd.qarray import Int4Tensor
+  from qwix_amd.core.qarray import Int4Tensor
   q = qa.qvalue
   if isinstance(q, Int4Tensor):
     return q.unpack().cpu().numpy()
