@@ -294,7 +294,6 @@ def _workspace(plan: _Plan, cal: int, device) -> tuple[torch.Tensor | None, int]
 
 def _alloc_q(shape, qtype: str, plan: _Plan, layout: int, device):
   """Allocates the qvalue buffer; returns (flat storage tensor, logical view)."""
-  n = math.prod(shape)
   is4 = qtype == numerics.INT4
   if layout == _lib.LAYOUT_NATURAL or plan.kind != '3d' or plan.dims[2] == 1:
     if is4:
@@ -314,7 +313,6 @@ def _alloc_q(shape, qtype: str, plan: _Plan, layout: int, device):
     return data, Int4Tensor(data.permute(*inv), shape, order[-1])
   data = torch.empty(phys_shape, dtype=numerics.storage_dtype(qtype), device=device)
   return data, data.permute(*inv)
-  del n
 
 
 def _default_layout(plan: _Plan, layout: str | None) -> int:
@@ -393,7 +391,8 @@ def quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = No
   """Dynamic-range quantization: calibrate, derive scale (and zero point), quantize -- one fused pass."""
   if how.noise_fn is not None:
     raise NotImplementedError('stochastic rounding is not part of the HIP path')
-  array = _check_float_input(array)
+  if not isinstance(array, torch.Tensor) or not numerics.should_quantize(array.dtype):
+    raise ValueError(f'Refuse to quantize: {getattr(array, "dtype", type(array))}')
   shape = tuple(array.shape)
   q = numerics.canonical_qtype(how.qtype)
   sshape = get_scale_shape(shape, how)
@@ -401,6 +400,24 @@ def quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = No
   if cal == _lib.MINMAX:
     numerics.get_asymmetric_bound(q)
   plan = _plan(shape, tuple(d // s for d, s in zip(shape, sshape)))
+  if not array.is_contiguous() and plan.kind == '3d' and plan.dims[2] > 1 and layout in (None, 'reduce_minor'):
+    # A strided view whose reduced axes are already the contiguous ones (e.g. a rotated weight kept
+    # K-contiguous): quantize its physical rows and hand back views with the logical shape.
+    order = plan.outer_axes + plan.inner_axes + plan.reduce_axes
+    phys = array.permute(*order)
+    if phys.is_contiguous():
+      nr = len(plan.reduce_axes)
+      phys_how = HowToQuantize(
+          qtype=q, channelwise_axes=tuple(range(phys.ndim - nr)),
+          tiled_axes={phys.ndim - nr: plan.tiles[0] // math.prod(shape[a] for a in plan.reduce_axes[1:])}
+          if plan.tiles[0] != plan.dims[1] else {},
+          calibration_method=how.calibration_method)
+      pq = quantize(phys, phys_how, layout='natural')
+      inv = [order.index(a) for a in range(len(shape))]
+      qv = pq.qvalue.permute(*inv)
+      zp = None if pq.zero_point is None else pq.zero_point.permute(*inv).contiguous()
+      return QArray(qv, pq.scale.permute(*inv).contiguous(), zp, q)
+  array = _check_float_input(array)
   scale = torch.empty(sshape, dtype=array.dtype, device=array.device)
   zp = torch.empty(sshape, dtype=torch.int8, device=array.device) if cal == _lib.MINMAX else None
   tag = _lib.float_tag(array.dtype)

@@ -1,0 +1,302 @@
+// Sub-channel quantized GEMM: int8 activations x int8/int4 weights with one weight scale per
+// group of `group` K-elements (and optionally per-group activation scales).
+//
+//   out[m,n] = cast( sum_g ((T(acc_g[m,n]) * sa[m,g']) * sb[g,n]) ),  acc_g = sum_{k in g} a[m,k] b[n,k]
+//
+// Same tiling as the per-channel kernel (128 x 256 output tile, 2 x 2 wavefronts, 128-byte K slabs
+// through two LDS stages, v_mfma_i32_32x32x32_i8) with two differences:
+//   * int4 weights travel packed through LDS and are widened in registers: every nibble becomes
+//     the HIGH nibble of a byte (value x 16, sign kept), which costs three bit-ops per 8 values;
+//     the activation fragment is byte-permuted to the same K order, and the factor 16 is folded
+//     into the weight scale (exact: a power of two);
+//   * at each group boundary the int32 partial is converted, scaled by sb[g, n] and added to an
+//     f32 accumulator; the int32 accumulator restarts from zero.
+// The lane that owns column n of the MFMA result owns it for all its registers, so one weight scale
+// per 32x32 tile and group is enough.  The result leaves through LDS so that global stores are
+// 16-byte and row-contiguous.
+#include "common.h"
+
+namespace qwix {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 256, BK = 128, TM = 2, TN = 4, kPad = 16;
+
+struct GroupedArgs {
+  const uint8_t* A; int64_t lda;
+  const uint8_t* B; int64_t ldb;
+  int M, N, K, group;
+  const void* sa; int sa_dtype; int ga;
+  const void* sb; int sb_dtype;
+  int t_dtype;      // dtype of the scaled partials (promotion of the scale dtypes)
+  uint8_t* out; int out_dtype; int64_t ldo;
+  int32_t* acc_out;
+};
+
+__device__ __forceinline__ float ld_scale(const void* p, int dtype, int64_t i) {
+  return dtype == QWIX_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i])
+                            : reinterpret_cast<const float*>(p)[i];
+}
+
+template <int BQT, bool EXACT>
+__global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
+  constexpr bool W4 = (BQT == QWIX_INT4);
+  constexpr int A_STRIDE = BK + kPad;
+  constexpr int B_ROW = W4 ? BK / 2 : BK;
+  constexpr int B_STRIDE = B_ROW + kPad;
+  constexpr int STAGE = BM * A_STRIDE + BN * B_STRIDE;
+  constexpr int A_CH = BK / 16, B_CH = B_ROW / 16;
+  constexpr int A_LOADS = BM * A_CH / 256, B_LOADS = BN * B_CH / 256;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_n = (p.N + BN - 1) / BN;
+  int pid = blockIdx.x;
+  if ((gridDim.x & 7) == 0) pid = (pid & 7) * (gridDim.x >> 3) + (pid >> 3);  // one XCD, one run of tiles
+  const int m0 = (pid / tiles_n) * BM, n0 = (pid % tiles_n) * BN;
+
+  v16i acc[TM][TN];
+  float accf[TM][TN][16];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc[i][j][r] = 0;
+        accf[i][j][r] = 0.f;
+      }
+
+  uint4 ra[A_LOADS], rb[B_LOADS];
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int c = tid + i * 256, row = c / A_CH, kc = c % A_CH;
+      const int m = m0 + row, k = k0 + kc * 16;
+      ra[i] = (m < p.M && k < p.K) ? *reinterpret_cast<const uint4*>(p.A + static_cast<int64_t>(m) * p.lda + k)
+                                   : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+      const int c = tid + i * 256, row = c / B_CH, kc = c % B_CH;
+      const int n = n0 + row, k = k0 + kc * (W4 ? 32 : 16);
+      rb[i] = (n < p.N && k < p.K)
+                  ? *reinterpret_cast<const uint4*>(p.B + static_cast<int64_t>(n) * p.ldb + (W4 ? k / 2 : k))
+                  : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store_lds = [&](int s) {
+    uint8_t* base = smem + s * STAGE;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int c = tid + i * 256, row = c / A_CH, kc = c % A_CH;
+      *reinterpret_cast<uint4*>(base + row * A_STRIDE + kc * 16) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+      const int c = tid + i * 256, row = c / B_CH, kc = c % B_CH;
+      *reinterpret_cast<uint4*>(base + BM * A_STRIDE + row * B_STRIDE + kc * 16) = rb[i];
+    }
+  };
+  auto compute = [&](int s) {
+    const uint8_t* pa = smem + s * STAGE + (wm * (BM / 2) + (lane & 31)) * A_STRIDE;
+    const uint8_t* pb = smem + s * STAGE + BM * A_STRIDE + (wn * (BN / 2) + (lane & 31)) * B_STRIDE;
+#pragma unroll
+    for (int ks = 0; ks < BK / 32; ++ks) {
+      v4i fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const v4i t = *reinterpret_cast<const v4i*>(pa + i * 32 * A_STRIDE + ks * 32 + (lane >> 5) * 16);
+        if constexpr (W4) {  // K order (0,2,4,6 | 1,3,5,7 | 8,10,12,14 | 9,11,13,15), as the widened nibbles
+          fa[i][0] = __builtin_amdgcn_perm(t[1], t[0], 0x06040200);
+          fa[i][1] = __builtin_amdgcn_perm(t[1], t[0], 0x07050301);
+          fa[i][2] = __builtin_amdgcn_perm(t[3], t[2], 0x06040200);
+          fa[i][3] = __builtin_amdgcn_perm(t[3], t[2], 0x07050301);
+        } else {
+          fa[i] = t;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        if constexpr (W4) {
+          const uint2 q = *reinterpret_cast<const uint2*>(pb + j * 32 * B_STRIDE + ks * 16 + (lane >> 5) * 8);
+          fb[j][0] = static_cast<int>((q.x << 4) & 0xF0F0F0F0u);
+          fb[j][1] = static_cast<int>(q.x & 0xF0F0F0F0u);
+          fb[j][2] = static_cast<int>((q.y << 4) & 0xF0F0F0F0u);
+          fb[j][3] = static_cast<int>(q.y & 0xF0F0F0F0u);
+        } else {
+          fb[j] = *reinterpret_cast<const v4i*>(pb + j * 32 * B_STRIDE + ks * 32 + (lane >> 5) * 16);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+  };
+
+  // acc[i][j][r]: m = m0 + wm*64 + i*32 + 8*(r/4) + 4*(lane/32) + r%4,  n = n0 + wn*128 + j*32 + lane%32.
+  auto row_of = [&](int i, int r) { return m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); };
+  auto col_of = [&](int j) { return n0 + wn * (BN / 2) + j * 32 + (lane & 31); };
+  constexpr float kUnscale = W4 ? 0.0625f : 1.0f;
+
+  auto flush = [&](int g) {
+    float sbv[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = col_of(j);
+      sbv[j] = n < p.N ? ld_scale(p.sb, p.sb_dtype, static_cast<int64_t>(g) * p.N + n) : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = row_of(i, r);
+        float sav = 1.f;
+        if (p.sa != nullptr && (EXACT || p.ga > 1) && m < p.M)
+          sav = ld_scale(p.sa, p.sa_dtype, static_cast<int64_t>(m) * p.ga + (p.ga > 1 ? g : 0));
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int raw = acc[i][j][r];
+          if (p.acc_out != nullptr && m < p.M && col_of(j) < p.N)
+            p.acc_out[(static_cast<int64_t>(g) * p.M + m) * p.N + col_of(j)] = W4 ? (raw >> 4) : raw;
+          float v = static_cast<float>(raw) * kUnscale;
+          if constexpr (EXACT) {
+            // (T(acc) * sa) * sb with one rounding per step, as the reference computes it.
+            if (p.sa != nullptr) {
+              if (p.sa_dtype == QWIX_BF16) v = round_bf16(round_bf16(v) * sav); else v = v * sav;
+            }
+            const bool tb = (p.t_dtype == QWIX_BF16);
+            if (tb) v = round_bf16(round_bf16(v) * sbv[j]); else v = v * sbv[j];
+            accf[i][j][r] += v;
+          } else {
+            accf[i][j][r] = __builtin_fmaf(v, (p.ga > 1 ? sav : 1.f) * sbv[j], accf[i][j][r]);
+          }
+          acc[i][j][r] = 0;
+        }
+      }
+  };
+
+  const int KT = (p.K + BK - 1) / BK;
+  const int tiles_per_group = p.group / BK;
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < KT) load_global((kt + 1) * BK);
+    compute(cur);
+    if ((kt + 1) % tiles_per_group == 0) flush(kt / tiles_per_group);
+    if (kt + 1 < KT) store_lds(cur ^ 1);
+    __syncthreads();
+  }
+
+  // Epilogue through LDS: each wavefront stages 32 rows x 128 columns of f32 at a time.
+  constexpr int ROW_F = 132;  // floats per staged row (128 + 4 padding)
+  float* stage = reinterpret_cast<float*>(smem) + wave * (32 * ROW_F);
+  const bool t_bf16 = (p.t_dtype == QWIX_BF16);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float v = accf[i][j][r];
+        if (!EXACT && p.sa != nullptr && p.ga == 1) {
+          const int m = row_of(i, r);
+          v *= (m < p.M) ? ld_scale(p.sa, p.sa_dtype, m) : 0.f;
+        }
+        if (t_bf16) v = round_bf16(v);  // the sum over groups is cast back to the partials' dtype
+        stage[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * ROW_F + j * 32 + (lane & 31)] = v;
+      }
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      const int chunk = lane + 64 * c, row = chunk >> 5, cc = chunk & 31;
+      const int m = m0 + wm * (BM / 2) + i * 32 + row, n = n0 + wn * (BN / 2) + cc * 4;
+      if (m >= p.M || n >= p.N) continue;
+      const float4 v = *reinterpret_cast<const float4*>(stage + row * ROW_F + cc * 4);
+      const float vv[4] = {v.x, v.y, v.z, v.w};
+      if (p.out_dtype == QWIX_BF16) {
+        uint16_t* o = reinterpret_cast<uint16_t*>(p.out) + static_cast<int64_t>(m) * p.ldo + n;
+        if (n + 3 < p.N && (p.ldo & 3) == 0) {
+          *reinterpret_cast<uint2*>(o) =
+              make_uint2(f32_to_bf16_bits(vv[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(vv[1])) << 16),
+                         f32_to_bf16_bits(vv[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(vv[3])) << 16));
+        } else {
+          for (int e = 0; e < 4 && n + e < p.N; ++e) o[e] = f32_to_bf16_bits(vv[e]);
+        }
+      } else {
+        float* o = reinterpret_cast<float*>(p.out) + static_cast<int64_t>(m) * p.ldo + n;
+        if (n + 3 < p.N && (p.ldo & 3) == 0) {
+          *reinterpret_cast<float4*>(o) = v;
+        } else {
+          for (int e = 0; e < 4 && n + e < p.N; ++e) o[e] = vv[e];
+        }
+      }
+    }
+  }
+}
+
+template <int BQT, bool EXACT>
+int launch_grouped(const GroupedArgs& p, hipStream_t st) {
+  constexpr bool W4 = (BQT == QWIX_INT4);
+  constexpr size_t stage = BM * (BK + kPad) + BN * ((W4 ? BK / 2 : BK) + kPad);
+  constexpr size_t epi = 4 * 32 * 132 * sizeof(float);
+  constexpr size_t smem = 2 * stage > epi ? 2 * stage : epi;
+  auto kern = qgemm_grouped_kernel<BQT, EXACT>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int64_t tiles = static_cast<int64_t>((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  kern<<<dim3(static_cast<unsigned>(tiles)), 256, smem, st>>>(p);
+  return check_launch("qgemm_grouped");
+}
+
+}  // namespace
+}  // namespace qwix
+
+using namespace qwix;
+
+extern "C" int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b, int64_t ldb_bytes, int b_qtype,
+                                      int64_t M, int64_t N, int64_t K, int64_t group, const void* sa, int sa_dtype,
+                                      int64_t ga, const void* sb, int sb_dtype, void* out, int out_dtype, int64_t ldo,
+                                      int exact, int32_t* acc_out, void* stream) {
+  if (!a || !b || !out || !sb) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/b/out/sb");
+  if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad GEMM shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
+                (long long)K);
+  if (b_qtype != QWIX_INT8 && b_qtype != QWIX_INT4)
+    return fail(QWIX_ERR_UNSUPPORTED, "grouped GEMM takes int8 or int4 weights (got qtype %d)", b_qtype);
+  if (group <= 0 || group % 128 || K % group)
+    return fail(QWIX_ERR_UNSUPPORTED, "group %lld must be a multiple of 128 that divides K=%lld", (long long)group,
+                (long long)K);
+  const int64_t brow = b_qtype == QWIX_INT4 ? K / 2 : K;
+  if (lda % 16 || ldb_bytes % 16 || lda < K || ldb_bytes < brow || !aligned16(a) || !aligned16(b))
+    return fail(QWIX_ERR_UNSUPPORTED, "lda/ldb must be multiples of 16 bytes and a/b 16-byte aligned");
+  if (ga != 1 && ga != K / group) return fail(QWIX_ERR_INVALID_ARGUMENT, "ga must be 1 or K/group, got %lld", (long long)ga);
+  auto ok_s = [](int d) { return d == QWIX_F32 || d == QWIX_BF16; };
+  if ((sa && !ok_s(sa_dtype)) || !ok_s(sb_dtype) || !ok_s(out_dtype))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "scale and output dtypes must be f32 or bf16");
+  if (ldo < N || !aligned16(out)) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad output leading dimension");
+  GroupedArgs p;
+  p.A = static_cast<const uint8_t*>(a); p.lda = lda;
+  p.B = static_cast<const uint8_t*>(b); p.ldb = ldb_bytes;
+  p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(K); p.group = static_cast<int>(group);
+  p.sa = sa; p.sa_dtype = sa_dtype; p.ga = static_cast<int>(ga);
+  p.sb = sb; p.sb_dtype = sb_dtype;
+  p.t_dtype = (sb_dtype == QWIX_F32 || (sa && sa_dtype == QWIX_F32)) ? QWIX_F32 : QWIX_BF16;
+  p.out = static_cast<uint8_t*>(out); p.out_dtype = out_dtype; p.ldo = ldo;
+  p.acc_out = acc_out;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (b_qtype == QWIX_INT4)
+    return exact ? launch_grouped<QWIX_INT4, true>(p, st) : launch_grouped<QWIX_INT4, false>(p, st);
+  return exact ? launch_grouped<QWIX_INT8, true>(p, st) : launch_grouped<QWIX_INT8, false>(p, st);
+}

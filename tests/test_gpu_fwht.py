@@ -1,0 +1,122 @@
+"""GPU parity: Walsh-Hadamard rotation and its fusion with quantization vs the CPU oracle.
+
+The reference computes x @ H as a dense bf16 matmul whose accumulation order is XLA's; the kernel
+uses f32 butterflies.  Hence: exact equality where every partial sum is exactly representable
+(small integers), <= 1 ulp on a tiny fraction otherwise, and bit-exact quantization *given the
+kernel's own rotated values*.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import qwix_oracle as O
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize('n', [2, 8, 64, 256, 1024, 8192, 16384])
+def test_fwht_exact_on_small_integers(n):
+  from qwix_amd.contrib import hadamard_rot as hr
+  g = util.rng(n)
+  x = g.integers(-4, 5, (6, n)).astype(np.float32)
+  p = int(np.log2(n))
+  want = x.astype(np.float64) @ O.hadamard_matrix(p).astype(np.float64)
+  y = hr.fwht(torch.from_numpy(x).to(util.DEV), 1)
+  assert np.array_equal(util.f32np(y), want.astype(np.float32))
+  if n <= 64:  # |sums| <= 256: exact in bf16 too
+    yb = hr.fwht(torch.from_numpy(x).to(torch.bfloat16).to(util.DEV), 1)
+    assert np.array_equal(util.f32np(yb), want.astype(np.float32))
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('n', [64, 512, 8192])
+def test_rotate_inputs_matches_oracle_and_preserves_product(n, dtype):
+  from qwix_amd.contrib import hadamard_rot as hr
+  x_np, x_t = util.make((16, n), dtype, seed=n)
+  w_np, w_t = util.make((n, 24), dtype, seed=n + 1, scale=0.02)
+  gen = torch.Generator().manual_seed(123)
+  xr, wr, _ = hr.hadamard_rotate_inputs(x_t, w_t, gen, row_sign_flip=True, col_sign_flip=True, lhs_reduction_dim=1, rhs_reduction_dim=0)
+  gen = torch.Generator().manual_seed(123)
+  rs = (torch.randint(0, 2, (n,), generator=gen, dtype=torch.int32) * 2 - 1).numpy().astype(np.float64)
+  cs = (torch.randint(0, 2, (n,), generator=gen, dtype=torch.int32) * 2 - 1).numpy().astype(np.float64)
+  oxr, owr = O.hadamard_rotate_inputs(O.FArr(x_np, dtype), O.FArr(w_np, dtype), rs, cs, lhs_reduction_dim=1, rhs_reduction_dim=0)
+  assert tuple(wr.shape) == (n, 24) and wr.stride(0) == 1
+  for got, want in ((util.f32np(xr), oxr.v), (util.f32np(wr), owr.v)):
+    if dtype == O.BF16:
+      ulp = np.abs(want) * 2.0**-7 + 1e-30
+      assert np.all(np.abs(got - want) <= ulp), 'more than one bf16 ulp away'
+      assert np.mean(got != want) < 2e-3
+    else:
+      assert np.allclose(got, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+  prod = util.f32np(xr).astype(np.float64) @ util.f32np(wr).astype(np.float64)
+  ref = x_np.astype(np.float64) @ w_np.astype(np.float64)
+  tol = 1e-4 if dtype == O.F32 else 3e-2
+  assert np.allclose(prod, ref, atol=tol * np.abs(ref).max())
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('qtype,tile', [('int8', None), ('int4', 128), ('float8_e4m3fn', None), ('int8', 64)])
+@pytest.mark.parametrize('n', [256, 8192])
+def test_fused_rotate_quantize_equals_rotate_then_quantize(n, qtype, tile, dtype):
+  from qwix_amd.contrib import hadamard_rot as hr
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make((12, n), dtype, seed=7 * n)
+  signs = torch.from_numpy(util.rng(5).choice([-1.0, 1.0], n).astype(np.float32)).to(util.TORCH_DT[dtype]).to(util.DEV)
+  kw = dict(qtype=qtype, channelwise_axes=[0])
+  if tile:
+    kw['tiled_axes'] = {1: tile}
+  how = qarray.HowToQuantize(**kw)
+  fused = hr.rotate_and_quantize(x_t, 1, how, pre_sign=signs)
+  rot = hr.fwht(x_t, 1, pre_sign=signs)
+  want = O.quantize(util.farr(rot), O.HowToQuantize(**kw))
+  util.assert_qarray_equal(fused, want, f'fused {qtype} {tile}')
+
+
+def test_weight_side_fused_rotation_feeds_the_grouped_gemm():
+  """BASELINE config 5 at reduced shape: rotate both sides, act int8 per token, weight int4 g128."""
+  from qwix_amd.contrib import hadamard_rot as hr
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  M, K, N = 64, 1024, 256
+  x_np, x_t = util.make((M, K), O.BF16, seed=1)
+  g = util.rng(2)
+  out_ch = g.choice(K, 11, replace=False)
+  x_np[:, out_ch] = O.round_to_bf16(x_np[:, out_ch] * 50)
+  x_t = torch.from_numpy(x_np).to(torch.bfloat16).to(util.DEV)
+  w_np, w_t = util.make((K, N), O.BF16, seed=3, scale=0.02)
+  s_np = g.choice([-1.0, 1.0], K).astype(np.float32)
+  s_t = torch.from_numpy(s_np).to(torch.bfloat16).to(util.DEV)
+  xq = hr.rotate_and_quantize(x_t, 1, qarray.HowToQuantize(qtype='int8', channelwise_axes=[0]), pre_sign=s_t)
+  wq = hr.rotate_and_quantize(w_t, 0, qarray.HowToQuantize(qtype='int4', channelwise_axes=[1], tiled_axes={0: 128}),
+                              pre_sign=s_t, out_scale=1.0 / K)
+  assert tuple(wq.shape) == (K, N) and tuple(wq.scale.shape) == (K // 128, N)
+  out = dg.dot_general(xq, wq, (((1,), (0,)), ((), ())))
+  # oracle on the kernel's own rotated values
+  xr = hr.fwht(x_t, 1, pre_sign=s_t)
+  wr = hr.fwht(w_t, 0, pre_sign=s_t, out_scale=1.0 / K)
+  oxq = O.quantize(util.farr(xr), O.HowToQuantize(qtype='int8', channelwise_axes=[0]))
+  owq = O.quantize(util.farr(wr.contiguous()), O.HowToQuantize(qtype='int4', channelwise_axes=[1], tiled_axes={0: 128}))
+  util.assert_qarray_equal(xq, oxq, 'rotated act')
+  util.assert_qarray_equal(wq, owq, 'rotated weight')
+  want, wacc = O.fast_dot_general(oxq, owq, (((1,), (0,)), ((), ())), return_acc=True)
+  got = util.f32np(out)
+  assert np.all(np.abs(got - want.v) <= 1e-2 * np.abs(want.v) + util.partials_envelope(wacc, oxq, owq))
+  exact = dg._fast_dot_general(xq, wq, (((1,), (0,)), ((), ())), exact=True)
+  assert np.array_equal(util.f32np(exact), want.v)
+  # the rotation spreads the outlier channels: quantization error vs the float product stays small
+  ref = x_np.astype(np.float64) @ w_np.astype(np.float64)
+  assert np.abs(got - ref).mean() / np.abs(ref).mean() < 0.15
+
+
+def test_fwht_errors():
+  from qwix_amd.contrib import hadamard_rot as hr
+  with pytest.raises(ValueError, match='power of 2'):
+    hr.hadamard_rotate_inputs(torch.ones(2, 6, device=util.DEV), torch.ones(6, 2, device=util.DEV), None,
+                              row_sign_flip=False, col_sign_flip=False, lhs_reduction_dim=1, rhs_reduction_dim=0)
+  with pytest.raises(ValueError, match='to be the same'):
+    hr.hadamard_rotate_inputs(torch.ones(2, 8, device=util.DEV), torch.ones(4, 2, device=util.DEV), None,
+                              row_sign_flip=False, col_sign_flip=False, lhs_reduction_dim=1, rhs_reduction_dim=0)
+  with pytest.raises(ValueError, match='Key must be provided'):
+    hr.hadamard_rotate_inputs(torch.ones(2, 8, device=util.DEV), torch.ones(8, 2, device=util.DEV), None,
+                              row_sign_flip=True, col_sign_flip=False, lhs_reduction_dim=1, rhs_reduction_dim=0)

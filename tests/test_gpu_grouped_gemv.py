@@ -1,0 +1,109 @@
+"""GPU parity: sub-channel (K-group) GEMM and the weight-only skinny GEMM vs the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import qwix_oracle as O
+from tests import util
+
+pytestmark = pytest.mark.gpu
+DN = (((1,), (0,)), ((), ()))
+
+
+def _pair(M, K, N, dtype, wq_type, group, seed, lhs_tile=None, layout=None):
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make((M, K), dtype, seed=seed)
+  w_np, w_t = util.make((K, N), dtype, seed=seed + 1, scale=0.02)
+  lkw = dict(qtype='int8', channelwise_axes=[0])
+  if lhs_tile:
+    lkw['tiled_axes'] = {1: lhs_tile}
+  rkw = dict(qtype=wq_type, channelwise_axes=[1])
+  if group:
+    rkw['tiled_axes'] = {0: group}
+  xq = qarray.quantize(x_t, qarray.HowToQuantize(**lkw))
+  wq = qarray.quantize(w_t, qarray.HowToQuantize(**rkw), layout=layout)
+  oxq = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(**lkw))
+  owq = O.quantize(O.FArr(w_np, dtype), O.HowToQuantize(**rkw))
+  util.assert_qarray_equal(xq, oxq, 'lhs')
+  util.assert_qarray_equal(wq, owq, 'rhs')
+  return xq, wq, oxq, owq, x_np, w_np
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('M,K,N,group', [(64, 256, 128, 128), (200, 512, 264, 128), (128, 1024, 256, 256), (300, 384, 520, 128)])
+def test_grouped_gemm_exact_mode_is_bit_exact(M, K, N, group, wq_type, dtype):
+  from qwix_amd.core import dot_general as dg
+  print('case grouped', M, K, N, group, wq_type, dtype, flush=True)
+  xq, wq, oxq, owq, _, _ = _pair(M, K, N, dtype, wq_type, group, seed=M + N)
+  out, acc = dg._fast_dot_general(xq, wq, DN, exact=True, return_accumulators=True)
+  torch.cuda.synchronize()
+  want, wacc = O.fast_dot_general(oxq, owq, DN, return_acc=True)
+  assert np.array_equal(acc.cpu().numpy(), wacc), 'per-group int32 partials differ'
+  got = util.f32np(out)
+  bad = np.flatnonzero(got.ravel() != want.v.ravel())
+  assert bad.size == 0, f'{bad.size} outputs differ: {got.ravel()[bad[:5]]} vs {want.v.ravel()[bad[:5]]}'
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+def test_grouped_gemm_fast_mode_within_tolerance(wq_type, dtype):
+  from qwix_amd.core import dot_general as dg
+  xq, wq, oxq, owq, x_np, w_np = _pair(256, 1024, 512, dtype, wq_type, 128, seed=3)
+  out = dg.dot_general(xq, wq, DN)
+  want, wacc = O.fast_dot_general(oxq, owq, DN, return_acc=True)
+  got = util.f32np(out)
+  assert np.all(np.abs(got - want.v) <= 1e-2 * np.abs(want.v) + util.partials_envelope(wacc, oxq, owq)), np.abs(got - want.v).max()
+  ref = x_np.astype(np.float64) @ w_np.astype(np.float64)
+  ceil = 0.12 if wq_type == 'int4' else 0.02   # einsum_test.py ceilings for w4a8 / w8a8
+  assert np.abs(got - ref).mean() / np.abs(ref).mean() < ceil * 1.1
+
+
+def test_both_sides_tiled_and_natural_layout_weight():
+  from qwix_amd.core import dot_general as dg
+  xq, wq, oxq, owq, _, _ = _pair(96, 512, 128, O.F32, 'int8', 128, seed=9, lhs_tile=128, layout='natural')
+  out, acc = dg._fast_dot_general(xq, wq, DN, exact=True, return_accumulators=True)
+  want, wacc = O.fast_dot_general(oxq, owq, DN, return_acc=True)
+  assert np.array_equal(acc.cpu().numpy(), wacc)
+  assert np.array_equal(util.f32np(out), want.v)
+  out = dg.dot_general(xq, wq, DN)
+  assert np.allclose(util.f32np(out), want.v, rtol=1e-4, atol=1e-5)
+
+
+def test_per_channel_int4_weight_and_tile_mismatch_error():
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  xq, wq, oxq, owq, _, _ = _pair(64, 256, 128, O.BF16, 'int4', None, seed=12)
+  out = dg._fast_dot_general(xq, wq, DN, exact=True)
+  want = O.fast_dot_general(oxq, owq, DN)
+  assert np.array_equal(util.f32np(out), want.v)
+  xq2, _, _, _, _, _ = _pair(64, 512, 128, O.BF16, 'int4', 128, seed=12, lhs_tile=256)
+  _, wq2, _, _, _, _ = _pair(64, 512, 128, O.BF16, 'int4', 128, seed=12)
+  with pytest.raises(ValueError, match='same tile size'):
+    dg._fast_dot_general(xq2, wq2, DN)
+
+
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('M', [1, 8, 16, 40])
+@pytest.mark.parametrize('K,N,group,sdt', [(512, 256, 128, torch.float32), (4096, 1024, 128, torch.float32), (1024, 200, 1024, torch.bfloat16)])
+def test_weight_only_gemv(M, K, N, group, sdt, wq_type):
+  """BASELINE config 2 at reduced N: bf16 activations x int4 g128 weight, f32 scales, bf16 out."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  print('case gemv', M, K, N, group, wq_type, flush=True)
+  x_np, x_t = util.make((M, K), O.BF16, seed=M + K)
+  w_np, w_t = util.make((K, N), O.BF16, seed=M + K + 1, scale=0.02)
+  tiled = {0: group} if group != K else {}
+  wq = qarray.quantize_api(w_t, wq_type, channelwise_axes=[1], tiled_axes=tiled, scale_dtype=sdt)
+  owq = O.quantize_api(O.FArr(w_np, O.BF16), wq_type, channelwise_axes=[1], tiled_axes=tiled, scale_dtype=util.ORACLE_DT[sdt])
+  util.assert_qarray_equal(wq, owq, 'weight')
+  out = dg.dot_general(x_t, wq, DN, preferred_element_type=torch.bfloat16)
+  torch.cuda.synchronize()
+  want = O.dot_general(O.FArr(x_np, O.BF16), owq, DN, O.BF16)
+  assert out.dtype == torch.bfloat16 and tuple(out.shape) == (M, N)
+  got = util.f32np(out)
+  scale = np.abs(want.v).mean()
+  assert np.allclose(got, want.v, rtol=1e-2, atol=1e-2 * scale), np.abs(got - want.v).max()
+  # default result type follows the scale dtype (bf16 x f32 -> f32)
+  out2 = dg.dot_general(x_t, wq, DN)
+  assert out2.dtype == sdt

@@ -60,3 +60,17 @@ def assert_qarray_equal(qa, want: O.QArray, what=''):
     assert np.array_equal(qa.zero_point.cpu().numpy(), want.zero_point), f'{what}: zero points differ'
   else:
     assert qa.zero_point is None
+
+
+def partials_envelope(acc, oxq, owq) -> np.ndarray:
+  """Rounding envelope of the reference's own sub-channel epilogue.
+
+  With bf16 scales the reference rounds every per-group partial three times (convert, * sx, * sy)
+  before summing, so two faithful evaluations may differ by up to 3 * 2^-9 * sum_g |partial_g|.
+  acc: (G, M, N) int32 partials.  Returns 2^-7 * sum_g |acc_g| * sx * sy_g (f32 scales: 2^-20).
+  """
+  sx = oxq.scale.v.reshape(oxq.scale.v.shape[0], -1)[:, :1]          # (M, 1)
+  sy = owq.scale.v                                                    # (G, N)
+  mag = (np.abs(acc).astype(np.float64) * sx[None] * sy[:, None, :]).sum(0)
+  eps = 2.0**-7 if O.BF16 in (oxq.scale.dtype, owq.scale.dtype) and O.F32 not in (oxq.scale.dtype, owq.scale.dtype) else 2.0**-20
+  return (eps * mag).astype(np.float32)
