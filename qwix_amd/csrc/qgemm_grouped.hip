@@ -3,7 +3,7 @@
 //
 //   out[m,n] = cast( sum_g ((T(acc_g[m,n]) * sa[m,g']) * sb[g,n]) ),  acc_g = sum_{k in g} a[m,k] b[n,k]
 //
-// Same tiling as the per-channel kernel (128 x 256 output tile, 2 x 2 wavefronts, 128-byte K slabs
+// Same tiling as the per-channel kernel (128 x 128 output tile, 2 x 2 wavefronts, 128-byte K slabs
 // through two LDS stages, v_mfma_i32_32x32x32_i8) with two differences:
 //   * int4 weights travel packed through LDS and are widened in registers: every nibble becomes
 //     the HIGH nibble of a byte (value x 16, sign kept), which costs three bit-ops per 8 values;
@@ -22,7 +22,7 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128, BN = 256, BK = 128, TM = 2, TN = 4, kPad = 16;
+constexpr int BM = 128, BN = 128, BK = 128, TM = 2, TN = 2, kPad = 16;
 
 struct GroupedArgs {
   const uint8_t* A; int64_t lda;
@@ -139,7 +139,7 @@ __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
     }
   };
 
-  // acc[i][j][r]: m = m0 + wm*64 + i*32 + 8*(r/4) + 4*(lane/32) + r%4,  n = n0 + wn*128 + j*32 + lane%32.
+  // acc[i][j][r]: m = m0 + wm*64 + i*32 + 8*(r/4) + 4*(lane/32) + r%4,  n = n0 + wn*(BN/2) + j*32 + lane%32.
   auto row_of = [&](int i, int r) { return m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); };
   auto col_of = [&](int j) { return n0 + wn * (BN / 2) + j * 32 + (lane & 31); };
   constexpr float kUnscale = W4 ? 0.0625f : 1.0f;
@@ -195,8 +195,10 @@ __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
     __syncthreads();
   }
 
-  // Epilogue through LDS: each wavefront stages 32 rows x 128 columns of f32 at a time.
-  constexpr int ROW_F = 132;  // floats per staged row (128 + 4 padding)
+  // Epilogue through LDS: each wavefront stages 32 rows x (BN/2) columns of f32 at a time.
+  constexpr int WCOLS = BN / 2;
+  constexpr int ROW_F = WCOLS + 4;  // floats per staged row (+ 4 padding)
+  constexpr int CPR = WCOLS / 4;    // 16-byte chunks per staged row
   float* stage = reinterpret_cast<float*>(smem) + wave * (32 * ROW_F);
   const bool t_bf16 = (p.t_dtype == QWIX_BF16);
 #pragma unroll
@@ -214,8 +216,8 @@ __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
         stage[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * ROW_F + j * 32 + (lane & 31)] = v;
       }
 #pragma unroll
-    for (int c = 0; c < 16; ++c) {
-      const int chunk = lane + 64 * c, row = chunk >> 5, cc = chunk & 31;
+    for (int c = 0; c < 32 * CPR / 64; ++c) {
+      const int chunk = lane + 64 * c, row = chunk / CPR, cc = chunk % CPR;
       const int m = m0 + wm * (BM / 2) + i * 32 + row, n = n0 + wn * (BN / 2) + cc * 4;
       if (m >= p.M || n >= p.N) continue;
       const float4 v = *reinterpret_cast<const float4*>(stage + row * ROW_F + cc * 4);
@@ -227,14 +229,16 @@ __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
               make_uint2(f32_to_bf16_bits(vv[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(vv[1])) << 16),
                          f32_to_bf16_bits(vv[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(vv[3])) << 16));
         } else {
-          for (int e = 0; e < 4 && n + e < p.N; ++e) o[e] = f32_to_bf16_bits(vv[e]);
+          _Pragma("unroll") for (int e = 0; e < 4; ++e)
+            if (n + e < p.N) o[e] = f32_to_bf16_bits(vv[e]);
         }
       } else {
         float* o = reinterpret_cast<float*>(p.out) + static_cast<int64_t>(m) * p.ldo + n;
         if (n + 3 < p.N && (p.ldo & 3) == 0) {
           *reinterpret_cast<float4*>(o) = v;
         } else {
-          for (int e = 0; e < 4 && n + e < p.N; ++e) o[e] = vv[e];
+          _Pragma("unroll") for (int e = 0; e < 4; ++e)
+            if (n + e < p.N) o[e] = vv[e];
         }
       }
     }
@@ -245,7 +249,7 @@ template <int BQT, bool EXACT>
 int launch_grouped(const GroupedArgs& p, hipStream_t st) {
   constexpr bool W4 = (BQT == QWIX_INT4);
   constexpr size_t stage = BM * (BK + kPad) + BN * ((W4 ? BK / 2 : BK) + kPad);
-  constexpr size_t epi = 4 * 32 * 132 * sizeof(float);
+  constexpr size_t epi = 4 * 32 * (BN / 2 + 4) * sizeof(float);
   constexpr size_t smem = 2 * stage > epi ? 2 * stage : epi;
   auto kern = qgemm_grouped_kernel<BQT, EXACT>;
   static bool configured = false;
