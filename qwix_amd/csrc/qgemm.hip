@@ -10,6 +10,7 @@
 // 4 consecutive n for a single m: output rows are written with 8/16-byte vector stores.
 // Workgroup ids are remapped so that the 8 XCDs (round-robin dispatch) each work on a compact
 // block of tiles and share their slabs through their own L2.
+#include <cstdlib>
 #include <type_traits>
 
 #include "common.h"
@@ -23,6 +24,24 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kPad = 16;
+
+// Optional in-kernel timing (development builds only: -DQWIX_GEMM_DEBUG).  Each wavefront records
+// s_memtime stamps / accumulated intervals into a device array that a test harness copies out.
+#ifdef QWIX_GEMM_DEBUG
+__device__ unsigned long long qwix_dbg[4096 * 8];
+#define QWIX_DBG_NOW() ([] { __builtin_amdgcn_sched_barrier(0); unsigned long long t_ = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0); return t_; }())
+#define QWIX_DBG_DECL unsigned long long dbg_t[8] = {0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long dbg_last = 0;
+#define QWIX_DBG_STAMP(i) dbg_t[i] = QWIX_DBG_NOW();
+#define QWIX_DBG_BEGIN() dbg_last = QWIX_DBG_NOW();
+#define QWIX_DBG_ACC(i) { unsigned long long n_ = QWIX_DBG_NOW(); dbg_t[i] += n_ - dbg_last; dbg_last = n_; }
+#define QWIX_DBG_FLUSH() if ((threadIdx.x & 63) == 0 && blockIdx.x < 512) { for (int i_ = 0; i_ < 8; ++i_) qwix_dbg[(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + i_] = dbg_t[i_]; }
+#else
+#define QWIX_DBG_DECL
+#define QWIX_DBG_STAMP(i)
+#define QWIX_DBG_BEGIN()
+#define QWIX_DBG_ACC(i)
+#define QWIX_DBG_FLUSH()
+#endif
 
 // Epilogue description.  The reference scales the accumulator as ((T(acc) * sa) * sb) with one
 // rounding per step in the promoted dtype; which of those roundings are to bf16 is decided on the
@@ -55,16 +74,52 @@ __device__ __forceinline__ float load_scale(const void* p, int dtype, int64_t i)
 }
 
 // acc[i][j][r]: m = m_base + i*32 + lane%32,  n = n_base + j*32 + 8*(r/4) + 4*(lane/32) + r%4.
+// All scales a lane needs are fetched before its first store, so that the stores (which the
+// compiler must keep ordered with loads that may alias) do not serialise the global-load latency.
 template <int OUT, int TM, int TN, typename AccT>
 __device__ __forceinline__ void write_tile(const AccT (&acc)[TM][TN], const Epilogue& ep, int m_base, int n_base,
                                            int lane, int M, int N, uint8_t* __restrict__ out, int64_t ldo) {
   const bool vec_ok = (N % 4 == 0);
   const bool r0 = ep.r0 != 0, r1 = ep.r1 != 0, r2 = ep.r2 != 0;
+  float sav[TM];
+  float sbv[TN][4][4];
+  if constexpr (OUT != QWIX_I32) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int m = m_base + i * 32 + (lane & 31);
+      sav[i] = (ep.sa != nullptr && m < M) ? load_scale(ep.sa, ep.sa_dtype, m) : 1.f;
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int n = n_base + j * 32 + 8 * qd + 4 * (lane >> 5);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sbv[j][qd][r] = 1.f;
+        if (ep.sb != nullptr) {
+          if (vec_ok && n < N) {  // n % 4 == 0: one 8- or 16-byte load
+            if (ep.sb_dtype == QWIX_BF16) {
+              const uint2 w = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(ep.sb) + n);
+              sbv[j][qd][0] = __uint_as_float(w.x << 16);
+              sbv[j][qd][1] = __uint_as_float(w.x & 0xFFFF0000u);
+              sbv[j][qd][2] = __uint_as_float(w.y << 16);
+              sbv[j][qd][3] = __uint_as_float(w.y & 0xFFFF0000u);
+            } else {
+              const float4 w = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(ep.sb) + n);
+              sbv[j][qd][0] = w.x; sbv[j][qd][1] = w.y; sbv[j][qd][2] = w.z; sbv[j][qd][3] = w.w;
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (n + r < N) sbv[j][qd][r] = load_scale(ep.sb, ep.sb_dtype, n + r);
+          }
+        }
+      }
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int m = m_base + i * 32 + (lane & 31);
     const bool m_ok = m < M;
-    const float sa = (ep.sa != nullptr && m_ok) ? load_scale(ep.sa, ep.sa_dtype, m) : 1.f;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
 #pragma unroll
@@ -85,12 +140,11 @@ __device__ __forceinline__ void write_tile(const AccT (&acc)[TM][TN], const Epil
             float v[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const float sb = (ep.sb != nullptr && n + r < N) ? load_scale(ep.sb, ep.sb_dtype, n + r) : 1.f;
               float t = static_cast<float>(acc[i][j][4 * qd + r]);
               t = r0 ? round_bf16(t) : t;
-              t *= sa;
+              t *= sav[i];
               t = r1 ? round_bf16(t) : t;
-              t *= sb;
+              t *= sbv[j][qd][r];
               v[r] = r2 ? round_bf16(t) : t;
             }
             if constexpr (OUT == QWIX_BF16) {
@@ -228,24 +282,33 @@ __global__ void __launch_bounds__(256)
   };
 
   const int KT = (K + BK - 1) / BK;
+  QWIX_DBG_DECL
+  QWIX_DBG_STAMP(0)
   load_global(0);
   store_lds(0);
   __syncthreads();
   read_frags(0, 0, 0);
+  QWIX_DBG_STAMP(1)
   for (int kt = 0; kt < KT; ++kt) {
     const int cur = kt & 1;
     const bool has_next = kt + 1 < KT;
+    QWIX_DBG_BEGIN()
     if (has_next) load_global((kt + 1) * BK);
 #pragma unroll
     for (int ks = 0; ks + 1 < NK; ++ks) {
       read_frags(cur, ks + 1, (ks + 1) & 1);
       mfma_step(ks & 1);
     }
+    QWIX_DBG_ACC(4)
     if (has_next) store_lds(cur ^ 1);
+    QWIX_DBG_ACC(5)
     __syncthreads();
+    QWIX_DBG_ACC(6)
     if (has_next) read_frags(cur ^ 1, 0, 0);
     mfma_step((NK - 1) & 1);
+    QWIX_DBG_ACC(7)
   }
+  QWIX_DBG_STAMP(2)
 
   const int m_base = m0 + wm * (BM / 2), n_base = n0 + wn * (BN / 2);
   if (ep.out_dtype == QWIX_BF16) {
@@ -255,6 +318,314 @@ __global__ void __launch_bounds__(256)
   } else {
     if constexpr (IS_INT) write_tile<QWIX_I32, TM, TN>(acc, ep, m_base, n_base, lane, M, N, out, ldo);
   }
+  QWIX_DBG_STAMP(3)
+  QWIX_DBG_FLUSH()
+}
+
+// Fast path (K % 128 == 0): the slabs go from global memory straight into LDS
+// (global_load_lds_dwordx4: no staging registers, no ds_write instructions).  Each wave-level load
+// fills one contiguous KiB of LDS = 8 tile rows x 128 bytes; inside a row the eight 16-byte k-chunks
+// are stored at position (chunk ^ (row & 7)), chosen by having each lane fetch the matching global
+// chunk, so that the fragment reads of 8 consecutive rows hit all 32 banks.  Rows past M / N are
+// clamped to the last valid row (their results are never stored).  Loads for slab kt+1 are issued
+// while the MFMAs of slab kt run; the workgroup barrier at the end of the slab waits for them.
+// The workgroup is WGM x WGN wavefronts; with 8 wavefronts (two per SIMD) the issue time of one
+// wavefront's loads and fragment reads hides behind the other's MFMAs.
+// EPI: 0 = no bf16 rounding in the epilogue, 1 = every step rounds to bf16, 2 = flags at run time.
+#define QWIX_GLDS16(gptr, lptr)                                                                       \
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),             \
+                                   (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
+
+template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI>
+__global__ void __launch_bounds__(WGM * WGN * 64)
+    qgemm_dma_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
+                     int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  constexpr bool IS_INT = (QT == QWIX_INT8);
+  constexpr int BK = 128;
+  constexpr int NWAVES = WGM * WGN;
+  constexpr int WTM = BM / WGM, WTN = BN / WGN;   // wave tile
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int KSTEP = IS_INT ? 32 : 64;
+  constexpr int NK = BK / KSTEP;
+  constexpr int ROWS = BM + BN;
+  constexpr int STAGE = ROWS * BK;
+  constexpr int LOADS = ROWS / 8 / NWAVES;  // 1 KiB loads per wavefront per slab
+  static_assert(ROWS % (8 * NWAVES) == 0 && (BM / 8) % LOADS == 0, "each wavefront loads from one operand");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+  int tile_m, tile_n;
+  tile_coords((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  using AccT = typename std::conditional<IS_INT, v16i, v16f>::type;
+  using FragT = typename std::conditional<IS_INT, v4i, v8i>::type;
+  AccT acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  // ---- loader: a wave-uniform base pointer plus this lane's 32-bit offset for each row group
+  const int lr = lane >> 3;                       // row inside the 8-row group
+  const int lc = (lane & 7) ^ lr;                 // global k-chunk that lands at LDS chunk position lane&7
+  const bool from_a = (wave * LOADS * 8) < BM;    // wave-uniform
+  const uint8_t* gbase = from_a ? A : B;
+  const int64_t gld = from_a ? lda : ldb;
+  const int glim = from_a ? (M - 1) : (N - 1);
+  const int grow0 = from_a ? (m0 + wave * LOADS * 8) : (n0 + wave * LOADS * 8 - BM);
+  uint32_t goff[LOADS];
+#pragma unroll
+  for (int j = 0; j < LOADS; ++j)
+    goff[j] = static_cast<uint32_t>(min(grow0 + j * 8 + lr, glim)) * static_cast<uint32_t>(gld) + lc * 16;
+  auto issue_loads = [&](int s, int k0) {
+    const uint8_t* gk = gbase + k0;
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) QWIX_GLDS16(gk + goff[j], smem + s * STAGE + (wave * LOADS + j) * 1024);
+  };
+
+  // ---- fragment addresses: row r, k-chunk c lives at r*128 + ((c ^ (r & 7)) << 4); r & 7 == lane & 7
+  const int a_row = (wm * WTM + (lane & 31)) * BK;
+  const int b_row = (BM + wn * WTN + (lane & 31)) * BK;
+  const int hx = lane >> 5, x7 = lane & 7;
+  FragT fa[2][TM], fb[2][TN];
+  auto read_frags = [&](int s, int ks, int buf) {
+    const uint8_t* base = smem + s * STAGE;
+    if constexpr (IS_INT) {
+      const int off = ((ks * 2 + hx) ^ x7) << 4;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const v4i*>(base + a_row + i * 32 * BK + off);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const v4i*>(base + b_row + j * 32 * BK + off);
+    } else {
+      const int off = ((ks * 4 + hx * 2) ^ x7) << 4;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const v4i lo = *reinterpret_cast<const v4i*>(base + a_row + i * 32 * BK + off);
+        const v4i hi = *reinterpret_cast<const v4i*>(base + a_row + i * 32 * BK + (off ^ 16));
+        fa[buf][i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const v4i lo = *reinterpret_cast<const v4i*>(base + b_row + j * 32 * BK + off);
+        const v4i hi = *reinterpret_cast<const v4i*>(base + b_row + j * 32 * BK + (off ^ 16));
+        fb[buf][j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+    }
+  };
+  auto mfma_step = [&](int buf) {
+#ifdef QWIX_DBG_SKIP_MFMA
+    for (int i = 0; i < TM; ++i)
+      for (int j = 0; j < TN; ++j) acc[i][j][0] += fb[buf][j][0] + fa[buf][i][0];
+    return;
+#endif
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        if constexpr (IS_INT)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+        else
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0, 0, 0, 0);
+      }
+  };
+  // Interleave hints for one k-step: MFMAs in pairs, a fragment read after each pair, and a slab load
+  // after each pair while loads remain.
+  auto hint_kstep = [&](int n_loads) {
+    constexpr int MF = TM * TN, RD = (IS_INT ? 1 : 2) * (TM + TN);
+#pragma unroll
+    for (int g = 0; g < MF; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // MFMA
+      if (g < RD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);           // DS read
+      if (g < n_loads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);      // VMEM read (LDS DMA)
+    }
+  };
+
+  const int KT = K / BK;
+  QWIX_DBG_DECL
+  QWIX_DBG_STAMP(0)
+  issue_loads(0, 0);
+  __syncthreads();
+  read_frags(0, 0, 0);
+  QWIX_DBG_STAMP(1)
+  // All loads of a slab are issued during its first k-step, giving them the rest of the slab to land.
+  for (int kt = 0; kt < KT - 1; ++kt) {
+    const int cur = kt & 1;
+    QWIX_DBG_BEGIN()
+#ifndef QWIX_DBG_SKIP_LOADS
+    issue_loads(cur ^ 1, (kt + 1) * BK);
+#endif
+#pragma unroll
+    for (int ks = 0; ks + 1 < NK; ++ks) {
+      read_frags(cur, ks + 1, (ks + 1) & 1);
+      mfma_step(ks & 1);
+      hint_kstep(ks == 0 ? LOADS : 0);
+    }
+    QWIX_DBG_ACC(4)
+    mfma_step((NK - 1) & 1);
+    QWIX_DBG_ACC(5)
+    __syncthreads();
+    QWIX_DBG_ACC(6)
+    read_frags(cur ^ 1, 0, 0);
+    QWIX_DBG_ACC(7)
+  }
+  {  // last slab: nothing left to fetch
+    const int cur = (KT - 1) & 1;
+#pragma unroll
+    for (int ks = 0; ks + 1 < NK; ++ks) {
+      read_frags(cur, ks + 1, (ks + 1) & 1);
+      mfma_step(ks & 1);
+    }
+    mfma_step((NK - 1) & 1);
+  }
+  QWIX_DBG_STAMP(2)
+
+  // ---- epilogue.  acc[i][j][r]: m = m_base + i*32 + lane%32, n = n_base + j*32 + 8*(r/4) + 4*(lane/32) + r%4.
+  // The scaled values are staged through this wavefront's own slice of LDS, 32 rows at a time, and
+  // leave with 16-byte stores that cover whole 128-byte row segments (a direct store from the MFMA
+  // layout would write 16-byte pieces of 32 different rows per instruction).
+  using OutT = typename std::conditional<OUT == QWIX_BF16, uint16_t, uint32_t>::type;
+  constexpr int ES = sizeof(OutT);
+  constexpr int ROWB = WTN * ES + 16;            // staged row pitch in bytes (padded against bank conflicts)
+  constexpr int CPR = WTN * ES / 16;             // 16-byte chunks per staged row
+  constexpr int EPC = 16 / ES;                   // elements per chunk
+  static_assert(NWAVES * 32 * ROWB <= 2 * STAGE, "epilogue staging does not fit in LDS");
+  const int m_base = m0 + wm * WTM, n_base = n0 + wn * WTN;
+  float sbv[TN][4][4];
+  float sav[TM];  // fetched up front: a load inside the store loop would wait for the stores before it
+  if constexpr (OUT != QWIX_I32) {
+    const bool vec_ok = (N % 4 == 0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int m = m_base + i * 32 + (lane & 31);
+      sav[i] = (ep.sa != nullptr && m < M) ? load_scale(ep.sa, ep.sa_dtype, m) : 1.f;
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int n = n_base + j * 32 + 8 * qd + 4 * (lane >> 5);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sbv[j][qd][r] = 1.f;
+        if (ep.sb != nullptr) {
+          if (vec_ok && n < N) {  // n % 4 == 0: one 8- or 16-byte load
+            if (ep.sb_dtype == QWIX_BF16) {
+              const uint2 w = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(ep.sb) + n);
+              sbv[j][qd][0] = __uint_as_float(w.x << 16);
+              sbv[j][qd][1] = __uint_as_float(w.x & 0xFFFF0000u);
+              sbv[j][qd][2] = __uint_as_float(w.y << 16);
+              sbv[j][qd][3] = __uint_as_float(w.y & 0xFFFF0000u);
+            } else {
+              const float4 w = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(ep.sb) + n);
+              sbv[j][qd][0] = w.x; sbv[j][qd][1] = w.y; sbv[j][qd][2] = w.z; sbv[j][qd][3] = w.w;
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (n + r < N) sbv[j][qd][r] = load_scale(ep.sb, ep.sb_dtype, n + r);
+          }
+        }
+      }
+  }
+  const bool r0 = EPI == 2 ? ep.r0 != 0 : EPI == 1, r1 = EPI == 2 ? ep.r1 != 0 : EPI == 1,
+             r2 = EPI == 2 ? ep.r2 != 0 : EPI == 1;
+  __syncthreads();  // every wavefront is done with the slabs; LDS becomes staging space
+  uint8_t* stg = smem + wave * (32 * ROWB);
+  const bool row_vec = (reinterpret_cast<uintptr_t>(out) % 16 == 0) && ((ldo * ES) % 16 == 0);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    float sa = 1.f;
+    if constexpr (OUT != QWIX_I32) sa = sav[i];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        uint8_t* dst = stg + (lane & 31) * ROWB + (j * 32 + 8 * qd + 4 * (lane >> 5)) * ES;
+        if constexpr (OUT == QWIX_I32) {
+          *reinterpret_cast<int4*>(dst) = make_int4(static_cast<int>(acc[i][j][4 * qd]), static_cast<int>(acc[i][j][4 * qd + 1]),
+                                                    static_cast<int>(acc[i][j][4 * qd + 2]), static_cast<int>(acc[i][j][4 * qd + 3]));
+        } else {
+          float v[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float t = static_cast<float>(acc[i][j][4 * qd + r]);
+            if (r0) t = round_bf16(t);
+            t *= sa;
+            if (r1) t = round_bf16(t);
+            t *= sbv[j][qd][r];
+            if (r2) t = round_bf16(t);
+            v[r] = t;
+          }
+          if constexpr (OUT == QWIX_BF16)
+            *reinterpret_cast<uint2*>(dst) =
+                make_uint2(f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16),
+                           f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16));
+          else
+            *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+      }
+    // read back row-major: chunk c of the 32 x CPR grid -> row c / CPR, 16-byte column c % CPR
+#pragma unroll
+    for (int c0 = 0; c0 < 32 * CPR; c0 += 64) {
+      const int c = c0 + lane, row = c / CPR, cc = c % CPR;
+      const uint4 v = *reinterpret_cast<const uint4*>(stg + row * ROWB + cc * 16);
+      const int mo = m_base + i * 32 + row, no = n_base + cc * EPC;
+      if (mo < M && no < N) {
+        OutT* o = reinterpret_cast<OutT*>(out) + static_cast<int64_t>(mo) * ldo + no;
+        if (row_vec && no + EPC <= N) {
+          *reinterpret_cast<uint4*>(o) = v;
+        } else {
+          const OutT* e = reinterpret_cast<const OutT*>(&v);
+#pragma unroll
+          for (int t = 0; t < EPC; ++t)
+            if (no + t < N) o[t] = e[t];
+        }
+      }
+    }
+  }
+  QWIX_DBG_STAMP(3)
+  QWIX_DBG_FLUSH()
+}
+
+template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI>
+int launch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
+               const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  constexpr size_t smem = 2 * (BM + BN) * 128;
+  auto kern = qgemm_dma_kernel<QT, BM, BN, WGM, WGN, OUT, EPI>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  kern<<<dim3(static_cast<unsigned>(tiles)), WGM * WGN * 64, smem, st>>>(
+      static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),
+      static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);
+  return check_launch("qgemm (dma)");
+}
+
+// Picks the epilogue specialisation: (bf16 out, all-bf16 rounding), (f32 out, no rounding), raw int32,
+// or the run-time-flag version for mixed scale dtypes.
+template <int QT, int BM, int BN, int WGM, int WGN>
+int dispatch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                 const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  const bool all = ep.r0 && ep.r1 && ep.r2, none = !ep.r0 && !ep.r1 && !ep.r2;
+  if (ep.out_dtype == QWIX_I32) {
+    if constexpr (QT == QWIX_INT8) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_I32, 0>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "int32 output needs int8 operands");
+  }
+  if (ep.out_dtype == QWIX_BF16) {
+    if (all) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_BF16, 1>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    return launch_dma<QT, BM, BN, WGM, WGN, QWIX_BF16, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+  }
+  if (none) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_F32, 0>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+  return launch_dma<QT, BM, BN, WGM, WGN, QWIX_F32, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
 }
 
 template <int QT, int BM, int BN, int BK>
@@ -281,6 +652,12 @@ int launch_qgemm(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t
 }  // namespace qwix
 
 using namespace qwix;
+
+#ifdef QWIX_GEMM_DEBUG
+extern "C" __attribute__((visibility("default"))) int qwix_dbg_read(unsigned long long* host, size_t n) {
+  return hipMemcpyFromSymbol(host, HIP_SYMBOL(qwix_dbg), n * sizeof(unsigned long long)) == hipSuccess ? 0 : 1;
+}
+#endif
 
 extern "C" int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M,
                               int64_t N, int64_t K, const void* sa, int sa_dtype, const void* sb, int sb_dtype,
@@ -319,6 +696,18 @@ extern "C" int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t
   step(sb, sb_dtype, &ep.r2);
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool big = (M >= 1024 && N >= 1024);
+  static const int variant = [] { const char* e = getenv("QWIX_GEMM_VARIANT"); return e ? atoi(e) : 1; }();
+  const bool off32 = M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);  // 32-bit lane offsets
+  if (K % 128 == 0 && off32 && variant != 0) {  // direct-to-LDS pipeline
+    if (qtype == QWIX_INT8) {
+      if (big) return variant == 2 ? dispatch_dma<QWIX_INT8, 256, 256, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st)
+                                   : dispatch_dma<QWIX_INT8, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      return dispatch_dma<QWIX_INT8, 128, 128, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    }
+    if (big) return variant == 2 ? dispatch_dma<QWIX_E4M3, 256, 256, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st)
+                                 : dispatch_dma<QWIX_E4M3, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    return dispatch_dma<QWIX_E4M3, 128, 128, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+  }
   if (qtype == QWIX_INT8) {
     if (big) return launch_qgemm<QWIX_INT8, 256, 256, 128>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     return launch_qgemm<QWIX_INT8, 128, 128, 128>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
