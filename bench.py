@@ -1,0 +1,409 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantize + quantized-dot hot path on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu-baseline]
+
+A "step" is one pass of the hot path over one batch of synthetic input that is already resident
+in HBM.  The default workload is the dynamic-range w8a8 int8 prefill GEMM at 4096^3 (the shape the
+metric "int8 qdot TOPS + % MFMA peak" is quoted on): per step the bf16 activations are quantized
+per token to int8 on the fly and multiplied with the pre-quantized int8 weight on the matrix
+cores, with the per-token x per-channel scale epilogue fused, bf16 out.  All launches go through
+the C ABI of libqwix_hip.so with preallocated buffers.
+
+Prints ONE JSON line.  `roofline` describes the dominant kernel (the MFMA GEMM): achieved =
+2*M*N*K / mean kernel time, measured with events on the launch stream inside the timed region.
+`cpu_baseline` times the NumPy oracle of the same step on a bounded sample on the host cores; it is
+a reported baseline, not a target.  `extra` carries the other workloads of the metric (quantize
+GB/s, fp8 GEMM, weight-only GEMV, Hadamard-rotated GEMM), each with its own roofline fraction.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_MFMA_TOPS = 5000.0   # MI355X dense int8 / fp8 matrix peak, TOP/s (TFLOP/s for fp8)
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak, GB/s
+
+
+def _events(n):
+  import torch
+  return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+class Workload:
+  """setup() allocates everything; step(rec) enqueues one step and may record (start, end) event pairs
+  of the dominant kernel through rec(); describe() gives the static numbers."""
+
+  name = ''
+  dtype = ''
+  metric = ''
+  unit = ''
+  bound = 'mfma'
+
+  def setup(self, dev): ...
+  def step(self, rec=None): ...
+  def work_per_step(self) -> float: ...      # ops (mfma) or bytes (hbm) of the whole step's headline figure
+  def kernel_work(self) -> float: ...        # algorithmic ops / bytes of ONE launch of the dominant kernel
+
+
+def _lib():
+  from qwix_amd import _lib as L
+  L.load()
+  return L
+
+
+class QdotW8A8(Workload):
+  """activation quantize (per token) + MFMA GEMM with fused scale epilogue; qtype int8 or e4m3."""
+
+  bound = 'mfma'
+
+  def __init__(self, name, M, K, N, qtype):
+    self.name, self.M, self.K, self.N, self.qtype = name, M, K, N, qtype
+    self.dtype = 'int8' if qtype == 'int8' else 'f8e4m3'
+    self.metric = ('int8' if qtype == 'int8' else 'fp8') + ' qdot TOPS (dynamic-range w8a8, activation quantize included)'
+    self.unit = 'TOPS'
+    self.kernel = 'qgemm_dma_kernel'
+
+  def setup(self, dev):
+    import torch
+    from qwix_amd.core import qarray
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(3000 + self.M)
+    self.x = torch.randn(self.M, self.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    w = (torch.randn(self.K, self.N, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(dev)
+    # PTQ: the weight is quantized once, per output channel, into the K-contiguous layout.
+    wq = qarray.quantize(w, qarray.HowToQuantize(qtype=self.qtype, channelwise_axes=[1]))
+    del w
+    self.wq = wq
+    self.b = wq.qvalue.permute(1, 0)          # (N, K) contiguous
+    assert self.b.is_contiguous()
+    self.sb = wq.scale.reshape(-1).contiguous()
+    self.xq = torch.empty(self.M, self.K, dtype=wq.qvalue.dtype, device=dev)
+    self.sa = torch.empty(self.M, dtype=torch.bfloat16, device=dev)
+    self.out = torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev)
+    self.qt = L.INT8 if self.qtype == 'int8' else L.E4M3
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, rec=None):
+    L = self.L
+    L.call('qwix_hip_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, 1, self.K, self.qt, L.ABSMAX, 0.0,
+           L.LAYOUT_NATURAL, self.xq.data_ptr(), self.sa.data_ptr(), None, None, 0, self.stream)
+    if rec:
+      rec(0)
+    L.call('qwix_hip_qgemm', self.xq.data_ptr(), self.K, self.b.data_ptr(), self.K, self.qt, self.M, self.N, self.K,
+           self.sa.data_ptr(), L.BF16, self.sb.data_ptr(), L.BF16, L.BF16, self.out.data_ptr(), L.BF16, self.N,
+           self.stream)
+    if rec:
+      rec(1)
+
+  def work_per_step(self):
+    return 2.0 * self.M * self.N * self.K
+
+  def kernel_work(self):
+    return 2.0 * self.M * self.N * self.K
+
+  def describe(self):
+    return {'workload': self.name, 'M': self.M, 'K': self.K, 'N': self.N,
+            'activation': 'bf16 N(0,1), per-token absmax -> ' + self.qtype + ' each step',
+            'weight': 'bf16 N(0,0.02) per-output-channel ' + self.qtype + ' (pre-quantized)', 'out': 'bf16'}
+
+  def cpu_baseline(self, budget_rows=4096, repeats=3):
+    """The oracle's version of one step on the first `budget_rows` tokens (best of `repeats`)."""
+    import numpy as np
+    from oracle import qwix_oracle as O
+    rows = min(budget_rows, self.M)
+    x = self.x[:rows].to('cpu').float().numpy()
+    wq = self.wq
+    wv = wq.qvalue.to('cpu')
+    if self.qtype == 'int8':
+      wnp = wv.numpy()
+    else:
+      import torch
+      wnp = wv.contiguous().view(torch.uint8).numpy()
+    owq = O.QArray(np.ascontiguousarray(wnp), O.FArr(wq.scale.to('cpu').float().numpy(), O.BF16), None, self.qtype)
+    how = O.HowToQuantize(qtype=self.qtype, channelwise_axes=[0])
+    dn = (((1,), (0,)), ((), ()))
+    dt = float('inf')
+    for _ in range(repeats):
+      t0 = time.perf_counter()
+      xq = O.quantize(O.FArr(x, O.BF16), how)
+      O.dot_general(xq, owq, dn)
+      dt = min(dt, time.perf_counter() - t0)
+    ops = 2.0 * rows * self.N * self.K
+    return {'value': round(ops / dt / 1e12, 5), 'unit': 'TOPS', 'cores': _blas_threads(), 'kind': 'port',
+            'sample': f'first {rows} of {self.M} tokens against the full ({self.K},{self.N}) weight: oracle quantize + '
+                      f'dot_general (float64 BLAS accumulate), best of {repeats}: {dt:.2f} s'}
+
+
+class QuantizeRows(Workload):
+  bound = 'hbm'
+
+  def __init__(self, name, M, K, qtype):
+    self.name, self.M, self.K, self.qtype = name, M, K, qtype
+    self.dtype = 'bf16->' + qtype
+    self.metric = 'quantize GB/s (per-token absmax, bf16 -> ' + qtype + ')'
+    self.unit = 'GB/s'
+    self.kernel = 'rows_kernel'
+
+  def setup(self, dev):
+    import torch
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(7)
+    self.x = torch.randn(self.M, self.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    qb = self.K // 2 if self.qtype == 'int4' else self.K
+    self.q = torch.empty(self.M, qb, dtype=torch.uint8, device=dev)
+    self.s = torch.empty(self.M, dtype=torch.bfloat16, device=dev)
+    self.qt = {'int8': L.INT8, 'int4': L.INT4, 'float8_e4m3fn': L.E4M3}[self.qtype]
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, rec=None):
+    L = self.L
+    if rec:
+      rec(0)
+    L.call('qwix_hip_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, 1, self.K, self.qt, L.ABSMAX, 0.0,
+           L.LAYOUT_NATURAL, self.q.data_ptr(), self.s.data_ptr(), None, None, 0, self.stream)
+    if rec:
+      rec(1)
+
+  def work_per_step(self):
+    return self.M * self.K * 2.0 + self.q.numel() + self.M * 2.0
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'M': self.M, 'K': self.K}
+
+
+class GemvW4(Workload):
+  bound = 'hbm'
+
+  def __init__(self, name, M, K, N, group):
+    self.name, self.M, self.K, self.N, self.group = name, M, K, N, group
+    self.dtype = 'bf16 x int4'
+    self.metric = 'weight-only int4 g128 GEMV GB/s'
+    self.unit = 'GB/s'
+    self.kernel = 'gemv_wq_kernel'
+
+  def setup(self, dev):
+    import torch
+    from qwix_amd.core import qarray
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(2000)
+    self.x = torch.randn(self.M, self.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    w = (torch.randn(self.K, self.N, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(dev)
+    wq = qarray.quantize_api(w, 'int4', channelwise_axes=[1], tiled_axes={0: self.group}, scale_dtype=torch.float32)
+    self.b = wq.qvalue.permute(1, 0).data
+    assert self.b.is_contiguous()
+    self.s = wq.scale.contiguous()
+    self.out = torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev)
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, rec=None):
+    L = self.L
+    if rec:
+      rec(0)
+    L.call('qwix_hip_gemv_wq', self.x.data_ptr(), self.K, self.b.data_ptr(), self.K // 2, L.INT4, self.M, self.N, self.K,
+           self.group, self.s.data_ptr(), L.F32, self.out.data_ptr(), L.BF16, self.N, self.stream)
+    if rec:
+      rec(1)
+
+  def work_per_step(self):
+    return self.K * self.N / 2.0 + (self.K // self.group) * self.N * 4.0 + self.M * self.K * 2.0 + self.M * self.N * 2.0
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'M': self.M, 'K': self.K, 'N': self.N, 'group': self.group}
+
+
+class HadamardQdot(Workload):
+  """C5: FWHT + per-token int8 quantize of the activations each step, then int8 x int4 g128 grouped GEMM
+  against the offline-rotated weight."""
+
+  bound = 'mfma'
+
+  def __init__(self, name, M, K, N):
+    self.name, self.M, self.K, self.N = name, M, K, N
+    self.dtype = 'int8 x int4'
+    self.metric = 'Hadamard-rotated a8w4 g128 qdot TOPS (FWHT + activation quantize included)'
+    self.unit = 'TOPS'
+    self.kernel = 'qgemm_grouped_kernel'
+
+  def setup(self, dev):
+    import torch
+    from qwix_amd.contrib import hadamard_rot as hr
+    from qwix_amd.core import qarray
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(5000)
+    x = torch.randn(self.M, self.K, generator=g, dtype=torch.float32)
+    idx = torch.randperm(self.K, generator=g)[: -(-self.K // 100)]
+    x[:, idx] *= 50.0
+    self.x = x.to(torch.bfloat16).to(dev)
+    w = (torch.randn(self.K, self.N, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(dev)
+    self.signs = hr.random_signs(g, self.K, torch.bfloat16, dev)
+    wq = hr.rotate_and_quantize(w, 0, qarray.HowToQuantize(qtype='int4', channelwise_axes=[1], tiled_axes={0: 128}),
+                                pre_sign=self.signs, out_scale=1.0 / self.K)
+    del w
+    self.b = wq.qvalue.permute(1, 0).data
+    assert self.b.is_contiguous()
+    self.sb = wq.scale.contiguous()
+    self.xq = torch.empty(self.M, self.K, dtype=torch.int8, device=dev)
+    self.sa = torch.empty(self.M, dtype=torch.bfloat16, device=dev)
+    self.out = torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev)
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, rec=None):
+    L = self.L
+    L.call('qwix_hip_fwht_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, self.signs.data_ptr(), None, 1.0, self.K,
+           L.INT8, self.xq.data_ptr(), self.sa.data_ptr(), self.stream)
+    if rec:
+      rec(0)
+    L.call('qwix_hip_qgemm_grouped', self.xq.data_ptr(), self.K, self.b.data_ptr(), self.K // 2, L.INT4, self.M, self.N,
+           self.K, 128, self.sa.data_ptr(), L.BF16, 1, self.sb.data_ptr(), L.BF16, self.out.data_ptr(), L.BF16, self.N, 0,
+           None, self.stream)
+    if rec:
+      rec(1)
+
+  def work_per_step(self):
+    return 2.0 * self.M * self.N * self.K
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'M': self.M, 'K': self.K, 'N': self.N, 'group': 128}
+
+
+WORKLOADS = {
+    'c3_int8_w8a8_4096': lambda: QdotW8A8('c3_int8_w8a8_4096', 4096, 4096, 4096, 'int8'),
+    'c4_fp8_w8a8_ffn': lambda: QdotW8A8('c4_fp8_w8a8_ffn', 8192, 8192, 28672, 'float8_e4m3fn'),
+    'c3_fp8_w8a8_4096': lambda: QdotW8A8('c3_fp8_w8a8_4096', 4096, 4096, 4096, 'float8_e4m3fn'),
+    'int8_w8a8_8192': lambda: QdotW8A8('int8_w8a8_8192', 8192, 8192, 8192, 'int8'),
+    'quantize_act_4096': lambda: QuantizeRows('quantize_act_4096', 4096, 4096, 'int8'),
+    'quantize_act_8192_fp8': lambda: QuantizeRows('quantize_act_8192_fp8', 8192, 8192, 'float8_e4m3fn'),
+    'c2_gemv_w4_m1': lambda: GemvW4('c2_gemv_w4_m1', 1, 4096, 14336, 128),
+    'c2_gemv_w4_m16': lambda: GemvW4('c2_gemv_w4_m16', 16, 4096, 14336, 128),
+    'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
+}
+DEFAULT = 'c3_int8_w8a8_4096'
+EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16',
+         'c5_hadamard_a8w4']
+
+
+def _blas_threads() -> int:
+  try:
+    from threadpoolctl import threadpool_info
+    n = [p.get('num_threads', 0) for p in threadpool_info() if p.get('user_api') == 'blas']
+    if n:
+      return int(max(n))
+  except Exception:
+    pass
+  return int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1))
+
+
+def run(wl: Workload, steps: int, warmup: int):
+  import torch
+  dev = torch.device('cuda:0')
+  wl.setup(dev)
+  for _ in range(warmup):
+    wl.step()
+  torch.cuda.synchronize()
+  ev = [_events(2) for _ in range(steps)]
+  cur = [0]
+
+  def rec(which):
+    ev[cur[0]][which].record()
+
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for i in range(steps):
+    cur[0] = i
+    wl.step(rec)
+  torch.cuda.synchronize()
+  dt = time.perf_counter() - t0
+  kt = sorted(a.elapsed_time(b) * 1e-3 for a, b in ev)
+  kmean = sum(kt) / len(kt)
+  return dt / steps, kmean, kt[len(kt) // 2]
+
+
+def summarize(wl: Workload, step_s: float, kern_s: float) -> dict:
+  peak = PEAK_MFMA_TOPS if wl.bound == 'mfma' else PEAK_HBM_GBS
+  scale = 1e12 if wl.bound == 'mfma' else 1e9
+  value = wl.work_per_step() / step_s / scale
+  achieved = wl.kernel_work() / kern_s / scale
+  return {
+      'value': round(value, 2), 'unit': wl.unit, 'ms_per_step': round(step_s * 1e3, 5),
+      'roofline': {'bound': wl.bound, 'kernel': wl.kernel, 'achieved': round(achieved, 2), 'peak': peak,
+                   'unit': 'TFLOP/s' if wl.bound == 'mfma' else 'GB/s', 'frac': round(achieved / peak, 4),
+                   'traffic': _traffic(wl.name)},
+  }
+
+
+def _traffic(name: str):
+  """HBM bytes per launch of the dominant kernel, from committed rocprofv3 --pmc measurements."""
+  p = os.path.join(ROOT, 'profiles', 'hbm_traffic.json')
+  if os.path.exists(p):
+    try:
+      return json.load(open(p)).get(name)
+    except Exception:
+      return None
+  return None
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument('--gpus', type=int, default=1)
+  ap.add_argument('--steps', type=int, default=50)
+  ap.add_argument('--warmup', type=int, default=5)
+  ap.add_argument('--workload', default=DEFAULT, choices=sorted(WORKLOADS))
+  ap.add_argument('--no-extra', action='store_true', help='skip the other workloads of the metric')
+  ap.add_argument('--no-cpu-baseline', action='store_true')
+  args = ap.parse_args()
+  if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
+    print('bench.py: this build runs on ONE GPU only (no collectives, no sharding); re-run with --gpus 1. '
+          'The reported value is the single GPU throughput.', file=sys.stderr)
+    sys.exit(2)
+  import torch
+  if not torch.cuda.is_available():
+    print('bench.py: no GPU visible; the hot path has no CPU fallback.', file=sys.stderr)
+    sys.exit(2)
+
+  wl = WORKLOADS[args.workload]()
+  step_s, kmean, _ = run(wl, args.steps, args.warmup)
+  res = summarize(wl, step_s, kmean)
+  line = {
+      'metric': wl.metric, 'value': res['value'], 'unit': res['unit'], 'n_gpus': 1, 'steps': args.steps,
+      'warmup': args.warmup, 'ms_per_step': res['ms_per_step'], 'higher_is_better': True, 'scaling': 'weak',
+      'vs_baseline': None, 'dtype': wl.dtype, 'data': 'synthetic', 'config': wl.describe(),
+      'roofline': res['roofline'],
+  }
+  if not args.no_cpu_baseline and hasattr(wl, 'cpu_baseline'):
+    line['cpu_baseline'] = wl.cpu_baseline()
+  else:
+    line['cpu_baseline'] = None
+  if not args.no_extra and args.workload == DEFAULT:
+    extra = {}
+    for name in EXTRA:
+      w = WORKLOADS[name]()
+      n = max(5, min(args.steps, 20))
+      s, km, _ = run(w, n, 3)
+      r = summarize(w, s, km)
+      extra[name] = {'metric': w.metric, 'value': r['value'], 'unit': r['unit'], 'ms_per_step': r['ms_per_step'],
+                     'roofline': r['roofline']}
+      del w
+      torch.cuda.empty_cache()
+    line['extra'] = extra
+  print(json.dumps(line))
+
+
+if __name__ == '__main__':
+  main()
