@@ -1,0 +1,58 @@
+"""Quantized einsum: string -> dimension numbers -> the HIP dot_general (host glue).
+
+Mirror of qwix/_src/core/einsum.py: `get_how_to_quantize` (:27-81) and `einsum` (:106-188) for
+the binary case; the contraction itself is `_qwix_dot_general` (default: the MFMA-backed
+qwix_amd dot_general).  N-ary einsums are contracted pairwise left to right.
+"""
+from __future__ import annotations
+
+from typing import Any, Mapping
+
+import torch
+
+from qwix_amd.core import dot_general as _dg
+from qwix_amd.core import einsum_info
+from qwix_amd.core import qarray
+
+
+def get_how_to_quantize(*, einsum_str: str, ndims: tuple[int, int], for_lhs: bool,
+                        tile_size: Mapping[int, int | float] | int | float | None, **kwargs: Any) -> qarray.HowToQuantize:
+  """Channelwise for every non-contracted subscript; tiles on the last contracted axis if tile_size."""
+  info = einsum_info.EinsumInfo.parse(einsum_str, ndims=ndims)
+  subs = info.lhs if for_lhs else info.rhs
+  channelwise, last = [], None
+  for axis, ch in enumerate(subs):
+    if ch in info.contract_chars:
+      last = axis
+    else:
+      channelwise.append(axis)
+  tiled: dict = {}
+  if isinstance(tile_size, Mapping):
+    tiled = dict(tile_size)
+    channelwise = [a for a in channelwise if a not in tiled]
+  elif tile_size and last is not None:
+    tiled[last] = tile_size
+  return qarray.HowToQuantize(channelwise_axes=channelwise, tiled_axes=tiled, **kwargs)
+
+
+def _binary(lhs, rhs, einsum_str: str, dot_general_fn, preferred_element_type, **kwargs):
+  info = einsum_info.EinsumInfo.parse(einsum_str, ndims=(len(lhs.shape), len(rhs.shape)))
+  out = dot_general_fn(lhs, rhs, info.dimension_numbers, preferred_element_type=preferred_element_type, **kwargs)
+  if info.output_perm is not None:
+    out = out.permute(*info.output_perm)
+  return out
+
+
+def einsum(*args, _qwix_dot_general=_dg.dot_general, preferred_element_type=None, **kwargs) -> torch.Tensor:
+  """Drop-in for jnp.einsum('subscripts', a, b) with QArray operands; the result dtype follows the
+  dequantized dtypes unless preferred_element_type is given."""
+  if not args or not isinstance(args[0], str):
+    raise NotImplementedError('einsum expects the subscripts string first')
+  einsum_str, operands = args[0], list(args[1:])
+  _, res_t = qarray.get_accumulator_and_result_type(*operands, preferred_element_type=preferred_element_type)
+  if len(operands) == 1:
+    op = operands[0]
+    return torch.einsum(einsum_str, qarray.dequantize(op) if isinstance(op, qarray.QArray) else op).to(res_t)
+  if len(operands) != 2:
+    raise NotImplementedError(f'einsum with {len(operands)} operands: contract them pairwise')
+  return _binary(operands[0], operands[1], einsum_str, _qwix_dot_general, res_t, **kwargs)

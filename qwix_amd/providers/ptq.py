@@ -1,0 +1,207 @@
+"""Post-training quantization provider on top of the HIP quantize / dot_general kernels.
+
+Mirror of qwix/_src/providers/ptq.py (`PtqProvider` :33-49, `quantize_params` :52-135) and of the
+parts of providers/boxed_param.py it inherits: `WithAux` (:37-77), `BoxedParamProvider.__init__`
+with its three injection points `_qarray_module`, `_dot_general_fn`, `_einsum_fn` (:92-107),
+`dot_general` (:109-171), `einsum` (:173-236), `quantize_act` (:416-455, dynamic and static
+range) and `create_quantized_param` (:458-499).
+
+Weights reach the provider either as `WithAux[QArray]` (already quantized: used as is) or as a
+`Param` (a named float tensor inside a params dict: quantized on first use and written back, which
+is how the reference turns float checkpoints into PTQ params); any other float tensor is an
+activation.  `precision` / `preferred_element_type` given by the caller are not forwarded, as in
+the reference (boxed_param.py:169-171).
+"""
+from __future__ import annotations
+
+import dataclasses
+import functools
+from typing import Any, Callable, Generic, Mapping, Sequence, TypeVar
+
+import torch
+
+from qwix_amd import qconfig
+from qwix_amd.core import dot_general as _dot_general
+from qwix_amd.core import einsum as _einsum
+from qwix_amd.core import qarray as _qarray
+
+T = TypeVar('T')
+
+
+@dataclasses.dataclass
+class WithAux(Generic[T]):
+  """A (quantized) array plus how it was / is to be quantized, so that quantize_params() can
+  quantize float weights without running the model."""
+
+  array: T
+  how: _qarray.HowToQuantize
+
+  value = property(lambda self: self.array)
+  shape = property(lambda self: tuple(self.array.shape))
+  ndim = property(lambda self: len(self.array.shape))
+  dtype = property(lambda self: self.array.dtype)
+
+  def replace(self, **kw) -> 'WithAux':
+    return dataclasses.replace(self, **kw)
+
+  def reshape(self, *shape):
+    if len(shape) == 1 and not isinstance(shape[0], int):
+      shape = tuple(shape[0])
+    if tuple(self.shape) != tuple(shape):
+      raise ValueError(f'Boxed weights should already have the target shape. Got {self.shape=} but {shape=} is requested.')
+    return self
+
+
+@dataclasses.dataclass
+class Param:
+  """A float weight together with where it lives: `store[name]` (a mutable params dict)."""
+
+  store: dict
+  name: str
+
+  value = property(lambda self: self.store[self.name])
+  shape = property(lambda self: tuple(self.value.shape))
+  ndim = property(lambda self: self.value.ndim)
+
+
+def create_quantized_param(param: Param, how: _qarray.HowToQuantize, *, _qarray_module=_qarray) -> WithAux:
+  """Quantizes a float weight, replaces it in its params dict, and returns the boxed QArray."""
+  value = param.value
+  if isinstance(value, WithAux):
+    return value
+  if not isinstance(value, torch.Tensor):
+    raise ValueError(f'Cannot quantize param {param.name!r} of type {type(value)}; feed float tensors or WithAux.')
+  boxed = WithAux(_qarray_module.quantize(value, how), how)
+  param.store[param.name] = boxed
+  return boxed
+
+
+def quantize_act(array: torch.Tensor, how: _qarray.HowToQuantize, rule: qconfig.QuantizationRule, act_name: str, *,
+                 quant_stats: Mapping[str, Any] | None = None, _qarray_module=_qarray) -> _qarray.QArray:
+  """Dynamic-range: one fused quantize.  Static-range (rule.act_static_scale): scale / zero point
+  come from `quant_stats[act_name + '_scale' / '_zero_point']` computed offline."""
+  if not rule.act_static_scale:
+    return _qarray_module.quantize(array, how)
+  if quant_stats is None or act_name + '_scale' not in quant_stats:
+    raise ValueError(f'static-range quantization of {act_name!r} needs a precomputed {act_name}_scale')
+  scale = quant_stats[act_name + '_scale']
+  scale = scale.array if isinstance(scale, WithAux) else scale
+  zp = quant_stats.get(act_name + '_zero_point')
+  return _qarray_module.quantize_with_scale_zero_point(array, how.qtype, scale, zp)
+
+
+class BoxedParamProvider(qconfig.QuantizationProvider):
+  """Runtime ops that substitute boxed (quantized) parameters; subclasses add policy."""
+
+  def __init__(self, rules: Sequence[qconfig.QuantizationRule], *, disable_jit: bool = False, _qarray_module=_qarray,
+               _dot_general_fn: Callable = _dot_general.dot_general, _einsum_fn: Callable = _einsum.einsum,
+               _conv_general_dilated_fn: Callable | None = None):
+    super().__init__(rules, disable_jit=disable_jit)
+    self._qarray_module = _qarray_module
+    self._dot_general_fn = _dot_general_fn
+    self._einsum_fn = _einsum_fn
+    self._conv_general_dilated_fn = _conv_general_dilated_fn
+    self.quant_stats: dict[str, Any] = {}
+
+  # -- helpers
+  def _prepare(self, lhs, rhs, rule, op_id, get_how):
+    if isinstance(rhs, WithAux):
+      rhs = rhs.array
+    elif isinstance(rhs, Param):
+      if isinstance(rhs.value, WithAux):
+        rhs = rhs.value.array
+      else:
+        how = get_how(for_lhs=False, qtype=rule.weight_qtype, calibration_method=rule.weight_calibration_method)
+        rhs = create_quantized_param(rhs, how, _qarray_module=self._qarray_module).array
+    elif rule.act_qtype is not None:
+      how = get_how(for_lhs=False, qtype=rule.act_qtype, calibration_method=rule.act_calibration_method or 'absmax')
+      rhs = quantize_act(rhs, how, rule, op_id + '_rhs', quant_stats=self.quant_stats, _qarray_module=self._qarray_module)
+    if rule.act_qtype is not None:
+      how = get_how(for_lhs=True, qtype=rule.act_qtype, calibration_method=rule.act_calibration_method or 'absmax')
+      lhs = quantize_act(lhs, how, rule, op_id + '_lhs', quant_stats=self.quant_stats, _qarray_module=self._qarray_module)
+    return lhs, rhs
+
+  @staticmethod
+  def _unbox_float(x):
+    if isinstance(x, Param):
+      x = x.value
+    if isinstance(x, WithAux):
+      x = x.array
+    return _qarray.dequantize(x) if isinstance(x, _qarray.QArray) else x
+
+  # -- ops
+  def dot_general(self, lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None, *, out_sharding=None):
+    rule, op_id = self._get_current_rule_and_op_id('dot_general')
+    if rule is None or rule.weight_qtype is None:
+      (lc, rc), _ = dimension_numbers
+      out = torch.tensordot(self._unbox_float(lhs), self._unbox_float(rhs), dims=(list(lc), list(rc)))
+      return out if preferred_element_type is None else out.to(preferred_element_type)
+    get_how = functools.partial(_dot_general.get_how_to_quantize, dimension_numbers=dimension_numbers,
+                                ndims=(len(lhs.shape), len(rhs.shape)), tile_size=rule.tile_size)
+    lhs, rhs = self._prepare(lhs, rhs, rule, op_id, get_how)
+    return self._dot_general_fn(lhs, rhs, dimension_numbers, out_sharding=out_sharding)
+
+  def einsum(self, einsum_str: str, *operands, precision=None, preferred_element_type=None, out_sharding=None):
+    rule, op_id = self._get_current_rule_and_op_id('einsum')
+    if rule is None or rule.weight_qtype is None:
+      out = torch.einsum(einsum_str, *[self._unbox_float(o) for o in operands])
+      return out if preferred_element_type is None else out.to(preferred_element_type)
+    if len(operands) != 2:
+      raise ValueError(f'Unsupported einsum format: {einsum_str=} {operands=}')
+    lhs, rhs = operands
+    get_how = functools.partial(_einsum.get_how_to_quantize, einsum_str=einsum_str,
+                                ndims=(len(lhs.shape), len(rhs.shape)), tile_size=rule.tile_size)
+    lhs, rhs = self._prepare(lhs, rhs, rule, op_id, get_how)
+    return self._einsum_fn(einsum_str, lhs, rhs)
+
+
+class PtqProvider(BoxedParamProvider):
+  """Quantization provider for PTQ: float weights are replaced by quantized ones when the ops run;
+  `quantize_params` does the same offline from the `how` recorded in the quantized param tree."""
+
+
+def _flatten(tree: Mapping, prefix=()) -> dict[tuple, Any]:
+  out = {}
+  for k, v in tree.items():
+    if isinstance(v, Mapping):
+      out.update(_flatten(v, prefix + (k,)))
+    else:
+      out[prefix + (k,)] = v
+  return out
+
+
+def _unflatten(flat: Mapping[tuple, Any]) -> dict:
+  out: dict = {}
+  for path, v in flat.items():
+    d = out
+    for k in path[:-1]:
+      d = d.setdefault(k, {})
+    d[path[-1]] = v
+  return out
+
+
+def quantize_params(params: Mapping, abstract_quantized_params: Mapping, quant_stats: Mapping | None = None, *,
+                    allow_extra_params: bool = False, _qarray_module=_qarray) -> dict:
+  """Quantizes a float param tree offline.
+
+  `abstract_quantized_params` is the param tree of the PTQ model (leaves that are `WithAux` carry
+  the `how`; their arrays may be real or shape-only).  Float leaves whose template is a `WithAux`
+  are reshaped to the template's shape and quantized with `_qarray_module.quantize`; other leaves
+  are passed through; leaves missing from the template raise unless allow_extra_params.
+  """
+  del quant_stats  # static-range statistics are applied by the provider (quant_stats attribute)
+  abstract = _flatten(abstract_quantized_params)
+  out = {}
+  for path, param in _flatten(params).items():
+    if not isinstance(param, torch.Tensor):
+      raise TypeError(f'params is not a pure dict of tensors: {type(param)}')
+    tmpl = abstract.get(path)
+    if tmpl is None:
+      if allow_extra_params:
+        continue
+      raise ValueError(f'{path} is not found in the abstract_quantized_params.')
+    if isinstance(tmpl, WithAux):
+      param = param.reshape(tmpl.shape)
+      param = tmpl.replace(array=_qarray_module.quantize(param, tmpl.how))
+    out[path] = param
+  return _unflatten(out)

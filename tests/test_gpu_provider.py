@@ -1,0 +1,143 @@
+"""GPU parity through the provider surface: QuantizationRule -> PtqProvider -> quantize_model /
+quantize_params, on the PTQ MLP of BASELINE config 1 and on an einsum layer."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import qwix_oracle as O
+from tests import util
+
+pytestmark = pytest.mark.gpu
+DN = (((1,), (0,)), ((), ()))
+
+
+def _mlp_setup(batch=256, d_in=1024, hidden=4096, d_out=1024):
+  import qwix_amd
+  from qwix_amd import nn
+  model = nn.MLP(hidden, d_out)
+  g = torch.Generator().manual_seed(1001)
+  params = model.init(g, d_in, torch.float32, util.DEV)
+  x = torch.rand(batch, d_in, generator=g, dtype=torch.float32).to(util.DEV)
+  rules = [qwix_amd.QuantizationRule(module_path='.*', weight_qtype='int8', act_qtype='int8')]
+  return model, params, x, rules
+
+
+def _oracle_mlp(params, x):
+  """The reference's flow restated with the oracle: per-channel int8 weights, per-token int8 activations."""
+  w1 = util.farr(params['Dense_0']['kernel'])
+  w2 = util.farr(params['Dense_1']['kernel'])
+  hw = O.HowToQuantize(qtype='int8', channelwise_axes=[1])
+  ha = O.HowToQuantize(qtype='int8', channelwise_axes=[0])
+  w1q, w2q = O.quantize(w1, hw), O.quantize(w2, hw)
+  xq = O.quantize(util.farr(x), ha)
+  h, acc1 = O.fast_dot_general(xq, w1q, DN, return_acc=True)
+  h = O.FArr(np.maximum(h.v, 0), O.F32)
+  hq = O.quantize(h, ha)
+  out, acc2 = O.fast_dot_general(hq, w2q, DN, return_acc=True)
+  return dict(w1q=w1q, w2q=w2q, xq=xq, hq=hq, acc1=acc1, acc2=acc2, out=out)
+
+
+def test_config1_ptq_mlp_quantize_params_then_apply():
+  import qwix_amd
+  from qwix_amd.providers.ptq import WithAux
+  model, params, x, rules = _mlp_setup()
+  ptq_model = qwix_amd.quantize_model(model, qwix_amd.PtqProvider(rules))
+  abstract = ptq_model.init(params, x)                        # PTQ param tree with `how`
+  qparams = qwix_amd.quantize_params(params, abstract)        # offline weight quantization
+  want = _oracle_mlp(params, x)
+  for name, key, n in (('Dense_0', 'w1q', 4096), ('Dense_1', 'w2q', 1024)):
+    leaf = qparams[name]['kernel']
+    assert isinstance(leaf, WithAux) and tuple(leaf.array.scale.shape) == (1, n) and leaf.array.scale.dtype == torch.float32
+    assert leaf.array.qvalue.dtype == torch.int8 and tuple(leaf.array.shape) == tuple(params[name]['kernel'].shape)
+    util.assert_qarray_equal(leaf.array, want[key], name)
+  out = ptq_model.apply(qparams, x)
+  assert out.dtype == torch.float32 and tuple(out.shape) == (256, 1024)
+  got = util.f32np(out)
+  assert np.array_equal(got, want['out'].v), np.abs(got - want['out'].v).max()
+  # quantize_params == implicit quantization on first use (ptq_test.py:68-80)
+  for name in ('Dense_0', 'Dense_1'):
+    a, b = abstract[name]['kernel'].array, qparams[name]['kernel'].array
+    assert torch.equal(a.qvalue, b.qvalue) and torch.equal(a.scale, b.scale)
+  # and close to the float model
+  ref = model(params, x)
+  assert (out - ref).abs().mean() / ref.abs().mean() < 0.02
+
+
+def test_config1_intermediate_accumulators_and_activation_quantization():
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  model, params, x, _ = _mlp_setup()
+  want = _oracle_mlp(params, x)
+  hw = qarray.HowToQuantize(qtype='int8', channelwise_axes=[1])
+  ha = qarray.HowToQuantize(qtype='int8', channelwise_axes=[0])
+  w1q, w2q = qarray.quantize(params['Dense_0']['kernel'], hw), qarray.quantize(params['Dense_1']['kernel'], hw)
+  xq = qarray.quantize(x, ha)
+  util.assert_qarray_equal(xq, want['xq'], 'x')
+  h, acc1 = dg._fast_dot_general(xq, w1q, DN, return_accumulators=True)
+  assert np.array_equal(acc1.cpu().numpy(), want['acc1'])
+  hq = qarray.quantize(torch.relu(h), ha)
+  util.assert_qarray_equal(hq, want['hq'], 'hidden')
+  _, acc2 = dg._fast_dot_general(hq, w2q, DN, return_accumulators=True)
+  assert np.array_equal(acc2.cpu().numpy(), want['acc2'])
+
+
+def test_unquantized_rule_and_unused_rules():
+  import qwix_amd
+  model, params, x, _ = _mlp_setup(batch=16, d_in=128, hidden=256, d_out=64)
+  rules = [qwix_amd.QuantizationRule(module_path='Dense_0', weight_qtype='int8'),
+           qwix_amd.QuantizationRule(module_path='nothing', weight_qtype='int4')]
+  prov = qwix_amd.PtqProvider(rules)
+  pm = qwix_amd.quantize_model(model, prov)
+  p = pm.init(params, x)
+  from qwix_amd.providers.ptq import WithAux
+  assert isinstance(p['Dense_0']['kernel'], WithAux) and isinstance(p['Dense_1']['kernel'], torch.Tensor)
+  assert [r.module_path for r in prov.get_unused_rules()] == ['nothing']
+  out = pm.apply(p, x)   # weight-only int8 on layer 0 (dequantize path), float layer 1
+  ref = model(params, x)
+  assert (out - ref).abs().mean() / ref.abs().mean() < 0.01
+  with pytest.raises(ValueError, match='not found in the abstract'):
+    qwix_amd.quantize_params({'Other': {'kernel': params['Dense_0']['kernel']}}, p)
+  assert qwix_amd.quantize_params({'Other': {'kernel': params['Dense_0']['kernel']}}, p, allow_extra_params=True) == {}
+
+
+def test_einsum_layer_with_subchannel_rule():
+  """'btd,dnh->btnh' weight (d, n, h) contracting d, tile 128: scale (d/128, n, h) (ptq_test.py shapes)."""
+  import qwix_amd
+  from qwix_amd import nn
+  layer = nn.Einsum('btd,dnh->btnh', (256, 4, 32))
+  g = torch.Generator().manual_seed(5)
+  params = layer.init(g, torch.bfloat16, util.DEV)
+  x = torch.randn(2, 24, 256, generator=g).to(torch.bfloat16).to(util.DEV)
+  rules = [qwix_amd.QuantizationRule(weight_qtype='int4', act_qtype='int8', tile_size=128)]
+  pm = qwix_amd.quantize_model(lambda p, x: layer(p, x), qwix_amd.PtqProvider(rules))
+  qp = pm.init(params, x)
+  wq = qp['kernel'].array
+  assert tuple(wq.scale.shape) == (2, 4, 32) and wq.qtype == 'int4'
+  out = pm.apply(qp, x)
+  assert tuple(out.shape) == (2, 24, 4, 32)
+  ow = O.quantize(util.farr(params['kernel']), O.HowToQuantize(qtype='int4', channelwise_axes=[1, 2], tiled_axes={0: 128}))
+  util.assert_qarray_equal(wq, ow, 'einsum weight')
+  ox = O.quantize(util.farr(x), O.HowToQuantize(qtype='int8', channelwise_axes=[0, 1], tiled_axes={2: 128}))
+  want, wacc = O.fast_dot_general(ox, ow, (((2,), (0,)), ((), ())), return_acc=True)
+  got = util.f32np(out)
+  sx = ox.scale.v.reshape(-1, 2)
+  mag = (np.abs(wacc.reshape(2, 48, 128)).astype(np.float64) * sx.T[:, :, None] * ow.scale.v.reshape(2, 1, 128)).sum(0).reshape(want.v.shape)
+  assert np.all(np.abs(got - want.v) <= 1e-2 * np.abs(want.v) + 2.0**-7 * mag)
+
+
+def test_small_tile_rule_takes_the_dequantize_path():
+  """(12, 5) kernel with tile 4 -> scale (3, 5) (ptq_test.py:698-730); tile < 128 => slow path."""
+  import qwix_amd
+  from qwix_amd import nn
+  layer = nn.Dense(5, name='Dense_0')
+  g = torch.Generator().manual_seed(6)
+  params = layer.init(g, 12, torch.float32, util.DEV, std=1.0)
+  x = torch.randn(3, 12, generator=g).to(util.DEV)
+  pm = qwix_amd.quantize_model(lambda p, x: layer(p, x), qwix_amd.PtqProvider([qwix_amd.QuantizationRule(weight_qtype='int8', tile_size=4)]))
+  qp = pm.init(params, x)
+  assert tuple(qp['kernel'].array.scale.shape) == (3, 5)
+  out = pm.apply(qp, x)
+  ow = O.quantize(util.farr(params['kernel']), O.HowToQuantize(qtype='int8', channelwise_axes=[1], tiled_axes={0: 4}))
+  util.assert_qarray_equal(qp['kernel'].array, ow, 'tile 4 weight')
+  want = O.dot_general(util.farr(x), ow, DN)
+  assert np.allclose(util.f32np(out), want.v, rtol=1e-5, atol=1e-6)

@@ -1,0 +1,173 @@
+"""CPU-only tests: host-side mirror of the reference interface, and the C-ABI library surface."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from oracle import qwix_oracle as O
+from qwix_amd import _lib, qconfig
+from qwix_amd.core import dot_general as dg
+from qwix_amd.core import einsum as es
+from qwix_amd.core import einsum_info, numerics, qarray
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+  header = open(os.path.join(ROOT, 'include', 'qwix_hip.h')).read()
+  declared = sorted(set(re.findall(r'\b(qwix_hip_\w+)\s*\(', header)))
+  assert len(declared) >= 15
+  lib = _lib.load()
+  for name in declared:
+    assert hasattr(lib, name), f'{name} is declared in include/qwix_hip.h but not exported'
+    assert name in _lib.SIGNATURES, f'{name} has no ctypes prototype'
+  assert sorted(_lib.SIGNATURES) == declared
+  assert lib.qwix_hip_abi_version() == 1
+  # a pure host-side entry point (no GPU work): workspace size query
+  assert lib.qwix_hip_quantize_workspace_bytes(1, 4096, 4096, 4096, _lib.ABSMAX) == 4096 * 4
+  assert lib.qwix_hip_quantize_workspace_bytes(8, 4096, 1, 4096, _lib.ABSMAX) == 0
+  assert lib.qwix_hip_quantize_workspace_bytes(1, 4096, 64, 128, _lib.MINMAX) == 32 * 64 * 4 * 2
+
+
+def test_argument_validation_happens_before_any_launch():
+  lib = _lib.load()
+  # null pointers / bad geometry are rejected on the host, with a message
+  assert lib.qwix_hip_quantize(None, 0, 1, 8, 1, 8, 0, 0, 0.0, 0, None, None, None, None, 0, None) == 1
+  assert b'null' in lib.qwix_hip_last_error()
+  assert lib.qwix_hip_fwht(ctypes.c_void_p(16), 0, 4, 6, None, None, 1.0, ctypes.c_void_p(16), None) == 1
+  assert b'power of 2' in lib.qwix_hip_last_error()
+  with pytest.raises(_lib.QwixHipError, match='no CPU path'):
+    qarray.quantize(torch.zeros(4, 8), qarray.HowToQuantize(qtype='int8'))
+
+
+def test_bounds_and_eligibility():
+  assert numerics.get_symmetric_bound('int8') == 127.5 and numerics.get_symmetric_bound(torch.int8) == 127.5
+  assert numerics.get_symmetric_bound('int4') == 7.5 and numerics.get_symmetric_bound(torch.float8_e4m3fn) == 448.0
+  assert numerics.get_asymmetric_bound('int4') == (-8.0, 7.0)
+  with pytest.raises(ValueError, match="doesn't support asymmetric"):
+    numerics.get_asymmetric_bound('nf4')
+  assert numerics.should_quantize(torch.bfloat16) and not numerics.should_quantize(torch.int8)
+  assert not numerics.can_dequant_on_output('nf4') and numerics.can_dequant_on_output('int4')
+
+
+def test_scale_shape_rules_match_oracle():
+  for shape, cw, tiled in [((2, 2, 6), [0], {2: 2}), ((128, 128), [], {0: 8, 1: 8}), ((16, 64), [1], {}), ((4, 12), [0], {1: 1 / 3})]:
+    a = qarray.get_scale_shape(shape, qarray.HowToQuantize(qtype='int8', channelwise_axes=cw, tiled_axes=tiled))
+    b = O.get_scale_shape(shape, O.HowToQuantize(qtype='int8', channelwise_axes=cw, tiled_axes=tiled))
+    assert a == b
+  with pytest.raises(ValueError, match='cannot be tiled'):
+    qarray.get_scale_shape((4, 10), qarray.HowToQuantize(qtype='int8', tiled_axes={1: 4}))
+  with pytest.raises(ValueError, match='both channelwise and tiled'):
+    qarray.get_scale_shape((4, 8), qarray.HowToQuantize(qtype='int8', channelwise_axes=[1], tiled_axes={1: 4}))
+
+
+def test_plan_maps_patterns_to_kernel_views():
+  P = qarray._plan
+  assert P((64, 4096), (1, 4096)).dims == (64, 4096, 1)
+  assert P((512, 256), (128, 1)).dims == (1, 512, 256) and P((512, 256), (128, 1)).tiles == (128,)
+  assert P((2, 3, 512), (1, 1, 512)).dims == (6, 512, 1)
+  assert P((256, 4, 32), (128, 1, 1)).dims == (1, 256, 128)
+  p = P((4, 64, 128), (4, 64, 1))
+  assert p.dims == (1, 256, 128) and p.tiles == (256,) and p.reduce_axes == (0, 1) and p.inner_axes == (2,)
+  assert P((128, 128), (8, 8)).kind == '5d'
+  assert P((4, 64, 128), (4, 32, 1)).dims == (1, 4, 1, 64, 128)
+  with pytest.raises(NotImplementedError):
+    P((4, 4, 4, 4, 4, 4), (2, 1, 2, 1, 2, 1))
+
+
+def test_get_how_to_quantize_matches_oracle():
+  dn = (((2, 3), (0, 1)), ((), ()))
+  for for_lhs in (True, False):
+    a = dg.get_how_to_quantize(dimension_numbers=dn, ndims=(4, 3), for_lhs=for_lhs, qtype='int8', tile_size=32)
+    b = O.dg_get_how_to_quantize(dimension_numbers=dn, ndims=(4, 3), for_lhs=for_lhs, qtype='int8', tile_size=32)
+    assert dict(a.tiled_axes) == dict(b.tiled_axes) and list(a.channelwise_axes) == list(b.channelwise_axes)
+    a = es.get_how_to_quantize(einsum_str='BTNH,NHO->BTO', ndims=(4, 3), for_lhs=for_lhs, qtype='int8', tile_size=32)
+    b = O.einsum_get_how_to_quantize(einsum_str='BTNH,NHO->BTO', ndims=(4, 3), for_lhs=for_lhs, qtype='int8', tile_size=32)
+    assert dict(a.tiled_axes) == dict(b.tiled_axes) and list(a.channelwise_axes) == list(b.channelwise_axes)
+  h = dg.get_how_to_quantize(dimension_numbers=(((1,), (0,)), ((), ())), ndims=(2, 2), for_lhs=False, qtype='int4', tile_size={0: 128})
+  assert dict(h.tiled_axes) == {0: 128} and list(h.channelwise_axes) == [1]
+
+
+@pytest.mark.parametrize(
+    's,ndims,batch,contract,nl,nr,no',
+    [('abc,bcd->acd', None, ['c'], ['b'], 3, 3, 3), ('ab,bc->ac', None, [], ['b'], 2, 2, 2), ('bth,thk->btk', None, ['t'], ['h'], 3, 3, 3),
+     (',i->i', None, [], [], 0, 1, 1), ('...a,ab->...b', (2, 2), [], ['a'], 2, 2, 2), ('ab,...b->...a', (2, 2), [], ['b'], 2, 2, 2),
+     ('...a,...b->...', (2, 2), None, [], 2, 2, 1)],
+)
+def test_einsum_info_parse_table(s, ndims, batch, contract, nl, nr, no):
+  """einsum_info_test.py:66-130 (subscript letters chosen for '...' may differ; structure may not)."""
+  info = einsum_info.EinsumInfo.parse(s, ndims=ndims)
+  assert (len(info.lhs), len(info.rhs), len(info.out)) == (nl, nr, no)
+  if batch is not None:
+    assert info.batch_chars == batch
+  else:
+    assert len(info.batch_chars) == 1
+  assert info.contract_chars == contract
+  o = O.EinsumInfo.parse(f'{info.lhs},{info.rhs}->{info.out}')
+  assert info.dimension_numbers == o.dimension_numbers and info.output_perm == o.output_perm
+
+
+def test_einsum_info_rejects_unsupported_strings():
+  with pytest.raises(NotImplementedError):
+    einsum_info.EinsumInfo.parse('ab,bc')
+  with pytest.raises(NotImplementedError):
+    einsum_info.EinsumInfo.parse('aab,bc->ac')
+
+
+@pytest.mark.parametrize(
+    'lhs,rhs,expect',
+    [(torch.bfloat16, torch.float32, torch.float32), (torch.bfloat16, ('int8', torch.bfloat16), torch.bfloat16),
+     (torch.bfloat16, ('int8', torch.float32), torch.float32), (('int4', torch.bfloat16), ('int8', torch.float32), torch.float32),
+     (('float8_e4m3fn', torch.bfloat16), ('float8_e4m3fn', torch.float32), torch.float32), (torch.bool, ('int8', torch.bfloat16), torch.bfloat16)],
+)
+def test_result_dtype_table(lhs, rhs, expect):
+  """dot_general_test.py:28-146, on CPU tensors (no kernels run)."""
+  def mk(spec):
+    if not isinstance(spec, tuple):
+      return torch.ones(10, 10).to(spec)
+    qt, st = spec
+    if qt == 'int4':
+      q = qarray.Int4Tensor(torch.zeros(10, 5, dtype=torch.uint8), (10, 10), 1)
+    else:
+      q = torch.ones(10, 10).to(numerics.storage_dtype(qt))
+    return qarray.QArray(q, torch.ones(1, 1, dtype=st), None, qt)
+  a, b = mk(lhs), mk(rhs)
+  for pref in (None, torch.bfloat16, torch.float32):
+    acc, res = qarray.get_accumulator_and_result_type(a, b, preferred_element_type=pref)
+    assert res == (pref or expect)
+  acc, _ = qarray.get_accumulator_and_result_type(mk(('int8', torch.bfloat16)), mk(('int4', torch.float32)), preferred_element_type=None)
+  assert acc == torch.int32
+
+
+def test_dispatcher_rule_and_validation():
+  q = qarray.QArray(torch.zeros(256, 8, dtype=torch.int8), torch.ones(2, 8), None, 'int8')
+  q64 = qarray.QArray(torch.zeros(256, 8, dtype=torch.int8), torch.ones(4, 8), None, 'int8')
+  lq = qarray.QArray(torch.zeros(4, 256, dtype=torch.int8), torch.ones(4, 1), None, 'int8')
+  dn = (((1,), (0,)), ((), ()))
+  assert not dg._use_fast_path(torch.zeros(4, 256, dtype=torch.bfloat16), q, dn)
+  assert dg._use_fast_path(torch.zeros(4, 256, dtype=torch.int8), q, dn)
+  assert dg._use_fast_path(lq, q, dn) and not dg._use_fast_path(lq, q64, dn)
+  with pytest.raises(ValueError, match='should be broadcastable'):
+    qarray.validate_qarray(qarray.QArray(torch.ones(10, 10, dtype=torch.int8), torch.ones(10, 3)))
+  assert qarray.get_tiled_axes(qarray.QArray(torch.ones(10, 256, 16, dtype=torch.int8), torch.ones(10, 8, 2))) == {1: 32, 2: 8}
+
+
+def test_rule_lookup_first_full_match_wins_and_op_ids():
+  rules = [qconfig.QuantizationRule(module_path='decoder/.*attn', weight_qtype='int4', tile_size=128),
+           qconfig.QuantizationRule(module_path='.*', op_names=('einsum',), weight_qtype='float8_e4m3fn'),
+           qconfig.QuantizationRule(module_path='.*', weight_qtype='int8', act_qtype='int8'),
+           qconfig.QuantizationRule(module_path='never', weight_qtype='int8')]
+  p = qconfig.QuantizationProvider(rules)
+  with qconfig.module_scope('decoder'), qconfig.module_scope('self_attn'):
+    r, op = p._get_current_rule_and_op_id('dot_general')
+    assert r.weight_qtype == 'int4' and op == 'dot_general0'
+    assert p._get_current_rule_and_op_id('dot_general')[1] == 'dot_general1'
+  with qconfig.module_scope('mlp'):
+    assert p._get_current_rule_and_op_id('einsum')[0].weight_qtype == 'float8_e4m3fn'
+    assert p._get_current_rule_and_op_id('dot_general')[0].act_qtype == 'int8'
+  assert qconfig.current_module_path() == ()
+  assert [r.module_path for r in p.get_unused_rules()] == ['never']
+  r = qconfig.QuantizationRule()
+  assert (r.module_path, r.weight_qtype, r.act_qtype, r.tile_size, r.weight_calibration_method, tuple(r.act_batch_axes)) == ('.*', None, None, None, 'absmax', (0,))
