@@ -11,7 +11,9 @@ cores, with the per-token x per-channel scale epilogue fused, bf16 out.  All lau
 the C ABI of libqwix_hip.so with preallocated buffers.
 
 Prints ONE JSON line.  `roofline` describes the dominant kernel (the MFMA GEMM): achieved =
-2*M*N*K / mean kernel time, measured with events on the launch stream inside the timed region.
+2*M*N*K / mean kernel time.  The kernel time comes from a second timed region of the same length in
+which only that kernel is launched, back to back, between two events on the launch stream: a pair of
+events around every single launch inside the step loop adds about 3 us of its own to a 10 us kernel.
 `cpu_baseline` times the NumPy oracle of the same step on a bounded sample on the host cores; it is
 a reported baseline, not a target.  `extra` carries the other workloads of the metric (quantize
 GB/s, fp8 GEMM, weight-only GEMV, Hadamard-rotated GEMM), each with its own roofline fraction.
@@ -37,8 +39,8 @@ def _events(n):
 
 
 class Workload:
-  """setup() allocates everything; step(rec) enqueues one step and may record (start, end) event pairs
-  of the dominant kernel through rec(); describe() gives the static numbers."""
+  """setup() allocates everything; step(i) enqueues step number i; kernel(i) enqueues only the dominant
+  kernel of that step on inputs a step has already produced; describe() gives the static numbers."""
 
   name = ''
   dtype = ''
@@ -47,7 +49,8 @@ class Workload:
   bound = 'mfma'
 
   def setup(self, dev): ...
-  def step(self, rec=None): ...
+  def step(self, i=0): ...
+  def kernel(self, i=0): ...
   def work_per_step(self) -> float: ...      # ops (mfma) or bytes (hbm) of the whole step's headline figure
   def kernel_work(self) -> float: ...        # algorithmic ops / bytes of ONE launch of the dominant kernel
 
@@ -68,7 +71,7 @@ class QdotW8A8(Workload):
     self.dtype = 'int8' if qtype == 'int8' else 'f8e4m3'
     self.metric = ('int8' if qtype == 'int8' else 'fp8') + ' qdot TOPS (dynamic-range w8a8, activation quantize included)'
     self.unit = 'TOPS'
-    self.kernel = 'qgemm_dma_kernel'
+    self.kernel_name = 'qgemm_dma_kernel'
 
   def setup(self, dev):
     import torch
@@ -91,17 +94,17 @@ class QdotW8A8(Workload):
     self.stream = torch.cuda.current_stream().cuda_stream
     self.L = L
 
-  def step(self, rec=None):
+  def step(self, i=0):
     L = self.L
     L.call('qwix_hip_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, 1, self.K, self.qt, L.ABSMAX, 0.0,
            L.LAYOUT_NATURAL, self.xq.data_ptr(), self.sa.data_ptr(), None, None, 0, self.stream)
-    if rec:
-      rec(0)
+    self.kernel(i)
+
+  def kernel(self, i=0):
+    L = self.L
     L.call('qwix_hip_qgemm', self.xq.data_ptr(), self.K, self.b.data_ptr(), self.K, self.qt, self.M, self.N, self.K,
            self.sa.data_ptr(), L.BF16, self.sb.data_ptr(), L.BF16, L.BF16, self.out.data_ptr(), L.BF16, self.N,
            self.stream)
-    if rec:
-      rec(1)
 
   def work_per_step(self):
     return 2.0 * self.M * self.N * self.K
@@ -150,7 +153,7 @@ class QuantizeRows(Workload):
     self.dtype = 'bf16->' + qtype
     self.metric = 'quantize GB/s (per-token absmax, bf16 -> ' + qtype + ')'
     self.unit = 'GB/s'
-    self.kernel = 'rows_kernel'
+    self.kernel_name = 'rows_kernel'
 
   def setup(self, dev):
     import torch
@@ -164,14 +167,12 @@ class QuantizeRows(Workload):
     self.stream = torch.cuda.current_stream().cuda_stream
     self.L = L
 
-  def step(self, rec=None):
+  def step(self, i=0):
     L = self.L
-    if rec:
-      rec(0)
     L.call('qwix_hip_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, 1, self.K, self.qt, L.ABSMAX, 0.0,
            L.LAYOUT_NATURAL, self.q.data_ptr(), self.s.data_ptr(), None, None, 0, self.stream)
-    if rec:
-      rec(1)
+
+  kernel = step
 
   def work_per_step(self):
     return self.M * self.K * 2.0 + self.q.numel() + self.M * 2.0
@@ -190,7 +191,7 @@ class GemvW4(Workload):
     self.dtype = 'bf16 x int4'
     self.metric = 'weight-only int4 g128 GEMV GB/s'
     self.unit = 'GB/s'
-    self.kernel = 'gemv_wq_kernel'
+    self.kernel_name = 'gemv_wq_kernel'
 
   def setup(self, dev):
     import torch
@@ -200,21 +201,25 @@ class GemvW4(Workload):
     self.x = torch.randn(self.M, self.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
     w = (torch.randn(self.K, self.N, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(dev)
     wq = qarray.quantize_api(w, 'int4', channelwise_axes=[1], tiled_axes={0: self.group}, scale_dtype=torch.float32)
-    self.b = wq.qvalue.permute(1, 0).data
-    assert self.b.is_contiguous()
-    self.s = wq.scale.contiguous()
+    b = wq.qvalue.permute(1, 0).data
+    assert b.is_contiguous()
+    s = wq.scale.contiguous()
+    # A decoder walks through a different weight matrix per layer: rotate over enough copies that a
+    # launch finds none of its weights in the 256 MB last-level cache.
+    self.copies = max(1, -(-(640 << 20) // (b.numel() * b.element_size())))
+    self.b = [b] + [b.clone() for _ in range(self.copies - 1)]
+    self.s = [s] + [s.clone() for _ in range(self.copies - 1)]
     self.out = torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev)
     self.stream = torch.cuda.current_stream().cuda_stream
     self.L = L
 
-  def step(self, rec=None):
+  def step(self, i=0):
     L = self.L
-    if rec:
-      rec(0)
-    L.call('qwix_hip_gemv_wq', self.x.data_ptr(), self.K, self.b.data_ptr(), self.K // 2, L.INT4, self.M, self.N, self.K,
-           self.group, self.s.data_ptr(), L.F32, self.out.data_ptr(), L.BF16, self.N, self.stream)
-    if rec:
-      rec(1)
+    c = i % self.copies
+    L.call('qwix_hip_gemv_wq', self.x.data_ptr(), self.K, self.b[c].data_ptr(), self.K // 2, L.INT4, self.M, self.N,
+           self.K, self.group, self.s[c].data_ptr(), L.F32, self.out.data_ptr(), L.BF16, self.N, self.stream)
+
+  kernel = step
 
   def work_per_step(self):
     return self.K * self.N / 2.0 + (self.K // self.group) * self.N * 4.0 + self.M * self.K * 2.0 + self.M * self.N * 2.0
@@ -222,7 +227,8 @@ class GemvW4(Workload):
   kernel_work = work_per_step
 
   def describe(self):
-    return {'workload': self.name, 'M': self.M, 'K': self.K, 'N': self.N, 'group': self.group}
+    return {'workload': self.name, 'M': self.M, 'K': self.K, 'N': self.N, 'group': self.group,
+            'weight_copies_rotated': self.copies}
 
 
 class HadamardQdot(Workload):
@@ -236,7 +242,7 @@ class HadamardQdot(Workload):
     self.dtype = 'int8 x int4'
     self.metric = 'Hadamard-rotated a8w4 g128 qdot TOPS (FWHT + activation quantize included)'
     self.unit = 'TOPS'
-    self.kernel = 'qgemm_grouped_kernel'
+    self.kernel_name = 'qgemm_grouped_kernel'
 
   def setup(self, dev):
     import torch
@@ -262,17 +268,17 @@ class HadamardQdot(Workload):
     self.stream = torch.cuda.current_stream().cuda_stream
     self.L = L
 
-  def step(self, rec=None):
+  def step(self, i=0):
     L = self.L
     L.call('qwix_hip_fwht_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, self.signs.data_ptr(), None, 1.0, self.K,
            L.INT8, self.xq.data_ptr(), self.sa.data_ptr(), self.stream)
-    if rec:
-      rec(0)
+    self.kernel(i)
+
+  def kernel(self, i=0):
+    L = self.L
     L.call('qwix_hip_qgemm_grouped', self.xq.data_ptr(), self.K, self.b.data_ptr(), self.K // 2, L.INT4, self.M, self.N,
            self.K, 128, self.sa.data_ptr(), L.BF16, 1, self.sb.data_ptr(), L.BF16, self.out.data_ptr(), L.BF16, self.N, 0,
            None, self.stream)
-    if rec:
-      rec(1)
 
   def work_per_step(self):
     return 2.0 * self.M * self.N * self.K
@@ -311,28 +317,29 @@ def _blas_threads() -> int:
 
 
 def run(wl: Workload, steps: int, warmup: int):
+  """Returns (seconds per step, seconds per launch of the dominant kernel)."""
   import torch
   dev = torch.device('cuda:0')
   wl.setup(dev)
-  for _ in range(warmup):
-    wl.step()
-  torch.cuda.synchronize()
-  ev = [_events(2) for _ in range(steps)]
-  cur = [0]
-
-  def rec(which):
-    ev[cur[0]][which].record()
-
+  for i in range(warmup):
+    wl.step(i)
   torch.cuda.synchronize()
   t0 = time.perf_counter()
   for i in range(steps):
-    cur[0] = i
-    wl.step(rec)
+    wl.step(i)
   torch.cuda.synchronize()
   dt = time.perf_counter() - t0
-  kt = sorted(a.elapsed_time(b) * 1e-3 for a, b in ev)
-  kmean = sum(kt) / len(kt)
-  return dt / steps, kmean, kt[len(kt) // 2]
+  # the dominant kernel alone, on the inputs the last step left behind
+  e0, e1 = _events(2)
+  for i in range(min(warmup, 3)):
+    wl.kernel(i)
+  torch.cuda.synchronize()
+  e0.record()
+  for i in range(steps):
+    wl.kernel(i)
+  e1.record()
+  torch.cuda.synchronize()
+  return dt / steps, e0.elapsed_time(e1) * 1e-3 / steps
 
 
 def summarize(wl: Workload, step_s: float, kern_s: float) -> dict:
@@ -342,7 +349,7 @@ def summarize(wl: Workload, step_s: float, kern_s: float) -> dict:
   achieved = wl.kernel_work() / kern_s / scale
   return {
       'value': round(value, 2), 'unit': wl.unit, 'ms_per_step': round(step_s * 1e3, 5),
-      'roofline': {'bound': wl.bound, 'kernel': wl.kernel, 'achieved': round(achieved, 2), 'peak': peak,
+      'roofline': {'bound': wl.bound, 'kernel': wl.kernel_name, 'achieved': round(achieved, 2), 'peak': peak,
                    'unit': 'TFLOP/s' if wl.bound == 'mfma' else 'GB/s', 'frac': round(achieved / peak, 4),
                    'traffic': _traffic(wl.name)},
   }
@@ -378,7 +385,7 @@ def main():
     sys.exit(2)
 
   wl = WORKLOADS[args.workload]()
-  step_s, kmean, _ = run(wl, args.steps, args.warmup)
+  step_s, kmean = run(wl, args.steps, args.warmup)
   res = summarize(wl, step_s, kmean)
   line = {
       'metric': wl.metric, 'value': res['value'], 'unit': res['unit'], 'n_gpus': 1, 'steps': args.steps,
@@ -395,7 +402,7 @@ def main():
     for name in EXTRA:
       w = WORKLOADS[name]()
       n = max(5, min(args.steps, 20))
-      s, km, _ = run(w, n, 3)
+      s, km = run(w, n, 3)
       r = summarize(w, s, km)
       extra[name] = {'metric': w.metric, 'value': r['value'], 'unit': r['unit'], 'ms_per_step': r['ms_per_step'],
                      'roofline': r['roofline']}

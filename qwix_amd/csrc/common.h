@@ -157,7 +157,8 @@ __device__ __forceinline__ float apply_factor(float v, float factor) {
 // it lies exactly on one, in which case it is representable in f32 and the residual step below
 // reproduces it exactly.  Hence one reciprocal + one Newton step gives RNE_bf16(RNE_f32(x/s)).
 // kSafe=false is for quotients known to be bounded (dynamic range: |x| <= absmax).
-template <typename D, bool kSafe = true>
+// kSignedZero keeps the sign of a zero quotient (matters for e4m3's -0 only).
+template <typename D, bool kSafe = true, bool kSignedZero = true>
 struct Divider {
   float s, r;
   __device__ __forceinline__ explicit Divider(float scale) : s(scale) {
@@ -172,7 +173,8 @@ struct Divider {
       if constexpr (kSafe)
         if (!(__builtin_fabsf(q0) < 0x1p100f)) q1 = x / s;
       // The residual step turns -0 into +0; the quotient always carries the sign of x (s > 0).
-      return __builtin_copysignf(round_bf16(q1), x);
+      if constexpr (kSignedZero) return __builtin_copysignf(round_bf16(q1), x);
+      return round_bf16(q1);
     } else {
       return x / s;
     }
@@ -195,6 +197,16 @@ __device__ __forceinline__ float wave_xor_min(float v, int width) {
 // NaN-propagating max of |x|: fmaxf drops NaNs, so track them separately where it matters.
 __device__ __forceinline__ float absmax_acc(float acc, float x) {
   return fmaxf(acc, __builtin_fabsf(x));
+}
+
+// Saturating round-half-even to a small integer in two float ops: clamp to [lo, hi] (one v_med3,
+// +-inf included), then add 1.5 * 2^23: the add rounds to the nearest (even) integer and leaves its
+// two's complement in the low mantissa bits.  NaN is not mapped to 0 here (unpinned either way).
+__device__ __forceinline__ uint32_t rne_bits_clamped(float v, float lo, float hi) {
+  return __float_as_uint(__builtin_amdgcn_fmed3f(v, lo, hi) + 12582912.0f);
+}
+__device__ __forceinline__ uint32_t pack4_low_bytes(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  return __builtin_amdgcn_perm(b, a, 0x0c0c0400u) | __builtin_amdgcn_perm(d, c, 0x04000c0cu);
 }
 
 // pack helpers

@@ -4,13 +4,14 @@
 //
 // HBM-bound: the weight bytes are read exactly once, the activations stay in L2.  Even at M = 16
 // the multiply-adds exceed what the vector ALUs can do in the time the weights stream in, so the
-// products run on v_mfma_f32_16x16x32_bf16 with the weights converted to bf16 in registers:
-//   int4: (nibble ^ 8) is OR-ed into the mantissa of bf16 128.0, giving 128 + (q + 8) exactly in
-//         two bit-ops per pair; the offset is removed after the MFMA with the row sums of x, which
-//         a second MFMA against an all-ones operand produces in the accumulator's own layout;
-//   int8: sign-extend, convert, pack.
-// A workgroup is 4 wavefronts that split K; each handles NT tiles of 16 output columns and the
-// four partial sums meet in LDS.
+// products run on v_mfma_f32_16x16x32_bf16 with the weights converted to bf16 in registers, in
+// offset binary so that the conversion is one or two bit-ops per pair of weights:
+//   int4: (nibble ^ 8) lands in the mantissa of bf16 128.0, giving 128 + (q + 8) exactly;
+//   int8: (byte ^ 0x80) is converted with v_cvt_f32_ubyte and truncated to bf16 (exact below 256).
+// The offset is removed by seeding each accumulator with -offset * rowsum(x), which four MFMAs against
+// a constant operand produce in the accumulator's own layout.
+// A workgroup is 16 wavefronts that split K; each handles NT tiles of 16 output columns with two K
+// blocks of loads in flight, and the partial sums meet in LDS.
 #include "common.h"
 
 namespace qwix {
@@ -20,109 +21,160 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
-constexpr int NT = 2;
 
 struct GemvArgs {
   const uint16_t* x; int64_t ldx;
   const uint8_t* q; int64_t ldb;
-  int M, N, K, group;
+  int M, N, K;
+  int bpg;         // 128-wide K blocks per scale group
+  uint64_t magic;  // ceil(2^32 / bpg): kb / bpg == (kb * magic) >> 32 while kb * bpg < 2^32
   const void* s; int s_dtype;
   void* out; int out_dtype; int64_t ldo;
 };
 
 __device__ __forceinline__ bf16x8 as_bf16x8(v4u v) { return __builtin_bit_cast(bf16x8, v); }
 
-template <int BQT>
-__global__ void __launch_bounds__(256) gemv_wq_kernel(GemvArgs p) {
+// Everything one wavefront needs for one 128-wide K block: its 4 activation fragments, and per
+// column tile the packed weights and the scale.
+template <int BQT, int NT>
+struct Block {
+  v4u xf[4];
+  v4u wq[NT][BQT == QWIX_INT4 ? 1 : 2];
+  unsigned sraw[NT];  // scale bits as loaded: bf16 in the low half, or f32
+};
+
+// Addresses are a wave-uniform 64-bit base plus a per-lane unsigned 32-bit byte offset that is fixed
+// for the whole kernel, so that a load costs no vector arithmetic.  Columns beyond N are clamped to
+// the last valid one instead of being predicated: an output element depends only on its own row of
+// x and its own column of the weights, and the clamped ones are never stored.
+template <int NT>
+struct LaneOff {
+  unsigned x;      // bytes from the first row of this workgroup's 16 rows of x
+  unsigned w[NT];  // bytes from row n_base of the weights
+  unsigned s[NT];  // elements from column n_base of the scales
+};
+
+template <int BQT, int NT, bool SBF>
+__device__ __forceinline__ void load_block(const GemvArgs& p, const LaneOff<NT>& a, bool xrow, int row0, int n_base,
+                                           int kb, Block<BQT, NT>* b) {
   constexpr bool W4 = (BQT == QWIX_INT4);
-  __shared__ float red[4][NT][4][64];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const char* xb = reinterpret_cast<const char*>(p.x + static_cast<int64_t>(row0) * p.ldx + kb * 128);
+  // every vector load occupies the texture path for as long as its active lanes need, also when they
+  // repeat an address: lanes whose row of x does not exist stay idle and feed zeros to the MFMA
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    b->xf[j] = v4u{0, 0, 0, 0};
+    if (xrow) b->xf[j] = *reinterpret_cast<const v4u*>(xb + a.x + j * 16);
+  }
+  const int sg = static_cast<int>((static_cast<uint64_t>(static_cast<unsigned>(kb)) * p.magic) >> 32);
+  const int64_t s0 = static_cast<int64_t>(sg) * p.N + n_base;
+  const uint8_t* wb = p.q + static_cast<int64_t>(n_base) * p.ldb + kb * (W4 ? 64 : 128);
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    b->wq[t][0] = *reinterpret_cast<const v4u*>(wb + a.w[t]);
+    if constexpr (!W4) b->wq[t][1] = *reinterpret_cast<const v4u*>(wb + a.w[t] + 16);
+    if constexpr (SBF)
+      b->sraw[t] = (reinterpret_cast<const uint16_t*>(p.s) + s0)[a.s[t]];
+    else
+      b->sraw[t] = (reinterpret_cast<const unsigned*>(p.s) + s0)[a.s[t]];
+  }
+}
+
+// Weights enter the MFMA in offset binary (int4: 128 + (q + 8), int8: q + 128, both exact in bf16);
+// the offset times the row sum of x is taken out by four MFMAs against the constant -offset, whose
+// result seeds the accumulator of every column tile.
+template <int BQT, int NT, bool SBF>
+__device__ __forceinline__ void compute_block(const Block<BQT, NT>& b, v4f (&outacc)[NT]) {
+  constexpr bool W4 = (BQT == QWIX_INT4);
+  constexpr unsigned kNegOff = W4 ? 0xC308C308u : 0xC300C300u;  // bf16 -136 / -128, twice
+  const v4u negoff = {kNegOff, kNegOff, kNegOff, kNegOff};
+  v4u xf[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if constexpr (W4) {  // element order (k0,k4,k1,k5,k2,k6,k3,k7): what the nibble widening yields
+      const v4u d = b.xf[j];
+      xf[j][0] = __builtin_amdgcn_perm(d[2], d[0], 0x05040100);
+      xf[j][1] = __builtin_amdgcn_perm(d[2], d[0], 0x07060302);
+      xf[j][2] = __builtin_amdgcn_perm(d[3], d[1], 0x05040100);
+      xf[j][3] = __builtin_amdgcn_perm(d[3], d[1], 0x07060302);
+    } else {
+      xf[j] = b.xf[j];
+    }
+  }
+  v4f base = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    base = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[j]), as_bf16x8(negoff), base, 0, 0, 0);
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    v4f acc = base;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v4u w;
+      if constexpr (W4) {
+        // (u & 0x000F000F) ^ 0x43084308: flips the nibble's sign bit and drops it into the mantissa of
+        // bf16 128.0, one three-input bit-op per pair of weights
+        const unsigned u = b.wq[t][0][j];
+        w[0] = (u & 0x000F000Fu) ^ 0x43084308u;          // (k0, k4)
+        w[1] = ((u >> 4) & 0x000F000Fu) ^ 0x43084308u;   // (k1, k5)
+        w[2] = ((u >> 8) & 0x000F000Fu) ^ 0x43084308u;   // (k2, k6)
+        w[3] = ((u >> 12) & 0x000F000Fu) ^ 0x43084308u;  // (k3, k7)
+      } else {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const unsigned u = b.wq[t][j >> 1][2 * (j & 1) + h] ^ 0x80808080u;
+          // integers up to 255 have 8 significant bits: the upper half of their f32 is their bf16
+          const unsigned f0 = __float_as_uint(static_cast<float>(u & 0xFFu));
+          const unsigned f1 = __float_as_uint(static_cast<float>((u >> 8) & 0xFFu));
+          const unsigned f2 = __float_as_uint(static_cast<float>((u >> 16) & 0xFFu));
+          const unsigned f3 = __float_as_uint(static_cast<float>(u >> 24));
+          w[2 * h] = __builtin_amdgcn_perm(f1, f0, 0x07060302);
+          w[2 * h + 1] = __builtin_amdgcn_perm(f3, f2, 0x07060302);
+        }
+      }
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[j]), as_bf16x8(w), acc, 0, 0, 0);
+    }
+    const float sc = __uint_as_float(SBF ? b.sraw[t] << 16 : b.sraw[t]);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) outacc[t][r] = fmaf(acc[r], sc, outacc[t][r]);
+  }
+}
+
+// NWAVE wavefronts per workgroup, each owning a slice of K; NT tiles of 16 output columns.
+template <int BQT, int NWAVE, int NT, bool SBF>
+__global__ void __launch_bounds__(NWAVE * 64) gemv_wq_kernel(GemvArgs p) {
+  __shared__ float red[NWAVE][NT][4][64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, kq = lane >> 4;
   const int n_base = blockIdx.x * (16 * NT);
-  const int m = blockIdx.y * 16 + col;  // row of x this lane feeds to the MFMA
   const int nblk = p.K / 128;
-  const int per_wave = (nblk + 3) / 4;
+  const int per_wave = (nblk + NWAVE - 1) / NWAVE;
   const int kb0 = wave * per_wave, kb1 = min(nblk, kb0 + per_wave);
+
+  const int row0 = blockIdx.y * 16;
+  LaneOff<NT> a;
+  const bool xrow = row0 + col < p.M;
+  a.x = static_cast<unsigned>(col) * static_cast<unsigned>(p.ldx) * 2u + kq * 64u;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    a.s[t] = static_cast<unsigned>(min(t * 16 + col, p.N - 1 - n_base));
+    a.w[t] = a.s[t] * static_cast<unsigned>(p.ldb) + kq * (BQT == QWIX_INT4 ? 16u : 32u);
+  }
 
   v4f outacc[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) outacc[t] = v4f{0.f, 0.f, 0.f, 0.f};
-  const v4u ones_u = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
 
-  for (int kb = kb0; kb < kb1; ++kb) {
-    const int k0 = kb * 128 + kq * 32;
-    // Four activation fragments of 8 consecutive k each.
-    v4u xf[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      xf[j] = v4u{0, 0, 0, 0};
-      if (m < p.M) xf[j] = *reinterpret_cast<const v4u*>(p.x + static_cast<int64_t>(m) * p.ldx + k0 + j * 8);
-      if constexpr (W4) {  // element order (k0,k4,k1,k5,k2,k6,k3,k7): what the nibble widening yields
-        const v4u d = xf[j];
-        xf[j][0] = __builtin_amdgcn_perm(d[2], d[0], 0x05040100);
-        xf[j][1] = __builtin_amdgcn_perm(d[2], d[0], 0x07060302);
-        xf[j][2] = __builtin_amdgcn_perm(d[3], d[1], 0x05040100);
-        xf[j][3] = __builtin_amdgcn_perm(d[3], d[1], 0x07060302);
-      }
-    }
-    v4f rowsum = {0.f, 0.f, 0.f, 0.f};
-    if constexpr (W4) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        rowsum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[j]), as_bf16x8(ones_u), rowsum, 0, 0, 0);
-    }
-    const int sg = (kb * 128) / p.group;
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const int n = n_base + t * 16 + col;
-      v4f acc = {0.f, 0.f, 0.f, 0.f};
-      float sc = 0.f;
-      if (n < p.N) {
-        sc = p.s_dtype == QWIX_BF16
-                 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.s)[static_cast<int64_t>(sg) * p.N + n])
-                 : reinterpret_cast<const float*>(p.s)[static_cast<int64_t>(sg) * p.N + n];
-      }
-      if constexpr (W4) {
-        v4u pk = {0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};  // zeros in two's complement
-        if (n < p.N) pk = *reinterpret_cast<const v4u*>(p.q + static_cast<int64_t>(n) * p.ldb + k0 / 2);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const unsigned u = pk[j] ^ 0x88888888u;  // offset binary: nibble = q + 8
-          v4u w;
-          w[0] = (u & 0x000F000Fu) | 0x43004300u;          // (k0, k4) as bf16 128 + nibble
-          w[1] = ((u >> 4) & 0x000F000Fu) | 0x43004300u;   // (k1, k5)
-          w[2] = ((u >> 8) & 0x000F000Fu) | 0x43004300u;   // (k2, k6)
-          w[3] = ((u >> 12) & 0x000F000Fu) | 0x43004300u;  // (k3, k7)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[j]), as_bf16x8(w), acc, 0, 0, 0);
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) outacc[t][r] += (acc[r] - 136.f * rowsum[r]) * sc;
-      } else {
-        v4u lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
-        if (n < p.N) {
-          lo = *reinterpret_cast<const v4u*>(p.q + static_cast<int64_t>(n) * p.ldb + k0);
-          hi = *reinterpret_cast<const v4u*>(p.q + static_cast<int64_t>(n) * p.ldb + k0 + 16);
-        }
-        const unsigned words[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          v4u w;
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            const unsigned d = words[2 * j + h];
-            const float f0 = static_cast<float>(static_cast<int>(d << 24) >> 24);
-            const float f1 = static_cast<float>(static_cast<int>(d << 16) >> 24);
-            const float f2 = static_cast<float>(static_cast<int>(d << 8) >> 24);
-            const float f3 = static_cast<float>(static_cast<int>(d) >> 24);
-            w[2 * h] = f32_to_bf16_bits(f0) | (static_cast<unsigned>(f32_to_bf16_bits(f1)) << 16);
-            w[2 * h + 1] = f32_to_bf16_bits(f2) | (static_cast<unsigned>(f32_to_bf16_bits(f3)) << 16);
-          }
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[j]), as_bf16x8(w), acc, 0, 0, 0);
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) outacc[t][r] += acc[r] * sc;
-      }
-    }
+  // Two K blocks per trip, all their loads issued before the first is consumed.  Nothing loaded is
+  // carried from one trip to the next; the other wavefronts of the SIMD cover the gap.
+  for (int kb = kb0; kb < kb1; kb += 2) {
+    Block<BQT, NT> b0, b1;
+    const bool two = kb + 1 < kb1;
+    load_block<BQT, NT, SBF>(p, a, xrow, row0, n_base, kb, &b0);
+    if (two) load_block<BQT, NT, SBF>(p, a, xrow, row0, n_base, kb + 1, &b1);
+    compute_block<BQT, NT, SBF>(b0, outacc);
+    if (two) compute_block<BQT, NT, SBF>(b1, outacc);
   }
 
 #pragma unroll
@@ -131,9 +183,11 @@ __global__ void __launch_bounds__(256) gemv_wq_kernel(GemvArgs p) {
     for (int r = 0; r < 4; ++r) red[wave][t][r][lane] = outacc[t][r];
   __syncthreads();
   // result lane layout: column n = lane % 16, row m = 4 * (lane / 16) + r
-  for (int idx = tid; idx < NT * 256; idx += 256) {
+  for (int idx = tid; idx < NT * 256; idx += NWAVE * 64) {
     const int t = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
-    const float v = red[0][t][r][l] + red[1][t][r][l] + red[2][t][r][l] + red[3][t][r][l];
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < NWAVE; ++w) v += red[w][t][r][l];
     const int mo = blockIdx.y * 16 + 4 * (l >> 4) + r, n = n_base + t * 16 + (l & 15);
     if (mo < p.M && n < p.N) {
       if (p.out_dtype == QWIX_BF16)
@@ -165,17 +219,37 @@ extern "C" int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64
     return fail(QWIX_ERR_UNSUPPORTED, "x rows and weight rows must be 16-byte aligned");
   auto ok = [](int d) { return d == QWIX_F32 || d == QWIX_BF16; };
   if (!ok(s_dtype) || !ok(out_dtype) || ldo < N) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad scale/output description");
+  if (16 * ldx * 2 > INT32_MAX || 64 * ldb_bytes > INT32_MAX)
+    return fail(QWIX_ERR_UNSUPPORTED, "row strides too large for 32-bit lane offsets");
   GemvArgs p;
   p.x = static_cast<const uint16_t*>(x); p.ldx = ldx;
   p.q = static_cast<const uint8_t*>(q); p.ldb = ldb_bytes;
-  p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(K); p.group = static_cast<int>(group);
+  p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(K);
+  p.bpg = static_cast<int>(group / 128);
+  p.magic = (0x100000000ull + p.bpg - 1) / p.bpg;
   p.s = s; p.s_dtype = s_dtype;
   p.out = out; p.out_dtype = out_dtype; p.ldo = ldo;
-  const dim3 grid(static_cast<unsigned>((N + 16 * NT - 1) / (16 * NT)), static_cast<unsigned>((M + 15) / 16));
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (b_qtype == QWIX_INT4)
-    gemv_wq_kernel<QWIX_INT4><<<grid, 256, 0, st>>>(p);
+#define QWIX_GEMV_LAUNCH(NW, NTT)                                                                          \
+  do {                                                                                                     \
+    const dim3 grid(static_cast<unsigned>((N + 16 * NTT - 1) / (16 * NTT)), static_cast<unsigned>((M + 15) / 16)); \
+    if (b_qtype == QWIX_INT4 && s_dtype == QWIX_BF16)                                                      \
+      gemv_wq_kernel<QWIX_INT4, NW, NTT, true><<<grid, NW * 64, 0, st>>>(p);                               \
+    else if (b_qtype == QWIX_INT4)                                                                         \
+      gemv_wq_kernel<QWIX_INT4, NW, NTT, false><<<grid, NW * 64, 0, st>>>(p);                              \
+    else if (s_dtype == QWIX_BF16)                                                                         \
+      gemv_wq_kernel<QWIX_INT8, NW, NTT, true><<<grid, NW * 64, 0, st>>>(p);                               \
+    else                                                                                                   \
+      gemv_wq_kernel<QWIX_INT8, NW, NTT, false><<<grid, NW * 64, 0, st>>>(p);                              \
+  } while (0)
+  // Wider column tiles reuse each activation fragment more often; narrower ones keep every CU busy
+  // when the weight matrix has few columns.
+  if (N >= 192 * 64)
+    QWIX_GEMV_LAUNCH(16, 4);
+  else if (N >= 192 * 32)
+    QWIX_GEMV_LAUNCH(16, 2);
   else
-    gemv_wq_kernel<QWIX_INT8><<<grid, 256, 0, st>>>(p);
+    QWIX_GEMV_LAUNCH(16, 1);
+#undef QWIX_GEMV_LAUNCH
   return check_launch("gemv_wq");
 }

@@ -10,6 +10,8 @@
 //           and merges panels with a 32-bit atomic max into a caller-provided workspace; pass 2
 //           re-reads each panel, quantizes it, and writes either the natural layout or the
 //           reduce-minor (transposed) layout the GEMM kernels consume.
+#include <cstdlib>
+
 #include "common.h"
 
 namespace qwix {
@@ -17,15 +19,21 @@ namespace {
 
 enum { MODE_QUANT = 0, MODE_CALIB = 1, MODE_GIVEN = 2 };
 
-// Quantize N consecutive values (already divided / shifted) and store them packed.
-template <int QT, int N>
+// Quantize N consecutive values (already divided / shifted) and store them packed.  BOUNDED selects
+// the two-op clamp-and-round converter (vector paths); the scalar paths keep NaN -> 0.
+template <int QT, int N, bool BOUNDED = false>
 __device__ __forceinline__ void store_q(const float* v, uint8_t* q, int64_t elem) {
   if constexpr (QT == QWIX_INT8) {
     uint32_t w[N / 4];
 #pragma unroll
-    for (int i = 0; i < N / 4; ++i)
-      w[i] = pack4_i8(to_int_q<QT>(v[4 * i]), to_int_q<QT>(v[4 * i + 1]), to_int_q<QT>(v[4 * i + 2]),
-                      to_int_q<QT>(v[4 * i + 3]));
+    for (int i = 0; i < N / 4; ++i) {
+      if constexpr (BOUNDED)
+        w[i] = pack4_low_bytes(rne_bits_clamped(v[4 * i], -128.f, 127.f), rne_bits_clamped(v[4 * i + 1], -128.f, 127.f),
+                               rne_bits_clamped(v[4 * i + 2], -128.f, 127.f), rne_bits_clamped(v[4 * i + 3], -128.f, 127.f));
+      else
+        w[i] = pack4_i8(to_int_q<QT>(v[4 * i]), to_int_q<QT>(v[4 * i + 1]), to_int_q<QT>(v[4 * i + 2]),
+                        to_int_q<QT>(v[4 * i + 3]));
+    }
     if constexpr (N == 8)
       *reinterpret_cast<uint2*>(q + elem) = make_uint2(w[0], w[1]);
     else
@@ -42,7 +50,12 @@ __device__ __forceinline__ void store_q(const float* v, uint8_t* q, int64_t elem
   } else {  // INT4: element `elem` is even; low nibble = even element.
     uint32_t w = 0;
 #pragma unroll
-    for (int i = 0; i < N; ++i) w |= static_cast<uint32_t>(to_int_q<QT>(v[i]) & 0xF) << (4 * i);
+    for (int i = 0; i < N; ++i) {
+      if constexpr (BOUNDED)
+        w |= (rne_bits_clamped(v[i], -8.f, 7.f) & 0xFu) << (4 * i);
+      else
+        w |= static_cast<uint32_t>(to_int_q<QT>(v[i]) & 0xF) << (4 * i);
+    }
     if constexpr (N == 8)
       *reinterpret_cast<uint32_t*>(q + elem / 2) = w;
     else
@@ -59,15 +72,19 @@ __device__ __forceinline__ uint8_t q_byte(float v) {  // one value -> one byte (
 }
 
 // ------------------------------------------------------------------------------------ rows
-// nseg segments of L = nvec * kVec contiguous elements.  log2g: threads per segment.
-template <typename D, int QT, int CAL, int MODE>
+// nseg segments of L = nvec * kVec contiguous elements.  log2g: threads per segment; NL: 16-byte
+// loads per thread.  The segment stays in registers in its packed form between the reduction and the
+// quantization (the empty asm keeps the compiler from re-issuing the loads instead), so HBM is read
+// exactly once.  bf16 absmax runs on the packed halves: |x| ordered like its 15 low bits.
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+template <typename D, int QT, int CAL, int MODE, int NL>
 __global__ void __launch_bounds__(256)
     rows_kernel(const uint8_t* __restrict__ x, int64_t nseg, int nvec, int log2g, float factor,
                 uint8_t* __restrict__ q, void* __restrict__ scale, int8_t* __restrict__ zp,
                 void* __restrict__ cal0, void* __restrict__ cal1) {
   constexpr int EV = D::kVec;
   constexpr bool ASYM = (CAL == QWIX_MINMAX);
-  constexpr int NL = 8;
   __shared__ float red[2][4];
   const int tid = threadIdx.x;
   const int g = 1 << log2g;
@@ -76,33 +93,45 @@ __global__ void __launch_bounds__(256)
   const bool seg_ok = seg < nseg;
   const uint4* xv = reinterpret_cast<const uint4*>(x) + seg * nvec;
 
-  float f[NL][EV];
+  uint4 raw[NL];
 #pragma unroll
   for (int j = 0; j < NL; ++j) {
     const int v = lane + (j << log2g);
-    if (seg_ok && v < nvec) {
-      unpack16<D>(xv[v], f[j]);
-    } else {
-#pragma unroll
-      for (int e = 0; e < EV; ++e) f[j][e] = 0.f;
-    }
+    raw[j] = make_uint4(0, 0, 0, 0);
+    if (seg_ok && v < nvec) raw[j] = xv[v];
   }
+#pragma unroll
+  for (int j = 0; j < NL; ++j) asm volatile("" : "+v"(raw[j].x), "+v"(raw[j].y), "+v"(raw[j].z), "+v"(raw[j].w));
 
   float s = 1.f;
   int z = 0;
   if constexpr (MODE != MODE_GIVEN) {
     float mx = 0.f, mn = 0.f;  // minmax clips to include 0; absmax >= 0
+    if constexpr (!ASYM && D::kTag == QWIX_BF16) {
+      u16x2 m = {0, 0};
 #pragma unroll
-    for (int j = 0; j < NL; ++j)
+      for (int j = 0; j < NL; ++j) {
+        const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
 #pragma unroll
-      for (int e = 0; e < EV; ++e) {
-        if constexpr (ASYM) {
-          mx = fmaxf(mx, f[j][e]);
-          mn = fminf(mn, f[j][e]);
-        } else {
-          mx = absmax_acc(mx, f[j][e]);
+        for (int e = 0; e < 4; ++e) m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2, w[e] & 0x7FFF7FFFu));
+      }
+      mx = bf16_bits_to_f32(m[0] > m[1] ? m[0] : m[1]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < NL; ++j) {
+        float f[EV];
+        unpack16<D>(raw[j], f);
+#pragma unroll
+        for (int e = 0; e < EV; ++e) {
+          if constexpr (ASYM) {
+            mx = fmaxf(mx, f[e]);
+            mn = fminf(mn, f[e]);
+          } else {
+            mx = absmax_acc(mx, f[e]);
+          }
         }
       }
+    }
     mx = wave_xor_max(mx, g < 64 ? g : 64);
     if constexpr (ASYM) mn = wave_xor_min(mn, g < 64 ? g : 64);
     if (g > 64) {  // uniform branch: segments span 2 or 4 waves
@@ -148,19 +177,20 @@ __global__ void __launch_bounds__(256)
     }
   }
 
-  const Divider<D, MODE == MODE_GIVEN> div(s);
+  const Divider<D, MODE == MODE_GIVEN, QT == QWIX_E4M3> div(s);
   const float zf = static_cast<float>(z);
 #pragma unroll
   for (int j = 0; j < NL; ++j) {
     const int v = lane + (j << log2g);
     if (seg_ok && v < nvec) {
       float t[EV];
+      unpack16<D>(raw[j], t);
 #pragma unroll
       for (int e = 0; e < EV; ++e) {
-        t[e] = div(f[j][e]);
+        t[e] = div(t[e]);
         if constexpr (ASYM) t[e] = rnd<D>(t[e] + zf);
       }
-      store_q<QT, EV>(t, q, (seg * nvec + v) * EV);
+      store_q<QT, EV, true>(t, q, (seg * nvec + v) * EV);
     }
   }
 }
@@ -401,7 +431,7 @@ __global__ void __launch_bounds__(256)
   }
 #pragma unroll
   for (int e = 0; e < EV; ++e) {
-    const Divider<D, SRC == 1> div(s[e]);
+    const Divider<D, SRC == 1, QT == QWIX_E4M3> div(s[e]);
     const float zf = static_cast<float>(z[e]);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -409,10 +439,11 @@ __global__ void __launch_bounds__(256)
       if constexpr (ASYM) v[j][e] = rnd<D>(v[j][e] + zf);
     }
   }
+  constexpr bool kBounded = true;
   if constexpr (LAYOUT == QWIX_LAYOUT_NATURAL) {
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-      if (r0 + j < row_end) store_q<QT, EV>(v[j], q, (o * gm.reduce + r0 + j) * gm.inner + c0);
+      if (r0 + j < row_end) store_q<QT, EV, kBounded>(v[j], q, (o * gm.reduce + r0 + j) * gm.inner + c0);
   } else {  // (outer, inner, reduce): 8 consecutive rows of one column are 8 consecutive bytes
     const bool full = r0 + 8 <= row_end;
 #pragma unroll
@@ -422,7 +453,7 @@ __global__ void __launch_bounds__(256)
         float col[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) col[j] = v[j][e];
-        store_q<QT, 8>(col, q, el);
+        store_q<QT, 8, kBounded>(col, q, el);
       } else if constexpr (QT == QWIX_INT4) {
         for (int j = 0; j + 1 < 8 && r0 + j + 1 < row_end; j += 2)
           q[(el + j) >> 1] = static_cast<uint8_t>(pack2_i4(to_int_q<QT>(v[j][e]), to_int_q<QT>(v[j + 1][e])));
@@ -639,12 +670,22 @@ int run_rows(const void* x, int dtype, int64_t nseg, int64_t L, int qtype, int c
                           (MODE == MODE_CALIB || (reinterpret_cast<uintptr_t>(q) & 7) == 0);
       if (vec_ok) {
         const int nvec = static_cast<int>(L / D::kVec);
-        int lg = log2_ceil((nvec + 3) / 4);  // aim at <= 4 loads per thread, 8 at most
+        static const int target = [] { const char* e = getenv("QWIX_ROWS_LOADS"); return e ? atoi(e) : 4; }();
+        int lg = log2_ceil((nvec + target - 1) / target);  // aim at `target` loads per thread, 8 at most
+        while ((nvec + (1 << lg) - 1) >> lg > 8) ++lg;
         if (lg > 8) lg = 8;
         const int64_t blocks = (nseg + (256 >> lg) - 1) / (256 >> lg);
-        rows_kernel<D, QT, CAL, MODE><<<dim3(static_cast<unsigned>(blocks)), 256, 0, st>>>(
-            static_cast<const uint8_t*>(x), nseg, nvec, lg, factor, static_cast<uint8_t*>(q), scale,
-            static_cast<int8_t*>(zp), c0, c1);
+        const int loads = (nvec + (1 << lg) - 1) >> lg;
+        const dim3 grid(static_cast<unsigned>(blocks));
+        const uint8_t* xb = static_cast<const uint8_t*>(x);
+        uint8_t* qb = static_cast<uint8_t*>(q);
+        int8_t* zb = static_cast<int8_t*>(zp);
+        if (loads <= 2)
+          rows_kernel<D, QT, CAL, MODE, 2><<<grid, 256, 0, st>>>(xb, nseg, nvec, lg, factor, qb, scale, zb, c0, c1);
+        else if (loads <= 4)
+          rows_kernel<D, QT, CAL, MODE, 4><<<grid, 256, 0, st>>>(xb, nseg, nvec, lg, factor, qb, scale, zb, c0, c1);
+        else
+          rows_kernel<D, QT, CAL, MODE, 8><<<grid, 256, 0, st>>>(xb, nseg, nvec, lg, factor, qb, scale, zb, c0, c1);
       } else {
         if (QT == QWIX_INT4 && MODE != MODE_CALIB && (L & 1))
           return fail(QWIX_ERR_UNSUPPORTED, "int4 needs an even contiguous length, got %lld", (long long)L);
