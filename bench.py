@@ -183,6 +183,37 @@ class QuantizeRows(Workload):
     return {'workload': self.name, 'M': self.M, 'K': self.K}
 
 
+class PlainCopy(Workload):
+  """A device-to-device copy of known size: the yardstick the HBM counters are scaled by."""
+
+  bound = 'hbm'
+
+  def __init__(self, name, nbytes):
+    self.name, self.nbytes = name, nbytes
+    self.dtype = 'u8'
+    self.metric = 'plain copy GB/s (read + write)'
+    self.unit = 'GB/s'
+    self.kernel_name = 'torch copy_'
+
+  def setup(self, dev):
+    import torch
+    self.src = torch.randint(0, 255, (self.nbytes,), dtype=torch.uint8, device=dev)
+    self.dst = torch.empty_like(self.src)
+
+  def step(self, i=0):
+    self.dst.copy_(self.src)
+
+  kernel = step
+
+  def work_per_step(self):
+    return 2.0 * self.nbytes
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'bytes_read': self.nbytes, 'bytes_written': self.nbytes}
+
+
 class GemvW4(Workload):
   bound = 'hbm'
 
@@ -298,6 +329,7 @@ WORKLOADS = {
     'quantize_act_8192_fp8': lambda: QuantizeRows('quantize_act_8192_fp8', 8192, 8192, 'float8_e4m3fn'),
     'c2_gemv_w4_m1': lambda: GemvW4('c2_gemv_w4_m1', 1, 4096, 14336, 128),
     'c2_gemv_w4_m16': lambda: GemvW4('c2_gemv_w4_m16', 16, 4096, 14336, 128),
+    'plain_copy_1g': lambda: PlainCopy('plain_copy_1g', 1 << 30),
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
 }
 DEFAULT = 'c3_int8_w8a8_4096'
