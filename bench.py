@@ -183,6 +183,46 @@ class QuantizeRows(Workload):
     return {'workload': self.name, 'M': self.M, 'K': self.K}
 
 
+class FwhtQuantize(Workload):
+  """C5 activations: Walsh-Hadamard rotation along K fused with per-token int8 quantization."""
+
+  bound = 'hbm'
+
+  def __init__(self, name, M, K):
+    self.name, self.M, self.K = name, M, K
+    self.dtype = 'bf16->int8'
+    self.metric = 'Hadamard rotate + quantize GB/s (per-token absmax, bf16 -> int8)'
+    self.unit = 'GB/s'
+    self.kernel_name = 'fwht_reg_kernel'
+
+  def setup(self, dev):
+    import torch
+    from qwix_amd.contrib import hadamard_rot as hr
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(5001)
+    self.x = torch.randn(self.M, self.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    self.signs = hr.random_signs(g, self.K, torch.bfloat16, dev)
+    self.q = torch.empty(self.M, self.K, dtype=torch.int8, device=dev)
+    self.s = torch.empty(self.M, dtype=torch.bfloat16, device=dev)
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, i=0):
+    L = self.L
+    L.call('qwix_hip_fwht_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, self.signs.data_ptr(), None, 1.0, self.K,
+           L.INT8, self.q.data_ptr(), self.s.data_ptr(), self.stream)
+
+  kernel = step
+
+  def work_per_step(self):
+    return self.M * self.K * 3.0 + self.M * 2.0
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'M': self.M, 'K': self.K}
+
+
 class PlainCopy(Workload):
   """A device-to-device copy of known size: the yardstick the HBM counters are scaled by."""
 
@@ -329,12 +369,14 @@ WORKLOADS = {
     'quantize_act_8192_fp8': lambda: QuantizeRows('quantize_act_8192_fp8', 8192, 8192, 'float8_e4m3fn'),
     'c2_gemv_w4_m1': lambda: GemvW4('c2_gemv_w4_m1', 1, 4096, 14336, 128),
     'c2_gemv_w4_m16': lambda: GemvW4('c2_gemv_w4_m16', 16, 4096, 14336, 128),
+    'c5_fwht_quantize_act': lambda: FwhtQuantize('c5_fwht_quantize_act', 2048, 8192),
+    'fwht_quantize_8192x8192': lambda: FwhtQuantize('fwht_quantize_8192x8192', 8192, 8192),
     'plain_copy_1g': lambda: PlainCopy('plain_copy_1g', 1 << 30),
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
 }
 DEFAULT = 'c3_int8_w8a8_4096'
 EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16',
-         'c5_hadamard_a8w4']
+         'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192']
 
 
 def _blas_threads() -> int:

@@ -14,6 +14,8 @@
 // The lane that owns column n of the MFMA result owns it for all its registers, so one weight scale
 // per 32x32 tile and group is enough.  The result leaves through LDS so that global stores are
 // 16-byte and row-contiguous.
+#include <type_traits>
+
 #include "common.h"
 
 namespace qwix {
@@ -264,6 +266,275 @@ int launch_grouped(const GroupedArgs& p, hipStream_t st) {
   return check_launch("qgemm_grouped");
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Fast path (no per-partial rounding, per-token or no activation scale, no accumulator dump).
+//
+// 128 x 256 output tile, 8 wavefronts side by side along N, each owning all 128 rows of 32 columns
+// (4 MFMA tiles that share one weight fragment, so the int4 widening is paid once per 4 MFMAs).  The
+// 128-wide K slabs travel global -> LDS directly in 1 KiB pieces, XOR-swizzled per 16-byte chunk so
+// that the fragment reads are bank-conflict free:
+//   A  (int8, 128 B per row):  8 rows per KiB, chunk c of row r sits at position c ^ (r & 7);
+//   B  (int4,  64 B per row): 16 rows per KiB, chunk c of row r sits at position c ^ ((r >> 2) & 3).
+// One 16-byte chunk of packed int4 holds 32 consecutive k; a lane consumes it over two k-steps, and
+// the A fragments of those two k-steps are the two 16-byte chunks with the same 32 k.  The widened
+// nibbles (x 16, sign kept) are byte-permuted into natural K order, so A goes to the MFMA untouched.
+// The first k-step of a group starts from a zero accumulator operand; at the end of a group each
+// int32 partial costs one convert and one FMA.  LDS then becomes staging space for row-contiguous
+// 16-byte stores, where the per-token scale is applied once per row.
+#define QWIX_GLDS16(gptr, lptr)                                                                       \
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),             \
+                                   (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
+
+struct Fast {
+  static constexpr int kBM = 128, kBN = 256, kBK = 128, kNW = 8, kTM = 4;
+};
+
+template <int BQT, bool SBF>
+__global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(GroupedArgs p) {
+  constexpr int BM = Fast::kBM, BN = Fast::kBN, BK = Fast::kBK, NW = Fast::kNW, TM = Fast::kTM;
+  constexpr bool W4 = (BQT == QWIX_INT4);
+  constexpr int B_ROWB = W4 ? 64 : 128;          // bytes of one B row in a slab
+  constexpr int A_BYTES = BM * BK, B_BYTES = BN * B_ROWB, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_LOADS = A_BYTES / 1024 / NW;   // KiB pieces per wavefront and slab
+  constexpr int B_LOADS = B_BYTES / 1024 / NW;
+  constexpr int B_RPL = 1024 / B_ROWB;           // B rows per KiB piece
+  constexpr int NK = BK / 32;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  int tile_m, tile_n;
+  {  // every XCD gets a contiguous run of tiles; tiles walk down 8 tile-rows before moving along N
+    const int nb = gridDim.x;
+    int pid = blockIdx.x;
+    if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);
+    constexpr int GM = 8;
+    const int per_group = GM * tiles_n, grp = pid / per_group, first_m = grp * GM;
+    const int gsz = min(tiles_m - first_m, GM);
+    tile_m = first_m + (pid % per_group) % gsz;
+    tile_n = (pid % per_group) / gsz;
+  }
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  // ---- loader: wave-uniform 64-bit tile base + per-lane 32-bit offset, rows clamped to the last valid one
+  const uint8_t* a_base = p.A + static_cast<int64_t>(m0) * p.lda;
+  const uint8_t* b_base = p.B + static_cast<int64_t>(n0) * p.ldb;
+  uint32_t a_off[A_LOADS], b_off[B_LOADS];
+#pragma unroll
+  for (int j = 0; j < A_LOADS; ++j) {
+    const int row = (j * NW + wave) * 8 + (lane >> 3);
+    a_off[j] = static_cast<uint32_t>(min(row, p.M - 1 - m0)) * static_cast<uint32_t>(p.lda) + (((lane & 7) ^ (lane >> 3)) << 4);
+  }
+#pragma unroll
+  for (int j = 0; j < B_LOADS; ++j) {
+    int row, chunk;
+    if constexpr (W4) {
+      row = (j * NW + wave) * 16 + (lane >> 2);
+      chunk = (lane & 3) ^ ((lane >> 4) & 3);
+    } else {
+      row = (j * NW + wave) * 8 + (lane >> 3);
+      chunk = (lane & 7) ^ (lane >> 3);
+    }
+    b_off[j] = static_cast<uint32_t>(min(row, p.N - 1 - n0)) * static_cast<uint32_t>(p.ldb) + (chunk << 4);
+  }
+  auto issue_loads = [&](int s, int kt) {
+    const uint8_t* ga = a_base + kt * BK;
+    const uint8_t* gb = b_base + kt * B_ROWB;
+    uint8_t* ls = smem + s * STAGE;
+#pragma unroll
+    for (int j = 0; j < A_LOADS; ++j) QWIX_GLDS16(ga + a_off[j], ls + (j * NW + wave) * 1024);
+#pragma unroll
+    for (int j = 0; j < B_LOADS; ++j) QWIX_GLDS16(gb + b_off[j], ls + A_BYTES + (j * NW + wave) * 1024);
+  };
+
+  // ---- fragments
+  const int frow = lane & 31, hx = lane >> 5;
+  const int a_row = frow * BK, a_sw = frow & 7;
+  const int b_row = (wave * 32 + frow) * B_ROWB, b_sw = W4 ? ((frow >> 2) & 3) : (frow & 7);
+  v4i fa[2][TM];
+  v4i fbr[2];  // int4: one chunk = two k-steps; int8: one chunk = one k-step
+  auto read_a = [&](int s, int ks, int buf) {
+    const int chunk = W4 ? (4 * (ks >> 1) + 2 * hx + (ks & 1)) : (2 * ks + hx);
+    const uint8_t* base = smem + s * STAGE + a_row + ((chunk ^ a_sw) << 4);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const v4i*>(base + i * 32 * BK);
+  };
+  auto read_b = [&](int s, int idx, int buf) {  // idx: pair of k-steps (int4) or k-step (int8)
+    const int chunk = 2 * idx + hx;
+    fbr[buf] = *reinterpret_cast<const v4i*>(smem + s * STAGE + A_BYTES + b_row + ((chunk ^ b_sw) << 4));
+  };
+  auto b_frag = [&](int ks) -> v4i {
+    if constexpr (W4) {
+      const v4i raw = fbr[(ks >> 1) & 1];
+      v4i f;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const unsigned w = static_cast<unsigned>(raw[2 * (ks & 1) + h]);
+        const unsigned ev = (w << 4) & 0xF0F0F0F0u, od = w & 0xF0F0F0F0u;  // nibbles 0,2,4,6 and 1,3,5,7, x 16
+        f[2 * h] = static_cast<int>(__builtin_amdgcn_perm(od, ev, 0x05010400));
+        f[2 * h + 1] = static_cast<int>(__builtin_amdgcn_perm(od, ev, 0x07030602));
+      }
+      return f;
+    } else {
+      return fbr[ks & 1];
+    }
+  };
+
+  v16i acc[TM];
+  float accf[TM][16];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      acc[i][r] = 0;
+      accf[i][r] = 0.f;
+    }
+
+  // acc[i][r]: m = m0 + i*32 + 8*(r/4) + 4*hx + r%4,  n = n0 + wave*32 + frow: one weight scale per lane and group
+  const int ncl = min(n0 + wave * 32 + frow, p.N - 1);
+  constexpr float kUnscale = W4 ? 0.0625f : 1.0f;
+  auto load_sb = [&](int g) -> unsigned {
+    const int64_t i = static_cast<int64_t>(g) * p.N + ncl;
+    if constexpr (SBF) return reinterpret_cast<const uint16_t*>(p.sb)[i];
+    return reinterpret_cast<const unsigned*>(p.sb)[i];
+  };
+
+  const int KT = p.K / BK;
+  const int tpg = p.group / BK;
+  unsigned sb_raw = load_sb(0);
+  issue_loads(0, 0);
+  __syncthreads();
+  read_a(0, 0, 0);
+  read_b(0, 0, 0);
+
+  auto slab = [&](int kt, auto first_tag) {
+    constexpr bool FIRST = decltype(first_tag)::value;
+    const int cur = kt & 1;
+    if (kt + 1 < KT) issue_loads(cur ^ 1, kt + 1);
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      if (ks + 1 < NK) {
+        read_a(cur, ks + 1, (ks + 1) & 1);
+        if constexpr (W4) {
+          if ((ks & 1) == 1) read_b(cur, (ks + 1) >> 1, ((ks + 1) >> 1) & 1);
+        } else {
+          read_b(cur, ks + 1, (ks + 1) & 1);
+        }
+      }
+      const v4i fb = b_frag(ks);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        if (FIRST && ks == 0) {
+          const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+          acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks & 1][i], fb, zero, 0, 0, 0);
+        } else {
+          acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks & 1][i], fb, acc[i], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  // The scale of the next group is fetched at the start of a group, together with the slab loads:
+  // a load issued just before the barrier would make the barrier's wait for the slab wait for it too.
+  unsigned sb_next = 0;
+  for (int kt = 0; kt < KT; ++kt) {
+    const int in_group = kt % tpg;
+    if (in_group == 0) {
+      if (kt + tpg < KT) sb_next = load_sb(kt / tpg + 1);
+      slab(kt, std::true_type{});
+    } else {
+      slab(kt, std::false_type{});
+    }
+    if (in_group == tpg - 1) {
+      const float sb = __uint_as_float(SBF ? sb_raw << 16 : sb_raw) * kUnscale;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) accf[i][r] = __builtin_fmaf(static_cast<float>(acc[i][r]), sb, accf[i][r]);
+      sb_raw = sb_next;
+    }
+    __syncthreads();
+    if (kt + 1 < KT) {
+      read_a((kt + 1) & 1, 0, 0);
+      read_b((kt + 1) & 1, 0, 0);
+    }
+  }
+
+  // ---- epilogue: 32 rows x 32 columns of f32 per wavefront and pass through LDS
+  constexpr int ROW_F = 36;  // floats per staged row (32 + padding)
+  float* stg = reinterpret_cast<float*>(smem) + wave * (32 * ROW_F);
+  const bool t_bf16 = (p.t_dtype == QWIX_BF16);
+  const bool vec_ok = (p.ldo % 8 == 0) && (p.N % 4 == 0);
+  // chunk c = lane + 64*q of the 32 x 8 grid of 16-byte pieces: row c/8, columns 4*(c%8) .. +3
+  float sav[TM][4];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int m = m0 + i * 32 + (lane + 64 * q) / 8;
+      sav[i][q] = (p.sa != nullptr && m < p.M) ? ld_scale(p.sa, p.sa_dtype, m) : 1.f;
+    }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) stg[(8 * (r >> 2) + 4 * hx + (r & 3)) * ROW_F + frow] = accf[i][r];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int c = lane + 64 * q, row = c >> 3, cc = c & 7;
+      const float4 v4 = *reinterpret_cast<const float4*>(stg + row * ROW_F + cc * 4);
+      float v[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[e] *= sav[i][q];
+        if (t_bf16) v[e] = round_bf16(v[e]);
+      }
+      const int m = m0 + i * 32 + row, n = n0 + wave * 32 + cc * 4;
+      if (m >= p.M || n >= p.N) continue;
+      if (p.out_dtype == QWIX_BF16) {
+        uint16_t* o = reinterpret_cast<uint16_t*>(p.out) + static_cast<int64_t>(m) * p.ldo + n;
+        if (vec_ok) {
+          *reinterpret_cast<uint2*>(o) =
+              make_uint2(f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16),
+                         f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16));
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < p.N) o[e] = f32_to_bf16_bits(v[e]);
+        }
+      } else {
+        float* o = reinterpret_cast<float*>(p.out) + static_cast<int64_t>(m) * p.ldo + n;
+        if (vec_ok) {
+          *reinterpret_cast<float4*>(o) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < p.N) o[e] = v[e];
+        }
+      }
+    }
+  }
+}
+
+template <int BQT, bool SBF>
+int launch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
+  constexpr int BM = Fast::kBM, BN = Fast::kBN, BK = Fast::kBK, NW = Fast::kNW;
+  constexpr size_t smem = 2 * (BM * BK + BN * (BQT == QWIX_INT4 ? 64 : 128));
+  static_assert(smem >= NW * 32 * 36 * sizeof(float), "epilogue staging must fit");
+  auto kern = qgemm_grouped_dma_kernel<BQT, SBF>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int64_t tiles = static_cast<int64_t>((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  kern<<<dim3(static_cast<unsigned>(tiles)), NW * 64, smem, st>>>(p);
+  return check_launch("qgemm_grouped (dma)");
+}
+
 }  // namespace
 }  // namespace qwix
 
@@ -300,6 +571,13 @@ extern "C" int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b,
   p.out = static_cast<uint8_t*>(out); p.out_dtype = out_dtype; p.ldo = ldo;
   p.acc_out = acc_out;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool row_strides_fit = 128 * lda < (int64_t{1} << 31) && 256 * ldb_bytes < (int64_t{1} << 31);
+  if (!exact && acc_out == nullptr && (sa == nullptr || ga == 1) && row_strides_fit) {
+    const bool sbf = (sb_dtype == QWIX_BF16);
+    if (b_qtype == QWIX_INT4)
+      return sbf ? launch_grouped_dma<QWIX_INT4, true>(p, st) : launch_grouped_dma<QWIX_INT4, false>(p, st);
+    return sbf ? launch_grouped_dma<QWIX_INT8, true>(p, st) : launch_grouped_dma<QWIX_INT8, false>(p, st);
+  }
   if (b_qtype == QWIX_INT4)
     return exact ? launch_grouped<QWIX_INT4, true>(p, st) : launch_grouped<QWIX_INT4, false>(p, st);
   return exact ? launch_grouped<QWIX_INT8, true>(p, st) : launch_grouped<QWIX_INT8, false>(p, st);

@@ -15,7 +15,7 @@ from tests import util
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize('n', [2, 8, 64, 256, 1024, 8192, 16384])
+@pytest.mark.parametrize('n', [2, 8, 64, 256, 1024, 2048, 4096, 8192, 16384])
 def test_fwht_exact_on_small_integers(n):
   from qwix_amd.contrib import hadamard_rot as hr
   g = util.rng(n)
@@ -57,7 +57,7 @@ def test_rotate_inputs_matches_oracle_and_preserves_product(n, dtype):
 
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
 @pytest.mark.parametrize('qtype,tile', [('int8', None), ('int4', 128), ('float8_e4m3fn', None), ('int8', 64)])
-@pytest.mark.parametrize('n', [256, 8192])
+@pytest.mark.parametrize('n', [256, 4096, 8192, 16384])
 def test_fused_rotate_quantize_equals_rotate_then_quantize(n, qtype, tile, dtype):
   from qwix_amd.contrib import hadamard_rot as hr
   from qwix_amd.core import qarray

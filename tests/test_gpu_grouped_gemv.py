@@ -47,16 +47,31 @@ def test_grouped_gemm_exact_mode_is_bit_exact(M, K, N, group, wq_type, dtype):
 
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
 @pytest.mark.parametrize('wq_type', ['int4', 'int8'])
-def test_grouped_gemm_fast_mode_within_tolerance(wq_type, dtype):
+@pytest.mark.parametrize('M,K,N,group', [(256, 1024, 512, 128), (200, 512, 264, 128), (130, 1024, 258, 256),
+                                         (520, 768, 1000, 384), (1, 128, 2, 128)])
+def test_grouped_gemm_fast_mode_within_tolerance(M, K, N, group, wq_type, dtype):
+  """The fast mode keeps the partial sums in f32 (no rounding per partial): it must agree with the exact
+  integer partials combined in float64 to f32 accuracy, and stay inside the envelope of the reference's
+  per-partial roundings."""
   from qwix_amd.core import dot_general as dg
-  xq, wq, oxq, owq, x_np, w_np = _pair(256, 1024, 512, dtype, wq_type, 128, seed=3)
+  print('case grouped fast', M, K, N, group, wq_type, dtype, flush=True)
+  xq, wq, oxq, owq, x_np, w_np = _pair(M, K, N, dtype, wq_type, group, seed=3 + M)
   out = dg.dot_general(xq, wq, DN)
+  torch.cuda.synchronize()
   want, wacc = O.fast_dot_general(oxq, owq, DN, return_acc=True)
   got = util.f32np(out)
   assert np.all(np.abs(got - want.v) <= 1e-2 * np.abs(want.v) + util.partials_envelope(wacc, oxq, owq)), np.abs(got - want.v).max()
-  ref = x_np.astype(np.float64) @ w_np.astype(np.float64)
-  ceil = 0.12 if wq_type == 'int4' else 0.02   # einsum_test.py ceilings for w4a8 / w8a8
-  assert np.abs(got - ref).mean() / np.abs(ref).mean() < ceil * 1.1
+  # closed form from the integer partials: sum_g acc_g[m,n] * sb[g,n], then * sa[m]
+  sa = np.asarray(oxq.scale.v, np.float64).reshape(M, 1)
+  sb = np.asarray(owq.scale.v, np.float64).reshape(K // group, 1, N)
+  exact = (np.asarray(wacc, np.float64).reshape(K // group, M, N) * sb).sum(0) * sa
+  tol = 2.0 ** -7 if dtype is O.BF16 else 1e-5
+  scale = np.abs(np.asarray(wacc, np.float64).reshape(K // group, M, N) * sb).sum(0) * sa
+  assert np.all(np.abs(got - exact) <= tol * scale + 1e-30), (np.abs(got - exact) / (scale + 1e-30)).max()
+  if M >= 128:
+    ref = x_np.astype(np.float64) @ w_np.astype(np.float64)
+    ceil = 0.12 if wq_type == 'int4' else 0.02   # einsum_test.py ceilings for w4a8 / w8a8
+    assert np.abs(got - ref).mean() / np.abs(ref).mean() < ceil * 1.1
 
 
 def test_both_sides_tiled_and_natural_layout_weight():
