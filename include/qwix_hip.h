@@ -125,6 +125,25 @@ QWIX_API int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t l
                    int sb_dtype, int acc_dtype, void* out, int out_dtype, int64_t ldo,
                    void* stream);
 
+/* Asymmetric (zero-point) operand on the quantized path.  Replaces the correction terms of
+ * _fast_dot_general (qwix/_src/core/dot_general.py:228-253): the reference subtracts
+ * dot(broadcast(zp_lhs), q_rhs) or dot(q_lhs, broadcast(zp_rhs)) from the int32 accumulator
+ * before scaling.  With one zero point per row (lhs) or per column (rhs) that term is the outer
+ * product zu[m] * zv[n]:
+ *     lhs asymmetric:  zu = zero points of the rows of a,  zv[n] = sum_k b[n,k]
+ *     rhs asymmetric:  zu[m] = sum_k a[m,k],               zv = zero points of the columns of b
+ *     out[m,n] = cast_R( (T(sum_k a[m,k] b[n,k] - zu[m] * zv[n]) * sa[m]) * sb[n] )
+ * int8 operands, int32 arithmetic (exact), otherwise as qwix_hip_qgemm. */
+QWIX_API int qwix_hip_qgemm_zp(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N,
+                      int64_t K, const void* sa, int sa_dtype, const void* sb, int sb_dtype,
+                      const int32_t* zu, const int32_t* zv, void* out, int out_dtype, int64_t ldo,
+                      void* stream);
+
+/* out[r] = sum_k q[r*ld + k] for int8 rows (K % 16 == 0): the K-sums qwix_hip_qgemm_zp needs
+ * (the reference obtains them as a dot_general against the broadcast zero point,
+ * dot_general.py:233-239,246-252). */
+QWIX_API int qwix_hip_ksum_i8(const void* q, int64_t ld, int64_t rows, int64_t K, int32_t* out, void* stream);
+
 /* Sub-channel GEMM (dot_general.py:186-203,255-260): K is split in groups of `group`
  * (multiple of 128); per-group int32 partials are scaled and summed:
  *     out[m,n] = cast_R( sum_g (T(acc_g[m,n]) * sa[m,g']) * sb[g,n] )

@@ -163,6 +163,25 @@ class _Canon:
     return s.reshape(gb, self.N).contiguous(), gb
 
 
+  # -- zero points (one per row of the lhs / per column of the rhs, like the scales)
+  def lhs_zero_point(self, lhs: QArray) -> torch.Tensor:
+    z = lhs.zero_point
+    if any(z.shape[a] != 1 for a in self.lca):
+      raise NotImplementedError('sub-channel zero points are not supported on the quantized path')
+    if tuple(z.shape[a] for a in self.lfree) != tuple(lhs.shape[a] for a in self.lfree):
+      z = z.expand(*[lhs.shape[a] if a in self.lfree else z.shape[a] for a in range(z.ndim)])
+    return z.reshape(self.M).contiguous()
+
+  def rhs_zero_point(self, rhs: QArray) -> torch.Tensor:
+    z = rhs.zero_point
+    if any(z.shape[a] != 1 for a in self.rca):
+      raise NotImplementedError('sub-channel zero points are not supported on the quantized path')
+    if tuple(z.shape[a] for a in self.rfree) != tuple(rhs.shape[a] for a in self.rfree):
+      z = z.expand(*[rhs.shape[a] if a in self.rfree else z.shape[a] for a in range(z.ndim)])
+    z = z.permute(*(self.rfree + self.rca))
+    return z.reshape(self.N).contiguous()
+
+
 def _tag_of(dtype: torch.dtype) -> int:
   if dtype == torch.int32:
     return _lib.I32
@@ -181,11 +200,10 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
                       return_accumulators: bool = False, **kwargs) -> torch.Tensor:
   """Contract the quantized values on the matrix cores, then scale: out = ((acc * sx) * sy)."""
   del kwargs
-  for x in (lhs, rhs):
-    if isinstance(x, QArray) and x.zero_point is not None:
-      if isinstance(lhs, QArray) and isinstance(rhs, QArray) and lhs.zero_point is not None and rhs.zero_point is not None:
-        raise ValueError('Only one operand can be asymmetric.')
-      raise NotImplementedError('zero-point operands are not supported on the fast path yet; dequantize first')
+  lzp = lhs.zero_point if isinstance(lhs, QArray) else None
+  rzp = rhs.zero_point if isinstance(rhs, QArray) else None
+  if lzp is not None and rzp is not None:
+    raise ValueError('Only one operand can be asymmetric.')
   c = _Canon(lhs, rhs, dimension_numbers)
   lt = qarray.get_tiled_axes(lhs) if isinstance(lhs, QArray) else {}
   rt = qarray.get_tiled_axes(rhs) if isinstance(rhs, QArray) else {}
@@ -209,6 +227,28 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
       qt = _lib.E4M3
     else:
       raise NotImplementedError(f'no MFMA kernel for {lq} x {rq} operands')
+    if lzp is not None or rzp is not None:
+      # dot_general.py:228-253: subtract dot(zp, q_other) from the int32 accumulator.  With one zero
+      # point per row (lhs) / column (rhs) that is the outer product zero_point x K-sum.
+      if qt != _lib.INT8:
+        raise NotImplementedError('zero-point operands need int8 x int8 values on the quantized path')
+      if return_accumulators:
+        raise NotImplementedError('raw accumulators are not returned for zero-point operands')
+      if c.K % 16:
+        raise NotImplementedError('zero-point correction needs K to be a multiple of 16')
+      if lzp is not None:
+        zu = c.lhs_zero_point(lhs).to(torch.int32)
+        zv = torch.empty(c.N, dtype=torch.int32, device=dev)
+        _lib.call('qwix_hip_ksum_i8', b.data_ptr(), b.stride(0), c.N, c.K, zv.data_ptr(), st)
+      else:
+        zv = c.rhs_zero_point(rhs).to(torch.int32)
+        zu = torch.empty(c.M, dtype=torch.int32, device=dev)
+        _lib.call('qwix_hip_ksum_i8', a.data_ptr(), a.stride(0), c.M, c.K, zu.data_ptr(), st)
+      _lib.call('qwix_hip_qgemm_zp', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), c.M, c.N, c.K,
+                _lib.ptr(sa), 0 if sa is None else _lib.float_tag(sa.dtype), _lib.ptr(sb),
+                0 if sb is None else _lib.float_tag(sb.dtype), zu.data_ptr(), zv.data_ptr(), out.data_ptr(),
+                _tag_of(res_t), c.N, st)
+      return out.reshape(c.out_shape)
     if return_accumulators:
       acc = torch.empty(c.M, c.N, dtype=torch.int32, device=dev)
       _lib.call('qwix_hip_qgemm', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), qt, c.M, c.N, c.K, None, 0,
@@ -220,6 +260,9 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
     out = out.reshape(c.out_shape)
     return (out, acc.reshape(c.out_shape)) if return_accumulators else out
   # sub-channel / int4 weights
+  if lzp is not None or rzp is not None:
+    raise NotImplementedError('zero-point operands with sub-channel scales or int4 values are not supported on the '
+                              'quantized path; dequantize first')
   if lq != numerics.INT8 or rq not in (numerics.INT8, numerics.INT4):
     raise NotImplementedError(f'sub-channel MFMA kernel needs int8 x int8/int4 operands, got {lq} x {rq}')
   ngroups = max(ga, gb)

@@ -51,6 +51,10 @@ struct Epilogue {
   const void* sb;  // per n, or null
   int sa_dtype, sb_dtype, out_dtype;
   int r0, r1, r2;
+  // Zero-point correction of an asymmetric operand (int8 only): acc[m,n] -= zu[m] * zv[n], where one
+  // vector holds the zero points and the other the K-sums of the opposite operand's quantized values.
+  const int32_t* zu;
+  const int32_t* zv;
 };
 
 // XCD-aware tile order: consecutive hardware workgroup ids go to different XCDs; give every XCD a
@@ -140,7 +144,14 @@ __device__ __forceinline__ void write_tile(const AccT (&acc)[TM][TN], const Epil
             float v[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              float t = static_cast<float>(acc[i][j][4 * qd + r]);
+              float t;
+              if constexpr (std::is_same<AccT, v16i>::value) {
+                int a = acc[i][j][4 * qd + r];
+                if (ep.zu != nullptr) a -= ep.zu[m] * ep.zv[min(n + r, N - 1)];
+                t = static_cast<float>(a);
+              } else {
+                t = static_cast<float>(acc[i][j][4 * qd + r]);
+              }
               t = r0 ? round_bf16(t) : t;
               t *= sav[i];
               t = r1 ? round_bf16(t) : t;
@@ -331,7 +342,8 @@ __global__ void __launch_bounds__(256)
 // while the MFMAs of slab kt run; the workgroup barrier at the end of the slab waits for them.
 // The workgroup is WGM x WGN wavefronts; with 8 wavefronts (two per SIMD) the issue time of one
 // wavefront's loads and fragment reads hides behind the other's MFMAs.
-// EPI: 0 = no bf16 rounding in the epilogue, 1 = every step rounds to bf16, 2 = flags at run time.
+// EPI: 0 = no bf16 rounding in the epilogue, 1 = every step rounds to bf16, 2 = flags at run time,
+// 3 = flags at run time and zero-point correction.
 #define QWIX_GLDS16(gptr, lptr)                                                                       \
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),             \
                                    (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
@@ -531,8 +543,14 @@ __global__ void __launch_bounds__(WGM * WGN * 64)
         }
       }
   }
-  const bool r0 = EPI == 2 ? ep.r0 != 0 : EPI == 1, r1 = EPI == 2 ? ep.r1 != 0 : EPI == 1,
-             r2 = EPI == 2 ? ep.r2 != 0 : EPI == 1;
+  constexpr bool ZP = (EPI == 3);  // run-time rounding flags plus zero-point correction
+  const bool r0 = EPI >= 2 ? ep.r0 != 0 : EPI == 1, r1 = EPI >= 2 ? ep.r1 != 0 : EPI == 1,
+             r2 = EPI >= 2 ? ep.r2 != 0 : EPI == 1;
+  int zuv[TM];
+  if constexpr (ZP) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) zuv[i] = ep.zu[min(m_base + i * 32 + (lane & 31), M - 1)];
+  }
   __syncthreads();  // every wavefront is done with the slabs; LDS becomes staging space
   uint8_t* stg = smem + wave * (32 * ROWB);
   const bool row_vec = (reinterpret_cast<uintptr_t>(out) % 16 == 0) && ((ldo * ES) % 16 == 0);
@@ -550,9 +568,17 @@ __global__ void __launch_bounds__(WGM * WGN * 64)
                                                     static_cast<int>(acc[i][j][4 * qd + 2]), static_cast<int>(acc[i][j][4 * qd + 3]));
         } else {
           float v[4];
+          int zvv[4] = {0, 0, 0, 0};
+          if constexpr (ZP) {
+            const int n = n_base + j * 32 + 8 * qd + 4 * (lane >> 5);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) zvv[r] = ep.zv[min(n + r, N - 1)];
+          }
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            float t = static_cast<float>(acc[i][j][4 * qd + r]);
+            float t;
+            if constexpr (ZP) t = static_cast<float>(static_cast<int>(acc[i][j][4 * qd + r]) - zuv[i] * zvv[r]);
+            else t = static_cast<float>(acc[i][j][4 * qd + r]);
             if (r0) t = round_bf16(t);
             t *= sa;
             if (r1) t = round_bf16(t);
@@ -620,6 +646,13 @@ int dispatch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t
     if constexpr (QT == QWIX_INT8) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_I32, 0>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     return fail(QWIX_ERR_INVALID_ARGUMENT, "int32 output needs int8 operands");
   }
+  if (ep.zu != nullptr) {
+    if constexpr (QT == QWIX_INT8) {
+      if (ep.out_dtype == QWIX_BF16) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_BF16, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      return launch_dma<QT, BM, BN, WGM, WGN, QWIX_F32, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    }
+    return fail(QWIX_ERR_UNSUPPORTED, "zero-point correction needs int8 operands");
+  }
   if (ep.out_dtype == QWIX_BF16) {
     if (all) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_BF16, 1>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     return launch_dma<QT, BM, BN, WGM, WGN, QWIX_BF16, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
@@ -659,9 +692,65 @@ extern "C" __attribute__((visibility("default"))) int qwix_dbg_read(unsigned lon
 }
 #endif
 
+namespace qwix {
+namespace {
+
+// out[r] = sum_k q[r, k] over int8 rows: one wavefront per row, 16 bytes per lane and trip.
+__global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__ q, int64_t ld, int rows, int K,
+                                                      int32_t* __restrict__ out) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const int8_t* p = q + static_cast<int64_t>(row) * ld;
+  int s = 0;
+  for (int k = lane * 16; k < K; k += 64 * 16) {  // K % 16 == 0
+    const int4 w = *reinterpret_cast<const int4*>(p + k);
+    const int u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s += (u[e] << 24 >> 24) + (u[e] << 16 >> 24) + (u[e] << 8 >> 24) + (u[e] >> 24);
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
+  if (lane == 0) out[row] = s;
+}
+
+}  // namespace
+}  // namespace qwix
+
+extern "C" int qwix_hip_ksum_i8(const void* q, int64_t ld, int64_t rows, int64_t K, int32_t* out, void* stream) {
+  if (!q || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null argument");
+  if (rows <= 0 || K <= 0 || rows > INT32_MAX || K > INT32_MAX || K % 16 || ld % 16 || ld < K || !aligned16(q))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "ksum_i8 needs K and ld multiples of 16 and a 16-byte aligned base "
+                "(rows=%lld K=%lld ld=%lld)", (long long)rows, (long long)K, (long long)ld);
+  ksum_i8_kernel<<<dim3(static_cast<unsigned>((rows + 3) / 4)), 256, 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const int8_t*>(q), ld, static_cast<int>(rows), static_cast<int>(K), out);
+  return check_launch("ksum_i8");
+}
+
+static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M, int64_t N, int64_t K,
+                      const void* sa, int sa_dtype, const void* sb, int sb_dtype, int acc_dtype, const int32_t* zu,
+                      const int32_t* zv, void* out, int out_dtype, int64_t ldo, void* stream);
+
 extern "C" int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M,
                               int64_t N, int64_t K, const void* sa, int sa_dtype, const void* sb, int sb_dtype,
                               int acc_dtype, void* out, int out_dtype, int64_t ldo, void* stream) {
+  return qgemm_impl(a, lda, b, ldb, qtype, M, N, K, sa, sa_dtype, sb, sb_dtype, acc_dtype, nullptr, nullptr, out,
+                    out_dtype, ldo, stream);
+}
+
+extern "C" int qwix_hip_qgemm_zp(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N,
+                                 int64_t K, const void* sa, int sa_dtype, const void* sb, int sb_dtype,
+                                 const int32_t* zu, const int32_t* zv, void* out, int out_dtype, int64_t ldo,
+                                 void* stream) {
+  if (!zu || !zv) return fail(QWIX_ERR_INVALID_ARGUMENT, "null zero-point vectors");
+  if (out_dtype != QWIX_F32 && out_dtype != QWIX_BF16)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "zero-point corrected output must be f32 or bf16");
+  return qgemm_impl(a, lda, b, ldb, QWIX_INT8, M, N, K, sa, sa_dtype, sb, sb_dtype, 0, zu, zv, out, out_dtype, ldo,
+                    stream);
+}
+
+static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M, int64_t N, int64_t K,
+                      const void* sa, int sa_dtype, const void* sb, int sb_dtype, int acc_dtype, const int32_t* zu,
+                      const int32_t* zv, void* out, int out_dtype, int64_t ldo, void* stream) {
   if (!a || !b || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/b/out");
   if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX)
     return fail(QWIX_ERR_INVALID_ARGUMENT, "bad GEMM shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
@@ -682,7 +771,7 @@ extern "C" int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t
   if (qtype == QWIX_E4M3 && !ok_s(acc_dtype)) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad accumulator dtype %d", acc_dtype);
   // Dtype chain of the reference epilogue: int32 adopts the first scale's dtype (through f32); a
   // float accumulator starts in acc_dtype; each multiply happens in the promotion of both sides.
-  Epilogue ep{sa, sb, sa_dtype, sb_dtype, out_dtype, 0, 0, 0};
+  Epilogue ep{sa, sb, sa_dtype, sb_dtype, out_dtype, 0, 0, 0, zu, zv};
   int cur = (qtype == QWIX_INT8) ? QWIX_I32 : acc_dtype;
   if (cur == QWIX_BF16) ep.r0 = 1;
   auto step = [&](const void* s, int s_dtype, int* r_after) {

@@ -107,3 +107,49 @@ def test_gemm_linearity_full_size_property():
   total = acc.to(torch.float64).sum().item()
   want_total = float(a.to(torch.float64).sum(0).cpu().numpy() @ b.numpy().astype(np.float64).sum(1))
   assert total == want_total
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('side', ['lhs', 'rhs'])
+@pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (100, 272, 60), (1100, 512, 1300), (3, 64, 5)])
+def test_int8_gemm_with_zero_point_operand_bit_exact(M, K, N, side, dtype):
+  """One asymmetric (minmax) operand: the int32 correction dot(zp, q_other) of dot_general.py:228-253 is
+  subtracted before scaling, so the output is again an elementwise function of exact integers."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  print('case zp', side, M, K, N, dtype, flush=True)
+  x_np, x_t = util.make((M, K), dtype, seed=M + 3 * N)
+  w_np, w_t = util.make((K, N), dtype, seed=M + 3 * N + 1, scale=0.02)
+  x_np = x_np + np.float32(0.75)          # shift the ranges so that the zero points are far from 0
+  x_t = x_t + 0.75
+  x_np = util.f32np(x_t)
+  lkw = dict(qtype='int8', channelwise_axes=[0], calibration_method='minmax' if side == 'lhs' else 'absmax')
+  rkw = dict(qtype='int8', channelwise_axes=[1], calibration_method='minmax' if side == 'rhs' else 'absmax')
+  xq = qarray.quantize(x_t, qarray.HowToQuantize(**lkw))
+  wq = qarray.quantize(w_t, qarray.HowToQuantize(**rkw))
+  oxq = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(**lkw))
+  owq = O.quantize(O.FArr(w_np, dtype), O.HowToQuantize(**rkw))
+  util.assert_qarray_equal(xq, oxq, 'lhs')
+  util.assert_qarray_equal(wq, owq, 'rhs')
+  assert (xq.zero_point is not None) == (side == 'lhs') and (wq.zero_point is not None) == (side == 'rhs')
+  out = dg.dot_general(xq, wq, DN)
+  torch.cuda.synchronize()
+  want = O.dot_general(oxq, owq, DN)
+  got = util.f32np(out)
+  bad = np.flatnonzero(got.ravel() != want.v.ravel())
+  assert bad.size == 0, f'{bad.size} outputs differ: {got.ravel()[bad[:5]]} vs {want.v.ravel()[bad[:5]]}'
+  # and it means what it should: close to the float product
+  ref = x_np.astype(np.float64) @ w_np.astype(np.float64)
+  if K >= 256:
+    assert np.abs(got - ref).mean() / np.abs(ref).mean() < 0.05
+
+
+def test_both_operands_asymmetric_is_an_error():
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  _, x_t = util.make((32, 64), O.F32, seed=1)
+  _, w_t = util.make((64, 32), O.F32, seed=2)
+  xq = qarray.quantize(x_t, qarray.HowToQuantize(qtype='int8', channelwise_axes=[0], calibration_method='minmax'))
+  wq = qarray.quantize(w_t, qarray.HowToQuantize(qtype='int8', channelwise_axes=[1], calibration_method='minmax'))
+  with pytest.raises(ValueError, match='Only one operand can be asymmetric'):
+    dg.dot_general(xq, wq, DN)
