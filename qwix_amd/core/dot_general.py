@@ -78,7 +78,7 @@ class _Canon:
     (lca, rca), (lba, rba) = dimension_numbers
     lca, rca = [int(a) for a in lca], [int(a) for a in rca]
     if len(lba) or len(rba):
-      raise NotImplementedError('batch dimensions are not supported by the HIP dot_general yet')
+      raise ValueError('batch dimensions are peeled off before the 2-D canonical form')
     if len(lca) != len(rca) or not lca:
       raise ValueError(f'bad contracting axes {lca} {rca}')
     lshape, rshape = tuple(lhs.shape), tuple(rhs.shape)
@@ -88,10 +88,6 @@ class _Canon:
     pairs = sorted(zip(lca, rca))
     self.lca = [p[0] for p in pairs]
     self.rca = [p[1] for p in pairs]
-    if self.lca != list(range(len(lshape) - len(lca), len(lshape))):
-      raise NotImplementedError(
-          f'lhs contracting axes {lca} must be the trailing axes of {lshape}; transpose the activation first'
-      )
     self.lfree = [a for a in range(len(lshape)) if a not in self.lca]
     self.rfree = [a for a in range(len(rshape)) if a not in self.rca]
     self.M = math.prod(lshape[a] for a in self.lfree)
@@ -104,6 +100,7 @@ class _Canon:
     v = lhs.qvalue if isinstance(lhs, QArray) else lhs
     if isinstance(v, Int4Tensor):
       raise NotImplementedError('an int4 left operand is not supported by the HIP GEMM kernels')
+    v = v.permute(*(self.lfree + self.lca))  # contracting axes last (a no-op view in the usual layout)
     v = v if v.is_contiguous() else v.contiguous()
     return v.reshape(self.M, self.K)
 
@@ -146,7 +143,7 @@ class _Canon:
     got = tuple(s.shape[a] for a in self.lfree)
     if got != want:
       s = s.expand(*[lhs.shape[a] if a in self.lfree else s.shape[a] for a in range(s.ndim)])
-    return s.reshape(self.M, ga).contiguous(), ga
+    return s.permute(*(self.lfree + self.lca)).reshape(self.M, ga).contiguous(), ga
 
   def rhs_scale(self, rhs: QArray) -> tuple[torch.Tensor | None, int]:
     """(scale as (gb, N) contiguous, gb)."""
@@ -170,7 +167,7 @@ class _Canon:
       raise NotImplementedError('sub-channel zero points are not supported on the quantized path')
     if tuple(z.shape[a] for a in self.lfree) != tuple(lhs.shape[a] for a in self.lfree):
       z = z.expand(*[lhs.shape[a] if a in self.lfree else z.shape[a] for a in range(z.ndim)])
-    return z.reshape(self.M).contiguous()
+    return z.permute(*(self.lfree + self.lca)).reshape(self.M).contiguous()
 
   def rhs_zero_point(self, rhs: QArray) -> torch.Tensor:
     z = rhs.zero_point
@@ -180,6 +177,52 @@ class _Canon:
       z = z.expand(*[rhs.shape[a] if a in self.rfree else z.shape[a] for a in range(z.ndim)])
     z = z.permute(*(self.rfree + self.rca))
     return z.reshape(self.N).contiguous()
+
+
+# ------------------------------------------------------------------------------------------
+# batch dimensions
+# ------------------------------------------------------------------------------------------
+
+
+def _index_batch(x, axes: Sequence[int], idx: Sequence[int]):
+  """x[..., idx_k at axes_k, ...] for a tensor or a QArray (scale / zero point axes of size 1 broadcast)."""
+  def take(t):
+    if isinstance(t, Int4Tensor):
+      raise NotImplementedError('batch dimensions with int4 operands are not supported')
+    sel = [slice(None)] * t.ndim
+    for a, i in zip(axes, idx):
+      sel[a] = i if t.shape[a] != 1 else 0
+    return t[tuple(sel)]
+  if isinstance(x, QArray):
+    return QArray(take(x.qvalue), take(x.scale), None if x.zero_point is None else take(x.zero_point), x.qtype)
+  return take(x)
+
+
+def _drop_axes(axes: Sequence[int], dropped: Sequence[int]) -> list[int]:
+  """Axis numbers after the `dropped` axes have been indexed away."""
+  return [a - sum(1 for d in dropped if d < a) for a in axes]
+
+
+def _over_batch(fn, lhs, rhs, dimension_numbers, **kwargs) -> torch.Tensor:
+  """Runs the 2-D operator once per batch element: out[b..., lhs free..., rhs free...], the layout of
+  lax.dot_general.  One kernel launch per element; the quantized values are sliced as views."""
+  (lca, rca), (lba, rba) = dimension_numbers
+  lba, rba = [int(a) for a in lba], [int(a) for a in rba]
+  if len(lba) != len(rba):
+    raise ValueError(f'batch axes differ in number: {lba} {rba}')
+  bshape = [lhs.shape[a] for a in lba]
+  if bshape != [rhs.shape[a] for a in rba]:
+    raise ValueError(f'batch dimensions differ: lhs {tuple(lhs.shape)} axes {lba} vs rhs {tuple(rhs.shape)} axes {rba}')
+  dn = ((_drop_axes(lca, lba), _drop_axes(rca, rba)), ((), ()))
+  outs = []
+  for flat in range(math.prod(bshape)):
+    idx, rem = [], flat
+    for d in reversed(bshape):
+      idx.append(rem % d)
+      rem //= d
+    idx.reverse()
+    outs.append(fn(_index_batch(lhs, lba, idx), _index_batch(rhs, rba, idx), dn, **kwargs))
+  return torch.stack(outs).reshape(*bshape, *outs[0].shape)
 
 
 def _tag_of(dtype: torch.dtype) -> int:
@@ -204,6 +247,11 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   rzp = rhs.zero_point if isinstance(rhs, QArray) else None
   if lzp is not None and rzp is not None:
     raise ValueError('Only one operand can be asymmetric.')
+  if len(dimension_numbers[1][0]) or len(dimension_numbers[1][1]):
+    if return_accumulators:
+      raise NotImplementedError('raw accumulators are not returned for batched contractions')
+    return _over_batch(_fast_dot_general, lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type,
+                       exact=exact)
   c = _Canon(lhs, rhs, dimension_numbers)
   lt = qarray.get_tiled_axes(lhs) if isinstance(lhs, QArray) else {}
   rt = qarray.get_tiled_axes(rhs) if isinstance(rhs, QArray) else {}
@@ -286,6 +334,8 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   """Dequantize-first path.  A bf16 activation against an int4/int8 weight runs in one fused
   kernel (dequantize in registers, bf16 MFMA); other combinations dequantize then use the vendor GEMM."""
   del kwargs
+  if len(dimension_numbers[1][0]) or len(dimension_numbers[1][1]):
+    return _over_batch(_slow_dot_general, lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type)
   if (_is_float_array(lhs) and lhs.dtype == torch.bfloat16 and isinstance(rhs, QArray) and rhs.zero_point is None
       and _qtype_of(rhs) in (numerics.INT4, numerics.INT8)):
     try:
@@ -307,9 +357,7 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
     lhs = qarray.dequantize(lhs)
   if isinstance(rhs, QArray):
     rhs = qarray.dequantize(rhs)
-  (lca, rca), (lba, rba) = dimension_numbers
-  if len(lba) or len(rba):
-    raise NotImplementedError('batch dimensions are not supported by the HIP dot_general yet')
+  (lca, rca), _ = dimension_numbers
   res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.dtype)
   ct = torch.promote_types(lhs.dtype, rhs.dtype)
   out = torch.tensordot(lhs.to(ct), rhs.to(ct), dims=(list(lca), list(rca)))

@@ -1,0 +1,81 @@
+"""GPU parity: general dimension numbers (batch axes, several contracting axes, contracting axes that are
+not trailing, permuted einsum outputs) through dot_general / einsum vs the CPU oracle.
+
+int8 x int8 per-channel contractions are exact integers followed by an elementwise epilogue, so every
+case here is compared bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import qwix_oracle as O
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+
+def _quantize_both(einsum_str, lshape, rshape, dtype, seed, qtype='int8'):
+  from qwix_amd.core import einsum as es
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make(lshape, dtype, seed=seed)
+  w_np, w_t = util.make(rshape, dtype, seed=seed + 1, scale=0.05)
+  nd = (len(lshape), len(rshape))
+  hl = es.get_how_to_quantize(einsum_str=einsum_str, ndims=nd, for_lhs=True, tile_size=None, qtype=qtype)
+  hr = es.get_how_to_quantize(einsum_str=einsum_str, ndims=nd, for_lhs=False, tile_size=None, qtype=qtype)
+  ohl = O.einsum_get_how_to_quantize(einsum_str=einsum_str, ndims=nd, for_lhs=True, tile_size=None, qtype=qtype)
+  ohr = O.einsum_get_how_to_quantize(einsum_str=einsum_str, ndims=nd, for_lhs=False, tile_size=None, qtype=qtype)
+  assert list(hl.channelwise_axes) == list(ohl.channelwise_axes) and list(hr.channelwise_axes) == list(ohr.channelwise_axes)
+  xq, wq = qarray.quantize(x_t, hl), qarray.quantize(w_t, hr)
+  oxq, owq = O.quantize(O.FArr(x_np, dtype), ohl), O.quantize(O.FArr(w_np, dtype), ohr)
+  util.assert_qarray_equal(xq, oxq, 'lhs')
+  util.assert_qarray_equal(wq, owq, 'rhs')
+  return xq, wq, oxq, owq
+
+
+CASES = [
+    ('btd,dnh->btnh', (2, 16, 64), (64, 4, 32)),       # attention projection: two free axes on the weight
+    ('btnh,nhd->btd', (2, 16, 4, 32), (4, 32, 48)),    # output projection: two contracting axes
+    ('bqd,bkd->bqk', (3, 40, 64), (3, 24, 64)),        # one batch axis, activation x activation
+    ('bhqd,bhkd->bhqk', (2, 3, 20, 64), (2, 3, 12, 64)),  # two batch axes
+    ('td,dn->nt', (50, 128), (128, 70)),               # permuted output
+    ('dt,dn->tn', (128, 50), (128, 70)),               # contracting axis of the lhs is not the last one
+    ('bdq,bkd->bkq', (2, 64, 10), (2, 12, 64)),        # batch + leading contraction + permuted output
+]
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('einsum_str,lshape,rshape', CASES)
+def test_einsum_general_dimension_numbers_bit_exact(einsum_str, lshape, rshape, dtype):
+  from qwix_amd.core import einsum as es
+  print('case einsum', einsum_str, lshape, rshape, dtype, flush=True)
+  xq, wq, oxq, owq = _quantize_both(einsum_str, lshape, rshape, dtype, seed=sum(lshape))
+  out = es.einsum(einsum_str, xq, wq)
+  torch.cuda.synchronize()
+  want = O.einsum(einsum_str, oxq, owq)
+  assert tuple(out.shape) == tuple(want.v.shape)
+  got = util.f32np(out)
+  bad = np.flatnonzero(got.ravel() != want.v.ravel())
+  assert bad.size == 0, f'{bad.size} outputs differ: {got.ravel()[bad[:5]]} vs {want.v.ravel()[bad[:5]]}'
+
+
+def test_batched_dot_general_on_the_dequantize_path():
+  """A float activation against a batched quantized operand takes the dequantize-first path."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make((2, 10, 64), O.F32, seed=11)
+  w_np, w_t = util.make((2, 64, 24), O.F32, seed=12, scale=0.05)
+  how = dict(qtype='int8', channelwise_axes=[0, 2])
+  wq = qarray.quantize(w_t, qarray.HowToQuantize(**how))
+  owq = O.quantize(O.FArr(w_np, O.F32), O.HowToQuantize(**how))
+  dn = (((2,), (1,)), ((0,), (0,)))
+  out = dg.dot_general(x_t, wq, dn)
+  want = O.dot_general(O.FArr(x_np, O.F32), owq, dn)
+  assert tuple(out.shape) == (2, 10, 24)
+  np.testing.assert_allclose(util.f32np(out), want.v, rtol=1e-5, atol=1e-6)
+
+
+def test_batch_shape_mismatch_is_an_error():
+  from qwix_amd.core import dot_general as dg
+  a = torch.zeros(2, 4, 16, device=util.DEV)
+  b = torch.zeros(3, 16, 4, device=util.DEV)
+  with pytest.raises(ValueError, match='batch dimensions differ'):
+    dg.dot_general(a, b, (((2,), (1,)), ((0,), (0,))))
