@@ -183,6 +183,52 @@ class QuantizeRows(Workload):
     return {'workload': self.name, 'M': self.M, 'K': self.K}
 
 
+class QuantizeWeight(Workload):
+  """PTQ of a (K, N) weight: per-output-channel absmax (reduction along the strided axis), written in the
+  K-contiguous layout the GEMM reads."""
+
+  bound = 'hbm'
+
+  def __init__(self, name, K, N, qtype, group=None):
+    self.name, self.K, self.N, self.qtype, self.group = name, K, N, qtype, group
+    self.dtype = 'bf16->' + qtype
+    self.metric = 'weight quantize GB/s (per-channel absmax along K, bf16 -> ' + qtype + ')'
+    self.unit = 'GB/s'
+    self.kernel_name = 'cols_quantize_kernel'
+
+  def setup(self, dev):
+    import torch
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(9)
+    self.w = (torch.randn(self.K, self.N, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(dev)
+    tile = self.group or self.K
+    qb = self.K // 2 if self.qtype == 'int4' else self.K
+    self.q = torch.empty(self.N, qb, dtype=torch.uint8, device=dev)
+    self.s = torch.empty(self.K // tile, self.N, dtype=torch.bfloat16, device=dev)
+    self.qt = {'int8': L.INT8, 'int4': L.INT4, 'float8_e4m3fn': L.E4M3}[self.qtype]
+    self.tile = tile
+    n = L.load().qwix_hip_quantize_workspace_bytes(1, self.K, self.N, tile, L.ABSMAX)
+    self.ws = torch.empty(max(int(n), 16), dtype=torch.uint8, device=dev)
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, i=0):
+    L = self.L
+    L.call('qwix_hip_quantize', self.w.data_ptr(), L.BF16, 1, self.K, self.N, self.tile, self.qt, L.ABSMAX, 0.0,
+           L.LAYOUT_REDUCE_MINOR, self.q.data_ptr(), self.s.data_ptr(), None, self.ws.data_ptr(), self.ws.numel(),
+           self.stream)
+
+  kernel = step
+
+  def work_per_step(self):
+    return self.K * self.N * 2.0 + self.q.numel() + self.s.numel() * 2.0
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'K': self.K, 'N': self.N, 'group': self.group}
+
+
 class FwhtQuantize(Workload):
   """C5 activations: Walsh-Hadamard rotation along K fused with per-token int8 quantization."""
 
@@ -313,7 +359,7 @@ class HadamardQdot(Workload):
     self.dtype = 'int8 x int4'
     self.metric = 'Hadamard-rotated a8w4 g128 qdot TOPS (FWHT + activation quantize included)'
     self.unit = 'TOPS'
-    self.kernel_name = 'qgemm_grouped_kernel'
+    self.kernel_name = 'qgemm_grouped_dma_kernel'
 
   def setup(self, dev):
     import torch
@@ -369,6 +415,9 @@ WORKLOADS = {
     'quantize_act_8192_fp8': lambda: QuantizeRows('quantize_act_8192_fp8', 8192, 8192, 'float8_e4m3fn'),
     'c2_gemv_w4_m1': lambda: GemvW4('c2_gemv_w4_m1', 1, 4096, 14336, 128),
     'c2_gemv_w4_m16': lambda: GemvW4('c2_gemv_w4_m16', 16, 4096, 14336, 128),
+    'c4_quantize_weight_fp8': lambda: QuantizeWeight('c4_quantize_weight_fp8', 8192, 28672, 'float8_e4m3fn'),
+    'c5_quantize_weight_int4_g128': lambda: QuantizeWeight('c5_quantize_weight_int4_g128', 8192, 8192, 'int4', 128),
+    'c3_quantize_weight_int8': lambda: QuantizeWeight('c3_quantize_weight_int8', 4096, 4096, 'int8'),
     'c5_fwht_quantize_act': lambda: FwhtQuantize('c5_fwht_quantize_act', 2048, 8192),
     'fwht_quantize_8192x8192': lambda: FwhtQuantize('fwht_quantize_8192x8192', 8192, 8192),
     'plain_copy_1g': lambda: PlainCopy('plain_copy_1g', 1 << 30),
