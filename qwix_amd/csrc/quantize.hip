@@ -378,7 +378,9 @@ __global__ void cols_finish_cal_kernel(const uint32_t* __restrict__ ws, int64_t 
   }
 }
 
-// Pass 2.  SRC 0: scale from ws (written out by chunk 0); SRC 1: scale given.
+// Pass 2.  SRC 0: scale from ws (written out by chunk 0); SRC 1: scale given; SRC 2: the whole
+// scale group (at most 128 rows) lies inside this block, which then calibrates on its own registers:
+// one read of the input, no workspace, no atomics.
 template <typename D, int QT, int CAL, int LAYOUT, int SRC>
 __global__ void __launch_bounds__(256)
     cols_quantize_kernel(const uint8_t* __restrict__ x, ColGeom gm, const uint32_t* __restrict__ ws,
@@ -386,48 +388,105 @@ __global__ void __launch_bounds__(256)
                          int8_t* __restrict__ zp) {
   constexpr int EV = D::kVec;
   constexpr bool ASYM = (CAL == QWIX_MINMAX);
+  __shared__ float red[SRC == 2 ? 2 : 1][SRC == 2 ? 4 : 1][SRC == 2 ? 16 : 1][EV];
   int64_t o, t, c0;
   int chunk;
   col_decode<D>(gm, blockIdx.x, &o, &t, &chunk, &c0);
-  if (c0 >= gm.inner) return;
+  const bool col_ok = c0 < gm.inner;  // idle threads stay for the barriers
   const int rb = threadIdx.x >> 4;
   const int64_t sidx = (o * gm.ntiles + t) * gm.inner + c0;
-  float s[EV];
-  int z[EV];
-#pragma unroll
-  for (int e = 0; e < EV; ++e) {
-    z[e] = 0;
-    if constexpr (SRC == 0) {
-      const float mx = apply_factor<D>(__uint_as_float(ws[sidx + e]), factor);
-      if constexpr (ASYM) {
-        const int64_t plane = gm.outer * gm.ntiles * gm.inner;
-        const float mn = apply_factor<D>(-__uint_as_float(ws[plane + sidx + e]), factor);
-        s[e] = asym_scale_zp<D, QT>(mn, mx, &z[e]);
-      } else {
-        s[e] = sym_scale<D, QT>(mx);
-      }
-      if (chunk == 0 && rb == 0) {
-        store1<D>(scale, sidx + e, s[e]);
-        if constexpr (ASYM) zp[sidx + e] = static_cast<int8_t>(z[e]);
-      }
-    } else {
-      s[e] = load1<D>(scale, sidx + e);
-      if constexpr (ASYM) z[e] = zp[sidx + e];
-    }
-  }
   const int64_t row_end = (t + 1) * gm.tile;
   const int64_t r0 = t * gm.tile + chunk * 128 + rb * 8;
   float v[8][EV];
+  auto load_rows = [&]() {
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    if (r0 + j < row_end) {
-      unpack16<D>(*reinterpret_cast<const uint4*>(
-                      x + ((o * gm.reduce + r0 + j) * gm.inner + c0) * sizeof(typename D::storage)),
-                  v[j]);
-    } else {
+    for (int j = 0; j < 8; ++j) {
+      if (col_ok && r0 + j < row_end) {
+        unpack16<D>(*reinterpret_cast<const uint4*>(
+                        x + ((o * gm.reduce + r0 + j) * gm.inner + c0) * sizeof(typename D::storage)),
+                    v[j]);
+      } else {
 #pragma unroll
-      for (int e = 0; e < EV; ++e) v[j][e] = 0.f;
+        for (int e = 0; e < EV; ++e) v[j][e] = 0.f;
+      }
     }
+  };
+  float s[EV];
+  int z[EV];
+  if constexpr (SRC == 2) {
+    load_rows();
+    float mx[EV], mn[EV];
+#pragma unroll
+    for (int e = 0; e < EV; ++e) {
+      mx[e] = mn[e] = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if constexpr (ASYM) {
+          mx[e] = fmaxf(mx[e], v[j][e]);
+          mn[e] = fminf(mn[e], v[j][e]);
+        } else {
+          mx[e] = absmax_acc(mx[e], v[j][e]);
+        }
+      }
+      // lanes l, l^16, l^32 hold the same columns
+      mx[e] = fmaxf(mx[e], __shfl_xor(mx[e], 16, 64));
+      mx[e] = fmaxf(mx[e], __shfl_xor(mx[e], 32, 64));
+      if constexpr (ASYM) {
+        mn[e] = fminf(mn[e], __shfl_xor(mn[e], 16, 64));
+        mn[e] = fminf(mn[e], __shfl_xor(mn[e], 32, 64));
+      }
+    }
+    const int tc = threadIdx.x & 15;
+    if ((threadIdx.x & 63) < 16) {
+#pragma unroll
+      for (int e = 0; e < EV; ++e) {
+        red[0][threadIdx.x >> 6][tc][e] = mx[e];
+        if constexpr (ASYM) red[1][threadIdx.x >> 6][tc][e] = mn[e];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < EV; ++e) {
+      z[e] = 0;
+      const float a = apply_factor<D>(
+          fmaxf(fmaxf(red[0][0][tc][e], red[0][1][tc][e]), fmaxf(red[0][2][tc][e], red[0][3][tc][e])), factor);
+      if constexpr (ASYM) {
+        const float b = apply_factor<D>(
+            fminf(fminf(red[1][0][tc][e], red[1][1][tc][e]), fminf(red[1][2][tc][e], red[1][3][tc][e])), factor);
+        s[e] = asym_scale_zp<D, QT>(b, a, &z[e]);
+      } else {
+        s[e] = sym_scale<D, QT>(a);
+      }
+      if (rb == 0 && col_ok) {
+        store1<D>(scale, sidx + e, s[e]);
+        if constexpr (ASYM) zp[sidx + e] = static_cast<int8_t>(z[e]);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < EV; ++e) {
+      z[e] = 0;
+      s[e] = 1.f;
+      if (!col_ok) continue;
+      if constexpr (SRC == 0) {
+        const float mx = apply_factor<D>(__uint_as_float(ws[sidx + e]), factor);
+        if constexpr (ASYM) {
+          const int64_t plane = gm.outer * gm.ntiles * gm.inner;
+          const float mn = apply_factor<D>(-__uint_as_float(ws[plane + sidx + e]), factor);
+          s[e] = asym_scale_zp<D, QT>(mn, mx, &z[e]);
+        } else {
+          s[e] = sym_scale<D, QT>(mx);
+        }
+        if (chunk == 0 && rb == 0) {
+          store1<D>(scale, sidx + e, s[e]);
+          if constexpr (ASYM) zp[sidx + e] = static_cast<int8_t>(z[e]);
+        }
+      } else {
+        s[e] = load1<D>(scale, sidx + e);
+        if constexpr (ASYM) z[e] = zp[sidx + e];
+      }
+    }
+    load_rows();
   }
 #pragma unroll
   for (int e = 0; e < EV; ++e) {
@@ -443,24 +502,39 @@ __global__ void __launch_bounds__(256)
   if constexpr (LAYOUT == QWIX_LAYOUT_NATURAL) {
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-      if (r0 + j < row_end) store_q<QT, EV, kBounded>(v[j], q, (o * gm.reduce + r0 + j) * gm.inner + c0);
-  } else {  // (outer, inner, reduce): 8 consecutive rows of one column are 8 consecutive bytes
-    const bool full = r0 + 8 <= row_end;
+      if (col_ok && r0 + j < row_end) store_q<QT, EV, kBounded>(v[j], q, (o * gm.reduce + r0 + j) * gm.inner + c0);
+  } else {
+    // (outer, inner, reduce): the block's 128 rows x 128 columns leave as 128 column pieces of 128 rows.
+    // A thread's 8 rows of one column are 8 consecutive output bytes, but a direct store would scatter
+    // 32-byte pieces over 128 output rows; staged through LDS the block writes whole 128-byte pieces.
+    constexpr int ROW_EL = 128 + 16;                       // staged row pitch in elements (keeps 8-byte alignment)
+    constexpr int EPB = (QT == QWIX_INT4) ? 2 : 1;         // elements per byte
+    __shared__ __attribute__((aligned(16))) uint8_t stage[16 * EV * ROW_EL / EPB];
+    const int tc = threadIdx.x & 15;
 #pragma unroll
     for (int e = 0; e < EV; ++e) {
-      const int64_t el = (o * gm.inner + c0 + e) * gm.reduce + r0;
-      if (full) {
-        float col[8];
+      float col[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) col[j] = v[j][e];
-        store_q<QT, 8, kBounded>(col, q, el);
-      } else if constexpr (QT == QWIX_INT4) {
-        for (int j = 0; j + 1 < 8 && r0 + j + 1 < row_end; j += 2)
-          q[(el + j) >> 1] = static_cast<uint8_t>(pack2_i4(to_int_q<QT>(v[j][e]), to_int_q<QT>(v[j + 1][e])));
+      for (int j = 0; j < 8; ++j) col[j] = v[j][e];
+      store_q<QT, 8, kBounded>(col, stage, (tc * EV + e) * ROW_EL + rb * 8);
+    }
+    __syncthreads();
+    // 16-byte pieces: piece p of column c covers rows 16*EPB*p .. of this block
+    constexpr int PIECES = 128 / (16 * EPB);
+    const int64_t row0 = t * gm.tile + chunk * 128;
+    const int64_t cb0 = c0 - tc * EV;                      // first column of the block
+    const bool vec = (gm.reduce % (16 * EPB) == 0) && (row0 % (16 * EPB) == 0);
+    for (int i = threadIdx.x; i < 16 * EV * PIECES; i += 256) {
+      const int c = i / PIECES, pc = i % PIECES;
+      const int64_t col = cb0 + c, r = row0 + pc * 16 * EPB;
+      if (col >= gm.inner || r >= row_end) continue;
+      const uint8_t* src = stage + (c * ROW_EL + pc * 16 * EPB) / EPB;
+      uint8_t* dst = q + ((o * gm.inner + col) * gm.reduce + r) / EPB;
+      if (vec && r + 16 * EPB <= row_end) {
+        *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);
       } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-          if (r0 + j < row_end) q[el + j] = q_byte<QT>(v[j][e]);
+        const int nb = static_cast<int>((min(row_end, r + 16 * EPB) - r + EPB - 1) / EPB);
+        for (int k = 0; k < nb; ++k) dst[k] = src[k];
       }
     }
   }
@@ -773,10 +847,13 @@ int qwix_hip_quantize(const void* x, int dtype, int64_t outer, int64_t reduce, i
     return run_rows<MODE_QUANT>(x, dtype, outer * (reduce / tile), tile, qtype, calibration, calib_factor, qvalue,
                                 scale, zero_point, nullptr, nullptr, st);
   if (int e = check_cols(x, dtype, reduce, inner, tile, q_layout, qvalue)) return e;
+  const ColGeom g = make_col_geom(outer, reduce, inner, tile, dtype == QWIX_BF16 ? 8 : 4);
+  if (g.chunks_per_tile == 1)  // a scale group fits one block: calibrate and quantize in one pass, no workspace
+    return run_cols_quantize<2>(x, dtype, g, qtype, calibration, q_layout, nullptr, calib_factor, qvalue, scale,
+                                zero_point, st);
   const size_t need = qwix_hip_quantize_workspace_bytes(outer, reduce, inner, tile, calibration);
   if (!workspace || workspace_bytes < need)
     return fail(QWIX_ERR_INVALID_ARGUMENT, "workspace of %zu bytes required, got %zu", need, workspace_bytes);
-  const ColGeom g = make_col_geom(outer, reduce, inner, tile, dtype == QWIX_BF16 ? 8 : 4);
   if (int e = run_cols_absmax(x, dtype, g, calibration, static_cast<uint32_t*>(workspace), st)) return e;
   return run_cols_quantize<0>(x, dtype, g, qtype, calibration, q_layout, static_cast<const uint32_t*>(workspace),
                               calib_factor, qvalue, scale, zero_point, st);
