@@ -46,6 +46,13 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) {
   __bf16 b = static_cast<__bf16>(x);  // RNE
   return __builtin_bit_cast(uint16_t, b);
 }
+// Two f32 -> two bf16 (RNE) in one v_cvt_pk_bf16_f32: a in the low half, b in the high half.
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
 // Round an f32 result to bf16 precision but keep it in an f32 register.
 __device__ __forceinline__ float round_bf16(float x) {
   return bf16_bits_to_f32(f32_to_bf16_bits(x));

@@ -566,6 +566,19 @@ __global__ void __launch_bounds__(WGM * WGN * 64)
         if constexpr (OUT == QWIX_I32) {
           *reinterpret_cast<int4*>(dst) = make_int4(static_cast<int>(acc[i][j][4 * qd]), static_cast<int>(acc[i][j][4 * qd + 1]),
                                                     static_cast<int>(acc[i][j][4 * qd + 2]), static_cast<int>(acc[i][j][4 * qd + 3]));
+        } else if constexpr (EPI == 1 && OUT == QWIX_BF16) {
+          // Every step rounds to bf16 and the result is bf16: round two values per v_cvt_pk_bf16_f32,
+          // and let the last rounding produce the packed output directly.
+          uint32_t w[2];
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            uint32_t pk = pack_bf16x2(static_cast<float>(acc[i][j][4 * qd + 2 * h]),
+                                      static_cast<float>(acc[i][j][4 * qd + 2 * h + 1]));
+            pk = pack_bf16x2(__uint_as_float(pk << 16) * sa, __uint_as_float(pk & 0xFFFF0000u) * sa);
+            w[h] = pack_bf16x2(__uint_as_float(pk << 16) * sbv[j][qd][2 * h],
+                               __uint_as_float(pk & 0xFFFF0000u) * sbv[j][qd][2 * h + 1]);
+          }
+          *reinterpret_cast<uint2*>(dst) = make_uint2(w[0], w[1]);
         } else {
           float v[4];
           int zvv[4] = {0, 0, 0, 0};
@@ -784,23 +797,18 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
   step(sa, sa_dtype, &ep.r1);
   step(sb, sb_dtype, &ep.r2);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const bool big = (M >= 1024 && N >= 1024);
-  static const int variant = [] { const char* e = getenv("QWIX_GEMM_VARIANT"); return e ? atoi(e) : 1; }();
+  // 256 x 256 tiles once they fill most of the chip's 256 CUs; smaller problems use 128 x 128 tiles.
+  const bool big = ((M + 255) / 256) * ((N + 255) / 256) >= 192;
   const bool off32 = M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);  // 32-bit lane offsets
-  if (K % 128 == 0 && off32 && variant != 0) {  // direct-to-LDS pipeline
+  if (K % 128 == 0 && off32) {  // direct-to-LDS pipeline
     if (qtype == QWIX_INT8) {
-      if (big) return variant == 2 ? dispatch_dma<QWIX_INT8, 256, 256, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st)
-                                   : dispatch_dma<QWIX_INT8, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      if (big) return dispatch_dma<QWIX_INT8, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       return dispatch_dma<QWIX_INT8, 128, 128, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     }
-    if (big) return variant == 2 ? dispatch_dma<QWIX_E4M3, 256, 256, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st)
-                                 : dispatch_dma<QWIX_E4M3, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    if (big) return dispatch_dma<QWIX_E4M3, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     return dispatch_dma<QWIX_E4M3, 128, 128, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
   }
-  if (qtype == QWIX_INT8) {
-    if (big) return launch_qgemm<QWIX_INT8, 256, 256, 128>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
-    return launch_qgemm<QWIX_INT8, 128, 128, 128>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
-  }
-  if (big) return launch_qgemm<QWIX_E4M3, 256, 256, 128>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+  // register-staged kernel: any K that is a multiple of 16
+  if (qtype == QWIX_INT8) return launch_qgemm<QWIX_INT8, 128, 128, 128>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
   return launch_qgemm<QWIX_E4M3, 128, 128, 128>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
 }

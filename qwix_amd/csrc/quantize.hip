@@ -744,7 +744,7 @@ int run_rows(const void* x, int dtype, int64_t nseg, int64_t L, int qtype, int c
                           (MODE == MODE_CALIB || (reinterpret_cast<uintptr_t>(q) & 7) == 0);
       if (vec_ok) {
         const int nvec = static_cast<int>(L / D::kVec);
-        static const int target = [] { const char* e = getenv("QWIX_ROWS_LOADS"); return e ? atoi(e) : 4; }();
+        constexpr int target = 4;  // 16-byte loads per thread
         int lg = log2_ceil((nvec + target - 1) / target);  // aim at `target` loads per thread, 8 at most
         while ((nvec + (1 << lg) - 1) >> lg > 8) ++lg;
         if (lg > 8) lg = 8;
