@@ -54,5 +54,28 @@ def einsum(*args, _qwix_dot_general=_dg.dot_general, preferred_element_type=None
     op = operands[0]
     return torch.einsum(einsum_str, qarray.dequantize(op) if isinstance(op, qarray.QArray) else op).to(res_t)
   if len(operands) != 2:
-    raise NotImplementedError(f'einsum with {len(operands)} operands: contract them pairwise')
+    return _nary(einsum_str, operands, _qwix_dot_general, res_t, **kwargs)
   return _binary(operands[0], operands[1], einsum_str, _qwix_dot_general, res_t, **kwargs)
+
+
+def _nary(einsum_str: str, operands: list, dot_general_fn, res_t, **kwargs):
+  """Three or more operands: contracted pairwise from the left (the reference follows the path chosen
+  by opt_einsum, einsum.py:137-152; the result is the same up to the order of the float roundings).
+  An intermediate keeps every subscript that a later operand or the output still needs."""
+  s = einsum_str.replace(' ', '')
+  if '->' not in s or '.' in s:
+    raise NotImplementedError(f'einsum with {len(operands)} operands needs explicit subscripts: "{einsum_str}"')
+  ins, out = s.split('->')
+  terms = ins.split(',')
+  if len(terms) != len(operands):
+    raise ValueError(f'"{einsum_str}" names {len(terms)} operands, got {len(operands)}')
+  cur, cur_sub = operands[0], terms[0]
+  for k in range(1, len(operands)):
+    later = set(out).union(*[set(t) for t in terms[k + 1:]])
+    keep = [c for c in cur_sub if c in later] + [c for c in terms[k] if c in later and c not in cur_sub]
+    last = k == len(operands) - 1
+    sub = out if last else ''.join(keep)
+    step = f'{cur_sub},{terms[k]}->{sub}'
+    cur = _binary(cur, operands[k], step, dot_general_fn, res_t if last else None, **kwargs)
+    cur_sub = sub
+  return cur

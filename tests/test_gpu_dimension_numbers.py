@@ -79,3 +79,21 @@ def test_batch_shape_mismatch_is_an_error():
   b = torch.zeros(3, 16, 4, device=util.DEV)
   with pytest.raises(ValueError, match='batch dimensions differ'):
     dg.dot_general(a, b, (((2,), (1,)), ((0,), (0,))))
+
+
+def test_three_operand_einsum_contracts_pairwise():
+  """activation x quantized weight x float matrix: the first contraction takes the quantized path."""
+  from qwix_amd.core import einsum as es
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make((24, 64), O.F32, seed=21)
+  w_np, w_t = util.make((64, 32), O.F32, seed=22, scale=0.05)
+  p_np, p_t = util.make((32, 8), O.F32, seed=23)
+  xq = qarray.quantize(x_t, qarray.HowToQuantize(qtype='int8', channelwise_axes=[0]))
+  wq = qarray.quantize(w_t, qarray.HowToQuantize(qtype='int8', channelwise_axes=[1]))
+  out = es.einsum('td,dn,nk->tk', xq, wq, p_t)
+  oxq = O.quantize(O.FArr(x_np, O.F32), O.HowToQuantize(qtype='int8', channelwise_axes=[0]))
+  owq = O.quantize(O.FArr(w_np, O.F32), O.HowToQuantize(qtype='int8', channelwise_axes=[1]))
+  first = O.einsum('td,dn->tn', oxq, owq)
+  want = first.v.astype(np.float64) @ p_np.astype(np.float64)
+  assert tuple(out.shape) == (24, 8)
+  np.testing.assert_allclose(util.f32np(out), want, rtol=1e-4, atol=1e-5)
