@@ -211,21 +211,29 @@ __device__ __forceinline__ void store_bytes(void* dst, const uint32_t (&w)[4]) {
   }
 }
 
-// Quantizes one run of consecutive finished elements with scale s and stores it.
+// Quantizes one run of consecutive finished elements with scale s and stores it.  |v| <= absmax, so
+// the quotients are bounded and the two-op clamp-and-round converter applies.
 template <typename D, int QT, int RUN>
 __device__ __forceinline__ void quantize_run(const float* v, float s, uint8_t* q, int64_t i) {
-  const Divider<D, false> div(s);
+  const Divider<D, false, QT == QWIX_E4M3> div(s);
   float t[RUN];
 #pragma unroll
   for (int e = 0; e < RUN; ++e) t[e] = div(v[e]);
   uint32_t w[4] = {0, 0, 0, 0};
   if constexpr (QT == QWIX_INT4) {
 #pragma unroll
-    for (int e = 0; e < RUN; ++e) w[0] |= static_cast<uint32_t>(to_int_q<QT>(t[e]) & 0xF) << (4 * e);
+    for (int e = 0; e < RUN; ++e) w[0] |= (rne_bits_clamped(t[e], -8.f, 7.f) & 0xFu) << (4 * e);
     store_bytes<RUN / 2>(q + i / 2, w);
   } else if constexpr (QT == QWIX_INT8) {
+    if constexpr (RUN >= 4) {
 #pragma unroll
-    for (int e = 0; e < RUN; ++e) w[e / 4] |= static_cast<uint32_t>(to_int_q<QT>(t[e]) & 0xFF) << (8 * (e & 3));
+      for (int e = 0; e < RUN; e += 4)
+        w[e / 4] = pack4_low_bytes(rne_bits_clamped(t[e], -128.f, 127.f), rne_bits_clamped(t[e + 1], -128.f, 127.f),
+                                   rne_bits_clamped(t[e + 2], -128.f, 127.f), rne_bits_clamped(t[e + 3], -128.f, 127.f));
+    } else {
+#pragma unroll
+      for (int e = 0; e < RUN; ++e) w[0] |= (rne_bits_clamped(t[e], -128.f, 127.f) & 0xFFu) << (8 * e);
+    }
     store_bytes<RUN>(q + i, w);
   } else {
 #pragma unroll
