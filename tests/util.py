@@ -13,14 +13,24 @@ def rng(seed):
   return np.random.Generator(np.random.PCG64(seed))
 
 
-def make(shape, dtype, seed, scale=1.0, dist='normal'):
-  """(numpy f32 holding dtype-representable values, torch tensor on the GPU)."""
+def make_np(shape, dtype, seed, scale=1.0, dist='normal'):
+  """numpy f32 array holding dtype-representable values from a seeded PCG64 stream."""
   g = rng(seed)
   x = g.standard_normal(shape) if dist == 'normal' else g.uniform(0, 1, shape)
   x = (x * scale).astype(np.float32)
   if dtype == O.BF16:
     x = O.round_to_bf16(x)
-  return x, torch.from_numpy(x).to(TORCH_DT[dtype]).to(DEV)
+  return x
+
+
+def to_gpu(x: np.ndarray, dtype) -> torch.Tensor:
+  return torch.from_numpy(x).to(TORCH_DT[dtype]).to(DEV)
+
+
+def make(shape, dtype, seed, scale=1.0, dist='normal'):
+  """(numpy f32 holding dtype-representable values, torch tensor on the GPU)."""
+  x = make_np(shape, dtype, seed, scale, dist)
+  return x, to_gpu(x, dtype)
 
 
 def farr(t: torch.Tensor) -> O.FArr:
