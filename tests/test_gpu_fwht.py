@@ -74,7 +74,7 @@ def test_fused_rotate_quantize_equals_rotate_then_quantize(n, qtype, tile, dtype
 
 
 def test_weight_side_fused_rotation_feeds_the_grouped_gemm():
-  """BASELINE config 5 at reduced shape: rotate both sides, act int8 per token, weight int4 g128."""
+  """The Hadamard a8w4 benchmark configuration at reduced shape: rotate both sides, act int8 per token, weight int4 g128."""
   from qwix_amd.contrib import hadamard_rot as hr
   from qwix_amd.core import dot_general as dg
   from qwix_amd.core import qarray

@@ -102,7 +102,7 @@ def test_per_channel_int4_weight_and_tile_mismatch_error():
 @pytest.mark.parametrize('M', [1, 8, 16, 40])
 @pytest.mark.parametrize('K,N,group,sdt', [(512, 256, 128, torch.float32), (4096, 1024, 128, torch.float32), (1024, 200, 1024, torch.bfloat16)])
 def test_weight_only_gemv(M, K, N, group, sdt, wq_type):
-  """BASELINE config 2 at reduced N: bf16 activations x int4 g128 weight, f32 scales, bf16 out."""
+  """The weight-only int4 benchmark configuration at reduced N: bf16 activations x int4 g128 weight, f32 scales, bf16 out."""
   from qwix_amd.core import dot_general as dg
   from qwix_amd.core import qarray
   print('case gemv', M, K, N, group, wq_type, flush=True)

@@ -1,5 +1,5 @@
 """GPU parity through the provider surface: QuantizationRule -> PtqProvider -> quantize_model /
-quantize_params, on the PTQ MLP of BASELINE config 1 and on an einsum layer."""
+quantize_params, on the PTQ MLP benchmark configuration and on an einsum layer."""
 import numpy as np
 import pytest
 import torch
