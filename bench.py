@@ -348,6 +348,61 @@ class GemvW4(Workload):
             'weight_copies_rotated': self.copies}
 
 
+class QdotDecode(Workload):
+  """Dynamic-range w8a8 at decode size: per-token int8 quantize of M <= 16 tokens + the skinny quantized
+  GEMM, which streams the int8 weight once (HBM-bound)."""
+
+  bound = 'hbm'
+  graph_ok = False
+
+  def __init__(self, name, M, K, N):
+    self.name, self.M, self.K, self.N = name, M, K, N
+    self.dtype = 'int8'
+    self.metric = 'w8a8 int8 decode GB/s (activation quantize included)'
+    self.unit = 'GB/s'
+    self.kernel_name = 'qgemm_skinny_kernel'
+
+  def setup(self, dev):
+    import torch
+    from qwix_amd.core import qarray
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(2100)
+    self.x = torch.randn(self.M, self.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    w = (torch.randn(self.K, self.N, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(dev)
+    wq = qarray.quantize(w, qarray.HowToQuantize(qtype='int8', channelwise_axes=[1]))
+    b = wq.qvalue.permute(1, 0)
+    assert b.is_contiguous()
+    self.copies = max(1, -(-(640 << 20) // (b.numel())))   # rotate: every launch reads its weight from HBM
+    self.b = [b] + [b.clone() for _ in range(self.copies - 1)]
+    self.sb = wq.scale.reshape(-1).contiguous()
+    self.xq = torch.empty(self.M, self.K, dtype=torch.int8, device=dev)
+    self.sa = torch.empty(self.M, dtype=torch.bfloat16, device=dev)
+    self.out = torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev)
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, i=0):
+    L = self.L
+    L.call('qwix_hip_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, 1, self.K, L.INT8, L.ABSMAX, 0.0,
+           L.LAYOUT_NATURAL, self.xq.data_ptr(), self.sa.data_ptr(), None, None, 0, self.stream)
+    self.kernel(i)
+
+  def kernel(self, i=0):
+    L = self.L
+    L.call('qwix_hip_qgemm', self.xq.data_ptr(), self.K, self.b[i % self.copies].data_ptr(), self.K, L.INT8, self.M,
+           self.N, self.K, self.sa.data_ptr(), L.BF16, self.sb.data_ptr(), L.BF16, L.BF16, self.out.data_ptr(), L.BF16,
+           self.N, self.stream)
+
+  def work_per_step(self):
+    return self.K * self.N + self.N * 2.0 + self.M * self.K * 3.0 + self.M * self.N * 2.0
+
+  def kernel_work(self):
+    return self.K * self.N + self.N * 2.0 + self.M * self.K * 1.0 + self.M * self.N * 2.0
+
+  def describe(self):
+    return {'workload': self.name, 'M': self.M, 'K': self.K, 'N': self.N, 'weight_copies_rotated': self.copies}
+
+
 class HadamardQdot(Workload):
   """C5: FWHT + per-token int8 quantize of the activations each step, then int8 x int4 g128 grouped GEMM
   against the offline-rotated weight."""
@@ -413,6 +468,7 @@ WORKLOADS = {
     'int8_w8a8_8192': lambda: QdotW8A8('int8_w8a8_8192', 8192, 8192, 8192, 'int8'),
     'quantize_act_4096': lambda: QuantizeRows('quantize_act_4096', 4096, 4096, 'int8'),
     'quantize_act_8192_fp8': lambda: QuantizeRows('quantize_act_8192_fp8', 8192, 8192, 'float8_e4m3fn'),
+    'w8a8_decode_m16': lambda: QdotDecode('w8a8_decode_m16', 16, 4096, 14336),
     'c2_gemv_w4_m1': lambda: GemvW4('c2_gemv_w4_m1', 1, 4096, 14336, 128),
     'c2_gemv_w4_m16': lambda: GemvW4('c2_gemv_w4_m16', 16, 4096, 14336, 128),
     'c4_quantize_weight_fp8': lambda: QuantizeWeight('c4_quantize_weight_fp8', 8192, 28672, 'float8_e4m3fn'),
@@ -424,7 +480,7 @@ WORKLOADS = {
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
 }
 DEFAULT = 'c3_int8_w8a8_4096'
-EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16',
+EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16',
          'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192']
 
 

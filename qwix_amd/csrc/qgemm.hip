@@ -708,6 +708,143 @@ extern "C" __attribute__((visibility("default"))) int qwix_dbg_read(unsigned lon
 namespace qwix {
 namespace {
 
+// ------------------------------------------------------------------------------------------------
+// Skinny GEMM (decode: a handful of tokens against a whole weight matrix).  The 128 x 128 tiles of
+// the kernels above would leave most CUs idle and most MFMA rows empty; here the weight matrix is
+// streamed exactly once: a workgroup owns NT tiles of 16 output columns, its 16 wavefronts split
+// K, each with two 128-byte blocks of loads in flight, and the int32 (or f32) partial tiles meet
+// in LDS.  int8: v_mfma_i32_16x16x64_i8, a lane holds 32 consecutive k of one row (two MFMAs);
+// e4m3: one v_mfma_f32_16x16x128_f8f6f4.  The int32 sum does not depend on the split, so results
+// are bit-identical to the tiled kernels'; the epilogue is the same rounding chain.
+typedef int v8i_s __attribute__((ext_vector_type(8)));
+typedef float v4f_s __attribute__((ext_vector_type(4)));
+constexpr int kSkinnyWaves = 16;
+
+template <int QT, int NT>
+__global__ void __launch_bounds__(kSkinnyWaves * 64)
+    qgemm_skinny_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb, int M,
+                        int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  constexpr bool IS_INT = (QT == QWIX_INT8);
+  using AccT = typename std::conditional<IS_INT, v4i, v4f_s>::type;
+  __shared__ AccT red[kSkinnyWaves][NT][64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15, kq = lane >> 4;
+  const int n_base = blockIdx.x * (16 * NT), row0 = blockIdx.y * 16;
+  const int nblk = K / 128;
+  const int per_wave = (nblk + kSkinnyWaves - 1) / kSkinnyWaves;
+  const int kb0 = wave * per_wave, kb1 = min(nblk, kb0 + per_wave);
+
+  // wave-uniform bases + fixed 32-bit lane offsets; rows of A past M and columns past N are clamped
+  const uint8_t* a_base = A + static_cast<int64_t>(row0) * lda;
+  const uint8_t* b_base = B + static_cast<int64_t>(n_base) * ldb;
+  const uint32_t a_off = static_cast<uint32_t>(min(col, M - 1 - row0)) * static_cast<uint32_t>(lda) + kq * 32;
+  uint32_t b_off[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+    b_off[t] = static_cast<uint32_t>(min(t * 16 + col, N - 1 - n_base)) * static_cast<uint32_t>(ldb) + kq * 32;
+
+  AccT acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[t][r] = 0;
+
+  struct Blk {
+    v4i x[2];
+    v4i w[NT][2];
+  };
+  auto load_blk = [&](int kb, Blk* b) {
+    const uint8_t* ap = a_base + kb * 128 + a_off;
+    b->x[0] = *reinterpret_cast<const v4i*>(ap);
+    b->x[1] = *reinterpret_cast<const v4i*>(ap + 16);
+    const uint8_t* bp = b_base + kb * 128;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      b->w[t][0] = *reinterpret_cast<const v4i*>(bp + b_off[t]);
+      b->w[t][1] = *reinterpret_cast<const v4i*>(bp + b_off[t] + 16);
+    }
+  };
+  auto compute_blk = [&](const Blk& b) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if constexpr (IS_INT) {
+        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b.x[0], b.w[t][0], acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b.x[1], b.w[t][1], acc[t], 0, 0, 0);
+      } else {
+        const v8i_s xa = {b.x[0][0], b.x[0][1], b.x[0][2], b.x[0][3], b.x[1][0], b.x[1][1], b.x[1][2], b.x[1][3]};
+        const v8i_s wb = {b.w[t][0][0], b.w[t][0][1], b.w[t][0][2], b.w[t][0][3],
+                          b.w[t][1][0], b.w[t][1][1], b.w[t][1][2], b.w[t][1][3]};
+        acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(xa, wb, acc[t], 0, 0, 0, 0, 0, 0);
+      }
+    }
+  };
+  for (int kb = kb0; kb < kb1; kb += 2) {
+    Blk b0, b1;
+    const bool two = kb + 1 < kb1;
+    load_blk(kb, &b0);
+    if (two) load_blk(kb + 1, &b1);
+    compute_blk(b0);
+    if (two) compute_blk(b1);
+  }
+
+#pragma unroll
+  for (int t = 0; t < NT; ++t) red[wave][t][lane] = acc[t];
+  __syncthreads();
+  // result lane layout: column n = lane % 16, row m = 4 * (lane / 16) + r
+  const bool r0 = ep.r0 != 0, r1 = ep.r1 != 0, r2 = ep.r2 != 0;
+  for (int idx = tid; idx < NT * 256; idx += kSkinnyWaves * 64) {
+    const int t = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
+    const int m = row0 + 4 * (l >> 4) + r, n = n_base + t * 16 + (l & 15);
+    if (m >= M || n >= N) continue;
+    float v;
+    if constexpr (IS_INT) {
+      int a = 0;
+#pragma unroll
+      for (int w = 0; w < kSkinnyWaves; ++w) a += red[w][t][l][r];
+      if (ep.out_dtype == QWIX_I32) {
+        reinterpret_cast<int*>(out)[static_cast<int64_t>(m) * ldo + n] = a;
+        continue;
+      }
+      if (ep.zu != nullptr) a -= ep.zu[m] * ep.zv[n];
+      v = static_cast<float>(a);
+    } else {
+      v = 0.f;
+#pragma unroll
+      for (int w = 0; w < kSkinnyWaves; ++w) v += red[w][t][l][r];
+    }
+    if (r0) v = round_bf16(v);
+    if (ep.sa != nullptr) v *= load_scale(ep.sa, ep.sa_dtype, m);
+    if (r1) v = round_bf16(v);
+    if (ep.sb != nullptr) v *= load_scale(ep.sb, ep.sb_dtype, n);
+    if (r2) v = round_bf16(v);
+    if (ep.out_dtype == QWIX_BF16)
+      reinterpret_cast<uint16_t*>(out)[static_cast<int64_t>(m) * ldo + n] = f32_to_bf16_bits(v);
+    else
+      reinterpret_cast<float*>(out)[static_cast<int64_t>(m) * ldo + n] = v;
+  }
+}
+
+template <int QT>
+int launch_skinny(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                  const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  const unsigned gy = static_cast<unsigned>((M + 15) / 16);
+#define QWIX_SKINNY(NTT)                                                                                         \
+  qgemm_skinny_kernel<QT, NTT><<<dim3(static_cast<unsigned>((N + 16 * NTT - 1) / (16 * NTT)), gy), kSkinnyWaves * 64, \
+                                 0, st>>>(static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, \
+                                          static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), ep,       \
+                                          static_cast<uint8_t*>(out), ldo)
+  // wider column groups reuse the activation fragments; narrower ones keep every CU busy
+  if (N >= 192 * 64)
+    QWIX_SKINNY(4);
+  else if (N >= 192 * 32)
+    QWIX_SKINNY(2);
+  else
+    QWIX_SKINNY(1);
+#undef QWIX_SKINNY
+  return check_launch("qgemm (skinny)");
+}
+
 // out[r] = sum_k q[r, k] over int8 rows: one wavefront per row, 16 bytes per lane and trip.
 __global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__ q, int64_t ld, int rows, int K,
                                                       int32_t* __restrict__ out) {
@@ -797,6 +934,10 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
   step(sa, sa_dtype, &ep.r1);
   step(sb, sb_dtype, &ep.r2);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (M <= 32 && K % 128 == 0 && 16 * lda < (int64_t{1} << 31) && 64 * ldb < (int64_t{1} << 31)) {
+    if (qtype == QWIX_INT8) return launch_skinny<QWIX_INT8>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    return launch_skinny<QWIX_E4M3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+  }
   // 256 x 256 tiles once they fill most of the chip's 256 CUs; smaller problems use 128 x 128 tiles.
   const bool big = ((M + 255) / 256) * ((N + 255) / 256) >= 192;
   const bool off32 = M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);  // 32-bit lane offsets

@@ -30,7 +30,8 @@ def _quantized_pair(M, K, N, dtype, qtype, seed):
 
 
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
-@pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (128, 64, 128), (100, 272, 60), (1, 4096, 1024), (1024, 512, 1024), (1300, 1024, 1100)])
+@pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (128, 64, 128), (100, 272, 60), (1, 4096, 1024), (1024, 512, 1024), (1300, 1024, 1100),
+                                   (16, 1024, 520), (32, 512, 96), (7, 256, 12300), (33, 256, 64)])
 def test_int8_gemm_bit_exact(M, K, N, dtype):
   from qwix_amd.core import dot_general as dg
   print('case int8', M, K, N, dtype, flush=True)
@@ -69,7 +70,7 @@ def test_raw_int8_operand_stays_on_fast_path():
 
 
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
-@pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (100, 320, 60), (1024, 2048, 1024)])
+@pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (100, 320, 60), (1024, 2048, 1024), (16, 1024, 264), (5, 4096, 12300)])
 def test_fp8_gemm_close(M, K, N, dtype):
   from qwix_amd.core import dot_general as dg
   print('case fp8', M, K, N, dtype, flush=True)
@@ -111,7 +112,7 @@ def test_gemm_linearity_full_size_property():
 
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
 @pytest.mark.parametrize('side', ['lhs', 'rhs'])
-@pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (100, 272, 60), (1100, 512, 1300), (3, 64, 5)])
+@pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (100, 272, 60), (1100, 512, 1300), (3, 64, 5), (8, 256, 200)])
 def test_int8_gemm_with_zero_point_operand_bit_exact(M, K, N, side, dtype):
   """One asymmetric (minmax) operand: the int32 correction dot(zp, q_other) of dot_general.py:228-253 is
   subtracted before scaling, so the output is again an elementwise function of exact integers."""
