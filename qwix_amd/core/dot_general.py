@@ -342,7 +342,9 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
       c = _Canon(lhs, rhs, dimension_numbers)
       sb, gb = c.rhs_scale(rhs)
       group = c.K // gb
-      if c.K % 128 == 0 and (group % 128 == 0):
+      # up to a few hundred rows the fused kernel (16 rows per pass over the weight) beats
+      # dequantize + float GEMM, which has to write and re-read the whole float weight
+      if c.K % 128 == 0 and (group % 128 == 0) and c.M <= 256:
         x = c.lhs_values(lhs)
         b, b_is4 = c.rhs_values(rhs)
         res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.scale.dtype)
