@@ -457,6 +457,45 @@ __global__ void __launch_bounds__(WGM * WGN * 64)
     }
   };
 
+  const int m_base = m0 + wm * WTM, n_base = n0 + wn * WTN;
+  float sbv[TN][4][4];
+  // The scale vectors are fetched before the main loop: at the start of the epilogue they would be a
+  // cold two-microsecond round trip with nothing to hide behind.
+  float sav[TM];
+  if constexpr (OUT != QWIX_I32) {
+    const bool vec_ok = (N % 4 == 0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int m = m_base + i * 32 + (lane & 31);
+      sav[i] = (ep.sa != nullptr && m < M) ? load_scale(ep.sa, ep.sa_dtype, m) : 1.f;
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int n = n_base + j * 32 + 8 * qd + 4 * (lane >> 5);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sbv[j][qd][r] = 1.f;
+        if (ep.sb != nullptr) {
+          if (vec_ok && n < N) {  // n % 4 == 0: one 8- or 16-byte load
+            if (ep.sb_dtype == QWIX_BF16) {
+              const uint2 w = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(ep.sb) + n);
+              sbv[j][qd][0] = __uint_as_float(w.x << 16);
+              sbv[j][qd][1] = __uint_as_float(w.x & 0xFFFF0000u);
+              sbv[j][qd][2] = __uint_as_float(w.y << 16);
+              sbv[j][qd][3] = __uint_as_float(w.y & 0xFFFF0000u);
+            } else {
+              const float4 w = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(ep.sb) + n);
+              sbv[j][qd][0] = w.x; sbv[j][qd][1] = w.y; sbv[j][qd][2] = w.z; sbv[j][qd][3] = w.w;
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (n + r < N) sbv[j][qd][r] = load_scale(ep.sb, ep.sb_dtype, n + r);
+          }
+        }
+      }
+  }
   const int KT = K / BK;
   QWIX_DBG_DECL
   QWIX_DBG_STAMP(0)
@@ -506,43 +545,6 @@ __global__ void __launch_bounds__(WGM * WGN * 64)
   constexpr int CPR = WTN * ES / 16;             // 16-byte chunks per staged row
   constexpr int EPC = 16 / ES;                   // elements per chunk
   static_assert(NWAVES * 32 * ROWB <= 2 * STAGE, "epilogue staging does not fit in LDS");
-  const int m_base = m0 + wm * WTM, n_base = n0 + wn * WTN;
-  float sbv[TN][4][4];
-  float sav[TM];  // fetched up front: a load inside the store loop would wait for the stores before it
-  if constexpr (OUT != QWIX_I32) {
-    const bool vec_ok = (N % 4 == 0);
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int m = m_base + i * 32 + (lane & 31);
-      sav[i] = (ep.sa != nullptr && m < M) ? load_scale(ep.sa, ep.sa_dtype, m) : 1.f;
-    }
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        const int n = n_base + j * 32 + 8 * qd + 4 * (lane >> 5);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) sbv[j][qd][r] = 1.f;
-        if (ep.sb != nullptr) {
-          if (vec_ok && n < N) {  // n % 4 == 0: one 8- or 16-byte load
-            if (ep.sb_dtype == QWIX_BF16) {
-              const uint2 w = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(ep.sb) + n);
-              sbv[j][qd][0] = __uint_as_float(w.x << 16);
-              sbv[j][qd][1] = __uint_as_float(w.x & 0xFFFF0000u);
-              sbv[j][qd][2] = __uint_as_float(w.y << 16);
-              sbv[j][qd][3] = __uint_as_float(w.y & 0xFFFF0000u);
-            } else {
-              const float4 w = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(ep.sb) + n);
-              sbv[j][qd][0] = w.x; sbv[j][qd][1] = w.y; sbv[j][qd][2] = w.z; sbv[j][qd][3] = w.w;
-            }
-          } else {
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (n + r < N) sbv[j][qd][r] = load_scale(ep.sb, ep.sb_dtype, n + r);
-          }
-        }
-      }
-  }
   constexpr bool ZP = (EPI == 3);  // run-time rounding flags plus zero-point correction
   const bool r0 = EPI >= 2 ? ep.r0 != 0 : EPI == 1, r1 = EPI >= 2 ? ep.r1 != 0 : EPI == 1,
              r2 = EPI >= 2 ? ep.r2 != 0 : EPI == 1;
