@@ -33,6 +33,9 @@ PEAK_MFMA_TOPS = 5000.0   # MI355X dense int8 / fp8 matrix peak, TOP/s (TFLOP/s 
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak, GB/s
 
 
+SPIN_UP_S = 0.5           # minimum duration of the untimed warm-up
+
+
 def _events(n):
   import torch
   return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
@@ -500,8 +503,15 @@ def run(wl: Workload, steps: int, warmup: int):
   import torch
   dev = torch.device('cuda:0')
   wl.setup(dev)
-  for i in range(warmup):
+  # Untimed warm-up: the requested steps, and at least SPIN_UP_S seconds of them -- the first few hundred
+  # milliseconds of GPU work after process start run at a lower clock than steady state.
+  t_start = time.perf_counter()
+  i = 0
+  while i < warmup or time.perf_counter() - t_start < SPIN_UP_S:
     wl.step(i)
+    i += 1
+    if i % 16 == 0:
+      torch.cuda.synchronize()
   torch.cuda.synchronize()
   t0 = time.perf_counter()
   for i in range(steps):
