@@ -498,7 +498,7 @@ def _blas_threads() -> int:
   return int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1))
 
 
-def run(wl: Workload, steps: int, warmup: int):
+def run(wl: Workload, steps: int, warmup: int, spin_up: float = None):
   """Returns (seconds per step, seconds per launch of the dominant kernel)."""
   import torch
   dev = torch.device('cuda:0')
@@ -507,7 +507,8 @@ def run(wl: Workload, steps: int, warmup: int):
   # milliseconds of GPU work after process start run at a lower clock than steady state.
   t_start = time.perf_counter()
   i = 0
-  while i < warmup or time.perf_counter() - t_start < SPIN_UP_S:
+  spin_up = SPIN_UP_S if spin_up is None else spin_up
+  while i < warmup or time.perf_counter() - t_start < spin_up:
     wl.step(i)
     i += 1
     if i % 16 == 0:
@@ -563,6 +564,8 @@ def main():
   ap.add_argument('--workload', default=DEFAULT, choices=sorted(WORKLOADS))
   ap.add_argument('--no-extra', action='store_true', help='skip the other workloads of the metric')
   ap.add_argument('--no-cpu-baseline', action='store_true')
+  ap.add_argument('--spin-up', type=float, default=SPIN_UP_S,
+                  help='minimum seconds of untimed warm-up (profiling runs shorten it to keep traces small)')
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
     print('bench.py: this build runs on ONE GPU only (no collectives, no sharding); re-run with --gpus 1. '
@@ -574,7 +577,7 @@ def main():
     sys.exit(2)
 
   wl = WORKLOADS[args.workload]()
-  step_s, kmean = run(wl, args.steps, args.warmup)
+  step_s, kmean = run(wl, args.steps, args.warmup, args.spin_up)
   res = summarize(wl, step_s, kmean)
   line = {
       'metric': wl.metric, 'value': res['value'], 'unit': res['unit'], 'n_gpus': 1, 'steps': args.steps,
@@ -591,7 +594,7 @@ def main():
     for name in EXTRA:
       w = WORKLOADS[name]()
       n = max(5, min(args.steps, 20))
-      s, km = run(w, n, 3)
+      s, km = run(w, n, 3, args.spin_up)
       r = summarize(w, s, km)
       extra[name] = {'metric': w.metric, 'value': r['value'], 'unit': r['unit'], 'ms_per_step': r['ms_per_step'],
                      'roofline': r['roofline']}
