@@ -139,6 +139,23 @@ QWIX_API int qwix_hip_qgemm_zp(const void* a, int64_t lda, const void* b, int64_
                       const int32_t* zu, const int32_t* zv, void* out, int out_dtype, int64_t ldo,
                       void* stream);
 
+/* Ragged quantized GEMM (mixture-of-experts).  Replaces _fast_ragged_dot_general
+ * (qwix/_src/core/ragged_dot.py:123-226) for the dimension numbers of qwix.ragged_dot
+ * (ragged_dot.py:24-29: lhs (M,K), rhs (G,K,N), lhs rows split into G consecutive groups):
+ *     out[m,n] = cast_R( (T(sum_k a[m,k] * b_g[n,k]) * sa[m]) * sb_g[n] ),   g = group of row m,
+ * with the same accumulator / rounding chain as qwix_hip_qgemm.  group_sizes (device memory, G
+ * int32 values) is read by the kernel, never by the host: negative sizes count as 0, groups are
+ * cut off at row M, and rows past the last group are written as zeros (what the masked sum of
+ * lax.ragged_dot_general gives them).  b is G panels of (N,K) K-contiguous values,
+ * b_group_stride bytes apart; sb holds one vector of N scales per group, sb_group_stride
+ * elements apart (the expanded per-group scale of ragged_dot.py:32-57,205-217), or a single shared
+ * vector when sb_group_stride is 0.  sa / sb may be null. */
+QWIX_API int qwix_hip_qgemm_ragged(const void* a, int64_t lda, const void* b, int64_t ldb,
+                          int64_t b_group_stride, int qtype, int64_t M, int64_t N, int64_t K,
+                          const int32_t* group_sizes, int64_t G, const void* sa, int sa_dtype,
+                          const void* sb, int sb_dtype, int64_t sb_group_stride, int acc_dtype,
+                          void* out, int out_dtype, int64_t ldo, void* stream);
+
 /* out[r] = sum_k q[r*ld + k] for int8 rows (K % 16 == 0): the K-sums qwix_hip_qgemm_zp needs
  * (the reference obtains them as a dot_general against the broadcast zero point,
  * dot_general.py:233-239,246-252). */

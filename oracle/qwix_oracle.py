@@ -17,6 +17,7 @@ What it restates (file:line refer to the google/qwix v0.1.8 source tree):
   dot_general qwix/_src/core/dot_general.py:28-76    get_how_to_quantize
               qwix/_src/core/dot_general.py:135-275  _fast_dot_general, _slow_dot_general
               qwix/_src/core/dot_general.py:407-491  dispatcher
+  ragged_dot  qwix/_src/core/ragged_dot.py:123-353   quantized / dequantize-first ragged dot
   einsum      qwix/_src/core/einsum.py:27-103        get_how_to_quantize, binary einsum
               qwix/_src/core/einsum_info.py:26-174   EinsumInfo
   hadamard    qwix/contrib/hadamard_rot.py:35-190    Sylvester matrix, sign flips, rotate
@@ -39,6 +40,9 @@ How each function is pinned (tests/test_oracle_*.py):
   * _fast == _slow == dequant-dot ... invariant of two_dim_scales_test.py:57-93.
   * dtype rule, tiling heuristics, EinsumInfo ... the reference's tables
     (dot_general_test.py:28-146,175-197; einsum_info_test.py).
+  * ragged dot ...................... reduces, group by group, to the pinned dot_general on
+    row slices; brute-force loops on tiny inputs; empty groups, rows of no group, groups
+    reaching past the last row (the group_sizes of ragged_dot_test.py:36-80).
   * hadamard ........................ H H^T = n I, (xH)(H^T w / n) = x w
     (hadamard_rot_test.py:24-41,92-147), popcount closed form.
 
@@ -712,6 +716,124 @@ def dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None):
   if use_fast_path(lhs, rhs, dimension_numbers):
     return fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type)
   return slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type)
+
+
+# ----------------------------------------------------------------------------
+# ragged_dot.py (the dimension numbers of qwix.ragged_dot: lhs (M,K), rhs (G,K,N))
+# ----------------------------------------------------------------------------
+
+
+def _ragged_dot_f64(lhs: np.ndarray, rhs: np.ndarray, group_sizes) -> np.ndarray:
+  """lax.ragged_dot as a masked sum: out = sum_g mask_g(lhs) @ rhs[g], mask_g = rows
+  [start_g, start_g + size_g).  Rows covered by no group come out as zeros; groups
+  reaching past the last row are cut off by the mask."""
+  m = lhs.shape[0]
+  out = np.zeros((m, rhs.shape[2]), np.float64)
+  rows = np.arange(m)
+  start = 0
+  for g, size in enumerate(group_sizes):
+    mask = (rows >= start) & (rows < start + int(size))
+    out += np.where(mask[:, None], lhs.astype(np.float64), 0.0) @ rhs[g].astype(np.float64)
+    start += int(size)
+  return out
+
+
+def fast_ragged_dot(lhs, rhs, group_sizes, preferred_element_type=None):
+  """ragged_dot.py:123-226 for _BASIC_RAGGED_DOT_DIMENSION_NUMBERS (:24-29).
+
+  Tiled contracting axes become a leading batch axis t of the ragged dot (:169-180); the
+  lhs scale is applied first, then the rhs scale -- expanded over the rows by a ragged dot
+  of ones with the scale when it has a group axis (:32-57,205-217; 1 * s is exact, rows of
+  no group get 0) -- and the tile axis is summed last (:222-224)."""
+  lv, ls, lzp, lt = _operand_fields(lhs)
+  rv, rs, rzp, rt = _operand_fields(rhs)
+  assert lzp is None and rzp is None, 'zero points take the slow path (ragged_dot.py:278-283)'
+  a, b = lt.get(1), rt.get(1)
+  if a and b and a != b:
+    raise ValueError('Contracting axes must be tiled with the same tile size.')
+  tile = a or b or lv.shape[1]
+  m, k = lv.shape
+  g, _, n = rv.shape
+  nt = k // tile
+  acc_t, res_t = get_accumulator_and_result_type(
+      lhs, rhs, preferred_element_type=preferred_element_type
+  )
+  parts = []
+  for t in range(nt):
+    d = _ragged_dot_f64(
+        lv[:, t * tile : (t + 1) * tile], rv[:, t * tile : (t + 1) * tile, :], group_sizes
+    )
+    if acc_t == INT32:
+      assert np.all(np.abs(d) < 2**31)
+      parts.append(d.astype(np.int64).astype(np.int32))
+    else:
+      parts.append(rnd(d.astype(np.float32), acc_t))
+  res = np.stack(parts)  # (nt, m, n)
+  cur_t = acc_t
+  scales = []
+  if ls is not None:
+    # (M|1, nt|1) -> (nt|1, M|1, 1)
+    scales.append(FArr(ls.v.T[:, :, None], ls.dtype))
+  if rs is not None:
+    # (G|1, nt|1, N|tiles) -> rows pick their group's vector
+    sv = rs.v
+    if sv.shape[2] not in (1, n):
+      sv = np.repeat(sv, n // sv.shape[2], axis=2)
+    if sv.shape[0] > 1:
+      ones = np.ones((m, 1), np.float32)
+      sv = np.stack([
+          _ragged_dot_f64(ones, sv[:, t : t + 1, :], group_sizes).astype(np.float32)
+          for t in range(sv.shape[1])
+      ])
+    else:
+      sv = np.transpose(sv, (1, 0, 2))  # (nt|1, 1, N|1)
+    scales.append(FArr(sv, rs.dtype))
+  for s in scales:
+    if cur_t == INT32:
+      res = rnd(res.astype(np.float32), s.dtype)
+      cur_t = s.dtype
+    else:
+      cur_t = promote(cur_t, s.dtype)
+      res = rnd(res, cur_t)
+    res = rnd(res * s.v, cur_t)
+  if a or b:
+    if cur_t == INT32:
+      res = res.sum(axis=0)
+    else:
+      out = np.zeros(res.shape[1:], np.float32)
+      for t in range(nt):
+        out = out + res[t].astype(np.float32)
+      res = rnd(out, cur_t)
+  else:
+    res = res[0]
+  if res_t == INT32:
+    return res.astype(np.int32)
+  return FArr(rnd(np.asarray(res, np.float32), res_t), res_t)
+
+
+def slow_ragged_dot(lhs, rhs, group_sizes, preferred_element_type=None):
+  """ragged_dot.py:229-241: dequantize, then a float ragged dot (f64 accumulate here)."""
+  if isinstance(lhs, QArray):
+    lhs = dequantize(lhs)
+  if isinstance(rhs, QArray):
+    rhs = dequantize(rhs)
+  res_t = preferred_element_type or promote(lhs.dtype, rhs.dtype)
+  d = _ragged_dot_f64(lhs.v, rhs.v, group_sizes)
+  return FArr(rnd(d.astype(np.float32), res_t), res_t)
+
+
+def ragged_dot(lhs, rhs, group_sizes, preferred_element_type=None):
+  """ragged_dot.py:244-353: the quantized path unless an operand has a zero point or is a
+  raw float array (:278-292)."""
+  fast = True
+  for operand in (lhs, rhs):
+    if isinstance(operand, QArray):
+      if operand.zero_point is not None:
+        fast = False
+    elif isinstance(operand, FArr):
+      fast = False
+  fn = fast_ragged_dot if fast else slow_ragged_dot
+  return fn(lhs, rhs, group_sizes, preferred_element_type)
 
 
 # ----------------------------------------------------------------------------

@@ -1,0 +1,187 @@
+"""Quantized ragged dot (mixture-of-experts matmul) on MI355X: host side of the ragged MFMA GEMM.
+
+Mirror of qwix/_src/core/ragged_dot.py: `ragged_dot` (:316-353), the dispatcher
+`ragged_dot_general` (:244-313: quantized path unless an operand has a zero point or is a raw float
+array), `_fast_ragged_dot_general` (:123-226) and `_slow_ragged_dot_general` (:229-241).
+
+lhs is (M, K), rhs is (G, K, N); the rows of lhs form G consecutive groups of `group_sizes` rows
+and group g is multiplied with rhs[g].  `group_sizes` stays in device memory: the kernel reads it,
+so the quantized path never synchronises with the host.  Rows past the last group come out as
+zeros.  Only the dimension numbers of `ragged_dot` are supported; others raise.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Sequence
+
+import torch
+
+from qwix_amd import _lib
+from qwix_amd.core import numerics
+from qwix_amd.core import qarray
+from qwix_amd.core.dot_general import DotDimensionNumbers, _is_float_array, _qtype_of, _tag_of
+from qwix_amd.core.qarray import Int4Tensor, QArray
+
+
+@dataclasses.dataclass(frozen=True)
+class RaggedDotDimensionNumbers:
+  """Counterpart of jax.lax.RaggedDotDimensionNumbers."""
+
+  dot_dimension_numbers: DotDimensionNumbers
+  lhs_ragged_dimensions: Sequence[int]
+  rhs_group_dimensions: Sequence[int]
+
+
+_BASIC_RAGGED_DOT_DIMENSION_NUMBERS = RaggedDotDimensionNumbers(
+    dot_dimension_numbers=(((1,), (1,)), ((), ())), lhs_ragged_dimensions=(0,), rhs_group_dimensions=(0,))
+
+
+def _check_basic(dn: RaggedDotDimensionNumbers, lhs, rhs, group_sizes, group_offset):
+  (lca, rca), (lba, rba) = dn.dot_dimension_numbers
+  basic = (tuple(lca), tuple(rca), tuple(lba), tuple(rba), tuple(dn.lhs_ragged_dimensions),
+           tuple(dn.rhs_group_dimensions)) == ((1,), (1,), (), (), (0,), (0,))
+  if not basic:
+    raise NotImplementedError(f'only the dimension numbers of ragged_dot are supported, got {dn}')
+  if group_offset is not None:
+    raise NotImplementedError('group_offset is not supported')
+  if len(lhs.shape) != 2 or len(rhs.shape) != 3 or lhs.shape[1] != rhs.shape[1]:
+    raise ValueError(f'ragged_dot expects lhs (M, K) and rhs (G, K, N), got {tuple(lhs.shape)} and {tuple(rhs.shape)}')
+  if group_sizes.ndim != 1 or group_sizes.shape[0] != rhs.shape[0]:
+    raise ValueError(f'group_sizes must have one entry per group: {tuple(group_sizes.shape)} vs G={rhs.shape[0]}')
+  if group_sizes.dtype not in (torch.int32, torch.int64):
+    raise TypeError(f'group_sizes must be an integer tensor, got {group_sizes.dtype}')
+
+
+def _rhs_values(v: torch.Tensor) -> torch.Tensor:
+  """(G, K, N) values as (G, N, K) K-contiguous storage: a view if the tensor already is a permuted
+  view of such storage, else one transposing pass per group."""
+  G, K, N = v.shape
+  p = v.permute(0, 2, 1)
+  if p.is_contiguous():
+    return p
+  if not v.is_contiguous():
+    v = v.contiguous()
+  dst = torch.empty(G, N, K, dtype=v.dtype, device=v.device)
+  for g in range(G):
+    _lib.call('qwix_hip_transpose_q', v[g].data_ptr(), _lib.INT8, K, N, dst[g].data_ptr(), _lib.stream_of(dst))
+  return dst
+
+
+def _fast_ragged_dot_general(lhs, rhs, group_sizes, dimension_numbers=_BASIC_RAGGED_DOT_DIMENSION_NUMBERS,
+                             precision=None, preferred_element_type=None, group_offset=None) -> torch.Tensor:
+  """Contract the quantized values group by group on the matrix cores, then scale:
+  out = ((acc * lhs_scale) * rhs_scale[group of the row]), tile partials summed last."""
+  del precision
+  _check_basic(dimension_numbers, lhs, rhs, group_sizes, group_offset)
+  for x in (lhs, rhs):
+    if isinstance(x, QArray) and x.zero_point is not None:
+      raise NotImplementedError('zero-point operands take the dequantize-first ragged dot')
+    if isinstance(x.qvalue if isinstance(x, QArray) else x, Int4Tensor):
+      raise NotImplementedError('int4 operands are not supported by the ragged MFMA kernel')
+  lq, rq = _qtype_of(lhs), _qtype_of(rhs)
+  if (lq, rq) == (numerics.INT8, numerics.INT8):
+    qt = _lib.INT8
+  elif (lq, rq) == (numerics.E4M3, numerics.E4M3):
+    qt = _lib.E4M3
+  else:
+    raise NotImplementedError(f'no ragged MFMA kernel for {lq} x {rq} operands')
+  lt = qarray.get_tiled_axes(lhs) if isinstance(lhs, QArray) else {}
+  rt = qarray.get_tiled_axes(rhs) if isinstance(rhs, QArray) else {}
+  if lt.get(1) and rt.get(1) and lt[1] != rt[1]:
+    raise ValueError(f'Contracting axes must be tiled with the same tile size. lhs_tiled_axes={lt} rhs_tiled_axes={rt} {dimension_numbers=}')
+  acc_t, res_t = qarray.get_accumulator_and_result_type(lhs, rhs, preferred_element_type=preferred_element_type)
+  M, K = lhs.shape
+  G, _, N = rhs.shape
+  tile = lt.get(1) or rt.get(1) or K
+  ntiles = K // tile
+  a = lhs.qvalue if isinstance(lhs, QArray) else lhs
+  a = a if a.is_contiguous() else a.contiguous()
+  b = _rhs_values(rhs.qvalue if isinstance(rhs, QArray) else rhs)
+  dev = a.device
+  st = _lib.stream_of(a)
+  gs = group_sizes.to(device=dev, dtype=torch.int32).contiguous()
+
+  # scales in kernel order: sa (M, ntiles or 1), sb (G or 1, ntiles or 1, N)
+  sa = sb = None
+  if isinstance(lhs, QArray):
+    sa = lhs.scale.expand(M, lhs.scale.shape[1]).contiguous()
+  if isinstance(rhs, QArray):
+    sb = rhs.scale
+    if sb.shape[2] not in (1, N):
+      sb = sb.repeat_interleave(N // sb.shape[2], dim=2)
+    sb = sb.expand(sb.shape[0], sb.shape[1], N).contiguous()
+  # dtype in which the scaled partials live: the accumulator's, promoted with each scale in turn
+  cur_t = None if acc_t == torch.int32 else acc_t
+  for s in (sa, sb):
+    if s is not None:
+      cur_t = s.dtype if cur_t is None else torch.promote_types(cur_t, s.dtype)
+  cur_t = cur_t or torch.int32
+
+  def launch(t: int, out: torch.Tensor):
+    sa_t = None if sa is None else sa[:, min(t, sa.shape[1] - 1)].contiguous()
+    sb_t = None if sb is None else sb[:, min(t, sb.shape[1] - 1), :].contiguous()
+    _lib.call('qwix_hip_qgemm_ragged', a.data_ptr() + t * tile, a.stride(0), b.data_ptr() + t * tile, b.stride(1),
+              b.stride(0), qt, M, N, tile, gs.data_ptr(), G, _lib.ptr(sa_t),
+              0 if sa_t is None else _lib.float_tag(sa_t.dtype), _lib.ptr(sb_t),
+              0 if sb_t is None else _lib.float_tag(sb_t.dtype), N if (sb_t is not None and sb_t.shape[0] > 1) else 0,
+              _tag_of(acc_t) if acc_t != torch.int32 else 0, out.data_ptr(), _tag_of(out.dtype), N, st)
+
+  if ntiles == 1:
+    out = torch.empty(M, N, dtype=res_t, device=dev)
+    launch(0, out)
+    return out
+  # Sub-channel scales along K: one launch per K tile, each partial scaled with its own scales; the
+  # partials are summed in f32 in tile order and rounded once (ragged_dot.py:222-224).
+  part = torch.empty(M, N, dtype=cur_t, device=dev)
+  total = torch.zeros(M, N, dtype=torch.int32 if cur_t == torch.int32 else torch.float32, device=dev)
+  for t in range(ntiles):
+    launch(t, part)
+    total += part
+  return total.to(cur_t).to(res_t)
+
+
+def _slow_ragged_dot_general(lhs, rhs, group_sizes, dimension_numbers=_BASIC_RAGGED_DOT_DIMENSION_NUMBERS,
+                             precision=None, preferred_element_type=None, group_offset=None) -> torch.Tensor:
+  """Dequantize (HIP kernel), then one float GEMM per group.  The group boundaries are needed on the
+  host to slice the rows, so this path waits for `group_sizes` to arrive there."""
+  del precision
+  _check_basic(dimension_numbers, lhs, rhs, group_sizes, group_offset)
+  if isinstance(lhs, QArray):
+    lhs = qarray.dequantize(lhs)
+  if isinstance(rhs, QArray):
+    rhs = qarray.dequantize(rhs)
+  res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.dtype)
+  ct = torch.promote_types(lhs.dtype, rhs.dtype)
+  M = lhs.shape[0]
+  out = torch.zeros(M, rhs.shape[2], dtype=res_t, device=lhs.device)
+  start = 0
+  for g, size in enumerate(group_sizes.tolist()):
+    stop = min(start + max(int(size), 0), M)
+    if stop > start:
+      out[start:stop] = torch.matmul(lhs[start:stop].to(ct), rhs[g].to(ct)).to(res_t)
+    start = stop
+  return out
+
+
+def ragged_dot_general(lhs, rhs, group_sizes: torch.Tensor, dimension_numbers: RaggedDotDimensionNumbers,
+                       precision=None, preferred_element_type=None, group_offset=None) -> torch.Tensor:
+  """Drop-in for lax.ragged_dot_general that accepts QArray operands."""
+  use_fast_path = True
+  for operand in (lhs, rhs):
+    if isinstance(operand, QArray):
+      if operand.zero_point is not None:
+        use_fast_path = False
+        break
+    elif _is_float_array(operand):
+      use_fast_path = False
+      break
+  fn = _fast_ragged_dot_general if use_fast_path else _slow_ragged_dot_general
+  return fn(lhs, rhs, group_sizes, dimension_numbers, precision=precision,
+            preferred_element_type=preferred_element_type, group_offset=group_offset)
+
+
+def ragged_dot(lhs, rhs, group_sizes: torch.Tensor, precision=None, preferred_element_type=None,
+               group_offset=None) -> torch.Tensor:
+  """Drop-in for lax.ragged_dot: lhs (M, K) . rhs (G, K, N) with the rows of lhs in G groups."""
+  return ragged_dot_general(lhs, rhs, group_sizes, _BASIC_RAGGED_DOT_DIMENSION_NUMBERS, precision=precision,
+                            preferred_element_type=preferred_element_type, group_offset=group_offset)

@@ -191,10 +191,11 @@ __device__ __forceinline__ void write_tile(const AccT (&acc)[TM][TN], const Epil
 // LDS into a second register set; the slab for the next iteration is fetched from global memory
 // at the top of the iteration, written to the other LDS stage before the last k-step, and the
 // workgroup barrier plus the first fragment read of the next slab hide behind that last k-step.
+// The tile at rows [m0, m0 + BM) x columns [n0, n0 + BN); rows from M on are neither read nor stored.
 template <int QT, int BM, int BN, int BK>
-__global__ void __launch_bounds__(256)
-    qgemm_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
-                 int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+__device__ __forceinline__ void qgemm_tile(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B,
+                                           int64_t ldb, int m0, int n0, int M, int N, int K, const Epilogue& ep,
+                                           uint8_t* __restrict__ out, int64_t ldo) {
   constexpr bool IS_INT = (QT == QWIX_INT8);
   constexpr int LDS_STRIDE = BK + kPad;
   constexpr int TM = BM / 64, TN = BN / 64;
@@ -209,9 +210,6 @@ __global__ void __launch_bounds__(256)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  int tile_m, tile_n;
-  tile_coords((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   using AccT = typename std::conditional<IS_INT, v16i, v16f>::type;
   using FragT = typename std::conditional<IS_INT, v4i, v8i>::type;
@@ -333,6 +331,15 @@ __global__ void __launch_bounds__(256)
   QWIX_DBG_FLUSH()
 }
 
+template <int QT, int BM, int BN, int BK>
+__global__ void __launch_bounds__(256)
+    qgemm_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
+                 int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  int tile_m, tile_n;
+  tile_coords((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
+  qgemm_tile<QT, BM, BN, BK>(A, lda, B, ldb, tile_m * BM, tile_n * BN, M, N, K, ep, out, ldo);
+}
+
 // Fast path (K % 128 == 0): the slabs go from global memory straight into LDS
 // (global_load_lds_dwordx4: no staging registers, no ds_write instructions).  Each wave-level load
 // fills one contiguous KiB of LDS = 8 tile rows x 128 bytes; inside a row the eight 16-byte k-chunks
@@ -349,9 +356,10 @@ __global__ void __launch_bounds__(256)
                                    (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
 
 template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI>
-__global__ void __launch_bounds__(WGM * WGN * 64)
-    qgemm_dma_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
-                     int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+__device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, int64_t lda,
+                                               const uint8_t* __restrict__ B, int64_t ldb, int m0, int n0, int M,
+                                               int N, int K, const Epilogue& ep, uint8_t* __restrict__ out,
+                                               int64_t ldo) {
   constexpr bool IS_INT = (QT == QWIX_INT8);
   constexpr int BK = 128;
   constexpr int NWAVES = WGM * WGN;
@@ -368,9 +376,6 @@ __global__ void __launch_bounds__(WGM * WGN * 64)
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
-  int tile_m, tile_n;
-  tile_coords((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   using AccT = typename std::conditional<IS_INT, v16i, v16f>::type;
   using FragT = typename std::conditional<IS_INT, v4i, v8i>::type;
@@ -633,6 +638,15 @@ __global__ void __launch_bounds__(WGM * WGN * 64)
 }
 
 template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI>
+__global__ void __launch_bounds__(WGM * WGN * 64)
+    qgemm_dma_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
+                     int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  int tile_m, tile_n;
+  tile_coords((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
+  qgemm_dma_tile<QT, BM, BN, WGM, WGN, OUT, EPI>(A, lda, B, ldb, tile_m * BM, tile_n * BN, M, N, K, ep, out, ldo);
+}
+
+template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI>
 int launch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
                const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   constexpr size_t smem = 2 * (BM + BN) * 128;
@@ -694,6 +708,156 @@ int launch_qgemm(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t
                                                               static_cast<int>(N), static_cast<int>(K), ep,
                                                               static_cast<uint8_t*>(out), ldo);
   return check_launch("qgemm");
+}
+
+// ------------------------------------------------------------------------------------------------
+// Ragged GEMM (mixture-of-experts): the rows of A are split into consecutive groups whose sizes are
+// read from device memory; the rows of group g meet B_g, the g-th (N, K) panel.  Rows that belong
+// to no group (past the sum of the sizes) come out as zeros.  No host synchronisation: the grid
+// is sized for the worst case, floor(M / BM) + G + 1 tile rows, and every workgroup finds its
+// tile by walking the group sizes (wave-uniform scalar work); workgroups past the last tile exit.
+struct Ragged {
+  const int32_t* group_sizes;  // G entries
+  int G;
+  int64_t b_group_stride;   // bytes between consecutive B panels
+  int64_t sb_group_stride;  // elements between the rhs scale vectors of consecutive groups (0: one shared vector)
+};
+
+constexpr int kRaggedChunk = 16;  // consecutive tile ids that run on one XCD
+
+// Returns 0: no tile, 1: a tile of group *g, 2: a tile of rows that belong to no group.
+// Tile ids are numbered group by group; inside a group they walk 8 tile rows per column so that
+// tiles that run together share operand panels.  Runs of kRaggedChunk ids are dealt out to the 8
+// XCDs in turn, which also spreads the unused ids at the end over all of them.
+template <int BM, int BN>
+__device__ __forceinline__ int ragged_tile(const Ragged& rg, int M, int N, int* g, int* m0, int* m_lim, int* n0) {
+  int pid = blockIdx.x;  // gridDim.x % (8 * kRaggedChunk) == 0
+  {
+    const int k = pid >> 3, x = pid & 7;
+    pid = ((k / kRaggedChunk) * 8 + x) * kRaggedChunk + k % kRaggedChunk;
+  }
+  const int tiles_n = (N + BN - 1) / BN;
+  int row = 0, first = 0, kind = 0;
+  for (int i = 0; i <= rg.G; ++i) {
+    // sizes are clamped so that no group reaches past row M; the pass i == G covers the rows left over
+    const int sz = i < rg.G ? min(max(rg.group_sizes[i], 0), M - row) : M - row;
+    const int nt = (sz + BM - 1) / BM;
+    const int cnt = nt * tiles_n;
+    if (kind == 0 && pid < first + cnt) {
+      constexpr int GM = 8;
+      const int r = pid - first, per = GM * tiles_n;
+      const int fm = (r / per) * GM, gsz = min(nt - fm, GM);
+      *g = i;
+      *m0 = row + (fm + (r % per) % gsz) * BM;
+      *m_lim = row + sz;
+      *n0 = ((r % per) / gsz) * BN;
+      kind = i < rg.G ? 1 : 2;
+    }
+    first += cnt;
+    row += sz;
+  }
+  return kind;
+}
+
+template <int BM, int BN, typename OutT>
+__device__ __forceinline__ void zero_tile(uint8_t* out, int64_t ldo, int m0, int m_lim, int n0, int N, int nthreads) {
+  const int rows = min(BM, m_lim - m0), cols = min(BN, N - n0);
+  for (int idx = threadIdx.x; idx < rows * cols; idx += nthreads)
+    reinterpret_cast<OutT*>(out)[static_cast<int64_t>(m0 + idx / cols) * ldo + n0 + idx % cols] = 0;
+}
+
+__device__ __forceinline__ Epilogue group_epilogue(const Epilogue& ep, const Ragged& rg, int g) {
+  Epilogue e = ep;
+  if (ep.sb != nullptr)
+    e.sb = static_cast<const uint8_t*>(ep.sb) + g * rg.sb_group_stride * (ep.sb_dtype == QWIX_BF16 ? 2 : 4);
+  return e;
+}
+
+template <int QT, int BM, int BN, int WGM, int WGN, int OUT>
+__global__ void __launch_bounds__(WGM * WGN * 64)
+    qgemm_ragged_dma_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
+                            Ragged rg, int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  int g, m0, m_lim, n0;
+  const int kind = ragged_tile<BM, BN>(rg, M, N, &g, &m0, &m_lim, &n0);
+  if (kind == 0) return;
+  using OutT = typename std::conditional<OUT == QWIX_BF16, uint16_t, uint32_t>::type;
+  if (kind == 2) {
+    zero_tile<BM, BN, OutT>(out, ldo, m0, m_lim, n0, N, WGM * WGN * 64);
+    return;
+  }
+  const Epilogue e = group_epilogue(ep, rg, g);
+  qgemm_dma_tile<QT, BM, BN, WGM, WGN, OUT, (OUT == QWIX_I32 ? 0 : 2)>(A, lda, B + g * rg.b_group_stride, ldb, m0, n0,
+                                                                        m_lim, N, K, e, out, ldo);
+}
+
+template <int QT, int BM, int BN, int BK>
+__global__ void __launch_bounds__(256)
+    qgemm_ragged_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
+                        Ragged rg, int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  int g, m0, m_lim, n0;
+  const int kind = ragged_tile<BM, BN>(rg, M, N, &g, &m0, &m_lim, &n0);
+  if (kind == 0) return;
+  if (kind == 2) {
+    if (ep.out_dtype == QWIX_BF16) zero_tile<BM, BN, uint16_t>(out, ldo, m0, m_lim, n0, N, 256);
+    else zero_tile<BM, BN, uint32_t>(out, ldo, m0, m_lim, n0, N, 256);
+    return;
+  }
+  const Epilogue e = group_epilogue(ep, rg, g);
+  qgemm_tile<QT, BM, BN, BK>(A, lda, B + g * rg.b_group_stride, ldb, m0, n0, m_lim, N, K, e, out, ldo);
+}
+
+inline unsigned ragged_grid(int64_t M, int64_t N, int64_t G, int BM, int BN) {
+  const int64_t tiles = (M / BM + G + 1) * ((N + BN - 1) / BN);
+  const int64_t unit = 8 * kRaggedChunk;
+  return static_cast<unsigned>((tiles + unit - 1) / unit * unit);
+}
+
+template <int QT, int BM, int BN, int WGM, int WGN, int OUT>
+int launch_ragged_dma(const void* a, int64_t lda, const void* b, int64_t ldb, const Ragged& rg, int64_t M, int64_t N,
+                      int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  constexpr size_t smem = 2 * (BM + BN) * 128;
+  auto kern = qgemm_ragged_dma_kernel<QT, BM, BN, WGM, WGN, OUT>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  kern<<<dim3(ragged_grid(M, N, rg.G, BM, BN)), WGM * WGN * 64, smem, st>>>(
+      static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, rg, static_cast<int>(M),
+      static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);
+  return check_launch("ragged qgemm (dma)");
+}
+
+template <int QT, int BM, int BN, int WGM, int WGN>
+int dispatch_ragged_dma(const void* a, int64_t lda, const void* b, int64_t ldb, const Ragged& rg, int64_t M, int64_t N,
+                        int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  if (ep.out_dtype == QWIX_I32) {
+    if constexpr (QT == QWIX_INT8) return launch_ragged_dma<QT, BM, BN, WGM, WGN, QWIX_I32>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "int32 output needs int8 operands");
+  }
+  if (ep.out_dtype == QWIX_BF16) return launch_ragged_dma<QT, BM, BN, WGM, WGN, QWIX_BF16>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+  return launch_ragged_dma<QT, BM, BN, WGM, WGN, QWIX_F32>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+}
+
+template <int QT>
+int launch_ragged(const void* a, int64_t lda, const void* b, int64_t ldb, const Ragged& rg, int64_t M, int64_t N,
+                  int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  constexpr int BM = 128, BN = 128, BK = 128;
+  constexpr size_t smem = 2 * (BM + BN) * (BK + kPad);
+  auto kern = qgemm_ragged_kernel<QT, BM, BN, BK>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  kern<<<dim3(ragged_grid(M, N, rg.G, BM, BN)), 256, smem, st>>>(
+      static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, rg, static_cast<int>(M),
+      static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);
+  return check_launch("ragged qgemm");
 }
 
 }  // namespace
@@ -882,6 +1046,85 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
                       const void* sa, int sa_dtype, const void* sb, int sb_dtype, int acc_dtype, const int32_t* zu,
                       const int32_t* zv, void* out, int out_dtype, int64_t ldo, void* stream);
 
+// Dtype chain of the reference epilogue: int32 adopts the first scale's dtype (through f32); a
+// float accumulator starts in acc_dtype; each multiply happens in the promotion of both sides.
+static Epilogue make_epilogue(int qtype, const void* sa, int sa_dtype, const void* sb, int sb_dtype, int acc_dtype,
+                              const int32_t* zu, const int32_t* zv, int out_dtype) {
+  Epilogue ep{sa, sb, sa_dtype, sb_dtype, out_dtype, 0, 0, 0, zu, zv};
+  int cur = (qtype == QWIX_INT8) ? QWIX_I32 : acc_dtype;
+  if (cur == QWIX_BF16) ep.r0 = 1;
+  auto step = [&](const void* s, int s_dtype, int* r_after) {
+    if (!s) return;
+    const int t = (cur == QWIX_I32) ? s_dtype : ((cur == QWIX_F32 || s_dtype == QWIX_F32) ? QWIX_F32 : QWIX_BF16);
+    if (cur == QWIX_I32 && t == QWIX_BF16) ep.r0 = 1;
+    *r_after = (t == QWIX_BF16);
+    cur = t;
+  };
+  step(sa, sa_dtype, &ep.r1);
+  step(sb, sb_dtype, &ep.r2);
+  return ep;
+}
+
+// Argument checks shared by the dense and the ragged entry points.
+static int check_gemm_args(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M, int64_t N,
+                           int64_t K, const void* sa, int sa_dtype, const void* sb, int sb_dtype, int acc_dtype,
+                           const void* out, int out_dtype, int64_t ldo) {
+  if (!a || !b || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/b/out");
+  if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad GEMM shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
+                (long long)K);
+  if (qtype != QWIX_INT8 && qtype != QWIX_E4M3)
+    return fail(QWIX_ERR_UNSUPPORTED, "qgemm supports int8 x int8 and e4m3 x e4m3 operands (got qtype %d)", qtype);
+  if (K % 16 || lda % 16 || ldb % 16 || lda < K || ldb < K || !aligned16(a) || !aligned16(b))
+    return fail(QWIX_ERR_UNSUPPORTED, "K, lda, ldb must be multiples of 16 bytes and a/b 16-byte aligned "
+                "(K=%lld lda=%lld ldb=%lld)", (long long)K, (long long)lda, (long long)ldb);
+  if (ldo < N || !aligned16(out) || (N % 4 == 0 && ldo % 4 != 0))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad output leading dimension %lld for N=%lld", (long long)ldo, (long long)N);
+  auto ok_s = [](int d) { return d == QWIX_F32 || d == QWIX_BF16; };
+  if ((sa && !ok_s(sa_dtype)) || (sb && !ok_s(sb_dtype)))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "scale dtypes must be f32 or bf16");
+  if (out_dtype == QWIX_I32 && qtype != QWIX_INT8)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "raw int32 accumulators exist for int8 operands only");
+  if (out_dtype != QWIX_I32 && !ok_s(out_dtype)) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad out dtype %d", out_dtype);
+  if (qtype == QWIX_E4M3 && !ok_s(acc_dtype)) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad accumulator dtype %d", acc_dtype);
+  return QWIX_OK;
+}
+
+extern "C" int qwix_hip_qgemm_ragged(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t b_group_stride,
+                                     int qtype, int64_t M, int64_t N, int64_t K, const int32_t* group_sizes,
+                                     int64_t G, const void* sa, int sa_dtype, const void* sb, int sb_dtype,
+                                     int64_t sb_group_stride, int acc_dtype, void* out, int out_dtype, int64_t ldo,
+                                     void* stream) {
+  if (const int rc = check_gemm_args(a, lda, b, ldb, qtype, M, N, K, sa, sa_dtype, sb, sb_dtype, acc_dtype, out,
+                                     out_dtype, ldo))
+    return rc;
+  if (!group_sizes || G <= 0 || G > 65536)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "ragged qgemm needs 1..65536 group sizes (G=%lld)", (long long)G);
+  if (b_group_stride % 16 || b_group_stride < 0 || sb_group_stride < 0 || (sb_group_stride % 4 != 0 && N % 4 == 0))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad group strides (b: %lld bytes, sb: %lld elements)",
+                (long long)b_group_stride, (long long)sb_group_stride);
+  if (M * lda >= (int64_t{1} << 31) || N * ldb >= (int64_t{1} << 31) ||
+      (M / 128 + G + 1) * ((N + 127) / 128) >= (int64_t{1} << 31))
+    return fail(QWIX_ERR_UNSUPPORTED, "ragged qgemm: operand too large for 32-bit offsets (M*lda=%lld N*ldb=%lld)",
+                (long long)(M * lda), (long long)(N * ldb));
+  const Epilogue ep = make_epilogue(qtype, sa, sa_dtype, sb, sb_dtype, acc_dtype, nullptr, nullptr, out_dtype);
+  const Ragged rg{group_sizes, static_cast<int>(G), b_group_stride, sb_group_stride};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (K % 128 == 0) {
+    // 256-row tiles pay off once the average group is several tiles tall; 128-row tiles waste fewer rows
+    // at the ragged end of each group.
+    const bool big = M / G >= 768 && ((M + 255) / 256) * ((N + 255) / 256) >= 192;
+    if (qtype == QWIX_INT8) {
+      if (big) return dispatch_ragged_dma<QWIX_INT8, 256, 256, 2, 4>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+      return dispatch_ragged_dma<QWIX_INT8, 128, 128, 2, 2>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+    }
+    if (big) return dispatch_ragged_dma<QWIX_E4M3, 256, 256, 2, 4>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+    return dispatch_ragged_dma<QWIX_E4M3, 128, 128, 2, 2>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+  }
+  if (qtype == QWIX_INT8) return launch_ragged<QWIX_INT8>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+  return launch_ragged<QWIX_E4M3>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+}
+
 extern "C" int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M,
                               int64_t N, int64_t K, const void* sa, int sa_dtype, const void* sb, int sb_dtype,
                               int acc_dtype, void* out, int out_dtype, int64_t ldo, void* stream) {
@@ -903,38 +1146,10 @@ extern "C" int qwix_hip_qgemm_zp(const void* a, int64_t lda, const void* b, int6
 static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M, int64_t N, int64_t K,
                       const void* sa, int sa_dtype, const void* sb, int sb_dtype, int acc_dtype, const int32_t* zu,
                       const int32_t* zv, void* out, int out_dtype, int64_t ldo, void* stream) {
-  if (!a || !b || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/b/out");
-  if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX)
-    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad GEMM shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
-                (long long)K);
-  if (qtype != QWIX_INT8 && qtype != QWIX_E4M3)
-    return fail(QWIX_ERR_UNSUPPORTED, "qgemm supports int8 x int8 and e4m3 x e4m3 operands (got qtype %d)", qtype);
-  if (K % 16 || lda % 16 || ldb % 16 || lda < K || ldb < K || !aligned16(a) || !aligned16(b))
-    return fail(QWIX_ERR_UNSUPPORTED, "K, lda, ldb must be multiples of 16 bytes and a/b 16-byte aligned "
-                "(K=%lld lda=%lld ldb=%lld)", (long long)K, (long long)lda, (long long)ldb);
-  if (ldo < N || !aligned16(out) || (N % 4 == 0 && ldo % 4 != 0))
-    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad output leading dimension %lld for N=%lld", (long long)ldo, (long long)N);
-  auto ok_s = [](int d) { return d == QWIX_F32 || d == QWIX_BF16; };
-  if ((sa && !ok_s(sa_dtype)) || (sb && !ok_s(sb_dtype)))
-    return fail(QWIX_ERR_INVALID_ARGUMENT, "scale dtypes must be f32 or bf16");
-  if (out_dtype == QWIX_I32 && qtype != QWIX_INT8)
-    return fail(QWIX_ERR_INVALID_ARGUMENT, "raw int32 accumulators exist for int8 operands only");
-  if (out_dtype != QWIX_I32 && !ok_s(out_dtype)) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad out dtype %d", out_dtype);
-  if (qtype == QWIX_E4M3 && !ok_s(acc_dtype)) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad accumulator dtype %d", acc_dtype);
-  // Dtype chain of the reference epilogue: int32 adopts the first scale's dtype (through f32); a
-  // float accumulator starts in acc_dtype; each multiply happens in the promotion of both sides.
-  Epilogue ep{sa, sb, sa_dtype, sb_dtype, out_dtype, 0, 0, 0, zu, zv};
-  int cur = (qtype == QWIX_INT8) ? QWIX_I32 : acc_dtype;
-  if (cur == QWIX_BF16) ep.r0 = 1;
-  auto step = [&](const void* s, int s_dtype, int* r_after) {
-    if (!s) return;
-    const int t = (cur == QWIX_I32) ? s_dtype : ((cur == QWIX_F32 || s_dtype == QWIX_F32) ? QWIX_F32 : QWIX_BF16);
-    if (cur == QWIX_I32 && t == QWIX_BF16) ep.r0 = 1;
-    *r_after = (t == QWIX_BF16);
-    cur = t;
-  };
-  step(sa, sa_dtype, &ep.r1);
-  step(sb, sb_dtype, &ep.r2);
+  if (const int rc = check_gemm_args(a, lda, b, ldb, qtype, M, N, K, sa, sa_dtype, sb, sb_dtype, acc_dtype, out,
+                                     out_dtype, ldo))
+    return rc;
+  const Epilogue ep = make_epilogue(qtype, sa, sa_dtype, sb, sb_dtype, acc_dtype, zu, zv, out_dtype);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (M <= 32 && K % 128 == 0 && 16 * lda < (int64_t{1} << 31) && 64 * ldb < (int64_t{1} << 31)) {
     if (qtype == QWIX_INT8) return launch_skinny<QWIX_INT8>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);

@@ -1,0 +1,161 @@
+"""GPU parity: ragged (mixture-of-experts) quantized GEMM through qwix_amd.ragged_dot vs the CPU oracle.
+
+int8 x int8: the int32 sums are exact and the epilogue is elementwise, so outputs are compared bit for
+bit.  e4m3 x e4m3: the matrix instruction's internal accumulation differs from the oracle's single
+rounding of an exact sum (up to 1e-4 of the largest output), so outputs are compared at rtol 1e-2 for
+bf16 results and 1e-3 for f32 results, the tolerances of the dense fp8 GEMM tests."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import qwix_oracle as O
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+
+def _how(qtype, channelwise, tiled=None):
+  from qwix_amd.core import qarray
+  return (qarray.HowToQuantize(qtype=qtype, channelwise_axes=list(channelwise), tiled_axes=dict(tiled or {})),
+          O.HowToQuantize(qtype=qtype, channelwise_axes=list(channelwise), tiled_axes=dict(tiled or {})))
+
+
+def _quantized(shape, dtype, seed, how, scale=1.0):
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make(shape, dtype, seed=seed, scale=scale)
+  q = qarray.quantize(x_t, how[0])
+  oq = O.quantize(O.FArr(x_np, dtype), how[1])
+  util.assert_qarray_equal(q, oq, 'operand')
+  return q, oq
+
+
+def _sizes(t):
+  return torch.tensor(t, dtype=torch.int32, device=util.DEV)
+
+
+def _check_exact(out, want):
+  got = util.f32np(out)
+  assert tuple(got.shape) == tuple(want.v.shape)
+  bad = np.flatnonzero(got.ravel() != want.v.ravel())
+  assert bad.size == 0, f'{bad.size} outputs differ: {got.ravel()[bad[:5]]} vs {want.v.ravel()[bad[:5]]}'
+
+
+INT8_CASES = [
+    # name, (M, K, G, N), group sizes, lhs channelwise, rhs channelwise, rhs tiled
+    ('per-tensor', (128, 256, 4, 64), (64, 32, 16, 16), (), (), None),
+    ('channelwise', (128, 256, 4, 64), (128, 100, 0, 28), (0,), (2,), None),
+    ('group+channel', (128, 256, 4, 64), (50, 50, 28, 0), (0,), (0, 2), None),
+    ('group only', (128, 256, 4, 64), (128, 0, 0, 0), (), (0,), None),
+    ('short of M', (300, 384, 5, 200), (10, 0, 130, 1, 70), (0,), (0, 2), None),
+    ('tile edges', (700, 128, 3, 260), (128, 129, 256), (0,), (0, 2), None),
+    ('K not a multiple of 128', (200, 80, 3, 72), (60, 0, 100), (0,), (0, 2), None),
+    ('many groups', (1000, 256, 64, 136), tuple((i * 7) % 31 for i in range(64)), (0,), (0, 2), None),
+    ('k tiled', (128, 256, 4, 512), (10, 20, 30, 68), (0,), (0, 2), {1: 128}),
+    ('k tiled, shared over groups', (128, 256, 4, 512), (10, 20, 30, 68), (0,), (2,), {1: 128}),
+    ('k and n tiled', (128, 256, 4, 512), (10, 20, 30, 68), (0,), (0,), {1: 128, 2: 128}),
+    ('big groups', (2100, 512, 2, 2304), (1100, 900), (0,), (0, 2), None),
+]
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('name,shape,sizes,lcw,rcw,rtiled', INT8_CASES)
+def test_ragged_dot_int8_bit_exact(name, shape, sizes, lcw, rcw, rtiled, dtype):
+  import qwix_amd
+  print('case ragged int8', name, shape, sizes, dtype, flush=True)
+  M, K, G, N = shape
+  xq, oxq = _quantized((M, K), dtype, 100 + M, _how('int8', lcw))
+  wq, owq = _quantized((G, K, N), dtype, 200 + N, _how('int8', rcw, rtiled), scale=0.05)
+  out = qwix_amd.ragged_dot(xq, wq, _sizes(sizes))
+  torch.cuda.synchronize()
+  _check_exact(out, O.ragged_dot(oxq, owq, sizes))
+
+
+def test_ragged_dot_both_sides_k_tiled():
+  import qwix_amd
+  xq, oxq = _quantized((128, 256), O.BF16, 7, _how('int8', (0,), {1: 128}))
+  wq, owq = _quantized((4, 256, 512), O.BF16, 8, _how('int8', (0, 2), {1: 128}), scale=0.05)
+  out = qwix_amd.ragged_dot(xq, wq, _sizes((10, 20, 30, 68)))
+  _check_exact(out, O.ragged_dot(oxq, owq, (10, 20, 30, 68)))
+  bad, _ = _quantized((128, 256), O.BF16, 7, _how('int8', (0,), {1: 64}))
+  with pytest.raises(ValueError, match='same tile size'):
+    qwix_amd.ragged_dot(bad, wq, _sizes((10, 20, 30, 68)))
+
+
+def test_ragged_dot_weights_stored_k_contiguous():
+  """A weight kept as (G, N, K) storage and handed over as its (G, K, N) view is used in place."""
+  import qwix_amd
+  from qwix_amd.core.qarray import QArray
+  xq, oxq = _quantized((256, 256), O.BF16, 17, _how('int8', (0,)))
+  wq, owq = _quantized((3, 256, 192), O.BF16, 18, _how('int8', (0, 2)), scale=0.05)
+  stored = wq.qvalue.permute(0, 2, 1).contiguous()
+  view = QArray(stored.permute(0, 2, 1), wq.scale, None, wq.qtype)
+  out = qwix_amd.ragged_dot(xq, view, _sizes((100, 56, 100)))
+  _check_exact(out, O.ragged_dot(oxq, owq, (100, 56, 100)))
+
+
+def test_ragged_dot_raw_int8_gives_int32():
+  import qwix_amd
+  rng = util.rng(3)
+  a = rng.integers(-128, 128, (260, 128)).astype(np.int8)
+  b = rng.integers(-128, 128, (3, 128, 136)).astype(np.int8)
+  sizes = (130, 0, 100)
+  out = qwix_amd.ragged_dot(torch.from_numpy(a).to(util.DEV), torch.from_numpy(b).to(util.DEV), _sizes(sizes))
+  assert out.dtype == torch.int32
+  assert np.array_equal(out.cpu().numpy(), O.ragged_dot(a, b, sizes))
+
+
+def test_ragged_dot_out_of_range_sizes_are_clamped():
+  """Negative sizes count as empty groups and a group that would pass the last row is cut off there
+  (the kernel takes group_sizes from device memory and must stay inside the operands whatever it holds)."""
+  import qwix_amd
+  xq, oxq = _quantized((200, 128), O.BF16, 27, _how('int8', (0,)))
+  wq, owq = _quantized((4, 128, 64), O.BF16, 28, _how('int8', (0, 2)), scale=0.05)
+  out = qwix_amd.ragged_dot(xq, wq, _sizes((50, -3, 400, 10)))
+  _check_exact(out, O.ragged_dot(oxq, owq, (50, 0, 150, 0)))
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('shape,sizes,rcw', [((128, 256, 4, 64), (128, 100, 0, 28), (2,)),
+                                             ((520, 512, 6, 384), (100, 3, 0, 257, 60, 50), (0, 2))])
+def test_ragged_dot_fp8(shape, sizes, rcw, dtype):
+  import qwix_amd
+  M, K, G, N = shape
+  xq, oxq = _quantized((M, K), dtype, 300 + M, _how(O.E4M3, (0,)))
+  wq, owq = _quantized((G, K, N), dtype, 400 + N, _how(O.E4M3, rcw), scale=0.05)
+  out = qwix_amd.ragged_dot(xq, wq, _sizes(sizes))
+  want = O.ragged_dot(oxq, owq, sizes).v
+  got = util.f32np(out)
+  tol = 1e-2 if dtype == O.BF16 else 1e-3
+  np.testing.assert_allclose(got, want, rtol=tol, atol=tol * np.abs(want).max())
+  assert np.all(got[min(sum(sizes), M):] == 0)
+
+
+def test_ragged_dot_dequantize_first_path():
+  """A raw float lhs or a zero point sends the call to the dequantize-first path (ragged_dot.py:278-292)."""
+  import qwix_amd
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make((128, 256), O.F32, seed=31)
+  wq, owq = _quantized((4, 256, 64), O.F32, 32, _how('int8', (0, 2)), scale=0.05)
+  sizes = (50, 50, 28, 0)
+  out = qwix_amd.ragged_dot(x_t, wq, _sizes(sizes))
+  want = O.ragged_dot(O.FArr(x_np, O.F32), owq, sizes).v
+  np.testing.assert_allclose(util.f32np(out), want, rtol=1e-4, atol=1e-4 * np.abs(want).max())
+  xz = qarray.quantize(x_t, qarray.HowToQuantize(qtype='int8', calibration_method='minmax'))
+  oxz = O.quantize(O.FArr(x_np, O.F32), O.HowToQuantize(qtype='int8', calibration_method='minmax'))
+  out = qwix_amd.ragged_dot(xz, wq, _sizes(sizes))
+  want = O.ragged_dot(oxz, owq, sizes).v
+  np.testing.assert_allclose(util.f32np(out), want, rtol=1e-4, atol=1e-4 * np.abs(want).max())
+
+
+def test_ragged_dot_errors():
+  import qwix_amd
+  from qwix_amd.core import ragged_dot as rd
+  xq, _ = _quantized((128, 256), O.BF16, 41, _how('int8', (0,)))
+  wq, _ = _quantized((4, 256, 64), O.BF16, 42, _how('int8', (0, 2)), scale=0.05)
+  with pytest.raises(ValueError, match='one entry per group'):
+    qwix_amd.ragged_dot(xq, wq, _sizes((64, 64)))
+  with pytest.raises(NotImplementedError, match='group_offset'):
+    qwix_amd.ragged_dot(xq, wq, _sizes((64, 64, 0, 0)), group_offset=_sizes((0,)))
+  dn = rd.RaggedDotDimensionNumbers((((0,), (1,)), ((), ())), (1,), (0,))
+  with pytest.raises(NotImplementedError, match='dimension numbers'):
+    qwix_amd.ragged_dot_general(xq, wq, _sizes((64, 64, 0, 0)), dn)
