@@ -464,6 +464,70 @@ class HadamardQdot(Workload):
     return {'workload': self.name, 'M': self.M, 'K': self.K, 'N': self.N, 'group': 128}
 
 
+class RaggedQdot(Workload):
+  """Mixture-of-experts matmul: the tokens are sorted by expert (uneven groups, sizes in device memory);
+  per-token int8 activation quantize + one ragged MFMA GEMM against G per-channel int8 expert weights."""
+
+  bound = 'mfma'
+
+  def __init__(self, name, M, K, N, G, qtype='int8'):
+    self.name, self.M, self.K, self.N, self.G, self.qtype = name, M, K, N, G, qtype
+    self.dtype = 'int8' if qtype == 'int8' else 'f8e4m3'
+    self.metric = self.dtype + ' ragged qdot TOPS (w8a8 mixture-of-experts matmul, activation quantize included)'
+    self.unit = 'TOPS'
+    self.kernel_name = 'qgemm_ragged_dma_kernel'
+
+  def setup(self, dev):
+    import numpy as np
+    import torch
+    from qwix_amd.core import qarray
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(5000 + self.G)
+    self.x = torch.randn(self.M, self.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    # expert weights, quantized once per (expert, output channel) and kept K-contiguous: (G, N, K)
+    self.b = torch.empty(self.G, self.N, self.K, dtype=torch.int8 if self.qtype == 'int8' else torch.float8_e4m3fn, device=dev)
+    self.sb = torch.empty(self.G, self.N, dtype=torch.bfloat16, device=dev)
+    for e in range(self.G):
+      w = (torch.randn(self.K, self.N, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(dev)
+      wq = qarray.quantize(w, qarray.HowToQuantize(qtype=self.qtype, channelwise_axes=[1]))
+      self.b[e].copy_(wq.qvalue.permute(1, 0))
+      self.sb[e].copy_(wq.scale.reshape(-1))
+    # uneven routing: sizes drawn around M / G, every token assigned
+    r = np.random.Generator(np.random.PCG64(17)).dirichlet(np.full(self.G, 8.0))
+    sizes = np.floor(r * self.M).astype(np.int64)
+    sizes[-1] += self.M - sizes.sum()
+    self.sizes_host = sizes.tolist()
+    self.sizes = torch.tensor(self.sizes_host, dtype=torch.int32, device=dev)
+    self.xq = torch.empty(self.M, self.K, dtype=self.b.dtype, device=dev)
+    self.sa = torch.empty(self.M, dtype=torch.bfloat16, device=dev)
+    self.out = torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev)
+    self.qt = L.INT8 if self.qtype == 'int8' else L.E4M3
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, i=0):
+    L = self.L
+    L.call('qwix_hip_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, 1, self.K, self.qt, L.ABSMAX, 0.0,
+           L.LAYOUT_NATURAL, self.xq.data_ptr(), self.sa.data_ptr(), None, None, 0, self.stream)
+    self.kernel(i)
+
+  def kernel(self, i=0):
+    L = self.L
+    L.call('qwix_hip_qgemm_ragged', self.xq.data_ptr(), self.K, self.b.data_ptr(), self.K, self.N * self.K, self.qt,
+           self.M, self.N, self.K, self.sizes.data_ptr(), self.G, self.sa.data_ptr(), L.BF16, self.sb.data_ptr(),
+           L.BF16, self.N, L.BF16, self.out.data_ptr(), L.BF16, self.N, self.stream)
+
+  def work_per_step(self):
+    return 2.0 * self.M * self.N * self.K
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'tokens': self.M, 'K': self.K, 'N': self.N, 'experts': self.G,
+            'group_sizes': f'uneven, {min(self.sizes_host)}..{max(self.sizes_host)} rows (device memory)',
+            'weight': 'per-expert per-output-channel ' + self.qtype + ' (pre-quantized)', 'out': 'bf16'}
+
+
 WORKLOADS = {
     'c3_int8_w8a8_4096': lambda: QdotW8A8('c3_int8_w8a8_4096', 4096, 4096, 4096, 'int8'),
     'c4_fp8_w8a8_ffn': lambda: QdotW8A8('c4_fp8_w8a8_ffn', 8192, 8192, 28672, 'float8_e4m3fn'),
@@ -480,11 +544,15 @@ WORKLOADS = {
     'c5_fwht_quantize_act': lambda: FwhtQuantize('c5_fwht_quantize_act', 2048, 8192),
     'fwht_quantize_8192x8192': lambda: FwhtQuantize('fwht_quantize_8192x8192', 8192, 8192),
     'plain_copy_1g': lambda: PlainCopy('plain_copy_1g', 1 << 30),
+    'moe_ragged_int8_8x1024': lambda: RaggedQdot('moe_ragged_int8_8x1024', 8192, 4096, 14336, 8),
+    'moe_ragged_int8_64x128': lambda: RaggedQdot('moe_ragged_int8_64x128', 8192, 2048, 4096, 64),
+    'moe_ragged_fp8_8x1024': lambda: RaggedQdot('moe_ragged_fp8_8x1024', 8192, 4096, 14336, 8, 'float8_e4m3fn'),
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
 }
 DEFAULT = 'c3_int8_w8a8_4096'
 EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16',
-         'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192']
+         'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'moe_ragged_int8_8x1024',
+         'moe_ragged_int8_64x128']
 
 
 def _blas_threads() -> int:
