@@ -156,6 +156,20 @@ QWIX_API int qwix_hip_qgemm_ragged(const void* a, int64_t lda, const void* b, in
                           const void* sb, int sb_dtype, int64_t sb_group_stride, int acc_dtype,
                           void* out, int out_dtype, int64_t ldo, void* stream);
 
+/* Batched quantized GEMM: `batch` independent problems of one shape in a single launch.  Replaces
+ * the batch dimensions of _fast_dot_general (qwix/_src/core/dot_general.py:135-261: lhs_ba / rhs_ba
+ * of dimension_numbers; the scale transposes of :79-90 put the batch axes first), e.g. the
+ * 'bqd,bkd->bqk' contractions of attention.  Problem z uses a + z*a_batch_stride and
+ * b + z*b_batch_stride (bytes), scale vectors sa + z*sa_batch_stride and sb + z*sb_batch_stride
+ * (elements; 0 = one vector shared by all problems) and writes out + z*out_batch_stride (elements).
+ * Everything else as qwix_hip_qgemm. */
+QWIX_API int qwix_hip_qgemm_batched(const void* a, int64_t lda, int64_t a_batch_stride, const void* b,
+                           int64_t ldb, int64_t b_batch_stride, int qtype, int64_t batch, int64_t M,
+                           int64_t N, int64_t K, const void* sa, int sa_dtype, int64_t sa_batch_stride,
+                           const void* sb, int sb_dtype, int64_t sb_batch_stride, int acc_dtype,
+                           void* out, int out_dtype, int64_t ldo, int64_t out_batch_stride,
+                           void* stream);
+
 /* out[r] = sum_k q[r*ld + k] for int8 rows (K % 16 == 0): the K-sums qwix_hip_qgemm_zp needs
  * (the reference obtains them as a dot_general against the broadcast zero point,
  * dot_general.py:233-239,246-252). */

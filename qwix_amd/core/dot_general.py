@@ -225,6 +225,61 @@ def _over_batch(fn, lhs, rhs, dimension_numbers, **kwargs) -> torch.Tensor:
   return torch.stack(outs).reshape(*bshape, *outs[0].shape)
 
 
+def _batched_qgemm(lhs, rhs, dimension_numbers, preferred_element_type):
+  """All batch elements in one launch (qwix_hip_qgemm_batched) for the common case: two QArrays of int8
+  or e4m3 values with per-row / per-column scales and no zero point.  Returns None when the operands
+  need the general route (one launch per batch element)."""
+  if not (isinstance(lhs, QArray) and isinstance(rhs, QArray)):
+    return None
+  if lhs.zero_point is not None or rhs.zero_point is not None:
+    return None
+  if isinstance(lhs.qvalue, Int4Tensor) or isinstance(rhs.qvalue, Int4Tensor):
+    return None
+  lq, rq = _qtype_of(lhs), _qtype_of(rhs)
+  if (lq, rq) == (numerics.INT8, numerics.INT8):
+    qt = _lib.INT8
+  elif (lq, rq) == (numerics.E4M3, numerics.E4M3):
+    qt = _lib.E4M3
+  else:
+    return None
+  (lca, rca), (lba, rba) = dimension_numbers
+  lca, rca, lba, rba = ([int(a) for a in x] for x in (lca, rca, lba, rba))
+  lshape, rshape = tuple(lhs.shape), tuple(rhs.shape)
+  if len(lba) != len(rba) or [lshape[a] for a in lba] != [rshape[a] for a in rba]:
+    return None  # the general route reports the error
+  if len(lca) != len(rca) or not lca or [lshape[a] for a in lca] != [rshape[a] for a in rca]:
+    return None
+  if any(lhs.scale.shape[a] != 1 for a in lca) or any(rhs.scale.shape[a] != 1 for a in rca):
+    return None  # sub-channel scales
+  lfree = [a for a in range(len(lshape)) if a not in lca and a not in lba]
+  rfree = [a for a in range(len(rshape)) if a not in rca and a not in rba]
+  bshape = [lshape[a] for a in lba]
+  Bt, M, N, K = (math.prod(bshape), math.prod(lshape[a] for a in lfree), math.prod(rshape[a] for a in rfree),
+                 math.prod(lshape[a] for a in lca))
+  if not (0 < Bt <= 65535) or M == 0 or N == 0 or K % 16:
+    return None
+  acc_t, res_t = qarray.get_accumulator_and_result_type(lhs, rhs, preferred_element_type=preferred_element_type)
+
+  def values(q, order, rows):
+    v = q.qvalue.permute(*order)
+    return (v if v.is_contiguous() else v.contiguous()).reshape(Bt, rows, K)
+
+  def scales(q, shape, contracting, order, rows):
+    s = q.scale.expand(*[1 if a in contracting else shape[a] for a in range(len(shape))])
+    return s.permute(*order).reshape(Bt, rows).contiguous()
+
+  a = values(lhs, lba + lfree + lca, M)
+  b = values(rhs, rba + rfree + rca, N)
+  sa = scales(lhs, lshape, lca, lba + lfree + lca, M)
+  sb = scales(rhs, rshape, rca, rba + rfree + rca, N)
+  out = torch.empty(Bt, M, N, dtype=res_t, device=a.device)
+  _lib.call('qwix_hip_qgemm_batched', a.data_ptr(), K, M * K, b.data_ptr(), K, N * K, qt, Bt, M, N, K,
+            sa.data_ptr(), _lib.float_tag(sa.dtype), M, sb.data_ptr(), _lib.float_tag(sb.dtype), N,
+            _tag_of(acc_t) if acc_t != torch.int32 else 0, out.data_ptr(), _tag_of(res_t), N, M * N,
+            _lib.stream_of(a))
+  return out.reshape(*bshape, *[lshape[a] for a in lfree], *[rshape[a] for a in rfree])
+
+
 def _tag_of(dtype: torch.dtype) -> int:
   if dtype == torch.int32:
     return _lib.I32
@@ -250,6 +305,9 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   if len(dimension_numbers[1][0]) or len(dimension_numbers[1][1]):
     if return_accumulators:
       raise NotImplementedError('raw accumulators are not returned for batched contractions')
+    out = _batched_qgemm(lhs, rhs, dimension_numbers, preferred_element_type)
+    if out is not None:
+      return out
     return _over_batch(_fast_dot_general, lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type,
                        exact=exact)
   c = _Canon(lhs, rhs, dimension_numbers)

@@ -860,6 +860,100 @@ int launch_ragged(const void* a, int64_t lda, const void* b, int64_t ldb, const 
   return check_launch("ragged qgemm");
 }
 
+// ------------------------------------------------------------------------------------------------
+// Batched GEMM: blockIdx.y selects one of `batch` independent problems of the same shape (the batch
+// axes of dot_general); operands, scale vectors and outputs of consecutive problems are a fixed
+// stride apart.  Same tile bodies as the dense kernels.
+struct Batched {
+  int64_t a_stride, b_stride;    // bytes
+  int64_t sa_stride, sb_stride;  // elements (0: the vector is shared by all problems)
+  int64_t out_stride;            // elements
+};
+
+__device__ __forceinline__ Epilogue batch_epilogue(const Epilogue& ep, const Batched& bs, int z) {
+  Epilogue e = ep;
+  if (ep.sa != nullptr)
+    e.sa = static_cast<const uint8_t*>(ep.sa) + z * bs.sa_stride * (ep.sa_dtype == QWIX_BF16 ? 2 : 4);
+  if (ep.sb != nullptr)
+    e.sb = static_cast<const uint8_t*>(ep.sb) + z * bs.sb_stride * (ep.sb_dtype == QWIX_BF16 ? 2 : 4);
+  return e;
+}
+
+template <int QT, int BM, int BN, int WGM, int WGN, int OUT>
+__global__ void __launch_bounds__(WGM * WGN * 64)
+    qgemm_batched_dma_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
+                             Batched bs, int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  const int z = blockIdx.y;
+  int tile_m, tile_n;
+  tile_coords((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
+  const Epilogue e = batch_epilogue(ep, bs, z);
+  constexpr int ES = OUT == QWIX_BF16 ? 2 : 4;
+  qgemm_dma_tile<QT, BM, BN, WGM, WGN, OUT, (OUT == QWIX_I32 ? 0 : 2)>(
+      A + z * bs.a_stride, lda, B + z * bs.b_stride, ldb, tile_m * BM, tile_n * BN, M, N, K, e,
+      out + z * bs.out_stride * ES, ldo);
+}
+
+template <int QT, int BM, int BN, int BK>
+__global__ void __launch_bounds__(256)
+    qgemm_batched_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
+                         Batched bs, int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  const int z = blockIdx.y;
+  int tile_m, tile_n;
+  tile_coords((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
+  const Epilogue e = batch_epilogue(ep, bs, z);
+  const int es = ep.out_dtype == QWIX_BF16 ? 2 : 4;
+  qgemm_tile<QT, BM, BN, BK>(A + z * bs.a_stride, lda, B + z * bs.b_stride, ldb, tile_m * BM, tile_n * BN, M, N, K, e,
+                             out + z * bs.out_stride * es, ldo);
+}
+
+template <int QT, int OUT>
+int launch_batched_dma(const void* a, int64_t lda, const void* b, int64_t ldb, const Batched& bs, int64_t batch,
+                       int64_t M, int64_t N, int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  constexpr int BM = 128, BN = 128;
+  constexpr size_t smem = 2 * (BM + BN) * 128;
+  auto kern = qgemm_batched_dma_kernel<QT, BM, BN, 2, 2, OUT>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  kern<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), 256, smem, st>>>(
+      static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, bs, static_cast<int>(M),
+      static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);
+  return check_launch("batched qgemm (dma)");
+}
+
+template <int QT>
+int launch_batched(const void* a, int64_t lda, const void* b, int64_t ldb, const Batched& bs, int64_t batch,
+                   int64_t M, int64_t N, int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  if (K % 128 == 0) {
+    if (ep.out_dtype == QWIX_I32) {
+      if constexpr (QT == QWIX_INT8) return launch_batched_dma<QT, QWIX_I32>(a, lda, b, ldb, bs, batch, M, N, K, ep, out, ldo, st);
+      return fail(QWIX_ERR_INVALID_ARGUMENT, "int32 output needs int8 operands");
+    }
+    if (ep.out_dtype == QWIX_BF16) return launch_batched_dma<QT, QWIX_BF16>(a, lda, b, ldb, bs, batch, M, N, K, ep, out, ldo, st);
+    return launch_batched_dma<QT, QWIX_F32>(a, lda, b, ldb, bs, batch, M, N, K, ep, out, ldo, st);
+  }
+  constexpr int BM = 128, BN = 128, BK = 128;
+  constexpr size_t smem = 2 * (BM + BN) * (BK + kPad);
+  auto kern = qgemm_batched_kernel<QT, BM, BN, BK>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  kern<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), 256, smem, st>>>(
+      static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, bs, static_cast<int>(M),
+      static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);
+  return check_launch("batched qgemm");
+}
+
 }  // namespace
 }  // namespace qwix
 
@@ -1141,6 +1235,32 @@ extern "C" int qwix_hip_qgemm_zp(const void* a, int64_t lda, const void* b, int6
     return fail(QWIX_ERR_INVALID_ARGUMENT, "zero-point corrected output must be f32 or bf16");
   return qgemm_impl(a, lda, b, ldb, QWIX_INT8, M, N, K, sa, sa_dtype, sb, sb_dtype, 0, zu, zv, out, out_dtype, ldo,
                     stream);
+}
+
+extern "C" int qwix_hip_qgemm_batched(const void* a, int64_t lda, int64_t a_batch_stride, const void* b, int64_t ldb,
+                                      int64_t b_batch_stride, int qtype, int64_t batch, int64_t M, int64_t N,
+                                      int64_t K, const void* sa, int sa_dtype, int64_t sa_batch_stride,
+                                      const void* sb, int sb_dtype, int64_t sb_batch_stride, int acc_dtype,
+                                      void* out, int out_dtype, int64_t ldo, int64_t out_batch_stride,
+                                      void* stream) {
+  if (const int rc = check_gemm_args(a, lda, b, ldb, qtype, M, N, K, sa, sa_dtype, sb, sb_dtype, acc_dtype, out,
+                                     out_dtype, ldo))
+    return rc;
+  if (batch <= 0 || batch > 65535)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "batched qgemm needs 1..65535 problems (batch=%lld)", (long long)batch);
+  if (a_batch_stride % 16 || b_batch_stride % 16 || a_batch_stride < 0 || b_batch_stride < 0 || sa_batch_stride < 0 ||
+      sb_batch_stride < 0 || out_batch_stride < 0 || (N % 4 == 0 && (sb_batch_stride % 4 || out_batch_stride % 4)))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad batch strides (a %lld b %lld bytes; sa %lld sb %lld out %lld elements)",
+                (long long)a_batch_stride, (long long)b_batch_stride, (long long)sa_batch_stride,
+                (long long)sb_batch_stride, (long long)out_batch_stride);
+  if (M * lda >= (int64_t{1} << 31) || N * ldb >= (int64_t{1} << 31))
+    return fail(QWIX_ERR_UNSUPPORTED, "batched qgemm: one problem must fit 32-bit offsets (M*lda=%lld N*ldb=%lld)",
+                (long long)(M * lda), (long long)(N * ldb));
+  const Epilogue ep = make_epilogue(qtype, sa, sa_dtype, sb, sb_dtype, acc_dtype, nullptr, nullptr, out_dtype);
+  const Batched bs{a_batch_stride, b_batch_stride, sa_batch_stride, sb_batch_stride, out_batch_stride};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (qtype == QWIX_INT8) return launch_batched<QWIX_INT8>(a, lda, b, ldb, bs, batch, M, N, K, ep, out, ldo, st);
+  return launch_batched<QWIX_E4M3>(a, lda, b, ldb, bs, batch, M, N, K, ep, out, ldo, st);
 }
 
 static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M, int64_t N, int64_t K,

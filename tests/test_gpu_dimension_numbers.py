@@ -39,6 +39,8 @@ CASES = [
     ('td,dn->nt', (50, 128), (128, 70)),               # permuted output
     ('dt,dn->tn', (128, 50), (128, 70)),               # contracting axis of the lhs is not the last one
     ('bdq,bkd->bkq', (2, 64, 10), (2, 12, 64)),        # batch + leading contraction + permuted output
+    ('bqd,bkd->bqk', (4, 200, 128), (4, 136, 128)),    # K a multiple of 128: the direct-to-LDS batched kernel, ragged tile edges
+    ('bhqd,bhkd->bhqk', (2, 2, 130, 256), (2, 2, 260, 256)),
 ]
 
 
@@ -55,6 +57,31 @@ def test_einsum_general_dimension_numbers_bit_exact(einsum_str, lshape, rshape, 
   got = util.f32np(out)
   bad = np.flatnonzero(got.ravel() != want.v.ravel())
   assert bad.size == 0, f'{bad.size} outputs differ: {got.ravel()[bad[:5]]} vs {want.v.ravel()[bad[:5]]}'
+
+
+def test_batch_axes_take_one_launch(monkeypatch):
+  """Quantized operands with batch axes go through the batched kernel, not through one launch per element,
+  and both routes give the same bits (int8) / the same values to the fp8 tolerance."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  dn = (((2,), (2,)), ((0,), (0,)))
+  for qtype in ('int8', O.E4M3):
+    x_np, x_t = util.make((3, 70, 128), O.BF16, seed=31)
+    w_np, w_t = util.make((3, 50, 128), O.BF16, seed=32)
+    xq = qarray.quantize(x_t, qarray.HowToQuantize(qtype=qtype, channelwise_axes=[0, 1]))
+    wq = qarray.quantize(w_t, qarray.HowToQuantize(qtype=qtype, channelwise_axes=[0, 1]))
+    looped = dg._over_batch(dg._fast_dot_general, xq, wq, dn)
+    with monkeypatch.context() as m:
+      m.setattr(dg, '_over_batch', lambda *a, **k: (_ for _ in ()).throw(AssertionError('looped over the batch')))
+      out = dg.dot_general(xq, wq, dn)
+    assert tuple(out.shape) == (3, 70, 50) and out.dtype == torch.bfloat16
+    if qtype == 'int8':
+      assert torch.equal(out, looped)
+      oxq = O.quantize(O.FArr(x_np, O.BF16), O.HowToQuantize(qtype=qtype, channelwise_axes=[0, 1]))
+      owq = O.quantize(O.FArr(w_np, O.BF16), O.HowToQuantize(qtype=qtype, channelwise_axes=[0, 1]))
+      assert np.array_equal(util.f32np(out), O.dot_general(oxq, owq, dn).v)
+    else:
+      np.testing.assert_allclose(util.f32np(out), util.f32np(looped), rtol=1e-2, atol=1e-2 * float(looped.abs().max()))
 
 
 def test_batched_dot_general_on_the_dequantize_path():
