@@ -74,7 +74,7 @@ class QdotW8A8(Workload):
     self.dtype = 'int8' if qtype == 'int8' else 'f8e4m3'
     self.metric = ('int8' if qtype == 'int8' else 'fp8') + ' qdot TOPS (dynamic-range w8a8, activation quantize included)'
     self.unit = 'TOPS'
-    self.kernel_name = 'qgemm_dma_kernel'
+    self.kernel_name = 'qgemm_pp_kernel' if ((M + 255) // 256) * ((N + 255) // 256) >= 192 and K >= 256 else 'qgemm_dma_kernel'
 
   def setup(self, dev):
     import torch
@@ -475,7 +475,8 @@ class RaggedQdot(Workload):
     self.dtype = 'int8' if qtype == 'int8' else 'f8e4m3'
     self.metric = self.dtype + ' ragged qdot TOPS (w8a8 mixture-of-experts matmul, activation quantize included)'
     self.unit = 'TOPS'
-    self.kernel_name = 'qgemm_ragged_dma_kernel'
+    big = M // G >= 768 and ((M + 255) // 256) * ((N + 255) // 256) >= 192 and K >= 256
+    self.kernel_name = 'qgemm_ragged_pp_kernel' if big else 'qgemm_ragged_dma_kernel'
 
   def setup(self, dev):
     import numpy as np

@@ -355,6 +355,148 @@ __global__ void __launch_bounds__(256)
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),             \
                                    (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
 
+// The per-row and per-column scales of one wavefront's part of the tile, in the accumulator layout
+// (acc[i][j][r]: m = m_base + i*32 + lane%32, n = n_base + j*32 + 8*(r/4) + 4*(lane/32) + r%4).
+template <int OUT, int TM, int TN>
+__device__ __forceinline__ void fetch_scales(const Epilogue& ep, int m_base, int n_base, int M, int N, int lane,
+                                             float (&sav)[TM], float (&sbv)[TN][4][4]) {
+  if constexpr (OUT != QWIX_I32) {
+    const bool vec_ok = (N % 4 == 0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int m = m_base + i * 32 + (lane & 31);
+      sav[i] = (ep.sa != nullptr && m < M) ? load_scale(ep.sa, ep.sa_dtype, m) : 1.f;
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int n = n_base + j * 32 + 8 * qd + 4 * (lane >> 5);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sbv[j][qd][r] = 1.f;
+        if (ep.sb != nullptr) {
+          if (vec_ok && n < N) {  // n % 4 == 0: one 8- or 16-byte load
+            if (ep.sb_dtype == QWIX_BF16) {
+              const uint2 w = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(ep.sb) + n);
+              sbv[j][qd][0] = __uint_as_float(w.x << 16);
+              sbv[j][qd][1] = __uint_as_float(w.x & 0xFFFF0000u);
+              sbv[j][qd][2] = __uint_as_float(w.y << 16);
+              sbv[j][qd][3] = __uint_as_float(w.y & 0xFFFF0000u);
+            } else {
+              const float4 w = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(ep.sb) + n);
+              sbv[j][qd][0] = w.x; sbv[j][qd][1] = w.y; sbv[j][qd][2] = w.z; sbv[j][qd][3] = w.w;
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (n + r < N) sbv[j][qd][r] = load_scale(ep.sb, ep.sb_dtype, n + r);
+          }
+        }
+      }
+  }
+}
+
+template <int OUT, int EPI, int TM, int TN, int NWAVES, int LDS_BYTES, typename AccT>
+__device__ __forceinline__ void staged_epilogue(const AccT (&acc)[TM][TN], const float (&sav)[TM],
+                                                const float (&sbv)[TN][4][4], const Epilogue& ep, int m_base,
+                                                int n_base, int M, int N, uint8_t* __restrict__ out, int64_t ldo,
+                                                uint8_t* smem, int wave, int lane) {
+  constexpr int WTN = TN * 32;
+  // ---- epilogue.  acc[i][j][r]: m = m_base + i*32 + lane%32, n = n_base + j*32 + 8*(r/4) + 4*(lane/32) + r%4.
+  // The scaled values are staged through this wavefront's own slice of LDS, 32 rows at a time, and
+  // leave with 16-byte stores that cover whole 128-byte row segments (a direct store from the MFMA
+  // layout would write 16-byte pieces of 32 different rows per instruction).
+  using OutT = typename std::conditional<OUT == QWIX_BF16, uint16_t, uint32_t>::type;
+  constexpr int ES = sizeof(OutT);
+  constexpr int ROWB = WTN * ES + 16;            // staged row pitch in bytes (padded against bank conflicts)
+  constexpr int CPR = WTN * ES / 16;             // 16-byte chunks per staged row
+  constexpr int EPC = 16 / ES;                   // elements per chunk
+  static_assert(NWAVES * 32 * ROWB <= LDS_BYTES, "epilogue staging does not fit in LDS");
+  constexpr bool ZP = (EPI == 3);  // run-time rounding flags plus zero-point correction
+  const bool r0 = EPI >= 2 ? ep.r0 != 0 : EPI == 1, r1 = EPI >= 2 ? ep.r1 != 0 : EPI == 1,
+             r2 = EPI >= 2 ? ep.r2 != 0 : EPI == 1;
+  int zuv[TM];
+  if constexpr (ZP) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) zuv[i] = ep.zu[min(m_base + i * 32 + (lane & 31), M - 1)];
+  }
+  __syncthreads();  // every wavefront is done with the slabs; LDS becomes staging space
+  uint8_t* stg = smem + wave * (32 * ROWB);
+  const bool row_vec = (reinterpret_cast<uintptr_t>(out) % 16 == 0) && ((ldo * ES) % 16 == 0);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    float sa = 1.f;
+    if constexpr (OUT != QWIX_I32) sa = sav[i];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        uint8_t* dst = stg + (lane & 31) * ROWB + (j * 32 + 8 * qd + 4 * (lane >> 5)) * ES;
+        if constexpr (OUT == QWIX_I32) {
+          *reinterpret_cast<int4*>(dst) = make_int4(static_cast<int>(acc[i][j][4 * qd]), static_cast<int>(acc[i][j][4 * qd + 1]),
+                                                    static_cast<int>(acc[i][j][4 * qd + 2]), static_cast<int>(acc[i][j][4 * qd + 3]));
+        } else if constexpr (EPI == 1 && OUT == QWIX_BF16) {
+          // Every step rounds to bf16 and the result is bf16: round two values per v_cvt_pk_bf16_f32,
+          // and let the last rounding produce the packed output directly.
+          uint32_t w[2];
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            uint32_t pk = pack_bf16x2(static_cast<float>(acc[i][j][4 * qd + 2 * h]),
+                                      static_cast<float>(acc[i][j][4 * qd + 2 * h + 1]));
+            pk = pack_bf16x2(__uint_as_float(pk << 16) * sa, __uint_as_float(pk & 0xFFFF0000u) * sa);
+            w[h] = pack_bf16x2(__uint_as_float(pk << 16) * sbv[j][qd][2 * h],
+                               __uint_as_float(pk & 0xFFFF0000u) * sbv[j][qd][2 * h + 1]);
+          }
+          *reinterpret_cast<uint2*>(dst) = make_uint2(w[0], w[1]);
+        } else {
+          float v[4];
+          int zvv[4] = {0, 0, 0, 0};
+          if constexpr (ZP) {
+            const int n = n_base + j * 32 + 8 * qd + 4 * (lane >> 5);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) zvv[r] = ep.zv[min(n + r, N - 1)];
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float t;
+            if constexpr (ZP) t = static_cast<float>(static_cast<int>(acc[i][j][4 * qd + r]) - zuv[i] * zvv[r]);
+            else t = static_cast<float>(acc[i][j][4 * qd + r]);
+            if (r0) t = round_bf16(t);
+            t *= sa;
+            if (r1) t = round_bf16(t);
+            t *= sbv[j][qd][r];
+            if (r2) t = round_bf16(t);
+            v[r] = t;
+          }
+          if constexpr (OUT == QWIX_BF16)
+            *reinterpret_cast<uint2*>(dst) =
+                make_uint2(f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16),
+                           f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16));
+          else
+            *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+      }
+    // read back row-major: chunk c of the 32 x CPR grid -> row c / CPR, 16-byte column c % CPR
+#pragma unroll
+    for (int c0 = 0; c0 < 32 * CPR; c0 += 64) {
+      const int c = c0 + lane, row = c / CPR, cc = c % CPR;
+      const uint4 v = *reinterpret_cast<const uint4*>(stg + row * ROWB + cc * 16);
+      const int mo = m_base + i * 32 + row, no = n_base + cc * EPC;
+      if (mo < M && no < N) {
+        OutT* o = reinterpret_cast<OutT*>(out) + static_cast<int64_t>(mo) * ldo + no;
+        if (row_vec && no + EPC <= N) {
+          *reinterpret_cast<uint4*>(o) = v;
+        } else {
+          const OutT* e = reinterpret_cast<const OutT*>(&v);
+#pragma unroll
+          for (int t = 0; t < EPC; ++t)
+            if (no + t < N) o[t] = e[t];
+        }
+      }
+    }
+  }
+}
+
 template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI>
 __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, int64_t lda,
                                                const uint8_t* __restrict__ B, int64_t ldb, int m0, int n0, int M,
@@ -467,40 +609,7 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
   // The scale vectors are fetched before the main loop: at the start of the epilogue they would be a
   // cold two-microsecond round trip with nothing to hide behind.
   float sav[TM];
-  if constexpr (OUT != QWIX_I32) {
-    const bool vec_ok = (N % 4 == 0);
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int m = m_base + i * 32 + (lane & 31);
-      sav[i] = (ep.sa != nullptr && m < M) ? load_scale(ep.sa, ep.sa_dtype, m) : 1.f;
-    }
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        const int n = n_base + j * 32 + 8 * qd + 4 * (lane >> 5);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) sbv[j][qd][r] = 1.f;
-        if (ep.sb != nullptr) {
-          if (vec_ok && n < N) {  // n % 4 == 0: one 8- or 16-byte load
-            if (ep.sb_dtype == QWIX_BF16) {
-              const uint2 w = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(ep.sb) + n);
-              sbv[j][qd][0] = __uint_as_float(w.x << 16);
-              sbv[j][qd][1] = __uint_as_float(w.x & 0xFFFF0000u);
-              sbv[j][qd][2] = __uint_as_float(w.y << 16);
-              sbv[j][qd][3] = __uint_as_float(w.y & 0xFFFF0000u);
-            } else {
-              const float4 w = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(ep.sb) + n);
-              sbv[j][qd][0] = w.x; sbv[j][qd][1] = w.y; sbv[j][qd][2] = w.z; sbv[j][qd][3] = w.w;
-            }
-          } else {
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (n + r < N) sbv[j][qd][r] = load_scale(ep.sb, ep.sb_dtype, n + r);
-          }
-        }
-      }
-  }
+  fetch_scales<OUT, TM, TN>(ep, m_base, n_base, M, N, lane, sav, sbv);
   const int KT = K / BK;
   QWIX_DBG_DECL
   QWIX_DBG_STAMP(0)
@@ -540,99 +649,8 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
   }
   QWIX_DBG_STAMP(2)
 
-  // ---- epilogue.  acc[i][j][r]: m = m_base + i*32 + lane%32, n = n_base + j*32 + 8*(r/4) + 4*(lane/32) + r%4.
-  // The scaled values are staged through this wavefront's own slice of LDS, 32 rows at a time, and
-  // leave with 16-byte stores that cover whole 128-byte row segments (a direct store from the MFMA
-  // layout would write 16-byte pieces of 32 different rows per instruction).
-  using OutT = typename std::conditional<OUT == QWIX_BF16, uint16_t, uint32_t>::type;
-  constexpr int ES = sizeof(OutT);
-  constexpr int ROWB = WTN * ES + 16;            // staged row pitch in bytes (padded against bank conflicts)
-  constexpr int CPR = WTN * ES / 16;             // 16-byte chunks per staged row
-  constexpr int EPC = 16 / ES;                   // elements per chunk
-  static_assert(NWAVES * 32 * ROWB <= 2 * STAGE, "epilogue staging does not fit in LDS");
-  constexpr bool ZP = (EPI == 3);  // run-time rounding flags plus zero-point correction
-  const bool r0 = EPI >= 2 ? ep.r0 != 0 : EPI == 1, r1 = EPI >= 2 ? ep.r1 != 0 : EPI == 1,
-             r2 = EPI >= 2 ? ep.r2 != 0 : EPI == 1;
-  int zuv[TM];
-  if constexpr (ZP) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i) zuv[i] = ep.zu[min(m_base + i * 32 + (lane & 31), M - 1)];
-  }
-  __syncthreads();  // every wavefront is done with the slabs; LDS becomes staging space
-  uint8_t* stg = smem + wave * (32 * ROWB);
-  const bool row_vec = (reinterpret_cast<uintptr_t>(out) % 16 == 0) && ((ldo * ES) % 16 == 0);
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    float sa = 1.f;
-    if constexpr (OUT != QWIX_I32) sa = sav[i];
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        uint8_t* dst = stg + (lane & 31) * ROWB + (j * 32 + 8 * qd + 4 * (lane >> 5)) * ES;
-        if constexpr (OUT == QWIX_I32) {
-          *reinterpret_cast<int4*>(dst) = make_int4(static_cast<int>(acc[i][j][4 * qd]), static_cast<int>(acc[i][j][4 * qd + 1]),
-                                                    static_cast<int>(acc[i][j][4 * qd + 2]), static_cast<int>(acc[i][j][4 * qd + 3]));
-        } else if constexpr (EPI == 1 && OUT == QWIX_BF16) {
-          // Every step rounds to bf16 and the result is bf16: round two values per v_cvt_pk_bf16_f32,
-          // and let the last rounding produce the packed output directly.
-          uint32_t w[2];
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            uint32_t pk = pack_bf16x2(static_cast<float>(acc[i][j][4 * qd + 2 * h]),
-                                      static_cast<float>(acc[i][j][4 * qd + 2 * h + 1]));
-            pk = pack_bf16x2(__uint_as_float(pk << 16) * sa, __uint_as_float(pk & 0xFFFF0000u) * sa);
-            w[h] = pack_bf16x2(__uint_as_float(pk << 16) * sbv[j][qd][2 * h],
-                               __uint_as_float(pk & 0xFFFF0000u) * sbv[j][qd][2 * h + 1]);
-          }
-          *reinterpret_cast<uint2*>(dst) = make_uint2(w[0], w[1]);
-        } else {
-          float v[4];
-          int zvv[4] = {0, 0, 0, 0};
-          if constexpr (ZP) {
-            const int n = n_base + j * 32 + 8 * qd + 4 * (lane >> 5);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) zvv[r] = ep.zv[min(n + r, N - 1)];
-          }
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            float t;
-            if constexpr (ZP) t = static_cast<float>(static_cast<int>(acc[i][j][4 * qd + r]) - zuv[i] * zvv[r]);
-            else t = static_cast<float>(acc[i][j][4 * qd + r]);
-            if (r0) t = round_bf16(t);
-            t *= sa;
-            if (r1) t = round_bf16(t);
-            t *= sbv[j][qd][r];
-            if (r2) t = round_bf16(t);
-            v[r] = t;
-          }
-          if constexpr (OUT == QWIX_BF16)
-            *reinterpret_cast<uint2*>(dst) =
-                make_uint2(f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16),
-                           f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16));
-          else
-            *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
-        }
-      }
-    // read back row-major: chunk c of the 32 x CPR grid -> row c / CPR, 16-byte column c % CPR
-#pragma unroll
-    for (int c0 = 0; c0 < 32 * CPR; c0 += 64) {
-      const int c = c0 + lane, row = c / CPR, cc = c % CPR;
-      const uint4 v = *reinterpret_cast<const uint4*>(stg + row * ROWB + cc * 16);
-      const int mo = m_base + i * 32 + row, no = n_base + cc * EPC;
-      if (mo < M && no < N) {
-        OutT* o = reinterpret_cast<OutT*>(out) + static_cast<int64_t>(mo) * ldo + no;
-        if (row_vec && no + EPC <= N) {
-          *reinterpret_cast<uint4*>(o) = v;
-        } else {
-          const OutT* e = reinterpret_cast<const OutT*>(&v);
-#pragma unroll
-          for (int t = 0; t < EPC; ++t)
-            if (no + t < N) o[t] = e[t];
-        }
-      }
-    }
-  }
+  staged_epilogue<OUT, EPI, TM, TN, NWAVES, 2 * STAGE>(acc, sav, sbv, ep, m_base, n_base, M, N, out, ldo, smem, wave,
+                                                         lane);
   QWIX_DBG_STAMP(3)
   QWIX_DBG_FLUSH()
 }
@@ -688,6 +706,219 @@ int dispatch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t
   }
   if (none) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_F32, 0>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
   return launch_dma<QT, BM, BN, WGM, WGN, QWIX_F32, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Ping-pong variant of the 256 x 256 kernel for long K.  The eight wavefronts form two groups (the
+// upper and the lower 128 rows of the tile; the two wavefronts that share a SIMD are in different
+// groups) that run half a slab out of phase: while one group is in its memory phase (read all
+// fragments of a slab from LDS into registers, issue its direct-to-LDS loads of A), the other is in
+// its compute phase (the slab's MFMAs back to back at raised priority, one load of B after each
+// k-step), so the matrix pipe of every SIMD always has a wavefront that does little else.  Two
+// workgroup barriers per slab keep the phases aligned; one extra barrier at the start of the lower
+// group and at the end of the upper group produces the offset.
+//   LDS: A in two stages of 32 KB, B in three (160 KB in all).  A wavefront loads 32 rows of A (its
+// group's half) for the next slab and 32 rows of B for the slab after that; the third B stage is
+// what makes room for loading B two slabs ahead, which gives those loads three phases to land and
+// lets them be issued from the compute phase without a wait behind them.  Every load is waited for
+// by the wavefront that issued it (vmcnt, oldest first) before the barrier that publishes it.
+template <int QT, int OUT, int EPI>
+__device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B,
+                                              int64_t ldb, int m0, int n0, int M, int N, int K, const Epilogue& ep,
+                                              uint8_t* __restrict__ out, int64_t ldo) {
+  constexpr bool IS_INT = (QT == QWIX_INT8);
+  constexpr int BM = 256, BN = 256, BK = 128, WGN = 4;
+  constexpr int TM = 4, TN = 2;                 // wave tile 128 x 64
+  constexpr int KSTEP = IS_INT ? 32 : 64, NK = BK / KSTEP;
+  constexpr int A_STAGE = BM * BK, B_STAGE = BN * BK, B_BASE = 2 * A_STAGE;
+  constexpr int LDS_BYTES = 2 * A_STAGE + 3 * B_STAGE;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;   // wm is also the phase group
+
+  using AccT = typename std::conditional<IS_INT, v16i, v16f>::type;
+  using FragT = typename std::conditional<IS_INT, v4i, v8i>::type;
+  AccT acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  // ---- loader: this wavefront brings rows [wm*128 + wn*32, +32) of A and of B, 8 rows per instruction
+  const int lr = lane >> 3, lc = (lane & 7) ^ lr;
+  const int lrow0 = wm * 128 + wn * 32;
+  uint32_t goffa[4], goffb[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    goffa[j] = static_cast<uint32_t>(min(m0 + lrow0 + j * 8 + lr, M - 1)) * static_cast<uint32_t>(lda) + lc * 16;
+    goffb[j] = static_cast<uint32_t>(min(n0 + lrow0 + j * 8 + lr, N - 1)) * static_cast<uint32_t>(ldb) + lc * 16;
+  }
+  auto load_a = [&](int kt) {  // own half of the A rows of slab kt
+    const uint8_t* gk = A + kt * BK;
+    uint8_t* dst = smem + (kt & 1) * A_STAGE + lrow0 * BK;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) QWIX_GLDS16(gk + goffa[j], dst + j * 1024);
+  };
+  auto load_b = [&](int kt, int stage) {  // own half of the B rows of slab kt
+    const uint8_t* gk = B + kt * BK;
+    uint8_t* dst = smem + B_BASE + stage * B_STAGE + lrow0 * BK;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) QWIX_GLDS16(gk + goffb[j], dst + j * 1024);
+  };
+
+  // ---- fragments of a whole slab
+  const int a_row = (wm * 128 + (lane & 31)) * BK;
+  const int b_row = B_BASE + (wn * 64 + (lane & 31)) * BK;
+  const int hx = lane >> 5, x7 = lane & 7;
+  FragT fa[NK][TM], fb[NK][TN];
+  auto read_slab = [&](int a_stage, int b_stage) {
+    const uint8_t* pa = smem + a_stage * A_STAGE + a_row;
+    const uint8_t* pb = smem + b_stage * B_STAGE + b_row;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      if constexpr (IS_INT) {
+        const int off = ((ks * 2 + hx) ^ x7) << 4;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[ks][i] = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + off);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[ks][j] = *reinterpret_cast<const v4i*>(pb + j * 32 * BK + off);
+      } else {
+        const int off = ((ks * 4 + hx * 2) ^ x7) << 4;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const v4i lo = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + off);
+          const v4i hi = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + (off ^ 16));
+          fa[ks][i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const v4i lo = *reinterpret_cast<const v4i*>(pb + j * 32 * BK + off);
+          const v4i hi = *reinterpret_cast<const v4i*>(pb + j * 32 * BK + (off ^ 16));
+          fb[ks][j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+      }
+    }
+  };
+  // s_waitcnt on vmcnt only (expcnt 7, lgkmcnt 15 stay open): all but the newest `left` direct-to-LDS
+  // loads of this wavefront have landed
+  auto wait_loads = [&](int left) {  // left: 0 or 4
+    if (left == 0) __builtin_amdgcn_s_waitcnt(0x0F70); else __builtin_amdgcn_s_waitcnt(0x0F74);
+  };
+  auto barrier = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  const int KT = K / BK;  // >= 2
+  // ---- prologue: A of slab 0, B of slabs 0 and 1 (each wavefront its rows)
+  load_a(0);
+  load_b(0, 0);
+  load_b(1, 1);
+  wait_loads(0);
+  barrier();
+  if (wm == 1) barrier();  // the lower group starts half a slab late
+
+  // B is loaded two slabs ahead, during the compute phase, one load after each k-step's MFMAs (those
+  // loads have three phases to land); A one slab ahead, in the memory phase.  The waits before the
+  // barriers leave the four loads just issued in flight and cover the four issued one phase earlier.
+  int bst = 0;  // B stage of slab kt = kt % 3
+  QWIX_DBG_DECL
+  QWIX_DBG_STAMP(0)
+  for (int kt = 0; kt < KT; ++kt) {
+    QWIX_DBG_BEGIN()
+    // memory phase
+    read_slab(kt & 1, bst);
+    __builtin_amdgcn_sched_barrier(0);  // fragment reads first: the loads below may not slip in front of them
+    const bool more_a = kt + 1 < KT, more_b = kt + 2 < KT;
+    if (more_a) load_a(kt + 1);
+    if (more_a) wait_loads(4); else wait_loads(0);
+    QWIX_DBG_ACC(2)
+    barrier();
+    QWIX_DBG_ACC(3)
+    // compute phase
+    const int bst2 = bst == 0 ? 2 : bst - 1;  // (kt + 2) % 3
+    const uint8_t* gkb = B + (kt + 2) * BK;
+    uint8_t* dstb = smem + B_BASE + bst2 * B_STAGE + lrow0 * BK;
+    __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          if constexpr (IS_INT)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+          else
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0, 0, 0, 0);
+        }
+      if (more_b) {
+#pragma unroll
+        for (int j = ks * (4 / NK); j < (ks + 1) * (4 / NK); ++j) QWIX_GLDS16(gkb + goffb[j], dstb + j * 1024);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_s_setprio(0);
+    QWIX_DBG_ACC(4)
+    if (more_b) wait_loads(4); else wait_loads(0);
+    QWIX_DBG_ACC(5)
+    barrier();
+    QWIX_DBG_ACC(6)
+    bst = bst == 2 ? 0 : bst + 1;
+  }
+  QWIX_DBG_STAMP(1)
+  if (wm == 0) barrier();
+
+  const int m_base = m0 + wm * 128, n_base = n0 + wn * 64;
+  float sav[TM];
+  float sbv[TN][4][4];
+  fetch_scales<OUT, TM, TN>(ep, m_base, n_base, M, N, lane, sav, sbv);
+  staged_epilogue<OUT, EPI, TM, TN, 8, LDS_BYTES>(acc, sav, sbv, ep, m_base, n_base, M, N, out, ldo, smem, wave, lane);
+  QWIX_DBG_FLUSH()
+}
+
+template <int QT, int OUT, int EPI>
+__global__ void __launch_bounds__(512)
+    qgemm_pp_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb, int M,
+                    int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  int tile_m, tile_n;
+  tile_coords((M + 255) / 256, (N + 255) / 256, &tile_m, &tile_n);
+  qgemm_pp_tile<QT, OUT, EPI>(A, lda, B, ldb, tile_m * 256, tile_n * 256, M, N, K, ep, out, ldo);
+}
+
+template <int QT, int OUT, int EPI>
+int launch_pp(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
+              const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  constexpr size_t smem = 5 * 256 * 128;
+  auto kern = qgemm_pp_kernel<QT, OUT, EPI>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  kern<<<dim3(static_cast<unsigned>(tiles)), 512, smem, st>>>(
+      static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),
+      static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);
+  return check_launch("qgemm (ping-pong)");
+}
+
+template <int QT>
+int dispatch_pp(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  const bool all = ep.r0 && ep.r1 && ep.r2, none = !ep.r0 && !ep.r1 && !ep.r2;
+  if (ep.out_dtype == QWIX_BF16) {
+    if (all) return launch_pp<QT, QWIX_BF16, 1>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    return launch_pp<QT, QWIX_BF16, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+  }
+  if (none) return launch_pp<QT, QWIX_F32, 0>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+  return launch_pp<QT, QWIX_F32, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
 }
 
 template <int QT, int BM, int BN, int BK>
@@ -790,6 +1021,46 @@ __global__ void __launch_bounds__(WGM * WGN * 64)
                                                                         m_lim, N, K, e, out, ldo);
 }
 
+inline unsigned ragged_grid(int64_t M, int64_t N, int64_t G, int BM, int BN) {
+  const int64_t tiles = (M / BM + G + 1) * ((N + BN - 1) / BN);
+  const int64_t unit = 8 * kRaggedChunk;
+  return static_cast<unsigned>((tiles + unit - 1) / unit * unit);
+}
+
+template <int QT, int OUT>
+__global__ void __launch_bounds__(512)
+    qgemm_ragged_pp_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
+                           Ragged rg, int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  int g, m0, m_lim, n0;
+  const int kind = ragged_tile<256, 256>(rg, M, N, &g, &m0, &m_lim, &n0);
+  if (kind == 0) return;
+  using OutT = typename std::conditional<OUT == QWIX_BF16, uint16_t, uint32_t>::type;
+  if (kind == 2) {
+    zero_tile<256, 256, OutT>(out, ldo, m0, m_lim, n0, N, 512);
+    return;
+  }
+  const Epilogue e = group_epilogue(ep, rg, g);
+  qgemm_pp_tile<QT, OUT, 2>(A, lda, B + g * rg.b_group_stride, ldb, m0, n0, m_lim, N, K, e, out, ldo);
+}
+
+template <int QT, int OUT>
+int launch_ragged_pp(const void* a, int64_t lda, const void* b, int64_t ldb, const Ragged& rg, int64_t M, int64_t N,
+                     int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  constexpr size_t smem = 5 * 256 * 128;
+  auto kern = qgemm_ragged_pp_kernel<QT, OUT>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  kern<<<dim3(ragged_grid(M, N, rg.G, 256, 256)), 512, smem, st>>>(
+      static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, rg, static_cast<int>(M),
+      static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);
+  return check_launch("ragged qgemm (ping-pong)");
+}
+
 template <int QT, int BM, int BN, int BK>
 __global__ void __launch_bounds__(256)
     qgemm_ragged_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
@@ -804,12 +1075,6 @@ __global__ void __launch_bounds__(256)
   }
   const Epilogue e = group_epilogue(ep, rg, g);
   qgemm_tile<QT, BM, BN, BK>(A, lda, B + g * rg.b_group_stride, ldb, m0, n0, m_lim, N, K, e, out, ldo);
-}
-
-inline unsigned ragged_grid(int64_t M, int64_t N, int64_t G, int BM, int BN) {
-  const int64_t tiles = (M / BM + G + 1) * ((N + BN - 1) / BN);
-  const int64_t unit = 8 * kRaggedChunk;
-  return static_cast<unsigned>((tiles + unit - 1) / unit * unit);
 }
 
 template <int QT, int BM, int BN, int WGM, int WGN, int OUT>
@@ -1208,6 +1473,14 @@ extern "C" int qwix_hip_qgemm_ragged(const void* a, int64_t lda, const void* b, 
     // 256-row tiles pay off once the average group is several tiles tall; 128-row tiles waste fewer rows
     // at the ragged end of each group.
     const bool big = M / G >= 768 && ((M + 255) / 256) * ((N + 255) / 256) >= 192;
+    if (big && K >= 256 && out_dtype != QWIX_I32) {
+      if (qtype == QWIX_INT8) {
+        if (out_dtype == QWIX_BF16) return launch_ragged_pp<QWIX_INT8, QWIX_BF16>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+        return launch_ragged_pp<QWIX_INT8, QWIX_F32>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+      }
+      if (out_dtype == QWIX_BF16) return launch_ragged_pp<QWIX_E4M3, QWIX_BF16>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+      return launch_ragged_pp<QWIX_E4M3, QWIX_F32>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+    }
     if (qtype == QWIX_INT8) {
       if (big) return dispatch_ragged_dma<QWIX_INT8, 256, 256, 2, 4>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
       return dispatch_ragged_dma<QWIX_INT8, 128, 128, 2, 2>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
@@ -1279,6 +1552,11 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
   const bool big = ((M + 255) / 256) * ((N + 255) / 256) >= 192;
   const bool off32 = M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);  // 32-bit lane offsets
   if (K % 128 == 0 && off32) {  // direct-to-LDS pipeline
+    // long K on a full chip: the ping-pong schedule (no raw-accumulator / zero-point variants of it exist)
+    if (big && K >= 256 && out_dtype != QWIX_I32 && zu == nullptr) {
+      if (qtype == QWIX_INT8) return dispatch_pp<QWIX_INT8>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      return dispatch_pp<QWIX_E4M3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    }
     if (qtype == QWIX_INT8) {
       if (big) return dispatch_dma<QWIX_INT8, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       return dispatch_dma<QWIX_INT8, 128, 128, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);

@@ -54,6 +54,7 @@ INT8_CASES = [
     ('k tiled, shared over groups', (128, 256, 4, 512), (10, 20, 30, 68), (0,), (2,), {1: 128}),
     ('k and n tiled', (128, 256, 4, 512), (10, 20, 30, 68), (0,), (0,), {1: 128, 2: 128}),
     ('big groups', (2100, 512, 2, 2304), (1100, 900), (0,), (0, 2), None),
+    ('big groups on a full chip (256-row tiles, ping-pong schedule)', (4096, 384, 4, 3072), (1000, 1100, 900, 1000), (0,), (0, 2), None),
 ]
 
 
@@ -116,7 +117,8 @@ def test_ragged_dot_out_of_range_sizes_are_clamped():
 
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
 @pytest.mark.parametrize('shape,sizes,rcw', [((128, 256, 4, 64), (128, 100, 0, 28), (2,)),
-                                             ((520, 512, 6, 384), (100, 3, 0, 257, 60, 50), (0, 2))])
+                                             ((520, 512, 6, 384), (100, 3, 0, 257, 60, 50), (0, 2)),
+                                             ((4096, 256, 4, 3072), (1000, 1100, 900, 1000), (0, 2))])
 def test_ragged_dot_fp8(shape, sizes, rcw, dtype):
   import qwix_amd
   M, K, G, N = shape
