@@ -2,14 +2,18 @@
 //
 //   out[m,n] = epilogue( sum_k a[m,k] * b[n,k] )      a: (M,K), b: (N,K), both K-contiguous
 //
-// One workgroup of 4 wavefronts (2 x 2) owns a BM x BN tile of the output.  K is walked in BK-byte
-// slabs: global -> registers -> LDS (two LDS stages, rows padded by 16 bytes so that the 16-byte
-// operand reads of 8 consecutive lanes touch all 32 banks once), operands are read back as
-// 16-byte fragments and fed to v_mfma_i32_32x32x32_i8 / v_mfma_f32_32x32x64_f8f6f4.
-// The MFMA "A" operand is fed from b and the "B" operand from a, so that each lane ends up with
-// 4 consecutive n for a single m: output rows are written with 8/16-byte vector stores.
-// Workgroup ids are remapped so that the 8 XCDs (round-robin dispatch) each work on a compact
-// block of tiles and share their slabs through their own L2.
+// Tile bodies (device functions of a tile origin and a row limit, shared by all entry points):
+//   qgemm_tile      register-staged 128 x 128 tile, any K that is a multiple of 16
+//   qgemm_dma_tile  K % 128 == 0: 128-byte K slabs go global -> LDS directly, two stages
+//   qgemm_pp_tile   256 x 256, long K: two wavefront groups half a slab out of phase (ping-pong)
+// Kernels around them: dense (one tile per workgroup, XCD-aware tile order), batched (blockIdx.y
+// selects the problem), ragged (rows in groups whose sizes live in device memory, one weight panel
+// per group), and a skinny kernel for M <= 32 that streams the weights once.
+// K is walked in slabs through LDS; rows are stored so that the 16-byte operand reads of 8
+// consecutive lanes touch all 32 banks once (padding in the register-staged body, an XOR swizzle in
+// the others); operands are read back as 16-byte fragments and fed to v_mfma_i32_32x32x32_i8 /
+// v_mfma_f32_32x32x64_f8f6f4.  The MFMA "A" operand is fed from b and the "B" operand from a, so
+// that each lane ends up with 4 consecutive n for a single m.
 #include <cstdlib>
 #include <type_traits>
 
@@ -577,11 +581,6 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
     }
   };
   auto mfma_step = [&](int buf) {
-#ifdef QWIX_DBG_SKIP_MFMA
-    for (int i = 0; i < TM; ++i)
-      for (int j = 0; j < TN; ++j) acc[i][j][0] += fb[buf][j][0] + fa[buf][i][0];
-    return;
-#endif
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -621,9 +620,7 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
   for (int kt = 0; kt < KT - 1; ++kt) {
     const int cur = kt & 1;
     QWIX_DBG_BEGIN()
-#ifndef QWIX_DBG_SKIP_LOADS
     issue_loads(cur ^ 1, (kt + 1) * BK);
-#endif
 #pragma unroll
     for (int ks = 0; ks + 1 < NK; ++ks) {
       read_frags(cur, ks + 1, (ks + 1) & 1);
