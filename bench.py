@@ -529,6 +529,127 @@ class RaggedQdot(Workload):
             'weight': 'per-expert per-output-channel ' + self.qtype + ' (pre-quantized)', 'out': 'bf16'}
 
 
+class QuantizeStatic(Workload):
+  """Static-range activation quantization: the scale was computed offline, one read and one write."""
+
+  bound = 'hbm'
+
+  def __init__(self, name, M, K):
+    self.name, self.M, self.K = name, M, K
+    self.dtype = 'bf16->int8'
+    self.metric = 'quantize GB/s (static range, per-tensor scale, bf16 -> int8)'
+    self.unit = 'GB/s'
+    self.kernel_name = 'rows_kernel'
+
+  def setup(self, dev):
+    import torch
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(11)
+    self.x = torch.randn(self.M, self.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    self.scale = (self.x.abs().max().float() / 127.5).to(torch.bfloat16).reshape(1)
+    self.q = torch.empty(self.M, self.K, dtype=torch.int8, device=dev)
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, i=0):
+    L = self.L
+    # one scale for the whole array: outer = 1, every element in one reduce group
+    L.call('qwix_hip_quantize_with_scale', self.x.data_ptr(), L.BF16, 1, self.M * self.K, 1, self.M * self.K, L.INT8,
+           self.scale.data_ptr(), None, L.LAYOUT_NATURAL, self.q.data_ptr(), self.stream)
+
+  kernel = step
+
+  def work_per_step(self):
+    return float(self.M * self.K * 3)
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'M': self.M, 'K': self.K, 'scale': 'per-tensor, precomputed'}
+
+
+class QdotZeroPoint(QdotW8A8):
+  """w8a8 with an asymmetric (minmax) int8 activation: quantize with zero point, K-sums of the weight rows,
+  GEMM with the zero-point correction in the epilogue."""
+
+  def __init__(self, name, M, K, N):
+    super().__init__(name, M, K, N, 'int8')
+    self.metric = 'int8 qdot TOPS (asymmetric activation, zero-point correction, activation quantize included)'
+    self.kernel_name = 'qgemm_dma_kernel'
+
+  def setup(self, dev):
+    import torch
+    super().setup(dev)
+    self.x = (self.x.float() + 0.5).to(torch.bfloat16)  # a shifted distribution, as minmax is meant for
+    self.zp = torch.empty(self.M, dtype=torch.int8, device=dev)
+    self.zu = torch.empty(self.M, dtype=torch.int32, device=dev)
+    self.zv = torch.empty(self.N, dtype=torch.int32, device=dev)
+    L = self.L
+    L.call('qwix_hip_ksum_i8', self.b.data_ptr(), self.K, self.N, self.K, self.zv.data_ptr(), self.stream)  # weights: once
+
+  def step(self, i=0):
+    L = self.L
+    L.call('qwix_hip_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, 1, self.K, self.qt, L.MINMAX, 0.0,
+           L.LAYOUT_NATURAL, self.xq.data_ptr(), self.sa.data_ptr(), self.zp.data_ptr(), None, 0, self.stream)
+    self.zu.copy_(self.zp)  # int8 -> int32 zero points (M values)
+    self.kernel(i)
+
+  def kernel(self, i=0):
+    L = self.L
+    L.call('qwix_hip_qgemm_zp', self.xq.data_ptr(), self.K, self.b.data_ptr(), self.K, self.M, self.N, self.K,
+           self.sa.data_ptr(), L.BF16, self.sb.data_ptr(), L.BF16, self.zu.data_ptr(), self.zv.data_ptr(),
+           self.out.data_ptr(), L.BF16, self.N, self.stream)
+
+  def cpu_baseline(self, *a, **k):
+    return None
+
+
+class QdotBatched(Workload):
+  """Batch axes of dot_general in one launch: 'bqd,bkd->bqk' with int8 operands (attention scores).  With
+  d = 128 the output write dominates: an HBM-bound contraction."""
+
+  bound = 'hbm'
+
+  def __init__(self, name, B, Q, Kv, D):
+    self.name, self.B, self.Q, self.Kv, self.D = name, B, Q, Kv, D
+    self.dtype = 'int8'
+    self.metric = 'batched int8 qdot GB/s (bqd,bkd->bqk, bf16 out)'
+    self.unit = 'GB/s'
+    self.kernel_name = 'qgemm_batched_dma_kernel'
+
+  def setup(self, dev):
+    import torch
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(21)
+    B, Q, Kv, D = self.B, self.Q, self.Kv, self.D
+    self.a = torch.randint(-127, 128, (B, Q, D), generator=g, dtype=torch.int8).to(dev)
+    self.b = torch.randint(-127, 128, (B, Kv, D), generator=g, dtype=torch.int8).to(dev)
+    self.sa = (torch.rand(B, Q, generator=g) * 0.01 + 0.001).to(torch.bfloat16).to(dev)
+    self.sb = (torch.rand(B, Kv, generator=g) * 0.01 + 0.001).to(torch.bfloat16).to(dev)
+    self.out = torch.empty(B, Q, Kv, dtype=torch.bfloat16, device=dev)
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, i=0):
+    L = self.L
+    B, Q, Kv, D = self.B, self.Q, self.Kv, self.D
+    L.call('qwix_hip_qgemm_batched', self.a.data_ptr(), D, Q * D, self.b.data_ptr(), D, Kv * D, L.INT8, B, Q, Kv, D,
+           self.sa.data_ptr(), L.BF16, Q, self.sb.data_ptr(), L.BF16, Kv, 0, self.out.data_ptr(), L.BF16, Kv, Q * Kv,
+           self.stream)
+
+  kernel = step
+
+  def work_per_step(self):
+    B, Q, Kv, D = self.B, self.Q, self.Kv, self.D
+    return float(B * (Q * D + Kv * D + 2 * (Q + Kv) + 2 * Q * Kv))
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'batch': self.B, 'q': self.Q, 'k': self.Kv, 'd': self.D,
+            'ops': 2.0 * self.B * self.Q * self.Kv * self.D}
+
+
 WORKLOADS = {
     'c3_int8_w8a8_4096': lambda: QdotW8A8('c3_int8_w8a8_4096', 4096, 4096, 4096, 'int8'),
     'c4_fp8_w8a8_ffn': lambda: QdotW8A8('c4_fp8_w8a8_ffn', 8192, 8192, 28672, 'float8_e4m3fn'),
@@ -548,12 +669,15 @@ WORKLOADS = {
     'moe_ragged_int8_8x1024': lambda: RaggedQdot('moe_ragged_int8_8x1024', 8192, 4096, 14336, 8),
     'moe_ragged_int8_64x128': lambda: RaggedQdot('moe_ragged_int8_64x128', 8192, 2048, 4096, 64),
     'moe_ragged_fp8_8x1024': lambda: RaggedQdot('moe_ragged_fp8_8x1024', 8192, 4096, 14336, 8, 'float8_e4m3fn'),
+    'srq_quantize_act_4096': lambda: QuantizeStatic('srq_quantize_act_4096', 4096, 4096),
+    'zp_int8_w8a8_4096': lambda: QdotZeroPoint('zp_int8_w8a8_4096', 4096, 4096, 4096),
+    'batched_qk_int8_32x2048': lambda: QdotBatched('batched_qk_int8_32x2048', 32, 2048, 2048, 128),
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
 }
 DEFAULT = 'c3_int8_w8a8_4096'
 EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16',
          'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'moe_ragged_int8_8x1024',
-         'moe_ragged_int8_64x128']
+         'moe_ragged_int8_64x128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048']
 
 
 def _blas_threads() -> int:

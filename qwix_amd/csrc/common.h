@@ -176,9 +176,15 @@ struct Divider {
       float q0 = x * r;
       float e = __builtin_fmaf(-q0, s, x);
       float q1 = __builtin_fmaf(e, r, q0);
-      // Overflowing or non-finite quotients (static scales only): take the IEEE path.
-      if constexpr (kSafe)
-        if (!(__builtin_fabsf(q0) < 0x1p100f)) q1 = x / s;
+      // Overflowing or non-finite quotients (static scales only): take the IEEE path.  The test is made
+      // wave-uniform first, so that the division sequence is branched over instead of being computed
+      // for every element and selected away.
+      if constexpr (kSafe) {
+        const bool odd = !(__builtin_fabsf(q0) < 0x1p100f);
+        if (__builtin_amdgcn_ballot_w64(odd) != 0) {
+          if (odd) q1 = x / s;
+        }
+      }
       // The residual step turns -0 into +0; the quotient always carries the sign of x (s > 0).
       if constexpr (kSignedZero) return __builtin_copysignf(round_bf16(q1), x);
       return round_bf16(q1);

@@ -12,6 +12,8 @@
 //           reduce-minor (transposed) layout the GEMM kernels consume.
 #include <cstdlib>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace qwix {
@@ -82,7 +84,7 @@ template <typename D, int QT, int CAL, int MODE, int NL>
 __global__ void __launch_bounds__(256)
     rows_kernel(const uint8_t* __restrict__ x, int64_t nseg, int nvec, int log2g, float factor,
                 uint8_t* __restrict__ q, void* __restrict__ scale, int8_t* __restrict__ zp,
-                void* __restrict__ cal0, void* __restrict__ cal1) {
+                void* __restrict__ cal0, void* __restrict__ cal1, int per_scale, int per_shift) {
   constexpr int EV = D::kVec;
   constexpr bool ASYM = (CAL == QWIX_MINMAX);
   __shared__ float red[2][4];
@@ -171,27 +173,54 @@ __global__ void __launch_bounds__(256)
       if constexpr (ASYM) zp[seg] = static_cast<int8_t>(z);
     }
   } else {
-    if (seg_ok) {
-      s = load1<D>(scale, seg);
-      if constexpr (ASYM) z = zp[seg];
+    if (seg_ok) {  // per_scale consecutive segments are pieces of one scale group
+      int64_t si = seg;  // per_shift: log2(per_scale) if that is a power of two, else -1
+      if (per_scale > 1)
+        si = per_shift >= 0 ? (seg >> per_shift)
+                            : (nseg <= 0xFFFFFFFFll ? static_cast<int64_t>(static_cast<uint32_t>(seg) / static_cast<uint32_t>(per_scale))
+                                                    : seg / per_scale);
+      s = load1<D>(scale, si);
+      if constexpr (ASYM) z = zp[si];
     }
   }
 
-  const Divider<D, MODE == MODE_GIVEN, QT == QWIX_E4M3> div(s);
   const float zf = static_cast<float>(z);
+  auto quantize_all = [&](auto safe_tag) {
+    const Divider<D, decltype(safe_tag)::value, QT == QWIX_E4M3> div(s);
 #pragma unroll
-  for (int j = 0; j < NL; ++j) {
-    const int v = lane + (j << log2g);
-    if (seg_ok && v < nvec) {
-      float t[EV];
-      unpack16<D>(raw[j], t);
+    for (int j = 0; j < NL; ++j) {
+      const int v = lane + (j << log2g);
+      if (seg_ok && v < nvec) {
+        float t[EV];
+        unpack16<D>(raw[j], t);
 #pragma unroll
-      for (int e = 0; e < EV; ++e) {
-        t[e] = div(t[e]);
-        if constexpr (ASYM) t[e] = rnd<D>(t[e] + zf);
+        for (int e = 0; e < EV; ++e) {
+          t[e] = div(t[e]);
+          if constexpr (ASYM) t[e] = rnd<D>(t[e] + zf);
+        }
+        store_q<QT, EV, true>(t, q, (seg * nvec + v) * EV);
       }
-      store_q<QT, EV, true>(t, q, (seg * nvec + v) * EV);
     }
+  };
+  if constexpr (MODE == MODE_GIVEN && D::kTag == QWIX_BF16) {
+    // A given scale can be anything: quotients may overflow or be NaN, which the reciprocal-based division
+    // does not reproduce.  One test per wavefront on the largest magnitude a thread holds decides whether
+    // all of its elements can take the plain path (as they always can when the scale comes from absmax).
+    u16x2 m = {0, 0};
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+      const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2, w[e] & 0x7FFF7FFFu));
+    }
+    const float big = bf16_bits_to_f32(m[0] > m[1] ? m[0] : m[1]);  // NaN / inf inputs order above finite ones
+    const bool odd = !(big * __builtin_fabsf(__builtin_amdgcn_rcpf(s)) < 0x1p100f);
+    if (__builtin_amdgcn_ballot_w64(odd) == 0)
+      quantize_all(std::false_type{});
+    else
+      quantize_all(std::true_type{});
+  } else {
+    quantize_all(std::integral_constant<bool, MODE == MODE_GIVEN>{});
   }
 }
 
@@ -354,6 +383,50 @@ __global__ void __launch_bounds__(256)
         atomicMax(ws + plane + wbase + e, __float_as_uint(-b));
       }
     }
+  }
+}
+
+// Long segments are calibrated in pieces (rows_kernel in calibration mode, one partial per piece); this
+// kernel merges the `pieces` partials of a segment (one wavefront per segment) and either writes the
+// calibration values (MODE_CALIB) or turns them into scale / zero point (MODE_QUANT).  The partials
+// already carry the calibration factor: rounding is monotone, so max and factor commute.
+template <typename D, int QT, int CAL, int MODE>
+__global__ void __launch_bounds__(256)
+    rows_merge_kernel(const void* __restrict__ p0, const void* __restrict__ p1, int64_t nseg, int pieces,
+                      void* __restrict__ scale, int8_t* __restrict__ zp, void* __restrict__ cal0,
+                      void* __restrict__ cal1) {
+  constexpr bool ASYM = (CAL == QWIX_MINMAX);
+  const int64_t seg = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (seg >= nseg) return;
+  float mx = 0.f, mn = 0.f;
+  for (int i = lane; i < pieces; i += 64) {
+    if constexpr (ASYM) {
+      mn = fminf(mn, load1<D>(p0, seg * pieces + i));
+      mx = fmaxf(mx, load1<D>(p1, seg * pieces + i));
+    } else {
+      mx = fmaxf(mx, load1<D>(p0, seg * pieces + i));
+    }
+  }
+  mx = wave_xor_max(mx, 64);
+  if constexpr (ASYM) mn = wave_xor_min(mn, 64);
+  if (lane != 0) return;
+  if constexpr (MODE == MODE_CALIB) {
+    if constexpr (ASYM) {
+      store1<D>(cal0, seg, mn);
+      store1<D>(cal1, seg, mx);
+    } else {
+      store1<D>(cal0, seg, mx);
+    }
+  } else {
+    int z = 0;
+    float s;
+    if constexpr (ASYM)
+      s = asym_scale_zp<D, QT>(mn, mx, &z);
+    else
+      s = sym_scale<D, QT>(mx);
+    store1<D>(scale, seg, s);
+    if constexpr (ASYM) zp[seg] = static_cast<int8_t>(z);
   }
 }
 
@@ -734,32 +807,68 @@ ColGeom make_col_geom(int64_t outer, int64_t reduce, int64_t inner, int64_t tile
   return g;
 }
 
-// mode: MODE_QUANT / MODE_CALIB / MODE_GIVEN.
+// Pieces a long contiguous segment of L elements is cut into: the smallest count that divides L into
+// pieces of at most 8192 elements that are multiples of 8 (one rule for both array dtypes, so that the
+// workspace size does not depend on the dtype).  0: no such cut (the strided kernel takes the segment).
+int64_t row_pieces(int64_t L) {
+  constexpr int64_t kMaxPiece = 8192;
+  if (L <= kMaxPiece || L % 8) return 0;
+  for (int64_t r = (L + kMaxPiece - 1) / kMaxPiece; r <= (int64_t{1} << 20) && r * 8 <= L; ++r)
+    if (L % r == 0 && (L / r) % 8 == 0) return r;
+  return 0;
+}
+
+template <typename D, int QT, int CAL, int MODE>
+void launch_rows(const void* x, int64_t nseg, int64_t L, float factor, void* q, void* scale, void* zp, void* c0,
+                 void* c1, int per_scale, hipStream_t st) {
+  const int nvec = static_cast<int>(L / D::kVec);
+  constexpr int target = 4;  // 16-byte loads per thread
+  int lg = log2_ceil((nvec + target - 1) / target);  // aim at `target` loads per thread, 8 at most
+  while ((nvec + (1 << lg) - 1) >> lg > 8) ++lg;
+  if (lg > 8) lg = 8;
+  const int64_t blocks = (nseg + (256 >> lg) - 1) / (256 >> lg);
+  const int loads = (nvec + (1 << lg) - 1) >> lg;
+  const dim3 grid(static_cast<unsigned>(blocks));
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  uint8_t* qb = static_cast<uint8_t*>(q);
+  int8_t* zb = static_cast<int8_t*>(zp);
+  const int sh = (per_scale & (per_scale - 1)) == 0 ? log2_ceil(per_scale) : -1;
+  if (loads <= 2)
+    rows_kernel<D, QT, CAL, MODE, 2><<<grid, 256, 0, st>>>(xb, nseg, nvec, lg, factor, qb, scale, zb, c0, c1, per_scale, sh);
+  else if (loads <= 4)
+    rows_kernel<D, QT, CAL, MODE, 4><<<grid, 256, 0, st>>>(xb, nseg, nvec, lg, factor, qb, scale, zb, c0, c1, per_scale, sh);
+  else
+    rows_kernel<D, QT, CAL, MODE, 8><<<grid, 256, 0, st>>>(xb, nseg, nvec, lg, factor, qb, scale, zb, c0, c1, per_scale, sh);
+}
+
+// mode: MODE_QUANT / MODE_CALIB / MODE_GIVEN.  ws: scratch for segments longer than one workgroup holds
+// in registers (qwix_hip_quantize_workspace_bytes says how much); not needed when the scale is given.
 template <int MODE>
 int run_rows(const void* x, int dtype, int64_t nseg, int64_t L, int qtype, int cal, float factor,
-             void* q, void* scale, void* zp, void* c0, void* c1, hipStream_t st) {
+             void* q, void* scale, void* zp, void* c0, void* c1, void* ws, size_t ws_bytes, hipStream_t st) {
   QWIX_DISPATCH_D(dtype, {
     QWIX_DISPATCH_QT_CAL(qtype, cal, {
-      const bool vec_ok = (L % D::kVec == 0) && aligned16(x) && (L / D::kVec <= 2048) &&
-                          (MODE == MODE_CALIB || (reinterpret_cast<uintptr_t>(q) & 7) == 0);
+      const bool aligned = aligned16(x) && (MODE == MODE_CALIB || (reinterpret_cast<uintptr_t>(q) & 7) == 0);
+      const bool vec_ok = (L % D::kVec == 0) && aligned && (L / D::kVec <= 2048);
+      const int64_t pieces = aligned ? row_pieces(L) : 0;
       if (vec_ok) {
-        const int nvec = static_cast<int>(L / D::kVec);
-        constexpr int target = 4;  // 16-byte loads per thread
-        int lg = log2_ceil((nvec + target - 1) / target);  // aim at `target` loads per thread, 8 at most
-        while ((nvec + (1 << lg) - 1) >> lg > 8) ++lg;
-        if (lg > 8) lg = 8;
-        const int64_t blocks = (nseg + (256 >> lg) - 1) / (256 >> lg);
-        const int loads = (nvec + (1 << lg) - 1) >> lg;
-        const dim3 grid(static_cast<unsigned>(blocks));
-        const uint8_t* xb = static_cast<const uint8_t*>(x);
-        uint8_t* qb = static_cast<uint8_t*>(q);
-        int8_t* zb = static_cast<int8_t*>(zp);
-        if (loads <= 2)
-          rows_kernel<D, QT, CAL, MODE, 2><<<grid, 256, 0, st>>>(xb, nseg, nvec, lg, factor, qb, scale, zb, c0, c1);
-        else if (loads <= 4)
-          rows_kernel<D, QT, CAL, MODE, 4><<<grid, 256, 0, st>>>(xb, nseg, nvec, lg, factor, qb, scale, zb, c0, c1);
-        else
-          rows_kernel<D, QT, CAL, MODE, 8><<<grid, 256, 0, st>>>(xb, nseg, nvec, lg, factor, qb, scale, zb, c0, c1);
+        launch_rows<D, QT, CAL, MODE>(x, nseg, L, factor, q, scale, zp, c0, c1, 1, st);
+      } else if (pieces > 0 && pieces <= INT32_MAX) {
+        // long segments: calibrate piece by piece, merge, then quantize the pieces with the merged scale
+        const int64_t n = nseg * pieces, piece = L / pieces;
+        if constexpr (MODE != MODE_GIVEN) {
+          const size_t need = static_cast<size_t>(n) * 4u * (CAL == QWIX_MINMAX ? 2u : 1u);
+          if (!ws || ws_bytes < need)
+            return fail(QWIX_ERR_INVALID_ARGUMENT, "workspace of %zu bytes required, got %zu", need, ws_bytes);
+          void* p0 = ws;
+          void* p1 = static_cast<uint8_t*>(ws) + static_cast<size_t>(n) * 4u;
+          launch_rows<D, QT, CAL, MODE_CALIB>(x, n, piece, factor, nullptr, nullptr, nullptr, p0, p1, 1, st);
+          rows_merge_kernel<D, QT, CAL, MODE><<<dim3(static_cast<unsigned>((nseg + 3) / 4)), 256, 0, st>>>(
+              p0, p1, nseg, static_cast<int>(pieces), scale, static_cast<int8_t*>(zp), c0, c1);
+        }
+        if constexpr (MODE != MODE_CALIB)
+          launch_rows<D, QT, CAL, MODE_GIVEN>(x, n, piece, 0.f, q, scale, zp, nullptr, nullptr,
+                                              static_cast<int>(pieces), st);
       } else {
         if (QT == QWIX_INT4 && MODE != MODE_CALIB && (L & 1))
           return fail(QWIX_ERR_UNSUPPORTED, "int4 needs an even contiguous length, got %lld", (long long)L);
@@ -831,8 +940,11 @@ const char* qwix_hip_last_error(void) { return err_buf(); }
 
 size_t qwix_hip_quantize_workspace_bytes(int64_t outer, int64_t reduce, int64_t inner, int64_t tile,
                                          int calibration) {
-  if (inner <= 1 || tile <= 0 || reduce % tile != 0) return 0;
-  return static_cast<size_t>(outer * (reduce / tile) * inner) * 4u * (calibration == QWIX_MINMAX ? 2u : 1u);
+  if (tile <= 0 || reduce % tile != 0) return 0;
+  const size_t per = 4u * (calibration == QWIX_MINMAX ? 2u : 1u);
+  if (inner <= 1)  // contiguous segments: partial calibration values of the pieces of long segments
+    return static_cast<size_t>(outer * (reduce / tile) * row_pieces(tile)) * per;
+  return static_cast<size_t>(outer * (reduce / tile) * inner) * per;
 }
 
 int qwix_hip_quantize(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner, int64_t tile,
@@ -845,7 +957,7 @@ int qwix_hip_quantize(const void* x, int dtype, int64_t outer, int64_t reduce, i
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (inner == 1)  // both layouts coincide
     return run_rows<MODE_QUANT>(x, dtype, outer * (reduce / tile), tile, qtype, calibration, calib_factor, qvalue,
-                                scale, zero_point, nullptr, nullptr, st);
+                                scale, zero_point, nullptr, nullptr, workspace, workspace_bytes, st);
   if (int e = check_cols(x, dtype, reduce, inner, tile, q_layout, qvalue)) return e;
   const ColGeom g = make_col_geom(outer, reduce, inner, tile, dtype == QWIX_BF16 ? 8 : 4);
   if (g.chunks_per_tile == 1)  // a scale group fits one block: calibrate and quantize in one pass, no workspace
@@ -868,7 +980,7 @@ int qwix_hip_calibrate(const void* x, int dtype, int64_t outer, int64_t reduce, 
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (inner == 1)
     return run_rows<MODE_CALIB>(x, dtype, outer * (reduce / tile), tile, QWIX_INT8, calibration, calib_factor,
-                                nullptr, nullptr, nullptr, out0, out1, st);
+                                nullptr, nullptr, nullptr, out0, out1, workspace, workspace_bytes, st);
   if (int e = check_cols(x, dtype, reduce, inner, tile, QWIX_LAYOUT_NATURAL, nullptr)) return e;
   const size_t need = qwix_hip_quantize_workspace_bytes(outer, reduce, inner, tile, calibration);
   if (!workspace || workspace_bytes < need)
@@ -910,7 +1022,8 @@ int qwix_hip_quantize_with_scale(const void* x, int dtype, int64_t outer, int64_
   const int cal = zero_point ? QWIX_MINMAX : QWIX_ABSMAX;
   if (inner == 1)
     return run_rows<MODE_GIVEN>(x, dtype, outer * (reduce / tile), tile, qtype, cal, 0.f, qvalue,
-                                const_cast<void*>(scale), const_cast<void*>(zero_point), nullptr, nullptr, st);
+                                const_cast<void*>(scale), const_cast<void*>(zero_point), nullptr, nullptr, nullptr, 0,
+                                st);
   if (int e = check_cols(x, dtype, reduce, inner, tile, q_layout, qvalue)) return e;
   const ColGeom g = make_col_geom(outer, reduce, inner, tile, dtype == QWIX_BF16 ? 8 : 4);
   return run_cols_quantize<1>(x, dtype, g, qtype, cal, q_layout, nullptr, 0.f, qvalue, const_cast<void*>(scale),

@@ -177,3 +177,52 @@ def test_errors_match_reference_behaviour():
     qarray.quantize(x.to(torch.int32), qarray.HowToQuantize(qtype='int8'))
   with pytest.raises(ValueError, match="doesn't support asymmetric"):
     qarray.quantize(x, qarray.HowToQuantize(qtype='float8_e4m3fn', calibration_method='minmax'))
+
+
+@pytest.mark.parametrize('qtype', QTYPES)
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('shape,kw', [
+    ((512, 1024), dict()),                                   # one scale for the whole array (524288 elements)
+    ((3, 40000), dict(channelwise_axes=[0])),                # rows longer than a workgroup keeps in registers
+    ((2, 6, 20480), dict(channelwise_axes=[0])),             # 122880 contiguous elements per scale
+    ((4, 98304), dict(channelwise_axes=[0], tiled_axes={1: 49152})),
+])
+def test_long_contiguous_groups(shape, kw, dtype, qtype):
+  """Scale groups of more than 16384 contiguous elements are calibrated in pieces and merged."""
+  x_np, x_t = util.make(shape, dtype, seed=len(shape) * 7 + shape[-1] % 13)
+  _check(x_np, x_t, dtype, dict(qtype=qtype, **kw), what='long rows')
+  if qtype == 'int8':
+    _check(x_np, x_t, dtype, dict(qtype=qtype, calibration_method='minmax', **kw), what='long rows minmax')
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+def test_long_contiguous_groups_calibrate_and_static(dtype):
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make((300, 2048), dtype, seed=99)
+  for cal in ('absmax', 'minmax'):
+    how = qarray.HowToQuantize(qtype='int8', calibration_method=cal)
+    ohow = O.HowToQuantize(qtype='int8', calibration_method=cal)
+    c = qarray.calibrate(x_t, how)
+    oc = O.calibrate(O.FArr(x_np, dtype), ohow)
+    for k in oc:
+      assert tuple(c[k].shape) == (1, 1) and np.array_equal(util.f32np(c[k]), oc[k].v), (cal, k)
+    s, zp = qarray.compute_scale_zero_point(c, 'int8')
+    qa = qarray.quantize_with_scale_zero_point(x_t, 'int8', s, zp)   # static range: the scale is given
+    util.assert_qarray_equal(qa, O.quantize(O.FArr(x_np, dtype), ohow), f'static per-tensor {cal}')
+
+
+@pytest.mark.parametrize('qtype', ['int8', 'float8_e4m3fn'])
+def test_static_scale_with_overflowing_quotients(qtype):
+  """A given scale need not come from the data: quotients that overflow or are infinite must still follow
+  true division (saturate), on rows that mix them with ordinary values and on rows that hold none."""
+  from qwix_amd.core import qarray
+  x_np = util.make_np((6, 512), O.BF16, seed=5)
+  x_np[0, :8] = [3e38, -3e38, 1e30, -1e30, np.inf, -np.inf, 0.0, 1.0]
+  x_np[3, 100] = 2e35
+  x_np = O.round_to_bf16(x_np)
+  x_t = util.to_gpu(x_np, O.BF16)
+  for s in (2.0 ** -120, 2.0 ** -20, 1.0):
+    scale_np = np.full((6, 1), s, np.float32)
+    qa = qarray.quantize_with_scale_zero_point(x_t, qtype, util.to_gpu(scale_np, O.BF16), None)
+    want = O.quantize_with_scale_zero_point(O.FArr(x_np, O.BF16), qtype, O.FArr(scale_np, O.BF16), None)
+    util.assert_qarray_equal(qa, want, f'static scale {s}')
