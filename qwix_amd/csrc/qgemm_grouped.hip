@@ -290,7 +290,10 @@ struct Fast {
   static constexpr int kBM = 128, kBN = 256, kBK = 128, kNW = 8, kTM = 4;
 };
 
-template <int BQT, bool SBF>
+// SAG: the activations carry one scale per row and group as well (both operands tiled along K): the
+// tile's (groups x 128 rows) scales are converted to f32 and parked in LDS behind the slab stages; folding a
+// group in then takes convert, multiply, FMA per accumulator instead of convert, FMA.
+template <int BQT, bool SBF, bool SAG>
 __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(GroupedArgs p) {
   constexpr int BM = Fast::kBM, BN = Fast::kBN, BK = Fast::kBK, NW = Fast::kNW, TM = Fast::kTM;
   constexpr bool W4 = (BQT == QWIX_INT4);
@@ -317,6 +320,16 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
     tile_n = (pid % per_group) / gsz;
   }
   const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  float* sa_lds = reinterpret_cast<float*>(smem + 2 * STAGE);  // [group][row of the tile]
+  if constexpr (SAG) {
+    const int ng = p.K / p.group;
+    for (int idx = tid; idx < ng * BM; idx += NW * 64) {
+      const int row = idx & (BM - 1), g = idx / BM;
+      const int m = min(m0 + row, p.M - 1);
+      sa_lds[idx] = ld_scale(p.sa, p.sa_dtype, static_cast<int64_t>(m) * p.ga + g);
+    }
+  }
 
   // ---- loader: wave-uniform 64-bit tile base + per-lane 32-bit offset, rows clamped to the last valid one
   const uint8_t* a_base = p.A + static_cast<int64_t>(m0) * p.lda;
@@ -449,10 +462,25 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
     }
     if (in_group == tpg - 1) {
       const float sb = __uint_as_float(SBF ? sb_raw << 16 : sb_raw) * kUnscale;
+      if constexpr (SAG) {
+        // rows of acc[i][4*qd .. 4*qd+3]: i*32 + 8*qd + 4*hx + 0..3, one 16-byte LDS read (a broadcast per half)
+        const float* sg = sa_lds + (kt / tpg) * BM + 4 * hx;
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) accf[i][r] = __builtin_fmaf(static_cast<float>(acc[i][r]), sb, accf[i][r]);
+          for (int qd = 0; qd < 4; ++qd) {
+            const float4 sa4 = *reinterpret_cast<const float4*>(sg + i * 32 + 8 * qd);
+            const float sv[4] = {sa4.x, sa4.y, sa4.z, sa4.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              accf[i][4 * qd + j] = __builtin_fmaf(static_cast<float>(acc[i][4 * qd + j]) * sv[j], sb, accf[i][4 * qd + j]);
+          }
+      } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) accf[i][r] = __builtin_fmaf(static_cast<float>(acc[i][r]), sb, accf[i][r]);
+      }
       sb_raw = sb_next;
     }
     __syncthreads();
@@ -474,7 +502,7 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int m = m0 + i * 32 + (lane + 64 * q) / 8;
-      sav[i][q] = (p.sa != nullptr && m < p.M) ? ld_scale(p.sa, p.sa_dtype, m) : 1.f;
+      sav[i][q] = (!SAG && p.sa != nullptr && m < p.M) ? ld_scale(p.sa, p.sa_dtype, m) : 1.f;
     }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
@@ -517,22 +545,34 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
   }
 }
 
-template <int BQT, bool SBF>
+// LDS of the fast kernel: two slab stages, plus the f32 activation scales of the tile when they are per group.
+template <int BQT>
+size_t grouped_dma_lds(bool sag, int64_t K, int64_t group) {
+  const size_t stages = 2 * (Fast::kBM * Fast::kBK + Fast::kBN * (BQT == QWIX_INT4 ? 64 : 128));
+  return stages + (sag ? static_cast<size_t>(K / group) * Fast::kBM * sizeof(float) : 0);
+}
+
+template <int BQT, bool SBF, bool SAG>
 int launch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
-  constexpr int BM = Fast::kBM, BN = Fast::kBN, BK = Fast::kBK, NW = Fast::kNW;
-  constexpr size_t smem = 2 * (BM * BK + BN * (BQT == QWIX_INT4 ? 64 : 128));
-  static_assert(smem >= NW * 32 * 36 * sizeof(float), "epilogue staging must fit");
-  auto kern = qgemm_grouped_dma_kernel<BQT, SBF>;
-  static bool configured = false;
-  if (!configured) {
+  constexpr int BM = Fast::kBM, BN = Fast::kBN, NW = Fast::kNW;
+  const size_t smem = grouped_dma_lds<BQT>(SAG, p.K, p.group);
+  static_assert(2 * (Fast::kBM * Fast::kBK + Fast::kBN * 64) >= NW * 32 * 36 * sizeof(float), "epilogue staging must fit");
+  auto kern = qgemm_grouped_dma_kernel<BQT, SBF, SAG>;
+  static size_t configured = 0;  // largest dynamic LDS size allowed so far
+  if (smem > configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
     if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
+    configured = smem;
   }
   const int64_t tiles = static_cast<int64_t>((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   kern<<<dim3(static_cast<unsigned>(tiles)), NW * 64, smem, st>>>(p);
   return check_launch("qgemm_grouped (dma)");
+}
+
+template <int BQT, bool SAG>
+int launch_grouped_dma_sb(const GroupedArgs& p, hipStream_t st) {
+  return p.sb_dtype == QWIX_BF16 ? launch_grouped_dma<BQT, true, SAG>(p, st) : launch_grouped_dma<BQT, false, SAG>(p, st);
 }
 
 }  // namespace
@@ -572,11 +612,17 @@ extern "C" int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b,
   p.acc_out = acc_out;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool row_strides_fit = 128 * lda < (int64_t{1} << 31) && 256 * ldb_bytes < (int64_t{1} << 31);
-  if (!exact && acc_out == nullptr && (sa == nullptr || ga == 1) && row_strides_fit) {
-    const bool sbf = (sb_dtype == QWIX_BF16);
-    if (b_qtype == QWIX_INT4)
-      return sbf ? launch_grouped_dma<QWIX_INT4, true>(p, st) : launch_grouped_dma<QWIX_INT4, false>(p, st);
-    return sbf ? launch_grouped_dma<QWIX_INT8, true>(p, st) : launch_grouped_dma<QWIX_INT8, false>(p, st);
+  if (!exact && acc_out == nullptr && row_strides_fit) {
+    // per-group activation scales ride along in LDS: the tile's scales must fit behind the slab stages
+    const bool sag = sa != nullptr && ga > 1;
+    constexpr size_t kLdsMax = 160 * 1024;
+    if (b_qtype == QWIX_INT4) {
+      if (!sag) return launch_grouped_dma_sb<QWIX_INT4, false>(p, st);
+      if (grouped_dma_lds<QWIX_INT4>(true, K, group) <= kLdsMax) return launch_grouped_dma_sb<QWIX_INT4, true>(p, st);
+    } else {
+      if (!sag) return launch_grouped_dma_sb<QWIX_INT8, false>(p, st);
+      if (grouped_dma_lds<QWIX_INT8>(true, K, group) <= kLdsMax) return launch_grouped_dma_sb<QWIX_INT8, true>(p, st);
+    }
   }
   if (b_qtype == QWIX_INT4)
     return exact ? launch_grouped<QWIX_INT4, true>(p, st) : launch_grouped<QWIX_INT4, false>(p, st);

@@ -74,6 +74,37 @@ def test_grouped_gemm_fast_mode_within_tolerance(M, K, N, group, wq_type, dtype)
     assert np.abs(got - ref).mean() / np.abs(ref).mean() < ceil * 1.1
 
 
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('M,K,N,group', [(256, 1024, 512, 128), (200, 512, 264, 128), (130, 1024, 258, 256), (300, 2048, 1000, 128)])
+def test_grouped_gemm_fast_mode_with_per_group_activation_scales(M, K, N, group, wq_type, dtype):
+  """Both operands tiled along K (what a rule with tile_size gives): the fast kernel folds group g in as
+  acc_g * sa[m, g] * sb[g, n] in f32.  Checked against that closed form built from the oracle's exact integer
+  partials, and against the envelope of the reference's per-partial roundings."""
+  from qwix_amd.core import dot_general as dg
+  print('case grouped fast, both tiled', M, K, N, group, wq_type, dtype, flush=True)
+  xq, wq, oxq, owq, x_np, w_np = _pair(M, K, N, dtype, wq_type, group, seed=5 + M, lhs_tile=group)
+  out = dg.dot_general(xq, wq, DN)
+  torch.cuda.synchronize()
+  want, wacc = O.fast_dot_general(oxq, owq, DN, return_acc=True)
+  got = util.f32np(out)
+  G = K // group
+  sa = np.asarray(oxq.scale.v, np.float64).reshape(M, G).T.reshape(G, M, 1)
+  sb = np.asarray(owq.scale.v, np.float64).reshape(G, 1, N)
+  parts = np.asarray(wacc, np.float64).reshape(G, M, N) * sa * sb
+  exact = parts.sum(0)
+  tol = 2.0 ** -7 if dtype is O.BF16 else 1e-5
+  scale = np.abs(parts).sum(0)
+  assert np.all(np.abs(got - exact) <= tol * scale + 1e-30), (np.abs(got - exact) / (scale + 1e-30)).max()
+  # the reference rounds every partial to the scale dtype: stay within a few roundings of it
+  rt = 2.0 ** -6 if dtype is O.BF16 else 1e-5
+  assert np.all(np.abs(got - want.v) <= rt * scale + 1e-30)
+  if M >= 128:
+    ref = x_np.astype(np.float64) @ w_np.astype(np.float64)
+    ceil = 0.12 if wq_type == 'int4' else 0.02
+    assert np.abs(got - ref).mean() / np.abs(ref).mean() < ceil * 1.1
+
+
 def test_both_sides_tiled_and_natural_layout_weight():
   from qwix_amd.core import dot_general as dg
   xq, wq, oxq, owq, _, _ = _pair(96, 512, 128, O.F32, 'int8', 128, seed=9, lhs_tile=128, layout='natural')
