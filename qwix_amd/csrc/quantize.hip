@@ -730,6 +730,137 @@ __global__ void dequant_kernel(const uint8_t* __restrict__ q, int layout, int64_
   store1<D>(out, idx, rnd<D>(v * load1<D>(scale, si)));
 }
 
+// Quantized byte (or nibble) -> float, as dequant_kernel does it.
+template <int QT>
+__device__ __forceinline__ float q_to_f32(uint32_t b) {
+  if constexpr (QT == QWIX_INT8) return static_cast<float>(static_cast<int>(b << 24) >> 24);
+  else if constexpr (QT == QWIX_E4M3) return e4m3_to_f32(b & 0xFF);
+  else return static_cast<float>(static_cast<int>((b & 0xF) ^ 8) - 8);
+}
+
+// Store 8 consecutive values of D at element index i (a multiple of 8).
+template <typename D>
+__device__ __forceinline__ void store8(void* out, int64_t i, const float* v) {
+  if constexpr (D::kTag == QWIX_BF16) {
+    uint4 w;
+    w.x = f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16);
+    w.y = f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16);
+    w.z = f32_to_bf16_bits(v[4]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[5])) << 16);
+    w.w = f32_to_bf16_bits(v[6]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[7])) << 16);
+    *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(out) + i) = w;
+  } else {
+    float4* o = reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + i);
+    o[0] = make_float4(v[0], v[1], v[2], v[3]);
+    o[1] = make_float4(v[4], v[5], v[6], v[7]);
+  }
+}
+
+// Natural layout, 8 consecutive elements (along the innermost axis) per thread.  inner == 1: the 8 share a
+// scale (tile % 8 == 0); inner > 1: they take 8 consecutive scales (inner % 8 == 0).
+template <typename D, int QT>
+__global__ void __launch_bounds__(256)
+    dequant_vec_kernel(const uint8_t* __restrict__ q, int64_t outer, int64_t reduce, int64_t inner, int64_t tile,
+                       const void* __restrict__ scale, const int8_t* __restrict__ zp, void* __restrict__ out) {
+  const int64_t n = outer * reduce * inner;
+  const int64_t idx = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 8;
+  if (idx >= n) return;
+  uint32_t b[8];
+  if constexpr (QT == QWIX_INT4) {
+    const uint32_t w = *reinterpret_cast<const uint32_t*>(q + idx / 2);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] = (w >> (4 * e)) & 0xF;
+  } else {
+    const uint2 w = *reinterpret_cast<const uint2*>(q + idx);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      b[e] = (w.x >> (8 * e)) & 0xFF;
+      b[4 + e] = (w.y >> (8 * e)) & 0xFF;
+    }
+  }
+  float s[8], z[8];
+  if (inner == 1) {
+    const int64_t si = idx / tile;
+    const float sv = load1<D>(scale, si);
+    const float zv = zp ? rnd<D>(static_cast<float>(zp[si])) : 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      s[e] = sv;
+      z[e] = zv;
+    }
+  } else {
+    const int64_t i = idx % inner, rest = idx / inner, r = rest % reduce, o = rest / reduce;
+    const int64_t si = (o * (reduce / tile) + r / tile) * inner + i;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      s[e] = load1<D>(scale, si + e);
+      z[e] = zp ? rnd<D>(static_cast<float>(zp[si + e])) : 0.f;
+    }
+  }
+  float v[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float t = rnd<D>(q_to_f32<QT>(b[e]));
+    if (zp != nullptr) t = rnd<D>(t - z[e]);
+    v[e] = rnd<D>(t * s[e]);
+  }
+  store8<D>(out, idx, v);
+}
+
+// Reduce-minor layout (values stored (outer, inner, reduce), output (outer, reduce, inner)): a 64 x 64 tile is
+// read along the reduced axis, turned in LDS, and written along the inner axis with its scales, 16 per thread.
+template <typename D, int QT>
+__global__ void __launch_bounds__(256)
+    dequant_rm_kernel(const uint8_t* __restrict__ q, int64_t reduce, int64_t inner, int64_t tile,
+                      const void* __restrict__ scale, const int8_t* __restrict__ zp, void* __restrict__ out) {
+  __shared__ __attribute__((aligned(16))) uint8_t turned[64][80];  // [r][i], rows padded to 80 bytes
+  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * 64, i0 = static_cast<int64_t>(blockIdx.y) * 64;
+  const int64_t o = blockIdx.z;
+  const int t = threadIdx.x;
+  {  // 64 rows (i) x 64 values (r): 16 values per thread
+    const int il = t >> 2, rc = (t & 3) * 16;
+    const int64_t i = i0 + il, r = r0 + rc;
+    uint32_t w[4] = {0, 0, 0, 0};
+    if (i < inner && r < reduce) {
+      const int64_t e = (o * inner + i) * reduce + r;
+      if constexpr (QT == QWIX_INT4) {
+        const uint2 p = *reinterpret_cast<const uint2*>(q + e / 2);
+        w[0] = p.x;
+        w[1] = p.y;
+      } else {
+        const uint4 p = *reinterpret_cast<const uint4*>(q + e);
+        w[0] = p.x; w[1] = p.y; w[2] = p.z; w[3] = p.w;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      uint32_t b;
+      if constexpr (QT == QWIX_INT4) b = (w[k >> 3] >> (4 * (k & 7))) & 0xF;
+      else b = (w[k >> 2] >> (8 * (k & 3))) & 0xFF;
+      turned[rc + k][il] = static_cast<uint8_t>(b);
+    }
+  }
+  __syncthreads();
+  const int rl = t >> 2, ic = (t & 3) * 16;
+  const int64_t r = r0 + rl, i = i0 + ic;
+  if (r >= reduce || i >= inner) return;
+  const uint4 pk = *reinterpret_cast<const uint4*>(&turned[rl][ic]);
+  const uint32_t w[4] = {pk.x, pk.y, pk.z, pk.w};
+  const int64_t si = (o * (reduce / tile) + r / tile) * inner + i;
+  const int64_t oi = (o * reduce + r) * inner + i;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int k = 8 * h + e;
+      float x = rnd<D>(q_to_f32<QT>((w[k >> 2] >> (8 * (k & 3))) & 0xFF));
+      if (zp != nullptr) x = rnd<D>(x - rnd<D>(static_cast<float>(zp[si + k])));
+      v[e] = rnd<D>(x * load1<D>(scale, si + k));
+    }
+    store8<D>(out, oi + 8 * h, v);
+  }
+}
+
 // (rows, cols) elements -> (cols, rows); int4 repacks along the new minor axis.
 template <int QT>
 __global__ void __launch_bounds__(256)
@@ -1074,6 +1205,35 @@ int qwix_hip_dequantize(const void* qvalue, int qtype, int q_layout, int64_t out
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint8_t* q = static_cast<const uint8_t*>(qvalue);
   const int8_t* zp = static_cast<const int8_t*>(zero_point);
+  const bool ptr_ok = aligned16(qvalue) && aligned16(out);
+  // fast paths; the one-thread-per-element kernel below takes every other shape
+  const bool natural = q_layout == QWIX_LAYOUT_NATURAL || inner == 1;
+  if (natural && ptr_ok && n % 8 == 0 && (inner == 1 ? tile % 8 == 0 : inner % 8 == 0)) {
+    const unsigned vb = static_cast<unsigned>((n / 8 + 255) / 256);
+#define QWIX_DEQ_VEC(QTT) dequant_vec_kernel<D, QTT><<<vb, 256, 0, st>>>(q, outer, reduce, inner, tile, scale, zp, out)
+    QWIX_DISPATCH_D(dtype, {
+      if (qtype == QWIX_INT8) QWIX_DEQ_VEC(QWIX_INT8);
+      else if (qtype == QWIX_INT4) QWIX_DEQ_VEC(QWIX_INT4);
+      else if (qtype == QWIX_E4M3) QWIX_DEQ_VEC(QWIX_E4M3);
+      else return fail(QWIX_ERR_INVALID_ARGUMENT, "unknown qtype %d", qtype);
+    })
+#undef QWIX_DEQ_VEC
+    return check_launch("dequantize");
+  }
+  if (!natural && ptr_ok && inner % 16 == 0 && reduce % (qtype == QWIX_INT4 ? 32 : 16) == 0 && outer <= 65535 &&
+      (inner + 63) / 64 <= 65535) {
+    const dim3 grid(static_cast<unsigned>((reduce + 63) / 64), static_cast<unsigned>((inner + 63) / 64),
+                    static_cast<unsigned>(outer));
+#define QWIX_DEQ_RM(QTT) dequant_rm_kernel<D, QTT><<<grid, 256, 0, st>>>(q, reduce, inner, tile, scale, zp, out)
+    QWIX_DISPATCH_D(dtype, {
+      if (qtype == QWIX_INT8) QWIX_DEQ_RM(QWIX_INT8);
+      else if (qtype == QWIX_INT4) QWIX_DEQ_RM(QWIX_INT4);
+      else if (qtype == QWIX_E4M3) QWIX_DEQ_RM(QWIX_E4M3);
+      else return fail(QWIX_ERR_INVALID_ARGUMENT, "unknown qtype %d", qtype);
+    })
+#undef QWIX_DEQ_RM
+    return check_launch("dequantize");
+  }
   QWIX_DISPATCH_D(dtype, {
     if (qtype == QWIX_INT8)
       dequant_kernel<D, QWIX_INT8><<<blocks, 256, 0, st>>>(q, q_layout, outer, reduce, inner, tile, scale, zp, out);

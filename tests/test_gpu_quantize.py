@@ -156,14 +156,27 @@ def test_calibrate_scale_static_pipeline(dtype):
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
 def test_dequantize(dtype, qtype):
   from qwix_amd.core import qarray
-  for shape, kw, layout in [((32, 512), dict(channelwise_axes=[0]), None), ((256, 64), dict(channelwise_axes=[1], tiled_axes={0: 128}), 'natural'),
-                            ((256, 64), dict(channelwise_axes=[1], tiled_axes={0: 128}), 'reduce_minor')]:
+  cases = [((32, 512), dict(channelwise_axes=[0]), None), ((256, 64), dict(channelwise_axes=[1], tiled_axes={0: 128}), 'natural'),
+           ((256, 64), dict(channelwise_axes=[1], tiled_axes={0: 128}), 'reduce_minor'),
+           # shapes that miss the vector paths (odd widths) and shapes with ragged 64 x 64 tiles
+           ((10, 130), dict(channelwise_axes=[0]), None), ((96, 36), dict(channelwise_axes=[1]), 'natural'),
+           ((96, 36), dict(channelwise_axes=[1]), 'reduce_minor'), ((160, 208), dict(channelwise_axes=[1]), 'reduce_minor'),
+           ((1024, 400), dict(channelwise_axes=[1], tiled_axes={0: 256}), 'reduce_minor'),
+           ((3, 128, 80), dict(channelwise_axes=[0, 2]), 'reduce_minor'), ((64, 4096), dict(channelwise_axes=[0], tiled_axes={1: 128}), None),
+           ((512, 96), dict(), None)]
+  for shape, kw, layout in cases:
     x_np, x_t = util.make(shape, dtype, seed=71)
     qa = qarray.quantize(x_t, qarray.HowToQuantize(qtype=qtype, **kw), layout=layout)
     dq = qarray.dequantize(qa)
     want = O.dequantize(O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(qtype=qtype, **kw)))
     assert dq.dtype == util.TORCH_DT[dtype]
     assert np.array_equal(util.f32np(dq), want.v), (shape, kw, layout)
+  if qtype == 'int8':  # zero points on each path
+    for shape, kw, layout in cases[:3] + cases[6:8]:
+      x_np, x_t = util.make(shape, dtype, seed=72, dist='uniform')
+      qa = qarray.quantize(x_t, qarray.HowToQuantize(qtype=qtype, calibration_method='minmax', **kw), layout=layout)
+      want = O.dequantize(O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(qtype=qtype, calibration_method='minmax', **kw)))
+      assert np.array_equal(util.f32np(qarray.dequantize(qa)), want.v), ('minmax', shape, kw, layout)
 
 
 def test_errors_match_reference_behaviour():
