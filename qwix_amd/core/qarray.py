@@ -17,6 +17,7 @@ Differences that come from the device layout, not from the numerics:
 from __future__ import annotations
 
 import dataclasses
+import functools
 import math
 from typing import Any, Callable, Collection, Mapping, Sequence
 
@@ -199,7 +200,7 @@ def validate_qarray(array: QArray) -> None:
 # ------------------------------------------------------------------------------------------
 
 
-@dataclasses.dataclass
+@dataclasses.dataclass(frozen=True)
 class _Plan:
   kind: str                      # '3d' or '5d'
   dims: tuple[int, ...]          # (outer, reduce, inner) or (d0, r1, d2, r3, d4)
@@ -211,6 +212,11 @@ class _Plan:
 
 def _plan(shape: Sequence[int], tiles: Sequence[int]) -> _Plan:
   """tiles[a] = elements of axis a that share one scale (1 = channelwise, dim = fully reduced)."""
+  return _plan_cached(tuple(int(d) for d in shape), tuple(int(t) for t in tiles))
+
+
+@functools.lru_cache(maxsize=4096)
+def _plan_cached(shape: tuple[int, ...], tiles: tuple[int, ...]) -> _Plan:
   blocks: list[list] = []  # ['c', size, axes] or ['r', reduce, tile, axes]
   for a, (d, t) in enumerate(zip(shape, tiles)):
     if d == 1:
