@@ -1172,12 +1172,16 @@ template <int QT, int OUT>
 int launch_batched_dma(const void* a, int64_t lda, const void* b, int64_t ldb, const Batched& bs, int64_t batch,
                        int64_t M, int64_t N, int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   constexpr int BM = 128, BN = 128;
-  constexpr size_t smem = 2 * (BM + BN) * 128;
+  constexpr size_t kStage = (BM + BN) * 128;
+  constexpr size_t kStaging = 4 * 32 * (64 * (OUT == QWIX_BF16 ? 2 : 4) + 16);  // epilogue: 4 wavefronts x 32 padded rows
+  // A single slab (K = 128, e.g. the head dimension of attention scores) never touches the second stage:
+  // half the LDS lets more workgroups share a CU, which is what hides the latency of such short tiles.
+  const size_t smem = K == 128 ? (kStage > kStaging ? kStage : kStaging) : 2 * kStage;
   auto kern = qgemm_batched_dma_kernel<QT, BM, BN, 2, 2, OUT>;
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(2 * kStage));
     if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     configured = true;
   }
