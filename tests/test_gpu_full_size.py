@@ -1,0 +1,130 @@
+"""GPU: size-independent properties at the full benchmark shapes, where the oracle would take minutes.
+
+Operands are small integers, so that every product and every partial sum is an exact integer in f32 whatever
+the accumulation order: sampled output rows must equal an int64 product computed on the host, and the sum of
+all outputs must equal (column sums of a) . (row sums of b), a checksum of checksums."""
+import numpy as np
+import pytest
+import torch
+
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+
+def _small_ints(shape, lo, hi, seed, dtype):
+  g = torch.Generator(device='cpu').manual_seed(seed)
+  return torch.randint(lo, hi + 1, shape, generator=g, dtype=torch.int8).to(util.DEV).to(dtype)
+
+
+def _check_rows_and_checksum(out, a_int, b_nk_int, rows):
+  """out (M, N) float/int tensor on the GPU; a_int (M, K), b_nk_int (N, K) int8 tensors on the GPU."""
+  want = a_int[rows].cpu().numpy().astype(np.int64) @ b_nk_int.cpu().numpy().astype(np.int64).T
+  assert np.array_equal(out[rows].cpu().to(torch.float64).numpy(), want.astype(np.float64))
+  total = out.to(torch.float64).sum().item()
+  want_total = float(a_int.to(torch.float64).sum(0).cpu().numpy() @ b_nk_int.to(torch.float64).sum(0).cpu().numpy())
+  assert total == want_total
+
+
+def test_fp8_gemm_at_the_ffn_shape():
+  """(8192, 8192) x (8192, 28672) e4m3, f32 out, no scales: values in -2..2 are exact in e4m3, sums stay below 2^24."""
+  from qwix_amd import _lib
+  M, K, N = 8192, 8192, 28672
+  a_i = _small_ints((M, K), -2, 2, 1, torch.int8)
+  b_i = _small_ints((N, K), -2, 2, 2, torch.int8)
+  a, b = a_i.to(torch.float32).to(torch.float8_e4m3fn), b_i.to(torch.float32).to(torch.float8_e4m3fn)
+  out = torch.empty(M, N, dtype=torch.float32, device=util.DEV)
+  print('case fp8 full size', M, K, N, flush=True)
+  _lib.call('qwix_hip_qgemm', a.data_ptr(), K, b.data_ptr(), K, _lib.E4M3, M, N, K, None, 0, None, 0, _lib.F32,
+            out.data_ptr(), _lib.F32, N, _lib.stream_of(a))
+  torch.cuda.synchronize()
+  rows = util.rng(3).choice(M, 8, replace=False)
+  _check_rows_and_checksum(out, a_i, b_i, rows)
+
+
+def test_int8_gemm_bf16_epilogue_at_8192():
+  """8192^3 int8 through the scaled epilogue (power-of-two scales keep every value exact in bf16)."""
+  from qwix_amd import _lib
+  M = N = K = 8192
+  a = _small_ints((M, K), -1, 1, 5, torch.int8)
+  b = _small_ints((N, K), -1, 1, 6, torch.int8)
+  # |sum| <= 8192 -> needs 14 bits: keep it exact in bf16 by making operands sparse enough: |sum| < 256
+  a = a * (torch.rand(M, K, device=util.DEV) < 0.01).to(torch.int8)
+  sa = torch.full((M,), 0.5, dtype=torch.bfloat16, device=util.DEV)
+  sb = torch.full((N,), 4.0, dtype=torch.bfloat16, device=util.DEV)
+  out = torch.empty(M, N, dtype=torch.bfloat16, device=util.DEV)
+  print('case int8 full size', M, K, N, flush=True)
+  _lib.call('qwix_hip_qgemm', a.data_ptr(), K, b.data_ptr(), K, _lib.INT8, M, N, K, sa.data_ptr(), _lib.BF16,
+            sb.data_ptr(), _lib.BF16, 0, out.data_ptr(), _lib.BF16, N, _lib.stream_of(a))
+  torch.cuda.synchronize()
+  rows = util.rng(4).choice(M, 8, replace=False)
+  want = a[rows].cpu().numpy().astype(np.int64) @ b.cpu().numpy().astype(np.int64).T
+  assert np.abs(want).max() < 256
+  assert np.array_equal(out[rows].float().cpu().numpy(), want.astype(np.float32) * 2.0)
+
+
+def test_grouped_a8w4_gemm_at_the_hadamard_shape():
+  """(2048, 8192) int8 x (8192, 8192) int4, groups of 128, unit scales: the f32 sum of the int32 partials is exact."""
+  from qwix_amd import _lib
+  from qwix_amd.core.qarray import Int4Tensor
+  M, K, N, G = 2048, 8192, 8192, 128
+  a = _small_ints((M, K), -127, 127, 7, torch.int8)
+  b_i = _small_ints((N, K), -8, 7, 8, torch.int8)           # (N, K) K-contiguous logical values
+  packed = Int4Tensor.pack(b_i).data if hasattr(Int4Tensor, 'pack') else None
+  if packed is None:
+    u = (b_i.to(torch.int16) & 0xF).to(torch.uint8)
+    packed = (u[:, 0::2] | (u[:, 1::2] << 4)).contiguous()
+  sb = torch.ones(K // G, N, dtype=torch.float32, device=util.DEV)
+  out = torch.empty(M, N, dtype=torch.float32, device=util.DEV)
+  print('case grouped full size', M, K, N, flush=True)
+  _lib.call('qwix_hip_qgemm_grouped', a.data_ptr(), K, packed.data_ptr(), K // 2, _lib.INT4, M, N, K, G, None, 0, 1,
+            sb.data_ptr(), _lib.F32, out.data_ptr(), _lib.F32, N, 0, None, _lib.stream_of(a))
+  torch.cuda.synchronize()
+  rows = util.rng(5).choice(M, 8, replace=False)
+  _check_rows_and_checksum(out, a, b_i, rows)
+
+
+def test_ragged_gemm_at_the_moe_shape():
+  """8192 tokens, 8 experts, K 4096, N 14336: every row against its own expert, leftover rows zero."""
+  from qwix_amd import _lib
+  M, K, N, G = 8192, 4096, 14336, 8
+  a = _small_ints((M, K), -15, 15, 9, torch.int8)
+  b = _small_ints((G, N, K), -15, 15, 10, torch.int8)
+  sizes_host = [1000, 1100, 900, 1024, 1500, 600, 1000, 1000]   # 8124 rows: the last 68 belong to no expert
+  sizes = torch.tensor(sizes_host, dtype=torch.int32, device=util.DEV)
+  out = torch.full((M, N), 7.0, dtype=torch.float32, device=util.DEV)
+  print('case ragged full size', M, K, N, G, flush=True)
+  _lib.call('qwix_hip_qgemm_ragged', a.data_ptr(), K, b.data_ptr(), K, N * K, _lib.INT8, M, N, K, sizes.data_ptr(), G,
+            None, 0, None, 0, 0, 0, out.data_ptr(), _lib.F32, N, _lib.stream_of(a))
+  torch.cuda.synchronize()
+  starts = np.concatenate([[0], np.cumsum(sizes_host)])
+  rows = np.array([0, 999, 1000, 2099, 2100, 4023, 4024, 8123])
+  for r in rows:
+    g = int(np.searchsorted(starts, r, side='right') - 1)
+    want = a[r].cpu().numpy().astype(np.int64) @ b[g].cpu().numpy().astype(np.int64).T
+    assert np.array_equal(out[r].cpu().numpy().astype(np.int64), want), (r, g)
+  assert torch.count_nonzero(out[starts[-1]:]).item() == 0
+  # checksum per expert: sum of its rows' outputs == (column sums of its rows) . (row sums of its weight)
+  for g in range(G):
+    blk = out[starts[g]:starts[g + 1]].to(torch.float64).sum().item()
+    want = float(a[starts[g]:starts[g + 1]].to(torch.float64).sum(0).cpu().numpy() @ b[g].to(torch.float64).sum(0).cpu().numpy())
+    assert blk == want, g
+
+
+def test_activation_quantize_at_8192_square():
+  """Per-token int8 / e4m3 quantize of (8192, 8192) bf16, checked by torch arithmetic as an independent hand:
+  scale = bf16(absmax / qmax) per row, and every value lies within half a step (one bf16 rounding of the
+  quotient included) of its reconstruction."""
+  from qwix_amd.core import qarray
+  g = torch.Generator(device='cpu').manual_seed(11)
+  x = torch.randn(8192, 8192, generator=g, dtype=torch.float32).to(torch.bfloat16).to(util.DEV)
+  for qtype, qmax in (('int8', 127.5), ('float8_e4m3fn', 448.0)):
+    q = qarray.quantize(x, qarray.HowToQuantize(qtype=qtype, channelwise_axes=[0]))
+    absmax = x.abs().amax(dim=1, keepdim=True)
+    want_scale = (absmax.float() / qmax).to(torch.bfloat16)
+    assert torch.equal(q.scale, want_scale), qtype
+    quot = (x.float() / q.scale.float()).to(torch.bfloat16).float()
+    if qtype == 'int8':
+      assert torch.equal(q.qvalue.float(), torch.clamp(torch.round(quot), -128, 127))
+    else:
+      assert torch.equal(q.qvalue.float(), torch.clamp(quot, -448, 448).to(torch.float8_e4m3fn).float())
