@@ -650,6 +650,63 @@ class QdotBatched(Workload):
             'ops': 2.0 * self.B * self.Q * self.Kv * self.D}
 
 
+class PtqMlpGraph(Workload):
+  """The reference's own example configuration (MLP 1024 -> 4096 -> 1024 on 256 tokens, int8 weights and
+  activations) through the provider surface: four small kernels per forward, launch-bound.  The forward is
+  captured once into a HIP graph and replayed; the eager time of the same forward is reported beside it."""
+
+  bound = 'mfma'
+
+  def __init__(self, name):
+    self.name = name
+    self.dtype = 'int8'
+    self.metric = 'PTQ MLP forward TOPS (int8 w8a8 through the provider, HIP graph replay)'
+    self.unit = 'TOPS'
+    self.kernel_name = 'graph'
+    self.ops = 2.0 * 2 * 256 * 1024 * 4096
+
+  def setup(self, dev):
+    import torch
+    import qwix_amd
+    from qwix_amd import nn
+    model = nn.MLP(4096, 1024)
+    g = torch.Generator().manual_seed(1001)
+    params = model.init(g, 1024, torch.float32, dev)
+    self.x = torch.rand(256, 1024, generator=g, dtype=torch.float32).to(dev)
+    rules = [qwix_amd.QuantizationRule(module_path='.*', weight_qtype='int8', act_qtype='int8')]
+    self.model = qwix_amd.quantize_model(model, qwix_amd.PtqProvider(rules))
+    self.qparams = qwix_amd.quantize_params(params, self.model.init(params, self.x))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+      for _ in range(3):
+        self.model.apply(self.qparams, self.x)
+    torch.cuda.current_stream().wait_stream(side)
+    self.graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(self.graph):
+      self.out = self.model.apply(self.qparams, self.x)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(200):
+      self.model.apply(self.qparams, self.x)
+    torch.cuda.synchronize()
+    self.eager_us = (time.perf_counter() - t0) / 200 * 1e6
+
+  def step(self, i=0):
+    self.graph.replay()
+
+  kernel = step
+
+  def work_per_step(self):
+    return self.ops
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'tokens': 256, 'layers': '1024 -> 4096 -> 1024', 'weights': 'int8 per channel',
+            'activations': 'int8 per token, quantized on the fly', 'eager_us_per_forward': round(self.eager_us, 1)}
+
+
 WORKLOADS = {
     'c3_int8_w8a8_4096': lambda: QdotW8A8('c3_int8_w8a8_4096', 4096, 4096, 4096, 'int8'),
     'c4_fp8_w8a8_ffn': lambda: QdotW8A8('c4_fp8_w8a8_ffn', 8192, 8192, 28672, 'float8_e4m3fn'),
@@ -672,12 +729,13 @@ WORKLOADS = {
     'srq_quantize_act_4096': lambda: QuantizeStatic('srq_quantize_act_4096', 4096, 4096),
     'zp_int8_w8a8_4096': lambda: QdotZeroPoint('zp_int8_w8a8_4096', 4096, 4096, 4096),
     'batched_qk_int8_32x2048': lambda: QdotBatched('batched_qk_int8_32x2048', 32, 2048, 2048, 128),
+    'c1_ptq_mlp_graph': lambda: PtqMlpGraph('c1_ptq_mlp_graph'),
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
 }
 DEFAULT = 'c3_int8_w8a8_4096'
 EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16',
          'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'moe_ragged_int8_8x1024',
-         'moe_ragged_int8_64x128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048']
+         'moe_ragged_int8_64x128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 
 
 def _blas_threads() -> int:

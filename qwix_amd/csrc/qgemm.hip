@@ -1545,7 +1545,16 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
     return rc;
   const Epilogue ep = make_epilogue(qtype, sa, sa_dtype, sb, sb_dtype, acc_dtype, zu, zv, out_dtype);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (M <= 32 && K % 128 == 0 && 16 * lda < (int64_t{1} << 31) && 64 * ldb < (int64_t{1} << 31)) {
+  // Few rows: stream the weights instead of tiling.  Up to 32 rows always; up to 256 rows while a rough cost
+  // model favours it: the skinny kernel makes one pass over the weights per 16 rows (from L2 after the first,
+  // about 0.5 us + 5.2 bytes/ns each) after a 4 us start, the tiled kernels walk K in 128-wide slabs of about
+  // 0.55 us after 5 us, however few of the chip's CUs their 128 x 128 tiles occupy.
+  const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+  const double passes = static_cast<double>((M + 15) / 16);
+  const double skinny_us = 4.0 + passes * (0.5 + static_cast<double>(N) * static_cast<double>(K) / 5.2e6);
+  const double tiled_us = 5.0 + 0.55 * static_cast<double>(K / 128);
+  const bool few_rows = M <= 32 || (M <= 256 && tiles128 <= 256 && skinny_us < tiled_us);
+  if (few_rows && K % 128 == 0 && M * lda < (int64_t{1} << 31) && 64 * ldb < (int64_t{1} << 31)) {
     if (qtype == QWIX_INT8) return launch_skinny<QWIX_INT8>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     return launch_skinny<QWIX_E4M3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
   }

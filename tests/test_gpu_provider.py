@@ -141,3 +141,32 @@ def test_small_tile_rule_takes_the_dequantize_path():
   util.assert_qarray_equal(qp['kernel'].array, ow, 'tile 4 weight')
   want = O.dot_general(util.farr(x), ow, DN)
   assert np.allclose(util.f32np(out), want.v, rtol=1e-5, atol=1e-6)
+
+
+def test_ptq_mlp_forward_replays_from_a_hip_graph():
+  """The launch-bound configuration (four small kernels per forward) captured once and replayed: no entry
+  point allocates or synchronises, so the whole quantized forward is graph-safe.  Every replay, with the
+  program's own eager work and synchronisations in between, must reproduce the eager result bit for bit."""
+  import qwix_amd
+  model, params, x, rules = _mlp_setup()
+  ptq_model = qwix_amd.quantize_model(model, qwix_amd.PtqProvider(rules))
+  qparams = qwix_amd.quantize_params(params, ptq_model.init(params, x))
+  static_x = x.clone()
+  s = torch.cuda.Stream()
+  s.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(s):
+    for _ in range(2):
+      ptq_model.apply(qparams, static_x)      # warm-up on the side stream (lazy initialisations)
+  torch.cuda.current_stream().wait_stream(s)
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    static_out = ptq_model.apply(qparams, static_x)
+  g = torch.Generator().manual_seed(5)
+  for i in range(4):
+    xi = torch.rand(x.shape, generator=g, dtype=torch.float32).to(util.DEV) * (i + 1)
+    eager = ptq_model.apply(qparams, xi)       # eager work between the replays
+    torch.cuda.synchronize()
+    static_x.copy_(xi)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(static_out, eager), i
