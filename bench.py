@@ -406,6 +406,28 @@ class QdotDecode(Workload):
     return {'workload': self.name, 'M': self.M, 'K': self.K, 'N': self.N, 'weight_copies_rotated': self.copies}
 
 
+class QdotDecodeFused(QdotDecode):
+  """The same decode step in one launch: the per-token quantization of the activations happens inside the
+  skinny GEMM (every workgroup re-derives the row scales from the bf16 activations it reads from L2)."""
+
+  def __init__(self, name, M, K, N):
+    super().__init__(name, M, K, N)
+    self.metric = 'w8a8 int8 decode GB/s (activation quantize fused into the GEMM launch)'
+    self.kernel_name = 'qgemm_skinny_fused_kernel'
+
+  def step(self, i=0):
+    L = self.L
+    L.call('qwix_hip_qgemm_fused_act', self.x.data_ptr(), L.BF16, self.K, self.b[i % self.copies].data_ptr(), self.K,
+           self.M, self.N, self.K, self.sb.data_ptr(), L.BF16, self.out.data_ptr(), L.BF16, self.N, self.stream)
+
+  kernel = step
+
+  def work_per_step(self):
+    return self.K * self.N + self.N * 2.0 + self.M * self.K * 2.0 + self.M * self.N * 2.0
+
+  kernel_work = work_per_step
+
+
 class HadamardQdot(Workload):
   """C5: FWHT + per-token int8 quantize of the activations each step, then int8 x int4 g128 grouped GEMM
   against the offline-rotated weight."""
@@ -715,6 +737,8 @@ WORKLOADS = {
     'quantize_act_4096': lambda: QuantizeRows('quantize_act_4096', 4096, 4096, 'int8'),
     'quantize_act_8192_fp8': lambda: QuantizeRows('quantize_act_8192_fp8', 8192, 8192, 'float8_e4m3fn'),
     'w8a8_decode_m16': lambda: QdotDecode('w8a8_decode_m16', 16, 4096, 14336),
+    'w8a8_decode_m16_k2048': lambda: QdotDecode('w8a8_decode_m16_k2048', 16, 2048, 8192),
+    'w8a8_decode_m16_k2048_fused': lambda: QdotDecodeFused('w8a8_decode_m16_k2048_fused', 16, 2048, 8192),
     'c2_gemv_w4_m1': lambda: GemvW4('c2_gemv_w4_m1', 1, 4096, 14336, 128),
     'c2_gemv_w4_m16': lambda: GemvW4('c2_gemv_w4_m16', 16, 4096, 14336, 128),
     'c4_quantize_weight_fp8': lambda: QuantizeWeight('c4_quantize_weight_fp8', 8192, 28672, 'float8_e4m3fn'),
@@ -733,7 +757,7 @@ WORKLOADS = {
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
 }
 DEFAULT = 'c3_int8_w8a8_4096'
-EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16',
+EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
          'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'moe_ragged_int8_8x1024',
          'moe_ragged_int8_64x128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 

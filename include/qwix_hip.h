@@ -170,6 +170,21 @@ QWIX_API int qwix_hip_qgemm_batched(const void* a, int64_t lda, int64_t a_batch_
                            void* out, int out_dtype, int64_t ldo, int64_t out_batch_stride,
                            void* stream);
 
+/* Decode-size w8a8 with the activation quantization folded into the GEMM: per-token absmax int8
+ * quantization of x (quantize, qwix/_src/core/qarray.py:638-644, as PtqProvider applies it to the
+ * lhs of dot_general, providers/boxed_param.py:416-455) followed by _fast_dot_general
+ * (dot_general.py:135-261) in one launch; the counterpart, for M <= 32, of the Pallas kernel
+ * qwix/contrib/kernels/lhs_fused_quantized_matmul.py.  Results are bit-identical to
+ * qwix_hip_quantize + qwix_hip_qgemm:
+ *     s[m] = D(max_k |x[m,k]| / 127.5) (1 if below 2^-63),  q = sat(rint(D(x / s))),
+ *     out[m,n] = cast_R( (T(sum_k q[m,k] b[n,k]) * s[m]) * sb[n] ),   D = dtype of x.
+ * x: (M, K) of x_dtype (QWIX_BF16 / QWIX_F32), row pitch ldx elements; b: (N, K) int8; M <= 32,
+ * K % 128 == 0, K <= 2048: every workgroup re-derives the quantized rows it needs, which beats a
+ * separate quantize launch only while K is short. */
+QWIX_API int qwix_hip_qgemm_fused_act(const void* x, int x_dtype, int64_t ldx, const void* b, int64_t ldb,
+                             int64_t M, int64_t N, int64_t K, const void* sb, int sb_dtype, void* out,
+                             int out_dtype, int64_t ldo, void* stream);
+
 /* out[r] = sum_k q[r*ld + k] for int8 rows (K % 16 == 0): the K-sums qwix_hip_qgemm_zp needs
  * (the reference obtains them as a dot_general against the broadcast zero point,
  * dot_general.py:233-239,246-252). */

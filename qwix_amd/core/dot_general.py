@@ -280,6 +280,37 @@ def _batched_qgemm(lhs, rhs, dimension_numbers, preferred_element_type):
   return out.reshape(*bshape, *[lshape[a] for a in lfree], *[rshape[a] for a in rfree])
 
 
+def fused_act_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None):
+  """Dynamic per-token int8 quantization of a float lhs and the quantized contraction in one launch
+  (qwix_hip_qgemm_fused_act), for decode-size calls: at most 32 rows and K <= 2048 against a per-channel int8 weight.
+  Bit-identical to quantize(lhs, channelwise over the non-contracting axes) followed by dot_general.
+  Returns None when the operands do not fit that kernel; the caller then takes the two-step route."""
+  if not (_is_float_array(lhs) and lhs.dtype in (torch.bfloat16, torch.float32) and isinstance(rhs, QArray)):
+    return None
+  if rhs.zero_point is not None or isinstance(rhs.qvalue, Int4Tensor) or _qtype_of(rhs) != numerics.INT8:
+    return None
+  (lca, rca), (lba, rba) = dimension_numbers
+  if len(lba) or len(rba) or any(rhs.scale.shape[int(a)] != 1 for a in rca):
+    return None
+  try:
+    c = _Canon(lhs, rhs, dimension_numbers)
+  except ValueError:
+    return None
+  if not (0 < c.M <= 32) or c.K % 128 or c.K > 2048:
+    return None
+  x = c.lhs_values(lhs)
+  b, _ = c.rhs_values(rhs)
+  sb, _ = c.rhs_scale(rhs)
+  res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.scale.dtype)
+  if res_t not in (torch.bfloat16, torch.float32):
+    return None
+  out = torch.empty(c.M, c.N, dtype=res_t, device=x.device)
+  _lib.call('qwix_hip_qgemm_fused_act', x.data_ptr(), _lib.float_tag(x.dtype), x.stride(0), b.data_ptr(), b.stride(0),
+            c.M, c.N, c.K, sb.data_ptr(), _lib.float_tag(sb.dtype), out.data_ptr(), _lib.float_tag(res_t), c.N,
+            _lib.stream_of(x))
+  return out.reshape(c.out_shape)
+
+
 def _tag_of(dtype: torch.dtype) -> int:
   if dtype == torch.int32:
     return _lib.I32

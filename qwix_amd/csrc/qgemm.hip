@@ -1371,6 +1371,159 @@ int launch_skinny(const void* a, int64_t lda, const void* b, int64_t ldb, int64_
   return check_launch("qgemm (skinny)");
 }
 
+// ------------------------------------------------------------------------------------------------
+// Decode with the activation quantization folded in (int8, M <= 32 per call): the float activations are
+// what the kernel reads.  Every workgroup keeps its 16 rows in registers (the 16 wavefronts split K as in
+// the skinny kernel, a lane holds the 32 consecutive k of one row that its MFMA operand needs), finds the
+// rows' absmax (lanes of a row by shuffle, wavefronts through LDS; a maximum does not depend on the order),
+// derives the scale exactly as the stand-alone quantize kernel does, quantizes its registers and goes on
+// as the skinny kernel.  The quantized values and scales are bit-identical to quantize-then-multiply; they
+// are recomputed by every workgroup from L2 (16 x K activations against 16 * NT x K weights), which is
+// cheaper than a kernel launch of its own as long as K is short.  KB: 128-wide K blocks per wavefront
+// (K <= 2048 * KB; only KB = 1 is instantiated).
+template <typename D, int NT, int KB>
+__global__ void __launch_bounds__(kSkinnyWaves * 64)
+    qgemm_skinny_fused_kernel(const uint8_t* __restrict__ X, int64_t ldx, const uint8_t* __restrict__ B, int64_t ldb,
+                              int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  constexpr int ES = D::kTag == QWIX_BF16 ? 2 : 4;   // bytes per activation
+  constexpr int XV = 32 * ES / 16;                    // 16-byte loads per lane and K block (32 elements)
+  __shared__ v4i red[kSkinnyWaves][NT][64];
+  __shared__ float rowmax[kSkinnyWaves][16];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15, kq = lane >> 4;
+  const int n_base = blockIdx.x * (16 * NT), row0 = blockIdx.y * 16;
+  const int nblk = K / 128;
+  const int kb0 = wave * KB, kb1 = min(nblk, kb0 + KB);  // nblk <= 16 * KB
+
+  const uint8_t* x_base = X + static_cast<int64_t>(row0) * ldx * ES;
+  const uint8_t* b_base = B + static_cast<int64_t>(n_base) * ldb;
+  const uint32_t x_off = static_cast<uint32_t>(min(col, M - 1 - row0)) * static_cast<uint32_t>(ldx * ES) + kq * 32 * ES;
+  uint32_t b_off[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+    b_off[t] = static_cast<uint32_t>(min(t * 16 + col, N - 1 - n_base)) * static_cast<uint32_t>(ldb) + kq * 32;
+
+  // ---- this lane's activations and weights for all of its K blocks
+  uint4 xr[KB][XV];
+  v4i w[KB][NT][2];
+#pragma unroll
+  for (int j = 0; j < KB; ++j) {
+    const int kb = kb0 + j;
+#pragma unroll
+    for (int v = 0; v < XV; ++v) xr[j][v] = make_uint4(0, 0, 0, 0);
+    if (kb < kb1) {
+      const uint8_t* xp = x_base + static_cast<int64_t>(kb) * 128 * ES + x_off;
+#pragma unroll
+      for (int v = 0; v < XV; ++v) xr[j][v] = *reinterpret_cast<const uint4*>(xp + 16 * v);
+      const uint8_t* bp = b_base + kb * 128;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        w[j][t][0] = *reinterpret_cast<const v4i*>(bp + b_off[t]);
+        w[j][t][1] = *reinterpret_cast<const v4i*>(bp + b_off[t] + 16);
+      }
+    }
+  }
+
+  // ---- absmax of the 16 rows
+  float mx = 0.f;
+#pragma unroll
+  for (int j = 0; j < KB; ++j)
+#pragma unroll
+    for (int v = 0; v < XV; ++v) {
+      float f[D::kVec];
+      unpack16<D>(xr[j][v], f);
+#pragma unroll
+      for (int e = 0; e < D::kVec; ++e) mx = fmaxf(mx, __builtin_fabsf(f[e]));
+    }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  if (lane < 16) rowmax[wave][lane] = mx;
+  __syncthreads();
+  mx = rowmax[0][col];
+#pragma unroll
+  for (int wv = 1; wv < kSkinnyWaves; ++wv) mx = fmaxf(mx, rowmax[wv][col]);
+  const float s = sym_scale<D, QWIX_INT8>(mx);  // the scale of row `col`, as the quantize kernel derives it
+  const Divider<D, false, false> div(s);
+
+  // ---- quantize the registers, multiply
+  v4i acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[t][e] = 0;
+#pragma unroll
+  for (int j = 0; j < KB; ++j) {
+    if (kb0 + j < kb1) {
+      uint32_t qw[8];  // 32 int8 values, 4 per word, in k order
+      constexpr int PER = D::kVec / 4;  // words a 16-byte vector turns into
+#pragma unroll
+      for (int v = 0; v < XV; ++v) {
+        float f[D::kVec];
+        unpack16<D>(xr[j][v], f);
+#pragma unroll
+        for (int h = 0; h < PER; ++h)
+          qw[v * PER + h] = pack4_low_bytes(rne_bits_clamped(div(f[4 * h]), -128.f, 127.f),
+                                            rne_bits_clamped(div(f[4 * h + 1]), -128.f, 127.f),
+                                            rne_bits_clamped(div(f[4 * h + 2]), -128.f, 127.f),
+                                            rne_bits_clamped(div(f[4 * h + 3]), -128.f, 127.f));
+      }
+      const v4i x0 = {static_cast<int>(qw[0]), static_cast<int>(qw[1]), static_cast<int>(qw[2]), static_cast<int>(qw[3])};
+      const v4i x1 = {static_cast<int>(qw[4]), static_cast<int>(qw[5]), static_cast<int>(qw[6]), static_cast<int>(qw[7])};
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(x0, w[j][t][0], acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(x1, w[j][t][1], acc[t], 0, 0, 0);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int t = 0; t < NT; ++t) red[wave][t][lane] = acc[t];
+  // the row scales in the result's lane layout: row m = 4 * (lane / 16) + e of the block
+  __shared__ float srow[16];
+  if (wave == 0 && lane < 16) srow[lane] = s;
+  __syncthreads();
+  const bool r0 = ep.r0 != 0, r1 = ep.r1 != 0, r2 = ep.r2 != 0;
+  for (int idx = tid; idx < NT * 256; idx += kSkinnyWaves * 64) {
+    const int t = idx >> 8, e = (idx >> 6) & 3, l = idx & 63;
+    const int mr = 4 * (l >> 4) + e;
+    const int m = row0 + mr, n = n_base + t * 16 + (l & 15);
+    if (m >= M || n >= N) continue;
+    int a = 0;
+#pragma unroll
+    for (int wv = 0; wv < kSkinnyWaves; ++wv) a += red[wv][t][l][e];
+    float v = static_cast<float>(a);
+    if (r0) v = round_bf16(v);
+    v *= srow[mr];
+    if (r1) v = round_bf16(v);
+    if (ep.sb != nullptr) v *= load_scale(ep.sb, ep.sb_dtype, n);
+    if (r2) v = round_bf16(v);
+    if (ep.out_dtype == QWIX_BF16)
+      reinterpret_cast<uint16_t*>(out)[static_cast<int64_t>(m) * ldo + n] = f32_to_bf16_bits(v);
+    else
+      reinterpret_cast<float*>(out)[static_cast<int64_t>(m) * ldo + n] = v;
+  }
+}
+
+template <typename D, int KB>
+int launch_skinny_fused(const void* x, int64_t ldx, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                        const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  const unsigned gy = static_cast<unsigned>((M + 15) / 16);
+#define QWIX_FUSED(NTT)                                                                                              \
+  qgemm_skinny_fused_kernel<D, NTT, KB><<<dim3(static_cast<unsigned>((N + 16 * NTT - 1) / (16 * NTT)), gy),         \
+                                          kSkinnyWaves * 64, 0, st>>>(static_cast<const uint8_t*>(x), ldx,           \
+                                                                      static_cast<const uint8_t*>(b), ldb,           \
+                                                                      static_cast<int>(M), static_cast<int>(N),      \
+                                                                      static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo)
+  if (N >= 192 * 32)
+    QWIX_FUSED(2);
+  else
+    QWIX_FUSED(1);
+#undef QWIX_FUSED
+  return check_launch("qgemm (skinny, fused activation quantize)");
+}
+
 // out[r] = sum_k q[r, k] over int8 rows: one wavefront per row, 16 bytes per lane and trip.
 __global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__ q, int64_t ld, int rows, int K,
                                                       int32_t* __restrict__ out) {
@@ -1448,6 +1601,32 @@ static int check_gemm_args(const void* a, int64_t lda, const void* b, int64_t ld
   if (out_dtype != QWIX_I32 && !ok_s(out_dtype)) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad out dtype %d", out_dtype);
   if (qtype == QWIX_E4M3 && !ok_s(acc_dtype)) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad accumulator dtype %d", acc_dtype);
   return QWIX_OK;
+}
+
+extern "C" int qwix_hip_qgemm_fused_act(const void* x, int x_dtype, int64_t ldx, const void* b, int64_t ldb,
+                                        int64_t M, int64_t N, int64_t K, const void* sb, int sb_dtype, void* out,
+                                        int out_dtype, int64_t ldo, void* stream) {
+  if (!x || !b || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null x/b/out");
+  if (x_dtype != QWIX_BF16 && x_dtype != QWIX_F32) return fail(QWIX_ERR_INVALID_ARGUMENT, "activations must be bf16 or f32");
+  if ((sb && sb_dtype != QWIX_BF16 && sb_dtype != QWIX_F32) || (out_dtype != QWIX_BF16 && out_dtype != QWIX_F32))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "scale and output dtypes must be f32 or bf16");
+  const int es = x_dtype == QWIX_BF16 ? 2 : 4;
+  // One 128-wide K block per wavefront: beyond K = 2048 the arithmetic of re-quantizing the rows in every
+  // workgroup costs more than the launch of a separate quantize kernel saves (measured: K = 1024 runs in half
+  // the time of the two launches, K = 4096 in the same time).
+  constexpr int64_t kMaxK = 128 * kSkinnyWaves;
+  if (M <= 0 || M > 32 || N <= 0 || N > INT32_MAX || K <= 0 || K % 128 || K > kMaxK)
+    return fail(QWIX_ERR_UNSUPPORTED, "fused activation quantize needs 1..32 rows and K a multiple of 128 up to %lld "
+                "(M=%lld K=%lld)", (long long)kMaxK, (long long)M, (long long)K);
+  if (ldx < K || (ldx * es) % 16 || ldb < K || ldb % 16 || !aligned16(x) || !aligned16(b) || ldo < N ||
+      32 * ldx * es >= (int64_t{1} << 31) || 64 * ldb >= (int64_t{1} << 31))
+    return fail(QWIX_ERR_UNSUPPORTED, "bad leading dimensions or alignment (ldx=%lld ldb=%lld ldo=%lld)", (long long)ldx,
+                (long long)ldb, (long long)ldo);
+  // the activation scale is computed in the activations' dtype, like the stand-alone quantize does
+  const Epilogue ep = make_epilogue(QWIX_INT8, x, x_dtype, sb, sb_dtype, 0, nullptr, nullptr, out_dtype);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (x_dtype == QWIX_BF16) return launch_skinny_fused<BF16, 1>(x, ldx, b, ldb, M, N, K, ep, out, ldo, st);
+  return launch_skinny_fused<F32, 1>(x, ldx, b, ldb, M, N, K, ep, out, ldo, st);
 }
 
 extern "C" int qwix_hip_qgemm_ragged(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t b_group_stride,

@@ -104,7 +104,7 @@ class BoxedParamProvider(qconfig.QuantizationProvider):
     self.quant_stats: dict[str, Any] = {}
 
   # -- helpers
-  def _prepare(self, lhs, rhs, rule, op_id, get_how):
+  def _prepare(self, lhs, rhs, rule, op_id, get_how, quantize_lhs: bool = True):
     if isinstance(rhs, WithAux):
       rhs = rhs.array
     elif isinstance(rhs, Param):
@@ -116,10 +116,17 @@ class BoxedParamProvider(qconfig.QuantizationProvider):
     elif rule.act_qtype is not None:
       how = get_how(for_lhs=False, qtype=rule.act_qtype, calibration_method=rule.act_calibration_method or 'absmax')
       rhs = quantize_act(rhs, how, rule, op_id + '_rhs', quant_stats=self.quant_stats, _qarray_module=self._qarray_module)
-    if rule.act_qtype is not None:
+    if rule.act_qtype is not None and quantize_lhs:
       how = get_how(for_lhs=True, qtype=rule.act_qtype, calibration_method=rule.act_calibration_method or 'absmax')
       lhs = quantize_act(lhs, how, rule, op_id + '_lhs', quant_stats=self.quant_stats, _qarray_module=self._qarray_module)
     return lhs, rhs
+
+  def _fusable(self, rule) -> bool:
+    """Decode-size calls may fold the lhs quantization into the GEMM launch: only with the stock kernels,
+    dynamic per-token int8 absmax, and no sub-channel tiling."""
+    return (self._dot_general_fn is _dot_general.dot_general and self._qarray_module is _qarray
+            and rule.act_qtype is not None and str(rule.act_qtype).replace('torch.', '') == 'int8'
+            and not rule.act_static_scale and (rule.act_calibration_method or 'absmax') == 'absmax' and not rule.tile_size)
 
   @staticmethod
   def _unbox_float(x):
@@ -138,7 +145,15 @@ class BoxedParamProvider(qconfig.QuantizationProvider):
       return out if preferred_element_type is None else out.to(preferred_element_type)
     get_how = functools.partial(_dot_general.get_how_to_quantize, dimension_numbers=dimension_numbers,
                                 ndims=(len(lhs.shape), len(rhs.shape)), tile_size=rule.tile_size)
-    lhs, rhs = self._prepare(lhs, rhs, rule, op_id, get_how)
+    if self._fusable(rule) and isinstance(lhs, torch.Tensor) and lhs.numel() // max(lhs.shape[-1], 1) <= 32:
+      lhs, rhs = self._prepare(lhs, rhs, rule, op_id, get_how, quantize_lhs=False)
+      out = _dot_general.fused_act_dot_general(lhs, rhs, dimension_numbers)
+      if out is not None:
+        return out
+      how = get_how(for_lhs=True, qtype=rule.act_qtype, calibration_method='absmax')
+      lhs = quantize_act(lhs, how, rule, op_id + '_lhs', quant_stats=self.quant_stats, _qarray_module=self._qarray_module)
+    else:
+      lhs, rhs = self._prepare(lhs, rhs, rule, op_id, get_how)
     return self._dot_general_fn(lhs, rhs, dimension_numbers, out_sharding=out_sharding)
 
   def einsum(self, einsum_str: str, *operands, precision=None, preferred_element_type=None, out_sharding=None):

@@ -170,3 +170,29 @@ def test_ptq_mlp_forward_replays_from_a_hip_graph():
     graph.replay()
     torch.cuda.synchronize()
     assert torch.equal(static_out, eager), i
+
+
+def test_decode_size_calls_fold_the_activation_quantization_into_the_gemm(monkeypatch):
+  """Through the provider, a call with at most 32 tokens takes the fused kernel (one launch) and gives the bits
+  of the two-step route; more tokens, static scales or sub-channel tiles keep the two-step route."""
+  import qwix_amd
+  from qwix_amd import nn
+  from qwix_amd.core import dot_general as dg
+  model = nn.MLP(2048, 512)
+  g = torch.Generator().manual_seed(3)
+  params = model.init(g, 1024, torch.bfloat16, util.DEV)
+  rules = [qwix_amd.QuantizationRule(module_path='.*', weight_qtype='int8', act_qtype='int8')]
+  ptq_model = qwix_amd.quantize_model(model, qwix_amd.PtqProvider(rules))
+  x = torch.rand(8, 1024, generator=g, dtype=torch.float32).to(torch.bfloat16).to(util.DEV)
+  qparams = qwix_amd.quantize_params(params, ptq_model.init(params, x))
+  calls = []
+  real = dg.fused_act_dot_general
+  monkeypatch.setattr(dg, 'fused_act_dot_general', lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+  out = ptq_model.apply(qparams, x)
+  assert len(calls) == 2
+  monkeypatch.setattr(dg, 'fused_act_dot_general', lambda *a, **k: None)   # force the two-step route
+  assert torch.equal(out, ptq_model.apply(qparams, x))
+  monkeypatch.setattr(dg, 'fused_act_dot_general', lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+  big = torch.rand(64, 1024, generator=g, dtype=torch.float32).to(torch.bfloat16).to(util.DEV)
+  ptq_model.apply(qparams, big)
+  assert len(calls) == 2                                                   # 64 tokens: not offered to the fused kernel

@@ -154,3 +154,30 @@ def test_both_operands_asymmetric_is_an_error():
   wq = qarray.quantize(w_t, qarray.HowToQuantize(qtype='int8', channelwise_axes=[1], calibration_method='minmax'))
   with pytest.raises(ValueError, match='Only one operand can be asymmetric'):
     dg.dot_general(xq, wq, DN)
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('M,K,N', [(1, 2048, 1024), (5, 128, 48), (16, 1024, 520), (17, 2048, 300), (32, 1536, 14336), (8, 640, 264)])
+def test_fused_activation_quantize_gemm_bit_exact(M, K, N, dtype):
+  """Activation quantization folded into the decode GEMM == quantize, then dot_general (the oracle's two steps)."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  print('case fused act', M, K, N, dtype, flush=True)
+  x_np, x_t = util.make((M, K), dtype, seed=M + K)
+  x_np[0, :] *= 0 if M > 4 else 1          # an all-zero row takes the scale guard
+  x_t = util.to_gpu(x_np, dtype)
+  w_np, w_t = util.make((K, N), dtype, seed=N, scale=0.02)
+  wq = qarray.quantize(w_t, qarray.HowToQuantize(qtype='int8', channelwise_axes=[1]))
+  out = dg.fused_act_dot_general(x_t, wq, DN)
+  assert out is not None and out.dtype == util.TORCH_DT[dtype]
+  torch.cuda.synchronize()
+  oxq = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(qtype='int8', channelwise_axes=[0]))
+  owq = O.quantize(O.FArr(w_np, dtype), O.HowToQuantize(qtype='int8', channelwise_axes=[1]))
+  want = O.fast_dot_general(oxq, owq, DN)
+  got = util.f32np(out)
+  bad = np.flatnonzero(got.ravel() != want.v.ravel())
+  assert bad.size == 0, f'{bad.size} outputs differ: {got.ravel()[bad[:5]]} vs {want.v.ravel()[bad[:5]]}'
+  # shapes the kernel does not take are handed back to the two-step route
+  assert dg.fused_act_dot_general(torch.zeros(40, K, device=util.DEV), wq, DN) is None
+  w4 = qarray.quantize(torch.zeros(4096, 64, device=util.DEV), qarray.HowToQuantize(qtype='int8', channelwise_axes=[1]))
+  assert dg.fused_act_dot_general(torch.zeros(8, 4096, device=util.DEV), w4, DN) is None   # K too long
