@@ -590,6 +590,47 @@ class QuantizeStatic(Workload):
     return {'workload': self.name, 'M': self.M, 'K': self.K, 'scale': 'per-tensor, precomputed'}
 
 
+class QuantizeBlocks(Workload):
+  """PTQ of a (K, N) weight with one scale per 128 x 128 block (tiles on both axes), natural layout."""
+
+  bound = 'hbm'
+
+  def __init__(self, name, K, N, qtype, block=128):
+    self.name, self.K, self.N, self.qtype, self.block = name, K, N, qtype, block
+    self.dtype = 'bf16->' + qtype
+    self.metric = 'weight quantize GB/s (absmax per %dx%d block, bf16 -> %s)' % (block, block, qtype)
+    self.unit = 'GB/s'
+    self.kernel_name = 'blocks_kernel'
+
+  def setup(self, dev):
+    import ctypes
+    import torch
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(13)
+    self.w = (torch.randn(self.K, self.N, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(dev)
+    self.q = torch.empty(self.K, self.N, dtype=torch.uint8, device=dev)
+    self.s = torch.empty(self.K // self.block, self.N // self.block, dtype=torch.bfloat16, device=dev)
+    self.qt = {'int8': L.INT8, 'float8_e4m3fn': L.E4M3}[self.qtype]
+    self.dims = (ctypes.c_int64 * 5)(1, self.K, 1, self.N, 1)
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, i=0):
+    L = self.L
+    L.call('qwix_hip_quantize_generic', self.w.data_ptr(), L.BF16, self.dims, self.block, self.block, self.qt,
+           L.ABSMAX, 0.0, self.q.data_ptr(), self.s.data_ptr(), None, self.stream)
+
+  kernel = step
+
+  def work_per_step(self):
+    return self.K * self.N * 3.0 + self.s.numel() * 2.0
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'K': self.K, 'N': self.N, 'block': self.block, 'qtype': self.qtype}
+
+
 class QdotZeroPoint(QdotW8A8):
   """w8a8 with an asymmetric (minmax) int8 activation: quantize with zero point, K-sums of the weight rows,
   GEMM with the zero-point correction in the epilogue."""
@@ -750,6 +791,7 @@ WORKLOADS = {
     'moe_ragged_int8_8x1024': lambda: RaggedQdot('moe_ragged_int8_8x1024', 8192, 4096, 14336, 8),
     'moe_ragged_int8_64x128': lambda: RaggedQdot('moe_ragged_int8_64x128', 8192, 2048, 4096, 64),
     'moe_ragged_fp8_8x1024': lambda: RaggedQdot('moe_ragged_fp8_8x1024', 8192, 4096, 14336, 8, 'float8_e4m3fn'),
+    'quantize_weight_fp8_block128': lambda: QuantizeBlocks('quantize_weight_fp8_block128', 4096, 14336, 'float8_e4m3fn'),
     'srq_quantize_act_4096': lambda: QuantizeStatic('srq_quantize_act_4096', 4096, 4096),
     'zp_int8_w8a8_4096': lambda: QdotZeroPoint('zp_int8_w8a8_4096', 4096, 4096, 4096),
     'batched_qk_int8_32x2048': lambda: QdotBatched('batched_qk_int8_32x2048', 32, 2048, 2048, 128),
@@ -759,7 +801,7 @@ WORKLOADS = {
 DEFAULT = 'c3_int8_w8a8_4096'
 EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
          'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'moe_ragged_int8_8x1024',
-         'moe_ragged_int8_64x128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
+         'moe_ragged_int8_64x128', 'quantize_weight_fp8_block128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 
 
 def _blas_threads() -> int:

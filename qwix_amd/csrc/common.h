@@ -58,6 +58,13 @@ __device__ __forceinline__ float round_bf16(float x) {
   return bf16_bits_to_f32(f32_to_bf16_bits(x));
 }
 
+// Two values at once: one convert for the pair.
+__device__ __forceinline__ void round_bf16_pair(float& a, float& b) {
+  const uint32_t w = pack_bf16x2(a, b);
+  a = __uint_as_float(w << 16);
+  b = __uint_as_float(w & 0xFFFF0000u);
+}
+
 template <typename D>
 __device__ __forceinline__ float rnd(float x) {
   if constexpr (D::kTag == QWIX_BF16) return round_bf16(x);
@@ -134,6 +141,12 @@ __device__ __forceinline__ uint32_t to_e4m3x2(float a, float b) {
   b = b > 448.f ? 448.f : (b < -448.f ? -448.f : b);
   return static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false)) & 0xFFFFu;
 }
+// The same for values that are not NaN: the clip is one v_med3 per value.
+__device__ __forceinline__ uint32_t to_e4m3x2_bounded(float a, float b) {
+  a = __builtin_amdgcn_fmed3f(a, -448.f, 448.f);
+  b = __builtin_amdgcn_fmed3f(b, -448.f, 448.f);
+  return static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false)) & 0xFFFFu;
+}
 __device__ __forceinline__ float e4m3_to_f32(uint32_t byte) {
   return __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(byte), 0);
 }
@@ -170,6 +183,37 @@ struct Divider {
   float s, r;
   __device__ __forceinline__ explicit Divider(float scale) : s(scale) {
     if constexpr (D::kTag == QWIX_BF16) r = __builtin_amdgcn_rcpf(scale);
+  }
+  // The quotient before its rounding to D (f32: the quotient itself).
+  __device__ __forceinline__ float raw(float x) const {
+    if constexpr (D::kTag == QWIX_BF16) {
+      float q0 = x * r;
+      float e = __builtin_fmaf(-q0, s, x);
+      float q1 = __builtin_fmaf(e, r, q0);
+      if constexpr (kSafe) {
+        const bool odd = !(__builtin_fabsf(q0) < 0x1p100f);
+        if (__builtin_amdgcn_ballot_w64(odd) != 0) {
+          if (odd) q1 = x / s;
+        }
+      }
+      return q1;
+    } else {
+      return x / s;
+    }
+  }
+  // Divides a pair; the bf16 rounding of both is one convert.  Zero quotients come out as +0.
+  __device__ __forceinline__ void pair_unsigned(float& a, float& b) const {
+    a = raw(a);
+    b = raw(b);
+    if constexpr (D::kTag == QWIX_BF16) round_bf16_pair(a, b);
+  }
+  __device__ __forceinline__ void pair(float& a, float& b) const {
+    const float xa = a, xb = b;
+    pair_unsigned(a, b);
+    if constexpr (kSignedZero && D::kTag == QWIX_BF16) {
+      a = __builtin_copysignf(a, xa);
+      b = __builtin_copysignf(b, xb);
+    }
   }
   __device__ __forceinline__ float operator()(float x) const {
     if constexpr (D::kTag == QWIX_BF16) {

@@ -24,7 +24,7 @@ enum { MODE_QUANT = 0, MODE_CALIB = 1, MODE_GIVEN = 2 };
 // Quantize N consecutive values (already divided / shifted) and store them packed.  BOUNDED selects
 // the two-op clamp-and-round converter (vector paths); the scalar paths keep NaN -> 0.
 template <int QT, int N, bool BOUNDED = false>
-__device__ __forceinline__ void store_q(const float* v, uint8_t* q, int64_t elem) {
+__device__ __forceinline__ void store_q(const float* v, uint8_t* q, int64_t elem, const uint32_t* bf16_signs = nullptr) {
   if constexpr (QT == QWIX_INT8) {
     uint32_t w[N / 4];
 #pragma unroll
@@ -43,8 +43,17 @@ __device__ __forceinline__ void store_q(const float* v, uint8_t* q, int64_t elem
   } else if constexpr (QT == QWIX_E4M3) {
     uint32_t w[N / 4];
 #pragma unroll
-    for (int i = 0; i < N / 4; ++i)
-      w[i] = to_e4m3x2(v[4 * i], v[4 * i + 1]) | (to_e4m3x2(v[4 * i + 2], v[4 * i + 3]) << 16);
+    for (int i = 0; i < N / 4; ++i) {
+      if constexpr (BOUNDED)
+        w[i] = to_e4m3x2_bounded(v[4 * i], v[4 * i + 1]) | (to_e4m3x2_bounded(v[4 * i + 2], v[4 * i + 3]) << 16);
+      else
+        w[i] = to_e4m3x2(v[4 * i], v[4 * i + 1]) | (to_e4m3x2(v[4 * i + 2], v[4 * i + 3]) << 16);
+      // bf16_signs: the packed bf16 words the values were divided from (two per output word).  A quotient
+      // carries the sign of its dividend, zero quotients included: take the four sign bits from there.
+      if (bf16_signs != nullptr)
+        w[i] = (__builtin_amdgcn_perm(bf16_signs[2 * i + 1], bf16_signs[2 * i], 0x07050301u) & 0x80808080u) |
+               (w[i] & 0x7F7F7F7Fu);
+    }
     if constexpr (N == 8)
       *reinterpret_cast<uint2*>(q + elem) = make_uint2(w[0], w[1]);
     else
@@ -185,8 +194,10 @@ __global__ void __launch_bounds__(256)
   }
 
   const float zf = static_cast<float>(z);
+  // With a given scale a NaN input must stay NaN in e4m3; the one-op clip does not keep it.
+  constexpr bool kBounded = !(MODE == MODE_GIVEN && QT == QWIX_E4M3);
   auto quantize_all = [&](auto safe_tag) {
-    const Divider<D, decltype(safe_tag)::value, QT == QWIX_E4M3> div(s);
+    const Divider<D, decltype(safe_tag)::value, false> div(s);  // the sign of a zero quotient is restored below
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
       const int v = lane + (j << log2g);
@@ -194,11 +205,20 @@ __global__ void __launch_bounds__(256)
         float t[EV];
         unpack16<D>(raw[j], t);
 #pragma unroll
-        for (int e = 0; e < EV; ++e) {
-          t[e] = div(t[e]);
-          if constexpr (ASYM) t[e] = rnd<D>(t[e] + zf);
+        for (int e = 0; e < EV; e += 2) {
+          div.pair_unsigned(t[e], t[e + 1]);
+          if constexpr (ASYM) {
+            t[e] += zf;
+            t[e + 1] += zf;
+            if constexpr (D::kTag == QWIX_BF16) round_bf16_pair(t[e], t[e + 1]);
+          }
         }
-        store_q<QT, EV, true>(t, q, (seg * nvec + v) * EV);
+        if constexpr (QT == QWIX_E4M3 && D::kTag == QWIX_BF16) {
+          const uint32_t signs[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+          store_q<QT, EV, kBounded>(t, q, (seg * nvec + v) * EV, signs);
+        } else {
+          store_q<QT, EV, kBounded>(t, q, (seg * nvec + v) * EV);
+        }
       }
     }
   };
@@ -566,12 +586,16 @@ __global__ void __launch_bounds__(256)
     const Divider<D, SRC == 1, QT == QWIX_E4M3> div(s[e]);
     const float zf = static_cast<float>(z[e]);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      v[j][e] = div(v[j][e]);
-      if constexpr (ASYM) v[j][e] = rnd<D>(v[j][e] + zf);
+    for (int j = 0; j < 8; j += 2) {
+      div.pair(v[j][e], v[j + 1][e]);
+      if constexpr (ASYM) {
+        v[j][e] += zf;
+        v[j + 1][e] += zf;
+        if constexpr (D::kTag == QWIX_BF16) round_bf16_pair(v[j][e], v[j + 1][e]);
+      }
     }
   }
-  constexpr bool kBounded = true;
+  constexpr bool kBounded = !(SRC == 1 && QT == QWIX_E4M3);  // a given scale: NaN inputs stay NaN in e4m3
   if constexpr (LAYOUT == QWIX_LAYOUT_NATURAL) {
 #pragma unroll
     for (int j = 0; j < 8; ++j)
@@ -687,6 +711,139 @@ __global__ void generic_quant_kernel(const void* __restrict__ x, Geom5 g, const 
     q[bi] = static_cast<uint8_t>(pack2_i4(to_int_q<QT>(t[0]), to_int_q<QT>(t[1])));
   else
     q[bi] = q_byte<QT>(t[0]);
+}
+
+// ------------------------------------------------------------------------------------ 2-D blocks
+// Scale groups that are t1 x t3 blocks of a matrix whose rows are `row_stride` elements apart (the 5-D
+// geometry with d4 == 1): 2^log2g threads hold one block in registers, read row piece by row piece with
+// 16-byte loads, so the array is read once and written once like the contiguous-segment kernel does.
+struct BlockGeom {
+  int64_t nblk;        // d0 * n1 * d2 * n3 = number of scales
+  int64_t row_stride;  // d2 * r3 elements between consecutive rows of a block
+  int64_t r1, r3;
+  uint32_t n1, d2, n3; // blocks along r1, middle kept axis, blocks along r3
+  uint32_t t1, t3;
+  uint32_t vpr;        // 16-byte vectors per block row
+  uint32_t vpr_magic;  // ceil(2^32 / vpr): v / vpr == (v * magic) >> 32 for v, vpr < 2^16 (unused when vpr == 1)
+  int nvec, log2g;
+};
+
+template <typename D, int QT, int CAL, int NL>
+__global__ void __launch_bounds__(256)
+    blocks_kernel(const uint8_t* __restrict__ x, BlockGeom gm, float factor, uint8_t* __restrict__ q,
+                  void* __restrict__ scale, int8_t* __restrict__ zp) {
+  constexpr int EV = D::kVec;
+  constexpr bool ASYM = (CAL == QWIX_MINMAX);
+  __shared__ float red[2][4];
+  const int tid = threadIdx.x;
+  const int log2g = gm.log2g, g = 1 << log2g;
+  const int64_t blk = (static_cast<int64_t>(blockIdx.x) << (8 - log2g)) + (tid >> log2g);
+  const int lane = tid & (g - 1);
+  const bool blk_ok = blk < gm.nblk;
+  int64_t base = 0;  // first element of the block
+  if (blk_ok) {
+    const uint32_t b = static_cast<uint32_t>(blk);
+    const uint32_t j3 = b % gm.n3, r = b / gm.n3;
+    const uint32_t i2 = r % gm.d2, r2 = r / gm.d2;
+    const uint32_t j1 = r2 % gm.n1, i0 = r2 / gm.n1;
+    base = ((static_cast<int64_t>(i0) * gm.r1 + static_cast<int64_t>(j1) * gm.t1) * gm.d2 + i2) * gm.r3 +
+           static_cast<int64_t>(j3) * gm.t3;
+  }
+  int64_t off[NL];  // element offset of each vector this thread owns
+  uint4 raw[NL];
+#pragma unroll
+  for (int j = 0; j < NL; ++j) {
+    const uint32_t v = lane + (j << log2g);
+    const uint32_t row = gm.vpr == 1 ? v : static_cast<uint32_t>((static_cast<uint64_t>(v) * gm.vpr_magic) >> 32);
+    off[j] = base + static_cast<int64_t>(row) * gm.row_stride + static_cast<int64_t>(v - row * gm.vpr) * EV;
+    raw[j] = make_uint4(0, 0, 0, 0);
+    if (blk_ok && static_cast<int>(v) < gm.nvec)
+      raw[j] = *reinterpret_cast<const uint4*>(x + off[j] * sizeof(typename D::storage));
+  }
+#pragma unroll
+  for (int j = 0; j < NL; ++j) asm volatile("" : "+v"(raw[j].x), "+v"(raw[j].y), "+v"(raw[j].z), "+v"(raw[j].w));
+
+  float mx = 0.f, mn = 0.f;
+  if constexpr (!ASYM && D::kTag == QWIX_BF16) {
+    u16x2 m = {0, 0};
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+      const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2, w[e] & 0x7FFF7FFFu));
+    }
+    mx = bf16_bits_to_f32(m[0] > m[1] ? m[0] : m[1]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+      float f[EV];
+      unpack16<D>(raw[j], f);
+#pragma unroll
+      for (int e = 0; e < EV; ++e) {
+        if constexpr (ASYM) {
+          mx = fmaxf(mx, f[e]);
+          mn = fminf(mn, f[e]);
+        } else {
+          mx = absmax_acc(mx, f[e]);
+        }
+      }
+    }
+  }
+  mx = wave_xor_max(mx, g < 64 ? g : 64);
+  if constexpr (ASYM) mn = wave_xor_min(mn, g < 64 ? g : 64);
+  if (g > 64) {  // uniform branch: a block spans 2 or 4 wavefronts
+    const int w = tid >> 6;
+    if ((tid & 63) == 0) {
+      red[0][w] = mx;
+      red[1][w] = mn;
+    }
+    __syncthreads();
+    const int w0 = (tid >> log2g) << (log2g - 6), nw = 1 << (log2g - 6);
+    mx = red[0][w0];
+    mn = red[1][w0];
+    for (int i = 1; i < nw; ++i) {
+      mx = fmaxf(mx, red[0][w0 + i]);
+      mn = fminf(mn, red[1][w0 + i]);
+    }
+  }
+  mx = apply_factor<D>(mx, factor);
+  float s;
+  int z = 0;
+  if constexpr (ASYM) {
+    mn = apply_factor<D>(mn, factor);
+    s = asym_scale_zp<D, QT>(mn, mx, &z);
+  } else {
+    s = sym_scale<D, QT>(mx);
+  }
+  if (blk_ok && lane == 0) {
+    store1<D>(scale, blk, s);
+    if constexpr (ASYM) zp[blk] = static_cast<int8_t>(z);
+  }
+  const float zf = static_cast<float>(z);
+  const Divider<D, false, false> div(s);  // the sign of a zero quotient is restored below
+#pragma unroll
+  for (int j = 0; j < NL; ++j) {
+    const int v = lane + (j << log2g);
+    if (blk_ok && v < gm.nvec) {
+      float t[EV];
+      unpack16<D>(raw[j], t);
+#pragma unroll
+      for (int e = 0; e < EV; e += 2) {
+        div.pair_unsigned(t[e], t[e + 1]);
+        if constexpr (ASYM) {
+          t[e] += zf;
+          t[e + 1] += zf;
+          if constexpr (D::kTag == QWIX_BF16) round_bf16_pair(t[e], t[e + 1]);
+        }
+      }
+      if constexpr (QT == QWIX_E4M3 && D::kTag == QWIX_BF16) {
+        const uint32_t signs[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+        store_q<QT, EV, true>(t, q, off[j], signs);
+      } else {
+        store_q<QT, EV, true>(t, q, off[j]);
+      }
+    }
+  }
 }
 
 // ------------------------------------------------------------------------------------ misc
@@ -1182,6 +1339,45 @@ int qwix_hip_quantize_generic(const void* x, int dtype, const int64_t dims[5], i
   const int64_t ns = dims[0] * (dims[1] / t1) * dims[2] * (dims[3] / t3) * dims[4];
   const int64_t nb = qtype == QWIX_INT4 ? n / 2 : n;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  {  // blocks of 16-byte row pieces that fit one workgroup's registers: the single-pass kernel
+    const int ev = dtype == QWIX_BF16 ? 8 : 4;
+    const int64_t nvec = t3 % ev == 0 ? t1 * (t3 / ev) : 0;
+    if (dims[4] == 1 && nvec >= 2 && nvec <= 256 * 16 && aligned16(x) && (reinterpret_cast<uintptr_t>(qvalue) & 7) == 0 &&
+        ns <= 0xFFFFFFFFll && (dtype == QWIX_F32 || dtype == QWIX_BF16)) {
+      BlockGeom bg;
+      bg.nblk = ns;
+      bg.row_stride = dims[2] * dims[3];
+      bg.r1 = dims[1];
+      bg.r3 = dims[3];
+      bg.n1 = static_cast<uint32_t>(dims[1] / t1);
+      bg.d2 = static_cast<uint32_t>(dims[2]);
+      bg.n3 = static_cast<uint32_t>(dims[3] / t3);
+      bg.t1 = static_cast<uint32_t>(t1);
+      bg.t3 = static_cast<uint32_t>(t3);
+      bg.vpr = static_cast<uint32_t>(t3 / ev);
+      bg.vpr_magic = bg.vpr == 1 ? 0u : static_cast<uint32_t>(((uint64_t{1} << 32) + bg.vpr - 1) / bg.vpr);
+      bg.nvec = static_cast<int>(nvec);
+      int lg = log2_ceil((nvec + 3) / 4);  // aim at 4 loads per thread, as many as 16 for the largest blocks
+      if (lg > 8) lg = 8;
+      bg.log2g = lg;
+      const int loads = static_cast<int>((nvec + (1 << lg) - 1) >> lg);
+      const dim3 grid(static_cast<unsigned>((ns + (256 >> lg) - 1) / (256 >> lg)));
+      const uint8_t* xb = static_cast<const uint8_t*>(x);
+      uint8_t* qb = static_cast<uint8_t*>(qvalue);
+      int8_t* zb = static_cast<int8_t*>(zero_point);
+      QWIX_DISPATCH_D(dtype, {
+        QWIX_DISPATCH_QT_CAL(qtype, calibration, {
+          if (loads <= 4)
+            blocks_kernel<D, QT, CAL, 4><<<grid, 256, 0, st>>>(xb, bg, calib_factor, qb, scale, zb);
+          else if (loads <= 8)
+            blocks_kernel<D, QT, CAL, 8><<<grid, 256, 0, st>>>(xb, bg, calib_factor, qb, scale, zb);
+          else
+            blocks_kernel<D, QT, CAL, 16><<<grid, 256, 0, st>>>(xb, bg, calib_factor, qb, scale, zb);
+        })
+      })
+      return check_launch("block quantize");
+    }
+  }
   QWIX_DISPATCH_D(dtype, {
     QWIX_DISPATCH_QT_CAL(qtype, calibration, {
       generic_scale_kernel<D, QT, CAL><<<dim3(static_cast<unsigned>((ns + 255) / 256)), 256, 0, st>>>(

@@ -128,3 +128,37 @@ def test_activation_quantize_at_8192_square():
       assert torch.equal(q.qvalue.float(), torch.clamp(torch.round(quot), -128, 127))
     else:
       assert torch.equal(q.qvalue.float(), torch.clamp(quot, -448, 448).to(torch.float8_e4m3fn).float())
+
+
+def test_weight_quantize_at_ffn_size_in_column_strips():
+  """Per-channel (reduction along the strided axis) e4m3 / int8 quantize of an (8192, 28672) bf16 weight, which
+  is larger than the memory-side cache and therefore taken in strips of columns; checked by torch arithmetic."""
+  from qwix_amd.core import qarray
+  g = torch.Generator(device='cpu').manual_seed(12)
+  w = (torch.randn(8192, 28672, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(util.DEV)
+  w *= torch.linspace(0.5, 2.0, 28672, device=util.DEV).to(torch.bfloat16)  # a scale in the wrong column shows
+  for qtype, qmax, layout in (('float8_e4m3fn', 448.0, None), ('int8', 127.5, 'natural')):
+    q = qarray.quantize(w, qarray.HowToQuantize(qtype=qtype, channelwise_axes=[1]), layout=layout)
+    want_scale = (w.abs().amax(dim=0, keepdim=True).float() / qmax).to(torch.bfloat16)
+    assert torch.equal(q.scale, want_scale), qtype
+    quot = (w.float() / q.scale.float()).to(torch.bfloat16).float()
+    if qtype == 'int8':
+      assert torch.equal(q.qvalue.float(), torch.clamp(torch.round(quot), -128, 127))
+    else:
+      assert torch.equal(q.qvalue.float(), torch.clamp(quot, -448, 448).to(torch.float8_e4m3fn).float())
+    del q, quot
+
+
+def test_block_quantize_at_ffn_size():
+  """One e4m3 scale per 128 x 128 block of a (4096, 14336) bf16 weight, checked by torch arithmetic."""
+  from qwix_amd.core import qarray
+  g = torch.Generator(device='cpu').manual_seed(13)
+  w = (torch.randn(4096, 14336, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(util.DEV)
+  w *= torch.linspace(0.5, 2.0, 14336, device=util.DEV).to(torch.bfloat16)
+  q = qarray.quantize(w, qarray.HowToQuantize(qtype='float8_e4m3fn', tiled_axes={0: 128, 1: 128}))
+  blocks = w.reshape(32, 128, 112, 128)
+  want_scale = (blocks.abs().amax(dim=(1, 3)).float() / 448.0).to(torch.bfloat16)
+  assert torch.equal(q.scale, want_scale)
+  s = q.scale.float().repeat_interleave(128, 0).repeat_interleave(128, 1)
+  quot = (w.float() / s).to(torch.bfloat16).float()
+  assert torch.equal(q.qvalue.float(), torch.clamp(quot, -448, 448).to(torch.float8_e4m3fn).float())

@@ -116,6 +116,34 @@ def test_2d_tiles_generic():
   _check(x_np, x_t, O.F32, dict(qtype='int4'), what='per tensor')
 
 
+@pytest.mark.parametrize('qtype', QTYPES)
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('shape,tiles', [
+    ((256, 384), {0: 128, 1: 128}),          # block-scaled weight, 16 loads per thread for f32
+    ((96, 160), {0: 32, 1: 32}),
+    ((64, 80), {0: 8, 1: 16}),               # several blocks per wavefront
+    ((64, 64), {0: 16, 1: 8}),               # one 16-byte vector per block row (bf16)
+    ((192, 96), {0: 96, 1: 48}),             # block row pieces that are not a power of two
+    ((3, 128, 256), {1: 64, 2: 128}),        # a stack of matrices (experts)
+    ((64, 3, 128), {0: 32, 2: 64}),          # a kept axis between the two tiled ones
+    ((512, 128), {0: 256, 1: 128}),          # the largest block the single-pass kernel holds (bf16)
+    ((40, 24), {0: 8, 1: 12}),               # row pieces shorter than a 16-byte vector: the scalar kernels
+])
+def test_2d_blocks(shape, tiles, dtype, qtype):
+  x_np, x_t = util.make(shape, dtype, seed=61, scale=0.05)
+  # different magnitudes per block, so that a scale written to the wrong block shows
+  ramp = np.linspace(0.25, 4.0, int(np.prod(shape)), dtype=np.float32).reshape(shape)
+  x_np = x_np * ramp if dtype == O.F32 else O.round_to_bf16(x_np * ramp)
+  x_t = torch.from_numpy(x_np).to(util.TORCH_DT[dtype]).to(util.DEV)
+  cw = [a for a in range(len(shape)) if a not in tiles]
+  _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=cw, tiled_axes=tiles), what='2d blocks')
+  if qtype != 'float8_e4m3fn':
+    x_np = x_np + np.float32(0.03) if dtype == O.F32 else O.round_to_bf16(x_np + np.float32(0.03))
+    x_t = torch.from_numpy(x_np).to(util.TORCH_DT[dtype]).to(util.DEV)
+    _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=cw, tiled_axes=tiles, calibration_method='minmax'),
+           what='2d blocks minmax')
+
+
 def test_zero_rows_and_reference_convert_vectors():
   from qwix_amd.core import qarray
   x = torch.zeros(4, 256, dtype=torch.bfloat16, device=util.DEV)
