@@ -406,6 +406,92 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// The same reduction for tall scale groups (tile >= 256 rows): a workgroup covers 256 rows x 64 vectors of
+// columns, each wavefront reading whole 1 KiB row pieces, and issues one atomic per column for 256 rows
+// instead of one for 128.
+constexpr int kWideRows = 256;
+template <typename D, int CAL>
+__global__ void __launch_bounds__(256)
+    cols_absmax_wide_kernel(const uint8_t* __restrict__ x, ColGeom gm, int wide_col_blocks, int wide_chunks,
+                            uint32_t* __restrict__ ws) {
+  constexpr int EV = D::kVec;
+  constexpr bool ASYM = (CAL == QWIX_MINMAX);
+  constexpr bool PACKED = !ASYM && D::kTag == QWIX_BF16;  // |x| of a bf16 pair orders like its low 15 bits
+  __shared__ float red[ASYM ? 2 : 1][4][EV][64];
+  int64_t b = blockIdx.x;
+  const int64_t cb = b % wide_col_blocks;
+  b /= wide_col_blocks;
+  const int chunk = static_cast<int>(b % wide_chunks);
+  b /= wide_chunks;
+  const int64_t t = b % gm.ntiles, o = b / gm.ntiles;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int64_t c0 = (cb * 64 + lane) * EV;
+  const bool col_ok = c0 < gm.inner;
+  const int64_t row_end = (t + 1) * gm.tile;
+  const int64_t row0 = t * gm.tile + static_cast<int64_t>(chunk) * kWideRows + w;  // rows row0 + 4 * i
+  float mx[EV], mn[EV];
+  u16x2 pm[4] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}};
+#pragma unroll
+  for (int e = 0; e < EV; ++e) mx[e] = mn[e] = 0.f;
+  const uint8_t* xp = x + ((o * gm.reduce + row0) * gm.inner + c0) * sizeof(typename D::storage);
+  const int64_t step = 4 * gm.inner * sizeof(typename D::storage);
+  for (int it = 0; it < kWideRows / 32; ++it) {
+    uint4 raw[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      raw[j] = make_uint4(0, 0, 0, 0);
+      if (col_ok && row0 + 4 * (it * 8 + j) < row_end) raw[j] = *reinterpret_cast<const uint4*>(xp + (it * 8 + j) * step);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if constexpr (PACKED) {
+        const uint32_t wd[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          pm[k] = __builtin_elementwise_max(pm[k], __builtin_bit_cast(u16x2, wd[k] & 0x7FFF7FFFu));
+      } else {
+        float f[EV];
+        unpack16<D>(raw[j], f);
+#pragma unroll
+        for (int e = 0; e < EV; ++e) {
+          if constexpr (ASYM) {
+            mx[e] = fmaxf(mx[e], f[e]);
+            mn[e] = fminf(mn[e], f[e]);
+          } else {
+            mx[e] = absmax_acc(mx[e], f[e]);
+          }
+        }
+      }
+    }
+  }
+  if constexpr (PACKED) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      mx[2 * k] = bf16_bits_to_f32(pm[k][0]);
+      mx[2 * k + 1] = bf16_bits_to_f32(pm[k][1]);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < EV; ++e) {
+    red[0][w][e][lane] = mx[e];
+    if constexpr (ASYM) red[1][w][e][lane] = mn[e];
+  }
+  __syncthreads();
+  // 64 * EV columns, 256 threads
+  const int64_t wbase = (o * gm.ntiles + t) * gm.inner + cb * 64 * EV;
+  const int64_t plane = gm.outer * gm.ntiles * gm.inner;
+  for (int c = tid; c < 64 * EV; c += 256) {
+    if (cb * 64 * EV + c >= gm.inner) break;
+    const int l = c / EV, e = c % EV;
+    const float a = fmaxf(fmaxf(red[0][0][e][l], red[0][1][e][l]), fmaxf(red[0][2][e][l], red[0][3][e][l]));
+    atomicMax(ws + wbase + c, __float_as_uint(a));  // a >= 0: bit patterns order like values
+    if constexpr (ASYM) {
+      const float m = fminf(fminf(red[1][0][e][l], red[1][1][e][l]), fminf(red[1][2][e][l], red[1][3][e][l]));
+      atomicMax(ws + plane + wbase + c, __float_as_uint(-m));
+    }
+  }
+}
+
 // Long segments are calibrated in pieces (rows_kernel in calibration mode, one partial per piece); this
 // kernel merges the `pieces` partials of a segment (one wavefront per segment) and either writes the
 // calibration values (MODE_CALIB) or turns them into scale / zero point (MODE_QUANT).  The partials
@@ -491,18 +577,17 @@ __global__ void __launch_bounds__(256)
   const int64_t row_end = (t + 1) * gm.tile;
   const int64_t r0 = t * gm.tile + chunk * 128 + rb * 8;
   float v[8][EV];
+  uint4 raw[8];
+  // The loads are issued before the scales are fetched, so that the two round trips overlap.
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    raw[j] = make_uint4(0, 0, 0, 0);
+    if (col_ok && r0 + j < row_end)
+      raw[j] = *reinterpret_cast<const uint4*>(x + ((o * gm.reduce + r0 + j) * gm.inner + c0) * sizeof(typename D::storage));
+  }
   auto load_rows = [&]() {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      if (col_ok && r0 + j < row_end) {
-        unpack16<D>(*reinterpret_cast<const uint4*>(
-                        x + ((o * gm.reduce + r0 + j) * gm.inner + c0) * sizeof(typename D::storage)),
-                    v[j]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < EV; ++e) v[j][e] = 0.f;
-      }
-    }
+    for (int j = 0; j < 8; ++j) unpack16<D>(raw[j], v[j]);
   };
   float s[EV];
   int z[EV];
@@ -1171,6 +1256,23 @@ int run_rows(const void* x, int dtype, int64_t nseg, int64_t L, int qtype, int c
 int run_cols_absmax(const void* x, int dtype, const ColGeom& g, int cal, uint32_t* ws, hipStream_t st) {
   const int64_t n = g.outer * g.ntiles * g.inner * (cal == QWIX_MINMAX ? 2 : 1);
   fill_u32_kernel<<<dim3(static_cast<unsigned>((n + 255) / 256)), 256, 0, st>>>(ws, n, 0u);
+  if (g.tile >= kWideRows) {
+    const int ev = dtype == QWIX_BF16 ? 8 : 4;
+    const int wcb = static_cast<int>((g.inner + 64 * ev - 1) / (64 * ev));
+    const int wch = static_cast<int>((g.tile + kWideRows - 1) / kWideRows);
+    const int64_t wblocks = g.outer * g.ntiles * wch * wcb;
+    if (wblocks <= INT32_MAX) {
+      QWIX_DISPATCH_D(dtype, {
+        if (cal == QWIX_MINMAX)
+          cols_absmax_wide_kernel<D, QWIX_MINMAX><<<dim3(static_cast<unsigned>(wblocks)), 256, 0, st>>>(
+              static_cast<const uint8_t*>(x), g, wcb, wch, ws);
+        else
+          cols_absmax_wide_kernel<D, QWIX_ABSMAX><<<dim3(static_cast<unsigned>(wblocks)), 256, 0, st>>>(
+              static_cast<const uint8_t*>(x), g, wcb, wch, ws);
+      })
+      return check_launch("cols absmax");
+    }
+  }
   const int64_t blocks = g.outer * g.ntiles * g.chunks_per_tile * g.col_blocks;
   QWIX_DISPATCH_D(dtype, {
     if (cal == QWIX_MINMAX)

@@ -93,6 +93,12 @@ def test_minmax(dtype, qtype):
   _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=[0], calibration_method='minmax'), what='minmax rows')
   _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=[1], calibration_method='minmax'), what='minmax cols')
   _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=[0], calibration_method='absmax,0.8'), what='absmax factor')
+  # tall groups: the strided reduction in 256-row pieces
+  x_np, x_t = util.make((600, 96), dtype, seed=42)
+  x_np = x_np + np.float32(0.25) if dtype == O.F32 else O.round_to_bf16(x_np + np.float32(0.25))
+  x_t = torch.from_numpy(x_np).to(util.TORCH_DT[dtype]).to(util.DEV)
+  _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=[1], calibration_method='minmax'), what='minmax tall cols')
+  _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=[1], tiled_axes={0: 300}), what='absmax tall cols, 2 groups')
 
 
 def test_reference_exact_minmax_vector():
