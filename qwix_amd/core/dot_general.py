@@ -455,6 +455,22 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   return out.to(res_t)
 
 
+def _degenerate(lhs, rhs, dimension_numbers, preferred_element_type):
+  """The result when an operand has no elements (nothing to launch): an empty array, or zeros when only
+  the contracted axes are empty -- what lax.dot_general returns for such shapes.  None otherwise."""
+  ls, rs = tuple(lhs.shape), tuple(rhs.shape)
+  if math.prod(ls) and math.prod(rs):
+    return None
+  (lc, rc), (lb, rb) = dimension_numbers
+  if [ls[a] for a in lc] != [rs[a] for a in rc] or [ls[a] for a in lb] != [rs[a] for a in rb]:
+    raise TypeError(f'dot_general: contracting / batch sizes of {ls} and {rs} differ for {dimension_numbers}')
+  out = ([ls[a] for a in lb] + [d for a, d in enumerate(ls) if a not in lc and a not in lb] +
+         [d for a, d in enumerate(rs) if a not in rc and a not in rb])
+  _, res_t = qarray.get_accumulator_and_result_type(lhs, rhs, preferred_element_type=preferred_element_type)
+  dev = (lhs.scale if isinstance(lhs, qarray.QArray) else lhs).device
+  return torch.zeros(out, dtype=res_t, device=dev)
+
+
 def dot_general(lhs: MaybeQ, rhs: MaybeQ, dimension_numbers: DotDimensionNumbers, precision=None,
                 preferred_element_type=None, **kwargs) -> torch.Tensor:
   """Drop-in for lax.dot_general that accepts QArray operands.
@@ -464,6 +480,9 @@ def dot_general(lhs: MaybeQ, rhs: MaybeQ, dimension_numbers: DotDimensionNumbers
   values directly.  `precision` and extra keywords (e.g. out_sharding) are accepted and ignored.
   """
   del precision
+  empty = _degenerate(lhs, rhs, dimension_numbers, preferred_element_type)
+  if empty is not None:
+    return empty
   if _use_fast_path(lhs, rhs, dimension_numbers):
     return _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type, **kwargs)
   return _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type, **kwargs)

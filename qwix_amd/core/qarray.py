@@ -181,7 +181,7 @@ def validate_qarray(array: QArray) -> None:
   qs, ss = array.shape, tuple(array.scale.shape)
   if len(qs) != len(ss):
     raise ValueError(f'Scale {ss} should have the same rank as qvalue {qs}.')
-  if not all(a % b == 0 for a, b in zip(qs, ss)):
+  if not all((a % b == 0) if b else a == 0 for a, b in zip(qs, ss)):
     raise ValueError(f'Scale {ss} should be broadcastable to qvalue {qs}.')
   if not numerics.should_quantize(array.scale.dtype):
     raise ValueError(f'{array.scale.dtype} is not a valid type for scale.')
@@ -189,7 +189,7 @@ def validate_qarray(array: QArray) -> None:
     zs = tuple(array.zero_point.shape)
     if len(zs) != len(qs):
       raise ValueError(f'Zero point {zs} should have the same rank as qvalue {qs}.')
-    if not all(a % b == 0 for a, b in zip(qs, zs)):
+    if not all((a % b == 0) if b else a == 0 for a, b in zip(qs, zs)):
       raise ValueError(f'Zero point {zs} should be broadcastable to qvalue {qs}.')
     if array.zero_point.dtype != torch.int8:
       raise ValueError(f'Zero point {array.zero_point.dtype} should be int8 (the storage dtype of int8/int4).')
@@ -321,6 +321,22 @@ def _alloc_q(shape, qtype: str, plan: _Plan, layout: int, device):
   return data, data.permute(*inv)
 
 
+def _empty_qvalue(shape, qtype: str, device):
+  """A qvalue with no elements (nothing is launched for it)."""
+  if qtype == numerics.INT4:
+    if shape[-1] % 2:
+      raise NotImplementedError(f'int4 needs an even last dimension, got {tuple(shape)}')
+    data = torch.empty(*shape[:-1], shape[-1] // 2, dtype=torch.uint8, device=device)
+    return Int4Tensor(data, shape, len(shape) - 1)
+  return torch.empty(tuple(shape), dtype=numerics.storage_dtype(qtype), device=device)
+
+
+def _check_empty_reduction(sshape) -> None:
+  # jnp.max over an empty axis has no identity; an empty scale means there is nothing to reduce at all.
+  if math.prod(sshape):
+    raise ValueError('zero-size array to reduction operation max which has no identity')
+
+
 def _default_layout(plan: _Plan, layout: str | None) -> int:
   if layout is None:
     layout = 'reduce_minor' if (plan.kind == '3d' and plan.dims[2] > 1 and plan.dims[1] % 8 == 0 and plan.tiles[0] % 8 == 0) else 'natural'
@@ -340,6 +356,10 @@ def calibrate(array: torch.Tensor, how: HowToQuantize) -> dict[str, torch.Tensor
   shape = tuple(array.shape)
   sshape = get_scale_shape(shape, how)
   cal, factor = _parse_calibration(how.calibration_method)
+  if array.numel() == 0:
+    _check_empty_reduction(sshape)
+    outs = [torch.empty(sshape, dtype=array.dtype, device=array.device) for _ in range(2 if cal == _lib.MINMAX else 1)]
+    return {'min': outs[0], 'max': outs[1]} if cal == _lib.MINMAX else {'absmax': outs[0]}
   plan = _plan(shape, _tiles_from_how(shape, how))
   if plan.kind != '3d':
     raise NotImplementedError('calibrate() alone supports a single reduced axis group')
@@ -378,10 +398,12 @@ def quantize_with_scale_zero_point(array: torch.Tensor, qtype, scale: torch.Tens
   if zero_point is not None and tuple(zero_point.shape) != tuple(scale.shape):
     raise ValueError(f'Expect zero_point shape {tuple(scale.shape)} but got {tuple(zero_point.shape)}')
   shape = tuple(array.shape)
-  if len(shape) != scale.ndim or any(d % s for d, s in zip(shape, scale.shape)):
+  if len(shape) != scale.ndim or any((d % s) if s else d for d, s in zip(shape, scale.shape)):
     raise ValueError(f'Cannot broadcast between {shape} {tuple(scale.shape)}')
   q = numerics.canonical_qtype(qtype)
   scale = scale.to(array.dtype).contiguous()
+  if array.numel() == 0:
+    return QArray(_empty_qvalue(shape, q, array.device), scale, zero_point, q)
   plan = _plan(shape, tuple(d // s for d, s in zip(shape, scale.shape)))
   if plan.kind != '3d':
     raise NotImplementedError('static-scale quantization supports a single reduced axis group')
@@ -405,6 +427,10 @@ def quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = No
   cal, factor = _parse_calibration(how.calibration_method)
   if cal == _lib.MINMAX:
     numerics.get_asymmetric_bound(q)
+  if array.numel() == 0:
+    _check_empty_reduction(sshape)
+    zp = torch.empty(sshape, dtype=torch.int8, device=array.device) if cal == _lib.MINMAX else None
+    return QArray(_empty_qvalue(shape, q, array.device), torch.empty(sshape, dtype=array.dtype, device=array.device), zp, q)
   plan = _plan(shape, tuple(d // s for d, s in zip(shape, sshape)))
   if not array.is_contiguous() and plan.kind == '3d' and plan.dims[2] > 1 and layout in (None, 'reduce_minor'):
     # A strided view whose reduced axes are already the contiguous ones (e.g. a rotated weight kept
@@ -492,6 +518,8 @@ def physical_layout(qa: QArray) -> tuple[_Plan, int, torch.Tensor]:
 def dequantize(array: QArray) -> torch.Tensor:
   """(qvalue - zero_point) * scale in the scale dtype; the reverse of quantize."""
   validate_qarray(array)
+  if math.prod(array.shape) == 0:
+    return torch.empty(array.shape, dtype=array.scale.dtype, device=array.scale.device)
   plan, lay, data = physical_layout(array)
   if plan.kind != '3d':
     raise NotImplementedError('dequantize supports a single reduced axis group')

@@ -12,6 +12,7 @@ zeros.  Only the dimension numbers of `ragged_dot` are supported; others raise.
 from __future__ import annotations
 
 import dataclasses
+import math
 from typing import Sequence
 
 import torch
@@ -166,6 +167,12 @@ def _slow_ragged_dot_general(lhs, rhs, group_sizes, dimension_numbers=_BASIC_RAG
 def ragged_dot_general(lhs, rhs, group_sizes: torch.Tensor, dimension_numbers: RaggedDotDimensionNumbers,
                        precision=None, preferred_element_type=None, group_offset=None) -> torch.Tensor:
   """Drop-in for lax.ragged_dot_general that accepts QArray operands."""
+  if math.prod(lhs.shape) == 0 or math.prod(rhs.shape) == 0:
+    # nothing to launch: no rows or no columns give an empty result, an empty contraction gives zeros
+    _check_basic(dimension_numbers, lhs, rhs, group_sizes, group_offset)
+    _, res_t = qarray.get_accumulator_and_result_type(lhs, rhs, preferred_element_type=preferred_element_type)
+    dev = (lhs.scale if isinstance(lhs, QArray) else lhs).device
+    return torch.zeros(lhs.shape[0], rhs.shape[2], dtype=res_t, device=dev)
   use_fast_path = True
   for operand in (lhs, rhs):
     if isinstance(operand, QArray):

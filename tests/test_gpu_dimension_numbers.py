@@ -124,3 +124,43 @@ def test_three_operand_einsum_contracts_pairwise():
   want = first.v.astype(np.float64) @ p_np.astype(np.float64)
   assert tuple(out.shape) == (24, 8)
   np.testing.assert_allclose(util.f32np(out), want, rtol=1e-4, atol=1e-5)
+
+
+def test_empty_operands_launch_nothing():
+  """Zero-size operands behave like lax.dot_general's: an empty result, zeros for an empty contraction, and
+  the reduction over an empty axis is refused as jnp.max refuses it."""
+  from qwix_amd.core import dot_general as dg, einsum, qarray, ragged_dot
+  dev = util.DEV
+  how_a = qarray.HowToQuantize(qtype='int8', channelwise_axes=[0])
+  how_w = qarray.HowToQuantize(qtype='int8', channelwise_axes=[1])
+  x0 = torch.empty(0, 128, device=dev, dtype=torch.bfloat16)
+  w = torch.randn(128, 64, device=dev, dtype=torch.bfloat16)
+  wq = qarray.quantize(w, how_w)
+  for qtype in ('int8', 'int4', 'float8_e4m3fn'):
+    q0 = qarray.quantize(x0, qarray.HowToQuantize(qtype=qtype, channelwise_axes=[0]))
+    assert tuple(q0.shape) == (0, 128) and tuple(q0.scale.shape) == (0, 1) and q0.scale.dtype == torch.bfloat16
+    qarray.validate_qarray(q0)
+    assert tuple(qarray.dequantize(q0).shape) == (0, 128)
+  with pytest.raises(ValueError, match='zero-size array'):
+    qarray.quantize(torch.empty(128, 0, device=dev, dtype=torch.bfloat16), how_a)
+  with pytest.raises(ValueError, match='zero-size array'):
+    qarray.calibrate(torch.empty(0, 128, device=dev, dtype=torch.bfloat16), how_w)
+  assert tuple(qarray.calibrate(x0, how_a)['absmax'].shape) == (0, 1)
+  dn = (((1,), (0,)), ((), ()))
+  q0 = qarray.quantize(x0, how_a)
+  out = dg.dot_general(q0, wq, dn)
+  assert tuple(out.shape) == (0, 64) and out.dtype == torch.bfloat16
+  out = dg.dot_general(x0, wq, dn, preferred_element_type=torch.float32)
+  assert tuple(out.shape) == (0, 64) and out.dtype == torch.float32
+  assert tuple(einsum.einsum('mk,kn->mn', x0, wq).shape) == (0, 64)
+  # an empty contraction: zeros
+  a = qarray.QArray(torch.empty(4, 0, dtype=torch.int8, device=dev), torch.ones(4, 1, device=dev), None, 'int8')
+  b = qarray.QArray(torch.empty(0, 8, dtype=torch.int8, device=dev), torch.ones(1, 8, device=dev), None, 'int8')
+  out = dg.dot_general(a, b, dn)
+  assert tuple(out.shape) == (4, 8) and torch.count_nonzero(out).item() == 0
+  with pytest.raises(TypeError):
+    dg.dot_general(q0, qarray.quantize(torch.randn(64, 64, device=dev, dtype=torch.bfloat16), how_w), dn)
+  wg = qarray.quantize(torch.randn(2, 128, 64, device=dev, dtype=torch.bfloat16),
+                       qarray.HowToQuantize(qtype='int8', channelwise_axes=[0, 2]))
+  out = ragged_dot.ragged_dot(q0, wg, torch.zeros(2, dtype=torch.int32, device=dev))
+  assert tuple(out.shape) == (0, 64)
