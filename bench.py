@@ -638,7 +638,6 @@ class QdotZeroPoint(QdotW8A8):
   def __init__(self, name, M, K, N):
     super().__init__(name, M, K, N, 'int8')
     self.metric = 'int8 qdot TOPS (asymmetric activation, zero-point correction, activation quantize included)'
-    self.kernel_name = 'qgemm_dma_kernel'
 
   def setup(self, dev):
     import torch

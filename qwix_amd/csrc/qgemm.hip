@@ -910,6 +910,13 @@ template <int QT>
 int dispatch_pp(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
                 const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   const bool all = ep.r0 && ep.r1 && ep.r2, none = !ep.r0 && !ep.r1 && !ep.r2;
+  if (ep.zu != nullptr) {
+    if constexpr (QT == QWIX_INT8) {
+      if (ep.out_dtype == QWIX_BF16) return launch_pp<QT, QWIX_BF16, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      return launch_pp<QT, QWIX_F32, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    }
+    return fail(QWIX_ERR_UNSUPPORTED, "zero-point correction needs int8 operands");
+  }
   if (ep.out_dtype == QWIX_BF16) {
     if (all) return launch_pp<QT, QWIX_BF16, 1>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     return launch_pp<QT, QWIX_BF16, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
@@ -1741,8 +1748,8 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
   const bool big = ((M + 255) / 256) * ((N + 255) / 256) >= 192;
   const bool off32 = M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);  // 32-bit lane offsets
   if (K % 128 == 0 && off32) {  // direct-to-LDS pipeline
-    // long K on a full chip: the ping-pong schedule (no raw-accumulator / zero-point variants of it exist)
-    if (big && K >= 256 && out_dtype != QWIX_I32 && zu == nullptr) {
+    // long K on a full chip: the ping-pong schedule (no raw-accumulator variant of it exists)
+    if (big && K >= 256 && out_dtype != QWIX_I32) {
       if (qtype == QWIX_INT8) return dispatch_pp<QWIX_INT8>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       return dispatch_pp<QWIX_E4M3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     }

@@ -162,3 +162,27 @@ def test_block_quantize_at_ffn_size():
   s = q.scale.float().repeat_interleave(128, 0).repeat_interleave(128, 1)
   quot = (w.float() / s).to(torch.bfloat16).float()
   assert torch.equal(q.qvalue.float(), torch.clamp(quot, -448, 448).to(torch.float8_e4m3fn).float())
+
+
+def test_zero_point_gemm_at_4096():
+  """4096^3 int8 with the zero-point correction in the epilogue of the large-tile kernel, f32 out, no scales:
+  out = a.b^T - zu (x) zv exactly."""
+  from qwix_amd import _lib
+  M = N = K = 4096
+  a = _small_ints((M, K), -3, 3, 21, torch.int8)
+  b = _small_ints((N, K), -3, 3, 22, torch.int8)
+  g = torch.Generator(device='cpu').manual_seed(23)
+  zu = torch.randint(-128, 128, (M,), generator=g, dtype=torch.int32).to(util.DEV)
+  zv = torch.empty(N, dtype=torch.int32, device=util.DEV)
+  _lib.call('qwix_hip_ksum_i8', b.data_ptr(), K, N, K, zv.data_ptr(), _lib.stream_of(b))
+  assert torch.equal(zv, b.to(torch.int32).sum(1, dtype=torch.int32))
+  out = torch.empty(M, N, dtype=torch.float32, device=util.DEV)
+  print('case zero point full size', M, K, N, flush=True)
+  _lib.call('qwix_hip_qgemm_zp', a.data_ptr(), K, b.data_ptr(), K, M, N, K, None, 0, None, 0, zu.data_ptr(),
+            zv.data_ptr(), out.data_ptr(), _lib.F32, N, _lib.stream_of(a))
+  torch.cuda.synchronize()
+  rows = util.rng(24).choice(M, 8, replace=False)
+  want = a[rows].cpu().numpy().astype(np.int64) @ b.cpu().numpy().astype(np.int64).T
+  want = want - zu[rows].cpu().numpy().astype(np.int64)[:, None] * zv.cpu().numpy().astype(np.int64)[None, :]
+  assert np.abs(want).max() < 2 ** 24
+  assert np.array_equal(out[rows].cpu().to(torch.float64).numpy(), want.astype(np.float64))
