@@ -334,7 +334,7 @@ def generic_broadcast(op, x: np.ndarray, y: np.ndarray) -> np.ndarray:
 
 
 def calibrate(array: FArr, how: HowToQuantize) -> dict[str, FArr]:
-  """qarray.py:470-534, absmax and minmax methods."""
+  """qarray.py:470-534: the absmax, minmax and fixed methods (rms is not restated)."""
   reduce_axes = []
   off = 0
   for axis in range(array.ndim):
@@ -362,6 +362,18 @@ def calibrate(array: FArr, how: HowToQuantize) -> dict[str, FArr]:
     if args:
       am = rnd(am * rnd(np.float32(args[0]), d), d)
     return {'absmax': FArr(am.reshape(shape), d)}
+  if method == 'fixed':  # qarray.py:518-532: a constant, per-tensor range
+    if len(args) not in (1, 2):
+      raise ValueError('A fixed range is required for fixed calibration.')
+    if len(args) == 1:
+      args = (-args[0], args[0])
+    if args[0] > 0 or args[1] < 0 or args[0] >= args[1]:
+      raise ValueError('The range must contain 0 and be non-empty.')
+    ones = tuple(1 for _ in shape)
+    if args[0] + args[1] == 0:
+      return {'absmax': FArr(np.full(ones, rnd(np.float32(args[1]), d), np.float32), d)}
+    return {'min': FArr(np.full(ones, rnd(np.float32(args[0]), d), np.float32), d),
+            'max': FArr(np.full(ones, rnd(np.float32(args[1]), d), np.float32), d)}
   raise ValueError(f'Unsupported calibration: {how.calibration_method}')
 
 

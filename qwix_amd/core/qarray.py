@@ -276,9 +276,31 @@ def _tiles_from_how(shape, how: HowToQuantize) -> tuple[int, ...]:
   return tuple(d // s for d, s in zip(shape, ss))
 
 
+def _fixed_calibration(method: str, array: torch.Tensor) -> dict[str, torch.Tensor] | None:
+  """'fixed,a[,b]' (qarray.py:518-532): a constant per-tensor range, nothing is read from the array.
+  None for the other methods."""
+  name, *args = method.lower().split(',')
+  if name != 'fixed':
+    return None
+  args = [float(a) for a in args]
+  if len(args) not in (1, 2):
+    raise ValueError('A fixed range is required for fixed calibration.')
+  if len(args) == 1:
+    args = [-args[0], args[0]]
+  if args[0] > 0 or args[1] < 0 or args[0] >= args[1]:
+    raise ValueError('The range must contain 0 and be non-empty.')
+  ones = (1,) * array.ndim
+  full = lambda v: torch.full(ones, v, dtype=array.dtype, device=array.device)
+  if args[0] + args[1] == 0:
+    return {'absmax': full(args[1])}
+  return {'min': full(args[0]), 'max': full(args[1])}
+
+
 def _parse_calibration(method: str) -> tuple[int, float]:
   name, *args = method.lower().split(',')
   args = [float(a) for a in args]
+  if name == 'rms':
+    raise NotImplementedError('rms calibration is not part of the HIP path (absmax, minmax and fixed are)')
   if name not in ('absmax', 'minmax'):
     raise ValueError(f'Unsupported calibration: {method}')
   return (_lib.ABSMAX if name == 'absmax' else _lib.MINMAX), (args[0] if args else 0.0)
@@ -355,6 +377,9 @@ def calibrate(array: torch.Tensor, how: HowToQuantize) -> dict[str, torch.Tensor
   array = _check_float_input(array)
   shape = tuple(array.shape)
   sshape = get_scale_shape(shape, how)
+  fixed = _fixed_calibration(how.calibration_method, array)
+  if fixed is not None:
+    return fixed
   cal, factor = _parse_calibration(how.calibration_method)
   if array.numel() == 0:
     _check_empty_reduction(sshape)
@@ -424,6 +449,10 @@ def quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = No
   shape = tuple(array.shape)
   q = numerics.canonical_qtype(how.qtype)
   sshape = get_scale_shape(shape, how)
+  fixed = _fixed_calibration(how.calibration_method, array)
+  if fixed is not None:  # a constant range: the static-scale kernel, with one scale for the whole array
+    scale, zp = compute_scale_zero_point(fixed, q)
+    return quantize_with_scale_zero_point(array, q, scale, zp, layout=layout)
   cal, factor = _parse_calibration(how.calibration_method)
   if cal == _lib.MINMAX:
     numerics.get_asymmetric_bound(q)

@@ -150,6 +150,22 @@ def test_2d_blocks(shape, tiles, dtype, qtype):
            what='2d blocks minmax')
 
 
+@pytest.mark.parametrize('qtype', QTYPES)
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+def test_fixed_calibration(dtype, qtype):
+  """'fixed,a[,b]': a constant per-tensor range, whatever axes are named channelwise."""
+  x_np, x_t = util.make((48, 256), dtype, seed=71, scale=2.0)
+  _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=[0], calibration_method='fixed,3'), what='fixed symmetric')
+  _check(x_np, x_t, dtype, dict(qtype=qtype, calibration_method='fixed,-2.5,2.5'), what='fixed symmetric pair')
+  if qtype != 'float8_e4m3fn':
+    _check(x_np, x_t, dtype, dict(qtype=qtype, channelwise_axes=[1], calibration_method='fixed,-1,3'), what='fixed asymmetric')
+  from qwix_amd.core import qarray
+  with pytest.raises(ValueError):
+    qarray.quantize(x_t, qarray.HowToQuantize(qtype=qtype, calibration_method='fixed,1,2'))
+  with pytest.raises(NotImplementedError):
+    qarray.quantize(x_t, qarray.HowToQuantize(qtype=qtype, calibration_method='rms,3'))
+
+
 def test_zero_rows_and_reference_convert_vectors():
   from qwix_amd.core import qarray
   x = torch.zeros(4, 256, dtype=torch.bfloat16, device=util.DEV)

@@ -293,3 +293,25 @@ def test_dequantize_closed_form():
   zp = np.array([[1, -1]], np.int8)
   dq = O.dequantize(O.QArray(q, s, zp, 'int4'))
   assert dq.v.tolist() == [[-4.5, 3.0, 1.0, 0.25]]
+
+
+def test_fixed_calibration_closed_form():
+  """qarray.py:518-532: 'fixed,a' is a per-tensor absmax of a, 'fixed,a,b' a per-tensor (min, max); with
+  a = 127.5 the int8 scale is exactly 1 and quantize reduces to convert_to (numerics_test.py:34-50)."""
+  x = O.FArr(np.array([[1.2, 3.5, -127.5, 129.0, -1300.0]], np.float32), O.F32)
+  how = O.HowToQuantize(qtype='int8', channelwise_axes=[0], calibration_method='fixed,127.5')
+  cal = O.calibrate(x, how)
+  assert set(cal) == {'absmax'} and cal['absmax'].v.shape == (1, 1) and cal['absmax'].v.item() == 127.5
+  q = O.quantize(x, how)
+  assert q.scale.v.shape == (1, 1) and q.scale.v.item() == 1.0
+  assert q.qvalue.tolist() == [[1, 4, -128, 127, -128]]
+  # asymmetric: range [-1, 3] on int8 -> scale = 4/255, zero point = rint(-128 + 1/scale) = -64
+  how = O.HowToQuantize(qtype='int8', calibration_method='fixed,-1,3')
+  q = O.quantize(O.FArr(np.array([[-1.0, 0.0, 3.0, 10.0]], np.float32), O.F32), how)
+  s = np.float32(4.0) / np.float32(255.0)
+  assert q.scale.v.item() == s
+  assert q.zero_point.item() == int(np.rint(np.float32(-128.0) - np.float32(-1.0) / s))
+  assert q.qvalue.tolist() == [[-128, int(q.zero_point.item()), 127, 127]]
+  for bad in ('fixed', 'fixed,1,2', 'fixed,-1,-0.5', 'fixed,0,0'):
+    with pytest.raises(ValueError):
+      O.calibrate(x, O.HowToQuantize(qtype='int8', calibration_method=bad))
