@@ -101,6 +101,14 @@ QWIX_API int qwix_hip_dequantize(const void* qvalue, int qtype, int q_layout, in
                         int64_t reduce, int64_t inner, int64_t tile, const void* scale,
                         const void* zero_point, int dtype, void* out, void* stream);
 
+/* dequantize for the 5-D geometry of qwix_hip_quantize_generic (two reduced axis groups, e.g. one
+ * scale per t1 x t3 block; two_dim_scales_test.py:29-56 dequantizes such an array):
+ * out[i] = D(D(q[i] - zp) * scale) with the scale / zero point of element i's block.  qvalue in the
+ * natural layout, scale (and zero_point, may be NULL) as qwix_hip_quantize_generic writes them. */
+QWIX_API int qwix_hip_dequantize_generic(const void* qvalue, int qtype, const int64_t dims[5], int64_t t1,
+                                int64_t t3, const void* scale, const void* zero_point, int dtype,
+                                void* out, void* stream);
+
 /* Layout helper: (rows, cols) bytes -> (cols, rows) bytes; int4: repacks so the pairs run
  * along the new contiguous axis.  Used to bring a NATURAL qvalue to REDUCE_MINOR. */
 QWIX_API int qwix_hip_transpose_q(const void* src, int qtype, int64_t rows, int64_t cols, void* dst,

@@ -32,6 +32,7 @@ SIGNATURES = {
     'qwix_hip_quantize_with_scale': (_int, [_vp, _int, _i64, _i64, _i64, _i64, _int, _vp, _vp, _int, _vp, _vp]),
     'qwix_hip_quantize_generic': (_int, [_vp, _int, _c.POINTER(_i64), _i64, _i64, _int, _int, _f32, _vp, _vp, _vp, _vp]),
     'qwix_hip_dequantize': (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64, _vp, _vp, _int, _vp, _vp]),
+    'qwix_hip_dequantize_generic': (_int, [_vp, _int, _c.POINTER(_i64), _i64, _i64, _vp, _vp, _int, _vp, _vp]),
     'qwix_hip_transpose_q': (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
     'qwix_hip_qgemm': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _vp, _int, _vp, _int, _int, _vp, _int, _i64, _vp]),
     'qwix_hip_qgemm_zp': (_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _int, _vp, _int, _vp, _vp, _vp, _int, _i64, _vp]),

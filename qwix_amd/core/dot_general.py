@@ -71,6 +71,18 @@ def _use_fast_path(lhs, rhs, dimension_numbers) -> bool:
 # ------------------------------------------------------------------------------------------
 
 
+def _broadcast_free(s: torch.Tensor, shape: Sequence[int], free: Sequence[int]) -> torch.Tensor:
+  """Brings the scale (or zero point) to full size along the non-contracted axes: a per-tensor entry is
+  expanded, a tiled axis repeats each entry over its tile -- the generic broadcast the reference applies to
+  the result (qarray.py:425-444), done on the small array instead."""
+  if all(s.shape[a] == shape[a] for a in free):
+    return s
+  for a in free:
+    if s.shape[a] not in (1, shape[a]):
+      s = s.repeat_interleave(shape[a] // s.shape[a], dim=a)
+  return s.expand(*[shape[a] if a in free else s.shape[a] for a in range(s.ndim)])
+
+
 class _Canon:
   """lhs as (M, K) row-major, rhs as (N, K) K-contiguous, plus scales in kernel order."""
 
@@ -139,10 +151,7 @@ class _Canon:
     ga = s.shape[self.lca[-1]]
     if ga > 1 and len(self.lca) > 1:
       raise NotImplementedError('sub-channel lhs scales with several contracting axes are not supported')
-    want = tuple(lhs.shape[a] for a in self.lfree)
-    got = tuple(s.shape[a] for a in self.lfree)
-    if got != want:
-      s = s.expand(*[lhs.shape[a] if a in self.lfree else s.shape[a] for a in range(s.ndim)])
+    s = _broadcast_free(s, lhs.shape, self.lfree)
     return s.permute(*(self.lfree + self.lca)).reshape(self.M, ga).contiguous(), ga
 
   def rhs_scale(self, rhs: QArray) -> tuple[torch.Tensor | None, int]:
@@ -154,8 +163,7 @@ class _Canon:
     gb = s.shape[self.rca[-1]]
     if gb > 1 and len(self.rca) > 1:
       raise NotImplementedError('sub-channel rhs scales with several contracting axes are not supported')
-    if tuple(s.shape[a] for a in self.rfree) != tuple(rhs.shape[a] for a in self.rfree):
-      s = s.expand(*[rhs.shape[a] if a in self.rfree else s.shape[a] for a in range(s.ndim)])
+    s = _broadcast_free(s, rhs.shape, self.rfree)
     s = s.permute(*([self.rca[-1]] + self.rfree + self.rca[:-1]))
     return s.reshape(gb, self.N).contiguous(), gb
 
@@ -165,16 +173,14 @@ class _Canon:
     z = lhs.zero_point
     if any(z.shape[a] != 1 for a in self.lca):
       raise NotImplementedError('sub-channel zero points are not supported on the quantized path')
-    if tuple(z.shape[a] for a in self.lfree) != tuple(lhs.shape[a] for a in self.lfree):
-      z = z.expand(*[lhs.shape[a] if a in self.lfree else z.shape[a] for a in range(z.ndim)])
+    z = _broadcast_free(z, lhs.shape, self.lfree)
     return z.permute(*(self.lfree + self.lca)).reshape(self.M).contiguous()
 
   def rhs_zero_point(self, rhs: QArray) -> torch.Tensor:
     z = rhs.zero_point
     if any(z.shape[a] != 1 for a in self.rca):
       raise NotImplementedError('sub-channel zero points are not supported on the quantized path')
-    if tuple(z.shape[a] for a in self.rfree) != tuple(rhs.shape[a] for a in self.rfree):
-      z = z.expand(*[rhs.shape[a] if a in self.rfree else z.shape[a] for a in range(z.ndim)])
+    z = _broadcast_free(z, rhs.shape, self.rfree)
     z = z.permute(*(self.rfree + self.rca))
     return z.reshape(self.N).contiguous()
 

@@ -550,11 +550,16 @@ def dequantize(array: QArray) -> torch.Tensor:
   if math.prod(array.shape) == 0:
     return torch.empty(array.shape, dtype=array.scale.dtype, device=array.scale.device)
   plan, lay, data = physical_layout(array)
-  if plan.kind != '3d':
-    raise NotImplementedError('dequantize supports a single reduced axis group')
   out = torch.empty(array.shape, dtype=array.scale.dtype, device=array.scale.device)
   scale = array.scale.contiguous()
   zp = None if array.zero_point is None else array.zero_point.contiguous()
+  if plan.kind != '3d':  # two reduced axis groups (block scales); physical_layout only passes the natural layout
+    import ctypes
+    dims = (ctypes.c_int64 * 5)(*plan.dims)
+    _lib.call('qwix_hip_dequantize_generic', data.data_ptr(), numerics.qtype_tag(array.qtype), dims, plan.tiles[0],
+              plan.tiles[1], scale.data_ptr(), _lib.ptr(zp), _lib.float_tag(scale.dtype), out.data_ptr(),
+              _lib.stream_of(scale))
+    return out
   _lib.call('qwix_hip_dequantize', data.data_ptr(), numerics.qtype_tag(array.qtype), lay, *plan.dims, plan.tiles[0],
             scale.data_ptr(), _lib.ptr(zp), _lib.float_tag(scale.dtype), out.data_ptr(), _lib.stream_of(scale))
   return out

@@ -1048,6 +1048,53 @@ __global__ void __launch_bounds__(256)
   store8<D>(out, idx, v);
 }
 
+// Dequantize for the 5-D geometry (two reduced axis groups: block scales).  VEC = 8: eight consecutive elements
+// of the innermost reduced axis share a scale (d4 == 1, t3 % 8 == 0); VEC = 1: anything.
+template <typename D, int QT, int VEC>
+__global__ void __launch_bounds__(256)
+    generic_dequant_kernel(const uint8_t* __restrict__ q, Geom5 g, const void* __restrict__ scale,
+                           const int8_t* __restrict__ zp, void* __restrict__ out) {
+  const int64_t n = g.d[0] * g.d[1] * g.d[2] * g.d[3] * g.d[4];
+  const int64_t idx = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * VEC;
+  if (idx >= n) return;
+  int64_t r = idx;
+  const int64_t i4 = r % g.d[4]; r /= g.d[4];
+  const int64_t i3 = r % g.d[3]; r /= g.d[3];
+  const int64_t i2 = r % g.d[2]; r /= g.d[2];
+  const int64_t i1 = r % g.d[1];
+  const int64_t i0 = r / g.d[1];
+  const int64_t si = scale_index5(g, i0, i1, i2, i3, i4);
+  const float sv = load1<D>(scale, si);
+  const float zv = zp ? rnd<D>(static_cast<float>(zp[si])) : 0.f;
+  uint32_t b[VEC];
+  if constexpr (VEC == 8) {
+    if constexpr (QT == QWIX_INT4) {
+      const uint32_t w = *reinterpret_cast<const uint32_t*>(q + idx / 2);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) b[e] = (w >> (4 * e)) & 0xF;
+    } else {
+      const uint2 w = *reinterpret_cast<const uint2*>(q + idx);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        b[e] = (w.x >> (8 * e)) & 0xFF;
+        b[4 + e] = (w.y >> (8 * e)) & 0xFF;
+      }
+    }
+  } else {
+    if constexpr (QT == QWIX_INT4) b[0] = (q[idx / 2] >> (4 * (idx & 1))) & 0xF;
+    else b[0] = q[idx];
+  }
+  float v[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    float t = rnd<D>(q_to_f32<QT>(b[e]));
+    if (zp != nullptr) t = rnd<D>(t - zv);
+    v[e] = rnd<D>(t * sv);
+  }
+  if constexpr (VEC == 8) store8<D>(out, idx, v);
+  else store1<D>(out, idx, v[0]);
+}
+
 // Reduce-minor layout (values stored (outer, inner, reduce), output (outer, reduce, inner)): a 64 x 64 tile is
 // read along the reduced axis, turned in LDS, and written along the inner axis with its scales, 16 per thread.
 template <typename D, int QT>
@@ -1489,6 +1536,42 @@ int qwix_hip_quantize_generic(const void* x, int dtype, const int64_t dims[5], i
     })
   })
   return check_launch("generic quantize");
+}
+
+int qwix_hip_dequantize_generic(const void* qvalue, int qtype, const int64_t dims[5], int64_t t1, int64_t t3,
+                                const void* scale, const void* zero_point, int dtype, void* out, void* stream) {
+  if (!qvalue || !scale || !out || !dims) return fail(QWIX_ERR_INVALID_ARGUMENT, "null argument");
+  Geom5 g;
+  int64_t n = 1;
+  for (int i = 0; i < 5; ++i) {
+    if (dims[i] <= 0) return fail(QWIX_ERR_INVALID_ARGUMENT, "dims[%d] = %lld", i, (long long)dims[i]);
+    g.d[i] = dims[i];
+    n *= dims[i];
+  }
+  if (t1 <= 0 || t3 <= 0 || dims[1] % t1 || dims[3] % t3)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "tiles (%lld, %lld) do not divide (%lld, %lld)", (long long)t1,
+                (long long)t3, (long long)dims[1], (long long)dims[3]);
+  if (qtype == QWIX_INT4 && (n & 1)) return fail(QWIX_ERR_UNSUPPORTED, "int4 needs an even element count");
+  g.t1 = t1;
+  g.t3 = t3;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint8_t* q = static_cast<const uint8_t*>(qvalue);
+  const int8_t* zp = static_cast<const int8_t*>(zero_point);
+  const bool vec = dims[4] == 1 && t3 % 8 == 0 && (reinterpret_cast<uintptr_t>(qvalue) & 7) == 0 && aligned16(out);
+  const int64_t threads = vec ? n / 8 : n;
+  const dim3 grid(static_cast<unsigned>((threads + 255) / 256));
+  if (threads + 255 >= (int64_t{256} << 31)) return fail(QWIX_ERR_UNSUPPORTED, "array too large");
+#define QWIX_DEQ_GEN(QTT)                                                                            \
+  if (vec) generic_dequant_kernel<D, QTT, 8><<<grid, 256, 0, st>>>(q, g, scale, zp, out);          \
+  else generic_dequant_kernel<D, QTT, 1><<<grid, 256, 0, st>>>(q, g, scale, zp, out)
+  QWIX_DISPATCH_D(dtype, {
+    if (qtype == QWIX_INT8) { QWIX_DEQ_GEN(QWIX_INT8); }
+    else if (qtype == QWIX_INT4) { QWIX_DEQ_GEN(QWIX_INT4); }
+    else if (qtype == QWIX_E4M3) { QWIX_DEQ_GEN(QWIX_E4M3); }
+    else return fail(QWIX_ERR_INVALID_ARGUMENT, "unknown qtype %d", qtype);
+  })
+#undef QWIX_DEQ_GEN
+  return check_launch("generic dequantize");
 }
 
 int qwix_hip_dequantize(const void* qvalue, int qtype, int q_layout, int64_t outer, int64_t reduce, int64_t inner,

@@ -153,3 +153,60 @@ def test_weight_only_gemv(M, K, N, group, sdt, wq_type):
   # default result type follows the scale dtype (bf16 x f32 -> f32)
   out2 = dg.dot_general(x_t, wq, DN)
   assert out2.dtype == sdt
+
+
+def _close(got, true, dtype):
+  """f32: the 1e-4 of the reference's test; bf16 results carry a rounding per epilogue step: 1 % mean error."""
+  if dtype == O.F32:
+    return np.allclose(got, true, rtol=1e-4, atol=1e-4)
+  return np.abs(got - true).mean() / np.abs(true).mean() < 1e-2
+
+
+def _two_dim_pair(M, K, N, lt, rt, dtype, seed):
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make((M, K), dtype, seed=seed)
+  w_np, w_t = util.make((K, N), dtype, seed=seed + 1)
+  lkw = dict(qtype='int8', tiled_axes={0: lt[0], 1: lt[1]})
+  rkw = dict(qtype='int8', tiled_axes={0: rt[0], 1: rt[1]})
+  xq = qarray.quantize(x_t, qarray.HowToQuantize(**lkw))
+  wq = qarray.quantize(w_t, qarray.HowToQuantize(**rkw))
+  oxq = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(**lkw))
+  owq = O.quantize(O.FArr(w_np, dtype), O.HowToQuantize(**rkw))
+  util.assert_qarray_equal(xq, oxq, 'lhs')
+  util.assert_qarray_equal(wq, owq, 'rhs')
+  return xq, wq, oxq, owq
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+def test_two_dim_scales_small_tiles(dtype):
+  """two_dim_scales_test.py:29-93: 8 x 8 tiles on both operands of a 128^3 product.  Tiles below 128 take the
+  dequantize-first path; dequantize is bit-exact, and dot_general == dequant . dequant within the 1e-4 the
+  reference test asks for."""
+  from qwix_amd.core import dot_general as dg, qarray
+  xq, wq, oxq, owq = _two_dim_pair(128, 128, 128, (8, 8), (8, 8), dtype, seed=81)
+  assert tuple(xq.scale.shape) == (16, 16)
+  for got, want in ((qarray.dequantize(xq), O.dequantize(oxq)), (qarray.dequantize(wq), O.dequantize(owq))):
+    assert tuple(got.shape) == (128, 128)
+    assert np.array_equal(util.f32np(got), want.v)
+  true = O.dequantize(oxq).v.astype(np.float64) @ O.dequantize(owq).v.astype(np.float64)
+  out = dg.dot_general(xq, wq, DN)
+  assert _close(util.f32np(out), true, dtype)
+  slow = dg._slow_dot_general(xq, wq, DN)
+  assert _close(util.f32np(slow), true, dtype)
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('lt,rt', [((64, 128), (128, 128)), ((32, 128), (128, 64)), ((256, 256), (256, 32))])
+def test_two_dim_scales_on_the_quantized_path(lt, rt, dtype):
+  """K tiles of at least 128 stay on the quantized path: the scales of the tiled non-contracted axes are
+  repeated over their tiles (the reference's generic broadcast), the per-K-tile int32 partials are exact."""
+  from qwix_amd.core import dot_general as dg
+  xq, wq, oxq, owq = _two_dim_pair(256, 512, 384, lt, rt, dtype, seed=83)
+  out, acc = dg._fast_dot_general(xq, wq, DN, exact=True, return_accumulators=True)
+  torch.cuda.synchronize()
+  want, wacc = O.fast_dot_general(oxq, owq, DN, return_acc=True)
+  assert np.array_equal(acc.cpu().numpy(), wacc), 'per-group int32 partials differ'
+  assert np.array_equal(util.f32np(out), want.v)
+  fast = dg.dot_general(xq, wq, DN)
+  true = O.dequantize(oxq).v.astype(np.float64) @ O.dequantize(owq).v.astype(np.float64)
+  assert _close(util.f32np(fast), true, dtype)
