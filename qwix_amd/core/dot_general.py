@@ -111,7 +111,7 @@ class _Canon:
   def lhs_values(self, lhs) -> torch.Tensor:
     v = lhs.qvalue if isinstance(lhs, QArray) else lhs
     if isinstance(v, Int4Tensor):
-      raise NotImplementedError('an int4 left operand is not supported by the HIP GEMM kernels')
+      v = v.unpack()  # int4 activations are widened to int8 (exact); the MFMA kernels take int8 rows
     v = v.permute(*(self.lfree + self.lca))  # contracting axes last (a no-op view in the usual layout)
     v = v if v.is_contiguous() else v.contiguous()
     return v.reshape(self.M, self.K)
@@ -335,6 +335,13 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
                       return_accumulators: bool = False, **kwargs) -> torch.Tensor:
   """Contract the quantized values on the matrix cores, then scale: out = ((acc * sx) * sy)."""
   del kwargs
+  if _is_float_array(lhs) or _is_float_array(rhs):
+    # The reference contracts a raw float operand with the other side's quantized values and scales the
+    # result (dot_general.py:135-261 with lhs_scale / rhs_scale None); the dispatcher never sends such a pair
+    # here.  It is served by the dequantize-first kernels: the same value up to the rounding of a float dot.
+    if return_accumulators:
+      raise NotImplementedError('raw accumulators need quantized operands on both sides')
+    return _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type)
   lzp = lhs.zero_point if isinstance(lhs, QArray) else None
   rzp = rhs.zero_point if isinstance(rhs, QArray) else None
   if lzp is not None and rzp is not None:
@@ -355,6 +362,8 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
       raise ValueError(f'Contracting axes must be tiled with the same tile size. lhs_tiled_axes={lt} rhs_tiled_axes={rt} {dimension_numbers=}')
   acc_t, res_t = qarray.get_accumulator_and_result_type(lhs, rhs, preferred_element_type=preferred_element_type)
   lq, rq = _qtype_of(lhs), _qtype_of(rhs)
+  if lq == numerics.INT4:
+    lq = numerics.INT8  # lhs_values widens int4 rows
   a = c.lhs_values(lhs)
   b, b_is4 = c.rhs_values(rhs)
   sa, ga = c.lhs_scale(lhs) if isinstance(lhs, QArray) else (None, 1)
@@ -363,6 +372,13 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   st = _lib.stream_of(a)
   out = torch.empty(c.M, c.N, dtype=res_t, device=dev)
   grouped = ga > 1 or gb > 1 or b_is4
+  K = c.K
+  if not grouped and K % 16:
+    # The kernels read K in 16-byte pieces: zero columns (+0 in e4m3 too) add nothing to any sum.
+    pad = 16 - K % 16
+    a = torch.nn.functional.pad(a.view(torch.uint8), (0, pad)).view(a.dtype)
+    b = torch.nn.functional.pad(b.view(torch.uint8), (0, pad)).view(b.dtype)
+    K += pad
   if not grouped:
     if (lq, rq) == (numerics.INT8, numerics.INT8):
       qt = _lib.INT8
@@ -377,26 +393,24 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
         raise NotImplementedError('zero-point operands need int8 x int8 values on the quantized path')
       if return_accumulators:
         raise NotImplementedError('raw accumulators are not returned for zero-point operands')
-      if c.K % 16:
-        raise NotImplementedError('zero-point correction needs K to be a multiple of 16')
       if lzp is not None:
         zu = c.lhs_zero_point(lhs).to(torch.int32)
         zv = torch.empty(c.N, dtype=torch.int32, device=dev)
-        _lib.call('qwix_hip_ksum_i8', b.data_ptr(), b.stride(0), c.N, c.K, zv.data_ptr(), st)
+        _lib.call('qwix_hip_ksum_i8', b.data_ptr(), b.stride(0), c.N, K, zv.data_ptr(), st)
       else:
         zv = c.rhs_zero_point(rhs).to(torch.int32)
         zu = torch.empty(c.M, dtype=torch.int32, device=dev)
-        _lib.call('qwix_hip_ksum_i8', a.data_ptr(), a.stride(0), c.M, c.K, zu.data_ptr(), st)
-      _lib.call('qwix_hip_qgemm_zp', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), c.M, c.N, c.K,
+        _lib.call('qwix_hip_ksum_i8', a.data_ptr(), a.stride(0), c.M, K, zu.data_ptr(), st)
+      _lib.call('qwix_hip_qgemm_zp', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), c.M, c.N, K,
                 _lib.ptr(sa), 0 if sa is None else _lib.float_tag(sa.dtype), _lib.ptr(sb),
                 0 if sb is None else _lib.float_tag(sb.dtype), zu.data_ptr(), zv.data_ptr(), out.data_ptr(),
                 _tag_of(res_t), c.N, st)
       return out.reshape(c.out_shape)
     if return_accumulators:
       acc = torch.empty(c.M, c.N, dtype=torch.int32, device=dev)
-      _lib.call('qwix_hip_qgemm', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), qt, c.M, c.N, c.K, None, 0,
+      _lib.call('qwix_hip_qgemm', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), qt, c.M, c.N, K, None, 0,
                 None, 0, 0, acc.data_ptr(), _lib.I32, c.N, st)
-    _lib.call('qwix_hip_qgemm', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), qt, c.M, c.N, c.K,
+    _lib.call('qwix_hip_qgemm', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), qt, c.M, c.N, K,
               _lib.ptr(sa), 0 if sa is None else _lib.float_tag(sa.dtype), _lib.ptr(sb),
               0 if sb is None else _lib.float_tag(sb.dtype), _tag_of(acc_t) if acc_t != torch.int32 else 0,
               out.data_ptr(), _tag_of(res_t), c.N, st)

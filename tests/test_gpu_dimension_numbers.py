@@ -164,3 +164,40 @@ def test_empty_operands_launch_nothing():
                        qarray.HowToQuantize(qtype='int8', channelwise_axes=[0, 2]))
   out = ragged_dot.ragged_dot(q0, wg, torch.zeros(2, dtype=torch.int32, device=dev))
   assert tuple(out.shape) == (0, 64)
+
+
+def test_reference_output_dtype_table_by_execution():
+  """dot_general_test.py:28-146 builds 10 x 10 operands of ones with per-tensor scales and checks the result
+  dtype of the slow path, the fast path, the dispatcher and einsum under every preferred_element_type.  Here
+  the four are run, not only shape-evaluated: K = 10 is not a multiple of the kernels' 16-byte pieces, the
+  int4 left operand is widened, and every output element must be exactly 10."""
+  from qwix_amd.core import dot_general as dg, einsum, qarray
+  dev = util.DEV
+
+  def mk(spec):
+    if not isinstance(spec, tuple):
+      return torch.ones(10, 10, dtype=spec, device=dev)
+    qd, sd = spec
+    if qd == 'int4':
+      qv = qarray.Int4Tensor(torch.full((10, 5), 0x11, dtype=torch.uint8, device=dev), (10, 10), 1)
+    elif qd == 'int8':
+      qv = torch.ones(10, 10, dtype=torch.int8, device=dev)
+    else:
+      qv = torch.ones(10, 10, device=dev).to(torch.float8_e4m3fn)
+    return qarray.QArray(qv, torch.ones(1, 1, dtype=sd, device=dev), None, qd)
+
+  bf16, f32 = torch.bfloat16, torch.float32
+  cases = [(bf16, f32, f32), (bf16, ('int8', bf16), bf16), (bf16, ('int8', f32), f32),
+           (('int4', bf16), ('int8', f32), f32), (('float8_e4m3fn', bf16), ('float8_e4m3fn', f32), f32)]
+  dn = (((1,), (0,)), ((), ()))
+  for l, r, expected in cases:
+    lhs, rhs = mk(l), mk(r)
+    for pet in (None, bf16, f32):
+      want = pet or expected
+      outs = [dg._slow_dot_general(lhs, rhs, dn, preferred_element_type=pet),
+              dg._fast_dot_general(lhs, rhs, dn, preferred_element_type=pet),
+              dg.dot_general(lhs, rhs, dn, preferred_element_type=pet),
+              einsum.einsum('ab,bc->ac', lhs, rhs, preferred_element_type=pet)]
+      for o in outs:
+        assert o.dtype == want, (l, r, pet, o.dtype)
+        assert tuple(o.shape) == (10, 10) and torch.all(o.float() == 10).item(), (l, r, pet)
