@@ -43,6 +43,20 @@ def _binary(lhs, rhs, einsum_str: str, dot_general_fn, preferred_element_type, *
   return out
 
 
+def broadcast_operands(operands: list, subs_list: list[str]) -> list:
+  """einsum_info.py:197-241: operands that share a subscript with different sizes are brought to the
+  largest one when it is a multiple of the others (size 1 included), values repeated tile-wise."""
+  size = {}
+  for op, subs in zip(operands, subs_list):
+    if len(subs) != len(op.shape):
+      return operands  # ellipsis or rank mismatch: left to the parser
+    for ch, d in zip(subs, op.shape):
+      d = int(d)
+      if ch not in size or size[ch] == 1 or (d > size[ch] and d % size[ch] == 0):
+        size[ch] = d
+  return [qarray.broadcast_to(op, tuple(size[c] for c in subs)) for op, subs in zip(operands, subs_list)]
+
+
 def einsum(*args, _qwix_dot_general=_dg.dot_general, preferred_element_type=None, **kwargs) -> torch.Tensor:
   """Drop-in for jnp.einsum('subscripts', a, b) with QArray operands; the result dtype follows the
   dequantized dtypes unless preferred_element_type is given."""
@@ -50,6 +64,9 @@ def einsum(*args, _qwix_dot_general=_dg.dot_general, preferred_element_type=None
     raise NotImplementedError('einsum expects the subscripts string first')
   einsum_str, operands = args[0], list(args[1:])
   _, res_t = qarray.get_accumulator_and_result_type(*operands, preferred_element_type=preferred_element_type)
+  flat = einsum_str.replace(' ', '')
+  if '.' not in flat:
+    operands = broadcast_operands(operands, flat.split('->')[0].split(','))
   if len(operands) == 1:
     op = operands[0]
     return torch.einsum(einsum_str, qarray.dequantize(op) if isinstance(op, qarray.QArray) else op).to(res_t)

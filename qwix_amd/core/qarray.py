@@ -538,8 +538,10 @@ def physical_layout(qa: QArray) -> tuple[_Plan, int, torch.Tensor]:
     phys = data.permute(*order)
     if phys.is_contiguous() and (not is4 or qa.qvalue.packed_axis == order[-1]):
       return plan, _lib.LAYOUT_REDUCE_MINOR, phys
+  if not is4:  # any other strided view (a slice of a batch, a transposed copy): one compaction
+    return plan, _lib.LAYOUT_NATURAL, data.contiguous()
   raise NotImplementedError(
-      f'QArray values of shape {shape} with strides {tuple(data.stride())} are neither row-major nor '
+      f'int4 values of shape {shape} with strides {tuple(data.stride())} are neither row-major nor '
       'reduce-minor; make them contiguous first.'
   )
 
@@ -563,6 +565,52 @@ def dequantize(array: QArray) -> torch.Tensor:
   _lib.call('qwix_hip_dequantize', data.data_ptr(), numerics.qtype_tag(array.qtype), lay, *plan.dims, plan.tiles[0],
             scale.data_ptr(), _lib.ptr(zp), _lib.float_tag(scale.dtype), out.data_ptr(), _lib.stream_of(scale))
   return out
+
+
+# ------------------------------------------------------------------------------------------
+# generic broadcast
+# ------------------------------------------------------------------------------------------
+
+
+def _broadcast_tensor(x: torch.Tensor, shape: tuple[int, ...]) -> torch.Tensor:
+  """An axis of size s grows to a multiple t * s by repeating each element t times (size 1: plain
+  broadcast) -- call_with_generic_broadcast of qarray.py:425-444 against an array of the target shape."""
+  if x.ndim < len(shape):
+    x = x.reshape((1,) * (len(shape) - x.ndim) + tuple(x.shape))
+  if x.ndim != len(shape):
+    raise ValueError(f'Cannot broadcast between {tuple(x.shape)} {shape}')
+  for axis, (have, want) in enumerate(zip(x.shape, shape)):
+    if have == want:
+      continue
+    if have == 0 or want % have:
+      raise ValueError(f'Cannot broadcast between {tuple(x.shape)} {shape}')
+    x = x.repeat_interleave(want // have, dim=axis) if have != 1 else x.expand(*[want if a == axis else d for a, d in enumerate(x.shape)])
+  return x
+
+
+def broadcast_to(operand, target_shape):
+  """qarray.py:447-467 for arrays and QArrays.  The values are repeated tile-wise; scale and zero point grow
+  only where they were finer than per-tensor along a growing axis (each element keeps its own scale, the
+  scale stays as small as it can), where the reference materialises them at the full target shape."""
+  target_shape = tuple(int(d) for d in target_shape)
+  if tuple(operand.shape) == target_shape:
+    return operand
+  if not isinstance(operand, QArray):
+    return _broadcast_tensor(operand, target_shape)
+  if isinstance(operand.qvalue, Int4Tensor):
+    raise NotImplementedError('broadcasting packed int4 values is not supported')
+  qs = tuple(operand.shape)
+  if len(qs) != len(target_shape):
+    raise ValueError(f'Cannot broadcast between {qs} {target_shape}')
+
+  def small(x):
+    if x is None:
+      return None
+    want = tuple(k if (s == t or k == 1) else k * (t // s) for k, s, t in zip(x.shape, qs, target_shape))
+    return _broadcast_tensor(x, want).contiguous()
+
+  return QArray(_broadcast_tensor(operand.qvalue, target_shape).contiguous(), small(operand.scale),
+                small(operand.zero_point), operand.qtype)
 
 
 # ------------------------------------------------------------------------------------------

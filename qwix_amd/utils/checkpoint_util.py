@@ -88,20 +88,10 @@ def load_nested_safetensors(path: str, device='cpu', rename_rules=None) -> dict:
 def broadcast_to(x: torch.Tensor, shape) -> torch.Tensor:
   """Tile-wise broadcast (qarray.py:447-467): an axis of size s grows to a multiple t*s by repeating
   each element t times, so a (4, 4) block scale of a 128 x 128 weight becomes (4, 128)."""
-  shape = tuple(shape)
-  if tuple(x.shape) == shape:
-    return x
-  if x.ndim < len(shape):
-    x = x.reshape((1,) * (len(shape) - x.ndim) + tuple(x.shape))
-  if x.ndim != len(shape):
-    raise ValueError(f'cannot broadcast {tuple(x.shape)} to {shape}')
-  for axis, (have, want) in enumerate(zip(x.shape, shape)):
-    if have == want:
-      continue
-    if have == 0 or want % have:
-      raise ValueError(f'cannot broadcast {tuple(x.shape)} to {shape}')
-    x = x.repeat_interleave(want // have, dim=axis)
-  return x
+  try:
+    return qarray._broadcast_tensor(x, tuple(shape))
+  except ValueError:
+    raise ValueError(f'cannot broadcast {tuple(x.shape)} to {tuple(shape)}') from None
 
 
 def _validate_prequantized_dict(checkpoint_param, path) -> None:

@@ -201,3 +201,81 @@ def test_reference_output_dtype_table_by_execution():
       for o in outs:
         assert o.dtype == want, (l, r, pet, o.dtype)
         assert tuple(o.shape) == (10, 10) and torch.all(o.float() == 10).item(), (l, r, pet)
+
+
+@pytest.mark.parametrize('einsum_str,explicit,lshape,rshape', [
+    ('a b c, b c d -> a d', 'abc,bcd->ad', (10, 256, 16), (256, 16, 128)),       # einsum_test.py:176-182
+    ('...ab,...bc->...ac', 'xab,xbc->xac', (10, 256, 16), (10, 16, 128)),        # :183-190
+    ('...ab,bc->...ac', 'xab,bc->xac', (10, 256, 16), (16, 128)),                # :191-198
+    ('abc,bcd->acd', 'abc,bcd->acd', (10, 256, 16), (256, 16, 128)),             # :199-207
+])
+def test_reference_einsum_strings_bit_exact(einsum_str, explicit, lshape, rshape):
+  """The einsum strings of the reference's own einsum test (spaces, ellipses, a shared kept axis), int8 per
+  channel: bit-exact against the oracle run on the equivalent explicit string."""
+  from qwix_amd.core import einsum as es
+  xq, wq, oxq, owq = _quantize_both(explicit, lshape, rshape, O.BF16, seed=91)
+  out = es.einsum(einsum_str, xq, wq)
+  want = O.einsum(explicit, oxq, owq)
+  assert tuple(out.shape) == tuple(want.v.shape)
+  assert np.array_equal(util.f32np(out), want.v)
+
+
+def test_einsum_asymmetric_subchannel_lhs():
+  """einsum_test.py:208-217: 'abc,bcd->acd' with a minmax lhs and tiles of a quarter of the contracted axis
+  (64 < 128: the dequantize-first path, over slices of the shared kept axis)."""
+  from qwix_amd.core import einsum as es, qarray
+  x_np, x_t = util.make((10, 256, 16), O.BF16, seed=92)
+  x_np = O.round_to_bf16(x_np + np.float32(1.0))
+  x_t = torch.from_numpy(x_np).to(torch.bfloat16).to(util.DEV)
+  w_np, w_t = util.make((256, 16, 128), O.BF16, seed=93)
+  nd = (3, 3)
+  hl = es.get_how_to_quantize(einsum_str='abc,bcd->acd', ndims=nd, for_lhs=True, tile_size=1 / 4, qtype='int8',
+                              calibration_method='minmax')
+  hr = es.get_how_to_quantize(einsum_str='abc,bcd->acd', ndims=nd, for_lhs=False, tile_size=1 / 4, qtype='int8')
+  out = es.einsum('abc,bcd->acd', qarray.quantize(x_t, hl), qarray.quantize(w_t, hr))
+  ref = np.einsum('abc,bcd->acd', x_np.astype(np.float64), w_np.astype(np.float64))
+  assert tuple(out.shape) == (10, 16, 128) and out.dtype == torch.bfloat16
+  assert np.abs(util.f32np(out) - ref).mean() / np.abs(ref).mean() < 0.012
+
+
+@pytest.mark.parametrize('einsum_str,lshape,rshape,expected', [
+    ('BTNH,BSNH->BTNS', (1, 2, 4, 8), (1, 3, 1, 8), (1, 2, 4, 3)),   # einsum_test.py:332-339: size-1 broadcast
+    ('BTNH,BSNH->BTNS', (1, 2, 4, 8), (1, 3, 8, 8), (1, 2, 8, 3)),   # :340-347: 4 heads against 8
+    ('BTNH,BSNH->BTNS', (1, 2, 8, 8), (1, 3, 4, 8), (1, 2, 8, 3)),   # :348-355
+    ('bth,thk->btk', (2, 3, 4), (3, 4, 5), (2, 3, 5)),               # :356-362
+])
+def test_einsum_generic_broadcasting(einsum_str, lshape, rshape, expected):
+  """Operands whose shared axes differ by a whole factor are repeated tile-wise first (einsum_info.py:197-241)."""
+  from qwix_amd.core import einsum as es, qarray
+  _, lhs = util.make(lshape, O.F32, seed=94)
+  _, rhs = util.make(rshape, O.F32, seed=95)
+  out = es.einsum(einsum_str, lhs, rhs)
+  assert tuple(out.shape) == expected
+  subs = einsum_str.split('->')[0].split(',')
+  size = {}
+  for sub, shp in zip(subs, (lshape, rshape)):
+    for ch, d in zip(sub, shp):
+      size[ch] = max(size.get(ch, 1), d)
+  grow = lambda t, sub: qarray.broadcast_to(t, tuple(size[c] for c in sub))
+  want = torch.einsum(einsum_str, grow(lhs, subs[0]), grow(rhs, subs[1]))
+  assert torch.allclose(out, want, rtol=1e-5, atol=1e-5)
+  # quantized operands broadcast the same way
+  ql = qarray.quantize(lhs, qarray.HowToQuantize(qtype='int8', channelwise_axes=list(range(len(lshape) - 1))))
+  qo = es.einsum(einsum_str, ql, rhs)
+  assert tuple(qo.shape) == expected
+  assert ((qo - want).abs().mean() / want.abs().mean()).item() < 0.02
+
+
+def test_einsum_mixed_operands_scalar_and_incompatible_shapes():
+  """einsum_test.py:363-383 (a quantized lhs with a float rhs, a scalar rhs) and :443-448."""
+  from qwix_amd.core import einsum as es, qarray
+  _, lhs = util.make((128, 128), O.F32, seed=96)
+  _, rhs = util.make((128, 32), O.F32, seed=97)
+  ql = qarray.quantize(lhs, qarray.HowToQuantize(qtype='int8'))
+  out = es.einsum('ij,jk->ik', ql, rhs)
+  want = lhs @ rhs
+  assert tuple(out.shape) == (128, 32) and ((out - want).abs().mean() / want.abs().mean()).item() < 0.02
+  out = es.einsum('ij,->ij', ql, torch.tensor(2.0, device=util.DEV))
+  assert tuple(out.shape) == (128, 128) and ((out - 2 * lhs).abs().mean() / (2 * lhs).abs().mean()).item() < 0.02
+  with pytest.raises(ValueError, match='Cannot broadcast'):
+    es.einsum('BTNH,BSNH->BTNS', torch.ones(1, 2, 3, 8, device=util.DEV), torch.ones(1, 3, 4, 8, device=util.DEV))
