@@ -129,6 +129,149 @@ class QArray:
     return self.transpose(*axes)
 
   T = property(lambda self: self.transpose())
+  mT = property(lambda self: self.swapaxes(-1, -2))
+
+  def reshape(self, *new_shape) -> 'QArray':
+    return reshape(self, *new_shape)
+
+  def __getitem__(self, idx) -> 'QArray':
+    return rewriting_take(self, idx)
+
+
+def _shape_groups(old: Sequence[int], new: Sequence[int]) -> list[tuple[tuple[int, ...], tuple[int, ...]]]:
+  """Cuts both shapes into the shortest runs of equal size, e.g. (2, 2, 6) -> (4, 1, 3, 2) gives
+  (2, 2)->(4,), ()->(1,), (6,)->(3, 2).  On a tie the old shape advances first unless its next entry is
+  the larger one (qarray.py:117-146)."""
+  groups, run_old, run_new = [], [], []
+  size_old = size_new = 1
+  i = j = 0
+  while i < len(old) or j < len(new):
+    if size_old < size_new:
+      from_old = True
+    elif size_old > size_new:
+      from_old = False
+    else:
+      from_old = i < len(old) and (j >= len(new) or old[i] <= new[j])
+    if from_old:
+      if i >= len(old):
+        break
+      run_old.append(old[i])
+      size_old *= old[i]
+      i += 1
+    else:
+      if j >= len(new):
+        break
+      run_new.append(new[j])
+      size_new *= new[j]
+      j += 1
+    if size_old == size_new:
+      groups.append((tuple(run_old), tuple(run_new)))
+      run_old, run_new, size_old, size_new = [], [], 1, 1
+  if run_old or run_new or i < len(old) or j < len(new):
+    raise ValueError(f'Cannot reshape {tuple(old)} into {tuple(new)}.')
+  return groups
+
+
+def reshape(array: QArray, *new_shape) -> QArray:
+  """qarray.py:106-171: reshapes values, scale and zero point together, which is possible when every run of
+  axes that is regrouped is either matched exactly by the scale, per-tensor in it, or channelwise on its
+  first axis only (that axis must then divide the first new axis)."""
+  if len(new_shape) == 1 and not isinstance(new_shape[0], int):
+    new_shape = tuple(new_shape[0])
+  new_shape = tuple(int(d) for d in new_shape)
+  old_shape = tuple(array.shape)
+  if math.prod(old_shape) != math.prod(new_shape):
+    raise ValueError(f'Cannot reshape {old_shape} into {new_shape}.')
+  groups = _shape_groups(old_shape, new_shape)
+
+  def target(x_shape: tuple[int, ...]) -> list[int]:
+    out, at = [], 0
+    for old, new in groups:
+      have = tuple(x_shape[at:at + len(old)])
+      n = math.prod(have)
+      if have == old:
+        out.extend(new)
+      elif n == 1:
+        out.extend([1] * len(new))
+      elif n == have[0] and new[0] % have[0] == 0:
+        out.extend([have[0]] + [1] * (len(new) - 1))
+      else:
+        raise ValueError(f'Cannot reshape {old_shape} into {new_shape} for {tuple(x_shape)}.')
+      at += len(old)
+    return out
+
+  q = array.qvalue
+  if isinstance(q, Int4Tensor):
+    if q.packed_axis != len(old_shape) - 1 or not q.data.is_contiguous() or not new_shape or new_shape[-1] % 2:
+      raise NotImplementedError('int4 values reshape only in the natural layout and to an even last dimension')
+    qv = Int4Tensor(q.data.reshape(*new_shape[:-1], new_shape[-1] // 2), new_shape, len(new_shape) - 1)
+  else:
+    qv = q.reshape(target(old_shape))
+  zp = None if array.zero_point is None else array.zero_point.reshape(target(tuple(array.zero_point.shape)))
+  return QArray(qv, array.scale.reshape(target(tuple(array.scale.shape))), zp, array.qtype)
+
+
+def rewriting_take(array: QArray, idx) -> QArray:
+  """array[idx] (qarray.py:174-209): integers, slices, None and one Ellipsis.  Scale and zero point follow:
+  a per-tensor axis keeps its single entry, an integer on a tiled axis picks that element's tile; a partial
+  slice of a tiled axis is refused."""
+  idx = list(idx) if isinstance(idx, (tuple, list)) else [idx]
+  named = sum(1 for it in idx if it is not None and it is not Ellipsis)
+  fill = [slice(None)] * (array.ndim - named)
+  if any(it is Ellipsis for it in idx):
+    at = [k for k, it in enumerate(idx) if it is Ellipsis]
+    if len(at) != 1:
+      raise ValueError('an index can hold a single Ellipsis')
+    idx[at[0]:at[0] + 1] = fill
+  else:
+    idx += fill
+  shape = tuple(array.shape)
+
+  def component_index(x_shape) -> tuple:
+    out, k = [], 0
+    for full, have in zip(shape, x_shape):
+      while idx[k] is None:
+        out.append(None)
+        k += 1
+      it = idx[k]
+      whole = isinstance(it, slice) and it == slice(None)
+      if full == have or whole:
+        out.append(it)
+      elif have == 1:
+        out.append(0 if isinstance(it, int) else slice(None))
+      elif isinstance(it, int):
+        out.append((it % full) // (full // have))
+      else:
+        raise ValueError(f'Unsupported indexing {idx} for {shape}.')
+      k += 1
+    out.extend(idx[k:])
+    return tuple(out)
+
+  q = array.qvalue
+  if isinstance(q, Int4Tensor):
+    ci = component_index(shape)
+    ax_items = [it for it in ci if it is not None]
+    if not (isinstance(ax_items[q.packed_axis], slice) and ax_items[q.packed_axis] == slice(None)):
+      raise NotImplementedError('the packed axis of int4 values can only be taken whole')
+    data = q.data[ci]
+    new_shape, packed, pos, src = [], None, 0, 0
+    for it in ci:
+      if it is None:
+        new_shape.append(1)
+        pos += 1
+        continue
+      if not isinstance(it, int):
+        if src == q.packed_axis:
+          packed = pos
+        new_shape.append(data.shape[pos] * (2 if src == q.packed_axis else 1))
+        pos += 1
+      src += 1
+    qv = Int4Tensor(data, new_shape, packed)
+  else:
+    qv = q[component_index(shape)]
+  zp = None if array.zero_point is None else array.zero_point[component_index(tuple(array.zero_point.shape))]
+  return QArray(qv, array.scale[component_index(tuple(array.scale.shape))], zp, array.qtype)
+
 
 
 @dataclasses.dataclass(frozen=True, kw_only=True)

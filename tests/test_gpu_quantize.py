@@ -289,3 +289,16 @@ def test_static_scale_with_overflowing_quotients(qtype):
     qa = qarray.quantize_with_scale_zero_point(x_t, qtype, util.to_gpu(scale_np, O.BF16), None)
     want = O.quantize_with_scale_zero_point(O.FArr(x_np, O.BF16), qtype, O.FArr(scale_np, O.BF16), None)
     util.assert_qarray_equal(qa, want, f'static scale {s}')
+
+
+def test_array_methods_commute_with_dequantize():
+  """qarray_test.py:244-283: dequantize(q.reshape(...)) == dequantize(q).reshape(...), and the same for a slice."""
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make((2, 2, 6), O.F32, seed=73)
+  q = qarray.quantize(x_t, qarray.HowToQuantize(qtype='int8', channelwise_axes=[0], tiled_axes={2: 2}))
+  assert tuple(q.scale.shape) == (2, 1, 3)
+  full = qarray.dequantize(q)
+  assert torch.equal(qarray.dequantize(q.reshape(4, 1, 3, 2)), full.reshape(4, 1, 3, 2))
+  assert torch.equal(qarray.dequantize(q[..., 1]), full[..., 1])
+  assert torch.equal(qarray.dequantize(q[1]), full[1])
+  assert torch.equal(qarray.dequantize(q.transpose(1, 2, 0)), full.permute(1, 2, 0))

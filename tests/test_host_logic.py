@@ -171,3 +171,45 @@ def test_rule_lookup_first_full_match_wins_and_op_ids():
   assert [r.module_path for r in p.get_unused_rules()] == ['never']
   r = qconfig.QuantizationRule()
   assert (r.module_path, r.weight_qtype, r.act_qtype, r.tile_size, r.weight_calibration_method, tuple(r.act_batch_axes)) == ('.*', None, None, None, 'absmax', (0,))
+
+
+def test_qarray_array_methods_follow_the_reference_table():
+  """qarray_test.py:228-302: scale shapes under reshape / transpose / slicing of a (2, 2, 6) array quantized
+  channelwise on axis 0 with tiles of 2 on axis 2 (scale (2, 1, 3))."""
+  import torch
+  from qwix_amd.core import qarray
+  q = qarray.QArray(torch.arange(24, dtype=torch.int8).reshape(2, 2, 6),
+                    torch.arange(1, 7, dtype=torch.float32).reshape(2, 1, 3), None, 'int8')
+  assert q.shape == (2, 2, 6) and q.ndim == 3
+  assert q.scale_tile_shape == (1, 2, 2) and q.zero_point_tile_shape is None
+  r = q.reshape(4, 1, 3, 2)
+  assert tuple(r.shape) == (4, 1, 3, 2) and tuple(r.scale.shape) == (2, 1, 3, 1)
+  assert tuple(q.reshape(2, 1, 2, 6).scale.shape) == (2, 1, 1, 3)
+  assert tuple(q.reshape(1, 4, 6).scale.shape) == (1, 2, 3)
+  assert tuple(r.reshape(4, 6).scale.shape) == (2, 3)
+  assert tuple(q.reshape((4, 6)).shape) == (4, 6) and tuple(q.reshape((4, 6)).scale.shape) == (2, 3)
+  with pytest.raises(ValueError):  # (2, 2, 6) -> (12, 2) would merge the tiled axis
+    q.reshape(12, 2)
+  with pytest.raises(ValueError):
+    q.reshape(5, 5)
+  with pytest.raises(ValueError):  # the tiled axis cannot be merged with its neighbour
+    qarray.QArray(torch.zeros(2, 2, 6, dtype=torch.int8), torch.ones(1, 2, 2), None, 'int8').reshape(4, 6)
+  t = q.transpose(1, 2, 0)
+  assert tuple(t.shape) == (2, 6, 2) and tuple(t.scale.shape) == (1, 3, 2)
+  assert tuple(q.T.shape) == (6, 2, 2) and tuple(q.T.scale.shape) == (3, 1, 2)
+  assert tuple(q.mT.shape) == (2, 6, 2) and tuple(q.mT.scale.shape) == (2, 3, 1)
+  s = q[..., 1]
+  assert tuple(s.shape) == (2, 2) and tuple(s.scale.shape) == (2, 1)
+  assert torch.equal(s.qvalue, q.qvalue[..., 1]) and torch.equal(s.scale, q.scale[..., 0])
+  assert tuple(q[0:1, 1:2, 4].scale.shape) == (1, 1) and q[0:1, 1:2, 4].scale.item() == 3.0
+  assert tuple(q[0].scale.shape) == (1, 3)
+  assert tuple(q[..., None].scale.shape) == (2, 1, 3, 1)
+  assert tuple(q[None].scale.shape) == (1, 2, 1, 3)
+  with pytest.raises(ValueError, match='Unsupported indexing'):
+    q[:, :, 1:3]
+  sw = q.swapaxes(1, 2)
+  assert tuple(sw.shape) == (2, 6, 2) and tuple(sw.scale.shape) == (2, 3, 1)
+  assert q.astype(torch.bfloat16).scale.dtype == torch.bfloat16
+  with pytest.raises(ValueError):
+    qarray.validate_qarray(qarray.QArray(torch.ones(10, 10, dtype=torch.int8), torch.ones(10, 3), None, 'int8'))
+  assert qarray.get_tiled_axes(qarray.QArray(torch.ones(10, 256, 16, dtype=torch.int8), torch.ones(10, 8, 2))) == {1: 32, 2: 8}
