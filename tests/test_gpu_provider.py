@@ -143,6 +143,38 @@ def test_small_tile_rule_takes_the_dequantize_path():
   assert np.allclose(util.f32np(out), want.v, rtol=1e-5, atol=1e-6)
 
 
+def test_two_dim_tile_rule():
+  """ptq_test.py:698-730: tile_size given as a mapping {0: 2, 1: 2} is used verbatim: an (8, 16) kernel gets
+  (4, 8) scales, through Dense and through an einsum, and the weight-only forward dequantizes per block."""
+  import qwix_amd
+  from qwix_amd import nn
+  layer = nn.Dense(16, name='Dense_0')
+  g = torch.Generator().manual_seed(7)
+  params = layer.init(g, 8, torch.float32, util.DEV, std=1.0)
+  x = torch.ones(2, 8, device=util.DEV)
+  rules = [qwix_amd.QuantizationRule(weight_qtype='int8', tile_size={0: 2, 1: 2})]
+  pm = qwix_amd.quantize_model(lambda p, x: layer(p, x), qwix_amd.PtqProvider(rules))
+  qp = pm.init(params, x)
+  assert tuple(qp['kernel'].array.scale.shape) == (4, 8)
+  out = pm.apply(qp, x)
+  assert tuple(out.shape) == (2, 16)
+  how = O.HowToQuantize(qtype='int8', tiled_axes={0: 2, 1: 2})
+  ow = O.quantize(util.farr(params['kernel']), how)
+  util.assert_qarray_equal(qp['kernel'].array, ow, '2 x 2 block weight')
+  want = O.dot_general(util.farr(x), ow, DN)
+  bias = util.f32np(params['bias']) if 'bias' in params else 0.0
+  assert np.allclose(util.f32np(out), want.v + bias, rtol=1e-5, atol=1e-6)
+
+  ein = nn.Einsum('ij,jk->ik', (8, 16))
+  eparams = ein.init(g, torch.float32, util.DEV)
+  pm = qwix_amd.quantize_model(lambda p, x: ein(p, x), qwix_amd.PtqProvider(rules))
+  qp = pm.init(eparams, x)
+  assert tuple(qp['kernel'].array.scale.shape) == (4, 8)
+  out = pm.apply(qp, x)
+  want = O.dot_general(util.farr(x), O.quantize(util.farr(eparams['kernel']), how), DN)
+  assert tuple(out.shape) == (2, 16) and np.allclose(util.f32np(out), want.v, rtol=1e-5, atol=1e-6)
+
+
 def test_ptq_mlp_forward_replays_from_a_hip_graph():
   """The launch-bound configuration (four small kernels per forward) captured once and replayed: no entry
   point allocates or synchronises, so the whole quantized forward is graph-safe.  Every replay, with the
