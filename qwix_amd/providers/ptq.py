@@ -20,6 +20,7 @@ from typing import Any, Callable, Generic, Mapping, Sequence, TypeVar
 
 import torch
 
+from qwix_amd import averaging
 from qwix_amd import qconfig
 from qwix_amd.core import dot_general as _dot_general
 from qwix_amd.core import einsum as _einsum
@@ -77,16 +78,39 @@ def create_quantized_param(param: Param, how: _qarray.HowToQuantize, *, _qarray_
 
 
 def quantize_act(array: torch.Tensor, how: _qarray.HowToQuantize, rule: qconfig.QuantizationRule, act_name: str, *,
-                 quant_stats: Mapping[str, Any] | None = None, _qarray_module=_qarray) -> _qarray.QArray:
-  """Dynamic-range: one fused quantize.  Static-range (rule.act_static_scale): scale / zero point
-  come from `quant_stats[act_name + '_scale' / '_zero_point']` computed offline."""
+                 store: dict | None = None, quant_stats: Mapping[str, Any] | None = None,
+                 _qarray_module=_qarray) -> _qarray.QArray:
+  """boxed_param.py:416-455.  Dynamic range: one fused quantize.  Static range (rule.act_static_scale): the
+  scale is a parameter `<act_name>_scale` (a WithAux, so that quantize_params can read the qtype; plus
+  `<act_name>_zero_point` for asymmetric methods) of the module that issues the op.  When it does not
+  exist yet it is created: from collected statistics `quant_stats[act_name]` ({'count', 'sum_of_*'}) if
+  there are any, else from the calibration of this very input averaged over rule.act_batch_axes.
+  `store` is the module's param dict; ops without one (two activations) use `quant_stats` itself, where a
+  precomputed `<act_name>_scale` may also be supplied directly."""
   if not rule.act_static_scale:
     return _qarray_module.quantize(array, how)
-  if quant_stats is None or act_name + '_scale' not in quant_stats:
-    raise ValueError(f'static-range quantization of {act_name!r} needs a precomputed {act_name}_scale')
-  scale = quant_stats[act_name + '_scale']
+  where = store if store is not None else quant_stats
+  if where is None:
+    raise ValueError(f'static-range quantization of {act_name!r} needs a param store or quant_stats')
+  name = act_name + '_scale'
+  if name not in where and quant_stats is not None and name in quant_stats:
+    where = quant_stats  # a scale computed offline and handed to the provider
+  if name not in where:
+    stat = None if quant_stats is None else quant_stats.get(act_name)
+    if isinstance(stat, Mapping) and 'count' in stat:
+      calibration = averaging.SimpleMovingAverage().get_calibration(stat)
+      calibration = {k: v.to(array.dtype) for k, v in calibration.items()}
+    else:
+      calibration = _qarray_module.calibrate(array, how)
+      axes = [a for a in rule.act_batch_axes]
+      calibration = {k: v.to(torch.float32).mean(dim=axes, keepdim=True).to(v.dtype) for k, v in calibration.items()}
+    scale, zp = _qarray_module.compute_scale_zero_point(calibration, how.qtype)
+    where[name] = WithAux(scale, how)
+    if zp is not None:
+      where[act_name + '_zero_point'] = zp
+  scale = where[name]
   scale = scale.array if isinstance(scale, WithAux) else scale
-  zp = quant_stats.get(act_name + '_zero_point')
+  zp = where.get(act_name + '_zero_point')
   return _qarray_module.quantize_with_scale_zero_point(array, how.qtype, scale, zp)
 
 
@@ -105,6 +129,7 @@ class BoxedParamProvider(qconfig.QuantizationProvider):
 
   # -- helpers
   def _prepare(self, lhs, rhs, rule, op_id, get_how, quantize_lhs: bool = True):
+    store = rhs.store if isinstance(rhs, Param) else None  # the issuing module's params: static scales live there
     if isinstance(rhs, WithAux):
       rhs = rhs.array
     elif isinstance(rhs, Param):
@@ -115,10 +140,12 @@ class BoxedParamProvider(qconfig.QuantizationProvider):
         rhs = create_quantized_param(rhs, how, _qarray_module=self._qarray_module).array
     elif rule.act_qtype is not None:
       how = get_how(for_lhs=False, qtype=rule.act_qtype, calibration_method=rule.act_calibration_method or 'absmax')
-      rhs = quantize_act(rhs, how, rule, op_id + '_rhs', quant_stats=self.quant_stats, _qarray_module=self._qarray_module)
+      rhs = quantize_act(rhs, how, rule, op_id + '_rhs', store=store, quant_stats=self.quant_stats,
+                         _qarray_module=self._qarray_module)
     if rule.act_qtype is not None and quantize_lhs:
       how = get_how(for_lhs=True, qtype=rule.act_qtype, calibration_method=rule.act_calibration_method or 'absmax')
-      lhs = quantize_act(lhs, how, rule, op_id + '_lhs', quant_stats=self.quant_stats, _qarray_module=self._qarray_module)
+      lhs = quantize_act(lhs, how, rule, op_id + '_lhs', store=store, quant_stats=self.quant_stats,
+                         _qarray_module=self._qarray_module)
     return lhs, rhs
 
   def _fusable(self, rule) -> bool:
@@ -204,7 +231,6 @@ def quantize_params(params: Mapping, abstract_quantized_params: Mapping, quant_s
   are reshaped to the template's shape and quantized with `_qarray_module.quantize`; other leaves
   are passed through; leaves missing from the template raise unless allow_extra_params.
   """
-  del quant_stats  # static-range statistics are applied by the provider (quant_stats attribute)
   abstract = _flatten(abstract_quantized_params)
   out = {}
   for path, param in _flatten(params).items():
@@ -219,4 +245,21 @@ def quantize_params(params: Mapping, abstract_quantized_params: Mapping, quant_s
       param = param.reshape(tmpl.shape)
       param = tmpl.replace(array=_qarray_module.quantize(param, tmpl.how))
     out[path] = param
+  # Static-range activations (ptq.py:106-129): scale and zero point from the collected statistics
+  # {module path...: {<act_name>: {'count', 'sum_of_absmax' | 'sum_of_min', 'sum_of_max'}}}.
+  stats = _flatten(quant_stats or {})
+  for path in sorted({p[:-1] for p in stats}):
+    stat = {p[-1]: v for p, v in stats.items() if p[:-1] == path}
+    if int(stat['count']) == 0:
+      raise ValueError(f'quant_stats is not initialized for {path}.')
+    scale_path = path[:-1] + (path[-1] + '_scale',)
+    tmpl = abstract.get(scale_path)
+    if not isinstance(tmpl, WithAux):
+      raise ValueError(f'{scale_path} is not a static scale of the abstract_quantized_params.')
+    calibration = averaging.SimpleMovingAverage().get_calibration(stat)
+    calibration = {k: v.to(tmpl.array.dtype) for k, v in calibration.items()}
+    scale, zero_point = _qarray_module.compute_scale_zero_point(calibration, tmpl.how.qtype)
+    out[scale_path] = tmpl.replace(array=scale)
+    if zero_point is not None:
+      out[path[:-1] + (path[-1] + '_zero_point',)] = zero_point
   return _unflatten(out)

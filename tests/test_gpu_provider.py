@@ -175,6 +175,67 @@ def test_two_dim_tile_rule():
   assert tuple(out.shape) == (2, 16) and np.allclose(util.f32np(out), want.v, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize('method', ['absmax', 'minmax'])
+def test_static_range_rule_end_to_end(method):
+  """ptq_test.py:86-143 without the training-time provider: statistics collected over three batches
+  ({'count', 'sum_of_*'}, averaging.py:38-64), the PTQ model's abstract params hold `dot_general0_lhs_scale`
+  as a (1, 1) WithAux (plus `_zero_point` for minmax), quantize_params turns the statistics into scale and
+  zero point (ptq.py:106-129), and the forward uses them; every stage is checked against the oracle."""
+  import qwix_amd
+  from qwix_amd import averaging, nn
+  from qwix_amd.core import qarray
+  from qwix_amd.providers import ptq
+  dense = nn.Dense(5, name='Dense_0')
+  g = torch.Generator().manual_seed(8)
+  params = dense.init(g, 12, torch.float32, util.DEV, std=1.0)
+  rules = [qwix_amd.QuantizationRule(module_path='.*', weight_qtype='int8', act_qtype='int8', act_static_scale=True,
+                                     act_calibration_method=method)]
+  how = qarray.HowToQuantize(qtype='int8', channelwise_axes=[0], calibration_method=method)
+  agg = averaging.SimpleMovingAverage()
+  stat, batches = None, []
+  for _ in range(3):
+    xb = (torch.randn(10, 12, generator=g) + 0.3).to(util.DEV)
+    batches.append(xb)
+    cal = {k: v.mean(dim=0, keepdim=True) for k, v in qarray.calibrate(xb, how).items()}  # act_batch_axes = (0,)
+    stat = agg.init(cal) if stat is None else stat
+    assert stat['count'].shape == () and all(v.shape == (1, 1) for k, v in stat.items() if k != 'count')
+    stat = agg.update(stat, cal)
+  assert int(stat['count']) == 3
+  with pytest.raises(ValueError, match='Shape mismatch'):
+    agg.update(stat, {k: v.reshape(1) for k, v in cal.items()})
+
+  x = batches[0]
+  pm = qwix_amd.quantize_model(lambda p, x: dense(p, x), qwix_amd.PtqProvider(rules))
+  abstract = pm.init(params, x)
+  assert isinstance(abstract['dot_general0_lhs_scale'], ptq.WithAux)
+  assert abstract['dot_general0_lhs_scale'].array.shape == (1, 1)
+  if method == 'minmax':
+    assert abstract['dot_general0_lhs_zero_point'].shape == (1, 1)
+  with pytest.raises(ValueError, match='not initialized'):
+    qwix_amd.quantize_params(params, abstract, {'dot_general0_lhs': agg.init(cal)})
+  qp = qwix_amd.quantize_params(params, abstract, {'dot_general0_lhs': stat})
+  assert set(qp) == set(abstract)
+
+  # the oracle's side of the same computation
+  keys = ['absmax'] if method == 'absmax' else ['min', 'max']
+  avg = {k: O.FArr((util.f32np(stat['sum_of_' + k]) / np.float32(3)).astype(np.float32), O.F32) for k in keys}
+  oscale, ozp = O.compute_scale_zero_point(avg, 'int8')
+  assert np.array_equal(util.f32np(qp['dot_general0_lhs_scale'].array), oscale.v)
+  if method == 'minmax':
+    assert np.array_equal(qp['dot_general0_lhs_zero_point'].cpu().numpy(), ozp)
+  out = pm.apply(qp, x)
+  oxq = O.quantize_with_scale_zero_point(util.farr(x), 'int8', oscale, ozp)
+  owq = O.quantize(util.farr(params['kernel']), O.HowToQuantize(qtype='int8', channelwise_axes=[1]))
+  util.assert_qarray_equal(qp['kernel'].array, owq, 'weight')
+  want = O.dot_general(oxq, owq, DN)
+  bias = util.f32np(params['bias']) if 'bias' in params else np.float32(0)
+  assert np.allclose(util.f32np(out), want.v + bias, rtol=1e-6, atol=1e-6)
+  # without statistics the scale comes from the first input itself
+  first = pm.init(params, x)['dot_general0_lhs_scale'].array
+  cal0 = {k: O.FArr(util.f32np(v.mean(dim=0, keepdim=True)), O.F32) for k, v in qarray.calibrate(x, how).items()}
+  assert np.allclose(util.f32np(first), O.compute_scale_zero_point(cal0, 'int8')[0].v, rtol=1e-6)
+
+
 def test_ptq_mlp_forward_replays_from_a_hip_graph():
   """The launch-bound configuration (four small kernels per forward) captured once and replayed: no entry
   point allocates or synchronises, so the whole quantized forward is graph-safe.  Every replay, with the

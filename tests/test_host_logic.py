@@ -213,3 +213,26 @@ def test_qarray_array_methods_follow_the_reference_table():
   with pytest.raises(ValueError):
     qarray.validate_qarray(qarray.QArray(torch.ones(10, 10, dtype=torch.int8), torch.ones(10, 3), None, 'int8'))
   assert qarray.get_tiled_axes(qarray.QArray(torch.ones(10, 256, 16, dtype=torch.int8), torch.ones(10, 8, 2))) == {1: 32, 2: 8}
+
+
+def test_simple_moving_average_statistics():
+  """averaging.py:38-99: float32 sums whatever the calibration dtype, plain average, the default calibration
+  while no more than bootstrap_steps samples have been seen."""
+  import torch
+  from qwix_amd import averaging
+  agg = averaging.SimpleMovingAverage()
+  cal = {'min': torch.tensor([[-1.0]], dtype=torch.bfloat16), 'max': torch.tensor([[3.0]], dtype=torch.bfloat16)}
+  stat = agg.init(cal)
+  assert stat['count'].dtype == torch.int32 and int(stat['count']) == 0
+  assert stat['sum_of_min'].dtype == torch.float32 and stat['sum_of_max'].shape == (1, 1)
+  stat = agg.update(stat, cal)
+  stat = agg.update(stat, {'min': torch.tensor([[-3.0]], dtype=torch.bfloat16), 'max': torch.tensor([[4.0]], dtype=torch.bfloat16)})
+  got = agg.get_calibration(stat)
+  assert int(stat['count']) == 2 and got['min'].item() == -2.0 and got['max'].item() == 3.5
+  with pytest.raises(ValueError, match='Shape mismatch'):
+    agg.update(stat, {'min': torch.zeros(2, 1), 'max': torch.zeros(2, 1)})
+  boot = averaging.SimpleMovingAverage(bootstrap_steps=2)
+  assert boot.get_calibration(stat, cal)['max'].item() == 3.0            # 2 samples: still the default
+  stat = agg.update(stat, cal)
+  out = boot.get_calibration(stat, cal)
+  assert out['max'].dtype == torch.bfloat16 and abs(out['max'].item() - 10.0 / 3) < 0.02
