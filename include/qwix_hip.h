@@ -78,6 +78,14 @@ QWIX_API int qwix_hip_calibrate(const void* x, int dtype, int64_t outer, int64_t
                        int64_t tile, int calibration, float calib_factor, void* out0,
                        void* out1, void* workspace, size_t workspace_bytes, void* stream);
 
+/* calibrate with the 'rms,s' method (qwix/_src/core/qarray.py:511-515): out[group] =
+ * D(D(sqrt(D(mean(D(x^2))))) * D(s)) for every scale group of the 5-D geometry of
+ * qwix_hip_quantize_generic (a single reduced group: dims = (outer, reduce, inner, 1, 1), t3 = 1).
+ * The result is an 'absmax' calibration: qwix_hip_compute_scale_zero_point turns it into a scale.
+ * The mean is summed in f32; the order of that sum is the one rounding XLA does not pin. */
+QWIX_API int qwix_hip_calibrate_rms(const void* x, int dtype, const int64_t dims[5], int64_t t1, int64_t t3,
+                           float factor, void* out, void* stream);
+
 /* compute_scale_zero_point (qarray.py:537-584) on n calibration values. */
 QWIX_API int qwix_hip_compute_scale_zero_point(const void* cal0, const void* cal1, int dtype, int64_t n,
                                       int qtype, int calibration, void* scale, void* zero_point,

@@ -9,7 +9,7 @@ What it restates (file:line refer to the google/qwix v0.1.8 source tree):
   numerics    qwix/_src/core/numerics.py:64-196      bounds, convert_to
   qarray      qwix/_src/core/qarray.py:332-349       get_scale_shape
               qwix/_src/core/qarray.py:390-444       split_axis, generic broadcast
-              qwix/_src/core/qarray.py:470-534       calibrate (absmax / minmax)
+              qwix/_src/core/qarray.py:470-534       calibrate (absmax / minmax / rms / fixed)
               qwix/_src/core/qarray.py:537-584       compute_scale_zero_point
               qwix/_src/core/qarray.py:594-644       quantize_with_scale_zero_point, quantize
               qwix/_src/core/qarray.py:647-708       quantize_api, dequantize
@@ -35,6 +35,9 @@ How each function is pinned (tests/test_oracle_*.py):
   * calibrate / scale / quantize ... reference vector qarray_test.py:191-219
     (arange(256)/255, minmax) + closed forms + brute-force Python loops on tiny
     tiled shapes + torch-CPU bf16 arithmetic as an independent implementation.
+  * calibrate 'fixed' .............. closed forms (scale exactly 1 reproduces the convert_to vectors).
+  * calibrate 'rms' ................ PARITY UNPINNED in its last bit: jnp.mean of the rounded squares is an
+    f32 sum in XLA's own order; pinned only by closed forms (constant arrays) and to one ulp.
   * integer dot ..................... exact integer arithmetic (any order agrees);
     checked against np.int64 matmul.
   * _fast == _slow == dequant-dot ... invariant of two_dim_scales_test.py:57-93.
@@ -334,7 +337,7 @@ def generic_broadcast(op, x: np.ndarray, y: np.ndarray) -> np.ndarray:
 
 
 def calibrate(array: FArr, how: HowToQuantize) -> dict[str, FArr]:
-  """qarray.py:470-534: the absmax, minmax and fixed methods (rms is not restated)."""
+  """qarray.py:470-534: the absmax, minmax, rms and fixed methods."""
   reduce_axes = []
   off = 0
   for axis in range(array.ndim):
@@ -362,6 +365,14 @@ def calibrate(array: FArr, how: HowToQuantize) -> dict[str, FArr]:
     if args:
       am = rnd(am * rnd(np.float32(args[0]), d), d)
     return {'absmax': FArr(am.reshape(shape), d)}
+  if method == 'rms':  # qarray.py:511-515.  Parity unpinned in its last bit: jnp.mean sums in f32 in XLA's own order
+    if not args:
+      raise ValueError('A scale factor is required for RMS calibration.')
+    sq = rnd(v * v, d)
+    n = np.float32(np.prod([v.shape[a] for a in ax]))
+    mean = rnd(np.sum(sq, axis=ax, keepdims=True, dtype=np.float32) / n, d)
+    rms = rnd(np.sqrt(mean), d)
+    return {'absmax': FArr(rnd(rms * rnd(np.float32(args[0]), d), d).reshape(shape), d)}
   if method == 'fixed':  # qarray.py:518-532: a constant, per-tensor range
     if len(args) not in (1, 2):
       raise ValueError('A fixed range is required for fixed calibration.')

@@ -439,11 +439,31 @@ def _fixed_calibration(method: str, array: torch.Tensor) -> dict[str, torch.Tens
   return {'min': full(args[0]), 'max': full(args[1])}
 
 
+def _rms_calibration(method: str, array: torch.Tensor, sshape, tiles) -> dict[str, torch.Tensor] | None:
+  """'rms,s' (qarray.py:511-515): an 'absmax' calibration of sqrt(mean(x^2)) * s per scale group.  None for
+  the other methods."""
+  name, *args = method.lower().split(',')
+  if name != 'rms':
+    return None
+  if not args:
+    raise ValueError('A scale factor is required for RMS calibration.')
+  array = _check_float_input(array)
+  if array.numel() == 0:
+    _check_empty_reduction(sshape)
+    return {'absmax': torch.empty(sshape, dtype=array.dtype, device=array.device)}
+  plan = _plan(tuple(array.shape), tuple(tiles))
+  dims5 = tuple(plan.dims) + (1, 1) if plan.kind == '3d' else tuple(plan.dims)
+  t1, t3 = (plan.tiles[0], 1) if plan.kind == '3d' else plan.tiles
+  import ctypes
+  out = torch.empty(sshape, dtype=array.dtype, device=array.device)
+  _lib.call('qwix_hip_calibrate_rms', array.data_ptr(), _lib.float_tag(array.dtype), (ctypes.c_int64 * 5)(*dims5), t1, t3,
+            float(args[0]), out.data_ptr(), _lib.stream_of(array))
+  return {'absmax': out}
+
+
 def _parse_calibration(method: str) -> tuple[int, float]:
   name, *args = method.lower().split(',')
   args = [float(a) for a in args]
-  if name == 'rms':
-    raise NotImplementedError('rms calibration is not part of the HIP path (absmax, minmax and fixed are)')
   if name not in ('absmax', 'minmax'):
     raise ValueError(f'Unsupported calibration: {method}')
   return (_lib.ABSMAX if name == 'absmax' else _lib.MINMAX), (args[0] if args else 0.0)
@@ -523,6 +543,9 @@ def calibrate(array: torch.Tensor, how: HowToQuantize) -> dict[str, torch.Tensor
   fixed = _fixed_calibration(how.calibration_method, array)
   if fixed is not None:
     return fixed
+  rms = _rms_calibration(how.calibration_method, array, sshape, _tiles_from_how(shape, how) if array.numel() else ())
+  if rms is not None:
+    return rms
   cal, factor = _parse_calibration(how.calibration_method)
   if array.numel() == 0:
     _check_empty_reduction(sshape)
@@ -593,6 +616,8 @@ def quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = No
   q = numerics.canonical_qtype(how.qtype)
   sshape = get_scale_shape(shape, how)
   fixed = _fixed_calibration(how.calibration_method, array)
+  if fixed is None:  # rms: its own reduction kernel, then the static-scale kernel
+    fixed = _rms_calibration(how.calibration_method, array, sshape, _tiles_from_how(shape, how) if array.numel() else ())
   if fixed is not None:  # a constant range: the static-scale kernel, with one scale for the whole array
     scale, zp = compute_scale_zero_point(fixed, q)
     return quantize_with_scale_zero_point(array, q, scale, zp, layout=layout)

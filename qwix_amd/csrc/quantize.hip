@@ -931,6 +931,39 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// rms calibration (qarray.py:511-515): sqrt(mean(x^2)) * factor per scale group, every step rounded to the
+// array dtype the way jnp does it (squares in D, the mean summed in f32 and cast to D, the root in D).  One
+// wavefront per group over the 5-D geometry; a rarely used method, kept simple rather than coalesced.
+template <typename D>
+__global__ void __launch_bounds__(256)
+    rms_kernel(const void* __restrict__ x, Geom5 g, float factor, void* __restrict__ out) {
+  const int64_t n1 = g.d[1] / g.t1, n3 = g.d[3] / g.t3;
+  const int64_t ns = g.d[0] * n1 * g.d[2] * n3 * g.d[4];
+  const int64_t si = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (si >= ns) return;
+  int64_t r = si;
+  const int64_t i4 = r % g.d[4]; r /= g.d[4];
+  const int64_t j3 = r % n3; r /= n3;
+  const int64_t i2 = r % g.d[2]; r /= g.d[2];
+  const int64_t j1 = r % n1;
+  const int64_t i0 = r / n1;
+  const int64_t count = g.t1 * g.t3;
+  float sum = 0.f;
+  for (int64_t e = lane; e < count; e += 64) {
+    const int64_t a = e / g.t3, b = e % g.t3;
+    const int64_t idx = ((((i0 * g.d[1]) + j1 * g.t1 + a) * g.d[2] + i2) * g.d[3] + j3 * g.t3 + b) * g.d[4] + i4;
+    const float v = load1<D>(x, idx);
+    sum += rnd<D>(v * v);
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, 64);
+  if (lane != 0) return;
+  const float mean = rnd<D>(sum / static_cast<float>(count));
+  const float rms = rnd<D>(__builtin_sqrtf(mean));
+  store1<D>(out, si, rnd<D>(rms * rnd<D>(factor)));
+}
+
 // ------------------------------------------------------------------------------------ misc
 template <typename D, int QT, int CAL>
 __global__ void scale_zp_kernel(const void* __restrict__ c0, const void* __restrict__ c1, int64_t n,
@@ -1536,6 +1569,29 @@ int qwix_hip_quantize_generic(const void* x, int dtype, const int64_t dims[5], i
     })
   })
   return check_launch("generic quantize");
+}
+
+int qwix_hip_calibrate_rms(const void* x, int dtype, const int64_t dims[5], int64_t t1, int64_t t3, float factor,
+                           void* out, void* stream) {
+  if (!x || !out || !dims) return fail(QWIX_ERR_INVALID_ARGUMENT, "null argument");
+  if (!(factor > 0.f)) return fail(QWIX_ERR_INVALID_ARGUMENT, "rms calibration needs a positive scale factor");
+  Geom5 g;
+  for (int i = 0; i < 5; ++i) {
+    if (dims[i] <= 0) return fail(QWIX_ERR_INVALID_ARGUMENT, "dims[%d] = %lld", i, (long long)dims[i]);
+    g.d[i] = dims[i];
+  }
+  if (t1 <= 0 || t3 <= 0 || dims[1] % t1 || dims[3] % t3)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "tiles (%lld, %lld) do not divide (%lld, %lld)", (long long)t1,
+                (long long)t3, (long long)dims[1], (long long)dims[3]);
+  g.t1 = t1;
+  g.t3 = t3;
+  const int64_t ns = dims[0] * (dims[1] / t1) * dims[2] * (dims[3] / t3) * dims[4];
+  if ((ns + 3) / 4 > INT32_MAX) return fail(QWIX_ERR_UNSUPPORTED, "too many scale groups");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  QWIX_DISPATCH_D(dtype, {
+    rms_kernel<D><<<dim3(static_cast<unsigned>((ns + 3) / 4)), 256, 0, st>>>(x, g, factor, out);
+  })
+  return check_launch("rms calibration");
 }
 
 int qwix_hip_dequantize_generic(const void* qvalue, int qtype, const int64_t dims[5], int64_t t1, int64_t t3,

@@ -162,8 +162,46 @@ def test_fixed_calibration(dtype, qtype):
   from qwix_amd.core import qarray
   with pytest.raises(ValueError):
     qarray.quantize(x_t, qarray.HowToQuantize(qtype=qtype, calibration_method='fixed,1,2'))
-  with pytest.raises(NotImplementedError):
-    qarray.quantize(x_t, qarray.HowToQuantize(qtype=qtype, calibration_method='rms,3'))
+  with pytest.raises(ValueError, match='scale factor'):
+    qarray.quantize(x_t, qarray.HowToQuantize(qtype=qtype, calibration_method='rms'))
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('shape,kw', [
+    ((64, 512), dict(channelwise_axes=[0], tiled_axes={1: 1 / 8})),   # qarray_test.py:92-100 ('rms,7', tiles of 1/8)
+    ((40, 256), dict(channelwise_axes=[0])),
+    ((256, 48), dict(channelwise_axes=[1])),                           # reduction along the strided axis
+    ((64, 64), dict(tiled_axes={0: 16, 1: 32})),                       # two reduced axis groups
+])
+def test_rms_calibration(shape, kw, dtype):
+  """'rms,7': scale = D(D(sqrt(D(mean(D(x^2))))) * 7) / qmax.  The mean is an f32 sum whose order neither XLA nor
+  this kernel pins: the calibration must match the oracle to one unit in the last place of the array dtype, and
+  where it matches exactly the quantized values must too (parity unpinned beyond that, as the oracle says)."""
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make(shape, dtype, seed=75)
+  how = dict(qtype='int8', calibration_method='rms,7', **kw)
+  cal = qarray.calibrate(x_t, qarray.HowToQuantize(**how))
+  want = O.calibrate(O.FArr(x_np, dtype), O.HowToQuantize(**how))
+  assert set(cal) == {'absmax'} and tuple(cal['absmax'].shape) == want['absmax'].v.shape
+  got = util.f32np(cal['absmax'])
+  ulp = 2.0 ** -7 if dtype == O.BF16 else 2.0 ** -22
+  assert np.all(np.abs(got - want['absmax'].v) <= ulp * np.abs(want['absmax'].v))
+  if dtype == O.BF16:  # f32 shows the summation order directly; bf16 hides it behind its rounding almost always
+    assert np.mean(got == want['absmax'].v) > 0.9
+  # closed form on a constant array: rms of all-c is |c|
+  c = torch.full(shape, -0.75, dtype=util.TORCH_DT[dtype], device=util.DEV)
+  assert torch.all(qarray.calibrate(c, qarray.HowToQuantize(**how))['absmax'] == 0.75 * 7).item()
+  if 'tiled_axes' in kw and len(kw['tiled_axes']) == 2:
+    return  # the static-scale kernel takes one reduced axis group
+  qa = qarray.quantize(x_t, qarray.HowToQuantize(**how))
+  oq = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(**how))
+  if np.array_equal(util.f32np(qa.scale), oq.scale.v):
+    util.assert_qarray_equal(qa, oq, 'rms')
+  else:
+    same = util.f32np(qa.scale) == oq.scale.v
+    for ax, (d, sd) in enumerate(zip(shape, same.shape)):
+      same = np.repeat(same, d // sd, axis=ax)
+    assert np.array_equal(util.qvalues_np(qa)[same], oq.qvalue[same])
 
 
 def test_zero_rows_and_reference_convert_vectors():

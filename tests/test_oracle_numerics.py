@@ -315,3 +315,17 @@ def test_fixed_calibration_closed_form():
   for bad in ('fixed', 'fixed,1,2', 'fixed,-1,-0.5', 'fixed,0,0'):
     with pytest.raises(ValueError):
       O.calibrate(x, O.HowToQuantize(qtype='int8', calibration_method=bad))
+
+
+def test_rms_calibration_closed_forms():
+  """qarray.py:511-515: rms of a constant array is |c|, of (+a, -a, +a, ...) is a; the factor multiplies it."""
+  x = O.FArr(np.full((4, 64), -0.75, np.float32), O.BF16)
+  how = O.HowToQuantize(qtype='int8', channelwise_axes=[0], calibration_method='rms,7')
+  cal = O.calibrate(x, how)
+  assert set(cal) == {'absmax'} and cal['absmax'].v.shape == (4, 1) and np.all(cal['absmax'].v == 0.75 * 7)
+  alt = np.tile(np.array([2.0, -2.0], np.float32), (3, 16))
+  cal = O.calibrate(O.FArr(alt, O.F32), O.HowToQuantize(qtype='int8', channelwise_axes=[0], tiled_axes={1: 8},
+                                                         calibration_method='rms,0.5'))
+  assert cal['absmax'].v.shape == (3, 4) and np.all(cal['absmax'].v == 1.0)
+  with pytest.raises(ValueError, match='scale factor'):
+    O.calibrate(x, O.HowToQuantize(qtype='int8', calibration_method='rms'))
