@@ -141,6 +141,20 @@ QWIX_API int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t l
                    int sb_dtype, int acc_dtype, void* out, int out_dtype, int64_t ldo,
                    void* stream);
 
+/* qwix_hip_qgemm with scratch memory.  A few hundred rows against a narrow weight with a long K leave most
+ * of the chip idle under 128 x 128 tiles; given a workspace the library may cut K into ranges that run as
+ * separate workgroups and add the partial tiles up in a second kernel (int32 partials: bit-identical to
+ * qwix_hip_qgemm for int8; e4m3 sums its f32 partials in range order).  qwix_hip_qgemm_workspace_bytes
+ * returns how many bytes that takes for a shape, 0 where splitting never pays; a NULL or smaller workspace
+ * makes the call behave exactly like qwix_hip_qgemm.  The workspace is 16-byte aligned device memory that
+ * only this call uses until it has finished on `stream`.  Same reference function as qwix_hip_qgemm
+ * (_fast_dot_general, qwix/_src/core/dot_general.py:135-261). */
+QWIX_API size_t qwix_hip_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+QWIX_API int qwix_hip_qgemm_ws(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M,
+                      int64_t N, int64_t K, const void* sa, int sa_dtype, const void* sb, int sb_dtype,
+                      int acc_dtype, void* out, int out_dtype, int64_t ldo, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
 /* Asymmetric (zero-point) operand on the quantized path.  Replaces the correction terms of
  * _fast_dot_general (qwix/_src/core/dot_general.py:228-253): the reference subtracts
  * dot(broadcast(zp_lhs), q_rhs) or dot(q_lhs, broadcast(zp_rhs)) from the int32 accumulator

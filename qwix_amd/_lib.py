@@ -36,6 +36,8 @@ SIGNATURES = {
     'qwix_hip_dequantize_generic': (_int, [_vp, _int, _c.POINTER(_i64), _i64, _i64, _vp, _vp, _int, _vp, _vp]),
     'qwix_hip_transpose_q': (_int, [_vp, _int, _i64, _i64, _vp, _vp]),
     'qwix_hip_qgemm': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _vp, _int, _vp, _int, _int, _vp, _int, _i64, _vp]),
+    'qwix_hip_qgemm_workspace_bytes': (_sz, [_i64, _i64, _i64]),
+    'qwix_hip_qgemm_ws': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _vp, _int, _vp, _int, _int, _vp, _int, _i64, _vp, _sz, _vp]),
     'qwix_hip_qgemm_zp': (_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _int, _vp, _int, _vp, _vp, _vp, _int, _i64, _vp]),
     'qwix_hip_qgemm_ragged': (_int, [_vp, _i64, _vp, _i64, _i64, _int, _i64, _i64, _i64, _vp, _i64, _vp, _int, _vp, _int, _i64, _int, _vp, _int, _i64, _vp]),
     'qwix_hip_qgemm_batched': (_int, [_vp, _i64, _i64, _vp, _i64, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp, _int, _i64, _int, _vp, _int, _i64, _i64, _vp]),

@@ -15,6 +15,7 @@ the vendor float GEMM.  Unsupported fast-path combinations raise; they never cha
 """
 from __future__ import annotations
 
+import functools
 import math
 from typing import Any, Mapping, Sequence
 
@@ -317,6 +318,12 @@ def fused_act_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=No
   return out.reshape(c.out_shape)
 
 
+@functools.lru_cache(maxsize=None)
+def _splitk_bytes(M: int, N: int, K: int) -> int:
+  """Scratch bytes with which the GEMM may split K for this shape (0: it would not)."""
+  return int(_lib.load().qwix_hip_qgemm_workspace_bytes(M, N, K))
+
+
 def _tag_of(dtype: torch.dtype) -> int:
   if dtype == torch.int32:
     return _lib.I32
@@ -410,10 +417,12 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
       acc = torch.empty(c.M, c.N, dtype=torch.int32, device=dev)
       _lib.call('qwix_hip_qgemm', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), qt, c.M, c.N, K, None, 0,
                 None, 0, 0, acc.data_ptr(), _lib.I32, c.N, st)
-    _lib.call('qwix_hip_qgemm', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), qt, c.M, c.N, K,
+    nws = _splitk_bytes(c.M, c.N, K)
+    ws = torch.empty(nws, dtype=torch.uint8, device=dev) if nws else None
+    _lib.call('qwix_hip_qgemm_ws', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), qt, c.M, c.N, K,
               _lib.ptr(sa), 0 if sa is None else _lib.float_tag(sa.dtype), _lib.ptr(sb),
               0 if sb is None else _lib.float_tag(sb.dtype), _tag_of(acc_t) if acc_t != torch.int32 else 0,
-              out.data_ptr(), _tag_of(res_t), c.N, st)
+              out.data_ptr(), _tag_of(res_t), c.N, _lib.ptr(ws), nws, st)
     out = out.reshape(c.out_shape)
     return (out, acc.reshape(c.out_shape)) if return_accumulators else out
   # sub-channel / int4 weights

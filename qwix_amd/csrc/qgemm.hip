@@ -1564,7 +1564,10 @@ extern "C" int qwix_hip_ksum_i8(const void* q, int64_t ld, int64_t rows, int64_t
 
 static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M, int64_t N, int64_t K,
                       const void* sa, int sa_dtype, const void* sb, int sb_dtype, int acc_dtype, const int32_t* zu,
-                      const int32_t* zv, void* out, int out_dtype, int64_t ldo, void* stream);
+                      const int32_t* zv, void* out, int out_dtype, int64_t ldo, void* stream, void* workspace = nullptr,
+                      size_t workspace_bytes = 0);
+static int splitk_plan(int64_t M, int64_t N, int64_t K, double other_us);
+static bool streams_weights(int64_t M, int64_t N, int64_t K);
 
 // Dtype chain of the reference epilogue: int32 adopts the first scale's dtype (through f32); a
 // float accumulator starts in acc_dtype; each multiply happens in the promotion of both sides.
@@ -1686,6 +1689,21 @@ extern "C" int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t
                     out_dtype, ldo, stream);
 }
 
+extern "C" size_t qwix_hip_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  // the split count qwix_hip_qgemm_ws would pick: the plan against the unsplit tiled kernel's model
+  const int splits = streams_weights(M, N, K) ? 0 : splitk_plan(M, N, K, 5.0 + 0.55 * static_cast<double>(K / 128));
+  return splits > 0 ? static_cast<size_t>(splits) * M * N * 4 : 0;
+}
+
+extern "C" int qwix_hip_qgemm_ws(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M,
+                                 int64_t N, int64_t K, const void* sa, int sa_dtype, const void* sb, int sb_dtype,
+                                 int acc_dtype, void* out, int out_dtype, int64_t ldo, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  return qgemm_impl(a, lda, b, ldb, qtype, M, N, K, sa, sa_dtype, sb, sb_dtype, acc_dtype, nullptr, nullptr, out,
+                    out_dtype, ldo, stream, workspace, workspace_bytes);
+}
+
 extern "C" int qwix_hip_qgemm_zp(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N,
                                  int64_t K, const void* sa, int sa_dtype, const void* sb, int sb_dtype,
                                  const int32_t* zu, const int32_t* zv, void* out, int out_dtype, int64_t ldo,
@@ -1723,9 +1741,144 @@ extern "C" int qwix_hip_qgemm_batched(const void* a, int64_t lda, int64_t a_batc
   return launch_batched<QWIX_E4M3>(a, lda, b, ldb, bs, batch, M, N, K, ep, out, ldo, st);
 }
 
+// ------------------------------------------------------------------------------------------------
+// Split-K for problems whose 128 x 128 tiles occupy a fraction of the chip while K is long (a few hundred
+// rows against a narrow weight): the grid gets a second dimension over ranges of K slabs, every workgroup
+// writes its raw partial tile (int32, or f32 for e4m3) to a caller workspace [split][M][N], and a second
+// kernel sums the splits and applies the epilogue.  Integer partials add exactly, so int8 results are the
+// bits of the unsplit kernels.
+template <int QT>
+__global__ void __launch_bounds__(256)
+    qgemm_splitk_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb, int M,
+                        int N, int K, int slabs_per_split, uint8_t* __restrict__ ws) {
+  int tile_m, tile_n;
+  tile_coords((M + 127) / 128, (N + 127) / 128, &tile_m, &tile_n);
+  const int k0 = blockIdx.y * slabs_per_split * 128;
+  const int klen = min(K - k0, slabs_per_split * 128);  // > 0: the host sizes the grid that way
+  const Epilogue raw{nullptr, nullptr, 0, 0, QT == QWIX_INT8 ? QWIX_I32 : QWIX_F32, 0, 0, 0, nullptr, nullptr};
+  uint8_t* part = ws + static_cast<int64_t>(blockIdx.y) * M * N * 4;
+  qgemm_dma_tile<QT, 128, 128, 2, 2, (QT == QWIX_INT8 ? QWIX_I32 : QWIX_F32), 0>(A + k0, lda, B + k0, ldb, tile_m * 128,
+                                                                                tile_n * 128, M, N, klen, raw, part, N);
+}
+
+// out[m, n] = epilogue(sum over splits of ws[s][m][n]); four consecutive elements of the flattened (m, n) per thread.
+template <bool IS_INT>
+__global__ void __launch_bounds__(256)
+    splitk_reduce_kernel(const uint8_t* __restrict__ ws, int splits, int M, int N, Epilogue ep, uint8_t* __restrict__ out,
+                         int64_t ldo) {
+  const int64_t total = static_cast<int64_t>(M) * N;
+  const int64_t i0 = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+  if (i0 >= total) return;
+  const bool vec = (N & 3) == 0;  // then the four share a row and the loads are 16-byte aligned
+  float v[4];
+  if constexpr (IS_INT) {
+    int a[4] = {0, 0, 0, 0};
+    for (int s = 0; s < splits; ++s) {
+      const int* p = reinterpret_cast<const int*>(ws) + s * total + i0;
+      if (vec) {
+        const int4 w = *reinterpret_cast<const int4*>(p);
+        a[0] += w.x; a[1] += w.y; a[2] += w.z; a[3] += w.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (i0 + e < total) a[e] += p[e];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = static_cast<float>(a[e]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float* p = reinterpret_cast<const float*>(ws) + s * total + i0;
+      if (vec) {
+        const float4 w = *reinterpret_cast<const float4*>(p);
+        v[0] += w.x; v[1] += w.y; v[2] += w.z; v[3] += w.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (i0 + e < total) v[e] += p[e];
+      }
+    }
+  }
+  const bool r0 = ep.r0 != 0, r1 = ep.r1 != 0, r2 = ep.r2 != 0;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int64_t i = i0 + e;
+    if (i >= total) break;
+    const int m = static_cast<int>(i / N), n = static_cast<int>(i % N);
+    float t = v[e];
+    if (r0) t = round_bf16(t);
+    if (ep.sa != nullptr) t *= load_scale(ep.sa, ep.sa_dtype, m);
+    if (r1) t = round_bf16(t);
+    if (ep.sb != nullptr) t *= load_scale(ep.sb, ep.sb_dtype, n);
+    if (r2) t = round_bf16(t);
+    if (ep.out_dtype == QWIX_BF16)
+      reinterpret_cast<uint16_t*>(out)[static_cast<int64_t>(m) * ldo + n] = f32_to_bf16_bits(t);
+    else
+      reinterpret_cast<float*>(out)[static_cast<int64_t>(m) * ldo + n] = t;
+  }
+}
+
+// Number of K ranges worth cutting the problem into (0: do not split).  Model, in microseconds, fitted to
+// measurements (256 x 4096 x 1024: 21.6 unsplit, 15.4 in 8 ranges; 256 x 8192 x 2048: 39.4 and 21.1): a
+// 128-wide K slab takes about 0.55, the two launches 9 together, and the partial tiles travel to the
+// workspace and back at about 4 bytes/ns.  Splitting has to win by 15 % to be chosen.
+// The rule of qgemm_impl for taking the weight-streaming kernel (see there for the model).
+static bool streams_weights(int64_t M, int64_t N, int64_t K) {
+  const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+  const double passes = static_cast<double>((M + 15) / 16);
+  const double skinny_us = 4.0 + passes * (0.5 + static_cast<double>(N) * static_cast<double>(K) / 5.2e6);
+  const double tiled_us = 5.0 + 0.55 * static_cast<double>(K / 128);
+  return M <= 32 || (M <= 256 && tiles128 <= 256 && skinny_us < tiled_us);
+}
+
+static int splitk_plan(int64_t M, int64_t N, int64_t K, double other_us) {
+  if (K % 128 != 0 || M <= 32) return 0;
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128), slabs = K / 128;
+  if (tiles > 128 || slabs < 8) return 0;
+  int best = 0;
+  double best_us = 1e30;
+  for (int s = 2; s <= 16 && s * 2 <= slabs && tiles * s <= 512; s *= 2) {
+    const double per = static_cast<double>((slabs + s - 1) / s);
+    const double waves = static_cast<double>((tiles * s + 255) / 256);
+    const double us = 9.0 + 0.55 * per * waves + static_cast<double>(s) * M * N * 8.0 / 4.0e6;
+    if (us < 0.85 * other_us && us < best_us) {
+      best_us = us;
+      best = s;
+    }
+  }
+  return best;
+}
+
+template <int QT>
+static int launch_splitk(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K, int splits,
+                         const Epilogue& ep, void* out, int64_t ldo, void* ws, hipStream_t st) {
+  constexpr size_t smem = 2 * (128 + 128) * 128;
+  auto kern = qgemm_splitk_kernel<QT>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128), slabs = K / 128;
+  const int per = static_cast<int>((slabs + splits - 1) / splits);
+  const int used = static_cast<int>((slabs + per - 1) / per);  // every range holds at least one slab
+  kern<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(used)), 256, smem, st>>>(
+      static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, static_cast<int>(M), static_cast<int>(N),
+      static_cast<int>(K), per, static_cast<uint8_t*>(ws));
+  const int64_t threads = (M * N + 3) / 4;
+  splitk_reduce_kernel<QT == QWIX_INT8><<<dim3(static_cast<unsigned>((threads + 255) / 256)), 256, 0, st>>>(
+      static_cast<const uint8_t*>(ws), used, static_cast<int>(M), static_cast<int>(N), ep, static_cast<uint8_t*>(out), ldo);
+  return check_launch("qgemm (split K)");
+}
+
 static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M, int64_t N, int64_t K,
                       const void* sa, int sa_dtype, const void* sb, int sb_dtype, int acc_dtype, const int32_t* zu,
-                      const int32_t* zv, void* out, int out_dtype, int64_t ldo, void* stream) {
+                      const int32_t* zv, void* out, int out_dtype, int64_t ldo, void* stream, void* workspace,
+                      size_t workspace_bytes) {
   if (const int rc = check_gemm_args(a, lda, b, ldb, qtype, M, N, K, sa, sa_dtype, sb, sb_dtype, acc_dtype, out,
                                      out_dtype, ldo))
     return rc;
@@ -1735,11 +1888,17 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
   // model favours it: the skinny kernel makes one pass over the weights per 16 rows (from L2 after the first,
   // about 0.5 us + 5.2 bytes/ns each) after a 4 us start, the tiled kernels walk K in 128-wide slabs of about
   // 0.55 us after 5 us, however few of the chip's CUs their 128 x 128 tiles occupy.
-  const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
-  const double passes = static_cast<double>((M + 15) / 16);
-  const double skinny_us = 4.0 + passes * (0.5 + static_cast<double>(N) * static_cast<double>(K) / 5.2e6);
   const double tiled_us = 5.0 + 0.55 * static_cast<double>(K / 128);
-  const bool few_rows = M <= 32 || (M <= 256 && tiles128 <= 256 && skinny_us < tiled_us);
+  const bool few_rows = streams_weights(M, N, K);
+  const bool off31 = M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);
+  if (workspace != nullptr && zu == nullptr && out_dtype != QWIX_I32 && off31) {
+    // only against the tiled kernels: where the weight-streaming kernel is chosen its own model has spoken
+    const int splits = few_rows ? 0 : splitk_plan(M, N, K, tiled_us);
+    if (splits > 0 && workspace_bytes >= static_cast<size_t>(splits) * M * N * 4 && aligned16(workspace)) {
+      if (qtype == QWIX_INT8) return launch_splitk<QWIX_INT8>(a, lda, b, ldb, M, N, K, splits, ep, out, ldo, workspace, st);
+      return launch_splitk<QWIX_E4M3>(a, lda, b, ldb, M, N, K, splits, ep, out, ldo, workspace, st);
+    }
+  }
   if (few_rows && K % 128 == 0 && M * lda < (int64_t{1} << 31) && 64 * ldb < (int64_t{1} << 31)) {
     if (qtype == QWIX_INT8) return launch_skinny<QWIX_INT8>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     return launch_skinny<QWIX_E4M3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);

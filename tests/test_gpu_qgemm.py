@@ -181,3 +181,59 @@ def test_fused_activation_quantize_gemm_bit_exact(M, K, N, dtype):
   assert dg.fused_act_dot_general(torch.zeros(40, K, device=util.DEV), wq, DN) is None
   w4 = qarray.quantize(torch.zeros(4096, 64, device=util.DEV), qarray.HowToQuantize(qtype='int8', channelwise_axes=[1]))
   assert dg.fused_act_dot_general(torch.zeros(8, 4096, device=util.DEV), w4, DN) is None   # K too long
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('M,K,N', [(256, 4096, 1024), (300, 4096, 520), (384, 4096, 512), (257, 8192, 1000), (512, 4096, 250)])
+def test_int8_gemm_split_k_bit_exact(M, K, N, dtype):
+  """A few hundred rows against a narrow weight with a long K: the library may cut K into ranges (it reports a
+  workspace size for these shapes); int32 partials add exactly, so the result is the oracle's, bit for bit,
+  with and without the workspace."""
+  from qwix_amd import _lib
+  from qwix_amd.core import dot_general as dg
+  print('case split-K', M, K, N, dtype, flush=True)
+  assert _lib.load().qwix_hip_qgemm_workspace_bytes(M, N, K) > 0
+  xq, wq, oxq, owq = _quantized_pair(M, K, N, dtype, 'int8', seed=M + K + N)
+  want = O.fast_dot_general(oxq, owq, DN)
+  out = dg.dot_general(xq, wq, DN)          # takes the workspace route
+  assert np.array_equal(util.f32np(out), want.v)
+  # the same call without scratch memory must give the same bits
+  c = dg._Canon(xq, wq, DN)
+  a, (b, _) = c.lhs_values(xq), c.rhs_values(wq)
+  sa, _ = c.lhs_scale(xq)
+  sb, _ = c.rhs_scale(wq)
+  plain = torch.empty(M, N, dtype=out.dtype, device=util.DEV)
+  tag = _lib.float_tag(out.dtype)
+  _lib.call('qwix_hip_qgemm', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), _lib.INT8, M, N, K, sa.data_ptr(),
+            _lib.float_tag(sa.dtype), sb.data_ptr(), _lib.float_tag(sb.dtype), 0, plain.data_ptr(), tag, N, _lib.stream_of(a))
+  assert torch.equal(plain, out)
+  # a workspace that is too small is ignored, not overrun
+  small = torch.empty(64, dtype=torch.uint8, device=util.DEV)
+  again = torch.empty_like(plain)
+  _lib.call('qwix_hip_qgemm_ws', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), _lib.INT8, M, N, K, sa.data_ptr(),
+            _lib.float_tag(sa.dtype), sb.data_ptr(), _lib.float_tag(sb.dtype), 0, again.data_ptr(), tag, N,
+            small.data_ptr(), 64, _lib.stream_of(a))
+  assert torch.equal(again, out)
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+def test_fp8_gemm_split_k_close(dtype):
+  from qwix_amd.core import dot_general as dg
+  M, K, N = 256, 4096, 1024
+  xq, wq, oxq, owq = _quantized_pair(M, K, N, dtype, 'float8_e4m3fn', seed=77)
+  out = dg.dot_general(xq, wq, DN)
+  want = O.fast_dot_general(oxq, owq, DN)
+  tol = 1e-2 if dtype == O.BF16 else 1e-3   # the tolerance of test_fp8_gemm_close
+  got = util.f32np(out)
+  assert np.allclose(got, want.v, rtol=tol, atol=tol * np.abs(want.v).mean()), np.abs(got - want.v).max()
+
+
+def test_split_k_is_not_offered_where_it_cannot_pay():
+  from qwix_amd import _lib
+  f = _lib.load().qwix_hip_qgemm_workspace_bytes
+  assert f(4096, 4096, 4096) == 0      # the tiles already fill the chip
+  assert f(16, 4096, 4096) == 0        # decode sizes stream the weight
+  assert f(256, 1024, 512) == 0        # too few slabs to cut
+  assert f(256, 4096, 1024) == 0       # a short K (M, N, K = 256, 4096, 1024): the second launch costs more than it saves
+  assert f(256, 256, 4096) == 0        # the weight-streaming kernel takes it
+  assert f(256, 1024, 4100) == 0       # K not a multiple of 128 (M, N, K)
