@@ -551,6 +551,25 @@ class RaggedQdot(Workload):
             'weight': 'per-expert per-output-channel ' + self.qtype + ' (pre-quantized)', 'out': 'bf16'}
 
 
+class RaggedDecode(RaggedQdot):
+  """Mixture-of-experts decode: a few tokens per expert, so the step is bound by reading every expert's
+  weight once; reported as the bytes of weights (+ activations, outputs) per second."""
+
+  bound = 'hbm'
+
+  def __init__(self, name, M, K, N, G):
+    super().__init__(name, M, K, N, G, 'int8')
+    self.metric = 'ragged qdot GB/s (w8a8 mixture-of-experts decode, weight streaming, activation quantize included)'
+    self.unit = 'GB/s'
+    self.kernel_name = 'qgemm_ragged_skinny_kernel'
+
+  def work_per_step(self):
+    return float(self.G * self.N * self.K + self.M * self.K * 3 + self.M * self.N * 2 + self.G * self.N * 2)
+
+  def kernel_work(self):
+    return float(self.G * self.N * self.K + self.M * self.K + self.M * self.N * 2 + self.G * self.N * 2)
+
+
 class QuantizeStatic(Workload):
   """Static-range activation quantization: the scale was computed offline, one read and one write."""
 
@@ -789,6 +808,7 @@ WORKLOADS = {
     'plain_copy_1g': lambda: PlainCopy('plain_copy_1g', 1 << 30),
     'moe_ragged_int8_8x1024': lambda: RaggedQdot('moe_ragged_int8_8x1024', 8192, 4096, 14336, 8),
     'moe_ragged_int8_64x128': lambda: RaggedQdot('moe_ragged_int8_64x128', 8192, 2048, 4096, 64),
+    'moe_decode_int8_64x4': lambda: RaggedDecode('moe_decode_int8_64x4', 256, 2048, 4096, 64),
     'moe_ragged_fp8_8x1024': lambda: RaggedQdot('moe_ragged_fp8_8x1024', 8192, 4096, 14336, 8, 'float8_e4m3fn'),
     'quantize_weight_fp8_block128': lambda: QuantizeBlocks('quantize_weight_fp8_block128', 4096, 14336, 'float8_e4m3fn'),
     'srq_quantize_act_4096': lambda: QuantizeStatic('srq_quantize_act_4096', 4096, 4096),
@@ -800,7 +820,7 @@ WORKLOADS = {
 DEFAULT = 'c3_int8_w8a8_4096'
 EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
          'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'moe_ragged_int8_8x1024',
-         'moe_ragged_int8_64x128', 'quantize_weight_fp8_block128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
+         'moe_ragged_int8_64x128', 'moe_decode_int8_64x4', 'quantize_weight_fp8_block128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 
 
 def _blas_threads() -> int:

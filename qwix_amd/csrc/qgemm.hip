@@ -1253,17 +1253,18 @@ typedef int v8i_s __attribute__((ext_vector_type(8)));
 typedef float v4f_s __attribute__((ext_vector_type(4)));
 constexpr int kSkinnyWaves = 16;
 
+// One 16-row block of the weight-streaming GEMM: rows row0 .. row0 + 15 (below M) against columns n_base ..
+// n_base + 16 * NT - 1, by a workgroup of kSkinnyWaves wavefronts that split K.
 template <int QT, int NT>
-__global__ void __launch_bounds__(kSkinnyWaves * 64)
-    qgemm_skinny_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb, int M,
-                        int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+__device__ __forceinline__ void skinny_block(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B,
+                                             int64_t ldb, int row0, int M, int n_base, int N, int K, const Epilogue& ep,
+                                             uint8_t* __restrict__ out, int64_t ldo) {
   constexpr bool IS_INT = (QT == QWIX_INT8);
   using AccT = typename std::conditional<IS_INT, v4i, v4f_s>::type;
   __shared__ AccT red[kSkinnyWaves][NT][64];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, kq = lane >> 4;
-  const int n_base = blockIdx.x * (16 * NT), row0 = blockIdx.y * 16;
   const int nblk = K / 128;
   const int per_wave = (nblk + kSkinnyWaves - 1) / kSkinnyWaves;
   const int kb0 = wave * per_wave, kb1 = min(nblk, kb0 + per_wave);
@@ -1358,6 +1359,13 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64)
   }
 }
 
+template <int QT, int NT>
+__global__ void __launch_bounds__(kSkinnyWaves * 64)
+    qgemm_skinny_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb, int M,
+                        int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  skinny_block<QT, NT>(A, lda, B, ldb, blockIdx.y * 16, M, blockIdx.x * (16 * NT), N, K, ep, out, ldo);
+}
+
 template <int QT>
 int launch_skinny(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
                   const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
@@ -1376,6 +1384,59 @@ int launch_skinny(const void* a, int64_t lda, const void* b, int64_t ldb, int64_
     QWIX_SKINNY(1);
 #undef QWIX_SKINNY
   return check_launch("qgemm (skinny)");
+}
+
+// Ragged variant for a few rows per group (mixture-of-experts decode): blockIdx.y is the group, whose rows are
+// found from the group sizes by every wavefront for itself; the workgroup streams that group's weight columns
+// once per 16 rows.  blockIdx.y == G clears the rows that belong to no group.
+template <int QT, int NT>
+__global__ void __launch_bounds__(kSkinnyWaves * 64)
+    qgemm_ragged_skinny_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
+                               Ragged rg, int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  const int g = blockIdx.y, lane = threadIdx.x & 63;
+  const int n_base = blockIdx.x * (16 * NT);
+  long long before = 0;
+  for (int i = lane; i < g; i += 64) before += max(rg.group_sizes[i], 0);
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) before += __shfl_xor(before, m, 64);
+  const int start = static_cast<int>(min(before, static_cast<long long>(M)));
+  if (g == rg.G) {  // rows past the last group: zeros
+    const int cols = min(16 * NT, N - n_base);
+    for (int idx = threadIdx.x; idx < (M - start) * cols; idx += kSkinnyWaves * 64) {
+      const int64_t at = static_cast<int64_t>(start + idx / cols) * ldo + n_base + idx % cols;
+      if (ep.out_dtype == QWIX_BF16) reinterpret_cast<uint16_t*>(out)[at] = 0;
+      else reinterpret_cast<uint32_t*>(out)[at] = 0;
+    }
+    return;
+  }
+  const int end = static_cast<int>(min(before + max(rg.group_sizes[g], 0), static_cast<long long>(M)));
+  const Epilogue e = group_epilogue(ep, rg, g);
+  const uint8_t* bg = B + g * rg.b_group_stride;
+  for (int row0 = start; row0 < end; row0 += 16) {  // the trip count is the same for the whole workgroup
+    skinny_block<QT, NT>(A, lda, bg, ldb, row0, end, n_base, N, K, e, out, ldo);
+    __syncthreads();  // the partial sums in LDS are reused by the next pass
+  }
+}
+
+template <int QT>
+int launch_ragged_skinny(const void* a, int64_t lda, const void* b, int64_t ldb, const Ragged& rg, int64_t M, int64_t N,
+                         int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  const unsigned gy = static_cast<unsigned>(rg.G + 1);
+#define QWIX_RSKINNY(NTT)                                                                                          \
+  qgemm_ragged_skinny_kernel<QT, NTT><<<dim3(static_cast<unsigned>((N + 16 * NTT - 1) / (16 * NTT)), gy),          \
+                                        kSkinnyWaves * 64, 0, st>>>(static_cast<const uint8_t*>(a), lda,            \
+                                                                    static_cast<const uint8_t*>(b), ldb, rg,          \
+                                                                    static_cast<int>(M), static_cast<int>(N),        \
+                                                                    static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo)
+  // wide column groups while that still leaves a thousand workgroups
+  if ((N / 64) * rg.G >= 1024)
+    QWIX_RSKINNY(4);
+  else if ((N / 32) * rg.G >= 1024)
+    QWIX_RSKINNY(2);
+  else
+    QWIX_RSKINNY(1);
+#undef QWIX_RSKINNY
+  return check_launch("ragged qgemm (skinny)");
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1659,6 +1720,12 @@ extern "C" int qwix_hip_qgemm_ragged(const void* a, int64_t lda, const void* b, 
   const Epilogue ep = make_epilogue(qtype, sa, sa_dtype, sb, sb_dtype, acc_dtype, nullptr, nullptr, out_dtype);
   const Ragged rg{group_sizes, static_cast<int>(G), b_group_stride, sb_group_stride};
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (K % 128 == 0 && M <= 16 * G && G + 1 <= 65535 && 64 * ldb < (int64_t{1} << 31)) {
+    // at most 16 rows per group on average (decode): stream every group's weight once instead of tiling
+    // (measured, 64 groups x 2048 x 4096: 146 -> 119 us; at 32 rows per group a second pass over the weights loses)
+    if (qtype == QWIX_INT8) return launch_ragged_skinny<QWIX_INT8>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+    return launch_ragged_skinny<QWIX_E4M3>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+  }
   if (K % 128 == 0) {
     // 256-row tiles pay off once the average group is several tiles tall; 128-row tiles waste fewer rows
     // at the ragged end of each group.

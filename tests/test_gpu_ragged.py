@@ -53,6 +53,10 @@ INT8_CASES = [
     ('k tiled', (128, 256, 4, 512), (10, 20, 30, 68), (0,), (0, 2), {1: 128}),
     ('k tiled, shared over groups', (128, 256, 4, 512), (10, 20, 30, 68), (0,), (2,), {1: 128}),
     ('k and n tiled', (128, 256, 4, 512), (10, 20, 30, 68), (0,), (0,), {1: 128, 2: 128}),
+    ('decode: a few rows per group (weight-streaming kernel), empty groups, rows of no group', (40, 256, 12, 200),
+     (0, 3, 16, 1, 0, 7, 2, 0, 5, 2, 1, 1), (0,), (0, 2), None),
+    ('decode: one group takes several 16-row passes', (60, 384, 6, 72), (0, 40, 1, 0, 9, 3), (0,), (0, 2), None),
+    ('decode: one row per group, shared weight scale', (16, 128, 16, 48), (1,) * 16, (0,), (2,), None),
     ('big groups', (2100, 512, 2, 2304), (1100, 900), (0,), (0, 2), None),
     ('big groups on a full chip (256-row tiles, ping-pong schedule)', (4096, 384, 4, 3072), (1000, 1100, 900, 1000), (0,), (0, 2), None),
 ]
@@ -118,7 +122,8 @@ def test_ragged_dot_out_of_range_sizes_are_clamped():
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
 @pytest.mark.parametrize('shape,sizes,rcw', [((128, 256, 4, 64), (128, 100, 0, 28), (2,)),
                                              ((520, 512, 6, 384), (100, 3, 0, 257, 60, 50), (0, 2)),
-                                             ((4096, 256, 4, 3072), (1000, 1100, 900, 1000), (0, 2))])
+                                             ((4096, 256, 4, 3072), (1000, 1100, 900, 1000), (0, 2)),
+                                             ((48, 256, 8, 200), (5, 0, 9, 1, 20, 3, 2, 4), (0, 2))])   # decode sizes
 def test_ragged_dot_fp8(shape, sizes, rcw, dtype):
   import qwix_amd
   M, K, G, N = shape
