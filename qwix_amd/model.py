@@ -24,7 +24,9 @@ class QuantizedModel:
     nn._tls.provider = self.provider
     self.provider.reset_op_ids()
     try:
-      return self.model(params, *inputs, **kwargs)
+      out = self.model(params, *inputs, **kwargs)
+      self.provider._initial_run_complete = True
+      return out
     finally:
       nn._tls.provider = old
 

@@ -54,10 +54,24 @@ class QuantizationProvider:
   """Holds the rules and resolves the rule that applies to the op being executed."""
 
   def __init__(self, rules: Sequence[QuantizationRule], *, disable_jit: bool = False):
-    self._rules = list(rules)
+    self._rules = [self._init_rule(rule) for rule in rules]
     self._rule_matches = [False] * len(self._rules)
     self._op_counts: dict[tuple[tuple[str, ...], str], int] = {}
+    self._initial_run_complete = False  # set by the model wrapper once the model has run under this provider
     self.disable_jit = disable_jit
+
+  @staticmethod
+  def _init_rule(rule: QuantizationRule) -> QuantizationRule:
+    """Validates a rule and fills its defaults (qconfig.py:122-135)."""
+    if rule.act_qtype is None and rule.act_static_scale is not None:
+      raise ValueError(f'Invalid rule: act_static_scale is set to {rule.act_static_scale} but act_qtype is None. '
+                       'Please either unset act_static_scale, or set act_qtype to enable activation quantization. '
+                       f'(Rule: {rule})')
+    if rule.act_static_scale is None:
+      rule = dataclasses.replace(rule, act_static_scale=False)
+    if rule.act_calibration_method is None:
+      rule = dataclasses.replace(rule, act_calibration_method='absmax')
+    return rule
 
   def reset_op_ids(self) -> None:
     """Op ids restart at 0 for every model call, so that the same op gets the same id each time."""
@@ -79,5 +93,8 @@ class QuantizationProvider:
     return rule, f'{op_name}{n}'
 
   def get_unused_rules(self) -> list[QuantizationRule]:
-    """Rules that never matched (qconfig.py:242-262)."""
+    """Rules that never matched (qconfig.py:242-262); only meaningful once the model has run."""
+    if not self._initial_run_complete:
+      raise ValueError('Quantization is not completed yet. Please call `quantize_model` and run the model '
+                       'before calling `get_unused_rules`.')
     return [r for r, used in zip(self._rules, self._rule_matches) if not used]

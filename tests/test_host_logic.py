@@ -168,7 +168,15 @@ def test_rule_lookup_first_full_match_wins_and_op_ids():
     assert p._get_current_rule_and_op_id('einsum')[0].weight_qtype == 'float8_e4m3fn'
     assert p._get_current_rule_and_op_id('dot_general')[0].act_qtype == 'int8'
   assert qconfig.current_module_path() == ()
+  with pytest.raises(ValueError, match='Quantization is not completed yet'):   # qconfig_test.py:97-115
+    p.get_unused_rules()
+  p._initial_run_complete = True   # what the model wrapper sets after the first run
   assert [r.module_path for r in p.get_unused_rules()] == ['never']
+  # qconfig_test.py:117-127 and the defaults of qconfig.py:122-135
+  with pytest.raises(ValueError, match='act_static_scale is set to True but act_qtype is None'):
+    qconfig.QuantizationProvider([qconfig.QuantizationRule(weight_qtype='int8', act_static_scale=True)])
+  filled = qconfig.QuantizationProvider([qconfig.QuantizationRule(weight_qtype='int8', act_qtype='int8')])._rules[0]
+  assert filled.act_static_scale is False and filled.act_calibration_method == 'absmax'
   r = qconfig.QuantizationRule()
   assert (r.module_path, r.weight_qtype, r.act_qtype, r.tile_size, r.weight_calibration_method, tuple(r.act_batch_axes)) == ('.*', None, None, None, 'absmax', (0,))
 
