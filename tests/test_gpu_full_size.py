@@ -186,3 +186,33 @@ def test_zero_point_gemm_at_4096():
   want = want - zu[rows].cpu().numpy().astype(np.int64)[:, None] * zv.cpu().numpy().astype(np.int64)[None, :]
   assert np.abs(want).max() < 2 ** 24
   assert np.array_equal(out[rows].cpu().to(torch.float64).numpy(), want.astype(np.float64))
+
+
+@pytest.mark.parametrize('n_extra', [0, 100])
+def test_int8_gemm_with_a_short_last_round(n_extra):
+  """2048 x 10240 x 512: 320 tiles of 256 x 256 are one full round of the chip plus a quarter (and, with 100
+  more columns, a ragged last tile column).  Scales differ per column, so a misplaced column shows; the
+  zero-point variant runs over the same shape."""
+  from qwix_amd import _lib
+  M, K, N = 2048, 512, 10240 + n_extra
+  a = _small_ints((M, K), -3, 3, 31, torch.int8)
+  b = _small_ints((N, K), -3, 3, 32, torch.int8)
+  sb = (2.0 ** torch.randint(-2, 3, (N,), generator=torch.Generator().manual_seed(33)).float()).to(util.DEV)
+  out = torch.empty(M, N, dtype=torch.float32, device=util.DEV)
+  print('case short last round', M, K, N, flush=True)
+  _lib.call('qwix_hip_qgemm', a.data_ptr(), K, b.data_ptr(), K, _lib.INT8, M, N, K, None, 0, sb.data_ptr(), _lib.F32, 0,
+            out.data_ptr(), _lib.F32, N, _lib.stream_of(a))
+  torch.cuda.synchronize()
+  rows = util.rng(34).choice(M, 8, replace=False)
+  want = a[rows].cpu().numpy().astype(np.int64) @ b.cpu().numpy().astype(np.int64).T
+  assert np.array_equal(out[rows].cpu().numpy().astype(np.float64), want * sb.cpu().numpy().astype(np.float64)[None, :])
+  total = (out.to(torch.float64) / sb.to(torch.float64)).sum().item()
+  assert total == float(a.to(torch.float64).sum(0).cpu().numpy() @ b.to(torch.float64).sum(0).cpu().numpy())
+  # zero-point correction across the same split
+  zu = torch.randint(-128, 128, (M,), generator=torch.Generator().manual_seed(35), dtype=torch.int32).to(util.DEV)
+  zv = b.to(torch.int32).sum(1, dtype=torch.int32)
+  _lib.call('qwix_hip_qgemm_zp', a.data_ptr(), K, b.data_ptr(), K, M, N, K, None, 0, sb.data_ptr(), _lib.F32, zu.data_ptr(),
+            zv.data_ptr(), out.data_ptr(), _lib.F32, N, _lib.stream_of(a))
+  torch.cuda.synchronize()
+  want = want - zu[rows].cpu().numpy().astype(np.int64)[:, None] * zv.cpu().numpy().astype(np.int64)[None, :]
+  assert np.array_equal(out[rows].cpu().numpy().astype(np.float64), want * sb.cpu().numpy().astype(np.float64)[None, :])
