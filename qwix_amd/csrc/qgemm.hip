@@ -1254,19 +1254,19 @@ typedef float v4f_s __attribute__((ext_vector_type(4)));
 constexpr int kSkinnyWaves = 16;
 
 // One 16-row block of the weight-streaming GEMM: rows row0 .. row0 + 15 (below M) against columns n_base ..
-// n_base + 16 * NT - 1, by a workgroup of kSkinnyWaves wavefronts that split K.
-template <int QT, int NT>
+// n_base + 16 * NT - 1, by a workgroup of WAVES wavefronts that split K.
+template <int QT, int NT, int WAVES = kSkinnyWaves>
 __device__ __forceinline__ void skinny_block(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B,
                                              int64_t ldb, int row0, int M, int n_base, int N, int K, const Epilogue& ep,
                                              uint8_t* __restrict__ out, int64_t ldo) {
   constexpr bool IS_INT = (QT == QWIX_INT8);
   using AccT = typename std::conditional<IS_INT, v4i, v4f_s>::type;
-  __shared__ AccT red[kSkinnyWaves][NT][64];
+  __shared__ AccT red[WAVES][NT][64];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, kq = lane >> 4;
   const int nblk = K / 128;
-  const int per_wave = (nblk + kSkinnyWaves - 1) / kSkinnyWaves;
+  const int per_wave = (nblk + WAVES - 1) / WAVES;
   const int kb0 = wave * per_wave, kb1 = min(nblk, kb0 + per_wave);
 
   // wave-uniform bases + fixed 32-bit lane offsets; rows of A past M and columns past N are clamped
@@ -1327,7 +1327,7 @@ __device__ __forceinline__ void skinny_block(const uint8_t* __restrict__ A, int6
   __syncthreads();
   // result lane layout: column n = lane % 16, row m = 4 * (lane / 16) + r
   const bool r0 = ep.r0 != 0, r1 = ep.r1 != 0, r2 = ep.r2 != 0;
-  for (int idx = tid; idx < NT * 256; idx += kSkinnyWaves * 64) {
+  for (int idx = tid; idx < NT * 256; idx += WAVES * 64) {
     const int t = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
     const int m = row0 + 4 * (l >> 4) + r, n = n_base + t * 16 + (l & 15);
     if (m >= M || n >= N) continue;
@@ -1335,7 +1335,7 @@ __device__ __forceinline__ void skinny_block(const uint8_t* __restrict__ A, int6
     if constexpr (IS_INT) {
       int a = 0;
 #pragma unroll
-      for (int w = 0; w < kSkinnyWaves; ++w) a += red[w][t][l][r];
+      for (int w = 0; w < WAVES; ++w) a += red[w][t][l][r];
       if (ep.out_dtype == QWIX_I32) {
         reinterpret_cast<int*>(out)[static_cast<int64_t>(m) * ldo + n] = a;
         continue;
@@ -1345,7 +1345,7 @@ __device__ __forceinline__ void skinny_block(const uint8_t* __restrict__ A, int6
     } else {
       v = 0.f;
 #pragma unroll
-      for (int w = 0; w < kSkinnyWaves; ++w) v += red[w][t][l][r];
+      for (int w = 0; w < WAVES; ++w) v += red[w][t][l][r];
     }
     if (r0) v = round_bf16(v);
     if (ep.sa != nullptr) v *= load_scale(ep.sa, ep.sa_dtype, m);
@@ -1389,8 +1389,8 @@ int launch_skinny(const void* a, int64_t lda, const void* b, int64_t ldb, int64_
 // Ragged variant for a few rows per group (mixture-of-experts decode): blockIdx.y is the group, whose rows are
 // found from the group sizes by every wavefront for itself; the workgroup streams that group's weight columns
 // once per 16 rows.  blockIdx.y == G clears the rows that belong to no group.
-template <int QT, int NT>
-__global__ void __launch_bounds__(kSkinnyWaves * 64)
+template <int QT, int NT, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
     qgemm_ragged_skinny_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
                                Ragged rg, int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
   const int g = blockIdx.y, lane = threadIdx.x & 63;
@@ -1402,7 +1402,7 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64)
   const int start = static_cast<int>(min(before, static_cast<long long>(M)));
   if (g == rg.G) {  // rows past the last group: zeros
     const int cols = min(16 * NT, N - n_base);
-    for (int idx = threadIdx.x; idx < (M - start) * cols; idx += kSkinnyWaves * 64) {
+    for (int idx = threadIdx.x; idx < (M - start) * cols; idx += WAVES * 64) {
       const int64_t at = static_cast<int64_t>(start + idx / cols) * ldo + n_base + idx % cols;
       if (ep.out_dtype == QWIX_BF16) reinterpret_cast<uint16_t*>(out)[at] = 0;
       else reinterpret_cast<uint32_t*>(out)[at] = 0;
@@ -1413,7 +1413,7 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64)
   const Epilogue e = group_epilogue(ep, rg, g);
   const uint8_t* bg = B + g * rg.b_group_stride;
   for (int row0 = start; row0 < end; row0 += 16) {  // the trip count is the same for the whole workgroup
-    skinny_block<QT, NT>(A, lda, bg, ldb, row0, end, n_base, N, K, e, out, ldo);
+    skinny_block<QT, NT, WAVES>(A, lda, bg, ldb, row0, end, n_base, N, K, e, out, ldo);
     __syncthreads();  // the partial sums in LDS are reused by the next pass
   }
 }
@@ -1422,19 +1422,23 @@ template <int QT>
 int launch_ragged_skinny(const void* a, int64_t lda, const void* b, int64_t ldb, const Ragged& rg, int64_t M, int64_t N,
                          int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   const unsigned gy = static_cast<unsigned>(rg.G + 1);
+  // Small workgroups: 4 wavefronts, and the fewer rows a group has, the narrower the column group (the
+  // activation fragment is re-read per column group, which costs as much as the weights once a group has 16
+  // rows).  Measured at 64 groups x 4 rows, K 2048, N 4096, in GB/s of weights: 16 wavefronts x 64 columns
+  // 4260, 8 x 32 4700, 4 x 64 4680, 4 x 32 4810, 4 x 16 5120, 2 x 16 5060, 1 x 16 4980.
+  constexpr int kWaves = 4;
 #define QWIX_RSKINNY(NTT)                                                                                          \
-  qgemm_ragged_skinny_kernel<QT, NTT><<<dim3(static_cast<unsigned>((N + 16 * NTT - 1) / (16 * NTT)), gy),          \
-                                        kSkinnyWaves * 64, 0, st>>>(static_cast<const uint8_t*>(a), lda,            \
-                                                                    static_cast<const uint8_t*>(b), ldb, rg,          \
-                                                                    static_cast<int>(M), static_cast<int>(N),        \
-                                                                    static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo)
-  // wide column groups while that still leaves a thousand workgroups
-  if ((N / 64) * rg.G >= 1024)
-    QWIX_RSKINNY(4);
-  else if ((N / 32) * rg.G >= 1024)
+  qgemm_ragged_skinny_kernel<QT, NTT, kWaves><<<dim3(static_cast<unsigned>((N + 16 * NTT - 1) / (16 * NTT)), gy), \
+                                                kWaves * 64, 0, st>>>(static_cast<const uint8_t*>(a), lda,          \
+                                                                      static_cast<const uint8_t*>(b), ldb, rg,        \
+                                                                      static_cast<int>(M), static_cast<int>(N),      \
+                                                                      static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo)
+  if (M <= 4 * static_cast<int64_t>(rg.G))
+    QWIX_RSKINNY(1);
+  else if (M <= 8 * static_cast<int64_t>(rg.G))
     QWIX_RSKINNY(2);
   else
-    QWIX_RSKINNY(1);
+    QWIX_RSKINNY(4);
 #undef QWIX_RSKINNY
   return check_launch("ragged qgemm (skinny)");
 }
@@ -1887,19 +1891,27 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// Number of K ranges worth cutting the problem into (0: do not split).  Model, in microseconds, fitted to
-// measurements (256 x 4096 x 1024: 21.6 unsplit, 15.4 in 8 ranges; 256 x 8192 x 2048: 39.4 and 21.1): a
-// 128-wide K slab takes about 0.55, the two launches 9 together, and the partial tiles travel to the
-// workspace and back at about 4 bytes/ns.  Splitting has to win by 15 % to be chosen.
 // The rule of qgemm_impl for taking the weight-streaming kernel (see there for the model).
 static bool streams_weights(int64_t M, int64_t N, int64_t K) {
   const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
   const double passes = static_cast<double>((M + 15) / 16);
   const double skinny_us = 4.0 + passes * (0.5 + static_cast<double>(N) * static_cast<double>(K) / 5.2e6);
-  const double tiled_us = 5.0 + 0.55 * static_cast<double>(K / 128);
-  return M <= 32 || (M <= 256 && tiles128 <= 256 && skinny_us < tiled_us);
+  // The tiled kernels, with weights that come from HBM (measured with rotating weights, 32 rows: K 4096 35 us
+  // whatever N up to 14336; K 8192, N 28672 71 us; K 4096, N 131072 148 us): about 0.95 us per 128-wide K slab
+  // and round of two tiles per CU, and never faster than about 3.8 bytes/ns of weights.
+  const double rounds = tiles128 <= 512 ? 1.0 : static_cast<double>(tiles128) / 512.0;
+  const double slab_us = 0.95 * static_cast<double>(K / 128) * rounds;
+  const double read_us = static_cast<double>(N) * static_cast<double>(K) / 3.8e6;
+  const double tiled_us = 5.0 + (slab_us > read_us ? slab_us : read_us);
+  if (M <= 32) return M <= 16 || skinny_us < tiled_us;
+  // more rows: the comparison that was tuned with weights that stay in the last-level cache between calls
+  return M <= 256 && tiles128 <= 256 && skinny_us < 5.0 + 0.55 * static_cast<double>(K / 128);
 }
 
+// Number of K ranges worth cutting the problem into (0: do not split).  Model, in microseconds, fitted to
+// measurements (256 x 4096 x 1024: 21.6 unsplit, 15.4 in 8 ranges; 256 x 8192 x 2048: 39.4 and 21.1): a
+// 128-wide K slab takes about 0.55, the two launches 9 together, and the partial tiles travel to the
+// workspace and back at about 4 bytes/ns.  Splitting has to win by 15 % to be chosen.
 static int splitk_plan(int64_t M, int64_t N, int64_t K, double other_us) {
   if (K % 128 != 0 || M <= 32) return 0;
   const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128), slabs = K / 128;
@@ -1951,10 +1963,10 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
     return rc;
   const Epilogue ep = make_epilogue(qtype, sa, sa_dtype, sb, sb_dtype, acc_dtype, zu, zv, out_dtype);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  // Few rows: stream the weights instead of tiling.  Up to 32 rows always; up to 256 rows while a rough cost
-  // model favours it: the skinny kernel makes one pass over the weights per 16 rows (from L2 after the first,
-  // about 0.5 us + 5.2 bytes/ns each) after a 4 us start, the tiled kernels walk K in 128-wide slabs of about
-  // 0.55 us after 5 us, however few of the chip's CUs their 128 x 128 tiles occupy.
+  // Few rows: stream the weights instead of tiling.  Up to 16 rows always; up to 256 rows while a rough cost
+  // model favours it (streams_weights): the skinny kernel makes one pass over the weights per 16 rows (about
+  // 0.5 us + 5.2 bytes/ns each) after a 4 us start; the tiled kernels walk K in 128-wide slabs after 5 us,
+  // however few of the chip's CUs their 128 x 128 tiles occupy.
   const double tiled_us = 5.0 + 0.55 * static_cast<double>(K / 128);
   const bool few_rows = streams_weights(M, N, K);
   const bool off31 = M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);
