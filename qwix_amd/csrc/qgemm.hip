@@ -1366,10 +1366,34 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64)
   skinny_block<QT, NT>(A, lda, B, ldb, blockIdx.y * 16, M, blockIdx.x * (16 * NT), N, K, ep, out, ldo);
 }
 
+// The same block with smaller workgroups, for weights of hundreds of megabytes (an output projection over a
+// large vocabulary): once there are several rounds of workgroups per CU, small ones overlap each other's load,
+// reduce and store phases (one row, K 4096, N 131072: 4.9 -> 6.0 TB/s with 4 wavefronts x 16 columns).  Taken for
+// up to 4 rows only: with 16 rows the narrow column groups re-read the activation fragment too often (8 wavefronts
+// x 32 columns: between -8 % and +10 % depending on K), and at decode sizes of tens of megabytes, where all
+// workgroups fit the chip at once, the 16-wavefront shape stays ahead (58.7 MB: 4.1 TB/s against 3.2 - 3.9).
+template <int QT, int NT, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+    qgemm_skinny_small_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
+                              int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  skinny_block<QT, NT, WAVES>(A, lda, B, ldb, blockIdx.y * 16, M, blockIdx.x * (16 * NT), N, K, ep, out, ldo);
+}
+
 template <int QT>
 int launch_skinny(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
                   const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   const unsigned gy = static_cast<unsigned>((M + 15) / 16);
+  if (N * K >= (int64_t{192} << 20) && M <= 4) {
+#define QWIX_SKINNY_SMALL(NTT, WVV)                                                                                \
+  qgemm_skinny_small_kernel<QT, NTT, WVV><<<dim3(static_cast<unsigned>((N + 16 * NTT - 1) / (16 * NTT)), gy), WVV * 64, \
+                                            0, st>>>(static_cast<const uint8_t*>(a), lda,                             \
+                                                     static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),        \
+                                                     static_cast<int>(N), static_cast<int>(K), ep,                     \
+                                                     static_cast<uint8_t*>(out), ldo)
+    QWIX_SKINNY_SMALL(1, 4);
+#undef QWIX_SKINNY_SMALL
+    return check_launch("qgemm (skinny)");
+  }
 #define QWIX_SKINNY(NTT)                                                                                         \
   qgemm_skinny_kernel<QT, NTT><<<dim3(static_cast<unsigned>((N + 16 * NTT - 1) / (16 * NTT)), gy), kSkinnyWaves * 64, \
                                  0, st>>>(static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, \

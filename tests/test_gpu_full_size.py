@@ -216,3 +216,20 @@ def test_int8_gemm_with_a_short_last_round(n_extra):
   torch.cuda.synchronize()
   want = want - zu[rows].cpu().numpy().astype(np.int64)[:, None] * zv.cpu().numpy().astype(np.int64)[None, :]
   assert np.array_equal(out[rows].cpu().numpy().astype(np.float64), want * sb.cpu().numpy().astype(np.float64)[None, :])
+
+
+def test_one_row_against_a_large_vocabulary_projection():
+  """1 x 4096 x 65536 int8 (256 MB of weights: the small-workgroup shape of the weight-streaming kernel), f32 out
+  with per-column power-of-two scales: every output is an exact integer times its scale."""
+  from qwix_amd import _lib
+  M, K, N = 3, 4096, 65536
+  a = _small_ints((M, K), -3, 3, 41, torch.int8)
+  b = _small_ints((N, K), -3, 3, 42, torch.int8)
+  sb = (2.0 ** torch.randint(-2, 3, (N,), generator=torch.Generator().manual_seed(43)).float()).to(util.DEV)
+  out = torch.empty(M, N, dtype=torch.float32, device=util.DEV)
+  print('case large vocabulary', M, K, N, flush=True)
+  _lib.call('qwix_hip_qgemm', a.data_ptr(), K, b.data_ptr(), K, _lib.INT8, M, N, K, None, 0, sb.data_ptr(), _lib.F32, 0,
+            out.data_ptr(), _lib.F32, N, _lib.stream_of(a))
+  torch.cuda.synchronize()
+  want = a.cpu().numpy().astype(np.int64) @ b.cpu().numpy().astype(np.int64).T
+  assert np.array_equal(out.cpu().numpy().astype(np.float64), want * sb.cpu().numpy().astype(np.float64)[None, :])
