@@ -706,6 +706,168 @@ int dispatch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t
 }
 
 // ------------------------------------------------------------------------------------------------
+// One tile row of at most 64 rows against a wide weight (a batch of decode tokens): the weight bytes dominate
+// and every one of them is needed once.  A workgroup is 4 wavefronts side by side along N, each with all
+// 32 * TM rows and 32 columns of its own; since no two wavefronts share a weight column, the weights go from
+// global memory straight into registers (64 contiguous bytes per lane and slab, K permuted to match: lane
+// half h holds bytes 64 h .. 64 h + 63 of the 128-byte slab row, and k-step s multiplies bytes 64 h + 16 s ..),
+// while the activations go through LDS by direct-to-LDS loads as in the other kernels.  Both are fetched three
+// slabs ahead (four LDS stages, four register sets): a wavefront waits until all but its newest two groups of
+// loads have landed (vmcnt counts in order), meets the others at a barrier, issues the group three slabs ahead
+// into the stage the barrier has just freed, and multiplies.  Measured with weights from HBM, K 4096, N 14336,
+// against the 128 x 128 two-stage tile and the weight-streaming kernel: 32 rows 26.8 / 36.6 / 26.1 us, 64 rows
+// 31.5 / 36.8 / 48.0 us; 64 rows, K 8192, N 28672: 65.0 / 73.6 / 156.6 us.  With 128 rows it is no faster than
+// the two-stage tile (40.8 / 37.8 us; nor under the ragged grid, 64 groups of 128 rows: 232 / 228 us): every
+// wavefront then reads all 128 activation rows from LDS for its 32 columns, and LDS reads, not loads in
+// flight, set the pace; it is instantiated for 32 and 64 rows only.
+template <int QT, int OUT, int EPI, int TM>
+__device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, int64_t lda,
+                                               const uint8_t* __restrict__ B, int64_t ldb, int m0, int n0, int M,
+                                               int N, int K, const Epilogue& ep, uint8_t* __restrict__ out,
+                                               int64_t ldo) {
+  constexpr bool IS_INT = (QT == QWIX_INT8);
+  constexpr int BK = 128, TN = 1, DEPTH = 4;  // TM: 32-row blocks of the tile (1, 2 or 4)
+  constexpr int KSTEP = IS_INT ? 32 : 64;
+  constexpr int NK = BK / KSTEP;
+  constexpr int ASTAGE = 32 * TM * BK;  // 4 KB of activations per 32 rows and slab
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  using AccT = typename std::conditional<IS_INT, v16i, v16f>::type;
+  using FragT = typename std::conditional<IS_INT, v4i, v8i>::type;
+  AccT acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][0][r] = 0;
+
+  const int m_base = m0, n_base = n0 + wave * 32;
+  float sav[TM];
+  float sbv[TN][4][4];
+  fetch_scales<OUT, TM, TN>(ep, m_base, n_base, M, N, lane, sav, sbv);  // oldest loads: done before any slab
+
+  // activations: 32 * TM rows of 128 bytes per slab = 4 * TM pieces of 1 KB (8 rows), TM per wavefront
+  const int lr = lane >> 3, lc = (lane & 7) ^ lr;
+  uint32_t aoff[TM];
+#pragma unroll
+  for (int j = 0; j < TM; ++j)
+    aoff[j] = static_cast<uint32_t>(min(m0 + (wave * TM + j) * 8 + lr, M - 1)) * static_cast<uint32_t>(lda) + lc * 16;
+  // weights: column n_base + lane % 32, bytes 64 * (lane / 32) .. of the slab
+  const int hx = lane >> 5, x7 = lane & 7;
+  const uint32_t boff = static_cast<uint32_t>(min(n_base + (lane & 31), N - 1)) * static_cast<uint32_t>(ldb) + hx * 64;
+  v4i breg[DEPTH][4];
+  auto issue_group = [&](int kt, int st) {  // TM direct-to-LDS loads + 4 register loads per lane
+    const uint8_t* ga = A + kt * BK;
+#pragma unroll
+    for (int j = 0; j < TM; ++j) QWIX_GLDS16(ga + aoff[j], smem + st * ASTAGE + (wave * TM + j) * 1024);
+    const uint8_t* gb = B + kt * BK + boff;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) breg[st][j] = *reinterpret_cast<const v4i*>(gb + 16 * j);
+  };
+  const int a_row = (lane & 31) * BK;
+  FragT fa[2][TM];
+  auto read_a = [&](int st, int ks, int buf) {
+    const uint8_t* base = smem + st * ASTAGE + a_row;
+    if constexpr (IS_INT) {
+      const int off = ((hx * 4 + ks) ^ x7) << 4;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const v4i*>(base + i * 32 * BK + off);
+    } else {
+      const int off = ((hx * 4 + ks * 2) ^ x7) << 4;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const v4i lo = *reinterpret_cast<const v4i*>(base + i * 32 * BK + off);
+        const v4i hi = *reinterpret_cast<const v4i*>(base + i * 32 * BK + (off ^ 16));
+        fa[buf][i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+    }
+  };
+  auto barrier = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  const int KT = K / BK;
+#pragma unroll
+  for (int d = 0; d < DEPTH - 1; ++d)
+    if (d < KT) issue_group(d, d);
+  for (int kt0 = 0; kt0 < KT; kt0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int kt = kt0 + d;
+      if (kt < KT) {  // the same for the whole workgroup
+        // groups kt + 1 and kt + 2 (TM + 4 loads each) may stay in flight; vmcnt only (expcnt 7, lgkmcnt 15 open)
+        constexpr int G1 = TM + 4, G2 = 2 * G1;
+        const int rem = KT - 1 - kt;
+        __builtin_amdgcn_sched_barrier(0);
+        if (rem >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (G2 & 15) | ((G2 >> 4) << 14));
+        else if (rem == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (G1 & 15) | ((G1 >> 4) << 14));
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
+        barrier();  // slab kt is in LDS from every wavefront, and everyone is done reading slab kt - 1
+        if (kt + DEPTH - 1 < KT) issue_group(kt + DEPTH - 1, (d + DEPTH - 1) % DEPTH);
+        __builtin_amdgcn_sched_barrier(0);
+        read_a(d, 0, 0);
+#pragma unroll
+        for (int ks = 0; ks < NK; ++ks) {
+          if (ks + 1 < NK) read_a(d, ks + 1, (ks + 1) & 1);
+          FragT fb;
+          if constexpr (IS_INT) {
+            fb = breg[d][ks];
+          } else {
+            const v4i lo = breg[d][2 * ks], hi = breg[d][2 * ks + 1];
+            fb = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          }
+#pragma unroll
+          for (int i = 0; i < TM; ++i) {
+            if constexpr (IS_INT)
+              acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb, fa[ks & 1][i], acc[i][0], 0, 0, 0);
+            else
+              acc[i][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb, fa[ks & 1][i], acc[i][0], 0, 0, 0, 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+  constexpr int kLds = DEPTH * ASTAGE > 20480 ? DEPTH * ASTAGE : 20480;  // the launch provides at least 20 KB
+  staged_epilogue<OUT, EPI, TM, TN, 4, kLds>(acc, sav, sbv, ep, m_base, n_base, M, N, out, ldo, smem, wave,
+                                                        lane);
+}
+
+template <int QT, int OUT, int EPI, int TM>
+__global__ void __launch_bounds__(256)
+    qgemm_mid_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb, int M,
+                     int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
+  qgemm_mid_tile<QT, OUT, EPI, TM>(A, lda, B, ldb, 0, blockIdx.x * 128, M, N, K, ep, out, ldo);
+}
+
+template <int QT, int OUT>
+int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
+               const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  // LDS: four stages of activations, and at least the 18 KB the epilogue stages through
+#define QWIX_MID(TMM)                                                                                             \
+  {                                                                                                               \
+    constexpr size_t smem = 4 * 32 * TMM * 128 > 20480 ? 4 * 32 * TMM * 128 : 20480;                               \
+    auto kern = qgemm_mid_kernel<QT, OUT, 2, TMM>;                                                                \
+    static bool configured = false;                                                                               \
+    if (!configured) {                                                                                            \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                     \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));     \
+      if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));         \
+      configured = true;                                                                                          \
+    }                                                                                                             \
+    kern<<<dim3(static_cast<unsigned>((N + 127) / 128)), 256, smem, st>>>(                                        \
+        static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),            \
+        static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);                           \
+  }
+  if (M <= 32) QWIX_MID(1)
+  else QWIX_MID(2)
+#undef QWIX_MID
+  return check_launch("qgemm (one tile row)");
+}
+
+// ------------------------------------------------------------------------------------------------
 // Ping-pong variant of the 256 x 256 kernel for long K.  The eight wavefronts form two groups (the
 // upper and the lower 128 rows of the tile; the two wavefronts that share a SIMD are in different
 // groups) that run half a slab out of phase: while one group is in its memory phase (read all
@@ -2014,6 +2176,16 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
     if (big && K >= 256 && out_dtype != QWIX_I32) {
       if (qtype == QWIX_INT8) return dispatch_pp<QWIX_INT8>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       return dispatch_pp<QWIX_E4M3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    }
+    if (M <= 64 && out_dtype != QWIX_I32 && zu == nullptr && N * K >= (int64_t{8} << 20)) {
+      // up to 64 rows against a weight of megabytes (and too many rows, or too large a weight, for the
+      // weight-streaming kernel): the tile that keeps three slabs of weights in flight per wavefront
+      if (qtype == QWIX_INT8) {
+        if (out_dtype == QWIX_BF16) return launch_mid<QWIX_INT8, QWIX_BF16>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+        return launch_mid<QWIX_INT8, QWIX_F32>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      }
+      if (out_dtype == QWIX_BF16) return launch_mid<QWIX_E4M3, QWIX_BF16>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      return launch_mid<QWIX_E4M3, QWIX_F32>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     }
     if (qtype == QWIX_INT8) {
       if (big) return dispatch_dma<QWIX_INT8, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);

@@ -233,3 +233,31 @@ def test_one_row_against_a_large_vocabulary_projection():
   torch.cuda.synchronize()
   want = a.cpu().numpy().astype(np.int64) @ b.cpu().numpy().astype(np.int64).T
   assert np.array_equal(out.cpu().numpy().astype(np.float64), want * sb.cpu().numpy().astype(np.float64)[None, :])
+
+
+@pytest.mark.parametrize('M,K,N', [(64, 4096, 14336), (33, 2048, 8200), (20, 8192, 28672), (48, 128, 66000), (64, 384, 22016)])
+def test_decode_batch_against_a_wide_weight(M, K, N):
+  """17 to 64 rows against megabytes of weights (the deep-prefetch tile): int8 with per-row and per-column
+  power-of-two scales, f32 out; every output is an exact integer times two exact scales.  K of one, three
+  and many 128-wide slabs exercise the start and the end of the prefetch pipeline; N = 8200 a ragged last tile."""
+  from qwix_amd import _lib
+  a = _small_ints((M, K), -127, 127, 51, torch.int8)
+  b = _small_ints((N, K), -127, 127, 52, torch.int8)
+  g = torch.Generator().manual_seed(53)
+  sa = (2.0 ** torch.randint(-3, 3, (M,), generator=g).float()).to(util.DEV)
+  sb = (2.0 ** torch.randint(-3, 3, (N,), generator=g).float()).to(util.DEV)
+  out = torch.full((M, N), float('nan'), dtype=torch.float32, device=util.DEV)
+  print('case decode batch', M, K, N, flush=True)
+  _lib.call('qwix_hip_qgemm', a.data_ptr(), K, b.data_ptr(), K, _lib.INT8, M, N, K, sa.data_ptr(), _lib.F32, sb.data_ptr(),
+            _lib.F32, 0, out.data_ptr(), _lib.F32, N, _lib.stream_of(a))
+  torch.cuda.synchronize()
+  want = (a.double() @ b.double().T) * sa.double()[:, None] * sb.double()[None, :]
+  assert torch.equal(out.double(), want)
+  # bf16 out through bf16 scales: the rounding flags of the run-time epilogue
+  outb = torch.empty(M, N, dtype=torch.bfloat16, device=util.DEV)
+  sab, sbb = sa.to(torch.bfloat16), sb.to(torch.bfloat16)
+  _lib.call('qwix_hip_qgemm', a.data_ptr(), K, b.data_ptr(), K, _lib.INT8, M, N, K, sab.data_ptr(), _lib.BF16,
+            sbb.data_ptr(), _lib.BF16, 0, outb.data_ptr(), _lib.BF16, N, _lib.stream_of(a))
+  accb = (a.double() @ b.double().T).float().to(torch.bfloat16)
+  wantb = (accb * sab[:, None]) * sbb[None, :]
+  assert torch.equal(outb, wantb)
