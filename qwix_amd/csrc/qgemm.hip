@@ -711,22 +711,29 @@ int dispatch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t
 // 32 * TM rows and 32 columns of its own; since no two wavefronts share a weight column, the weights go from
 // global memory straight into registers (64 contiguous bytes per lane and slab, K permuted to match: lane
 // half h holds bytes 64 h .. 64 h + 63 of the 128-byte slab row, and k-step s multiplies bytes 64 h + 16 s ..),
-// while the activations go through LDS by direct-to-LDS loads as in the other kernels.  Both are fetched three
-// slabs ahead (four LDS stages, four register sets): a wavefront waits until all but its newest two groups of
-// loads have landed (vmcnt counts in order), meets the others at a barrier, issues the group three slabs ahead
-// into the stage the barrier has just freed, and multiplies.  Measured with weights from HBM, K 4096, N 14336,
-// against the 128 x 128 two-stage tile and the weight-streaming kernel: 32 rows 26.8 / 36.6 / 26.1 us, 64 rows
-// 31.5 / 36.8 / 48.0 us; 64 rows, K 8192, N 28672: 65.0 / 73.6 / 156.6 us.  With 128 rows it is no faster than
+// while the activations go through LDS by direct-to-LDS loads as in the other kernels.  Both are fetched
+// DEPTH - 1 slabs ahead (DEPTH LDS stages, DEPTH register sets; 8 in the build): a wavefront waits until all
+// but its newest DEPTH - 2 groups of loads have landed (vmcnt counts in order; 6 groups of at most 6 loads stay
+// under the counter's limit of 63), meets the others at a barrier, issues the group DEPTH - 1 slabs ahead into
+// the stage the barrier has just freed, and multiplies.  Measured with weights from HBM, K 4096, N 14336,
+// against the 128 x 128 two-stage tile and the weight-streaming kernel: 32 rows 26.2 / 36.6 / 26.1 us, 64 rows
+// 26.6 / 36.8 / 48.0 us; 64 rows, K 8192, N 28672: 57.0 / 73.6 / 156.6 us (with four stages and compiler-
+// tracked loads: 31.5 and 65.0 us for the two 64-row cases).  With 128 rows it is no faster than
 // the two-stage tile (40.8 / 37.8 us; nor under the ragged grid, 64 groups of 128 rows: 232 / 228 us): every
 // wavefront then reads all 128 activation rows from LDS for its 32 columns, and LDS reads, not loads in
 // flight, set the pace; it is instantiated for 32 and 64 rows only.
-template <int QT, int OUT, int EPI, int TM>
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {  // vmcnt only: expcnt 7 and lgkmcnt 15 stay open
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+template <int QT, int OUT, int EPI, int TM, int DEPTH>
 __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, int64_t lda,
                                                const uint8_t* __restrict__ B, int64_t ldb, int m0, int n0, int M,
                                                int N, int K, const Epilogue& ep, uint8_t* __restrict__ out,
                                                int64_t ldo) {
   constexpr bool IS_INT = (QT == QWIX_INT8);
-  constexpr int BK = 128, TN = 1, DEPTH = 4;  // TM: 32-row blocks of the tile (1, 2 or 4)
+  constexpr int BK = 128, TN = 1;  // TM: 32-row blocks of the tile; DEPTH: slabs of loads kept going, plus one
   constexpr int KSTEP = IS_INT ? 32 : 64;
   constexpr int NK = BK / KSTEP;
   constexpr int ASTAGE = 32 * TM * BK;  // 4 KB of activations per 32 rows and slab
@@ -761,9 +768,17 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
     const uint8_t* ga = A + kt * BK;
 #pragma unroll
     for (int j = 0; j < TM; ++j) QWIX_GLDS16(ga + aoff[j], smem + st * ASTAGE + (wave * TM + j) * 1024);
-    const uint8_t* gb = B + kt * BK + boff;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) breg[st][j] = *reinterpret_cast<const v4i*>(gb + 16 * j);
+    // Issued as asm so that the compiler does not track them: its own waits for these registers, merged over
+    // the loop's back edge, come out as vmcnt(0) once per trip and would drain every load in flight.  The
+    // explicit waits below are what guarantees that a register set has landed before it is multiplied.
+    const uint8_t* gb = B + kt * BK;
+    asm volatile("global_load_dwordx4 %0, %4, %5\n\t"
+                 "global_load_dwordx4 %1, %4, %5 offset:16\n\t"
+                 "global_load_dwordx4 %2, %4, %5 offset:32\n\t"
+                 "global_load_dwordx4 %3, %4, %5 offset:48"
+                 : "=&v"(breg[st][0]), "=&v"(breg[st][1]), "=&v"(breg[st][2]), "=&v"(breg[st][3])
+                 : "v"(boff), "s"(gb)
+                 : "memory");
   };
   const int a_row = (lane & 31) * BK;
   FragT fa[2][TM];
@@ -798,13 +813,20 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
     for (int d = 0; d < DEPTH; ++d) {
       const int kt = kt0 + d;
       if (kt < KT) {  // the same for the whole workgroup
-        // groups kt + 1 and kt + 2 (TM + 4 loads each) may stay in flight; vmcnt only (expcnt 7, lgkmcnt 15 open)
-        constexpr int G1 = TM + 4, G2 = 2 * G1;
+        // the groups after kt (TM + 4 loads each, at most DEPTH - 2 of them) may stay in flight
+        constexpr int G = TM + 4;
+        static_assert(DEPTH == 4 || DEPTH == 8, "the wait below lists the cases");
         const int rem = KT - 1 - kt;
         __builtin_amdgcn_sched_barrier(0);
-        if (rem >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (G2 & 15) | ((G2 >> 4) << 14));
-        else if (rem == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (G1 & 15) | ((G1 >> 4) << 14));
-        else __builtin_amdgcn_s_waitcnt(0x0F70);
+        switch (rem < DEPTH - 2 ? rem : DEPTH - 2) {
+          case 0: wait_vmcnt<0>(); break;
+          case 1: wait_vmcnt<G>(); break;
+          case 2: wait_vmcnt<2 * G>(); break;
+          case 3: wait_vmcnt<3 * G>(); break;
+          case 4: wait_vmcnt<4 * G>(); break;
+          case 5: wait_vmcnt<5 * G>(); break;
+          default: wait_vmcnt<6 * G>(); break;
+        }
         barrier();  // slab kt is in LDS from every wavefront, and everyone is done reading slab kt - 1
         if (kt + DEPTH - 1 < KT) issue_group(kt + DEPTH - 1, (d + DEPTH - 1) % DEPTH);
         __builtin_amdgcn_sched_barrier(0);
@@ -835,21 +857,22 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
                                                         lane);
 }
 
-template <int QT, int OUT, int EPI, int TM>
+template <int QT, int OUT, int EPI, int TM, int DEPTH>
 __global__ void __launch_bounds__(256)
     qgemm_mid_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb, int M,
                      int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
-  qgemm_mid_tile<QT, OUT, EPI, TM>(A, lda, B, ldb, 0, blockIdx.x * 128, M, N, K, ep, out, ldo);
+  qgemm_mid_tile<QT, OUT, EPI, TM, DEPTH>(A, lda, B, ldb, 0, blockIdx.x * 128, M, N, K, ep, out, ldo);
 }
 
 template <int QT, int OUT>
 int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
                const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
-  // LDS: four stages of activations, and at least the 18 KB the epilogue stages through
+  constexpr int kDepth = 8;
+  // LDS: kDepth stages of activations, and at least the 18 KB the epilogue stages through
 #define QWIX_MID(TMM)                                                                                             \
   {                                                                                                               \
-    constexpr size_t smem = 4 * 32 * TMM * 128 > 20480 ? 4 * 32 * TMM * 128 : 20480;                               \
-    auto kern = qgemm_mid_kernel<QT, OUT, 2, TMM>;                                                                \
+    constexpr size_t smem = kDepth * 32 * TMM * 128 > 20480 ? kDepth * 32 * TMM * 128 : 20480;                     \
+    auto kern = qgemm_mid_kernel<QT, OUT, 2, TMM, kDepth>;                                                        \
     static bool configured = false;                                                                               \
     if (!configured) {                                                                                            \
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                     \
