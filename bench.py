@@ -352,18 +352,18 @@ class GemvW4(Workload):
 
 
 class QdotDecode(Workload):
-  """Dynamic-range w8a8 at decode size: per-token int8 quantize of M <= 16 tokens + the skinny quantized
-  GEMM, which streams the int8 weight once (HBM-bound)."""
+  """Dynamic-range w8a8 at decode size: per-token int8 quantize of a few tokens + the quantized GEMM that
+  streams the int8 weight once (HBM-bound): the skinny kernel up to 16 tokens, the 64-row tile above."""
 
   bound = 'hbm'
   graph_ok = False
 
-  def __init__(self, name, M, K, N):
+  def __init__(self, name, M, K, N, kernel_name='qgemm_skinny_kernel'):
     self.name, self.M, self.K, self.N = name, M, K, N
     self.dtype = 'int8'
     self.metric = 'w8a8 int8 decode GB/s (activation quantize included)'
     self.unit = 'GB/s'
-    self.kernel_name = 'qgemm_skinny_kernel'
+    self.kernel_name = kernel_name
 
   def setup(self, dev):
     import torch
@@ -796,6 +796,8 @@ WORKLOADS = {
     'quantize_act_4096': lambda: QuantizeRows('quantize_act_4096', 4096, 4096, 'int8'),
     'quantize_act_8192_fp8': lambda: QuantizeRows('quantize_act_8192_fp8', 8192, 8192, 'float8_e4m3fn'),
     'w8a8_decode_m16': lambda: QdotDecode('w8a8_decode_m16', 16, 4096, 14336),
+    'w8a8_decode_m64': lambda: QdotDecode('w8a8_decode_m64', 64, 4096, 14336, 'qgemm_mid_kernel'),
+    'w8a8_decode_m64_k8192': lambda: QdotDecode('w8a8_decode_m64_k8192', 64, 8192, 28672, 'qgemm_mid_kernel'),
     'w8a8_decode_m16_k2048': lambda: QdotDecode('w8a8_decode_m16_k2048', 16, 2048, 8192),
     'w8a8_decode_m16_k2048_fused': lambda: QdotDecodeFused('w8a8_decode_m16_k2048_fused', 16, 2048, 8192),
     'c2_gemv_w4_m1': lambda: GemvW4('c2_gemv_w4_m1', 1, 4096, 14336, 128),
@@ -818,7 +820,7 @@ WORKLOADS = {
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
 }
 DEFAULT = 'c3_int8_w8a8_4096'
-EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
+EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
          'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'moe_ragged_int8_8x1024',
          'moe_ragged_int8_64x128', 'moe_decode_int8_64x4', 'quantize_weight_fp8_block128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 

@@ -707,7 +707,7 @@ int dispatch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t
 
 // ------------------------------------------------------------------------------------------------
 // One tile row of at most 64 rows against a wide weight (a batch of decode tokens): the weight bytes dominate
-// and every one of them is needed once.  A workgroup is 4 wavefronts side by side along N, each with all
+// and every one of them is needed once.  A workgroup is NW (2 or 4) wavefronts side by side along N, each with all
 // 32 * TM rows and 32 columns of its own; since no two wavefronts share a weight column, the weights go from
 // global memory straight into registers (64 contiguous bytes per lane and slab, K permuted to match: lane
 // half h holds bytes 64 h .. 64 h + 63 of the 128-byte slab row, and k-step s multiplies bytes 64 h + 16 s ..),
@@ -727,7 +727,7 @@ __device__ __forceinline__ void wait_vmcnt() {  // vmcnt only: expcnt 7 and lgkm
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <int QT, int OUT, int EPI, int TM, int DEPTH>
+template <int QT, int OUT, int EPI, int TM, int DEPTH, int NW>
 __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, int64_t lda,
                                                const uint8_t* __restrict__ B, int64_t ldb, int m0, int n0, int M,
                                                int N, int K, const Epilogue& ep, uint8_t* __restrict__ out,
@@ -737,6 +737,8 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
   constexpr int KSTEP = IS_INT ? 32 : 64;
   constexpr int NK = BK / KSTEP;
   constexpr int ASTAGE = 32 * TM * BK;  // 4 KB of activations per 32 rows and slab
+  constexpr int PW = 4 * TM / NW;       // 1 KB pieces (8 rows) of a slab of activations that a wavefront fetches
+  static_assert(PW * NW == 4 * TM, "the wavefronts share the activation rows evenly");
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -754,20 +756,20 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
   float sbv[TN][4][4];
   fetch_scales<OUT, TM, TN>(ep, m_base, n_base, M, N, lane, sav, sbv);  // oldest loads: done before any slab
 
-  // activations: 32 * TM rows of 128 bytes per slab = 4 * TM pieces of 1 KB (8 rows), TM per wavefront
+  // activations: 32 * TM rows of 128 bytes per slab = 4 * TM pieces of 1 KB (8 rows), PW per wavefront
   const int lr = lane >> 3, lc = (lane & 7) ^ lr;
-  uint32_t aoff[TM];
+  uint32_t aoff[PW];
 #pragma unroll
-  for (int j = 0; j < TM; ++j)
-    aoff[j] = static_cast<uint32_t>(min(m0 + (wave * TM + j) * 8 + lr, M - 1)) * static_cast<uint32_t>(lda) + lc * 16;
+  for (int j = 0; j < PW; ++j)
+    aoff[j] = static_cast<uint32_t>(min(m0 + (wave * PW + j) * 8 + lr, M - 1)) * static_cast<uint32_t>(lda) + lc * 16;
   // weights: column n_base + lane % 32, bytes 64 * (lane / 32) .. of the slab
   const int hx = lane >> 5, x7 = lane & 7;
   const uint32_t boff = static_cast<uint32_t>(min(n_base + (lane & 31), N - 1)) * static_cast<uint32_t>(ldb) + hx * 64;
   v4i breg[DEPTH][4];
-  auto issue_group = [&](int kt, int st) {  // TM direct-to-LDS loads + 4 register loads per lane
+  auto issue_group = [&](int kt, int st) {  // PW direct-to-LDS loads + 4 register loads per lane
     const uint8_t* ga = A + kt * BK;
 #pragma unroll
-    for (int j = 0; j < TM; ++j) QWIX_GLDS16(ga + aoff[j], smem + st * ASTAGE + (wave * TM + j) * 1024);
+    for (int j = 0; j < PW; ++j) QWIX_GLDS16(ga + aoff[j], smem + st * ASTAGE + (wave * PW + j) * 1024);
     // Issued as asm so that the compiler does not track them: its own waits for these registers, merged over
     // the loop's back edge, come out as vmcnt(0) once per trip and would drain every load in flight.  The
     // explicit waits below are what guarantees that a register set has landed before it is multiplied.
@@ -813,8 +815,9 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
     for (int d = 0; d < DEPTH; ++d) {
       const int kt = kt0 + d;
       if (kt < KT) {  // the same for the whole workgroup
-        // the groups after kt (TM + 4 loads each, at most DEPTH - 2 of them) may stay in flight
-        constexpr int G = TM + 4;
+        // the groups after kt (PW + 4 loads each, at most DEPTH - 2 of them) may stay in flight
+        constexpr int G = PW + 4;
+        static_assert(6 * G <= 63, "vmcnt is a 6-bit counter");
         static_assert(DEPTH == 4 || DEPTH == 8, "the wait below lists the cases");
         const int rem = KT - 1 - kt;
         __builtin_amdgcn_sched_barrier(0);
@@ -853,15 +856,15 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
     }
   }
   constexpr int kLds = DEPTH * ASTAGE > 20480 ? DEPTH * ASTAGE : 20480;  // the launch provides at least 20 KB
-  staged_epilogue<OUT, EPI, TM, TN, 4, kLds>(acc, sav, sbv, ep, m_base, n_base, M, N, out, ldo, smem, wave,
-                                                        lane);
+  staged_epilogue<OUT, EPI, TM, TN, NW, kLds>(acc, sav, sbv, ep, m_base, n_base, M, N, out, ldo, smem, wave,
+                                                         lane);
 }
 
-template <int QT, int OUT, int EPI, int TM, int DEPTH>
-__global__ void __launch_bounds__(256)
+template <int QT, int OUT, int EPI, int TM, int DEPTH, int NW>
+__global__ void __launch_bounds__(64 * NW)
     qgemm_mid_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb, int M,
                      int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
-  qgemm_mid_tile<QT, OUT, EPI, TM, DEPTH>(A, lda, B, ldb, 0, blockIdx.x * 128, M, N, K, ep, out, ldo);
+  qgemm_mid_tile<QT, OUT, EPI, TM, DEPTH, NW>(A, lda, B, ldb, 0, blockIdx.x * (32 * NW), M, N, K, ep, out, ldo);
 }
 
 template <int QT, int OUT>
@@ -869,10 +872,10 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
                const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   constexpr int kDepth = 8;
   // LDS: kDepth stages of activations, and at least the 18 KB the epilogue stages through
-#define QWIX_MID(TMM)                                                                                             \
+#define QWIX_MID(TMM, NWW)                                                                                        \
   {                                                                                                               \
     constexpr size_t smem = kDepth * 32 * TMM * 128 > 20480 ? kDepth * 32 * TMM * 128 : 20480;                     \
-    auto kern = qgemm_mid_kernel<QT, OUT, 2, TMM, kDepth>;                                                        \
+    auto kern = qgemm_mid_kernel<QT, OUT, 2, TMM, kDepth, NWW>;                                                   \
     static bool configured = false;                                                                               \
     if (!configured) {                                                                                            \
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                     \
@@ -880,12 +883,21 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
       if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));         \
       configured = true;                                                                                          \
     }                                                                                                             \
-    kern<<<dim3(static_cast<unsigned>((N + 127) / 128)), 256, smem, st>>>(                                        \
+    kern<<<dim3(static_cast<unsigned>((N + 32 * NWW - 1) / (32 * NWW))), 64 * NWW, smem, st>>>(                   \
         static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),            \
         static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);                           \
   }
-  if (M <= 32) QWIX_MID(1)
-  else QWIX_MID(2)
+  // Workgroups of 2 wavefronts (64 columns) for up to 32 rows, and for 64 rows while 128-column workgroups
+  // would leave CUs without one: twice the workgroups, twice the CUs that pull weights.  Measured, weights
+  // from HBM, 2 / 4 wavefronts, K 4096, N 14336: 32 rows 17.5 / 23.4 us, 64 rows 20.3 / 26.4 us; K 8192,
+  // N 8192: 23.9 / 37.4 and 30.5 / 42.8 us; K 8192, N 28672: 51.8 / 54.2 and 62.6 / 55.0 us.
+  const bool narrow = (N + 127) / 128 < 192;
+  if (M <= 32) {
+    QWIX_MID(1, 2)
+  } else {
+    if (narrow) QWIX_MID(2, 2)
+    else QWIX_MID(2, 4)
+  }
 #undef QWIX_MID
   return check_launch("qgemm (one tile row)");
 }
@@ -1841,7 +1853,7 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
                       const int32_t* zv, void* out, int out_dtype, int64_t ldo, void* stream, void* workspace = nullptr,
                       size_t workspace_bytes = 0);
 static int splitk_plan(int64_t M, int64_t N, int64_t K, double other_us);
-static bool streams_weights(int64_t M, int64_t N, int64_t K);
+static bool streams_weights(int64_t M, int64_t N, int64_t K, bool one_tile_row = false);
 
 // Dtype chain of the reference epilogue: int32 adopts the first scale's dtype (through f32); a
 // float accumulator starts in acc_dtype; each multiply happens in the promotion of both sides.
@@ -2101,7 +2113,7 @@ __global__ void __launch_bounds__(256)
 }
 
 // The rule of qgemm_impl for taking the weight-streaming kernel (see there for the model).
-static bool streams_weights(int64_t M, int64_t N, int64_t K) {
+static bool streams_weights(int64_t M, int64_t N, int64_t K, bool one_tile_row) {
   const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
   const double passes = static_cast<double>((M + 15) / 16);
   const double skinny_us = 4.0 + passes * (0.5 + static_cast<double>(N) * static_cast<double>(K) / 5.2e6);
@@ -2112,7 +2124,18 @@ static bool streams_weights(int64_t M, int64_t N, int64_t K) {
   const double slab_us = 0.95 * static_cast<double>(K / 128) * rounds;
   const double read_us = static_cast<double>(N) * static_cast<double>(K) / 3.8e6;
   const double tiled_us = 5.0 + (slab_us > read_us ? slab_us : read_us);
-  if (M <= 32) return M <= 16 || skinny_us < tiled_us;
+  if (M <= 16) return true;
+  if (M <= 32 && one_tile_row) {
+    // The one-tile-row kernel is there for this call (qgemm_impl checks what it needs).  With 32 rows and
+    // 64-column workgroups it was measured, weights from HBM, at K 4096, N 4096 / 14336 / 28672: 14.2 / 17.5 /
+    // 29.5 us; K 8192, N 8192 / 28672: 23.9 / 51.8 us; K 2048, N 8192: 9.7 us (the two passes of the
+    // weight-streaming kernel: 11.3 / 25.9 / 30.0, 33.4 / 54.1, 9.7 us): 0.29 us per slab of K while the
+    // workgroups are few, 4.8 bytes/ns of weights once they fill the chip.
+    const double slabs_us = 0.29 * static_cast<double>(K / 128);
+    const double bytes_us = static_cast<double>(N) * static_cast<double>(K) / 4.8e6;
+    return skinny_us < 5.0 + (slabs_us > bytes_us ? slabs_us : bytes_us);
+  }
+  if (M <= 32) return skinny_us < tiled_us;
   // more rows: the comparison that was tuned with weights that stay in the last-level cache between calls
   return M <= 256 && tiles128 <= 256 && skinny_us < 5.0 + 0.55 * static_cast<double>(K / 128);
 }
@@ -2177,7 +2200,10 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
   // 0.5 us + 5.2 bytes/ns each) after a 4 us start; the tiled kernels walk K in 128-wide slabs after 5 us,
   // however few of the chip's CUs their 128 x 128 tiles occupy.
   const double tiled_us = 5.0 + 0.55 * static_cast<double>(K / 128);
-  const bool few_rows = streams_weights(M, N, K);
+  // what the one-tile-row kernel (launch_mid) needs
+  const bool mid_ok = M > 16 && M <= 64 && K % 128 == 0 && out_dtype != QWIX_I32 && zu == nullptr &&
+                      N * K >= (int64_t{8} << 20) && M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);
+  const bool few_rows = streams_weights(M, N, K, mid_ok);
   const bool off31 = M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);
   if (workspace != nullptr && zu == nullptr && out_dtype != QWIX_I32 && off31) {
     // only against the tiled kernels: where the weight-streaming kernel is chosen its own model has spoken
@@ -2200,7 +2226,7 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
       if (qtype == QWIX_INT8) return dispatch_pp<QWIX_INT8>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       return dispatch_pp<QWIX_E4M3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     }
-    if (M <= 64 && out_dtype != QWIX_I32 && zu == nullptr && N * K >= (int64_t{8} << 20)) {
+    if (mid_ok) {
       // up to 64 rows against a weight of megabytes (and too many rows, or too large a weight, for the
       // weight-streaming kernel): the tile that keeps three slabs of weights in flight per wavefront
       if (qtype == QWIX_INT8) {

@@ -570,7 +570,9 @@ __global__ void __launch_bounds__(256)
   __shared__ float red[SRC == 2 ? 2 : 1][SRC == 2 ? 4 : 1][SRC == 2 ? 16 : 1][EV];
   int64_t o, t, c0;
   int chunk;
-  col_decode<D>(gm, blockIdx.x, &o, &t, &chunk, &c0);
+  // After a calibration pass over the same array the blocks run in the opposite order: what that pass read
+  // last is what the last-level cache still holds, so it is re-read first.
+  col_decode<D>(gm, SRC == 0 ? gridDim.x - 1 - blockIdx.x : blockIdx.x, &o, &t, &chunk, &c0);
   const bool col_ok = c0 < gm.inner;  // idle threads stay for the barriers
   const int rb = threadIdx.x >> 4;
   const int64_t sidx = (o * gm.ntiles + t) * gm.inner + c0;

@@ -235,11 +235,13 @@ def test_one_row_against_a_large_vocabulary_projection():
   assert np.array_equal(out.cpu().numpy().astype(np.float64), want * sb.cpu().numpy().astype(np.float64)[None, :])
 
 
-@pytest.mark.parametrize('M,K,N', [(64, 4096, 14336), (33, 2048, 8200), (20, 8192, 28672), (48, 128, 66000), (64, 384, 22016)])
+@pytest.mark.parametrize('M,K,N', [(64, 4096, 14336), (33, 2048, 8200), (20, 8192, 28672), (48, 128, 66000), (64, 384, 22016),
+                                   (32, 4096, 14336), (24, 8192, 8192), (17, 2048, 28700), (64, 4096, 28672)])
 def test_decode_batch_against_a_wide_weight(M, K, N):
   """17 to 64 rows against megabytes of weights (the deep-prefetch tile): int8 with per-row and per-column
   power-of-two scales, f32 out; every output is an exact integer times two exact scales.  K of one, three
-  and many 128-wide slabs exercise the start and the end of the prefetch pipeline; N = 8200 a ragged last tile."""
+  and many 128-wide slabs exercise the start and the end of the prefetch pipeline; N = 8200 a ragged last tile.
+  The shapes cover the 32-row and the 64-row tile, and workgroups of 64 and of 128 columns."""
   from qwix_amd import _lib
   a = _small_ints((M, K), -127, 127, 51, torch.int8)
   b = _small_ints((N, K), -127, 127, 52, torch.int8)
@@ -261,3 +263,23 @@ def test_decode_batch_against_a_wide_weight(M, K, N):
   accb = (a.double() @ b.double().T).float().to(torch.bfloat16)
   wantb = (accb * sab[:, None]) * sbb[None, :]
   assert torch.equal(outb, wantb)
+
+
+@pytest.mark.parametrize('M,K,N', [(64, 4096, 14336), (32, 8192, 8192), (40, 2048, 28700)])
+def test_fp8_decode_batch_against_a_wide_weight(M, K, N):
+  """The same tile with e4m3 operands: values in -2..2 are exact in e4m3 and every sum stays below 2^24, so the
+  f32 output must equal the integer product; power-of-two scales keep the bf16 epilogue exact as well."""
+  from qwix_amd import _lib
+  a_i = _small_ints((M, K), -2, 2, 61, torch.int8)
+  b_i = _small_ints((N, K), -2, 2, 62, torch.int8)
+  a, b = a_i.to(torch.float32).to(torch.float8_e4m3fn), b_i.to(torch.float32).to(torch.float8_e4m3fn)
+  g = torch.Generator().manual_seed(63)
+  sa = (2.0 ** torch.randint(-3, 3, (M,), generator=g).float()).to(util.DEV)
+  sb = (2.0 ** torch.randint(-3, 3, (N,), generator=g).float()).to(util.DEV)
+  out = torch.full((M, N), float('nan'), dtype=torch.float32, device=util.DEV)
+  print('case fp8 decode batch', M, K, N, flush=True)
+  _lib.call('qwix_hip_qgemm', a.data_ptr(), K, b.data_ptr(), K, _lib.E4M3, M, N, K, sa.data_ptr(), _lib.F32, sb.data_ptr(),
+            _lib.F32, _lib.F32, out.data_ptr(), _lib.F32, N, _lib.stream_of(a))
+  torch.cuda.synchronize()
+  want = (a_i.double() @ b_i.double().T) * sa.double()[:, None] * sb.double()[None, :]
+  assert torch.equal(out.double(), want)
