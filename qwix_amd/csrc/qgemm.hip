@@ -718,10 +718,11 @@ int dispatch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t
 // the stage the barrier has just freed, and multiplies.  Measured with weights from HBM, K 4096, N 14336,
 // against the 128 x 128 two-stage tile and the weight-streaming kernel: 32 rows 26.2 / 36.6 / 26.1 us, 64 rows
 // 26.6 / 36.8 / 48.0 us; 64 rows, K 8192, N 28672: 57.0 / 73.6 / 156.6 us (with four stages and compiler-
-// tracked loads: 31.5 and 65.0 us for the two 64-row cases).  With 128 rows it is no faster than
-// the two-stage tile (40.8 / 37.8 us; nor under the ragged grid, 64 groups of 128 rows: 232 / 228 us): every
-// wavefront then reads all 128 activation rows from LDS for its 32 columns, and LDS reads, not loads in
-// flight, set the pace; it is instantiated for 32 and 64 rows only.
+// tracked loads: 31.5 and 65.0 us for the two 64-row cases).  Workgroups of 64 columns then brought the 64-row
+// case at N 14336 to 20.4 us and the 32-row case to 17.6 us.  With 128 rows every wavefront reads all 128
+// activation rows from LDS per slab for its 32 columns, and a workgroup's stages take 96 KB, one workgroup per
+// CU: that variant (six stages) pays while one round of 64-column workgroups covers N, and not under the
+// ragged grid (64 groups of 128 rows: 232 against 228 us for the two-stage tile).
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {  // vmcnt only: expcnt 7 and lgkmcnt 15 stay open
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
@@ -817,8 +818,8 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
       if (kt < KT) {  // the same for the whole workgroup
         // the groups after kt (PW + 4 loads each, at most DEPTH - 2 of them) may stay in flight
         constexpr int G = PW + 4;
-        static_assert(6 * G <= 63, "vmcnt is a 6-bit counter");
-        static_assert(DEPTH == 4 || DEPTH == 8, "the wait below lists the cases");
+        static_assert((DEPTH - 2) * G <= 63, "vmcnt is a 6-bit counter");
+        static_assert(DEPTH >= 4 && DEPTH <= 8, "the wait below lists the cases");
         const int rem = KT - 1 - kt;
         __builtin_amdgcn_sched_barrier(0);
         switch (rem < DEPTH - 2 ? rem : DEPTH - 2) {
@@ -827,8 +828,8 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
           case 2: wait_vmcnt<2 * G>(); break;
           case 3: wait_vmcnt<3 * G>(); break;
           case 4: wait_vmcnt<4 * G>(); break;
-          case 5: wait_vmcnt<5 * G>(); break;
-          default: wait_vmcnt<6 * G>(); break;
+          case 5: wait_vmcnt<(5 * G < 63 ? 5 * G : 63)>(); break;  // 5, 6: not reached unless DEPTH is 7, 8
+          default: wait_vmcnt<(6 * G < 63 ? 6 * G : 63)>(); break;
         }
         barrier();  // slab kt is in LDS from every wavefront, and everyone is done reading slab kt - 1
         if (kt + DEPTH - 1 < KT) issue_group(kt + DEPTH - 1, (d + DEPTH - 1) % DEPTH);
@@ -870,10 +871,10 @@ __global__ void __launch_bounds__(64 * NW)
 template <int QT, int OUT>
 int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
                const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
-  constexpr int kDepth = 8;
   // LDS: kDepth stages of activations, and at least the 18 KB the epilogue stages through
 #define QWIX_MID(TMM, NWW)                                                                                        \
   {                                                                                                               \
+    constexpr int kDepth = TMM == 4 ? 6 : 8; /* 128 rows: 12 loads per group, 4 groups stay under vmcnt's 63 */    \
     constexpr size_t smem = kDepth * 32 * TMM * 128 > 20480 ? kDepth * 32 * TMM * 128 : 20480;                     \
     auto kern = qgemm_mid_kernel<QT, OUT, 2, TMM, kDepth, NWW>;                                                   \
     static bool configured = false;                                                                               \
@@ -894,6 +895,8 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
   const bool narrow = (N + 127) / 128 < 192;
   if (M <= 32) {
     QWIX_MID(1, 2)
+  } else if (M > 64) {
+    QWIX_MID(4, 2)
   } else {
     if (narrow) QWIX_MID(2, 2)
     else QWIX_MID(2, 4)
@@ -2201,7 +2204,11 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
   // however few of the chip's CUs their 128 x 128 tiles occupy.
   const double tiled_us = 5.0 + 0.55 * static_cast<double>(K / 128);
   // what the one-tile-row kernel (launch_mid) needs
-  const bool mid_ok = M > 16 && M <= 64 && K % 128 == 0 && out_dtype != QWIX_I32 && zu == nullptr &&
+  // (65 to 128 rows: one workgroup per CU for its 96 KB of LDS stages, so only while one round of 64-column
+  // workgroups covers N.  Measured against the 128 x 128 tile, int8, weights from HBM, K 4096, N 4096 / 14336:
+  // 25.9 / 29.3 against 37.1 / 38.7 us; K 8192, N 8192: 43.1 against 67.7 us; but K 8192, N 28672: 90.4
+  // against 77.0 us.)
+  const bool mid_ok = M > 16 && (M <= 64 || (M <= 128 && (N + 63) / 64 <= 256)) && K % 128 == 0 && out_dtype != QWIX_I32 && zu == nullptr &&
                       N * K >= (int64_t{8} << 20) && M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);
   const bool few_rows = streams_weights(M, N, K, mid_ok);
   const bool off31 = M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);
