@@ -874,7 +874,7 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
   // LDS: kDepth stages of activations, and at least the 18 KB the epilogue stages through
 #define QWIX_MID(TMM, NWW)                                                                                        \
   {                                                                                                               \
-    constexpr int kDepth = TMM == 4 ? 6 : 8; /* 128 rows: 12 loads per group, 4 groups stay under vmcnt's 63 */    \
+    constexpr int kDepth = (4 * TMM / NWW + 4) * 6 <= 63 ? 8 : 6; /* groups in flight stay under vmcnt's 63 */      \
     constexpr size_t smem = kDepth * 32 * TMM * 128 > 20480 ? kDepth * 32 * TMM * 128 : 20480;                     \
     auto kern = qgemm_mid_kernel<QT, OUT, 2, TMM, kDepth, NWW>;                                                   \
     static bool configured = false;                                                                               \
@@ -893,10 +893,16 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
   // from HBM, 2 / 4 wavefronts, K 4096, N 14336: 32 rows 17.5 / 23.4 us, 64 rows 20.3 / 26.4 us; K 8192,
   // N 8192: 23.9 / 37.4 and 30.5 / 42.8 us; K 8192, N 28672: 51.8 / 54.2 and 62.6 / 55.0 us.
   const bool narrow = (N + 127) / 128 < 192;
-  if (M <= 32) {
+  // Up to N 8192 and 64 rows a workgroup is a single wavefront (32 columns): 10 to 15 % less again (64 rows,
+  // K 4096, N 4096 / 6144: 16.6 / 16.3 against 19.6 / 18.7 us; K 14336, N 4096: 44.1 against 52.6 us).
+  if (M <= 64 && (N + 63) / 64 <= 128) {
+    if (M <= 32) QWIX_MID(1, 1)
+    else QWIX_MID(2, 1)
+  } else if (M <= 32) {
     QWIX_MID(1, 2)
   } else if (M > 64) {
-    QWIX_MID(4, 2)
+    if ((N + 63) / 64 <= 256) QWIX_MID(4, 2)
+    else QWIX_MID(4, 4)
   } else {
     if (narrow) QWIX_MID(2, 2)
     else QWIX_MID(2, 4)
@@ -2134,9 +2140,18 @@ static bool streams_weights(int64_t M, int64_t N, int64_t K, bool one_tile_row) 
     // 29.5 us; K 8192, N 8192 / 28672: 23.9 / 51.8 us; K 2048, N 8192: 9.7 us (the two passes of the
     // weight-streaming kernel: 11.3 / 25.9 / 30.0, 33.4 / 54.1, 9.7 us): 0.29 us per slab of K while the
     // workgroups are few, 4.8 bytes/ns of weights once they fill the chip.
-    const double slabs_us = 0.29 * static_cast<double>(K / 128);
+    // Single-wavefront workgroups (N up to 8192): 0.26 us per slab (K 4096, N 4096 / 6144: 13.1 / 13.0 us,
+    // K 8192, N 8192: 22.2 us, K 14336, N 4096: 34.6 us against 11.6 / 14.5, 23.9, 28.9 us).
+    const double slabs_us = (N <= 8192 ? 0.26 : 0.29) * static_cast<double>(K / 128);
     const double bytes_us = static_cast<double>(N) * static_cast<double>(K) / 4.8e6;
     return skinny_us < 5.0 + (slabs_us > bytes_us ? slabs_us : bytes_us);
+  }
+  if (M <= 64 && one_tile_row) {
+    // 33 to 64 rows, the same comparison: 0.34 us per slab (K 4096 / 8192 / 14336, N 4096: 16.6 / 27.4 / 44.1
+    // us, where three or four passes of the weight-streaming kernel took 19.6 / 31.9 / 52.6 us), 4 bytes/ns.
+    const double slabs_us = 0.34 * static_cast<double>(K / 128);
+    const double bytes_us = static_cast<double>(N) * static_cast<double>(K) / 4.0e6;
+    return skinny_us < 5.8 + (slabs_us > bytes_us ? slabs_us : bytes_us);
   }
   if (M <= 32) return skinny_us < tiled_us;
   // more rows: the comparison that was tuned with weights that stay in the last-level cache between calls
@@ -2204,11 +2219,12 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
   // however few of the chip's CUs their 128 x 128 tiles occupy.
   const double tiled_us = 5.0 + 0.55 * static_cast<double>(K / 128);
   // what the one-tile-row kernel (launch_mid) needs
-  // (65 to 128 rows: one workgroup per CU for its 96 KB of LDS stages, so only while one round of 64-column
-  // workgroups covers N.  Measured against the 128 x 128 tile, int8, weights from HBM, K 4096, N 4096 / 14336:
-  // 25.9 / 29.3 against 37.1 / 38.7 us; K 8192, N 8192: 43.1 against 67.7 us; but K 8192, N 28672: 90.4
-  // against 77.0 us.)
-  const bool mid_ok = M > 16 && (M <= 64 || (M <= 128 && (N + 63) / 64 <= 256)) && K % 128 == 0 && out_dtype != QWIX_I32 && zu == nullptr &&
+  // (65 to 128 rows: one workgroup per CU for its 96 or 128 KB of LDS stages, so only while one round of
+  // workgroups covers N: 64-column ones up to N 16384, 128-column ones up to N 32768.  Measured against the
+  // 128 x 128 tile, int8, weights from HBM, K 4096, N 4096 / 14336: 25.9 / 29.3 against 37.1 / 38.7 us; K 8192,
+  // N 8192: 43.1 against 67.7 us; K 8192, N 28672: 68.9 against 77.0 us with 128-column workgroups, 90.4 with
+  // two rounds of 64-column ones.)
+  const bool mid_ok = M > 16 && (M <= 64 || (M <= 128 && (N + 127) / 128 <= 256)) && K % 128 == 0 && out_dtype != QWIX_I32 && zu == nullptr &&
                       N * K >= (int64_t{8} << 20) && M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);
   const bool few_rows = streams_weights(M, N, K, mid_ok);
   const bool off31 = M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);
