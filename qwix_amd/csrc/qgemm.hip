@@ -400,7 +400,7 @@ __device__ __forceinline__ void fetch_scales(const Epilogue& ep, int m_base, int
   }
 }
 
-template <int OUT, int EPI, int TM, int TN, int NWAVES, int LDS_BYTES, typename AccT>
+template <int OUT, int EPI, int TM, int TN, int NWAVES, int LDS_BYTES, bool SYNC = true, typename AccT>
 __device__ __forceinline__ void staged_epilogue(const AccT (&acc)[TM][TN], const float (&sav)[TM],
                                                 const float (&sbv)[TN][4][4], const Epilogue& ep, int m_base,
                                                 int n_base, int M, int N, uint8_t* __restrict__ out, int64_t ldo,
@@ -424,7 +424,7 @@ __device__ __forceinline__ void staged_epilogue(const AccT (&acc)[TM][TN], const
 #pragma unroll
     for (int i = 0; i < TM; ++i) zuv[i] = ep.zu[min(m_base + i * 32 + (lane & 31), M - 1)];
   }
-  __syncthreads();  // every wavefront is done with the slabs; LDS becomes staging space
+  if constexpr (SYNC) __syncthreads();  // every wavefront is done with the slabs; LDS becomes staging space
   uint8_t* stg = smem + wave * (32 * ROWB);
   const bool row_vec = (reinterpret_cast<uintptr_t>(out) % 16 == 0) && ((ldo * ES) % 16 == 0);
 #pragma unroll
@@ -732,7 +732,7 @@ template <int QT, int OUT, int EPI, int TM, int DEPTH, int NW>
 __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, int64_t lda,
                                                const uint8_t* __restrict__ B, int64_t ldb, int m0, int n0, int M,
                                                int N, int K, const Epilogue& ep, uint8_t* __restrict__ out,
-                                               int64_t ldo) {
+                                               int64_t ldo, int kshift) {
   constexpr bool IS_INT = (QT == QWIX_INT8);
   constexpr int BK = 128, TN = 1;  // TM: 32-row blocks of the tile; DEPTH: slabs of loads kept going, plus one
   constexpr int KSTEP = IS_INT ? 32 : 64;
@@ -767,7 +767,10 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
   const int hx = lane >> 5, x7 = lane & 7;
   const uint32_t boff = static_cast<uint32_t>(min(n_base + (lane & 31), N - 1)) * static_cast<uint32_t>(ldb) + hx * 64;
   v4i breg[DEPTH][4];
+  const int KT = K / BK;
   auto issue_group = [&](int kt, int st) {  // PW direct-to-LDS loads + 4 register loads per lane
+    kt += kshift;  // this workgroup's first slab (below KT): the slabs are walked from there, wrapping around
+    if (kt >= KT) kt -= KT;
     const uint8_t* ga = A + kt * BK;
 #pragma unroll
     for (int j = 0; j < PW; ++j) QWIX_GLDS16(ga + aoff[j], smem + st * ASTAGE + (wave * PW + j) * 1024);
@@ -807,7 +810,6 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  const int KT = K / BK;
 #pragma unroll
   for (int d = 0; d < DEPTH - 1; ++d)
     if (d < KT) issue_group(d, d);
@@ -864,8 +866,150 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
 template <int QT, int OUT, int EPI, int TM, int DEPTH, int NW>
 __global__ void __launch_bounds__(64 * NW)
     qgemm_mid_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb, int M,
-                     int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
-  qgemm_mid_tile<QT, OUT, EPI, TM, DEPTH, NW>(A, lda, B, ldb, 0, blockIdx.x * (32 * NW), M, N, K, ep, out, ldo);
+                     int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo, int kmul) {
+  const int kshift = static_cast<int>((blockIdx.x * static_cast<unsigned>(kmul)) % static_cast<unsigned>(K / 128));
+  qgemm_mid_tile<QT, OUT, EPI, TM, DEPTH, NW>(A, lda, B, ldb, 0, blockIdx.x * (32 * NW), M, N, K, ep, out, ldo,
+                                              kshift);
+}
+
+// ------------------------------------------------------------------------------------------------
+// The same one tile row when N is so small that 32-column workgroups do not fill the chip (N up to 8192): the
+// KW wavefronts of a workgroup share its 32 columns and split K instead, wavefront w taking slabs w, w + KW, ...
+// Activations and weights both go from global memory straight into registers, in the same permuted K order
+// (lane half h holds bytes 64 h .. 64 h + 63 of a row's 128-byte slab, for its activation rows as for its
+// weight column), so the main loop touches no LDS and has no barrier: every wavefront runs its own pipeline
+// of DEPTH register sets, waiting only on its own loads (explicit vmcnt, loads issued as asm as above).  At the
+// end the partial accumulators meet in LDS, and wavefront i adds up and stores the i-th block of 32 rows.
+// int32 partials add exactly; for e4m3 the f32 sums are those of K / (128 KW) slabs each, added in wavefront order.
+template <int QT, int OUT, int EPI, int TM, int DEPTH, int KW>
+__global__ void __launch_bounds__(64 * KW)
+    qgemm_ksplit_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb, int M,
+                        int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo, int kmul) {
+  constexpr bool IS_INT = (QT == QWIX_INT8);
+  constexpr int BK = 128;
+  constexpr int NK = IS_INT ? 4 : 2;  // MFMAs per slab and 32-row block
+  constexpr int G = 4 * TM + 4;       // loads per slab and lane
+  static_assert((DEPTH - 2) * G <= 63, "vmcnt is a 6-bit counter");
+  static_assert(DEPTH >= 3 && DEPTH <= 8 && TM <= KW, "the waits and the final reduction list these cases");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n0 = blockIdx.x * 32;
+
+  using AccT = typename std::conditional<IS_INT, v16i, v16f>::type;
+  using FragT = typename std::conditional<IS_INT, v4i, v8i>::type;
+  AccT acc[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+  float sav[TM];
+  float sbv[1][4][4];
+  fetch_scales<OUT, TM, 1>(ep, 0, n0, M, N, lane, sav, sbv);  // oldest loads: done before any slab is used
+
+  const int hx = lane >> 5;
+  uint32_t aoff[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+    aoff[i] = static_cast<uint32_t>(min(i * 32 + (lane & 31), M - 1)) * static_cast<uint32_t>(lda) + hx * 64;
+  const uint32_t boff = static_cast<uint32_t>(min(n0 + (lane & 31), N - 1)) * static_cast<uint32_t>(ldb) + hx * 64;
+  v4i areg[DEPTH][TM][4], breg[DEPTH][4];
+  const int KT = K / BK;
+  const int kshift = static_cast<int>((blockIdx.x * static_cast<unsigned>(kmul)) % static_cast<unsigned>(KT));
+  auto issue_group = [&](int kt, int st) {  // 4 TM + 4 register loads per lane, not tracked by the compiler
+    kt += kshift;
+    if (kt >= KT) kt -= KT;
+    const uint8_t* ga = A + kt * BK;
+    const uint8_t* gb = B + kt * BK;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      asm volatile("global_load_dwordx4 %0, %4, %5\n\t"
+                   "global_load_dwordx4 %1, %4, %5 offset:16\n\t"
+                   "global_load_dwordx4 %2, %4, %5 offset:32\n\t"
+                   "global_load_dwordx4 %3, %4, %5 offset:48"
+                   : "=&v"(areg[st][i][0]), "=&v"(areg[st][i][1]), "=&v"(areg[st][i][2]), "=&v"(areg[st][i][3])
+                   : "v"(aoff[i]), "s"(ga)
+                   : "memory");
+    asm volatile("global_load_dwordx4 %0, %4, %5\n\t"
+                 "global_load_dwordx4 %1, %4, %5 offset:16\n\t"
+                 "global_load_dwordx4 %2, %4, %5 offset:32\n\t"
+                 "global_load_dwordx4 %3, %4, %5 offset:48"
+                 : "=&v"(breg[st][0]), "=&v"(breg[st][1]), "=&v"(breg[st][2]), "=&v"(breg[st][3])
+                 : "v"(boff), "s"(gb)
+                 : "memory");
+  };
+
+  const int mine = KT > wave ? (KT - wave + KW - 1) / KW : 0;  // slabs of this wavefront: wave + j * KW
+#pragma unroll
+  for (int d = 0; d < DEPTH - 1; ++d)
+    if (d < mine) issue_group(wave + d * KW, d);
+  for (int j0 = 0; j0 < mine; j0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int j = j0 + d;
+      if (j < mine) {  // the same for the whole wavefront
+        const int rem = mine - 1 - j;  // the groups after j (at most DEPTH - 2 of them) may stay in flight
+        __builtin_amdgcn_sched_barrier(0);
+        switch (rem < DEPTH - 2 ? rem : DEPTH - 2) {
+          case 0: wait_vmcnt<0>(); break;
+          case 1: wait_vmcnt<G>(); break;
+          case 2: wait_vmcnt<(2 * G < 63 ? 2 * G : 63)>(); break;
+          case 3: wait_vmcnt<(3 * G < 63 ? 3 * G : 63)>(); break;
+          case 4: wait_vmcnt<(4 * G < 63 ? 4 * G : 63)>(); break;
+          case 5: wait_vmcnt<(5 * G < 63 ? 5 * G : 63)>(); break;
+          default: wait_vmcnt<(6 * G < 63 ? 6 * G : 63)>(); break;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // set (d - 1) was multiplied one slab ago: refill it DEPTH - 1 slabs ahead
+        if (j + DEPTH - 1 < mine) issue_group(wave + (j + DEPTH - 1) * KW, (d + DEPTH - 1) % DEPTH);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < NK; ++ks) {
+          FragT fb;
+          if constexpr (IS_INT) {
+            fb = breg[d][ks];
+          } else {
+            const v4i lo = breg[d][2 * ks], hi = breg[d][2 * ks + 1];
+            fb = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          }
+#pragma unroll
+          for (int i = 0; i < TM; ++i) {
+            if constexpr (IS_INT) {
+              acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb, areg[d][i][ks], acc[i], 0, 0, 0);
+            } else {
+              const v4i lo = areg[d][i][2 * ks], hi = areg[d][i][2 * ks + 1];
+              const v8i fa = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+              acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb, fa, acc[i], 0, 0, 0, 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+  }
+  // partial accumulators -> LDS (behind the 20 KB that the epilogue stages through), [wave][block][register][lane]
+  constexpr int kStage = 20480;
+  using Word = typename std::conditional<IS_INT, int, float>::type;
+  Word* part = reinterpret_cast<Word*>(smem + kStage);
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) part[((wave * TM + i) * 16 + r) * 64 + lane] = acc[i][r];
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    if (wave == i) {  // wavefront i finishes block i
+      AccT total[1][1];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        Word t = part[((0 * TM + i) * 16 + r) * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < KW; ++w) t += part[((w * TM + i) * 16 + r) * 64 + lane];
+        total[0][0][r] = t;
+      }
+      const float sav1[1] = {sav[i]};
+      staged_epilogue<OUT, EPI, 1, 1, KW, kStage, false>(total, sav1, sbv, ep, i * 32, n0, M, N, out, ldo, smem, wave, lane);
+    }
+  }
 }
 
 template <int QT, int OUT>
@@ -886,7 +1030,7 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
     }                                                                                                             \
     kern<<<dim3(static_cast<unsigned>((N + 32 * NWW - 1) / (32 * NWW))), 64 * NWW, smem, st>>>(                   \
         static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),            \
-        static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);                           \
+        static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo, kmul);                     \
   }
   // Workgroups of 2 wavefronts (64 columns) for up to 32 rows, and for 64 rows while 128-column workgroups
   // would leave CUs without one: twice the workgroups, twice the CUs that pull weights.  Measured, weights
@@ -895,7 +1039,34 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
   const bool narrow = (N + 127) / 128 < 192;
   // Up to N 8192 and 64 rows a workgroup is a single wavefront (32 columns): 10 to 15 % less again (64 rows,
   // K 4096, N 4096 / 6144: 16.6 / 16.3 against 19.6 / 18.7 us; K 14336, N 4096: 44.1 against 52.6 us).
-  if (M <= 64 && (N + 63) / 64 <= 128) {
+  // Workgroup b starts at slab 5 b (mod K / 128) and wraps around: with a power-of-two row pitch all workgroups
+  // would otherwise ask the same few memory channels for the same K offset of their rows at the same time
+  // (K 8192, N 28672, 64 rows: 49.3 against 54.9 us; K 4096, N 14336, 32 rows: 16.2 against 17.6 us).  Integer
+  // sums do not depend on the order; e4m3 sums are then added in an order that depends on the column block.
+  constexpr int kmul = 5;
+  // N up to 8192: four wavefronts split K over the same 32 columns (32 rows, K 4096, N 6144: 12.3 against 14.2 us
+  // for single-wavefront workgroups, K 8192, N 8192: 19.5 against 22.0 us; 64 rows: 5 % less).
+  if (M <= 64 && (N + 63) / 64 <= 128 && K >= 1024) {
+#define QWIX_KSPLIT(TMM, DD)                                                                                      \
+  {                                                                                                               \
+    constexpr int kKW = 4;                                                                                        \
+    constexpr size_t smem = 20480 + kKW * TMM * 4096;                                                             \
+    auto kern = qgemm_ksplit_kernel<QT, OUT, 2, TMM, DD, kKW>;                                                    \
+    static bool configured = false;                                                                               \
+    if (!configured) {                                                                                            \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                     \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));     \
+      if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));         \
+      configured = true;                                                                                          \
+    }                                                                                                             \
+    kern<<<dim3(static_cast<unsigned>((N + 31) / 32)), 64 * kKW, smem, st>>>(                                     \
+        static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),            \
+        static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo, kmul);                     \
+  }
+    if (M <= 32) QWIX_KSPLIT(1, 6)
+    else QWIX_KSPLIT(2, 4)
+#undef QWIX_KSPLIT
+  } else if (M <= 64 && (N + 63) / 64 <= 128) {
     if (M <= 32) QWIX_MID(1, 1)
     else QWIX_MID(2, 1)
   } else if (M <= 32) {
