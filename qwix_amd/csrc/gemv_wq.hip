@@ -36,9 +36,9 @@ __device__ __forceinline__ bf16x8 as_bf16x8(v4u v) { return __builtin_bit_cast(b
 
 // Everything one wavefront needs for one 128-wide K block: its 4 activation fragments, and per
 // column tile the packed weights and the scale.
-template <int BQT, int NT>
+template <int BQT, int NT, int RT>
 struct Block {
-  v4u xf[4];
+  v4u xf[RT][4];  // RT tiles of 16 rows of x
   v4u wq[NT][BQT == QWIX_INT4 ? 1 : 2];
   unsigned sraw[NT];  // scale bits as loaded: bf16 in the low half, or f32
 };
@@ -54,17 +54,21 @@ struct LaneOff {
   unsigned s[NT];  // elements from column n_base of the scales
 };
 
-template <int BQT, int NT, bool SBF>
-__device__ __forceinline__ void load_block(const GemvArgs& p, const LaneOff<NT>& a, bool xrow, int row0, int n_base,
-                                           int kb, Block<BQT, NT>* b) {
+template <int BQT, int NT, bool SBF, int RT>
+__device__ __forceinline__ void load_block(const GemvArgs& p, const LaneOff<NT>& a, const bool (&xrow)[RT], int row0,
+                                           int n_base, int kb, Block<BQT, NT, RT>* b) {
   constexpr bool W4 = (BQT == QWIX_INT4);
   const char* xb = reinterpret_cast<const char*>(p.x + static_cast<int64_t>(row0) * p.ldx + kb * 128);
   // every vector load occupies the texture path for as long as its active lanes need, also when they
   // repeat an address: lanes whose row of x does not exist stay idle and feed zeros to the MFMA
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    b->xf[j] = v4u{0, 0, 0, 0};
-    if (xrow) b->xf[j] = *reinterpret_cast<const v4u*>(xb + a.x + j * 16);
+  for (int rt = 0; rt < RT; ++rt) {
+    const char* xr = xb + static_cast<int64_t>(rt) * 32 * p.ldx;  // 16 rows of bf16 further down
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      b->xf[rt][j] = v4u{0, 0, 0, 0};
+      if (xrow[rt]) b->xf[rt][j] = *reinterpret_cast<const v4u*>(xr + a.x + j * 16);
+    }
   }
   const int sg = static_cast<int>((static_cast<uint64_t>(static_cast<unsigned>(kb)) * p.magic) >> 32);
   const int64_t s0 = static_cast<int64_t>(sg) * p.N + n_base;
@@ -82,32 +86,39 @@ __device__ __forceinline__ void load_block(const GemvArgs& p, const LaneOff<NT>&
 
 // Weights enter the MFMA in offset binary (int4: 128 + (q + 8), int8: q + 128, both exact in bf16);
 // the offset times the row sum of x is taken out by four MFMAs against the constant -offset, whose
-// result seeds the accumulator of every column tile.
-template <int BQT, int NT, bool SBF>
-__device__ __forceinline__ void compute_block(const Block<BQT, NT>& b, v4f (&outacc)[NT]) {
+// result seeds the accumulator of every column tile.  A widened weight fragment serves all RT row tiles; every
+// output element sees the same operations in the same order whatever RT is.
+template <int BQT, int NT, bool SBF, int RT>
+__device__ __forceinline__ void compute_block(Block<BQT, NT, RT>& b, v4f (&outacc)[RT][NT]) {
   constexpr bool W4 = (BQT == QWIX_INT4);
   constexpr unsigned kNegOff = W4 ? 0xC308C308u : 0xC300C300u;  // bf16 -136 / -128, twice
   const v4u negoff = {kNegOff, kNegOff, kNegOff, kNegOff};
-  v4u xf[4];
+  v4u (&xf)[RT][4] = b.xf;
+  if constexpr (W4) {  // element order (k0,k4,k1,k5,k2,k6,k3,k7): what the nibble widening yields (in place)
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    if constexpr (W4) {  // element order (k0,k4,k1,k5,k2,k6,k3,k7): what the nibble widening yields
-      const v4u d = b.xf[j];
-      xf[j][0] = __builtin_amdgcn_perm(d[2], d[0], 0x05040100);
-      xf[j][1] = __builtin_amdgcn_perm(d[2], d[0], 0x07060302);
-      xf[j][2] = __builtin_amdgcn_perm(d[3], d[1], 0x05040100);
-      xf[j][3] = __builtin_amdgcn_perm(d[3], d[1], 0x07060302);
-    } else {
-      xf[j] = b.xf[j];
-    }
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const v4u d = xf[rt][j];
+        xf[rt][j][0] = __builtin_amdgcn_perm(d[2], d[0], 0x05040100);
+        xf[rt][j][1] = __builtin_amdgcn_perm(d[2], d[0], 0x07060302);
+        xf[rt][j][2] = __builtin_amdgcn_perm(d[3], d[1], 0x05040100);
+        xf[rt][j][3] = __builtin_amdgcn_perm(d[3], d[1], 0x07060302);
+      }
   }
-  v4f base = {0.f, 0.f, 0.f, 0.f};
+  v4f base[RT];
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
-    base = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[j]), as_bf16x8(negoff), base, 0, 0, 0);
+  for (int rt = 0; rt < RT; ++rt) {
+    base[rt] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      base[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[rt][j]), as_bf16x8(negoff), base[rt], 0, 0, 0);
+  }
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    v4f acc = base;
+    v4f acc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt] = base[rt];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       v4u w;
@@ -132,18 +143,24 @@ __device__ __forceinline__ void compute_block(const Block<BQT, NT>& b, v4f (&out
           w[2 * h + 1] = __builtin_amdgcn_perm(f3, f2, 0x07060302);
         }
       }
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[j]), as_bf16x8(w), acc, 0, 0, 0);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+        acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[rt][j]), as_bf16x8(w), acc[rt], 0, 0, 0);
     }
     const float sc = __uint_as_float(SBF ? b.sraw[t] << 16 : b.sraw[t]);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) outacc[t][r] = fmaf(acc[r], sc, outacc[t][r]);
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) outacc[rt][t][r] = fmaf(acc[rt][r], sc, outacc[rt][t][r]);
   }
 }
 
-// NWAVE wavefronts per workgroup, each owning a slice of K; NT tiles of 16 output columns.
-template <int BQT, int NWAVE, int NT, bool SBF>
+// NWAVE wavefronts per workgroup, each owning a slice of K; NT tiles of 16 output columns, RT tiles of 16 rows
+// (the weights are read, and widened, once per workgroup whatever RT is).
+template <int BQT, int NWAVE, int NT, bool SBF, int RT = 1>
 __global__ void __launch_bounds__(NWAVE * 64) gemv_wq_kernel(GemvArgs p) {
-  __shared__ float red[NWAVE][NT][4][64];
+  extern __shared__ float red_raw[];
+  float (*red)[RT * NT][4][64] = reinterpret_cast<float (*)[RT * NT][4][64]>(red_raw);  // [NWAVE]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, kq = lane >> 4;
@@ -152,9 +169,11 @@ __global__ void __launch_bounds__(NWAVE * 64) gemv_wq_kernel(GemvArgs p) {
   const int per_wave = (nblk + NWAVE - 1) / NWAVE;
   const int kb0 = wave * per_wave, kb1 = min(nblk, kb0 + per_wave);
 
-  const int row0 = blockIdx.y * 16;
+  const int row0 = blockIdx.y * (16 * RT);
   LaneOff<NT> a;
-  const bool xrow = row0 + col < p.M;
+  bool xrow[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) xrow[rt] = row0 + rt * 16 + col < p.M;
   a.x = static_cast<unsigned>(col) * static_cast<unsigned>(p.ldx) * 2u + kq * 64u;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
@@ -162,33 +181,38 @@ __global__ void __launch_bounds__(NWAVE * 64) gemv_wq_kernel(GemvArgs p) {
     a.w[t] = a.s[t] * static_cast<unsigned>(p.ldb) + kq * (BQT == QWIX_INT4 ? 16u : 32u);
   }
 
-  v4f outacc[NT];
+  v4f outacc[RT][NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) outacc[t] = v4f{0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) outacc[rt][t] = v4f{0.f, 0.f, 0.f, 0.f};
 
   // Two K blocks per trip, all their loads issued before the first is consumed.  Nothing loaded is
   // carried from one trip to the next; the other wavefronts of the SIMD cover the gap.
   for (int kb = kb0; kb < kb1; kb += 2) {
-    Block<BQT, NT> b0, b1;
+    Block<BQT, NT, RT> b0, b1;
     const bool two = kb + 1 < kb1;
-    load_block<BQT, NT, SBF>(p, a, xrow, row0, n_base, kb, &b0);
-    if (two) load_block<BQT, NT, SBF>(p, a, xrow, row0, n_base, kb + 1, &b1);
-    compute_block<BQT, NT, SBF>(b0, outacc);
-    if (two) compute_block<BQT, NT, SBF>(b1, outacc);
+    load_block<BQT, NT, SBF, RT>(p, a, xrow, row0, n_base, kb, &b0);
+    if (two) load_block<BQT, NT, SBF, RT>(p, a, xrow, row0, n_base, kb + 1, &b1);
+    compute_block<BQT, NT, SBF, RT>(b0, outacc);
+    if (two) compute_block<BQT, NT, SBF, RT>(b1, outacc);
   }
 
 #pragma unroll
-  for (int t = 0; t < NT; ++t)
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][t][r][lane] = outacc[t][r];
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][rt * NT + t][r][lane] = outacc[rt][t][r];
   __syncthreads();
   // result lane layout: column n = lane % 16, row m = 4 * (lane / 16) + r
-  for (int idx = tid; idx < NT * 256; idx += NWAVE * 64) {
-    const int t = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
+  for (int idx = tid; idx < RT * NT * 256; idx += NWAVE * 64) {
+    const int t2 = idx >> 8, r = (idx >> 6) & 3, l = idx & 63;
+    const int rt = t2 / NT, t = t2 % NT;
     float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < NWAVE; ++w) v += red[w][t][r][l];
-    const int mo = blockIdx.y * 16 + 4 * (l >> 4) + r, n = n_base + t * 16 + (l & 15);
+    for (int w = 0; w < NWAVE; ++w) v += red[w][t2][r][l];
+    const int mo = row0 + rt * 16 + 4 * (l >> 4) + r, n = n_base + t * 16 + (l & 15);
     if (mo < p.M && n < p.N) {
       if (p.out_dtype == QWIX_BF16)
         reinterpret_cast<uint16_t*>(p.out)[static_cast<int64_t>(mo) * p.ldo + n] = f32_to_bf16_bits(v);
@@ -230,17 +254,35 @@ extern "C" int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64
   p.s = s; p.s_dtype = s_dtype;
   p.out = out; p.out_dtype = out_dtype; p.ldo = ldo;
   hipStream_t st = static_cast<hipStream_t>(stream);
+#define QWIX_GEMV_KERNEL(KERN, NW, NTT, RTT)                                                                \
+  do {                                                                                                     \
+    constexpr size_t smem = sizeof(float) * NW * RTT * NTT * 4 * 64;                                       \
+    static bool configured = false;                                                                        \
+    if (!configured && smem >= 65536) {                                                                     \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(KERN),                              \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)); \
+      if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));  \
+      configured = true;                                                                                   \
+    }                                                                                                      \
+    KERN<<<grid, NW * 64, smem, st>>>(p);                                                                  \
+  } while (0)
+#define QWIX_GEMV_LAUNCH_RT(NW, NTT, RTT)                                                                  \
+  do {                                                                                                     \
+    const dim3 grid(static_cast<unsigned>((N + 16 * NTT - 1) / (16 * NTT)),                                \
+                    static_cast<unsigned>((M + 16 * RTT - 1) / (16 * RTT)));                               \
+    if (b_qtype == QWIX_INT4 && s_dtype == QWIX_BF16)                                                      \
+      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT4, NW, NTT, true, RTT>), NW, NTT, RTT);                     \
+    else if (b_qtype == QWIX_INT4)                                                                         \
+      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT4, NW, NTT, false, RTT>), NW, NTT, RTT);                    \
+    else if (s_dtype == QWIX_BF16)                                                                         \
+      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT8, NW, NTT, true, RTT>), NW, NTT, RTT);                     \
+    else                                                                                                   \
+      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT8, NW, NTT, false, RTT>), NW, NTT, RTT);                    \
+  } while (0)
 #define QWIX_GEMV_LAUNCH(NW, NTT)                                                                          \
   do {                                                                                                     \
-    const dim3 grid(static_cast<unsigned>((N + 16 * NTT - 1) / (16 * NTT)), static_cast<unsigned>((M + 15) / 16)); \
-    if (b_qtype == QWIX_INT4 && s_dtype == QWIX_BF16)                                                      \
-      gemv_wq_kernel<QWIX_INT4, NW, NTT, true><<<grid, NW * 64, 0, st>>>(p);                               \
-    else if (b_qtype == QWIX_INT4)                                                                         \
-      gemv_wq_kernel<QWIX_INT4, NW, NTT, false><<<grid, NW * 64, 0, st>>>(p);                              \
-    else if (s_dtype == QWIX_BF16)                                                                         \
-      gemv_wq_kernel<QWIX_INT8, NW, NTT, true><<<grid, NW * 64, 0, st>>>(p);                               \
-    else                                                                                                   \
-      gemv_wq_kernel<QWIX_INT8, NW, NTT, false><<<grid, NW * 64, 0, st>>>(p);                              \
+    if (M <= 16) QWIX_GEMV_LAUNCH_RT(NW, NTT, 1);                                                          \
+    else QWIX_GEMV_LAUNCH_RT(8, NTT, 2);                                                                   \
   } while (0)
   // Wider column tiles reuse each activation fragment more often; narrower ones keep every CU busy
   // when the weight matrix has few columns.
@@ -251,5 +293,7 @@ extern "C" int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64
   else
     QWIX_GEMV_LAUNCH(16, 1);
 #undef QWIX_GEMV_LAUNCH
+#undef QWIX_GEMV_LAUNCH_RT
+#undef QWIX_GEMV_KERNEL
   return check_launch("gemv_wq");
 }

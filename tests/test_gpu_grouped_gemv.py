@@ -130,7 +130,7 @@ def test_per_channel_int4_weight_and_tile_mismatch_error():
 
 
 @pytest.mark.parametrize('wq_type', ['int4', 'int8'])
-@pytest.mark.parametrize('M', [1, 8, 16, 40])
+@pytest.mark.parametrize('M', [1, 8, 16, 24, 40, 100])
 @pytest.mark.parametrize('K,N,group,sdt', [(512, 256, 128, torch.float32), (4096, 1024, 128, torch.float32), (1024, 200, 1024, torch.bfloat16)])
 def test_weight_only_gemv(M, K, N, group, sdt, wq_type):
   """The weight-only int4 benchmark configuration at reduced N: bf16 activations x int4 g128 weight, f32 scales, bf16 out."""
@@ -153,6 +153,26 @@ def test_weight_only_gemv(M, K, N, group, sdt, wq_type):
   # default result type follows the scale dtype (bf16 x f32 -> f32)
   out2 = dg.dot_general(x_t, wq, DN)
   assert out2.dtype == sdt
+
+
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('M,K,N', [(30, 1024, 520), (50, 4096, 14336), (130, 512, 6400)])
+def test_weight_only_rows_do_not_depend_on_the_batch(M, K, N, wq_type):
+  """More than 16 rows share a pass over the weights (2 tiles of 16 rows per workgroup, half as many wavefronts
+  along K): the f32 partial sums meet in another order, nothing else changes, so the result equals the rows
+  computed 16 at a time up to that reordering."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  print('case gemv batch', M, K, N, wq_type, flush=True)
+  _, x_t = util.make((M, K), O.BF16, seed=M + K)
+  _, w_t = util.make((K, N), O.BF16, seed=M + K + 1, scale=0.02)
+  wq = qarray.quantize_api(w_t, wq_type, channelwise_axes=[1], tiled_axes={0: 128}, scale_dtype=torch.float32)
+  out = dg.dot_general(x_t, wq, DN, preferred_element_type=torch.float32)
+  parts = [dg.dot_general(x_t[i:i + 16].contiguous(), wq, DN, preferred_element_type=torch.float32)
+           for i in range(0, M, 16)]
+  torch.cuda.synchronize()
+  want = torch.cat(parts, 0)
+  assert torch.allclose(out, want, rtol=1e-5, atol=1e-5 * want.abs().mean().item())
 
 
 def _close(got, true, dtype):
