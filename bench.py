@@ -802,6 +802,7 @@ WORKLOADS = {
     'w8a8_decode_m16_k2048_fused': lambda: QdotDecodeFused('w8a8_decode_m16_k2048_fused', 16, 2048, 8192),
     'c2_gemv_w4_m1': lambda: GemvW4('c2_gemv_w4_m1', 1, 4096, 14336, 128),
     'c2_gemv_w4_m16': lambda: GemvW4('c2_gemv_w4_m16', 16, 4096, 14336, 128),
+    'c2_gemv_w4_m32': lambda: GemvW4('c2_gemv_w4_m32', 32, 4096, 14336, 128),
     'c4_quantize_weight_fp8': lambda: QuantizeWeight('c4_quantize_weight_fp8', 8192, 28672, 'float8_e4m3fn'),
     'c5_quantize_weight_int4_g128': lambda: QuantizeWeight('c5_quantize_weight_int4_g128', 8192, 8192, 'int4', 128),
     'c3_quantize_weight_int8': lambda: QuantizeWeight('c3_quantize_weight_int8', 4096, 4096, 'int8'),
