@@ -57,6 +57,8 @@ INT8_CASES = [
      (0, 3, 16, 1, 0, 7, 2, 0, 5, 2, 1, 1), (0,), (0, 2), None),
     ('decode: one group takes several 16-row passes', (60, 384, 6, 72), (0, 40, 1, 0, 9, 3), (0,), (0, 2), None),
     ('decode: one row per group, shared weight scale', (16, 128, 16, 48), (1,) * 16, (0,), (2,), None),
+    ('a few dozen rows per group (64-row tiles, deep weight prefetch), some groups empty or taller than a tile',
+     (1700, 1024, 40, 520), tuple((i * 37) % 60 if i % 9 else (0 if i % 2 else 130) for i in range(40)), (0,), (0, 2), None),
     ('big groups', (2100, 512, 2, 2304), (1100, 900), (0,), (0, 2), None),
     ('big groups on a full chip (256-row tiles, ping-pong schedule)', (4096, 384, 4, 3072), (1000, 1100, 900, 1000), (0,), (0, 2), None),
 ]
