@@ -282,7 +282,8 @@ extern "C" int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64
 #define QWIX_GEMV_LAUNCH(NW, NTT)                                                                          \
   do {                                                                                                     \
     if (M <= 16) QWIX_GEMV_LAUNCH_RT(NW, NTT, 1);                                                          \
-    else QWIX_GEMV_LAUNCH_RT(8, NTT, 2);                                                                   \
+    else if (M <= 32) QWIX_GEMV_LAUNCH_RT(8, NTT, 2);                                                      \
+    else QWIX_GEMV_LAUNCH_RT(4, NTT, 2); /* several passes side by side: smaller workgroups, two per CU */  \
   } while (0)
   // Wider column tiles reuse each activation fragment more often; narrower ones keep every CU busy
   // when the weight matrix has few columns.

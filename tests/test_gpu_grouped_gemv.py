@@ -158,7 +158,7 @@ def test_weight_only_gemv(M, K, N, group, sdt, wq_type):
 @pytest.mark.parametrize('wq_type', ['int4', 'int8'])
 @pytest.mark.parametrize('M,K,N', [(30, 1024, 520), (50, 4096, 14336), (130, 512, 6400)])
 def test_weight_only_rows_do_not_depend_on_the_batch(M, K, N, wq_type):
-  """More than 16 rows share a pass over the weights (2 tiles of 16 rows per workgroup, half as many wavefronts
+  """More than 16 rows share a pass over the weights (2 tiles of 16 rows per workgroup, fewer wavefronts
   along K): the f32 partial sums meet in another order, nothing else changes, so the result equals the rows
   computed 16 at a time up to that reordering."""
   from qwix_amd.core import dot_general as dg
