@@ -868,8 +868,8 @@ __global__ void __launch_bounds__(64 * NW)
     qgemm_mid_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb, int M,
                      int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo, int kmul) {
   const int kshift = static_cast<int>((blockIdx.x * static_cast<unsigned>(kmul)) % static_cast<unsigned>(K / 128));
-  qgemm_mid_tile<QT, OUT, EPI, TM, DEPTH, NW>(A, lda, B, ldb, 0, blockIdx.x * (32 * NW), M, N, K, ep, out, ldo,
-                                              kshift);
+  qgemm_mid_tile<QT, OUT, EPI, TM, DEPTH, NW>(A, lda, B, ldb, blockIdx.y * (32 * TM), blockIdx.x * (32 * NW), M, N, K,
+                                              ep, out, ldo, kshift);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1016,9 +1016,10 @@ template <int QT, int OUT>
 int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
                const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   // LDS: kDepth stages of activations, and at least the 18 KB the epilogue stages through
-#define QWIX_MID(TMM, NWW)                                                                                        \
+#define QWIX_MID(TMM, NWW) QWIX_MID_D(TMM, NWW, ((4 * TMM / NWW + 4) * 6 <= 63 ? 8 : 6))
+#define QWIX_MID_D(TMM, NWW, DD)                                                                                  \
   {                                                                                                               \
-    constexpr int kDepth = (4 * TMM / NWW + 4) * 6 <= 63 ? 8 : 6; /* groups in flight stay under vmcnt's 63 */      \
+    constexpr int kDepth = DD; /* the groups in flight must stay under vmcnt's 63 */                               \
     constexpr size_t smem = kDepth * 32 * TMM * 128 > 20480 ? kDepth * 32 * TMM * 128 : 20480;                     \
     auto kern = qgemm_mid_kernel<QT, OUT, 2, TMM, kDepth, NWW>;                                                   \
     static bool configured = false;                                                                               \
@@ -1028,7 +1029,8 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
       if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));         \
       configured = true;                                                                                          \
     }                                                                                                             \
-    kern<<<dim3(static_cast<unsigned>((N + 32 * NWW - 1) / (32 * NWW))), 64 * NWW, smem, st>>>(                   \
+    kern<<<dim3(static_cast<unsigned>((N + 32 * NWW - 1) / (32 * NWW)),                                           \
+                static_cast<unsigned>((M + 32 * TMM - 1) / (32 * TMM))), 64 * NWW, smem, st>>>(                    \
         static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),            \
         static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo, kmul);                     \
   }
@@ -1071,6 +1073,8 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
     else QWIX_MID(2, 1)
   } else if (M <= 32) {
     QWIX_MID(1, 2)
+  } else if (M > 128) {
+    QWIX_MID_D(4, 2, 4)  // two tile rows side by side: four stages, 64 KB, two workgroups per CU
   } else if (M > 64) {
     if ((N + 63) / 64 <= 256) QWIX_MID(4, 2)
     else QWIX_MID(4, 4)
@@ -1079,6 +1083,7 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
     else QWIX_MID(2, 4)
   }
 #undef QWIX_MID
+#undef QWIX_MID_D
   return check_launch("qgemm (one tile row)");
 }
 
@@ -2447,7 +2452,11 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
   // 128 x 128 tile, int8, weights from HBM, K 4096, N 4096 / 14336: 25.9 / 29.3 against 37.1 / 38.7 us; K 8192,
   // N 8192: 43.1 against 67.7 us; K 8192, N 28672: 68.9 against 77.0 us with 128-column workgroups, 90.4 with
   // two rounds of 64-column ones.)
-  const bool mid_ok = M > 16 && (M <= 64 || (M <= 128 && (N + 127) / 128 <= 256)) && K % 128 == 0 && out_dtype != QWIX_I32 && zu == nullptr &&
+  // 129 to 256 rows, N up to 8192: two tile rows of 128 side by side (four stages, two workgroups per CU) where
+  // the 128 x 128 tiles would occupy a quarter of the chip: 256 rows, K 4096, N 4096: 24.6 against 36.5 us;
+  // K 8192, N 8192: 43.8 against 65.0 us; K 14336, N 4096: 67.3 against 112.8 us; no gain from N 14336 on.
+  const bool mid_ok = M > 16 && (M <= 64 || (M <= 128 && (N + 127) / 128 <= 256) ||
+                                 (M <= 256 && (N + 63) / 64 <= 128)) && K % 128 == 0 && out_dtype != QWIX_I32 && zu == nullptr &&
                       N * K >= (int64_t{8} << 20) && M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);
   const bool few_rows = streams_weights(M, N, K, mid_ok);
   const bool off31 = M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);

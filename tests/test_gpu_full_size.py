@@ -238,12 +238,13 @@ def test_one_row_against_a_large_vocabulary_projection():
 @pytest.mark.parametrize('M,K,N', [(64, 4096, 14336), (33, 2048, 8200), (20, 8192, 28672), (48, 128, 66000), (64, 384, 22016),
                                    (32, 4096, 14336), (24, 8192, 8192), (17, 2048, 28700), (64, 4096, 28672),
                                    (128, 4096, 14336), (100, 2048, 8200), (65, 512, 16384), (128, 1024, 28672),
-                                   (64, 4096, 4096), (24, 2048, 6100), (20, 1152, 8100), (50, 1024, 8190)])
+                                   (64, 4096, 4096), (24, 2048, 6100), (20, 1152, 8100), (50, 1024, 8190),
+                                   (256, 4096, 4096), (200, 2048, 8192), (130, 1280, 8000)])
 def test_decode_batch_against_a_wide_weight(M, K, N):
-  """17 to 128 rows against megabytes of weights (the deep-prefetch tile): int8 with per-row and per-column
+  """17 to 256 rows against megabytes of weights (the deep-prefetch tile): int8 with per-row and per-column
   power-of-two scales, f32 out; every output is an exact integer times two exact scales.  K of one, three
   and many 128-wide slabs exercise the start and the end of the prefetch pipeline; N = 8200 a ragged last tile.
-  The shapes cover the 32-, 64- and 128-row tiles, and workgroups of 32, 64 and 128 columns; up to N 8192 the
+  The shapes cover the 32-, 64- and 128-row tiles (also two 128-row tiles one above the other), and workgroups of 32, 64 and 128 columns; up to N 8192 the
   wavefronts of a workgroup split K instead (9 slabs over 4 wavefronts: uneven shares; 8: fewer than the pipeline is deep)."""
   from qwix_amd import _lib
   a = _small_ints((M, K), -127, 127, 51, torch.int8)
@@ -268,7 +269,7 @@ def test_decode_batch_against_a_wide_weight(M, K, N):
   assert torch.equal(outb, wantb)
 
 
-@pytest.mark.parametrize('M,K,N', [(64, 4096, 14336), (32, 8192, 8192), (40, 2048, 28700), (128, 4096, 8192), (48, 4096, 4096), (40, 2304, 4000), (30, 8192, 2048)])
+@pytest.mark.parametrize('M,K,N', [(64, 4096, 14336), (32, 8192, 8192), (40, 2048, 28700), (128, 4096, 8192), (48, 4096, 4096), (40, 2304, 4000), (30, 8192, 2048), (250, 2048, 4096)])
 def test_fp8_decode_batch_against_a_wide_weight(M, K, N):
   """The same tile with e4m3 operands: values in -2..2 are exact in e4m3 and every sum stays below 2^24, so the
   f32 output must equal the integer product; power-of-two scales keep the bf16 epilogue exact as well."""
