@@ -1012,7 +1012,7 @@ __global__ void __launch_bounds__(64 * KW)
   }
 }
 
-template <int QT, int OUT>
+template <int QT, int OUT, int EPI = 2>
 int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
                const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   // LDS: kDepth stages of activations, and at least the 18 KB the epilogue stages through
@@ -1021,7 +1021,7 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
   {                                                                                                               \
     constexpr int kDepth = DD; /* the groups in flight must stay under vmcnt's 63 */                               \
     constexpr size_t smem = kDepth * 32 * TMM * 128 > 20480 ? kDepth * 32 * TMM * 128 : 20480;                     \
-    auto kern = qgemm_mid_kernel<QT, OUT, 2, TMM, kDepth, NWW>;                                                   \
+    auto kern = qgemm_mid_kernel<QT, OUT, EPI, TMM, kDepth, NWW>;                                                 \
     static bool configured = false;                                                                               \
     if (!configured) {                                                                                            \
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                     \
@@ -1053,7 +1053,7 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
   {                                                                                                               \
     constexpr int kKW = 4;                                                                                        \
     constexpr size_t smem = 20480 + kKW * TMM * 4096;                                                             \
-    auto kern = qgemm_ksplit_kernel<QT, OUT, 2, TMM, DD, kKW>;                                                    \
+    auto kern = qgemm_ksplit_kernel<QT, OUT, EPI, TMM, DD, kKW>;                                                  \
     static bool configured = false;                                                                               \
     if (!configured) {                                                                                            \
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                     \
@@ -2456,7 +2456,8 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
   // the 128 x 128 tiles would occupy a quarter of the chip: 256 rows, K 4096, N 4096: 24.6 against 36.5 us;
   // K 8192, N 8192: 43.8 against 65.0 us; K 14336, N 4096: 67.3 against 112.8 us; no gain from N 14336 on.
   const bool mid_ok = M > 16 && (M <= 64 || (M <= 128 && (N + 127) / 128 <= 256) ||
-                                 (M <= 256 && (N + 63) / 64 <= 128)) && K % 128 == 0 && out_dtype != QWIX_I32 && zu == nullptr &&
+                                 (M <= 256 && (N + 63) / 64 <= 128)) && K % 128 == 0 && out_dtype != QWIX_I32 &&
+                      (zu == nullptr || qtype == QWIX_INT8) &&
                       N * K >= (int64_t{8} << 20) && M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);
   const bool few_rows = streams_weights(M, N, K, mid_ok);
   const bool off31 = M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);
@@ -2484,6 +2485,10 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
     if (mid_ok) {
       // up to 64 rows against a weight of megabytes (and too many rows, or too large a weight, for the
       // weight-streaming kernel): the tile that keeps three slabs of weights in flight per wavefront
+      if (qtype == QWIX_INT8 && zu != nullptr) {  // zero-point correction in the epilogue
+        if (out_dtype == QWIX_BF16) return launch_mid<QWIX_INT8, QWIX_BF16, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+        return launch_mid<QWIX_INT8, QWIX_F32, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      }
       if (qtype == QWIX_INT8) {
         if (out_dtype == QWIX_BF16) return launch_mid<QWIX_INT8, QWIX_BF16>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
         return launch_mid<QWIX_INT8, QWIX_F32>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);

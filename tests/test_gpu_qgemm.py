@@ -112,7 +112,8 @@ def test_gemm_linearity_full_size_property():
 
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
 @pytest.mark.parametrize('side', ['lhs', 'rhs'])
-@pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (100, 272, 60), (1100, 512, 1300), (3, 64, 5), (8, 256, 200)])
+@pytest.mark.parametrize('M,K,N', [(256, 1024, 512), (100, 272, 60), (1100, 512, 1300), (3, 64, 5), (8, 256, 200),
+                                   (48, 2048, 4608), (100, 1024, 9000), (200, 2048, 4100), (30, 640, 14000)])  # decode batches against wide weights
 def test_int8_gemm_with_zero_point_operand_bit_exact(M, K, N, side, dtype):
   """One asymmetric (minmax) operand: the int32 correction dot(zp, q_other) of dot_general.py:228-253 is
   subtracted before scaling, so the output is again an elementwise function of exact integers."""
