@@ -2361,7 +2361,13 @@ static bool streams_weights(int64_t M, int64_t N, int64_t K, bool one_tile_row) 
   const double slab_us = 0.95 * static_cast<double>(K / 128) * rounds;
   const double read_us = static_cast<double>(N) * static_cast<double>(K) / 3.8e6;
   const double tiled_us = 5.0 + (slab_us > read_us ? slab_us : read_us);
-  if (M <= 16) return true;
+  if (M <= 16) {
+    // One pass either way.  From about 100 MB of weights on, while one or two rounds of 64-column workgroups
+    // cover N, the one-tile-row kernel streams them faster (16 rows, K 8192, N 28672: 47.4 against 53.0 us, the
+    // rate of a plain device copy; K 4096, N 28672: 27.3 against 30.2 us); with more rounds it falls behind
+    // (K 8192, N 57344: 126 against 100 us).
+    return !(one_tile_row && N * K >= (int64_t{96} << 20) && N <= 32768);
+  }
   if (M <= 32 && one_tile_row) {
     // The one-tile-row kernel is there for this call (qgemm_impl checks what it needs).  With 32 rows and
     // 64-column workgroups it was measured, weights from HBM, at K 4096, N 4096 / 14336 / 28672: 14.2 / 17.5 /
@@ -2455,7 +2461,7 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
   // 129 to 256 rows, N up to 8192: two tile rows of 128 side by side (four stages, two workgroups per CU) where
   // the 128 x 128 tiles would occupy a quarter of the chip: 256 rows, K 4096, N 4096: 24.6 against 36.5 us;
   // K 8192, N 8192: 43.8 against 65.0 us; K 14336, N 4096: 67.3 against 112.8 us; no gain from N 14336 on.
-  const bool mid_ok = M > 16 && (M <= 64 || (M <= 128 && (N + 127) / 128 <= 256) ||
+  const bool mid_ok = (M > 16 || (N * K >= (int64_t{96} << 20) && N <= 32768)) && (M <= 64 || (M <= 128 && (N + 127) / 128 <= 256) ||
                                  (M <= 256 && (N + 63) / 64 <= 128)) && K % 128 == 0 && out_dtype != QWIX_I32 &&
                       (zu == nullptr || qtype == QWIX_INT8) &&
                       N * K >= (int64_t{8} << 20) && M * lda < (int64_t{1} << 31) && N * ldb < (int64_t{1} << 31);

@@ -239,9 +239,9 @@ def test_one_row_against_a_large_vocabulary_projection():
                                    (32, 4096, 14336), (24, 8192, 8192), (17, 2048, 28700), (64, 4096, 28672),
                                    (128, 4096, 14336), (100, 2048, 8200), (65, 512, 16384), (128, 1024, 28672),
                                    (64, 4096, 4096), (24, 2048, 6100), (20, 1152, 8100), (50, 1024, 8190),
-                                   (256, 4096, 4096), (200, 2048, 8192), (130, 1280, 8000)])
+                                   (256, 4096, 4096), (200, 2048, 8192), (130, 1280, 8000), (16, 4096, 28672), (3, 8192, 14000)])
 def test_decode_batch_against_a_wide_weight(M, K, N):
-  """17 to 256 rows against megabytes of weights (the deep-prefetch tile): int8 with per-row and per-column
+  """17 to 256 rows against megabytes of weights (fewer rows too from about 100 MB of weights on) (the deep-prefetch tile): int8 with per-row and per-column
   power-of-two scales, f32 out; every output is an exact integer times two exact scales.  K of one, three
   and many 128-wide slabs exercise the start and the end of the prefetch pipeline; N = 8200 a ragged last tile.
   The shapes cover the 32-, 64- and 128-row tiles (also two 128-row tiles one above the other), and workgroups of 32, 64 and 128 columns; up to N 8192 the
