@@ -72,6 +72,20 @@ QWIX_API int qwix_hip_quantize(const void* x, int dtype, int64_t outer, int64_t 
                       int q_layout, void* qvalue, void* scale, void* zero_point,
                       void* workspace, size_t workspace_bytes, void* stream);
 
+/* qwix_hip_quantize for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments and results as qwix_hip_quantize without the workspace: the calibration scratch
+ * (partial absmax / min / max values of scale groups that span several workgroups) lives in a
+ * file-scope device array of qwix_hip_quantize_static_max_bytes() = 1 MiB that every GPU the library
+ * runs on holds until the process ends.  Shapes whose qwix_hip_quantize_workspace_bytes(...) exceeds
+ * that are refused with QWIX_ERR_UNSUPPORTED.  The call allocates nothing and frees nothing.  All calls
+ * on one GPU share that GPU's array: calls that overlap on one GPU (different streams, or threads)
+ * race; calls ordered on one stream do not (every call clears what it accumulates into). */
+QWIX_API size_t qwix_hip_quantize_static_max_bytes(void);
+QWIX_API int qwix_hip_quantize_static(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner,
+                             int64_t tile, int qtype, int calibration, float calib_factor,
+                             int q_layout, void* qvalue, void* scale, void* zero_point, void* stream);
+
 /* calibrate alone (qarray.py:470-534): writes absmax (QWIX_ABSMAX: out0) or min/max
  * (QWIX_MINMAX: out0=min, out1=max), each `dtype`, shaped like the scale. */
 QWIX_API int qwix_hip_calibrate(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner,

@@ -27,6 +27,8 @@ SIGNATURES = {
     'qwix_hip_last_error': (_c.c_char_p, []),
     'qwix_hip_quantize_workspace_bytes': (_sz, [_i64, _i64, _i64, _i64, _int]),
     'qwix_hip_quantize': (_int, [_vp, _int, _i64, _i64, _i64, _i64, _int, _int, _f32, _int, _vp, _vp, _vp, _vp, _sz, _vp]),
+    'qwix_hip_quantize_static_max_bytes': (_sz, []),
+    'qwix_hip_quantize_static': (_int, [_vp, _int, _i64, _i64, _i64, _i64, _int, _int, _f32, _int, _vp, _vp, _vp, _vp]),
     'qwix_hip_calibrate': (_int, [_vp, _int, _i64, _i64, _i64, _i64, _int, _f32, _vp, _vp, _vp, _sz, _vp]),
     'qwix_hip_calibrate_rms': (_int, [_vp, _int, _c.POINTER(_i64), _i64, _i64, _f32, _vp, _vp]),
     'qwix_hip_compute_scale_zero_point': (_int, [_vp, _vp, _int, _i64, _int, _int, _vp, _vp, _vp]),

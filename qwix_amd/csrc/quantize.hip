@@ -11,6 +11,7 @@
 //           re-reads each panel, quantizes it, and writes either the natural layout or the
 //           reduce-minor (transposed) layout the GEMM kernels consume.
 #include <cstdlib>
+#include <mutex>
 
 #include <type_traits>
 
@@ -1405,6 +1406,40 @@ int check_cols(const void* x, int dtype, int64_t reduce, int64_t inner, int64_t 
 
 using namespace qwix;
 
+// ------------------------------------------------------------------------------------ static scratch
+// Calibration scratch of qwix_hip_quantize_static: one array per GPU, held from the moment the code
+// object is loaded on that GPU until the process ends.  `quantize_scratch` is only a host-side handle of
+// the symbol; the device address differs per GPU and comes from hipGetSymbolAddress, once per device.
+constexpr size_t kStaticScratchBytes = size_t{1} << 20;
+static __device__ __align__(256) unsigned char quantize_scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxScratchDevices = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[kMaxScratchDevices] = {nullptr};
+
+// Device address of the current device's copy of quantize_scratch (looked up on the first call on
+// that device, cached afterwards), or nullptr with the error text set.
+void* static_scratch() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxScratchDevices) {
+    fail(QWIX_ERR_LAUNCH, "no current HIP device (or device index %d >= %d)", dev, kMaxScratchDevices);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(quantize_scratch));
+    if (e != hipSuccess || p == nullptr) {
+      fail(QWIX_ERR_LAUNCH, "hipGetSymbolAddress(quantize_scratch) on device %d: %s", dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    scratch_ptr[dev] = p;
+  }
+  return scratch_ptr[dev];
+}
+}  // namespace
+
 extern "C" {
 
 int qwix_hip_abi_version(void) { return 1; }
@@ -1441,6 +1476,25 @@ int qwix_hip_quantize(const void* x, int dtype, int64_t outer, int64_t reduce, i
   if (int e = run_cols_absmax(x, dtype, g, calibration, static_cast<uint32_t*>(workspace), st)) return e;
   return run_cols_quantize<0>(x, dtype, g, qtype, calibration, q_layout, static_cast<const uint32_t*>(workspace),
                               calib_factor, qvalue, scale, zero_point, st);
+}
+
+size_t qwix_hip_quantize_static_max_bytes(void) { return kStaticScratchBytes; }
+
+int qwix_hip_quantize_static(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner, int64_t tile,
+                             int qtype, int calibration, float calib_factor, int q_layout, void* qvalue,
+                             void* scale, void* zero_point, void* stream) {
+  if (int e = check_geom(outer, reduce, inner, tile)) return e;
+  const size_t need = qwix_hip_quantize_workspace_bytes(outer, reduce, inner, tile, calibration);
+  if (need > kStaticScratchBytes)
+    return fail(QWIX_ERR_UNSUPPORTED,
+                "this shape needs %zu bytes of calibration scratch, the static buffer holds %zu: call "
+                "qwix_hip_quantize with a workspace instead", need, kStaticScratchBytes);
+  void* ws = static_scratch();  // device address of this GPU's array; never the symbol itself
+  if (ws == nullptr) return QWIX_ERR_LAUNCH;
+  // The kernels behind qwix_hip_quantize clear what they accumulate into (a fill kernel on `stream`), so
+  // what an earlier call left in the array does not matter.
+  return qwix_hip_quantize(x, dtype, outer, reduce, inner, tile, qtype, calibration, calib_factor, q_layout, qvalue,
+                           scale, zero_point, ws, kStaticScratchBytes, stream);
 }
 
 int qwix_hip_calibrate(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner, int64_t tile,
