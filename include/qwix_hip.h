@@ -250,6 +250,30 @@ QWIX_API int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b, i
                            int sb_dtype, void* out, int out_dtype, int64_t ldo, int exact,
                            int32_t* acc_out, void* stream);
 
+/* Sub-channel GEMM with one asymmetric operand.  Replaces the zero-point terms of _fast_dot_general when a
+ * contracting axis is tiled (qwix/_src/core/dot_general.py:196-203: the zero point is split with the tiles;
+ * :228-253: the correction dot is subtracted from every tile's int32 partial before it is scaled):
+ *     out[m,n] = cast_R( sum_g (T(acc_g[m,n] - zu[m,g] * zv[g,n]) * sa[m,g']) * sb[g,n] )
+ *   lhs asymmetric:  zu = zero points of a (per row, or per row and group), zv[g,n] = sum of b[n, k in group g]
+ *   rhs asymmetric:  zu[m,g] = sum of a[m, k in group g],  zv = zero points of b (per column, or per group and column)
+ * zu[m,g] is read at zu[m * zu_row_stride + g * zu_group_stride], zv[g,n] at zv[n * zv_col_stride +
+ * g * zv_group_stride] (int32, element strides; a group stride of 0 = one value for all groups).
+ * qwix_hip_ksum_groups writes the K-sums.  acc_out, when given, receives the corrected partials.
+ * Everything else as qwix_hip_qgemm_grouped. */
+QWIX_API int qwix_hip_qgemm_grouped_zp(const void* a, int64_t lda, const void* b, int64_t ldb_bytes, int b_qtype,
+                              int64_t M, int64_t N, int64_t K, int64_t group, const void* sa, int sa_dtype,
+                              int64_t ga, const void* sb, int sb_dtype, const int32_t* zu,
+                              int64_t zu_row_stride, int64_t zu_group_stride, const int32_t* zv,
+                              int64_t zv_col_stride, int64_t zv_group_stride, void* out, int out_dtype,
+                              int64_t ldo, int exact, int32_t* acc_out, void* stream);
+
+/* out[r, g] = sum of the g-th group of `group` values of row r, for rows of int8 or packed int4 values
+ * (ld_bytes apart, 16-byte aligned; group a multiple of 128 that divides K); out is (rows, K/group) int32.
+ * The reference obtains these sums as a dot_general of the broadcast zero point against the quantized
+ * values of the other operand (dot_general.py:233-239, 246-252). */
+QWIX_API int qwix_hip_ksum_groups(const void* q, int qtype, int64_t ld_bytes, int64_t rows, int64_t K, int64_t group,
+                         int32_t* out, void* stream);
+
 /* Weight-only skinny GEMM (the reference's _slow_dot_general, dot_general.py:264-275, with
  * the dequantize fused): out[m,n] = sum_k x[m,k] * (q[k,n] * s[k/group, n]).
  *   x   (M,K) bf16 row-major; q int4/int8 K-contiguous rows (n*ldb_bytes); s (K/group, N)

@@ -169,21 +169,29 @@ class _Canon:
     return s.reshape(gb, self.N).contiguous(), gb
 
 
-  # -- zero points (one per row of the lhs / per column of the rhs, like the scales)
-  def lhs_zero_point(self, lhs: QArray) -> torch.Tensor:
+  # -- zero points: shaped like the scales; int32 for the kernels
+  def lhs_zero_point(self, lhs: QArray) -> tuple[torch.Tensor, int]:
+    """(zero points as (M, gz) int32 contiguous, gz): gz > 1 when the last contracting axis is tiled."""
     z = lhs.zero_point
-    if any(z.shape[a] != 1 for a in self.lca):
-      raise NotImplementedError('sub-channel zero points are not supported on the quantized path')
+    if any(z.shape[a] != 1 for a in self.lca[:-1]):
+      raise NotImplementedError('only the last contracting axis of the lhs may carry sub-channel zero points')
+    gz = z.shape[self.lca[-1]]
+    if gz > 1 and len(self.lca) > 1:
+      raise NotImplementedError('sub-channel lhs zero points with several contracting axes are not supported')
     z = _broadcast_free(z, lhs.shape, self.lfree)
-    return z.permute(*(self.lfree + self.lca)).reshape(self.M).contiguous()
+    return z.permute(*(self.lfree + self.lca)).reshape(self.M, gz).to(torch.int32).contiguous(), gz
 
-  def rhs_zero_point(self, rhs: QArray) -> torch.Tensor:
+  def rhs_zero_point(self, rhs: QArray) -> tuple[torch.Tensor, int]:
+    """(zero points as (gz, N) int32 contiguous, gz)."""
     z = rhs.zero_point
-    if any(z.shape[a] != 1 for a in self.rca):
-      raise NotImplementedError('sub-channel zero points are not supported on the quantized path')
+    if any(z.shape[a] != 1 for a in self.rca[:-1]):
+      raise NotImplementedError('only the last contracting axis of the rhs may carry sub-channel zero points')
+    gz = z.shape[self.rca[-1]]
+    if gz > 1 and len(self.rca) > 1:
+      raise NotImplementedError('sub-channel rhs zero points with several contracting axes are not supported')
     z = _broadcast_free(z, rhs.shape, self.rfree)
-    z = z.permute(*(self.rfree + self.rca))
-    return z.reshape(self.N).contiguous()
+    z = z.permute(*([self.rca[-1]] + self.rfree + self.rca[:-1]))
+    return z.reshape(gz, self.N).to(torch.int32).contiguous(), gz
 
 
 # ------------------------------------------------------------------------------------------
@@ -401,11 +409,11 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
       if return_accumulators:
         raise NotImplementedError('raw accumulators are not returned for zero-point operands')
       if lzp is not None:
-        zu = c.lhs_zero_point(lhs).to(torch.int32)
+        zu = c.lhs_zero_point(lhs)[0].reshape(c.M)
         zv = torch.empty(c.N, dtype=torch.int32, device=dev)
         _lib.call('qwix_hip_ksum_i8', b.data_ptr(), b.stride(0), c.N, K, zv.data_ptr(), st)
       else:
-        zv = c.rhs_zero_point(rhs).to(torch.int32)
+        zv = c.rhs_zero_point(rhs)[0].reshape(c.N)
         zu = torch.empty(c.M, dtype=torch.int32, device=dev)
         _lib.call('qwix_hip_ksum_i8', a.data_ptr(), a.stride(0), c.M, K, zu.data_ptr(), st)
       _lib.call('qwix_hip_qgemm_zp', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), c.M, c.N, K,
@@ -426,9 +434,6 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
     out = out.reshape(c.out_shape)
     return (out, acc.reshape(c.out_shape)) if return_accumulators else out
   # sub-channel / int4 weights
-  if lzp is not None or rzp is not None:
-    raise NotImplementedError('zero-point operands with sub-channel scales or int4 values are not supported on the '
-                              'quantized path; dequantize first')
   if lq != numerics.INT8 or rq not in (numerics.INT8, numerics.INT4):
     raise NotImplementedError(f'sub-channel MFMA kernel needs int8 x int8/int4 operands, got {lq} x {rq}')
   ngroups = max(ga, gb)
@@ -440,48 +445,110 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   if gb != ngroups:  # rhs per-channel, lhs tiled: repeat the rhs scale per group
     sb = sb.expand(ngroups, c.N).contiguous()
   acc = torch.empty(ngroups, c.M, c.N, dtype=torch.int32, device=dev) if return_accumulators else None
-  _lib.call('qwix_hip_qgemm_grouped', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
-            _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, group, _lib.ptr(sa),
-            0 if sa is None else _lib.float_tag(sa.dtype), ga, sb.data_ptr(), _lib.float_tag(sb.dtype), out.data_ptr(),
-            _tag_of(res_t), c.N, int(exact), _lib.ptr(acc), st)
+  bq = _lib.INT4 if b_is4 else _lib.INT8
+  if lzp is not None or rzp is not None:
+    # dot_general.py:196-203, 228-253: the zero point is split with the tiles and every tile's partial is
+    # corrected by zero_point x (K-sum of the other operand over that tile) before it is scaled.
+    if lzp is not None:
+      zu, gz = c.lhs_zero_point(lhs)                       # (M, gz)
+      zu_strides = (gz, 1 if gz > 1 else 0)
+      zv = torch.empty(c.N, ngroups, dtype=torch.int32, device=dev)
+      _lib.call('qwix_hip_ksum_groups', b.data_ptr(), bq, b.stride(0), c.N, c.K, group, zv.data_ptr(), st)
+      zv_strides = (ngroups, 1)
+    else:
+      zv, gz = c.rhs_zero_point(rhs)                       # (gz, N)
+      zv_strides = (1, c.N if gz > 1 else 0)
+      zu = torch.empty(c.M, ngroups, dtype=torch.int32, device=dev)
+      _lib.call('qwix_hip_ksum_groups', a.data_ptr(), _lib.INT8, a.stride(0), c.M, c.K, group, zu.data_ptr(), st)
+      zu_strides = (ngroups, 1)
+    if gz not in (1, ngroups):
+      raise ValueError(f'zero points come in {gz} groups along K, the scales in {ngroups}')
+    _lib.call('qwix_hip_qgemm_grouped_zp', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), bq, c.M, c.N, c.K,
+              group, _lib.ptr(sa), 0 if sa is None else _lib.float_tag(sa.dtype), ga, sb.data_ptr(),
+              _lib.float_tag(sb.dtype), zu.data_ptr(), zu_strides[0], zu_strides[1], zv.data_ptr(), zv_strides[0],
+              zv_strides[1], out.data_ptr(), _tag_of(res_t), c.N, int(exact), _lib.ptr(acc), st)
+  else:
+    _lib.call('qwix_hip_qgemm_grouped', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), bq, c.M, c.N, c.K, group,
+              _lib.ptr(sa), 0 if sa is None else _lib.float_tag(sa.dtype), ga, sb.data_ptr(), _lib.float_tag(sb.dtype),
+              out.data_ptr(), _tag_of(res_t), c.N, int(exact), _lib.ptr(acc), st)
   out = out.reshape(c.out_shape)
   return (out, acc.reshape((ngroups,) + c.out_shape)) if return_accumulators else out
 
 
+def _weight_only_fit(lhs, rhs, dimension_numbers):
+  """The canonical form when the fused weight-only kernels (dequantize in registers, bf16 MFMA) take this pair,
+  else None.  The conditions are the kernels' own: a bf16 activation, a symmetric int4/int8 weight whose
+  scales are tiled along the last contracting axis only, in groups that are multiples of 128."""
+  if not (_is_float_array(lhs) and lhs.dtype == torch.bfloat16 and isinstance(rhs, QArray)):
+    return None
+  if rhs.zero_point is not None or _qtype_of(rhs) not in (numerics.INT4, numerics.INT8):
+    return None
+  c = _Canon(lhs, rhs, dimension_numbers)
+  if any(rhs.scale.shape[a] != 1 for a in c.rca[:-1]):
+    return None
+  gb = rhs.scale.shape[c.rca[-1]]
+  if (gb > 1 and len(c.rca) > 1) or c.K % 128 or (c.K // gb) % 128:
+    return None
+  if isinstance(rhs.qvalue, Int4Tensor):  # packed pairs must run along K or along N (one re-layout)
+    order = c.rfree + c.rca
+    packed = (rhs.qvalue.permute(*order).packed_axis, rhs.qvalue.permute(*(c.rca + c.rfree)).packed_axis)
+    if len(order) - 1 not in packed:
+      return None
+  return c
+
+
+# Rows up to which the fused weight-only kernel (one pass over the weight per 16 or 32 rows) is used; above
+# it the weight is dequantized once (HIP kernel) and contracted by the float GEMM.
+WEIGHT_ONLY_MAX_ROWS = 256
+
+
 def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, **kwargs) -> torch.Tensor:
-  """Dequantize-first path.  A bf16 activation against an int4/int8 weight runs in one fused
-  kernel (dequantize in registers, bf16 MFMA); other combinations dequantize then use the vendor GEMM."""
+  """Dequantize-first path (dot_general.py:264-275).  A bf16 activation against an int4/int8 weight runs in one
+  fused kernel (dequantize in registers, bf16 MFMA) when `_weight_only_fit` says the kernel takes it; every
+  other combination is dequantized by the HIP dequantize kernel and contracted by the float GEMM.  Which of
+  the two runs is decided here from the operands alone; a kernel that refuses its arguments raises."""
   del kwargs
   if len(dimension_numbers[1][0]) or len(dimension_numbers[1][1]):
     return _over_batch(_slow_dot_general, lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type)
-  if (_is_float_array(lhs) and lhs.dtype == torch.bfloat16 and isinstance(rhs, QArray) and rhs.zero_point is None
-      and _qtype_of(rhs) in (numerics.INT4, numerics.INT8)):
-    try:
-      c = _Canon(lhs, rhs, dimension_numbers)
-      sb, gb = c.rhs_scale(rhs)
-      group = c.K // gb
-      # up to a few hundred rows the fused kernel (16 rows per pass over the weight) beats
-      # dequantize + float GEMM, which has to write and re-read the whole float weight
-      if c.K % 128 == 0 and (group % 128 == 0) and c.M <= 256:
-        x = c.lhs_values(lhs)
-        b, b_is4 = c.rhs_values(rhs)
-        res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.scale.dtype)
-        out = torch.empty(c.M, c.N, dtype=res_t, device=x.device)
-        _lib.call('qwix_hip_gemv_wq', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0),
-                  _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, group, sb.data_ptr(), _lib.float_tag(sb.dtype),
-                  out.data_ptr(), _lib.float_tag(res_t), c.N, _lib.stream_of(x))
-        return out.reshape(c.out_shape)
-    except NotImplementedError:
-      pass
+  c = _weight_only_fit(lhs, rhs, dimension_numbers)
+  if c is not None and c.M <= WEIGHT_ONLY_MAX_ROWS:
+    sb, gb = c.rhs_scale(rhs)
+    x = c.lhs_values(lhs)
+    b, b_is4 = c.rhs_values(rhs)
+    res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.scale.dtype)
+    out = torch.empty(c.M, c.N, dtype=res_t, device=x.device)
+    _lib.call('qwix_hip_gemv_wq', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0),
+              _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
+              out.data_ptr(), _lib.float_tag(res_t), c.N, _lib.stream_of(x))
+    return out.reshape(c.out_shape)
   if isinstance(lhs, QArray):
     lhs = qarray.dequantize(lhs)
   if isinstance(rhs, QArray):
     rhs = qarray.dequantize(rhs)
-  (lca, rca), _ = dimension_numbers
   res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.dtype)
+  return float_dot_general(lhs, rhs, dimension_numbers, res_t)
+
+
+def float_dot_general(lhs: torch.Tensor, rhs: torch.Tensor, dimension_numbers, preferred_element_type=None) -> torch.Tensor:
+  """lax.dot_general on two float tensors: contracting AND batch axes honoured, result laid out as
+  (batch..., lhs free..., rhs free...).  The float GEMM itself is the vendor library's (torch.einsum)."""
+  (lca, rca), (lba, rba) = dimension_numbers
+  lca, rca, lba, rba = ([int(a) for a in x] for x in (lca, rca, lba, rba))
+  if len(lca) != len(rca) or len(lba) != len(rba):
+    raise TypeError(f'dot_general: contracting / batch axes differ in number: {dimension_numbers}')
+  letters = iter('abcdefghijklmnopqrstuvwxyzABCDEFGHIJKLMNOPQRSTUVWXYZ')
+  lsub = [next(letters) for _ in range(lhs.ndim)]
+  rsub = [None] * rhs.ndim
+  for l, r in list(zip(lca, rca)) + list(zip(lba, rba)):
+    if lhs.shape[l] != rhs.shape[r]:
+      raise TypeError(f'dot_general: sizes of {tuple(lhs.shape)} axis {l} and {tuple(rhs.shape)} axis {r} differ')
+    rsub[r] = lsub[l]
+  rsub = [c if c is not None else next(letters) for c in rsub]
+  out = ([lsub[a] for a in lba] + [lsub[a] for a in range(lhs.ndim) if a not in lca and a not in lba] +
+         [rsub[a] for a in range(rhs.ndim) if a not in rca and a not in rba])
   ct = torch.promote_types(lhs.dtype, rhs.dtype)
-  out = torch.tensordot(lhs.to(ct), rhs.to(ct), dims=(list(lca), list(rca)))
-  return out.to(res_t)
+  res = torch.einsum(f"{''.join(lsub)},{''.join(rsub)}->{''.join(out)}", lhs.to(ct), rhs.to(ct))
+  return res if preferred_element_type is None else res.to(preferred_element_type)
 
 
 def _degenerate(lhs, rhs, dimension_numbers, preferred_element_type):

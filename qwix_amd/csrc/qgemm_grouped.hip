@@ -35,6 +35,11 @@ struct GroupedArgs {
   int t_dtype;      // dtype of the scaled partials (promotion of the scale dtypes)
   uint8_t* out; int out_dtype; int64_t ldo;
   int32_t* acc_out;
+  // Zero-point correction of an asymmetric operand, per group: acc_g[m,n] -= zu[m,g] * zv[g,n].  One array
+  // holds zero points, the other the per-group K-sums of the opposite operand; element strides, 0 along the
+  // group axis for an array that is the same for all groups.  Both null: symmetric operands.
+  const int32_t* zu; int64_t zu_sm, zu_sg;
+  const int32_t* zv; int64_t zv_sn, zv_sg;
 };
 
 __device__ __forceinline__ float ld_scale(const void* p, int dtype, int64_t i) {
@@ -144,14 +149,15 @@ __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
   // acc[i][j][r]: m = m0 + wm*64 + i*32 + 8*(r/4) + 4*(lane/32) + r%4,  n = n0 + wn*(BN/2) + j*32 + lane%32.
   auto row_of = [&](int i, int r) { return m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); };
   auto col_of = [&](int j) { return n0 + wn * (BN / 2) + j * 32 + (lane & 31); };
-  constexpr float kUnscale = W4 ? 0.0625f : 1.0f;
 
   auto flush = [&](int g) {
     float sbv[TN];
+    int zvv[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n = col_of(j);
       sbv[j] = n < p.N ? ld_scale(p.sb, p.sb_dtype, static_cast<int64_t>(g) * p.N + n) : 0.f;
+      zvv[j] = (p.zu != nullptr && n < p.N) ? p.zv[n * p.zv_sn + g * p.zv_sg] : 0;
     }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -161,12 +167,14 @@ __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
         float sav = 1.f;
         if (p.sa != nullptr && (EXACT || p.ga > 1) && m < p.M)
           sav = ld_scale(p.sa, p.sa_dtype, static_cast<int64_t>(m) * p.ga + (p.ga > 1 ? g : 0));
+        const int zuv = (p.zu != nullptr && m < p.M) ? p.zu[m * p.zu_sm + g * p.zu_sg] : 0;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          const int raw = acc[i][j][r];
+          // int4 weights were widened to 16 x value: the partial is an exact multiple of 16
+          const int raw = (W4 ? (acc[i][j][r] >> 4) : acc[i][j][r]) - zuv * zvv[j];
           if (p.acc_out != nullptr && m < p.M && col_of(j) < p.N)
-            p.acc_out[(static_cast<int64_t>(g) * p.M + m) * p.N + col_of(j)] = W4 ? (raw >> 4) : raw;
-          float v = static_cast<float>(raw) * kUnscale;
+            p.acc_out[(static_cast<int64_t>(g) * p.M + m) * p.N + col_of(j)] = raw;
+          float v = static_cast<float>(raw);
           if constexpr (EXACT) {
             // (T(acc) * sa) * sb with one rounding per step, as the reference computes it.
             if (p.sa != nullptr) {
@@ -293,7 +301,11 @@ struct Fast {
 // SAG: the activations carry one scale per row and group as well (both operands tiled along K): the
 // tile's (groups x 128 rows) scales are converted to f32 and parked in LDS behind the slab stages; folding a
 // group in then takes convert, multiply, FMA per accumulator instead of convert, FMA.
-template <int BQT, bool SBF, bool SAG>
+// AUX: the instantiation for asymmetric operands and for parity runs.  Loads, LDS layout, MFMA sequence and
+// epilogue are the ones of the plain instantiation; only the fold of a finished group differs: the int32
+// partial is taken as a plain integer (int4: shifted back by the factor 16 of the widening), corrected by
+// zu[m,g] * zv[g,n] when an operand is asymmetric, written to acc_out when that is given, then scaled.
+template <int BQT, bool SBF, bool SAG, bool AUX>
 __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(GroupedArgs p) {
   constexpr int BM = Fast::kBM, BN = Fast::kBN, BK = Fast::kBK, NW = Fast::kNW, TM = Fast::kTM;
   constexpr bool W4 = (BQT == QWIX_INT4);
@@ -461,6 +473,35 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
       slab(kt, std::false_type{});
     }
     if (in_group == tpg - 1) {
+      const int g = kt / tpg;
+      if constexpr (AUX) {
+        // acc[i][r]: row i*32 + 8*(r/4) + 4*hx + r%4 of the tile, column ncol
+        const int ncol = n0 + wave * 32 + frow;
+        const bool zp = p.zu != nullptr;
+        const int zvl = zp ? p.zv[ncl * p.zv_sn + g * p.zv_sg] : 0;
+        const float sbz = __uint_as_float(SBF ? sb_raw << 16 : sb_raw);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int row = i * 32 + 8 * (r >> 2) + 4 * hx + (r & 3);
+            const int m = m0 + row;
+            int val = W4 ? (acc[i][r] >> 4) : acc[i][r];  // the widened weights carry a factor 16, exactly
+            if (zp) val -= p.zu[min(m, p.M - 1) * p.zu_sm + g * p.zu_sg] * zvl;
+            if (p.acc_out != nullptr && m < p.M && ncol < p.N)
+              p.acc_out[(static_cast<int64_t>(g) * p.M + m) * p.N + ncol] = val;
+            float f = static_cast<float>(val);
+            if constexpr (SAG) f *= sa_lds[g * BM + row];
+            accf[i][r] = __builtin_fmaf(f, sbz, accf[i][r]);
+          }
+        sb_raw = sb_next;
+        __syncthreads();
+        if (kt + 1 < KT) {
+          read_a((kt + 1) & 1, 0, 0);
+          read_b((kt + 1) & 1, 0, 0);
+        }
+        continue;
+      }
       const float sb = __uint_as_float(SBF ? sb_raw << 16 : sb_raw) * kUnscale;
       if constexpr (SAG) {
         // rows of acc[i][4*qd .. 4*qd+3]: i*32 + 8*qd + 4*hx + 0..3, one 16-byte LDS read (a broadcast per half)
@@ -552,12 +593,12 @@ size_t grouped_dma_lds(bool sag, int64_t K, int64_t group) {
   return stages + (sag ? static_cast<size_t>(K / group) * Fast::kBM * sizeof(float) : 0);
 }
 
-template <int BQT, bool SBF, bool SAG>
+template <int BQT, bool SBF, bool SAG, bool AUX>
 int launch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
   constexpr int BM = Fast::kBM, BN = Fast::kBN, NW = Fast::kNW;
   const size_t smem = grouped_dma_lds<BQT>(SAG, p.K, p.group);
   static_assert(2 * (Fast::kBM * Fast::kBK + Fast::kBN * 64) >= NW * 32 * 36 * sizeof(float), "epilogue staging must fit");
-  auto kern = qgemm_grouped_dma_kernel<BQT, SBF, SAG>;
+  auto kern = qgemm_grouped_dma_kernel<BQT, SBF, SAG, AUX>;
   static size_t configured = 0;  // largest dynamic LDS size allowed so far
   if (smem > configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -572,7 +613,49 @@ int launch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
 
 template <int BQT, bool SAG>
 int launch_grouped_dma_sb(const GroupedArgs& p, hipStream_t st) {
-  return p.sb_dtype == QWIX_BF16 ? launch_grouped_dma<BQT, true, SAG>(p, st) : launch_grouped_dma<BQT, false, SAG>(p, st);
+  if (p.zu != nullptr || p.acc_out != nullptr)
+    return p.sb_dtype == QWIX_BF16 ? launch_grouped_dma<BQT, true, SAG, true>(p, st)
+                                   : launch_grouped_dma<BQT, false, SAG, true>(p, st);
+  return p.sb_dtype == QWIX_BF16 ? launch_grouped_dma<BQT, true, SAG, false>(p, st)
+                                 : launch_grouped_dma<BQT, false, SAG, false>(p, st);
+}
+
+// Per-group K-sums of quantized rows: out[row, g] = sum over the g-th group of `group` values of row `row`
+// (int8, or packed int4).  One 16-byte chunk per thread; the chunks of a group that sit in `seg` adjacent
+// lanes (a power of two that divides the chunks per group) are added by shuffles, the rest by integer
+// atomics into the zero-filled output -- integer addition, so the order does not matter.
+__global__ void __launch_bounds__(256) fill_i32_kernel(int32_t* p, int64_t n) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+template <bool W4>
+__global__ void __launch_bounds__(256)
+    ksum_groups_kernel(const uint8_t* __restrict__ q, int64_t ld, int64_t rows, int chunks_per_row, int cpg, int seg,
+                       int G, int32_t* __restrict__ out) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t row = idx / chunks_per_row;
+  const int c = static_cast<int>(idx % chunks_per_row);
+  const bool valid = row < rows;
+  int s = 0;
+  if (valid) {
+    const uint4 w = *reinterpret_cast<const uint4*>(q + row * ld + static_cast<int64_t>(c) * 16);
+    const unsigned u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if constexpr (W4) {  // signed nibble = (nibble ^ 8) - 8
+        const unsigned x = u[e] ^ 0x88888888u;
+        const unsigned t = (x & 0x0F0F0F0Fu) + ((x >> 4) & 0x0F0F0F0Fu);
+        s += static_cast<int>((t * 0x01010101u) >> 24) - 64;
+      } else {             // signed byte = (byte ^ 0x80) - 128
+        const unsigned x = u[e] ^ 0x80808080u;
+        const unsigned t = (x & 0x00FF00FFu) + ((x >> 8) & 0x00FF00FFu);
+        s += static_cast<int>((t & 0xFFFFu) + (t >> 16)) - 512;
+      }
+    }
+  }
+  for (int m = seg >> 1; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
+  if (valid && (c & (seg - 1)) == 0) atomicAdd(out + row * G + c / cpg, s);
 }
 
 }  // namespace
@@ -580,10 +663,42 @@ int launch_grouped_dma_sb(const GroupedArgs& p, hipStream_t st) {
 
 using namespace qwix;
 
-extern "C" int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b, int64_t ldb_bytes, int b_qtype,
-                                      int64_t M, int64_t N, int64_t K, int64_t group, const void* sa, int sa_dtype,
-                                      int64_t ga, const void* sb, int sb_dtype, void* out, int out_dtype, int64_t ldo,
-                                      int exact, int32_t* acc_out, void* stream) {
+extern "C" int qwix_hip_ksum_groups(const void* q, int qtype, int64_t ld_bytes, int64_t rows, int64_t K, int64_t group,
+                                    int32_t* out, void* stream) {
+  if (!q || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null argument");
+  if (qtype != QWIX_INT8 && qtype != QWIX_INT4)
+    return fail(QWIX_ERR_UNSUPPORTED, "K-sums are taken of int8 or int4 values (got qtype %d)", qtype);
+  if (rows <= 0 || K <= 0 || group <= 0 || group % 128 || K % group)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "group %lld must be a multiple of 128 that divides K=%lld (rows=%lld)",
+                (long long)group, (long long)K, (long long)rows);
+  const int64_t row_bytes = qtype == QWIX_INT4 ? K / 2 : K, group_bytes = qtype == QWIX_INT4 ? group / 2 : group;
+  if (ld_bytes % 16 || ld_bytes < row_bytes || !aligned16(q))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "rows must be 16-byte aligned and at least K values long");
+  const int64_t chunks_per_row = row_bytes / 16, cpg = group_bytes / 16, G = K / group;
+  if (chunks_per_row > INT32_MAX || rows * G > (int64_t{1} << 40))
+    return fail(QWIX_ERR_UNSUPPORTED, "shape too large for the K-sum kernel");
+  int seg = 1;
+  while (seg < 64 && cpg % (2 * seg) == 0) seg *= 2;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t n_out = rows * G, n_chunks = rows * chunks_per_row;
+  fill_i32_kernel<<<dim3(static_cast<unsigned>((n_out + 255) / 256)), 256, 0, st>>>(out, n_out);
+  const dim3 grid(static_cast<unsigned>((n_chunks + 255) / 256));
+  if (qtype == QWIX_INT4)
+    ksum_groups_kernel<true><<<grid, 256, 0, st>>>(static_cast<const uint8_t*>(q), ld_bytes, rows,
+                                                   static_cast<int>(chunks_per_row), static_cast<int>(cpg), seg,
+                                                   static_cast<int>(G), out);
+  else
+    ksum_groups_kernel<false><<<grid, 256, 0, st>>>(static_cast<const uint8_t*>(q), ld_bytes, rows,
+                                                    static_cast<int>(chunks_per_row), static_cast<int>(cpg), seg,
+                                                    static_cast<int>(G), out);
+  return check_launch("ksum_groups");
+}
+
+static int grouped_impl(const void* a, int64_t lda, const void* b, int64_t ldb_bytes, int b_qtype, int64_t M, int64_t N,
+                        int64_t K, int64_t group, const void* sa, int sa_dtype, int64_t ga, const void* sb, int sb_dtype,
+                        const int32_t* zu, int64_t zu_row_stride, int64_t zu_group_stride, const int32_t* zv,
+                        int64_t zv_col_stride, int64_t zv_group_stride, void* out, int out_dtype, int64_t ldo,
+                        int exact, int32_t* acc_out, void* stream) {
   if (!a || !b || !out || !sb) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/b/out/sb");
   if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX)
     return fail(QWIX_ERR_INVALID_ARGUMENT, "bad GEMM shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
@@ -601,6 +716,10 @@ extern "C" int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b,
   if ((sa && !ok_s(sa_dtype)) || !ok_s(sb_dtype) || !ok_s(out_dtype))
     return fail(QWIX_ERR_INVALID_ARGUMENT, "scale and output dtypes must be f32 or bf16");
   if (ldo < N || !aligned16(out)) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad output leading dimension");
+  if ((zu == nullptr) != (zv == nullptr))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "zu and zv come together (zero points and the other operand's K-sums)");
+  if (zu && (zu_row_stride < 0 || zu_group_stride < 0 || zv_col_stride < 0 || zv_group_stride < 0))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "negative zero-point stride");
   GroupedArgs p;
   p.A = static_cast<const uint8_t*>(a); p.lda = lda;
   p.B = static_cast<const uint8_t*>(b); p.ldb = ldb_bytes;
@@ -610,9 +729,11 @@ extern "C" int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b,
   p.t_dtype = (sb_dtype == QWIX_F32 || (sa && sa_dtype == QWIX_F32)) ? QWIX_F32 : QWIX_BF16;
   p.out = static_cast<uint8_t*>(out); p.out_dtype = out_dtype; p.ldo = ldo;
   p.acc_out = acc_out;
+  p.zu = zu; p.zu_sm = zu_row_stride; p.zu_sg = zu_group_stride;
+  p.zv = zv; p.zv_sn = zv_col_stride; p.zv_sg = zv_group_stride;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool row_strides_fit = 128 * lda < (int64_t{1} << 31) && 256 * ldb_bytes < (int64_t{1} << 31);
-  if (!exact && acc_out == nullptr && row_strides_fit) {
+  if (!exact && row_strides_fit) {
     // per-group activation scales ride along in LDS: the tile's scales must fit behind the slab stages
     const bool sag = sa != nullptr && ga > 1;
     constexpr size_t kLdsMax = 160 * 1024;
@@ -627,4 +748,23 @@ extern "C" int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b,
   if (b_qtype == QWIX_INT4)
     return exact ? launch_grouped<QWIX_INT4, true>(p, st) : launch_grouped<QWIX_INT4, false>(p, st);
   return exact ? launch_grouped<QWIX_INT8, true>(p, st) : launch_grouped<QWIX_INT8, false>(p, st);
+}
+
+extern "C" int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b, int64_t ldb_bytes, int b_qtype,
+                                      int64_t M, int64_t N, int64_t K, int64_t group, const void* sa, int sa_dtype,
+                                      int64_t ga, const void* sb, int sb_dtype, void* out, int out_dtype, int64_t ldo,
+                                      int exact, int32_t* acc_out, void* stream) {
+  return grouped_impl(a, lda, b, ldb_bytes, b_qtype, M, N, K, group, sa, sa_dtype, ga, sb, sb_dtype, nullptr, 0, 0,
+                      nullptr, 0, 0, out, out_dtype, ldo, exact, acc_out, stream);
+}
+
+extern "C" int qwix_hip_qgemm_grouped_zp(const void* a, int64_t lda, const void* b, int64_t ldb_bytes, int b_qtype,
+                                         int64_t M, int64_t N, int64_t K, int64_t group, const void* sa, int sa_dtype,
+                                         int64_t ga, const void* sb, int sb_dtype, const int32_t* zu,
+                                         int64_t zu_row_stride, int64_t zu_group_stride, const int32_t* zv,
+                                         int64_t zv_col_stride, int64_t zv_group_stride, void* out, int out_dtype,
+                                         int64_t ldo, int exact, int32_t* acc_out, void* stream) {
+  if (!zu || !zv) return fail(QWIX_ERR_INVALID_ARGUMENT, "null zu/zv");
+  return grouped_impl(a, lda, b, ldb_bytes, b_qtype, M, N, K, group, sa, sa_dtype, ga, sb, sb_dtype, zu, zu_row_stride,
+                      zu_group_stride, zv, zv_col_stride, zv_group_stride, out, out_dtype, ldo, exact, acc_out, stream);
 }

@@ -167,9 +167,9 @@ class BoxedParamProvider(qconfig.QuantizationProvider):
   def dot_general(self, lhs, rhs, dimension_numbers, precision=None, preferred_element_type=None, *, out_sharding=None):
     rule, op_id = self._get_current_rule_and_op_id('dot_general')
     if rule is None or rule.weight_qtype is None:
-      (lc, rc), _ = dimension_numbers
-      out = torch.tensordot(self._unbox_float(lhs), self._unbox_float(rhs), dims=(list(lc), list(rc)))
-      return out if preferred_element_type is None else out.to(preferred_element_type)
+      # no rule for this op: the float contraction, batch axes included (boxed_param.py:119-127)
+      return _dot_general.float_dot_general(self._unbox_float(lhs), self._unbox_float(rhs), dimension_numbers,
+                                            preferred_element_type)
     get_how = functools.partial(_dot_general.get_how_to_quantize, dimension_numbers=dimension_numbers,
                                 ndims=(len(lhs.shape), len(rhs.shape)), tile_size=rule.tile_size)
     if self._fusable(rule) and isinstance(lhs, torch.Tensor) and lhs.numel() // max(lhs.shape[-1], 1) <= 32:

@@ -230,3 +230,86 @@ def test_two_dim_scales_on_the_quantized_path(lt, rt, dtype):
   fast = dg.dot_general(xq, wq, DN)
   true = O.dequantize(oxq).v.astype(np.float64) @ O.dequantize(owq).v.astype(np.float64)
   assert _close(util.f32np(fast), true, dtype)
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('M,K,N,group,lhs_tile', [(256, 1024, 512, 128, None), (200, 512, 264, 128, None),
+                                                  (130, 1024, 258, 256, None), (300, 2048, 1000, 128, 128)])
+def test_fast_kernel_int32_partials_are_bit_exact(M, K, N, group, lhs_tile, wq_type, dtype):
+  """The kernel that serves dot_general by default (global -> LDS slabs, f32 sum of the scaled partials)
+  dumps its per-group int32 partials on request: they are the reference's accumulators, bit for bit, and
+  the outputs of the run that dumps equal those of the run that does not."""
+  from qwix_amd.core import dot_general as dg
+  print('case grouped fast acc', M, K, N, group, lhs_tile, wq_type, dtype, flush=True)
+  xq, wq, oxq, owq, _, _ = _pair(M, K, N, dtype, wq_type, group, seed=21 + M, lhs_tile=lhs_tile)
+  out, acc = dg._fast_dot_general(xq, wq, DN, exact=False, return_accumulators=True)
+  plain = dg._fast_dot_general(xq, wq, DN, exact=False)
+  torch.cuda.synchronize()
+  _, wacc = O.fast_dot_general(oxq, owq, DN, return_acc=True)
+  assert np.array_equal(acc.cpu().numpy(), wacc), 'per-group int32 partials of the fast kernel differ'
+  assert torch.equal(out, plain)
+
+
+def _zp_pair(M, K, N, dtype, wq_type, group, seed, side, zp_tiled):
+  """One asymmetric (minmax) operand; `zp_tiled`: that operand is tiled along K, so its zero point is per group."""
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make((M, K), dtype, seed=seed, dist='uniform')
+  w_np, w_t = util.make((K, N), dtype, seed=seed + 1, scale=0.02)
+  w_np = w_np + np.float32(0.01)  # off-centre weights: a zero point that matters
+  w_np = O.round_to_bf16(w_np) if dtype is O.BF16 else w_np
+  w_t = util.to_gpu(w_np, dtype)
+  lkw = dict(qtype='int8', channelwise_axes=[0])
+  rkw = dict(qtype=wq_type, channelwise_axes=[1])
+  if side == 'lhs':
+    lkw['calibration_method'] = 'minmax'
+    if zp_tiled:
+      lkw['tiled_axes'] = {1: group}
+    rkw['tiled_axes'] = {0: group}
+  else:
+    rkw['calibration_method'] = 'minmax'
+    if zp_tiled:
+      rkw['tiled_axes'] = {0: group}
+    else:
+      lkw['tiled_axes'] = {1: group}
+  xq = qarray.quantize(x_t, qarray.HowToQuantize(**lkw))
+  wq = qarray.quantize(w_t, qarray.HowToQuantize(**rkw))
+  oxq = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(**lkw))
+  owq = O.quantize(O.FArr(w_np, dtype), O.HowToQuantize(**rkw))
+  util.assert_qarray_equal(xq, oxq, 'lhs')
+  util.assert_qarray_equal(wq, owq, 'rhs')
+  return xq, wq, oxq, owq
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('zp_tiled', [True, False])
+@pytest.mark.parametrize('side', ['lhs', 'rhs'])
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('M,K,N,group', [(200, 512, 264, 128), (130, 1024, 258, 256)])
+def test_sub_channel_zero_points_bit_exact(M, K, N, group, wq_type, side, zp_tiled, dtype):
+  """A tiled contraction with one asymmetric operand (dot_general.py:196-203, 228-253): the zero point is split
+  with the tiles and zero_point x K-sum is subtracted from every tile's partial.  Corrected int32 partials and
+  (exact mode) outputs equal the oracle's bit for bit, from both kernels; the default mode stays within the
+  envelope of the reference's own per-partial roundings."""
+  from qwix_amd.core import dot_general as dg
+  print('case grouped zp', M, K, N, group, wq_type, side, zp_tiled, dtype, flush=True)
+  xq, wq, oxq, owq = _zp_pair(M, K, N, dtype, wq_type, group, 31 + M, side, zp_tiled)
+  want, wacc = O.fast_dot_general(oxq, owq, DN, return_acc=True)
+  out, acc = dg._fast_dot_general(xq, wq, DN, exact=True, return_accumulators=True)
+  torch.cuda.synchronize()
+  assert np.array_equal(acc.cpu().numpy(), wacc), 'corrected partials differ (register-staged kernel)'
+  got = util.f32np(out)
+  bad = np.flatnonzero(got.ravel() != want.v.ravel())
+  assert bad.size == 0, f'{bad.size} outputs differ: {got.ravel()[bad[:5]]} vs {want.v.ravel()[bad[:5]]}'
+  out, acc = dg._fast_dot_general(xq, wq, DN, exact=False, return_accumulators=True)
+  plain = dg.dot_general(xq, wq, DN)   # the dispatcher sends the pair to the quantized path, as the reference does
+  torch.cuda.synchronize()
+  assert np.array_equal(acc.cpu().numpy(), wacc), 'corrected partials differ (global -> LDS kernel)'
+  assert torch.equal(out, plain)
+  G = K // group
+  sa = np.asarray(oxq.scale.v, np.float64)
+  sa = sa.reshape(M, -1).T.reshape(-1, M, 1)               # (1 or G, M, 1)
+  sb = np.asarray(owq.scale.v, np.float64).reshape(-1, 1, N)  # (1 or G, 1, N)
+  parts = np.asarray(wacc, np.float64).reshape(G, M, N) * sa * sb
+  rt = 2.0 ** -6 if dtype is O.BF16 else 1e-5
+  assert np.all(np.abs(util.f32np(plain) - want.v) <= rt * np.abs(parts).sum(0) + 1e-30)

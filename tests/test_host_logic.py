@@ -244,3 +244,29 @@ def test_simple_moving_average_statistics():
   stat = agg.update(stat, cal)
   out = boot.get_calibration(stat, cal)
   assert out['max'].dtype == torch.bfloat16 and abs(out['max'].item() - 10.0 / 3) < 0.02
+
+
+def test_provider_pass_through_honours_batch_axes():
+  """An op that no rule covers (or whose rule has no weight_qtype) is the float lax.dot_general, batch axes
+  included (boxed_param.py:119-127): (2,3,4) x (2,5,4) over batch 0 gives (2,3,5), not (2,3,2,5)."""
+  from qwix_amd.providers import ptq
+  g = torch.Generator().manual_seed(0)
+  a, b = torch.randn(2, 3, 4, generator=g), torch.randn(2, 5, 4, generator=g)
+  dn = (((2,), (2,)), ((0,), (0,)))
+  want = torch.einsum('bik,bjk->bij', a, b)
+  out = ptq.PtqProvider([]).dot_general(a, b, dn)
+  assert out.shape == (2, 3, 5) and torch.allclose(out, want, atol=1e-6)
+  # a rule exists but does not match this module path; and a rule that matches but quantizes nothing
+  for rules in ([qconfig.QuantizationRule(module_path='elsewhere', weight_qtype='int8')],
+                [qconfig.QuantizationRule(module_path='.*', weight_qtype=None)]):
+    with qconfig.module_scope('attn'):
+      out = ptq.PtqProvider(rules).dot_general(a, b, dn, preferred_element_type=torch.bfloat16)
+    assert out.dtype == torch.bfloat16 and out.shape == (2, 3, 5)
+    assert torch.allclose(out.float(), want, atol=2e-2, rtol=2e-2)
+  # several batch axes, batch axes not leading, two contracting axes: layout (batch..., lhs free..., rhs free...)
+  a, b = torch.randn(3, 2, 4, 5, generator=g), torch.randn(5, 4, 6, 2, 3, generator=g)
+  dn = (((2, 3), (1, 0)), ((1, 0), (3, 4)))
+  out = dg.float_dot_general(a, b, dn)
+  assert torch.allclose(out, torch.einsum('cbkl,lknbc->bcn', a, b), atol=1e-5)
+  with pytest.raises(TypeError, match='differ'):
+    dg.float_dot_general(torch.zeros(2, 3), torch.zeros(4, 3), (((0,), (0,)), ((), ())))
