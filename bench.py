@@ -801,6 +801,7 @@ class PtqMlpGraph(Workload):
 
 
 WORKLOADS = {
+    'quantize_act_8192': lambda: QuantizeRows('quantize_act_8192', 8192, 8192, 'int8'),
     'c3_int8_w8a8_4096': lambda: QdotW8A8('c3_int8_w8a8_4096', 4096, 4096, 4096, 'int8'),
     'c4_fp8_w8a8_ffn': lambda: QdotW8A8('c4_fp8_w8a8_ffn', 8192, 8192, 28672, 'float8_e4m3fn'),
     'c3_fp8_w8a8_4096': lambda: QdotW8A8('c3_fp8_w8a8_4096', 4096, 4096, 4096, 'float8_e4m3fn'),
@@ -833,7 +834,7 @@ WORKLOADS = {
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
 }
 DEFAULT = 'c3_int8_w8a8_4096'
-EXTRA = ['quantize_act_4096', 'quantize_act_8192_fp8', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
+EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
          'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'moe_ragged_int8_8x1024',
          'moe_ragged_int8_64x128', 'moe_decode_int8_64x4', 'quantize_weight_fp8_block128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 
@@ -849,8 +850,15 @@ def _blas_threads() -> int:
   return int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1))
 
 
-def run(wl: Workload, steps: int, warmup: int, spin_up: float = None):
-  """Returns (seconds per step, seconds per launch of the dominant kernel)."""
+REPEATS = 7               # the timed region (exactly `steps` steps) is repeated; the median is reported
+
+
+def run(wl: Workload, steps: int, warmup: int, spin_up: float = None, repeats: int = REPEATS):
+  """Returns (seconds per step, seconds per launch of the dominant kernel, timing summary).
+
+  Both figures are medians over `repeats` repetitions of a timed region of exactly `steps` steps, each
+  bracketed by a device synchronisation on both sides: a single region of 50 x 80 us is 4 ms, short enough
+  for one clock excursion to decide it."""
   import torch
   dev = torch.device('cuda:0')
   wl.setup(dev)
@@ -865,22 +873,32 @@ def run(wl: Workload, steps: int, warmup: int, spin_up: float = None):
     if i % 16 == 0:
       torch.cuda.synchronize()
   torch.cuda.synchronize()
-  t0 = time.perf_counter()
-  for i in range(steps):
-    wl.step(i)
-  torch.cuda.synchronize()
-  dt = time.perf_counter() - t0
+  step_t = []
+  for _ in range(repeats):
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+      wl.step(i)
+    torch.cuda.synchronize()
+    step_t.append((time.perf_counter() - t0) / steps)
   # the dominant kernel alone, on the inputs the last step left behind
   e0, e1 = _events(2)
   for i in range(min(warmup, 3)):
     wl.kernel(i)
-  torch.cuda.synchronize()
-  e0.record()
-  for i in range(steps):
-    wl.kernel(i)
-  e1.record()
-  torch.cuda.synchronize()
-  return dt / steps, e0.elapsed_time(e1) * 1e-3 / steps
+  kern_t = []
+  for _ in range(repeats):
+    torch.cuda.synchronize()
+    e0.record()
+    for i in range(steps):
+      wl.kernel(i)
+    e1.record()
+    torch.cuda.synchronize()
+    kern_t.append(e0.elapsed_time(e1) * 1e-3 / steps)
+  med = lambda v: sorted(v)[len(v) // 2]
+  timing = {'repeats': repeats, 'step_ms_min': round(min(step_t) * 1e3, 5), 'step_ms_median': round(med(step_t) * 1e3, 5),
+            'step_ms_max': round(max(step_t) * 1e3, 5), 'kernel_us_min': round(min(kern_t) * 1e6, 3),
+            'kernel_us_median': round(med(kern_t) * 1e6, 3)}
+  return med(step_t), med(kern_t), timing
 
 
 def summarize(wl: Workload, step_s: float, kern_s: float) -> dict:
@@ -895,7 +913,7 @@ def summarize(wl: Workload, step_s: float, kern_s: float) -> dict:
       'value': round(value, 2), 'unit': wl.unit, 'ms_per_step': round(step_s * 1e3, 5),
       'roofline': {'bound': rb, 'kernel': wl.kernel_name, 'achieved': round(achieved, 2), 'peak': peak,
                    'unit': 'TFLOP/s' if rb == 'mfma' else 'GB/s', 'frac': round(achieved / peak, 4),
-                   'traffic': _traffic(wl.name)},
+                   'traffic': _traffic(wl.name), **_mfma_util(wl.name)},
   }
 
 
@@ -910,12 +928,27 @@ def _traffic(name: str):
   return None
 
 
+def _mfma_util(name: str) -> dict:
+  """Matrix-core utilisation of the dominant kernel from committed rocprofv3 --pmc measurements
+  (SQ_VALU_MFMA_BUSY_CYCLES / SQ_BUSY_CYCLES and friends; profiles/mfma_util.json), {} when not measured."""
+  p = os.path.join(ROOT, 'profiles', 'mfma_util.json')
+  if os.path.exists(p):
+    try:
+      v = json.load(open(p)).get(name)
+      return {'mfma_util': v} if v is not None else {}
+    except Exception:
+      return {}
+  return {}
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument('--gpus', type=int, default=1)
   ap.add_argument('--steps', type=int, default=50)
   ap.add_argument('--warmup', type=int, default=5)
   ap.add_argument('--workload', default=DEFAULT, choices=sorted(WORKLOADS))
+  ap.add_argument('--repeats', type=int, default=REPEATS,
+                  help='repetitions of the timed region of --steps steps; the median is reported')
   ap.add_argument('--no-extra', action='store_true', help='skip the other workloads of the metric')
   ap.add_argument('--no-cpu-baseline', action='store_true')
   ap.add_argument('--spin-up', type=float, default=SPIN_UP_S,
@@ -931,13 +964,13 @@ def main():
     sys.exit(2)
 
   wl = WORKLOADS[args.workload]()
-  step_s, kmean = run(wl, args.steps, args.warmup, args.spin_up)
+  step_s, kmean, timing = run(wl, args.steps, args.warmup, args.spin_up, args.repeats)
   res = summarize(wl, step_s, kmean)
   line = {
       'metric': wl.metric, 'value': res['value'], 'unit': res['unit'], 'n_gpus': 1, 'steps': args.steps,
       'warmup': args.warmup, 'ms_per_step': res['ms_per_step'], 'higher_is_better': True, 'scaling': 'weak',
       'vs_baseline': None, 'dtype': wl.dtype, 'data': 'synthetic', 'config': wl.describe(),
-      'roofline': res['roofline'],
+      'roofline': res['roofline'], 'timing': timing,
   }
   if not args.no_cpu_baseline and hasattr(wl, 'cpu_baseline'):
     line['cpu_baseline'] = wl.cpu_baseline()
@@ -948,7 +981,7 @@ def main():
     for name in EXTRA:
       w = WORKLOADS[name]()
       n = max(5, min(args.steps, 20))
-      s, km = run(w, n, 3, args.spin_up)
+      s, km, _ = run(w, n, 3, args.spin_up, min(args.repeats, 5))
       r = summarize(w, s, km)
       extra[name] = {'metric': w.metric, 'value': r['value'], 'unit': r['unit'], 'ms_per_step': r['ms_per_step'],
                      'roofline': r['roofline']}

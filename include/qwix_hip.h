@@ -7,7 +7,8 @@
  *   - only enqueues work on that stream (no hipMalloc/hipFree, no device sync),
  *   - returns QWIX_OK or an error code; qwix_hip_last_error() gives the text of
  *     the calling thread's last error,
- *   - is re-entrant and keeps no mutable global state.
+ *   - is re-entrant; the only state the library keeps is, per kernel and device, the dynamic-LDS limit it has
+ *     already raised (an atomic), and the per-device address of the scratch array of qwix_hip_quantize_static.
  * These are exactly the symbols a jax.ffi custom-call handler (or ctypes, or a
  * torch extension) binds; the reference functions they replace are cited per
  * entry (paths relative to the google/qwix tree).

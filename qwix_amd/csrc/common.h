@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
@@ -25,6 +26,24 @@ inline int fail(int code, const char* fmt, ...) {
 inline int check_launch(const char* what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return QWIX_OK;
+}
+// Dynamic-LDS limit of a kernel (hipFuncAttributeMaxDynamicSharedMemorySize), raised when a launch needs more
+// than was granted so far on the current device.  Safe to call from several threads: the attribute call is
+// idempotent and the record of what was granted is atomic; the library keeps no other mutable state.
+struct LdsGrant {
+  static constexpr int kDevices = 64;
+  std::atomic<size_t> bytes[kDevices];
+};
+inline int grant_lds(const void* kernel, size_t bytes, LdsGrant& g) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= LdsGrant::kDevices)
+    return fail(QWIX_ERR_LAUNCH, "no current HIP device (index %d)", dev);
+  size_t have = g.bytes[dev].load(std::memory_order_acquire);
+  if (bytes <= have) return QWIX_OK;
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes));
+  if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  while (have < bytes && !g.bytes[dev].compare_exchange_weak(have, bytes, std::memory_order_release)) {}
   return QWIX_OK;
 }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }

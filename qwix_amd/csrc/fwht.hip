@@ -381,13 +381,8 @@ int launch_fwht_reg(const void* x, int64_t rows, const void* pre, const void* po
   constexpr int n = 1 << B;
   constexpr size_t smem = static_cast<size_t>(n + n / 32 + 32) * sizeof(float);
   auto kern = fwht_reg_kernel<D, MODE, QT, B>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   kern<<<dim3(static_cast<unsigned>(rows)), RegFwht<B>::kThreads, smem, st>>>(x, pre, post, out_scale, ltile, y, scale);
   return check_launch("fwht (register passes)");
 }

@@ -257,13 +257,8 @@ extern "C" int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64
 #define QWIX_GEMV_KERNEL(KERN, NW, NTT, RTT)                                                                \
   do {                                                                                                     \
     constexpr size_t smem = sizeof(float) * NW * RTT * NTT * 4 * 64;                                       \
-    static bool configured = false;                                                                        \
-    if (!configured && smem >= 65536) {                                                                     \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(KERN),                              \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)); \
-      if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));  \
-      configured = true;                                                                                   \
-    }                                                                                                      \
+    static LdsGrant granted;                                                                               \
+    if (smem >= 65536) if (int e_ = grant_lds(reinterpret_cast<const void*>(KERN), smem, granted)) return e_;\
     KERN<<<grid, NW * 64, smem, st>>>(p);                                                                  \
   } while (0)
 #define QWIX_GEMV_LAUNCH_RT(NW, NTT, RTT)                                                                  \

@@ -29,24 +29,6 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kPad = 16;
 
-// Optional in-kernel timing (development builds only: -DQWIX_GEMM_DEBUG).  Each wavefront records
-// s_memtime stamps / accumulated intervals into a device array that a test harness copies out.
-#ifdef QWIX_GEMM_DEBUG
-__device__ unsigned long long qwix_dbg[4096 * 8];
-#define QWIX_DBG_NOW() ([] { __builtin_amdgcn_sched_barrier(0); unsigned long long t_ = __builtin_readcyclecounter(); __builtin_amdgcn_sched_barrier(0); return t_; }())
-#define QWIX_DBG_DECL unsigned long long dbg_t[8] = {0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long dbg_last = 0;
-#define QWIX_DBG_STAMP(i) dbg_t[i] = QWIX_DBG_NOW();
-#define QWIX_DBG_BEGIN() dbg_last = QWIX_DBG_NOW();
-#define QWIX_DBG_ACC(i) { unsigned long long n_ = QWIX_DBG_NOW(); dbg_t[i] += n_ - dbg_last; dbg_last = n_; }
-#define QWIX_DBG_FLUSH() if ((threadIdx.x & 63) == 0 && blockIdx.x < 512) { for (int i_ = 0; i_ < 8; ++i_) qwix_dbg[(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + i_] = dbg_t[i_]; }
-#else
-#define QWIX_DBG_DECL
-#define QWIX_DBG_STAMP(i)
-#define QWIX_DBG_BEGIN()
-#define QWIX_DBG_ACC(i)
-#define QWIX_DBG_FLUSH()
-#endif
-
 // Epilogue description.  The reference scales the accumulator as ((T(acc) * sa) * sb) with one
 // rounding per step in the promoted dtype; which of those roundings are to bf16 is decided on the
 // host (r0: the converted accumulator, r1: after the lhs scale, r2: after the rhs scale).
@@ -295,33 +277,24 @@ __device__ __forceinline__ void qgemm_tile(const uint8_t* __restrict__ A, int64_
   };
 
   const int KT = (K + BK - 1) / BK;
-  QWIX_DBG_DECL
-  QWIX_DBG_STAMP(0)
   load_global(0);
   store_lds(0);
   __syncthreads();
   read_frags(0, 0, 0);
-  QWIX_DBG_STAMP(1)
   for (int kt = 0; kt < KT; ++kt) {
     const int cur = kt & 1;
     const bool has_next = kt + 1 < KT;
-    QWIX_DBG_BEGIN()
     if (has_next) load_global((kt + 1) * BK);
 #pragma unroll
     for (int ks = 0; ks + 1 < NK; ++ks) {
       read_frags(cur, ks + 1, (ks + 1) & 1);
       mfma_step(ks & 1);
     }
-    QWIX_DBG_ACC(4)
     if (has_next) store_lds(cur ^ 1);
-    QWIX_DBG_ACC(5)
     __syncthreads();
-    QWIX_DBG_ACC(6)
     if (has_next) read_frags(cur ^ 1, 0, 0);
     mfma_step((NK - 1) & 1);
-    QWIX_DBG_ACC(7)
   }
-  QWIX_DBG_STAMP(2)
 
   const int m_base = m0 + wm * (BM / 2), n_base = n0 + wn * (BN / 2);
   if (ep.out_dtype == QWIX_BF16) {
@@ -331,8 +304,6 @@ __device__ __forceinline__ void qgemm_tile(const uint8_t* __restrict__ A, int64_
   } else {
     if constexpr (IS_INT) write_tile<QWIX_I32, TM, TN>(acc, ep, m_base, n_base, lane, M, N, out, ldo);
   }
-  QWIX_DBG_STAMP(3)
-  QWIX_DBG_FLUSH()
 }
 
 template <int QT, int BM, int BN, int BK>
@@ -610,16 +581,12 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
   float sav[TM];
   fetch_scales<OUT, TM, TN>(ep, m_base, n_base, M, N, lane, sav, sbv);
   const int KT = K / BK;
-  QWIX_DBG_DECL
-  QWIX_DBG_STAMP(0)
   issue_loads(0, 0);
   __syncthreads();
   read_frags(0, 0, 0);
-  QWIX_DBG_STAMP(1)
   // All loads of a slab are issued during its first k-step, giving them the rest of the slab to land.
   for (int kt = 0; kt < KT - 1; ++kt) {
     const int cur = kt & 1;
-    QWIX_DBG_BEGIN()
     issue_loads(cur ^ 1, (kt + 1) * BK);
 #pragma unroll
     for (int ks = 0; ks + 1 < NK; ++ks) {
@@ -627,13 +594,9 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
       mfma_step(ks & 1);
       hint_kstep(ks == 0 ? LOADS : 0);
     }
-    QWIX_DBG_ACC(4)
     mfma_step((NK - 1) & 1);
-    QWIX_DBG_ACC(5)
     __syncthreads();
-    QWIX_DBG_ACC(6)
     read_frags(cur ^ 1, 0, 0);
-    QWIX_DBG_ACC(7)
   }
   {  // last slab: nothing left to fetch
     const int cur = (KT - 1) & 1;
@@ -644,12 +607,9 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
     }
     mfma_step((NK - 1) & 1);
   }
-  QWIX_DBG_STAMP(2)
 
   staged_epilogue<OUT, EPI, TM, TN, NWAVES, 2 * STAGE>(acc, sav, sbv, ep, m_base, n_base, M, N, out, ldo, smem, wave,
                                                          lane);
-  QWIX_DBG_STAMP(3)
-  QWIX_DBG_FLUSH()
 }
 
 template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI>
@@ -666,13 +626,8 @@ int launch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
                const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   constexpr size_t smem = 2 * (BM + BN) * 128;
   auto kern = qgemm_dma_kernel<QT, BM, BN, WGM, WGN, OUT, EPI>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   kern<<<dim3(static_cast<unsigned>(tiles)), WGM * WGN * 64, smem, st>>>(
       static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),
@@ -1022,13 +977,8 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
     constexpr int kDepth = DD; /* the groups in flight must stay under vmcnt's 63 */                               \
     constexpr size_t smem = kDepth * 32 * TMM * 128 > 20480 ? kDepth * 32 * TMM * 128 : 20480;                     \
     auto kern = qgemm_mid_kernel<QT, OUT, EPI, TMM, kDepth, NWW>;                                                 \
-    static bool configured = false;                                                                               \
-    if (!configured) {                                                                                            \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                     \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));     \
-      if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));         \
-      configured = true;                                                                                          \
-    }                                                                                                             \
+    static LdsGrant granted;                                                                                      \
+    if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;                        \
     kern<<<dim3(static_cast<unsigned>((N + 32 * NWW - 1) / (32 * NWW)),                                           \
                 static_cast<unsigned>((M + 32 * TMM - 1) / (32 * TMM))), 64 * NWW, smem, st>>>(                    \
         static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),            \
@@ -1054,13 +1004,8 @@ int launch_mid(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
     constexpr int kKW = 4;                                                                                        \
     constexpr size_t smem = 20480 + kKW * TMM * 4096;                                                             \
     auto kern = qgemm_ksplit_kernel<QT, OUT, EPI, TMM, DD, kKW>;                                                  \
-    static bool configured = false;                                                                               \
-    if (!configured) {                                                                                            \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                     \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));     \
-      if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));         \
-      configured = true;                                                                                          \
-    }                                                                                                             \
+    static LdsGrant granted;                                                                                      \
+    if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;                        \
     kern<<<dim3(static_cast<unsigned>((N + 31) / 32)), 64 * kKW, smem, st>>>(                                     \
         static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),            \
         static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo, kmul);                     \
@@ -1194,11 +1139,31 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
   };
 
   const int KT = K / BK;  // >= 2
+  // The scale vectors are first needed in the epilogue, where a cold fetch (address translation plus a trip
+  // to HBM) would stall every wavefront with nothing to hide behind.  Touch this wavefront's pieces of them
+  // now, under the equally cold first slab loads: 128 row scales and 64 column scales, 8 / 4 bytes per lane.
+  uint32_t warm_a = 0, warm_b = 0;
+  if constexpr (OUT != QWIX_I32) {
+    const int m_base = m0 + wm * 128, n_base = n0 + wn * 64;
+    if (ep.sa != nullptr) {
+      const int64_t es = ep.sa_dtype == QWIX_BF16 ? 2 : 4;
+      const int64_t want = (static_cast<int64_t>(m_base) * es + lane * 8) & ~int64_t{3}, last = (M * es - 4) & ~int64_t{3};
+      const int64_t off = want < last ? want : last;
+      warm_a = *reinterpret_cast<const uint32_t*>(static_cast<const uint8_t*>(ep.sa) + off);
+    }
+    if (ep.sb != nullptr) {
+      const int64_t es = ep.sb_dtype == QWIX_BF16 ? 2 : 4;
+      const int64_t want = (static_cast<int64_t>(n_base) * es + lane * 4) & ~int64_t{3}, last = (N * es - 4) & ~int64_t{3};
+      const int64_t off = want < last ? want : last;
+      warm_b = *reinterpret_cast<const uint32_t*>(static_cast<const uint8_t*>(ep.sb) + off);
+    }
+  }
   // ---- prologue: A of slab 0, B of slabs 0 and 1 (each wavefront its rows)
   load_a(0);
   load_b(0, 0);
   load_b(1, 1);
   wait_loads(0);
+  asm volatile("" ::"v"(warm_a), "v"(warm_b));  // the touches above have landed too; their values are not used
   barrier();
   if (wm == 1) barrier();  // the lower group starts half a slab late
 
@@ -1206,19 +1171,14 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
   // loads have three phases to land); A one slab ahead, in the memory phase.  The waits before the
   // barriers leave the four loads just issued in flight and cover the four issued one phase earlier.
   int bst = 0;  // B stage of slab kt = kt % 3
-  QWIX_DBG_DECL
-  QWIX_DBG_STAMP(0)
   for (int kt = 0; kt < KT; ++kt) {
-    QWIX_DBG_BEGIN()
     // memory phase
     read_slab(kt & 1, bst);
     __builtin_amdgcn_sched_barrier(0);  // fragment reads first: the loads below may not slip in front of them
     const bool more_a = kt + 1 < KT, more_b = kt + 2 < KT;
     if (more_a) load_a(kt + 1);
     if (more_a) wait_loads(4); else wait_loads(0);
-    QWIX_DBG_ACC(2)
     barrier();
-    QWIX_DBG_ACC(3)
     // compute phase
     const int bst2 = bst == 0 ? 2 : bst - 1;  // (kt + 2) % 3
     const uint8_t* gkb = B + (kt + 2) * BK;
@@ -1242,14 +1202,10 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
       __builtin_amdgcn_sched_barrier(0);
     }
     __builtin_amdgcn_s_setprio(0);
-    QWIX_DBG_ACC(4)
     if (more_b) wait_loads(4); else wait_loads(0);
-    QWIX_DBG_ACC(5)
     barrier();
-    QWIX_DBG_ACC(6)
     bst = bst == 2 ? 0 : bst + 1;
   }
-  QWIX_DBG_STAMP(1)
   if (wm == 0) barrier();
 
   const int m_base = m0 + wm * 128, n_base = n0 + wn * 64;
@@ -1257,7 +1213,6 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
   float sbv[TN][4][4];
   fetch_scales<OUT, TM, TN>(ep, m_base, n_base, M, N, lane, sav, sbv);
   staged_epilogue<OUT, EPI, TM, TN, 8, LDS_BYTES>(acc, sav, sbv, ep, m_base, n_base, M, N, out, ldo, smem, wave, lane);
-  QWIX_DBG_FLUSH()
 }
 
 template <int QT, int OUT, int EPI>
@@ -1274,13 +1229,8 @@ int launch_pp(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M,
               const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   constexpr size_t smem = 5 * 256 * 128;
   auto kern = qgemm_pp_kernel<QT, OUT, EPI>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
   kern<<<dim3(static_cast<unsigned>(tiles)), 512, smem, st>>>(
       static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),
@@ -1312,13 +1262,8 @@ int launch_qgemm(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t
                  const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   constexpr size_t smem = 2 * (BM + BN) * (BK + kPad);
   auto kern = qgemm_kernel<QT, BM, BN, BK>;
-  static bool configured = false;  // idempotent attribute, benign if raced
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   kern<<<dim3(static_cast<unsigned>(tiles)), 256, smem, st>>>(static_cast<const uint8_t*>(a), lda,
                                                               static_cast<const uint8_t*>(b), ldb, static_cast<int>(M),
@@ -1434,13 +1379,8 @@ int launch_ragged_pp(const void* a, int64_t lda, const void* b, int64_t ldb, con
                      int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   constexpr size_t smem = 5 * 256 * 128;
   auto kern = qgemm_ragged_pp_kernel<QT, OUT>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   kern<<<dim3(ragged_grid(M, N, rg.G, 256, 256)), 512, smem, st>>>(
       static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, rg, static_cast<int>(M),
       static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);
@@ -1468,13 +1408,8 @@ int launch_ragged_dma(const void* a, int64_t lda, const void* b, int64_t ldb, co
                       int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   constexpr size_t smem = 2 * (BM + BN) * 128;
   auto kern = qgemm_ragged_dma_kernel<QT, BM, BN, WGM, WGN, OUT>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   kern<<<dim3(ragged_grid(M, N, rg.G, BM, BN)), WGM * WGN * 64, smem, st>>>(
       static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, rg, static_cast<int>(M),
       static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);
@@ -1509,13 +1444,8 @@ int launch_ragged_mid(const void* a, int64_t lda, const void* b, int64_t ldb, co
   constexpr int TM = 2, NW = 4, kDepth = 8;
   constexpr size_t smem = kDepth * 32 * TM * 128;  // 64 KB of activation stages (the epilogue needs 18 KB)
   auto kern = qgemm_ragged_mid_kernel<QT, OUT, TM, kDepth, NW>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   kern<<<dim3(ragged_grid(M, N, rg.G, 32 * TM, 32 * NW)), 64 * NW, smem, st>>>(
       static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, rg, static_cast<int>(M),
       static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);
@@ -1539,13 +1469,8 @@ int launch_ragged(const void* a, int64_t lda, const void* b, int64_t ldb, const 
   constexpr int BM = 128, BN = 128, BK = 128;
   constexpr size_t smem = 2 * (BM + BN) * (BK + kPad);
   auto kern = qgemm_ragged_kernel<QT, BM, BN, BK>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   kern<<<dim3(ragged_grid(M, N, rg.G, BM, BN)), 256, smem, st>>>(
       static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, rg, static_cast<int>(M),
       static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);
@@ -1608,13 +1533,8 @@ int launch_batched_dma(const void* a, int64_t lda, const void* b, int64_t ldb, c
   // half the LDS lets more workgroups share a CU, which is what hides the latency of such short tiles.
   const size_t smem = K == 128 ? (kStage > kStaging ? kStage : kStaging) : 2 * kStage;
   auto kern = qgemm_batched_dma_kernel<QT, BM, BN, 2, 2, OUT>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(2 * kStage));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   kern<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), 256, smem, st>>>(
       static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, bs, static_cast<int>(M),
@@ -1636,13 +1556,8 @@ int launch_batched(const void* a, int64_t lda, const void* b, int64_t ldb, const
   constexpr int BM = 128, BN = 128, BK = 128;
   constexpr size_t smem = 2 * (BM + BN) * (BK + kPad);
   auto kern = qgemm_batched_kernel<QT, BM, BN, BK>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   kern<<<dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(batch)), 256, smem, st>>>(
       static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, bs, static_cast<int>(M),
@@ -1654,12 +1569,6 @@ int launch_batched(const void* a, int64_t lda, const void* b, int64_t ldb, const
 }  // namespace qwix
 
 using namespace qwix;
-
-#ifdef QWIX_GEMM_DEBUG
-extern "C" __attribute__((visibility("default"))) int qwix_dbg_read(unsigned long long* host, size_t n) {
-  return hipMemcpyFromSymbol(host, HIP_SYMBOL(qwix_dbg), n * sizeof(unsigned long long)) == hipSuccess ? 0 : 1;
-}
-#endif
 
 namespace qwix {
 namespace {
@@ -2419,13 +2328,8 @@ static int launch_splitk(const void* a, int64_t lda, const void* b, int64_t ldb,
                          const Epilogue& ep, void* out, int64_t ldo, void* ws, hipStream_t st) {
   constexpr size_t smem = 2 * (128 + 128) * 128;
   auto kern = qgemm_splitk_kernel<QT>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128), slabs = K / 128;
   const int per = static_cast<int>((slabs + splits - 1) / splits);
   const int used = static_cast<int>((slabs + per - 1) / per);  // every range holds at least one slab

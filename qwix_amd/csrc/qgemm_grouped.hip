@@ -262,13 +262,8 @@ int launch_grouped(const GroupedArgs& p, hipStream_t st) {
   constexpr size_t epi = 4 * 32 * (BN / 2 + 4) * sizeof(float);
   constexpr size_t smem = 2 * stage > epi ? 2 * stage : epi;
   auto kern = qgemm_grouped_kernel<BQT, EXACT>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   const int64_t tiles = static_cast<int64_t>((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   kern<<<dim3(static_cast<unsigned>(tiles)), 256, smem, st>>>(p);
   return check_launch("qgemm_grouped");
@@ -282,7 +277,7 @@ int launch_grouped(const GroupedArgs& p, hipStream_t st) {
 // (4 MFMA tiles that share one weight fragment, so the int4 widening is paid once per 4 MFMAs).  The
 // 128-wide K slabs travel global -> LDS directly in 1 KiB pieces, XOR-swizzled per 16-byte chunk so
 // that the fragment reads are bank-conflict free:
-//   A  (int8, 128 B per row):  8 rows per KiB, chunk c of row r sits at position c ^ (r & 7);
+//   A  (int8, 128 B per row):  8 rows per KiB, chunk c of row r sits at position c ^ ((r >> 1) & 7);
 //   B  (int4,  64 B per row): 16 rows per KiB, chunk c of row r sits at position c ^ ((r >> 2) & 3).
 // One 16-byte chunk of packed int4 holds 32 consecutive k; a lane consumes it over two k-steps, and
 // the A fragments of those two k-steps are the two 16-byte chunks with the same 32 k.  The widened
@@ -293,6 +288,12 @@ int launch_grouped(const GroupedArgs& p, hipStream_t st) {
 #define QWIX_GLDS16(gptr, lptr)                                                                       \
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),             \
                                    (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
+
+// Swizzle key of a 128-byte row in LDS: 16-byte chunk c of row r sits at chunk position c ^ swz128(r).  The LDS
+// serves a ds_read_b128 sixteen lanes at a time out of 64 banks (256 bytes): sixteen consecutive rows must land
+// in sixteen different 16-byte bank groups.  Row parity already selects the upper or lower 128 bytes, so the key
+// is taken from the next three bits of the row number.
+__device__ __forceinline__ int swz128(int row) { return (row >> 1) & 7; }
 
 struct Fast {
   static constexpr int kBM = 128, kBN = 256, kBK = 128, kNW = 8, kTM = 4;
@@ -305,9 +306,21 @@ struct Fast {
 // epilogue are the ones of the plain instantiation; only the fold of a finished group differs: the int32
 // partial is taken as a plain integer (int4: shifted back by the factor 16 of the widening), corrected by
 // zu[m,g] * zv[g,n] when an operand is asymmetric, written to acc_out when that is given, then scaled.
-template <int BQT, bool SBF, bool SAG, bool AUX>
-__global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(GroupedArgs p) {
+// MAGIC (groups of exactly 128, bf16 partials, per-token or no activation scale): the first MFMA of a group
+// starts from the integer 0x4B400000 in every accumulator instead of 0.  The group's partial p satisfies
+// |p| < 2^22, so the finished accumulator, read as a float, IS 1.5 * 2^23 + p exactly, and folding the group in
+// is one FMA per accumulator (no integer-to-float conversion).  The constants C * sb[g,n] that this adds are
+// tracked per lane (a lane owns one column) and taken out every fourth group, so the running sums stay within
+// 4 * C * sb and the f32 rounding they pick up is about 2^-12 of a partial: far inside the 2^-9 the reference
+// itself spends on rounding every scaled partial to bf16.
+// ST: slab stages in LDS.  With 3, the loads of slab k+2 are issued at the start of slab k and get two slabs of
+// time to land; the wait before the barrier that ends slab k leaves them in flight (vmcnt counts oldest first).
+// ONE: every group is one slab (group == 128): the main loop then has a single straight-line body.
+template <int BQT, bool SBF, bool SAG, bool AUX, bool MAGIC = false, int ST = 2, bool ONE = false>
+__global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+    qgemm_grouped_dma_kernel(GroupedArgs p) {
   constexpr int BM = Fast::kBM, BN = Fast::kBN, BK = Fast::kBK, NW = Fast::kNW, TM = Fast::kTM;
+  constexpr int WR = 1;  // every wavefront owns all rows of its 32 columns
   constexpr bool W4 = (BQT == QWIX_INT4);
   constexpr int B_ROWB = W4 ? 64 : 128;          // bytes of one B row in a slab
   constexpr int A_BYTES = BM * BK, B_BYTES = BN * B_ROWB, STAGE = A_BYTES + B_BYTES;
@@ -319,6 +332,8 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wc = wave % (NW / WR), wr = wave / (NW / WR);   // column group, row group of this wavefront
+  constexpr int WROWS = BM / WR;                              // rows per wavefront
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   int tile_m, tile_n;
   {  // every XCD gets a contiguous run of tiles; tiles walk down 8 tile-rows before moving along N
@@ -333,7 +348,7 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
   }
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-  float* sa_lds = reinterpret_cast<float*>(smem + 2 * STAGE);  // [group][row of the tile]
+  float* sa_lds = reinterpret_cast<float*>(smem + ST * STAGE);  // [group][row of the tile]
   if constexpr (SAG) {
     const int ng = p.K / p.group;
     for (int idx = tid; idx < ng * BM; idx += NW * 64) {
@@ -350,7 +365,7 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
 #pragma unroll
   for (int j = 0; j < A_LOADS; ++j) {
     const int row = (j * NW + wave) * 8 + (lane >> 3);
-    a_off[j] = static_cast<uint32_t>(min(row, p.M - 1 - m0)) * static_cast<uint32_t>(p.lda) + (((lane & 7) ^ (lane >> 3)) << 4);
+    a_off[j] = static_cast<uint32_t>(min(row, p.M - 1 - m0)) * static_cast<uint32_t>(p.lda) + (((lane & 7) ^ swz128(row)) << 4);
   }
 #pragma unroll
   for (int j = 0; j < B_LOADS; ++j) {
@@ -360,11 +375,11 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
       chunk = (lane & 3) ^ ((lane >> 4) & 3);
     } else {
       row = (j * NW + wave) * 8 + (lane >> 3);
-      chunk = (lane & 7) ^ (lane >> 3);
+      chunk = (lane & 7) ^ swz128(row);
     }
     b_off[j] = static_cast<uint32_t>(min(row, p.N - 1 - n0)) * static_cast<uint32_t>(p.ldb) + (chunk << 4);
   }
-  auto issue_loads = [&](int s, int kt) {
+  auto issue_loads = [&](int s, int kt) __attribute__((always_inline)) {
     const uint8_t* ga = a_base + kt * BK;
     const uint8_t* gb = b_base + kt * B_ROWB;
     uint8_t* ls = smem + s * STAGE;
@@ -376,21 +391,21 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
 
   // ---- fragments
   const int frow = lane & 31, hx = lane >> 5;
-  const int a_row = frow * BK, a_sw = frow & 7;
-  const int b_row = (wave * 32 + frow) * B_ROWB, b_sw = W4 ? ((frow >> 2) & 3) : (frow & 7);
+  const int a_row = (wr * WROWS + frow) * BK, a_sw = swz128(wr * WROWS + frow);
+  const int b_row = (wc * 32 + frow) * B_ROWB, b_sw = W4 ? ((frow >> 2) & 3) : swz128(wc * 32 + frow);
   v4i fa[2][TM];
   v4i fbr[2];  // int4: one chunk = two k-steps; int8: one chunk = one k-step
-  auto read_a = [&](int s, int ks, int buf) {
+  auto read_a = [&](int s, int ks, int buf) __attribute__((always_inline)) {
     const int chunk = W4 ? (4 * (ks >> 1) + 2 * hx + (ks & 1)) : (2 * ks + hx);
     const uint8_t* base = smem + s * STAGE + a_row + ((chunk ^ a_sw) << 4);
 #pragma unroll
     for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const v4i*>(base + i * 32 * BK);
   };
-  auto read_b = [&](int s, int idx, int buf) {  // idx: pair of k-steps (int4) or k-step (int8)
+  auto read_b = [&](int s, int idx, int buf) __attribute__((always_inline)) {  // idx: pair of k-steps (int4) or k-step (int8)
     const int chunk = 2 * idx + hx;
     fbr[buf] = *reinterpret_cast<const v4i*>(smem + s * STAGE + A_BYTES + b_row + ((chunk ^ b_sw) << 4));
   };
-  auto b_frag = [&](int ks) -> v4i {
+  auto b_frag = [&](int ks) __attribute__((always_inline)) -> v4i {
     if constexpr (W4) {
       const v4i raw = fbr[(ks >> 1) & 1];
       v4i f;
@@ -416,11 +431,21 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
       acc[i][r] = 0;
       accf[i][r] = 0.f;
     }
+  constexpr int kMagicBits = 0x4B400000;           // 1.5 * 2^23 as a float
+  constexpr float kMagic = 12582912.0f;
+  v16i magic;
+  if constexpr (MAGIC) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) magic[r] = kMagicBits;
+    // keep the sixteen copies in registers of their own: the MFMA reads its addend from consecutive registers
+    asm volatile("" : "+v"(magic));
+  }
+  float corr = 0.f;  // MAGIC: sum of C * sb over the groups folded in since the constants were last taken out
 
-  // acc[i][r]: m = m0 + i*32 + 8*(r/4) + 4*hx + r%4,  n = n0 + wave*32 + frow: one weight scale per lane and group
-  const int ncl = min(n0 + wave * 32 + frow, p.N - 1);
+  // acc[i][r]: m = m0 + wr*WROWS + i*32 + 8*(r/4) + 4*hx + r%4,  n = n0 + wc*32 + frow: one weight scale per lane and group
+  const int ncl = min(n0 + wc * 32 + frow, p.N - 1);
   constexpr float kUnscale = W4 ? 0.0625f : 1.0f;
-  auto load_sb = [&](int g) -> unsigned {
+  auto load_sb = [&](int g) __attribute__((always_inline)) -> unsigned {
     const int64_t i = static_cast<int64_t>(g) * p.N + ncl;
     if constexpr (SBF) return reinterpret_cast<const uint16_t*>(p.sb)[i];
     return reinterpret_cast<const unsigned*>(p.sb)[i];
@@ -428,18 +453,89 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
 
   const int KT = p.K / BK;
   const int tpg = p.group / BK;
+  // The same load, hidden from the compiler's own wait-count bookkeeping: at the loop's back edge it would
+  // otherwise wait for every outstanding load (vmcnt 0), the slab loads issued two slabs ahead included.  The
+  // result is valid once the explicit wait at the end of the slab has passed (the load is older than the slab
+  // loads of its iteration, and loads complete in order); until then nothing may read or copy `dst`.
+  auto load_sb_async = [&](int g, unsigned& dst) __attribute__((always_inline)) {
+    const int64_t i = static_cast<int64_t>(g) * p.N + ncl;
+    if constexpr (SBF) {
+      const uint16_t* ptr = reinterpret_cast<const uint16_t*>(p.sb) + i;
+      asm volatile("global_load_ushort %0, %1, off" : "=v"(dst) : "v"(ptr) : "memory");
+    } else {
+      const unsigned* ptr = reinterpret_cast<const unsigned*>(p.sb) + i;
+      asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(ptr) : "memory");
+    }
+  };
   unsigned sb_raw = load_sb(0);
   issue_loads(0, 0);
+  if (ST == 3 && KT > 1) issue_loads(1, 1);
   __syncthreads();
   read_a(0, 0, 0);
   read_b(0, 0, 0);
 
-  auto slab = [&](int kt, auto first_tag) {
-    constexpr bool FIRST = decltype(first_tag)::value;
-    const int cur = kt & 1;
-    if (kt + 1 < KT) issue_loads(cur ^ 1, kt + 1);
+  int cs = 0;  // stage that holds the current slab
+  auto next_stage = [&](int s, int by) __attribute__((always_inline)) { return s + by >= ST ? s + by - ST : s + by; };
+  // End of slab kt: every wavefront's loads of slab kt+1 have landed (what was issued during this slab may stay
+  // in flight when there are three stages), all wavefronts are done reading slab kt; then the first fragments
+  // of slab kt+1.
+  auto end_slab = [&](int kt) __attribute__((always_inline)) {
+    if constexpr (ST == 3) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (kt + 2 < KT) __builtin_amdgcn_s_waitcnt(0x0F70 | (A_LOADS + B_LOADS)); else __builtin_amdgcn_s_waitcnt(0x0F70);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    } else {
+      __syncthreads();
+    }
+    cs = next_stage(cs, 1);
+    if (kt + 1 < KT) {
+      read_a(cs, 0, 0);
+      read_b(cs, 0, 0);
+    }
+  };
+
+  // Folding a finished group into the f32 sums, one 32 x 32 tile at a time: acc[i] of group g, weight scale sbg
+  // (with the 1/16 of the int4 widening folded in).
+  auto fold_tile = [&](int i, int g, float sbg, bool recentre) __attribute__((always_inline)) {
+    if constexpr (SAG) {
+      // rows of acc[i][4*qd .. 4*qd+3]: i*32 + 8*qd + 4*hx + 0..3, one 16-byte LDS read (a broadcast per half)
+      const float* sg = sa_lds + g * BM + wr * WROWS + 4 * hx;
 #pragma unroll
-    for (int ks = 0; ks < NK; ++ks) {
+      for (int qd = 0; qd < 4; ++qd) {
+        const float4 sa4 = *reinterpret_cast<const float4*>(sg + i * 32 + 8 * qd);
+        const float sv[4] = {sa4.x, sa4.y, sa4.z, sa4.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          accf[i][4 * qd + j] = __builtin_fmaf(static_cast<float>(acc[i][4 * qd + j]) * sv[j], sbg, accf[i][4 * qd + j]);
+      }
+    } else if constexpr (MAGIC) {
+      if (i == 0) corr = __builtin_fmaf(kMagic, sbg, corr);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) accf[i][r] = __builtin_fmaf(__int_as_float(acc[i][r]), sbg, accf[i][r]);
+      if (recentre) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) accf[i][r] -= corr;
+        if (i == TM - 1) corr = 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) accf[i][r] = __builtin_fmaf(static_cast<float>(acc[i][r]), sbg, accf[i][r]);
+    }
+  };
+
+  // One slab.  FIRST: it opens a group (the accumulators restart from zero, or from the magic constant).
+  // LAST: it closes one.  Then the last two k-steps run tile by tile instead of k-step by k-step, and the fold of
+  // tile i sits behind the MFMAs of tile i+1: its sixteen accumulators are complete by then, and the vector work
+  // runs while the matrix core multiplies the next tile; only the last tile's fold has nothing to hide behind.
+  // (A wavefront issues in order: vector work placed after all MFMAs of a group would run with the matrix
+  // core idle, and the other wavefront of the SIMD is at the same point of its own program.)
+  auto slab = [&](int kt, auto first_tag, auto last_tag, int g, float sbg, bool recentre) __attribute__((always_inline)) {
+    constexpr bool FIRST = decltype(first_tag)::value;
+    constexpr bool LAST = decltype(last_tag)::value && !AUX;
+    const int cur = cs;
+    if (kt + ST - 1 < KT) issue_loads(next_stage(cs, ST - 1), kt + ST - 1);
+    auto read_next = [&](int ks) __attribute__((always_inline)) {  // fragments of k-step ks + 1
       if (ks + 1 < NK) {
         read_a(cur, ks + 1, (ks + 1) & 1);
         if constexpr (W4) {
@@ -448,43 +544,85 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
           read_b(cur, ks + 1, (ks + 1) & 1);
         }
       }
-      const v4i fb = b_frag(ks);
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        if (FIRST && ks == 0) {
+    };
+    auto mfma = [&](int ks, int i, const v4i& fb) __attribute__((always_inline)) {
+      if (FIRST && ks == 0) {
+        if constexpr (MAGIC) {
+          acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks & 1][i], fb, magic, 0, 0, 0);
+        } else {
           const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
           acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks & 1][i], fb, zero, 0, 0, 0);
-        } else {
-          acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks & 1][i], fb, acc[i], 0, 0, 0);
         }
+      } else {
+        acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks & 1][i], fb, acc[i], 0, 0, 0);
       }
+    };
+    constexpr int NKM = LAST ? NK - 2 : NK;  // k-steps that run k-step by k-step
+#pragma unroll
+    for (int ks = 0; ks < NKM; ++ks) {
+      read_next(ks);
+      const v4i fb = b_frag(ks);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) mfma(ks, i, fb);
+    }
+    if constexpr (LAST) {
+      read_next(NK - 2);
+      const v4i fb2 = b_frag(NK - 2), fb3 = b_frag(NK - 1);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        mfma(NK - 2, i, fb2);
+        mfma(NK - 1, i, fb3);
+        if (i > 0) fold_tile(i - 1, g, sbg, recentre);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      fold_tile(TM - 1, g, sbg, recentre);
     }
   };
 
   // The scale of the next group is fetched at the start of a group, together with the slab loads:
   // a load issued just before the barrier would make the barrier's wait for the slab wait for it too.
-  unsigned sb_next = 0;
+  auto to_scale = [&](unsigned raw) __attribute__((always_inline)) {
+    return __uint_as_float(SBF ? raw << 16 : raw) * (AUX ? 1.0f : kUnscale);
+  };
+  unsigned sb_cur = sb_raw, sb_next = 0;
+  using T = std::true_type;
+  using F = std::false_type;
+  if constexpr (ONE && !AUX) {
+    // every slab is a group of its own (always so for the conversion-free fold): one loop body
+    for (int kt = 0; kt < KT; ++kt) {
+      if (kt + 1 < KT) load_sb_async(kt + 1, sb_next);
+      slab(kt, T{}, T{}, kt, to_scale(sb_cur), (kt & 3) == 3 || kt == KT - 1);
+      end_slab(kt);  // its wait covers the scale load above
+      asm volatile("" : "+v"(sb_next));
+      sb_cur = sb_next;
+    }
+  } else
   for (int kt = 0; kt < KT; ++kt) {
     const int in_group = kt % tpg;
-    if (in_group == 0) {
-      if (kt + tpg < KT) sb_next = load_sb(kt / tpg + 1);
-      slab(kt, std::true_type{});
-    } else {
-      slab(kt, std::false_type{});
-    }
-    if (in_group == tpg - 1) {
-      const int g = kt / tpg;
+    const int g = kt / tpg;
+    const float sbg = to_scale(sb_cur);
+    const bool recentre = false;
+    const bool first = in_group == 0, last = in_group == tpg - 1;
+    if (first && kt + tpg < KT) sb_next = load_sb(g + 1);
+    // (groups of several slabs: two loop bodies, the fold after the group's last MFMA)
+    if (first) slab(kt, T{}, F{}, g, sbg, recentre);
+    else slab(kt, F{}, F{}, g, sbg, recentre);
+    if (last) {
+      if constexpr (!AUX) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fold_tile(i, g, sbg, false);
+      }
       if constexpr (AUX) {
-        // acc[i][r]: row i*32 + 8*(r/4) + 4*hx + r%4 of the tile, column ncol
-        const int ncol = n0 + wave * 32 + frow;
+        // Asymmetric operands and parity runs: the partials as plain integers, folded at the end of the group.
+        // acc[i][r]: row i*32 + 8*(r/4) + 4*hx + r%4 of the wavefront's rows, column ncol
+        const int ncol = n0 + wc * 32 + frow;
         const bool zp = p.zu != nullptr;
         const int zvl = zp ? p.zv[ncl * p.zv_sn + g * p.zv_sg] : 0;
-        const float sbz = __uint_as_float(SBF ? sb_raw << 16 : sb_raw);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const int row = i * 32 + 8 * (r >> 2) + 4 * hx + (r & 3);
+            const int row = wr * WROWS + i * 32 + 8 * (r >> 2) + 4 * hx + (r & 3);
             const int m = m0 + row;
             int val = W4 ? (acc[i][r] >> 4) : acc[i][r];  // the widened weights carry a factor 16, exactly
             if (zp) val -= p.zu[min(m, p.M - 1) * p.zu_sm + g * p.zu_sg] * zvl;
@@ -492,44 +630,14 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
               p.acc_out[(static_cast<int64_t>(g) * p.M + m) * p.N + ncol] = val;
             float f = static_cast<float>(val);
             if constexpr (SAG) f *= sa_lds[g * BM + row];
-            accf[i][r] = __builtin_fmaf(f, sbz, accf[i][r]);
+            accf[i][r] = __builtin_fmaf(f, sbg, accf[i][r]);
           }
-        sb_raw = sb_next;
-        __syncthreads();
-        if (kt + 1 < KT) {
-          read_a((kt + 1) & 1, 0, 0);
-          read_b((kt + 1) & 1, 0, 0);
-        }
-        continue;
       }
-      const float sb = __uint_as_float(SBF ? sb_raw << 16 : sb_raw) * kUnscale;
-      if constexpr (SAG) {
-        // rows of acc[i][4*qd .. 4*qd+3]: i*32 + 8*qd + 4*hx + 0..3, one 16-byte LDS read (a broadcast per half)
-        const float* sg = sa_lds + (kt / tpg) * BM + 4 * hx;
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int qd = 0; qd < 4; ++qd) {
-            const float4 sa4 = *reinterpret_cast<const float4*>(sg + i * 32 + 8 * qd);
-            const float sv[4] = {sa4.x, sa4.y, sa4.z, sa4.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-              accf[i][4 * qd + j] = __builtin_fmaf(static_cast<float>(acc[i][4 * qd + j]) * sv[j], sb, accf[i][4 * qd + j]);
-          }
-      } else {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) accf[i][r] = __builtin_fmaf(static_cast<float>(acc[i][r]), sb, accf[i][r]);
-      }
-      sb_raw = sb_next;
+      sb_cur = sb_next;
     }
-    __syncthreads();
-    if (kt + 1 < KT) {
-      read_a((kt + 1) & 1, 0, 0);
-      read_b((kt + 1) & 1, 0, 0);
-    }
+    end_slab(kt);
   }
+  if constexpr (ST == 3) __syncthreads();  // before LDS turns into staging space for the output
 
   // ---- epilogue: 32 rows x 32 columns of f32 per wavefront and pass through LDS
   constexpr int ROW_F = 36;  // floats per staged row (32 + padding)
@@ -542,7 +650,7 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int m = m0 + i * 32 + (lane + 64 * q) / 8;
+      const int m = m0 + wr * WROWS + i * 32 + (lane + 64 * q) / 8;
       sav[i][q] = (!SAG && p.sa != nullptr && m < p.M) ? ld_scale(p.sa, p.sa_dtype, m) : 1.f;
     }
 #pragma unroll
@@ -559,7 +667,7 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
         v[e] *= sav[i][q];
         if (t_bf16) v[e] = round_bf16(v[e]);
       }
-      const int m = m0 + i * 32 + row, n = n0 + wave * 32 + cc * 4;
+      const int m = m0 + wr * WROWS + i * 32 + row, n = n0 + wc * 32 + cc * 4;
       if (m >= p.M || n >= p.N) continue;
       if (p.out_dtype == QWIX_BF16) {
         uint16_t* o = reinterpret_cast<uint16_t*>(p.out) + static_cast<int64_t>(m) * p.ldo + n;
@@ -586,38 +694,50 @@ __global__ void __launch_bounds__(Fast::kNW * 64) qgemm_grouped_dma_kernel(Group
   }
 }
 
-// LDS of the fast kernel: two slab stages, plus the f32 activation scales of the tile when they are per group.
+// LDS of the fast kernel: `st` slab stages, plus the f32 activation scales of the tile when they are per group.
 template <int BQT>
-size_t grouped_dma_lds(bool sag, int64_t K, int64_t group) {
-  const size_t stages = 2 * (Fast::kBM * Fast::kBK + Fast::kBN * (BQT == QWIX_INT4 ? 64 : 128));
+size_t grouped_dma_lds(bool sag, int64_t K, int64_t group, int st) {
+  const size_t stages = st * (Fast::kBM * Fast::kBK + Fast::kBN * (BQT == QWIX_INT4 ? 64 : 128));
   return stages + (sag ? static_cast<size_t>(K / group) * Fast::kBM * sizeof(float) : 0);
 }
+constexpr size_t kLdsMax = 160 * 1024;
 
-template <int BQT, bool SBF, bool SAG, bool AUX>
+template <int BQT, bool SBF, bool SAG, bool AUX, bool MAGIC, int ST, bool ONE>
 int launch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
   constexpr int BM = Fast::kBM, BN = Fast::kBN, NW = Fast::kNW;
-  const size_t smem = grouped_dma_lds<BQT>(SAG, p.K, p.group);
-  static_assert(2 * (Fast::kBM * Fast::kBK + Fast::kBN * 64) >= NW * 32 * 36 * sizeof(float), "epilogue staging must fit");
-  auto kern = qgemm_grouped_dma_kernel<BQT, SBF, SAG, AUX>;
-  static size_t configured = 0;  // largest dynamic LDS size allowed so far
-  if (smem > configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return fail(QWIX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = smem;
-  }
+  const size_t smem = grouped_dma_lds<BQT>(SAG, p.K, p.group, ST);
+  static_assert(ST * (Fast::kBM * Fast::kBK + BN * 64) >= NW * 32 * 36 * sizeof(float), "epilogue staging must fit");
+  auto kern = qgemm_grouped_dma_kernel<BQT, SBF, SAG, AUX, MAGIC, ST, ONE>;
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   const int64_t tiles = static_cast<int64_t>((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   kern<<<dim3(static_cast<unsigned>(tiles)), NW * 64, smem, st>>>(p);
   return check_launch("qgemm_grouped (dma)");
 }
 
+// Picks the instantiation.  Returns -1 when the tile's per-group activation scales do not fit in LDS (the caller
+// then takes the register-staged kernel).
 template <int BQT, bool SAG>
-int launch_grouped_dma_sb(const GroupedArgs& p, hipStream_t st) {
-  if (p.zu != nullptr || p.acc_out != nullptr)
-    return p.sb_dtype == QWIX_BF16 ? launch_grouped_dma<BQT, true, SAG, true>(p, st)
-                                   : launch_grouped_dma<BQT, false, SAG, true>(p, st);
-  return p.sb_dtype == QWIX_BF16 ? launch_grouped_dma<BQT, true, SAG, false>(p, st)
-                                 : launch_grouped_dma<BQT, false, SAG, false>(p, st);
+int dispatch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
+  const bool sbf = p.sb_dtype == QWIX_BF16;
+  const bool three = grouped_dma_lds<BQT>(SAG, p.K, p.group, 3) <= kLdsMax;  // room for a third slab stage
+  if (!three && grouped_dma_lds<BQT>(SAG, p.K, p.group, 2) > kLdsMax) return -1;
+  if (p.zu != nullptr || p.acc_out != nullptr)  // asymmetric operands, parity runs
+    return sbf ? launch_grouped_dma<BQT, true, SAG, true, false, 2, false>(p, st)
+               : launch_grouped_dma<BQT, false, SAG, true, false, 2, false>(p, st);
+  if (p.group == Fast::kBK) {  // one slab per group
+    if constexpr (!SAG) {
+      // scaled partials that the reference keeps in bf16: the conversion-free fold
+      if (sbf && p.t_dtype == QWIX_BF16) return launch_grouped_dma<BQT, true, false, false, true, 3, true>(p, st);
+    }
+    if (three)
+      return sbf ? launch_grouped_dma<BQT, true, SAG, false, false, 3, true>(p, st)
+                 : launch_grouped_dma<BQT, false, SAG, false, false, 3, true>(p, st);
+    return sbf ? launch_grouped_dma<BQT, true, SAG, false, false, 2, true>(p, st)
+               : launch_grouped_dma<BQT, false, SAG, false, false, 2, true>(p, st);
+  }
+  return sbf ? launch_grouped_dma<BQT, true, SAG, false, false, 2, false>(p, st)
+             : launch_grouped_dma<BQT, false, SAG, false, false, 2, false>(p, st);
 }
 
 // Per-group K-sums of quantized rows: out[row, g] = sum over the g-th group of `group` values of row `row`
@@ -736,14 +856,12 @@ static int grouped_impl(const void* a, int64_t lda, const void* b, int64_t ldb_b
   if (!exact && row_strides_fit) {
     // per-group activation scales ride along in LDS: the tile's scales must fit behind the slab stages
     const bool sag = sa != nullptr && ga > 1;
-    constexpr size_t kLdsMax = 160 * 1024;
-    if (b_qtype == QWIX_INT4) {
-      if (!sag) return launch_grouped_dma_sb<QWIX_INT4, false>(p, st);
-      if (grouped_dma_lds<QWIX_INT4>(true, K, group) <= kLdsMax) return launch_grouped_dma_sb<QWIX_INT4, true>(p, st);
-    } else {
-      if (!sag) return launch_grouped_dma_sb<QWIX_INT8, false>(p, st);
-      if (grouped_dma_lds<QWIX_INT8>(true, K, group) <= kLdsMax) return launch_grouped_dma_sb<QWIX_INT8, true>(p, st);
-    }
+    int rc;
+    if (b_qtype == QWIX_INT4)
+      rc = sag ? dispatch_grouped_dma<QWIX_INT4, true>(p, st) : dispatch_grouped_dma<QWIX_INT4, false>(p, st);
+    else
+      rc = sag ? dispatch_grouped_dma<QWIX_INT8, true>(p, st) : dispatch_grouped_dma<QWIX_INT8, false>(p, st);
+    if (rc >= 0) return rc;
   }
   if (b_qtype == QWIX_INT4)
     return exact ? launch_grouped<QWIX_INT4, true>(p, st) : launch_grouped<QWIX_INT4, false>(p, st);
