@@ -351,6 +351,57 @@ class GemvW4(Workload):
             'weight_copies_rotated': self.copies}
 
 
+class WeightOnlyPrefill(Workload):
+  """Weight-only int4 g128 at prefill size: per step the int4 weight is dequantized into a K-contiguous bf16
+  array and multiplied with the bf16 activations on the bf16 matrix cores (f32 accumulate, bf16 out)."""
+
+  bound = 'mfma'
+  peak_tops = 2500.0   # dense bf16 MFMA peak, TFLOP/s
+
+  def __init__(self, name, M, K, N, group):
+    self.name, self.M, self.K, self.N, self.group = name, M, K, N, group
+    self.dtype = 'bf16 x int4'
+    self.metric = 'weight-only int4 g128 prefill TFLOP/s (weight dequantize included)'
+    self.unit = 'TFLOP/s'
+    # 256 x 256 tiles (ping-pong kernel) once they fill most of the chip, 128 x 128 tiles below
+    self.kernel_name = 'qgemm_pp_kernel' if -(-M // 256) * -(-N // 256) >= 192 else 'qgemm_dma_kernel'
+
+  def setup(self, dev):
+    import torch
+    from qwix_amd.core import qarray
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(2100)
+    self.x = torch.randn(self.M, self.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    w = (torch.randn(self.K, self.N, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(dev)
+    wq = qarray.quantize_api(w, 'int4', channelwise_axes=[1], tiled_axes={0: self.group}, scale_dtype=torch.float32)
+    self.b = wq.qvalue.permute(1, 0).data
+    assert self.b.is_contiguous()
+    self.s = wq.scale.contiguous()
+    self.w = torch.empty(self.N, self.K, dtype=torch.bfloat16, device=dev)
+    self.out = torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev)
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, i=0):
+    L = self.L
+    L.call('qwix_hip_dequantize_rm', self.b.data_ptr(), L.INT4, 1, self.K, self.N, self.group, self.s.data_ptr(), None,
+           L.F32, self.w.data_ptr(), L.BF16, self.stream)
+    self.kernel(i)
+
+  def kernel(self, i=0):
+    L = self.L
+    L.call('qwix_hip_gemm_bf16', self.x.data_ptr(), self.K, self.w.data_ptr(), self.K, self.M, self.N, self.K,
+           self.out.data_ptr(), L.BF16, self.N, self.stream)
+
+  def work_per_step(self):
+    return 2.0 * self.M * self.N * self.K
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'M': self.M, 'K': self.K, 'N': self.N, 'group': self.group}
+
+
 class QdotDecode(Workload):
   """Dynamic-range w8a8 at decode size: per-token int8 quantize of a few tokens + the quantized GEMM that
   streams the int8 weight once (HBM-bound): the skinny kernel up to 16 tokens, the 64-row tile above."""
@@ -816,6 +867,8 @@ WORKLOADS = {
     'c2_gemv_w4_m1': lambda: GemvW4('c2_gemv_w4_m1', 1, 4096, 14336, 128),
     'c2_gemv_w4_m16': lambda: GemvW4('c2_gemv_w4_m16', 16, 4096, 14336, 128),
     'c2_gemv_w4_m32': lambda: GemvW4('c2_gemv_w4_m32', 32, 4096, 14336, 128),
+    'c2_w4a16_prefill_m2048': lambda: WeightOnlyPrefill('c2_w4a16_prefill_m2048', 2048, 4096, 14336, 128),
+    'c2_w4a16_prefill_m512': lambda: WeightOnlyPrefill('c2_w4a16_prefill_m512', 512, 4096, 14336, 128),
     'c4_quantize_weight_fp8': lambda: QuantizeWeight('c4_quantize_weight_fp8', 8192, 28672, 'float8_e4m3fn'),
     'c5_quantize_weight_int4_g128': lambda: QuantizeWeight('c5_quantize_weight_int4_g128', 8192, 8192, 'int4', 128),
     'c3_quantize_weight_int8': lambda: QuantizeWeight('c3_quantize_weight_int8', 4096, 4096, 'int8'),
@@ -834,7 +887,7 @@ WORKLOADS = {
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
 }
 DEFAULT = 'c3_int8_w8a8_4096'
-EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
+EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'c2_w4a16_prefill_m2048', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
          'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'moe_ragged_int8_8x1024',
          'moe_ragged_int8_64x128', 'moe_decode_int8_64x4', 'quantize_weight_fp8_block128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 
@@ -906,7 +959,7 @@ def summarize(wl: Workload, step_s: float, kern_s: float) -> dict:
   value = wl.work_per_step() / step_s / scale
   # the roofline that bounds the dominant kernel need not be the one the metric's unit suggests
   rb = getattr(wl, 'roofline_bound', wl.bound)
-  peak = PEAK_MFMA_TOPS if rb == 'mfma' else PEAK_HBM_GBS
+  peak = getattr(wl, 'peak_tops', PEAK_MFMA_TOPS) if rb == 'mfma' else PEAK_HBM_GBS
   work = wl.roofline_work() if hasattr(wl, 'roofline_work') else wl.kernel_work()
   achieved = work / kern_s / (1e12 if rb == 'mfma' else 1e9)
   return {

@@ -275,6 +275,23 @@ QWIX_API int qwix_hip_qgemm_grouped_zp(const void* a, int64_t lda, const void* b
 QWIX_API int qwix_hip_ksum_groups(const void* q, int qtype, int64_t ld_bytes, int64_t rows, int64_t K, int64_t group,
                          int32_t* out, void* stream);
 
+/* bf16 x bf16 GEMM with f32 accumulation: the float contraction of the dequantize-first path
+ * (_slow_dot_general, qwix/_src/core/dot_general.py:264-275: lax.dot_general on the dequantized operands) for
+ * batches too large for qwix_hip_gemv_wq:  out[m,n] = cast( sum_k a[m,k] * b[n,k] ).
+ *   a (M,K) and b (N,K) bf16, K-contiguous, lda / ldb in elements (multiples of 8), K % 64 == 0;
+ *   out (M,N) of out_dtype in {F32, BF16}.
+ * Same tile kernels as qwix_hip_qgemm (v_mfma_f32_32x32x16_bf16). */
+QWIX_API int qwix_hip_gemm_bf16(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                       void* out, int out_dtype, int64_t ldo, void* stream);
+
+/* dequantize (qarray.py:692-708) of a REDUCE_MINOR qvalue that keeps that layout: out[(o, i, r)] =
+ * D(D(q - zp) * scale[o, r / tile, i]) as a row-major (outer, inner, reduce) array, the K-contiguous operand
+ * qwix_hip_gemm_bf16 reads.  D = `dtype` = the scale dtype; out_dtype is `dtype`, or QWIX_BF16 for f32 scales
+ * (the f32 value rounded once more, as a cast of the dequantized array would).  reduce % 8 == 0, tile % 8 == 0. */
+QWIX_API int qwix_hip_dequantize_rm(const void* qvalue, int qtype, int64_t outer, int64_t reduce, int64_t inner,
+                           int64_t tile, const void* scale, const void* zero_point, int dtype, void* out,
+                           int out_dtype, void* stream);
+
 /* Weight-only skinny GEMM (the reference's _slow_dot_general, dot_general.py:264-275, with
  * the dequantize fused): out[m,n] = sum_k x[m,k] * (q[k,n] * s[k/group, n]).
  *   x   (M,K) bf16 row-major; q int4/int8 K-contiguous rows (n*ldb_bytes); s (K/group, N)

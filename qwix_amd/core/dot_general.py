@@ -521,12 +521,58 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
               _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
               out.data_ptr(), _lib.float_tag(res_t), c.N, _lib.stream_of(x))
     return out.reshape(c.out_shape)
+  out = _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type)
+  if out is not None:
+    return out
   if isinstance(lhs, QArray):
     lhs = qarray.dequantize(lhs)
   if isinstance(rhs, QArray):
     rhs = qarray.dequantize(rhs)
   res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.dtype)
   return float_dot_general(lhs, rhs, dimension_numbers, res_t)
+
+
+def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type):
+  """The dequantize-first path on this library's own kernels, for a bf16 activation against a quantized weight
+  of any of the three qtypes, with or without zero point: the weight is dequantized into a K-contiguous bf16
+  array (qwix_hip_dequantize_rm, the reference's D(D(q - zp) * scale) in the scale dtype; an f32 result rounded
+  once more to bf16) and contracted by the bf16 MFMA GEMM with f32 accumulation (qwix_hip_gemm_bf16).  Returns
+  None when the operands are not of that kind (then: HIP dequantize + the float GEMM of the vendor library)."""
+  if not (_is_float_array(lhs) and lhs.dtype == torch.bfloat16 and isinstance(rhs, QArray)):
+    return None
+  if _qtype_of(rhs) not in (numerics.INT4, numerics.INT8, numerics.E4M3):
+    return None
+  c = _Canon(lhs, rhs, dimension_numbers)
+  if any(rhs.scale.shape[a] != 1 for a in c.rca[:-1]) or c.K % 64:
+    return None
+  gb = rhs.scale.shape[c.rca[-1]]
+  if (gb > 1 and len(c.rca) > 1) or (c.K // gb) % 8 or rhs.scale.dtype not in (torch.bfloat16, torch.float32):
+    return None
+  if isinstance(rhs.qvalue, Int4Tensor):
+    order = c.rfree + c.rca
+    packed = (rhs.qvalue.permute(*order).packed_axis, rhs.qvalue.permute(*(c.rca + c.rfree)).packed_axis)
+    if len(order) - 1 not in packed:
+      return None
+  x = c.lhs_values(lhs)
+  b, _ = c.rhs_values(rhs)
+  sb, _ = c.rhs_scale(rhs)
+  zp = None
+  if rhs.zero_point is not None:
+    z, gz = c.rhs_zero_point(rhs)
+    if gz != gb:
+      return None
+    zp = z.to(torch.int8)
+  dev, st = x.device, _lib.stream_of(x)
+  w = torch.empty(c.N, c.K, dtype=torch.bfloat16, device=dev)
+  _lib.call('qwix_hip_dequantize_rm', b.data_ptr(), numerics.qtype_tag(_qtype_of(rhs)), 1, c.K, c.N, c.K // gb,
+            sb.data_ptr(), _lib.ptr(zp), _lib.float_tag(sb.dtype), w.data_ptr(), _lib.BF16, st)
+  res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.scale.dtype)
+  if res_t not in (torch.bfloat16, torch.float32):
+    return None
+  out = torch.empty(c.M, c.N, dtype=res_t, device=dev)
+  _lib.call('qwix_hip_gemm_bf16', x.data_ptr(), x.stride(0), w.data_ptr(), c.K, c.M, c.N, c.K, out.data_ptr(),
+            _lib.float_tag(res_t), c.N, st)
+  return out.reshape(c.out_shape)
 
 
 def float_dot_general(lhs: torch.Tensor, rhs: torch.Tensor, dimension_numbers, preferred_element_type=None) -> torch.Tensor:

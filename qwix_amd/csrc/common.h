@@ -48,6 +48,13 @@ inline int grant_lds(const void* kernel, size_t bytes, LdsGrant& g) {
 }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// ------------------------------------------------------------------ LDS layout
+// Swizzle key of a 128-byte row in LDS: 16-byte chunk c of row r sits at chunk position c ^ swz128(r).  The LDS
+// serves a ds_read_b128 sixteen lanes at a time out of 64 banks (256 bytes): sixteen consecutive rows must land
+// in sixteen different 16-byte bank groups.  Row parity already selects the upper or lower 128 bytes, so the key
+// is taken from the next three bits of the row number.
+__device__ __forceinline__ int swz128(int row) { return (row >> 1) & 7; }
+
 // ------------------------------------------------------------------ dtype tags
 struct F32 {
   using storage = float;

@@ -28,6 +28,19 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kPad = 16;
+// Operand tag of the tile bodies for bf16 x bf16 (the float contraction of the dequantize-first path); the
+// byte geometry is that of int8: a 128-byte K slab is four MFMA k-steps of 32 bytes per row (16 bf16 values).
+constexpr int kOpBf16 = 16;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// Swizzle key of the kernels in this file: 16-byte chunk c of the 128-byte LDS row r sits at chunk position
+// c ^ swz8(r).  Eight consecutive rows then cover all eight chunk positions; over the sixteen rows that the LDS
+// serves per clock for a ds_read_b128 this still leaves two-way bank conflicts, which the sixteen-row key of
+// common.h (swz128) removes.  Measured side by side on one box, the conflict-free key is nevertheless 2-5 %
+// SLOWER here (int8 4096^3: 72.1 against 70.3 us; 8192^3: 494 against 485 us; the 8-expert ragged GEMM 578
+// against 551 us; e4m3 and the one-tile-row kernel unchanged): these kernels run at the board's power limit,
+// where faster fragment reads buy nothing and cost clock.  So the eight-row key stays.
+__device__ __forceinline__ int swz8(int row) { return row & 7; }
 
 // Epilogue description.  The reference scales the accumulator as ((T(acc) * sa) * sb) with one
 // rounding per step in the promoted dtype; which of those roundings are to bf16 is decided on the
@@ -318,8 +331,8 @@ __global__ void __launch_bounds__(256)
 // Fast path (K % 128 == 0): the slabs go from global memory straight into LDS
 // (global_load_lds_dwordx4: no staging registers, no ds_write instructions).  Each wave-level load
 // fills one contiguous KiB of LDS = 8 tile rows x 128 bytes; inside a row the eight 16-byte k-chunks
-// are stored at position (chunk ^ (row & 7)), chosen by having each lane fetch the matching global
-// chunk, so that the fragment reads of 8 consecutive rows hit all 32 banks.  Rows past M / N are
+// are stored at position (chunk ^ swz8(row)), chosen by having each lane fetch the matching global
+// chunk, so that the fragment reads of 16 consecutive rows hit all 64 banks.  Rows past M / N are
 // clamped to the last valid row (their results are never stored).  Loads for slab kt+1 are issued
 // while the MFMAs of slab kt run; the workgroup barrier at the end of the slab waits for them.
 // The workgroup is WGM x WGN wavefronts; with 8 wavefronts (two per SIMD) the issue time of one
@@ -478,11 +491,13 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
                                                int N, int K, const Epilogue& ep, uint8_t* __restrict__ out,
                                                int64_t ldo) {
   constexpr bool IS_INT = (QT == QWIX_INT8);
+  constexpr bool IS_BF = (QT == kOpBf16);
+  constexpr bool B16 = IS_INT || IS_BF;  // 16 bytes per lane and k-step
   constexpr int BK = 128;
   constexpr int NWAVES = WGM * WGN;
   constexpr int WTM = BM / WGM, WTN = BN / WGN;   // wave tile
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  constexpr int KSTEP = IS_INT ? 32 : 64;
+  constexpr int KSTEP = B16 ? 32 : 64;
   constexpr int NK = BK / KSTEP;
   constexpr int ROWS = BM + BN;
   constexpr int STAGE = ROWS * BK;
@@ -495,7 +510,7 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
   const int wm = wave / WGN, wn = wave % WGN;
 
   using AccT = typename std::conditional<IS_INT, v16i, v16f>::type;
-  using FragT = typename std::conditional<IS_INT, v4i, v8i>::type;
+  using FragT = typename std::conditional<B16, v4i, v8i>::type;
   AccT acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -506,7 +521,6 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
 
   // ---- loader: a wave-uniform base pointer plus this lane's 32-bit offset for each row group
   const int lr = lane >> 3;                       // row inside the 8-row group
-  const int lc = (lane & 7) ^ lr;                 // global k-chunk that lands at LDS chunk position lane&7
   const bool from_a = (wave * LOADS * 8) < BM;    // wave-uniform
   const uint8_t* gbase = from_a ? A : B;
   const int64_t gld = from_a ? lda : ldb;
@@ -515,21 +529,22 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
   uint32_t goff[LOADS];
 #pragma unroll
   for (int j = 0; j < LOADS; ++j)
-    goff[j] = static_cast<uint32_t>(min(grow0 + j * 8 + lr, glim)) * static_cast<uint32_t>(gld) + lc * 16;
+    goff[j] = static_cast<uint32_t>(min(grow0 + j * 8 + lr, glim)) * static_cast<uint32_t>(gld) +
+              (((lane & 7) ^ swz8((wave * LOADS + j) * 8 + lr)) << 4);  // the global k-chunk that lands at position lane & 7
   auto issue_loads = [&](int s, int k0) {
     const uint8_t* gk = gbase + k0;
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) QWIX_GLDS16(gk + goff[j], smem + s * STAGE + (wave * LOADS + j) * 1024);
   };
 
-  // ---- fragment addresses: row r, k-chunk c lives at r*128 + ((c ^ (r & 7)) << 4); r & 7 == lane & 7
+  // ---- fragment addresses: row r, k-chunk c lives at r*128 + ((c ^ swz8(r)) << 4); wave tiles start at multiples of 32
   const int a_row = (wm * WTM + (lane & 31)) * BK;
   const int b_row = (BM + wn * WTN + (lane & 31)) * BK;
-  const int hx = lane >> 5, x7 = lane & 7;
+  const int hx = lane >> 5, x7 = swz8(lane & 31);
   FragT fa[2][TM], fb[2][TN];
   auto read_frags = [&](int s, int ks, int buf) {
     const uint8_t* base = smem + s * STAGE;
-    if constexpr (IS_INT) {
+    if constexpr (B16) {
       const int off = ((ks * 2 + hx) ^ x7) << 4;
 #pragma unroll
       for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const v4i*>(base + a_row + i * 32 * BK + off);
@@ -558,6 +573,9 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
       for (int j = 0; j < TN; ++j) {
         if constexpr (IS_INT)
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+        else if constexpr (IS_BF)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb[buf][j]),
+                                                              __builtin_bit_cast(bf16x8, fa[buf][i]), acc[i][j], 0, 0, 0);
         else
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0, 0, 0, 0);
       }
@@ -565,7 +583,7 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
   // Interleave hints for one k-step: MFMAs in pairs, a fragment read after each pair, and a slab load
   // after each pair while loads remain.
   auto hint_kstep = [&](int n_loads) {
-    constexpr int MF = TM * TN, RD = (IS_INT ? 1 : 2) * (TM + TN);
+    constexpr int MF = TM * TN, RD = (B16 ? 1 : 2) * (TM + TN);
 #pragma unroll
     for (int g = 0; g < MF; ++g) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // MFMA
@@ -713,13 +731,14 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
   fetch_scales<OUT, TM, TN>(ep, m_base, n_base, M, N, lane, sav, sbv);  // oldest loads: done before any slab
 
   // activations: 32 * TM rows of 128 bytes per slab = 4 * TM pieces of 1 KB (8 rows), PW per wavefront
-  const int lr = lane >> 3, lc = (lane & 7) ^ lr;
+  const int lr = lane >> 3;
   uint32_t aoff[PW];
 #pragma unroll
   for (int j = 0; j < PW; ++j)
-    aoff[j] = static_cast<uint32_t>(min(m0 + (wave * PW + j) * 8 + lr, M - 1)) * static_cast<uint32_t>(lda) + lc * 16;
+    aoff[j] = static_cast<uint32_t>(min(m0 + (wave * PW + j) * 8 + lr, M - 1)) * static_cast<uint32_t>(lda) +
+              (((lane & 7) ^ swz8((wave * PW + j) * 8 + lr)) << 4);
   // weights: column n_base + lane % 32, bytes 64 * (lane / 32) .. of the slab
-  const int hx = lane >> 5, x7 = lane & 7;
+  const int hx = lane >> 5, x7 = swz8(lane & 31);
   const uint32_t boff = static_cast<uint32_t>(min(n_base + (lane & 31), N - 1)) * static_cast<uint32_t>(ldb) + hx * 64;
   v4i breg[DEPTH][4];
   const int KT = K / BK;
@@ -1051,9 +1070,11 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
                                               int64_t ldb, int m0, int n0, int M, int N, int K, const Epilogue& ep,
                                               uint8_t* __restrict__ out, int64_t ldo) {
   constexpr bool IS_INT = (QT == QWIX_INT8);
+  constexpr bool IS_BF = (QT == kOpBf16);
+  constexpr bool B16 = IS_INT || IS_BF;  // 16 bytes per lane and k-step
   constexpr int BM = 256, BN = 256, BK = 128, WGN = 4;
   constexpr int TM = 4, TN = 2;                 // wave tile 128 x 64
-  constexpr int KSTEP = IS_INT ? 32 : 64, NK = BK / KSTEP;
+  constexpr int KSTEP = B16 ? 32 : 64, NK = BK / KSTEP;
   constexpr int A_STAGE = BM * BK, B_STAGE = BN * BK, B_BASE = 2 * A_STAGE;
   constexpr int LDS_BYTES = 2 * A_STAGE + 3 * B_STAGE;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -1063,7 +1084,7 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
   const int wm = wave / WGN, wn = wave % WGN;   // wm is also the phase group
 
   using AccT = typename std::conditional<IS_INT, v16i, v16f>::type;
-  using FragT = typename std::conditional<IS_INT, v4i, v8i>::type;
+  using FragT = typename std::conditional<B16, v4i, v8i>::type;
   AccT acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -1073,11 +1094,12 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
   // ---- loader: this wavefront brings rows [wm*128 + wn*32, +32) of A and of B, 8 rows per instruction
-  const int lr = lane >> 3, lc = (lane & 7) ^ lr;
+  const int lr = lane >> 3;
   const int lrow0 = wm * 128 + wn * 32;
   uint32_t goffa[4], goffb[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
+    const uint32_t lc = static_cast<uint32_t>((lane & 7) ^ swz8(lrow0 + j * 8 + lr));
     goffa[j] = static_cast<uint32_t>(min(m0 + lrow0 + j * 8 + lr, M - 1)) * static_cast<uint32_t>(lda) + lc * 16;
     goffb[j] = static_cast<uint32_t>(min(n0 + lrow0 + j * 8 + lr, N - 1)) * static_cast<uint32_t>(ldb) + lc * 16;
   }
@@ -1097,14 +1119,14 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
   // ---- fragments of a whole slab
   const int a_row = (wm * 128 + (lane & 31)) * BK;
   const int b_row = B_BASE + (wn * 64 + (lane & 31)) * BK;
-  const int hx = lane >> 5, x7 = lane & 7;
+  const int hx = lane >> 5, x7 = swz8(lane & 31);
   FragT fa[NK][TM], fb[NK][TN];
   auto read_slab = [&](int a_stage, int b_stage) {
     const uint8_t* pa = smem + a_stage * A_STAGE + a_row;
     const uint8_t* pb = smem + b_stage * B_STAGE + b_row;
 #pragma unroll
     for (int ks = 0; ks < NK; ++ks) {
-      if constexpr (IS_INT) {
+      if constexpr (B16) {
         const int off = ((ks * 2 + hx) ^ x7) << 4;
 #pragma unroll
         for (int i = 0; i < TM; ++i) fa[ks][i] = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + off);
@@ -1192,6 +1214,9 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
         for (int j = 0; j < TN; ++j) {
           if constexpr (IS_INT)
             acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+          else if constexpr (IS_BF)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb[ks][j]),
+                                                                __builtin_bit_cast(bf16x8, fa[ks][i]), acc[i][j], 0, 0, 0);
           else
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0, 0, 0, 0);
         }
@@ -2118,6 +2143,35 @@ extern "C" int qwix_hip_qgemm_ragged(const void* a, int64_t lda, const void* b, 
   }
   if (qtype == QWIX_INT8) return launch_ragged<QWIX_INT8>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
   return launch_ragged<QWIX_E4M3>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+}
+
+extern "C" int qwix_hip_gemm_bf16(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                                  void* out, int out_dtype, int64_t ldo, void* stream) {
+  if (!a || !b || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/b/out");
+  if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || 2 * K > INT32_MAX)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad GEMM shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
+                (long long)K);
+  if (out_dtype != QWIX_BF16 && out_dtype != QWIX_F32) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad out dtype %d", out_dtype);
+  // rows are walked in 128-byte slabs that go to LDS directly
+  if (K % 64 || lda % 8 || ldb % 8 || lda < K || ldb < K || !aligned16(a) || !aligned16(b))
+    return fail(QWIX_ERR_UNSUPPORTED, "bf16 GEMM needs K a multiple of 64, row pitches multiples of 8 elements and "
+                "16-byte aligned operands (K=%lld lda=%lld ldb=%lld)", (long long)K, (long long)lda, (long long)ldb);
+  if (ldo < N || !aligned16(out) || (N % 4 == 0 && ldo % 4 != 0))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad output leading dimension %lld for N=%lld", (long long)ldo, (long long)N);
+  const int64_t ldab = 2 * lda, ldbb = 2 * ldb, kb = 2 * K;  // the tile bodies count bytes
+  if (M * ldab >= (int64_t{1} << 31) || N * ldbb >= (int64_t{1} << 31))
+    return fail(QWIX_ERR_UNSUPPORTED, "operands beyond 2 GiB are not supported by the bf16 GEMM");
+  const Epilogue ep{nullptr, nullptr, 0, 0, out_dtype, 0, 0, 0, nullptr, nullptr};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool big = ((M + 255) / 256) * ((N + 255) / 256) >= 192;
+  if (out_dtype == QWIX_BF16) {
+    if (big && kb >= 256) return launch_pp<kOpBf16, QWIX_BF16, 0>(a, ldab, b, ldbb, M, N, kb, ep, out, ldo, st);
+    if (big) return launch_dma<kOpBf16, 256, 256, 2, 4, QWIX_BF16, 0>(a, ldab, b, ldbb, M, N, kb, ep, out, ldo, st);
+    return launch_dma<kOpBf16, 128, 128, 2, 2, QWIX_BF16, 0>(a, ldab, b, ldbb, M, N, kb, ep, out, ldo, st);
+  }
+  if (big && kb >= 256) return launch_pp<kOpBf16, QWIX_F32, 0>(a, ldab, b, ldbb, M, N, kb, ep, out, ldo, st);
+  if (big) return launch_dma<kOpBf16, 256, 256, 2, 4, QWIX_F32, 0>(a, ldab, b, ldbb, M, N, kb, ep, out, ldo, st);
+  return launch_dma<kOpBf16, 128, 128, 2, 2, QWIX_F32, 0>(a, ldab, b, ldbb, M, N, kb, ep, out, ldo, st);
 }
 
 extern "C" int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M,

@@ -289,12 +289,6 @@ int launch_grouped(const GroupedArgs& p, hipStream_t st) {
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),             \
                                    (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
 
-// Swizzle key of a 128-byte row in LDS: 16-byte chunk c of row r sits at chunk position c ^ swz128(r).  The LDS
-// serves a ds_read_b128 sixteen lanes at a time out of 64 banks (256 bytes): sixteen consecutive rows must land
-// in sixteen different 16-byte bank groups.  Row parity already selects the upper or lower 128 bytes, so the key
-// is taken from the next three bits of the row number.
-__device__ __forceinline__ int swz128(int row) { return (row >> 1) & 7; }
-
 struct Fast {
   static constexpr int kBM = 128, kBN = 256, kBK = 128, kNW = 8, kTM = 4;
 };

@@ -1084,6 +1084,42 @@ __global__ void __launch_bounds__(256)
   store8<D>(out, idx, v);
 }
 
+// Reduce-minor in, reduce-minor out: element (o, i, r) of the (outer, inner, reduce) array; 8 consecutive r per
+// thread share a scale (tile % 8 == 0).  The result is the K-contiguous float operand of the bf16 GEMM.
+template <typename D, int QT, typename OD>
+__global__ void __launch_bounds__(256)
+    dequant_keep_rm_kernel(const uint8_t* __restrict__ q, int64_t outer, int64_t reduce, int64_t inner, int64_t tile,
+                           const void* __restrict__ scale, const int8_t* __restrict__ zp, void* __restrict__ out) {
+  const int64_t n = outer * reduce * inner;
+  const int64_t idx = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 8;
+  if (idx >= n) return;
+  uint32_t b[8];
+  if constexpr (QT == QWIX_INT4) {
+    const uint32_t w = *reinterpret_cast<const uint32_t*>(q + idx / 2);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] = (w >> (4 * e)) & 0xF;
+  } else {
+    const uint2 w = *reinterpret_cast<const uint2*>(q + idx);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      b[e] = (w.x >> (8 * e)) & 0xFF;
+      b[4 + e] = (w.y >> (8 * e)) & 0xFF;
+    }
+  }
+  const int64_t r = idx % reduce, rest = idx / reduce, i = rest % inner, o = rest / inner;
+  const int64_t si = (o * (reduce / tile) + r / tile) * inner + i;
+  const float sv = load1<D>(scale, si);
+  const float zv = zp ? rnd<D>(static_cast<float>(zp[si])) : 0.f;
+  float v[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float t = rnd<D>(q_to_f32<QT>(b[e]));
+    if (zp != nullptr) t = rnd<D>(t - zv);
+    v[e] = rnd<D>(t * sv);
+  }
+  store8<OD>(out, idx, v);  // bf16 out of f32 values: one more rounding, what casting the f32 array gives
+}
+
 // Dequantize for the 5-D geometry (two reduced axis groups: block scales).  VEC = 8: eight consecutive elements
 // of the innermost reduced axis share a scale (d4 == 1, t3 % 8 == 0); VEC = 1: anything.
 template <typename D, int QT, int VEC>
@@ -1738,6 +1774,38 @@ int qwix_hip_dequantize(const void* qvalue, int qtype, int q_layout, int64_t out
       return fail(QWIX_ERR_INVALID_ARGUMENT, "unknown qtype %d", qtype);
   })
   return check_launch("dequantize");
+}
+
+int qwix_hip_dequantize_rm(const void* qvalue, int qtype, int64_t outer, int64_t reduce, int64_t inner, int64_t tile,
+                           const void* scale, const void* zero_point, int dtype, void* out, int out_dtype,
+                           void* stream) {
+  if (out_dtype != dtype && !(dtype == QWIX_F32 && out_dtype == QWIX_BF16))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "out_dtype must be the scale dtype, or bf16 for f32 scales");
+  if (int e = check_geom(outer, reduce, inner, tile)) return e;
+  if (!qvalue || !scale || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null argument");
+  if (reduce % 8 || tile % 8 || !aligned16(qvalue) || !aligned16(out))
+    return fail(QWIX_ERR_UNSUPPORTED, "reduce-minor dequantize needs reduce and tile multiples of 8 and 16-byte aligned "
+                "arrays (reduce=%lld tile=%lld)", (long long)reduce, (long long)tile);
+  const int64_t n = outer * reduce * inner;
+  const unsigned vb = static_cast<unsigned>((n / 8 + 255) / 256);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint8_t* q = static_cast<const uint8_t*>(qvalue);
+  const int8_t* zp = static_cast<const int8_t*>(zero_point);
+#define QWIX_DEQ_KEEP(QTT)                                                                                       \
+  do {                                                                                                           \
+    if (out_dtype == dtype)                                                                                      \
+      dequant_keep_rm_kernel<D, QTT, D><<<vb, 256, 0, st>>>(q, outer, reduce, inner, tile, scale, zp, out);      \
+    else                                                                                                         \
+      dequant_keep_rm_kernel<D, QTT, BF16><<<vb, 256, 0, st>>>(q, outer, reduce, inner, tile, scale, zp, out);   \
+  } while (0)
+  QWIX_DISPATCH_D(dtype, {
+    if (qtype == QWIX_INT8) QWIX_DEQ_KEEP(QWIX_INT8);
+    else if (qtype == QWIX_INT4) QWIX_DEQ_KEEP(QWIX_INT4);
+    else if (qtype == QWIX_E4M3) QWIX_DEQ_KEEP(QWIX_E4M3);
+    else return fail(QWIX_ERR_INVALID_ARGUMENT, "unknown qtype %d", qtype);
+  })
+#undef QWIX_DEQ_KEEP
+  return check_launch("dequantize (reduce-minor)");
 }
 
 int qwix_hip_transpose_q(const void* src, int qtype, int64_t rows, int64_t cols, void* dst, void* stream) {

@@ -326,3 +326,71 @@ def test_sub_channel_zero_points_bit_exact(M, K, N, group, wq_type, side, zp_til
   parts = np.asarray(wacc, np.float64).reshape(G, M, N) * sa * sb
   rt = 2.0 ** -6 if dtype is O.BF16 else 1e-5
   assert np.all(np.abs(util.f32np(plain) - want.v) <= rt * np.abs(parts).sum(0) + 1e-30)
+
+
+@pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('M,K,N', [(64, 64, 64), (300, 448, 200), (512, 2048, 1024), (4096, 512, 4096), (2048, 256, 14336)])
+def test_bf16_gemm_against_float64(M, K, N, out_dtype):
+  """qwix_hip_gemm_bf16 through the C ABI: bf16 operands are exact in f64, so the product against numpy's f64
+  matmul bounds the kernel's f32 accumulation (and the one bf16 rounding of the result)."""
+  from qwix_amd import _lib
+  print('case bf16 gemm', M, K, N, out_dtype, flush=True)
+  a_np, a = util.make((M, K), O.BF16, seed=M + N)
+  b_np, b = util.make((N, K), O.BF16, seed=M + N + 1)
+  out = torch.full((M, N), float('nan'), dtype=out_dtype, device=util.DEV)
+  _lib.call('qwix_hip_gemm_bf16', a.data_ptr(), K, b.data_ptr(), K, M, N, K, out.data_ptr(), _lib.float_tag(out_dtype),
+            N, _lib.stream_of(a))
+  torch.cuda.synchronize()
+  want = a_np.astype(np.float64) @ b_np.astype(np.float64).T
+  got = util.f32np(out).astype(np.float64)
+  mag = np.abs(a_np).astype(np.float64) @ np.abs(b_np).astype(np.float64).T   # sum of |products|
+  tol = 2.0 ** -18 * mag + (2.0 ** -8 * np.abs(want) if out_dtype == torch.bfloat16 else 0)
+  assert np.all(np.abs(got - want) <= tol + 1e-30), (np.abs(got - want) / (tol + 1e-30)).max()
+
+
+@pytest.mark.parametrize('case', [('int4', 128, False, torch.float32), ('int8', 128, False, torch.bfloat16),
+                                  ('int4', 256, True, torch.bfloat16), ('int8', None, True, torch.float32),
+                                  ('float8_e4m3fn', None, False, torch.bfloat16)])
+@pytest.mark.parametrize('M,K,N', [(64, 512, 384), (512, 1024, 1024), (2048, 4096, 1536)])
+def test_weight_only_prefill_on_hip_kernels(M, K, N, case):
+  """bf16 activations x quantized weight beyond the decode batch: dequantize into a K-contiguous bf16 array, then
+  the bf16 MFMA GEMM -- both this library's kernels.  The dequantized operand equals the oracle's dequantize bit
+  for bit (bf16 scales) or after one bf16 rounding (f32 scales); the result is compared with the oracle's
+  dequantize-first dot (f64 accumulate) at the tolerance of the weight-only configuration, rtol 1e-2."""
+  from qwix_amd import _lib
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  wq_type, group, asym, sdt = case
+  print('case weight-only prefill', M, K, N, case, flush=True)
+  x_np, x_t = util.make((M, K), O.BF16, seed=M + K)
+  w_np, w_t = util.make((K, N), O.BF16, seed=M + K + 1, scale=0.02)
+  kw = dict(channelwise_axes=[1], tiled_axes={0: group} if group else {}, scale_dtype=sdt)
+  okw = dict(channelwise_axes=[1], tiled_axes={0: group} if group else {}, scale_dtype=util.ORACLE_DT[sdt])
+  if asym:
+    kw['calibration_method'] = okw['calibration_method'] = 'minmax'
+  wq = qarray.quantize_api(w_t, wq_type, **kw)
+  owq = O.quantize_api(O.FArr(w_np, O.BF16), wq_type, **okw)
+  util.assert_qarray_equal(wq, owq, 'weight')
+  # the decode kernel is bypassed by its own row limit (M > 256) or by the operand kind (zero point, e4m3)
+  fit = dg._weight_only_fit(x_t, wq, DN)
+  assert (fit is None) == (asym or wq_type == 'float8_e4m3fn')
+  out = dg._dequantize_then_bf16_gemm(x_t, wq, DN, torch.bfloat16)
+  assert out is not None and out.dtype == torch.bfloat16
+  torch.cuda.synchronize()
+  want = O.dot_general(O.FArr(x_np, O.BF16), owq, DN, O.BF16)
+  got = util.f32np(out)
+  assert np.allclose(got, want.v, rtol=1e-2, atol=1e-2 * np.abs(want.v).mean()), np.abs(got - want.v).max()
+  if M > dg.WEIGHT_ONLY_MAX_ROWS or fit is None:
+    assert torch.equal(dg.dot_general(x_t, wq, DN, preferred_element_type=torch.bfloat16), out)
+  # the dequantized operand itself, against the oracle's dequantize
+  c = dg._Canon(x_t, wq, DN)
+  b, _ = c.rhs_values(wq)
+  sb, gb = c.rhs_scale(wq)
+  zp = None if wq.zero_point is None else c.rhs_zero_point(wq)[0].to(torch.int8)
+  w = torch.empty(N, K, dtype=torch.bfloat16, device=util.DEV)
+  from qwix_amd.core import numerics
+  _lib.call('qwix_hip_dequantize_rm', b.data_ptr(), numerics.qtype_tag(wq.qtype), 1, K, N, K // gb, sb.data_ptr(),
+            _lib.ptr(zp), _lib.float_tag(sb.dtype), w.data_ptr(), _lib.BF16, _lib.stream_of(w))
+  deq = O.dequantize(owq)
+  want_w = O.round_to_bf16(deq.v) if sdt == torch.float32 else deq.v
+  assert np.array_equal(util.f32np(w).T, want_w)
