@@ -808,6 +808,10 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
           default: wait_vmcnt<(6 * G < 63 ? 6 * G : 63)>(); break;
         }
         barrier();  // slab kt is in LDS from every wavefront, and everyone is done reading slab kt - 1
+        // The compiler does not know that these registers were in flight until the wait above: pin them here, so
+        // that no read or copy of them can be scheduled (or have been hoisted) in front of that wait.
+#pragma unroll
+        for (int r = 0; r < 4; ++r) asm volatile("" : "+v"(breg[d][r]));
         if (kt + DEPTH - 1 < KT) issue_group(kt + DEPTH - 1, (d + DEPTH - 1) % DEPTH);
         __builtin_amdgcn_sched_barrier(0);
         read_a(d, 0, 0);
@@ -934,6 +938,13 @@ __global__ void __launch_bounds__(64 * KW)
           default: wait_vmcnt<(6 * G < 63 ? 6 * G : 63)>(); break;
         }
         __builtin_amdgcn_sched_barrier(0);
+        // pin the set that has just landed: nothing may read or copy it in front of the wait above
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          asm volatile("" : "+v"(breg[d][r]));
+#pragma unroll
+          for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(areg[d][i][r]));
+        }
         // set (d - 1) was multiplied one slab ago: refill it DEPTH - 1 slabs ahead
         if (j + DEPTH - 1 < mine) issue_group(wave + (j + DEPTH - 1) * KW, (d + DEPTH - 1) % DEPTH);
         __builtin_amdgcn_sched_barrier(0);

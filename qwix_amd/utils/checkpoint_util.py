@@ -114,8 +114,10 @@ def _as_tensor(x, device) -> torch.Tensor:
   return torch.from_numpy(np.ascontiguousarray(x)).to(device)
 
 
-def _coerce(value, template: torch.Tensor, path, allow_broadcast=False) -> torch.Tensor:
-  """Device, dtype (a value conversion, e.g. int8 codes into an e4m3 template) and shape of the template."""
+def _coerce(value, template: torch.Tensor, path, allow_broadcast=False, follow_layout=False) -> torch.Tensor:
+  """Device, dtype (a value conversion, e.g. int8 codes into an e4m3 template) and shape of the template.
+  follow_layout: also the template's memory layout (a weight that quantize() stores with its contracted axis
+  contiguous keeps that layout when its codes come from a file, so that no GEMM has to re-lay it out)."""
   if isinstance(template, qarray.Int4Tensor) or not isinstance(template, torch.Tensor):
     raise TypeError(f'{path} does not resolve to a dense tensor in the template_params.')
   value = _as_tensor(value, template.device)
@@ -128,7 +130,17 @@ def _coerce(value, template: torch.Tensor, path, allow_broadcast=False) -> torch
       value = broadcast_to(value, template.shape)
     except ValueError as e:
       raise ValueError(f'{path} has shape {tuple(value.shape)}, expected {tuple(template.shape)}.') from e
+  if follow_layout and not template.is_contiguous() and value.numel() and _is_dense_permutation(template):
+    out = torch.empty_strided(tuple(template.shape), template.stride(), dtype=value.dtype, device=value.device)
+    out.copy_(value)  # one re-layout at load time
+    return out
   return value.contiguous()
+
+
+def _is_dense_permutation(t: torch.Tensor) -> bool:
+  """True when t is a permuted view of a dense row-major block (what empty_strided can reproduce)."""
+  order = sorted(range(t.ndim), key=lambda a: (-t.stride(a), a))
+  return t.permute(*order).is_contiguous()
 
 
 def _template_fields(template_param):
@@ -142,7 +154,7 @@ def _template_fields(template_param):
 def _process_quantized_param(checkpoint_param, template_param, path):
   _validate_prequantized_dict(checkpoint_param, path)
   t_q, t_s, t_zp = _template_fields(template_param)
-  qvalue = _coerce(checkpoint_param['qvalue'], t_q, path)
+  qvalue = _coerce(checkpoint_param['qvalue'], t_q, path, follow_layout=True)
   scale = _coerce(checkpoint_param['scale'], t_s, path, allow_broadcast=True)
   zero_point = checkpoint_param.get('zero_point')
   if t_zp is None and zero_point is not None:

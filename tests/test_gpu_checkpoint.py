@@ -44,6 +44,14 @@ def test_prequantized_safetensors_round_trip(tmp_path):
   for name in ('Dense_0', 'Dense_1'):
     a, b = processed[name]['kernel'].array, qparams[name]['kernel'].array
     assert a.qvalue.device.type == 'cuda' and torch.equal(a.qvalue, b.qvalue) and torch.equal(a.scale, b.scale)
+  # codes from the file take the layout quantize() gives such a weight (contracted axis contiguous): the GEMM
+  # reads them as they are, no per-call re-layout
+  from qwix_amd import _lib
+  from qwix_amd.core import qarray as qa_mod
+  for name in ('Dense_0', 'Dense_1'):
+    a, b = processed[name]['kernel'].array, qparams[name]['kernel'].array
+    assert qa_mod.physical_layout(a)[1] == qa_mod.physical_layout(b)[1] == _lib.LAYOUT_REDUCE_MINOR
+    assert a.qvalue.stride() == b.qvalue.stride()
   out = ptq_model.apply(processed, x)
   assert torch.equal(out, ptq_model.apply(qparams, x))
   # the rules can be rebuilt from the payload alone

@@ -287,3 +287,36 @@ def test_fp8_decode_batch_against_a_wide_weight(M, K, N):
   torch.cuda.synchronize()
   want = (a_i.double() @ b_i.double().T) * sa.double()[:, None] * sb.double()[None, :]
   assert torch.equal(out.double(), want)
+
+
+def test_weight_only_int4_prefill_at_the_gemv_weight_shape():
+  """(2048, 4096) bf16 x (4096, 14336) int4 in groups of 128 with power-of-two scales, through reduce-minor
+  dequantize + the bf16 MFMA GEMM: the dequantized weights are small multiples of the scales, exact in bf16, and
+  every partial sum is exact in f32."""
+  from qwix_amd import _lib
+  M, K, N, G = 2048, 4096, 14336, 128
+  x_i = _small_ints((M, K), -3, 3, 11, torch.int8)
+  b_i = _small_ints((N, K), -8, 7, 12, torch.int8)
+  u = (b_i.to(torch.int16) & 0xF).to(torch.uint8)
+  packed = (u[:, 0::2] | (u[:, 1::2] << 4)).contiguous()
+  # scale 2^(g mod 3 - 1) per group, the same for every column: out = sum_g 2^e_g * (x_g . b_g)
+  e = (torch.arange(K // G, device=util.DEV) % 3 - 1).to(torch.float32)
+  sb = torch.pow(2.0, e)[:, None].expand(K // G, N).contiguous()
+  x = x_i.to(torch.bfloat16)
+  w = torch.empty(N, K, dtype=torch.bfloat16, device=util.DEV)
+  out = torch.empty(M, N, dtype=torch.float32, device=util.DEV)
+  print('case weight-only prefill full size', M, K, N, flush=True)
+  st = _lib.stream_of(x)
+  _lib.call('qwix_hip_dequantize_rm', packed.data_ptr(), _lib.INT4, 1, K, N, G, sb.data_ptr(), None, _lib.F32, w.data_ptr(),
+            _lib.BF16, st)
+  _lib.call('qwix_hip_gemm_bf16', x.data_ptr(), K, w.data_ptr(), K, M, N, K, out.data_ptr(), _lib.F32, N, st)
+  torch.cuda.synchronize()
+  # the weights in units of 1/2: exact integers
+  w2 = (b_i.to(torch.int32).reshape(N, K // G, G) * torch.pow(2.0, e + 1).to(torch.int32)[None, :, None]).reshape(N, K)
+  assert torch.equal((w.to(torch.float32) * 2).to(torch.int32), w2)
+  rows = util.rng(13).choice(M, 8, replace=False)
+  want = x_i[rows].cpu().numpy().astype(np.int64) @ w2.cpu().numpy().astype(np.int64).T
+  assert np.abs(want).max() < 2 ** 24
+  assert np.array_equal(out[rows].cpu().to(torch.float64).numpy() * 2, want.astype(np.float64))
+  total = out.to(torch.float64).sum().item() * 2
+  assert total == float(x_i.to(torch.float64).sum(0).cpu().numpy() @ w2.to(torch.float64).sum(0).cpu().numpy())
