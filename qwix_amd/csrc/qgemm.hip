@@ -473,7 +473,7 @@ __device__ __forceinline__ void staged_epilogue(const AccT (&acc)[TM][TN], const
       if (mo < M && no < N) {
         OutT* o = reinterpret_cast<OutT*>(out) + static_cast<int64_t>(mo) * ldo + no;
         if (row_vec && no + EPC <= N) {
-          *reinterpret_cast<uint4*>(o) = v;
+          __builtin_nontemporal_store(__builtin_bit_cast(v4i, v), reinterpret_cast<v4i*>(o));
         } else {
           const OutT* e = reinterpret_cast<const OutT*>(&v);
 #pragma unroll
