@@ -48,6 +48,20 @@ inline int grant_lds(const void* kernel, size_t bytes, LdsGrant& g) {
 }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// ------------------------------------------------------------------ streaming accesses
+// 16-byte load / store of data that this kernel touches exactly once (nontemporal: not kept in the caches).
+typedef int qwix_v4i __attribute__((ext_vector_type(4)));
+typedef int qwix_v2i __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 nt_load16(const uint4* p) {
+  return __builtin_bit_cast(uint4, __builtin_nontemporal_load(reinterpret_cast<const qwix_v4i*>(p)));
+}
+__device__ __forceinline__ void nt_store16(uint4* p, uint4 v) {
+  __builtin_nontemporal_store(__builtin_bit_cast(qwix_v4i, v), reinterpret_cast<qwix_v4i*>(p));
+}
+__device__ __forceinline__ void nt_store8(uint2* p, uint2 v) {
+  __builtin_nontemporal_store(__builtin_bit_cast(qwix_v2i, v), reinterpret_cast<qwix_v2i*>(p));
+}
+
 // ------------------------------------------------------------------ LDS layout
 // Swizzle key of a 128-byte row in LDS: 16-byte chunk c of row r sits at chunk position c ^ swz128(r).  The LDS
 // serves a ds_read_b128 sixteen lanes at a time out of 64 banks (256 bytes): sixteen consecutive rows must land

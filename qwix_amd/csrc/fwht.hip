@@ -204,10 +204,10 @@ __device__ __forceinline__ void store_bytes(void* dst, const uint32_t (&w)[4]) {
   if constexpr (BYTES == 1) *reinterpret_cast<uint8_t*>(dst) = static_cast<uint8_t>(w[0]);
   else if constexpr (BYTES == 2) *reinterpret_cast<uint16_t*>(dst) = static_cast<uint16_t>(w[0]);
   else if constexpr (BYTES == 4) *reinterpret_cast<uint32_t*>(dst) = w[0];
-  else if constexpr (BYTES == 8) *reinterpret_cast<uint2*>(dst) = make_uint2(w[0], w[1]);
+  else if constexpr (BYTES == 8) nt_store8(reinterpret_cast<uint2*>(dst), make_uint2(w[0], w[1]));
   else {
     static_assert(BYTES % 16 == 0, "unsupported store width");
-    *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+    nt_store16(reinterpret_cast<uint4*>(dst), make_uint4(w[0], w[1], w[2], w[3]));
   }
 }
 

@@ -666,9 +666,9 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
       if (p.out_dtype == QWIX_BF16) {
         uint16_t* o = reinterpret_cast<uint16_t*>(p.out) + static_cast<int64_t>(m) * p.ldo + n;
         if (vec_ok) {
-          *reinterpret_cast<uint2*>(o) =
-              make_uint2(f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16),
-                         f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16));
+          nt_store8(reinterpret_cast<uint2*>(o),
+                    make_uint2(f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16),
+                               f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16)));
         } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e)
@@ -677,7 +677,8 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
       } else {
         float* o = reinterpret_cast<float*>(p.out) + static_cast<int64_t>(m) * p.ldo + n;
         if (vec_ok) {
-          *reinterpret_cast<float4*>(o) = make_float4(v[0], v[1], v[2], v[3]);
+          nt_store16(reinterpret_cast<uint4*>(o), make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]),
+                                                             __float_as_uint(v[2]), __float_as_uint(v[3])));
         } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e)

@@ -38,7 +38,7 @@ __device__ __forceinline__ void store_q(const float* v, uint8_t* q, int64_t elem
                         to_int_q<QT>(v[4 * i + 3]));
     }
     if constexpr (N == 8)
-      *reinterpret_cast<uint2*>(q + elem) = make_uint2(w[0], w[1]);
+      nt_store8(reinterpret_cast<uint2*>(q + elem), make_uint2(w[0], w[1]));
     else
       *reinterpret_cast<uint32_t*>(q + elem) = w[0];
   } else if constexpr (QT == QWIX_E4M3) {
@@ -56,7 +56,7 @@ __device__ __forceinline__ void store_q(const float* v, uint8_t* q, int64_t elem
                (w[i] & 0x7F7F7F7Fu);
     }
     if constexpr (N == 8)
-      *reinterpret_cast<uint2*>(q + elem) = make_uint2(w[0], w[1]);
+      nt_store8(reinterpret_cast<uint2*>(q + elem), make_uint2(w[0], w[1]));
     else
       *reinterpret_cast<uint32_t*>(q + elem) = w[0];
   } else {  // INT4: element `elem` is even; low nibble = even element.
@@ -716,7 +716,7 @@ __global__ void __launch_bounds__(256)
       const uint8_t* src = stage + (c * ROW_EL + pc * 16 * EPB) / EPB;
       uint8_t* dst = q + ((o * gm.inner + col) * gm.reduce + r) / EPB;
       if (vec && r + 16 * EPB <= row_end) {
-        *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);
+        nt_store16(reinterpret_cast<uint4*>(dst), *reinterpret_cast<const uint4*>(src));
       } else {
         const int nb = static_cast<int>((min(row_end, r + 16 * EPB) - r + EPB - 1) / EPB);
         for (int k = 0; k < nb; ++k) dst[k] = src[k];
