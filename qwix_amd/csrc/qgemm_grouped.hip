@@ -310,7 +310,8 @@ struct Fast {
 // ST: slab stages in LDS.  With 3, the loads of slab k+2 are issued at the start of slab k and get two slabs of
 // time to land; the wait before the barrier that ends slab k leaves them in flight (vmcnt counts oldest first).
 // ONE: every group is one slab (group == 128): the main loop then has a single straight-line body.
-template <int BQT, bool SBF, bool SAG, bool AUX, bool MAGIC = false, int ST = 2, bool ONE = false>
+// DUMP (with AUX): the corrected partials are also written to acc_out (parity runs).
+template <int BQT, bool SBF, bool SAG, bool AUX, bool MAGIC = false, int ST = 2, bool ONE = false, bool DUMP = false>
 __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     qgemm_grouped_dma_kernel(GroupedArgs p) {
   constexpr int BM = Fast::kBM, BN = Fast::kBN, BK = Fast::kBK, NW = Fast::kNW, TM = Fast::kTM;
@@ -349,6 +350,17 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
       const int row = idx & (BM - 1), g = idx / BM;
       const int m = min(m0 + row, p.M - 1);
       sa_lds[idx] = ld_scale(p.sa, p.sa_dtype, static_cast<int64_t>(m) * p.ga + g);
+    }
+  }
+  // zero-point side values of the tile's rows, [group or 0][row], behind the activation scales
+  int* zu_lds = reinterpret_cast<int*>(smem + ST * STAGE) + (SAG ? (p.K / p.group) * BM : 0);
+  if constexpr (AUX) {
+    if (p.zu != nullptr) {
+      const int gz = p.zu_sg != 0 ? p.K / p.group : 1;
+      for (int idx = tid; idx < gz * BM; idx += NW * 64) {
+        const int row = idx & (BM - 1), g = idx / BM;
+        zu_lds[idx] = p.zu[static_cast<int64_t>(min(m0 + row, p.M - 1)) * p.zu_sm + g * p.zu_sg];
+      }
     }
   }
 
@@ -608,23 +620,36 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
       }
       if constexpr (AUX) {
         // Asymmetric operands and parity runs: the partials as plain integers, folded at the end of the group.
-        // acc[i][r]: row i*32 + 8*(r/4) + 4*hx + r%4 of the wavefront's rows, column ncol
+        // acc[i][4*qd + j]: row i*32 + 8*qd + 4*hx + j of the wavefront's rows, column ncol
         const int ncol = n0 + wc * 32 + frow;
         const bool zp = p.zu != nullptr;
         const int zvl = zp ? p.zv[ncl * p.zv_sn + g * p.zv_sg] : 0;
+        const int* zrow = zu_lds + (p.zu_sg != 0 ? g * BM : 0) + wr * WROWS + 4 * hx;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int row = wr * WROWS + i * 32 + 8 * (r >> 2) + 4 * hx + (r & 3);
-            const int m = m0 + row;
-            int val = W4 ? (acc[i][r] >> 4) : acc[i][r];  // the widened weights carry a factor 16, exactly
-            if (zp) val -= p.zu[min(m, p.M - 1) * p.zu_sm + g * p.zu_sg] * zvl;
-            if (p.acc_out != nullptr && m < p.M && ncol < p.N)
-              p.acc_out[(static_cast<int64_t>(g) * p.M + m) * p.N + ncol] = val;
-            float f = static_cast<float>(val);
-            if constexpr (SAG) f *= sa_lds[g * BM + row];
-            accf[i][r] = __builtin_fmaf(f, sbg, accf[i][r]);
+          for (int qd = 0; qd < 4; ++qd) {
+            int4 z4 = make_int4(0, 0, 0, 0);
+            if (zp) z4 = *reinterpret_cast<const int4*>(zrow + i * 32 + 8 * qd);  // a broadcast per wavefront half
+            const int zz[4] = {z4.x, z4.y, z4.z, z4.w};
+            float sv[4] = {1.f, 1.f, 1.f, 1.f};
+            if constexpr (SAG) {
+              const float4 s4 = *reinterpret_cast<const float4*>(sa_lds + g * BM + wr * WROWS + 4 * hx + i * 32 + 8 * qd);
+              sv[0] = s4.x; sv[1] = s4.y; sv[2] = s4.z; sv[3] = s4.w;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int r = 4 * qd + j;
+              // the widened weights carry a factor 16, exactly
+              const int val = (W4 ? (acc[i][r] >> 4) : acc[i][r]) - zz[j] * zvl;
+              if constexpr (DUMP) {
+                const int m = m0 + wr * WROWS + i * 32 + 8 * qd + 4 * hx + j;
+                if (m < p.M && ncol < p.N) p.acc_out[(static_cast<int64_t>(g) * p.M + m) * p.N + ncol] = val;
+              }
+              float f = static_cast<float>(val);
+              if constexpr (SAG) f *= sv[j];
+              accf[i][r] = __builtin_fmaf(f, sbg, accf[i][r]);
+            }
           }
       }
       sb_cur = sb_next;
@@ -691,18 +716,21 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
 
 // LDS of the fast kernel: `st` slab stages, plus the f32 activation scales of the tile when they are per group.
 template <int BQT>
-size_t grouped_dma_lds(bool sag, int64_t K, int64_t group, int st) {
+size_t grouped_dma_lds(bool sag, int64_t K, int64_t group, int st, int64_t zu_groups = 0) {
   const size_t stages = st * (Fast::kBM * Fast::kBK + Fast::kBN * (BQT == QWIX_INT4 ? 64 : 128));
-  return stages + (sag ? static_cast<size_t>(K / group) * Fast::kBM * sizeof(float) : 0);
+  return stages + (sag ? static_cast<size_t>(K / group) * Fast::kBM * sizeof(float) : 0) +
+         static_cast<size_t>(zu_groups) * Fast::kBM * sizeof(int);
 }
+// rows of zero-point side values that ride along in LDS: one per group, one in all, or none
+inline int64_t zu_groups_of(const GroupedArgs& p) { return p.zu == nullptr ? 0 : (p.zu_sg != 0 ? p.K / p.group : 1); }
 constexpr size_t kLdsMax = 160 * 1024;
 
-template <int BQT, bool SBF, bool SAG, bool AUX, bool MAGIC, int ST, bool ONE>
+template <int BQT, bool SBF, bool SAG, bool AUX, bool MAGIC, int ST, bool ONE, bool DUMP = false>
 int launch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
   constexpr int BM = Fast::kBM, BN = Fast::kBN, NW = Fast::kNW;
-  const size_t smem = grouped_dma_lds<BQT>(SAG, p.K, p.group, ST);
+  const size_t smem = grouped_dma_lds<BQT>(SAG, p.K, p.group, ST, zu_groups_of(p));
   static_assert(ST * (Fast::kBM * Fast::kBK + BN * 64) >= NW * 32 * 36 * sizeof(float), "epilogue staging must fit");
-  auto kern = qgemm_grouped_dma_kernel<BQT, SBF, SAG, AUX, MAGIC, ST, ONE>;
+  auto kern = qgemm_grouped_dma_kernel<BQT, SBF, SAG, AUX, MAGIC, ST, ONE, DUMP>;
   static LdsGrant granted;
   if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   const int64_t tiles = static_cast<int64_t>((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
@@ -716,8 +744,11 @@ template <int BQT, bool SAG>
 int dispatch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
   const bool sbf = p.sb_dtype == QWIX_BF16;
   const bool three = grouped_dma_lds<BQT>(SAG, p.K, p.group, 3) <= kLdsMax;  // room for a third slab stage
-  if (!three && grouped_dma_lds<BQT>(SAG, p.K, p.group, 2) > kLdsMax) return -1;
-  if (p.zu != nullptr || p.acc_out != nullptr)  // asymmetric operands, parity runs
+  if (grouped_dma_lds<BQT>(SAG, p.K, p.group, 2, zu_groups_of(p)) > kLdsMax) return -1;
+  if (p.acc_out != nullptr)  // parity runs
+    return sbf ? launch_grouped_dma<BQT, true, SAG, true, false, 2, false, true>(p, st)
+               : launch_grouped_dma<BQT, false, SAG, true, false, 2, false, true>(p, st);
+  if (p.zu != nullptr)  // an asymmetric operand
     return sbf ? launch_grouped_dma<BQT, true, SAG, true, false, 2, false>(p, st)
                : launch_grouped_dma<BQT, false, SAG, true, false, 2, false>(p, st);
   if (p.group == Fast::kBK) {  // one slab per group
