@@ -230,6 +230,22 @@ QWIX_API int qwix_hip_qgemm_fused_act(const void* x, int x_dtype, int64_t ldx, c
                              int64_t M, int64_t N, int64_t K, const void* sb, int sb_dtype, void* out,
                              int out_dtype, int64_t ldo, void* stream);
 
+/* Dynamic-range w8a8 in one call at any batch size: per-token absmax quantization of x to int8 or e4m3
+ * (qarray.quantize, qwix/_src/core/qarray.py:638-644, as PtqProvider applies it to the lhs of dot_general,
+ * providers/boxed_param.py:416-455) followed by _fast_dot_general (dot_general.py:135-261): the operation that
+ * qwix/contrib/kernels/lhs_fused_quantized_matmul.py specifies, with the numerics of the two reference
+ * functions (per-token scales over the whole of K, scale in the dtype of x).  Decode-size int8 calls run as
+ * one launch (qwix_hip_qgemm_fused_act); every other shape runs the quantize kernel and then the GEMM on the
+ * caller's scratch memory (qwix_hip_qgemm_dynamic_act_workspace_bytes(M, N, K, x_dtype) bytes, 16-byte aligned,
+ * used only by this call until it has finished on `stream`), with dense rows (ldx == K).  Results are
+ * bit-identical to qwix_hip_quantize + qwix_hip_qgemm.  At prefill sizes the two kernels stay separate on
+ * purpose: with per-token scales every column tile of a row panel would redo the panel's quantization. */
+QWIX_API size_t qwix_hip_qgemm_dynamic_act_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtype);
+QWIX_API int qwix_hip_qgemm_dynamic_act(const void* x, int x_dtype, int64_t ldx, const void* b, int64_t ldb, int qtype,
+                               int64_t M, int64_t N, int64_t K, const void* sb, int sb_dtype, int acc_dtype,
+                               void* out, int out_dtype, int64_t ldo, void* workspace,
+                               size_t workspace_bytes, void* stream);
+
 /* out[r] = sum_k q[r*ld + k] for int8 rows (K % 16 == 0): the K-sums qwix_hip_qgemm_zp needs
  * (the reference obtains them as a dot_general against the broadcast zero point,
  * dot_general.py:233-239,246-252). */

@@ -295,14 +295,18 @@ def _batched_qgemm(lhs, rhs, dimension_numbers, preferred_element_type):
   return out.reshape(*bshape, *[lshape[a] for a in lfree], *[rshape[a] for a in rfree])
 
 
-def fused_act_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None):
-  """Dynamic per-token int8 quantization of a float lhs and the quantized contraction in one launch
-  (qwix_hip_qgemm_fused_act), for decode-size calls: at most 32 rows and K <= 2048 against a per-channel int8 weight.
-  Bit-identical to quantize(lhs, channelwise over the non-contracting axes) followed by dot_general.
-  Returns None when the operands do not fit that kernel; the caller then takes the two-step route."""
+def fused_act_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, act_qtype=numerics.INT8):
+  """Dynamic per-token quantization of a float lhs (absmax over the whole contraction, to the weight's own
+  qtype: int8 or e4m3) and the quantized contraction against a per-channel weight in one library call
+  (qwix_hip_qgemm_dynamic_act): one launch at decode sizes, the quantize kernel and the GEMM back to back on a
+  scratch buffer otherwise.  Bit-identical to quantize(lhs, channelwise over the non-contracting axes)
+  followed by dot_general.  Returns None when the operands are not of that kind; the caller then takes the
+  two-step route."""
   if not (_is_float_array(lhs) and lhs.dtype in (torch.bfloat16, torch.float32) and isinstance(rhs, QArray)):
     return None
-  if rhs.zero_point is not None or isinstance(rhs.qvalue, Int4Tensor) or _qtype_of(rhs) != numerics.INT8:
+  if rhs.zero_point is not None or isinstance(rhs.qvalue, Int4Tensor):
+    return None
+  if act_qtype not in (numerics.INT8, numerics.E4M3) or _qtype_of(rhs) != act_qtype:
     return None
   (lca, rca), (lba, rba) = dimension_numbers
   if len(lba) or len(rba) or any(rhs.scale.shape[int(a)] != 1 for a in rca):
@@ -311,19 +315,32 @@ def fused_act_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=No
     c = _Canon(lhs, rhs, dimension_numbers)
   except ValueError:
     return None
-  if not (0 < c.M <= 32) or c.K % 128 or c.K > 2048:
+  if c.M <= 0 or c.K % 16:
     return None
-  x = c.lhs_values(lhs)
-  b, _ = c.rhs_values(rhs)
-  sb, _ = c.rhs_scale(rhs)
+  # qarray.py:781-821 for a (quantized lhs with scales in lhs.dtype, rhs) pair: integer values accumulate in
+  # int32, e4m3 values in the result type.
   res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.scale.dtype)
+  acc_t = torch.int32 if act_qtype == numerics.INT8 else res_t
   if res_t not in (torch.bfloat16, torch.float32):
     return None
+  x = c.lhs_values(lhs)
+  if x.stride(1) != 1 or x.stride(0) != c.K:
+    x = x.contiguous()
+  b, _ = c.rhs_values(rhs)
+  sb, _ = c.rhs_scale(rhs)
   out = torch.empty(c.M, c.N, dtype=res_t, device=x.device)
-  _lib.call('qwix_hip_qgemm_fused_act', x.data_ptr(), _lib.float_tag(x.dtype), x.stride(0), b.data_ptr(), b.stride(0),
-            c.M, c.N, c.K, sb.data_ptr(), _lib.float_tag(sb.dtype), out.data_ptr(), _lib.float_tag(res_t), c.N,
-            _lib.stream_of(x))
+  nws = _dynamic_act_bytes(c.M, c.N, c.K, _lib.float_tag(x.dtype))
+  ws = torch.empty(nws, dtype=torch.uint8, device=x.device) if nws else None
+  _lib.call('qwix_hip_qgemm_dynamic_act', x.data_ptr(), _lib.float_tag(x.dtype), x.stride(0), b.data_ptr(), b.stride(0),
+            _lib.INT8 if act_qtype == numerics.INT8 else _lib.E4M3, c.M, c.N, c.K, sb.data_ptr(),
+            _lib.float_tag(sb.dtype), _tag_of(acc_t) if acc_t != torch.int32 else 0, out.data_ptr(),
+            _lib.float_tag(res_t), c.N, _lib.ptr(ws), nws, _lib.stream_of(x))
   return out.reshape(c.out_shape)
+
+
+@functools.lru_cache(maxsize=None)
+def _dynamic_act_bytes(M: int, N: int, K: int, x_tag: int) -> int:
+  return int(_lib.load().qwix_hip_qgemm_dynamic_act_workspace_bytes(M, N, K, x_tag))
 
 
 @functools.lru_cache(maxsize=None)

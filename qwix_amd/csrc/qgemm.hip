@@ -2156,6 +2156,50 @@ extern "C" int qwix_hip_qgemm_ragged(const void* a, int64_t lda, const void* b, 
   return launch_ragged<QWIX_E4M3>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
 }
 
+// Workspace of qwix_hip_qgemm_dynamic_act: the quantized rows, their scales, what the quantize kernel itself needs
+// for rows too long for one workgroup, and the GEMM's split-K partials; each part 256-byte aligned.
+static size_t dyn_align(size_t v) { return (v + 255) & ~size_t{255}; }
+extern "C" size_t qwix_hip_qgemm_dynamic_act_workspace_bytes(int64_t M, int64_t N, int64_t K, int x_dtype) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const size_t es = x_dtype == QWIX_BF16 ? 2 : 4;
+  return dyn_align(static_cast<size_t>(M) * K) + dyn_align(static_cast<size_t>(M) * es) +
+         dyn_align(qwix_hip_quantize_workspace_bytes(M, K, 1, K, QWIX_ABSMAX)) +
+         dyn_align(qwix_hip_qgemm_workspace_bytes(M, N, K));
+}
+
+extern "C" int qwix_hip_qgemm_dynamic_act(const void* x, int x_dtype, int64_t ldx, const void* b, int64_t ldb, int qtype,
+                                          int64_t M, int64_t N, int64_t K, const void* sb, int sb_dtype, int acc_dtype,
+                                          void* out, int out_dtype, int64_t ldo, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+  if (!x || !b || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null x/b/out");
+  if (x_dtype != QWIX_BF16 && x_dtype != QWIX_F32) return fail(QWIX_ERR_INVALID_ARGUMENT, "activations must be bf16 or f32");
+  if (qtype != QWIX_INT8 && qtype != QWIX_E4M3)
+    return fail(QWIX_ERR_UNSUPPORTED, "dynamic activation quantization to int8 or e4m3 (got qtype %d)", qtype);
+  if (M <= 0 || N <= 0 || K <= 0) return fail(QWIX_ERR_INVALID_ARGUMENT, "bad shape M=%lld N=%lld K=%lld", (long long)M,
+                                             (long long)N, (long long)K);
+  // decode-size int8 calls: one launch (the rows are quantized in the GEMM's prologue)
+  if (qtype == QWIX_INT8 && M <= 32 && K % 128 == 0 && K <= 128 * kSkinnyWaves && sb != nullptr)
+    return qwix_hip_qgemm_fused_act(x, x_dtype, ldx, b, ldb, M, N, K, sb, sb_dtype, out, out_dtype, ldo, stream);
+  // otherwise: the quantize kernel, then the GEMM, on the caller's scratch memory
+  if (ldx != K) return fail(QWIX_ERR_UNSUPPORTED, "the two-launch route needs dense activation rows (ldx=%lld K=%lld)",
+                            (long long)ldx, (long long)K);
+  const size_t need = qwix_hip_qgemm_dynamic_act_workspace_bytes(M, N, K, x_dtype);
+  if (!workspace || workspace_bytes < need || !aligned16(workspace))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "workspace of %zu bytes required, got %zu", need, workspace_bytes);
+  const size_t es = x_dtype == QWIX_BF16 ? 2 : 4;
+  uint8_t* q = static_cast<uint8_t*>(workspace);
+  uint8_t* sa = q + dyn_align(static_cast<size_t>(M) * K);
+  uint8_t* qws = sa + dyn_align(static_cast<size_t>(M) * es);
+  const size_t qws_bytes = qwix_hip_quantize_workspace_bytes(M, K, 1, K, QWIX_ABSMAX);
+  uint8_t* gws = qws + dyn_align(qws_bytes);
+  const size_t gws_bytes = qwix_hip_qgemm_workspace_bytes(M, N, K);
+  if (int e = qwix_hip_quantize(x, x_dtype, M, K, 1, K, qtype, QWIX_ABSMAX, 0.f, QWIX_LAYOUT_NATURAL, q, sa, nullptr,
+                                qws_bytes ? qws : nullptr, qws_bytes, stream))
+    return e;
+  return qgemm_impl(q, K, b, ldb, qtype, M, N, K, sa, x_dtype, sb, sb_dtype, acc_dtype, nullptr, nullptr, out, out_dtype,
+                    ldo, stream, gws_bytes ? gws : nullptr, gws_bytes);
+}
+
 extern "C" int qwix_hip_gemm_bf16(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
                                   void* out, int out_dtype, int64_t ldo, void* stream) {
   if (!a || !b || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/b/out");

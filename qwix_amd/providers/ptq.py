@@ -148,12 +148,17 @@ class BoxedParamProvider(qconfig.QuantizationProvider):
                          _qarray_module=self._qarray_module)
     return lhs, rhs
 
-  def _fusable(self, rule) -> bool:
-    """Decode-size calls may fold the lhs quantization into the GEMM launch: only with the stock kernels,
-    dynamic per-token int8 absmax, and no sub-channel tiling."""
-    return (self._dot_general_fn is _dot_general.dot_general and self._qarray_module is _qarray
-            and rule.act_qtype is not None and str(rule.act_qtype).replace('torch.', '') == 'int8'
-            and not rule.act_static_scale and (rule.act_calibration_method or 'absmax') == 'absmax' and not rule.tile_size)
+  def _fusable(self, rule):
+    """The qtype with which the lhs quantization and the GEMM run as one library call, else None: only with the
+    stock kernels, dynamic per-token absmax to int8 or e4m3, and no sub-channel tiling."""
+    if not (self._dot_general_fn is _dot_general.dot_general and self._qarray_module is _qarray):
+      return None
+    if rule.act_qtype is None or rule.act_static_scale or rule.tile_size:
+      return None
+    if (rule.act_calibration_method or 'absmax') != 'absmax':
+      return None
+    qt = str(rule.act_qtype).replace('torch.', '')
+    return qt if qt in ('int8', 'float8_e4m3fn') else None
 
   @staticmethod
   def _unbox_float(x):
@@ -172,9 +177,10 @@ class BoxedParamProvider(qconfig.QuantizationProvider):
                                             preferred_element_type)
     get_how = functools.partial(_dot_general.get_how_to_quantize, dimension_numbers=dimension_numbers,
                                 ndims=(len(lhs.shape), len(rhs.shape)), tile_size=rule.tile_size)
-    if self._fusable(rule) and isinstance(lhs, torch.Tensor) and lhs.numel() // max(lhs.shape[-1], 1) <= 32:
+    fused_qtype = self._fusable(rule)
+    if fused_qtype is not None and isinstance(lhs, torch.Tensor):
       lhs, rhs = self._prepare(lhs, rhs, rule, op_id, get_how, quantize_lhs=False)
-      out = _dot_general.fused_act_dot_general(lhs, rhs, dimension_numbers)
+      out = _dot_general.fused_act_dot_general(lhs, rhs, dimension_numbers, act_qtype=fused_qtype)
       if out is not None:
         return out
       how = get_how(for_lhs=True, qtype=rule.act_qtype, calibration_method='absmax')

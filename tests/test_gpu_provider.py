@@ -287,5 +287,7 @@ def test_decode_size_calls_fold_the_activation_quantization_into_the_gemm(monkey
   assert torch.equal(out, ptq_model.apply(qparams, x))
   monkeypatch.setattr(dg, 'fused_act_dot_general', lambda *a, **k: (calls.append(1), real(*a, **k))[1])
   big = torch.rand(64, 1024, generator=g, dtype=torch.float32).to(torch.bfloat16).to(util.DEV)
-  ptq_model.apply(qparams, big)
-  assert len(calls) == 2                                                   # 64 tokens: not offered to the fused kernel
+  fused = ptq_model.apply(qparams, big)
+  assert len(calls) == 4                                                   # 64 tokens: the same entry point, two launches
+  monkeypatch.setattr(dg, 'fused_act_dot_general', lambda *a, **k: None)
+  assert torch.equal(fused, ptq_model.apply(qparams, big))

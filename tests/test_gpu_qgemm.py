@@ -178,10 +178,74 @@ def test_fused_activation_quantize_gemm_bit_exact(M, K, N, dtype):
   got = util.f32np(out)
   bad = np.flatnonzero(got.ravel() != want.v.ravel())
   assert bad.size == 0, f'{bad.size} outputs differ: {got.ravel()[bad[:5]]} vs {want.v.ravel()[bad[:5]]}'
-  # shapes the kernel does not take are handed back to the two-step route
-  assert dg.fused_act_dot_general(torch.zeros(40, K, device=util.DEV), wq, DN) is None
-  w4 = qarray.quantize(torch.zeros(4096, 64, device=util.DEV), qarray.HowToQuantize(qtype='int8', channelwise_axes=[1]))
-  assert dg.fused_act_dot_general(torch.zeros(8, 4096, device=util.DEV), w4, DN) is None   # K too long
+  # operands of another kind are handed back to the two-step route
+  w4 = qarray.quantize(torch.zeros(256, 64, device=util.DEV), qarray.HowToQuantize(qtype='int4', channelwise_axes=[1]))
+  assert dg.fused_act_dot_general(torch.zeros(8, 256, device=util.DEV), w4, DN) is None
+  assert dg.fused_act_dot_general(x_t, wq, DN, act_qtype='float8_e4m3fn') is None   # weight is int8
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('qtype', ['int8', 'float8_e4m3fn'])
+@pytest.mark.parametrize('M,K,N', [(40, 2048, 520), (8, 4096, 264), (300, 1024, 1000), (512, 4096, 250), (1024, 512, 2048),
+                                   (3, 20000, 64), (2048, 2048, 2048)])
+def test_dynamic_activation_gemm_in_one_call_bit_exact(M, K, N, qtype, dtype):
+  """qwix_hip_qgemm_dynamic_act at sizes beyond the one-launch kernel (the quantize kernel and the GEMM back to
+  back on one scratch buffer; split-K shapes and rows too long for one workgroup included) == the oracle's
+  quantize followed by its fast dot_general, bit for bit with int8; with e4m3 the f32 accumulation order is the
+  kernel's, so the library's own two-step result is the bit-exact reference and the oracle the tolerance one."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  print('case dynamic act', M, K, N, qtype, dtype, flush=True)
+  x_np, x_t = util.make((M, K), dtype, seed=M + K + 1)
+  x_np[M // 2, :] = 0                        # an all-zero row takes the scale guard
+  x_t = util.to_gpu(x_np, dtype)
+  w_np, w_t = util.make((K, N), dtype, seed=N + 3, scale=0.02)
+  wq = qarray.quantize(w_t, qarray.HowToQuantize(qtype=qtype, channelwise_axes=[1]))
+  out = dg.fused_act_dot_general(x_t, wq, DN, act_qtype=qtype)
+  assert out is not None and out.dtype == util.TORCH_DT[dtype]
+  xq = qarray.quantize(x_t, qarray.HowToQuantize(qtype=qtype, channelwise_axes=[0]))
+  two_step = dg.dot_general(xq, wq, DN)
+  assert torch.equal(out, two_step)
+  oxq = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(qtype=qtype, channelwise_axes=[0]))
+  owq = O.quantize(O.FArr(w_np, dtype), O.HowToQuantize(qtype=qtype, channelwise_axes=[1]))
+  want = O.fast_dot_general(oxq, owq, DN)
+  got = util.f32np(out)
+  if qtype == 'int8':
+    bad = np.flatnonzero(got.ravel() != want.v.ravel())
+    assert bad.size == 0, f'{bad.size} outputs differ: {got.ravel()[bad[:5]]} vs {want.v.ravel()[bad[:5]]}'
+  else:
+    # e4m3 accumulates in f32 in the kernel's own order; with a bf16 result the accumulator and both scalings
+    # are rounded to bf16 in turn, so a last-bit difference of the f32 sum can move the result by two bf16 steps
+    # (2^-6): that bounds every element, and all but 1 in 10^4 must meet the 1e-2 bar.
+    tol = 1e-2 if dtype == O.BF16 else 1e-3
+    atol = tol * float(np.abs(want.v).mean())
+    err = np.abs(got - want.v)
+    assert np.all(err <= (2.0 ** -6 if dtype == O.BF16 else tol) * np.abs(want.v) + atol), err.max()
+    assert np.mean(err <= tol * np.abs(want.v) + atol) >= 1 - 1e-4
+
+
+def test_dynamic_activation_gemm_argument_checks():
+  """The one-call entry point refuses a missing or short scratch buffer and strided rows with an error code and
+  a message instead of launching."""
+  from qwix_amd import _lib
+  L = _lib.load()
+  M, N, K = 64, 128, 256
+  x = torch.zeros(M, K, dtype=torch.bfloat16, device=util.DEV)
+  b = torch.zeros(N, K, dtype=torch.int8, device=util.DEV)
+  sb = torch.ones(N, dtype=torch.bfloat16, device=util.DEV)
+  out = torch.empty(M, N, dtype=torch.bfloat16, device=util.DEV)
+  need = L.qwix_hip_qgemm_dynamic_act_workspace_bytes(M, N, K, _lib.BF16)
+  assert need >= M * K + 2 * M
+  ws = torch.empty(need, dtype=torch.uint8, device=util.DEV)
+  args = lambda ldx, wsp, nws: (x.data_ptr(), _lib.BF16, ldx, b.data_ptr(), K, _lib.INT8, M, N, K, sb.data_ptr(), _lib.BF16, 0,
+                                out.data_ptr(), _lib.BF16, N, wsp, nws, None)
+  assert L.qwix_hip_qgemm_dynamic_act(*args(K, ws.data_ptr(), need)) == 0
+  assert L.qwix_hip_qgemm_dynamic_act(*args(K, None, 0)) != 0
+  assert b'workspace' in L.qwix_hip_last_error()
+  assert L.qwix_hip_qgemm_dynamic_act(*args(K, ws.data_ptr(), need - 1)) != 0
+  assert L.qwix_hip_qgemm_dynamic_act(*args(2 * K, ws.data_ptr(), need)) != 0
+  assert b'dense' in L.qwix_hip_last_error()
+  torch.cuda.synchronize()
 
 
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
