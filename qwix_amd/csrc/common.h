@@ -312,4 +312,20 @@ __device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d) {
 }
 __device__ __forceinline__ uint32_t pack2_i4(int lo, int hi) { return (lo & 0xF) | ((hi & 0xF) << 4); }
 
+// ---- buffer loads: a wave-uniform descriptor plus a 32-bit per-lane byte offset plus a wave-uniform offset ----
+// A descriptor without a bound of its own (the callers' offsets are in range by construction): raw, untyped.
+__device__ __forceinline__ auto buffer_from(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7FFFFFFF, 0x00020000);
+}
+
+// 16 bytes per lane from a buffer straight into LDS (lane l lands at lds + 16 l).  The host pass of the compiler
+// does not know the 16-byte form of this builtin (it checks against its own target), hence the guard: there is
+// nothing to compile on that side.
+template <typename R>
+__device__ __forceinline__ void buffer_to_lds16(R rsrc, uint8_t* lds, unsigned voffset, int soffset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(lds), 16, voffset, soffset, 0, 0);
+#endif
+}
+
 }  // namespace qwix

@@ -60,21 +60,6 @@ struct LaneOff {
   const void *bx, *bw, *bs;  // wave-uniform: x from row row0, weights from row n_base, scales from column n_base
 };
 
-// A descriptor without a bound of its own (the callers' offsets are in range by construction): raw, untyped.
-__device__ __forceinline__ auto buffer_from(const void* base) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7FFFFFFF, 0x00020000);
-}
-
-// 16 bytes per lane from a buffer straight into LDS (lane l lands at lds + 16 l).  The host pass of the compiler
-// does not know the 16-byte form of this builtin (it checks against its own target), hence the guard: there is
-// nothing to compile on that side.
-template <typename R>
-__device__ __forceinline__ void buffer_to_lds16(R rsrc, uint8_t* lds, unsigned voffset, int soffset) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(lds), 16, voffset, soffset, 0, 0);
-#endif
-}
-
 // How the weight bytes are requested decides the speed of this kernel.  The memory side works in 128-byte lines;
 // the 64 bytes that the four lanes of a column need from a weight row per K block are half a line, and reading the
 // 4096 x 14336 int4 weight as 16 rows x 64 bytes per instruction takes 7.9 us (halves requested far apart) or

@@ -1635,7 +1635,10 @@ __device__ __forceinline__ void skinny_block(const uint8_t* __restrict__ A, int6
   const int col = lane & 15, kq = lane >> 4;
   const int nblk = K / 128;
   const int per_wave = (nblk + WAVES - 1) / WAVES;
-  const int kb0 = wave * per_wave, kb1 = min(nblk, kb0 + per_wave);
+  // Which slice of K a wavefront takes rotates with the workgroup: in step, all workgroups would ask the same few
+  // memory channels for the same K offset of their rows at the same time (4096 x 14336 int8, 16 rows: 14.5 -> 13.9 us).
+  const int slice = (wave + static_cast<int>(blockIdx.x)) % WAVES;
+  const int kb0 = min(nblk, slice * per_wave), kb1 = min(nblk, kb0 + per_wave);
 
   // wave-uniform bases + fixed 32-bit lane offsets; rows of A past M and columns past N are clamped
   const uint8_t* a_base = A + static_cast<int64_t>(row0) * lda;
