@@ -156,6 +156,29 @@ def test_weight_only_gemv(M, K, N, group, sdt, wq_type):
 
 
 @pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('M', [1, 20, 40])
+@pytest.mark.parametrize('K,N,group', [(384, 72, 128), (4224, 136, 128), (16384, 264, 256), (8192, 2048, 128), (128, 48, 128)])
+def test_weight_only_gemv_k_splits(M, K, N, group, wq_type):
+  """How the wavefronts of the weight-only kernel share K: an odd number of 128-wide blocks (a last, single block
+  after the pairs), one block in all, and so many blocks that a wavefront makes several trips (the next pair's
+  weights are requested while this pair is multiplied); N that ends inside a column tile."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  print('case gemv k-split', M, K, N, group, wq_type, flush=True)
+  x_np, x_t = util.make((M, K), O.BF16, seed=M + K + 5)
+  w_np, w_t = util.make((K, N), O.BF16, seed=N + K + 6, scale=0.02)
+  wq = qarray.quantize_api(w_t, wq_type, channelwise_axes=[1], tiled_axes={0: group}, scale_dtype=torch.float32)
+  owq = O.quantize_api(O.FArr(w_np, O.BF16), wq_type, channelwise_axes=[1], tiled_axes={0: group}, scale_dtype=O.F32)
+  util.assert_qarray_equal(wq, owq, 'weight')
+  out = dg.dot_general(x_t, wq, DN, preferred_element_type=torch.float32)
+  torch.cuda.synchronize()
+  want = O.dot_general(O.FArr(x_np, O.BF16), owq, DN, O.F32)
+  got = util.f32np(out)
+  # f32 sums in another order than the oracle's: 1e-3 of the typical magnitude
+  assert np.allclose(got, want.v, rtol=1e-3, atol=1e-3 * np.abs(want.v).mean()), np.abs(got - want.v).max()
+
+
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
 @pytest.mark.parametrize('M,K,N', [(30, 1024, 520), (50, 4096, 14336), (130, 512, 6400)])
 def test_weight_only_rows_do_not_depend_on_the_batch(M, K, N, wq_type):
   """More than 16 rows share a pass over the weights (2 tiles of 16 rows per workgroup, fewer wavefronts
