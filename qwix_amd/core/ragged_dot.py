@@ -7,7 +7,9 @@ array), `_fast_ragged_dot_general` (:123-226) and `_slow_ragged_dot_general` (:2
 lhs is (M, K), rhs is (G, K, N); the rows of lhs form G consecutive groups of `group_sizes` rows
 and group g is multiplied with rhs[g].  `group_sizes` stays in device memory: the kernel reads it,
 so the quantized path never synchronises with the host.  Rows past the last group come out as
-zeros.  Only the dimension numbers of `ragged_dot` are supported; others raise.
+zeros.  int4 expert weights and the dequantize-first path run the dense kernels of dot_general group by
+group (these need the group boundaries on the host).  Only the dimension numbers of `ragged_dot` are
+supported; others raise.
 """
 from __future__ import annotations
 
@@ -20,6 +22,7 @@ import torch
 from qwix_amd import _lib
 from qwix_amd.core import numerics
 from qwix_amd.core import qarray
+from qwix_amd.core import dot_general as _dot_general
 from qwix_amd.core.dot_general import DotDimensionNumbers, _is_float_array, _qtype_of, _tag_of
 from qwix_amd.core.qarray import Int4Tensor, QArray
 
@@ -68,6 +71,55 @@ def _rhs_values(v: torch.Tensor) -> torch.Tensor:
   return dst
 
 
+_PLAIN_DOT = (((1,), (0,)), ((), ()))
+
+
+def _rows(x, start: int, stop: int):
+  """Rows start .. stop - 1 of an (M, K) operand: a view, scales and zero points sliced where they are per row."""
+  if not isinstance(x, QArray):
+    return x[start:stop]
+  cut = lambda t: None if t is None else (t[start:stop] if t.shape[0] > 1 else t)
+  q = x.qvalue
+  if isinstance(q, Int4Tensor):
+    if q.packed_axis == 0:
+      raise NotImplementedError('int4 rows packed along the ragged axis cannot be sliced by groups')
+    q = Int4Tensor(q.data[start:stop], (stop - start,) + tuple(q.shape[1:]), q.packed_axis)
+  else:
+    q = q[start:stop]
+  return QArray(qvalue=q, scale=cut(x.scale), zero_point=cut(x.zero_point), qtype=x.qtype)
+
+
+def _group(w, g: int):
+  """Group g of a (G, K, N) operand as a (K, N) operand: a view."""
+  if not isinstance(w, QArray):
+    return w[g]
+  pick = lambda t: None if t is None else t[g if t.shape[0] > 1 else 0]
+  q = w.qvalue
+  if isinstance(q, Int4Tensor):
+    if q.packed_axis == 0:
+      raise NotImplementedError('int4 weights packed along the group axis cannot be sliced by groups')
+    q = Int4Tensor(q.data[g], tuple(q.shape[1:]), q.packed_axis - 1)
+  else:
+    q = q[g]
+  return QArray(qvalue=q, scale=pick(w.scale), zero_point=pick(w.zero_point), qtype=w.qtype)
+
+
+def _group_by_group(fn, lhs, rhs, group_sizes, res_t, **kwargs) -> torch.Tensor:
+  """out[rows of group g] = fn(those rows of lhs, rhs[g]): one call of a dense kernel path per non-empty group.
+  The group boundaries are needed on the host to slice the rows, so this waits for `group_sizes` to arrive there.
+  Rows past the last group stay zero."""
+  M, N = lhs.shape[0], rhs.shape[2]
+  dev = (lhs.scale if isinstance(lhs, QArray) else lhs).device
+  out = torch.zeros(M, N, dtype=res_t, device=dev)
+  start = 0
+  for g, size in enumerate(group_sizes.tolist()):
+    stop = min(start + max(int(size), 0), M)
+    if stop > start:
+      out[start:stop] = fn(_rows(lhs, start, stop), _group(rhs, g), _PLAIN_DOT, preferred_element_type=res_t, **kwargs)
+    start = stop
+  return out
+
+
 def _fast_ragged_dot_general(lhs, rhs, group_sizes, dimension_numbers=_BASIC_RAGGED_DOT_DIMENSION_NUMBERS,
                              precision=None, preferred_element_type=None, group_offset=None) -> torch.Tensor:
   """Contract the quantized values group by group on the matrix cores, then scale:
@@ -77,8 +129,11 @@ def _fast_ragged_dot_general(lhs, rhs, group_sizes, dimension_numbers=_BASIC_RAG
   for x in (lhs, rhs):
     if isinstance(x, QArray) and x.zero_point is not None:
       raise NotImplementedError('zero-point operands take the dequantize-first ragged dot')
-    if isinstance(x.qvalue if isinstance(x, QArray) else x, Int4Tensor):
-      raise NotImplementedError('int4 operands are not supported by the ragged MFMA kernel')
+  if any(isinstance(x.qvalue if isinstance(x, QArray) else x, Int4Tensor) for x in (lhs, rhs)):
+    # int4 values (int8 activations x int4 expert weights): the sub-channel MFMA GEMM of dot_general, group by
+    # group; the ragged kernel itself reads int8 / e4m3 values only
+    _, res_t = qarray.get_accumulator_and_result_type(lhs, rhs, preferred_element_type=preferred_element_type)
+    return _group_by_group(_dot_general._fast_dot_general, lhs, rhs, group_sizes, res_t)
   lq, rq = _qtype_of(lhs), _qtype_of(rhs)
   if (lq, rq) == (numerics.INT8, numerics.INT8):
     qt = _lib.INT8
@@ -143,25 +198,17 @@ def _fast_ragged_dot_general(lhs, rhs, group_sizes, dimension_numbers=_BASIC_RAG
 
 def _slow_ragged_dot_general(lhs, rhs, group_sizes, dimension_numbers=_BASIC_RAGGED_DOT_DIMENSION_NUMBERS,
                              precision=None, preferred_element_type=None, group_offset=None) -> torch.Tensor:
-  """Dequantize (HIP kernel), then one float GEMM per group.  The group boundaries are needed on the
-  host to slice the rows, so this path waits for `group_sizes` to arrive there."""
+  """Dequantize first (ragged_dot.py:229-241), group by group on the dense dequantize-first path: a bf16
+  activation against an expert's int4 / int8 / e4m3 weight runs on this library's weight-only kernels (the fused
+  dequantize + bf16 MFMA kernel up to 256 rows, dequantize + the bf16 MFMA GEMM beyond), every other combination
+  is dequantized by the HIP kernel and contracted by the float GEMM."""
   del precision
   _check_basic(dimension_numbers, lhs, rhs, group_sizes, group_offset)
   if isinstance(lhs, QArray):
     lhs = qarray.dequantize(lhs)
-  if isinstance(rhs, QArray):
-    rhs = qarray.dequantize(rhs)
-  res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.dtype)
-  ct = torch.promote_types(lhs.dtype, rhs.dtype)
-  M = lhs.shape[0]
-  out = torch.zeros(M, rhs.shape[2], dtype=res_t, device=lhs.device)
-  start = 0
-  for g, size in enumerate(group_sizes.tolist()):
-    stop = min(start + max(int(size), 0), M)
-    if stop > start:
-      out[start:stop] = torch.matmul(lhs[start:stop].to(ct), rhs[g].to(ct)).to(res_t)
-    start = stop
-  return out
+  rhs_t = rhs.scale.dtype if isinstance(rhs, QArray) else rhs.dtype
+  res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs_t)
+  return _group_by_group(_dot_general._slow_dot_general, lhs, rhs, group_sizes, res_t)
 
 
 def ragged_dot_general(lhs, rhs, group_sizes: torch.Tensor, dimension_numbers: RaggedDotDimensionNumbers,

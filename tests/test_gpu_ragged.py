@@ -139,6 +139,52 @@ def test_ragged_dot_fp8(shape, sizes, rcw, dtype):
   assert np.all(got[min(sum(sizes), M):] == 0)
 
 
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('shape,sizes,rtiled', [((200, 256, 4, 136), (50, 0, 130, 20), None),
+                                                ((300, 512, 3, 264), (100, 100, 60), {1: 128}),
+                                                ((64, 1024, 6, 128), (1, 0, 30, 3, 0, 9), {1: 256})])
+def test_ragged_dot_int4_expert_weights(shape, sizes, rtiled, dtype):
+  """int8 activations x int4 expert weights (per channel and sub-channel along K): the sub-channel MFMA GEMM of
+  dot_general, group by group.  Its f32 sum of the scaled partials is ordered differently from the oracle's, so
+  the comparison is the one of the dense sub-channel tests (rtol 1e-2 for bf16 results, 1e-3 for f32)."""
+  import qwix_amd
+  M, K, G, N = shape
+  xq, oxq = _quantized((M, K), dtype, 61, _how('int8', (0,)))
+  wq, owq = _quantized((G, K, N), dtype, 62, _how('int4', (0, 2), rtiled), scale=0.05)
+  out = qwix_amd.ragged_dot(xq, wq, _sizes(sizes))
+  torch.cuda.synchronize()
+  want = O.ragged_dot(oxq, owq, sizes).v
+  got = util.f32np(out)
+  assert out.dtype == util.TORCH_DT[dtype] and tuple(got.shape) == (M, N)
+  # The reference rounds every K tile's scaled partial to the result dtype before summing them; the default
+  # kernel keeps them in f32 (as for dot_general): with bf16 results that is up to half a bf16 step of the
+  # largest partial per tile, on top of the 1e-2 bar.
+  tol = 1e-2 if dtype == O.BF16 else 1e-3
+  ntiles = K // (rtiled or {1: K})[1]
+  atol = tol * np.abs(want).mean() + (ntiles * 2.0 ** -8 * np.abs(want).max() if dtype == O.BF16 else 0.0)
+  np.testing.assert_allclose(got, want, rtol=tol, atol=atol)
+  assert np.all(got[min(sum(sizes), M):] == 0)
+
+
+@pytest.mark.parametrize('wq_type,tiled', [('int4', {1: 128}), ('int8', None), ('float8_e4m3fn', None)])
+@pytest.mark.parametrize('sizes', [(3, 0, 20, 1), (300, 40, 0, 172)])
+def test_ragged_dot_weight_only_experts(sizes, wq_type, tiled):
+  """bf16 activations x quantized expert weights (the dequantize-first path, ragged_dot.py:229-241), group by group
+  on this library's weight-only kernels: a few rows per expert (fused dequantize + bf16 MFMA) and hundreds
+  (dequantize, then the bf16 MFMA GEMM)."""
+  import qwix_amd
+  M, K, G, N = 512, 512, 4, 192
+  x_np, x_t = util.make((M, K), O.BF16, seed=71)
+  wq, owq = _quantized((G, K, N), O.BF16, 72, _how(wq_type, (0, 2), tiled), scale=0.05)
+  out = qwix_amd.ragged_dot(x_t, wq, _sizes(sizes))
+  torch.cuda.synchronize()
+  want = O.ragged_dot(O.FArr(x_np, O.BF16), owq, sizes).v
+  got = util.f32np(out)
+  assert out.dtype == torch.bfloat16
+  np.testing.assert_allclose(got, want, rtol=1e-2, atol=1e-2 * np.abs(want).max())   # as for the fp8 experts above
+  assert np.all(got[min(sum(sizes), M):] == 0)
+
+
 def test_ragged_dot_dequantize_first_path():
   """A raw float lhs or a zero point sends the call to the dequantize-first path (ragged_dot.py:278-292)."""
   import qwix_amd
