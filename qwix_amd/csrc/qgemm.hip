@@ -2321,17 +2321,28 @@ __global__ void __launch_bounds__(256)
   if (i0 >= total) return;
   const bool vec = (N & 3) == 0;  // then the four share a row and the loads are 16-byte aligned
   float v[4];
+  // Eight partials are requested before the first is added: one trip to memory per eight splits, not per split.
+  // They are added in split order (int32 sums do not depend on it; the f32 sums of e4m3 partials do).
+  constexpr int kBatch = 8;
   if constexpr (IS_INT) {
     int a[4] = {0, 0, 0, 0};
-    for (int s = 0; s < splits; ++s) {
-      const int* p = reinterpret_cast<const int*>(ws) + s * total + i0;
+    for (int s0 = 0; s0 < splits; s0 += kBatch) {
       if (vec) {
-        const int4 w = *reinterpret_cast<const int4*>(p);
-        a[0] += w.x; a[1] += w.y; a[2] += w.z; a[3] += w.w;
-      } else {
+        int4 w[kBatch];
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (i0 + e < total) a[e] += p[e];
+        for (int j = 0; j < kBatch; ++j) {
+          w[j] = make_int4(0, 0, 0, 0);
+          if (s0 + j < splits) w[j] = *reinterpret_cast<const int4*>(reinterpret_cast<const int*>(ws) + (s0 + j) * total + i0);
+        }
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) { a[0] += w[j].x; a[1] += w[j].y; a[2] += w[j].z; a[3] += w[j].w; }
+      } else {
+        for (int s = s0; s < min(splits, s0 + kBatch); ++s) {
+          const int* p = reinterpret_cast<const int*>(ws) + s * total + i0;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (i0 + e < total) a[e] += p[e];
+        }
       }
     }
 #pragma unroll
@@ -2339,15 +2350,25 @@ __global__ void __launch_bounds__(256)
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e) v[e] = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float* p = reinterpret_cast<const float*>(ws) + s * total + i0;
+    for (int s0 = 0; s0 < splits; s0 += kBatch) {
       if (vec) {
-        const float4 w = *reinterpret_cast<const float4*>(p);
-        v[0] += w.x; v[1] += w.y; v[2] += w.z; v[3] += w.w;
-      } else {
+        float4 w[kBatch];
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (i0 + e < total) v[e] += p[e];
+        for (int j = 0; j < kBatch; ++j) {
+          w[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (s0 + j < splits) w[j] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(ws) + (s0 + j) * total + i0);
+        }
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+          if (s0 + j < splits) { v[0] += w[j].x; v[1] += w[j].y; v[2] += w[j].z; v[3] += w[j].w; }
+        }
+      } else {
+        for (int s = s0; s < min(splits, s0 + kBatch); ++s) {
+          const float* p = reinterpret_cast<const float*>(ws) + s * total + i0;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (i0 + e < total) v[e] += p[e];
+        }
       }
     }
   }
