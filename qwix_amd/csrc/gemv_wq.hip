@@ -263,7 +263,10 @@ __global__ void __launch_bounds__(NWAVE * 64) gemv_wq_kernel(GemvArgs p) {
   a.panel = reinterpret_cast<uint8_t*>(red_raw) + wave * (NT * 2048);
   // int4: the first pair of K blocks is on its way to LDS before anything else is worked out.  The key of panel
   // row 8 i + r is (4 i + (r >> 1)) & 7: it alternates between two values per lane.
-  constexpr int H = (NT + 1) / 2;  // column tiles whose weights are requested before the activations and scales
+  // Column tiles whose weights are requested before the activations and scales: one (M = 1, K 4096, N 14336 by the
+  // number of early tiles out of four: one 8.44 us, two 8.82 us, three 9.00 us; with one the first products start
+  // when a quarter of the wavefront's bytes are there).
+  constexpr int H = 1;
   const unsigned grow = lane >> 3;
   unsigned gchunk[2];
   if constexpr (BQT == QWIX_INT4) {
@@ -296,8 +299,8 @@ __global__ void __launch_bounds__(NWAVE * 64) gemv_wq_kernel(GemvArgs p) {
     for (int t = 0; t < NT; ++t) outacc[rt][t] = v4f{0.f, 0.f, 0.f, 0.f};
 
   // Two K blocks per trip, all their loads issued before the first is consumed.  With int4 weights the first
-  // half of the column tiles is requested first of all (for the first trip: before the address arithmetic of
-  // everything else), then activations and scales, then the second half; the fences keep the scheduler from
+  // column tile is requested first of all (for the first trip: before the address arithmetic of
+  // everything else), then activations and scales, then the other tiles; the fences keep the scheduler from
   // moving anything across the hand-counted waits.
   int kb = kb0;
   for (; kb + 1 < kb1; kb += 2) {
