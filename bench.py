@@ -352,8 +352,9 @@ class GemvW4(Workload):
 
 
 class WeightOnlyPrefill(Workload):
-  """Weight-only int4 g128 at prefill size: per step the int4 weight is dequantized into a K-contiguous bf16
-  array and multiplied with the bf16 activations on the bf16 matrix cores (f32 accumulate, bf16 out)."""
+  """Weight-only int4 g128 at prefill size on the bf16 matrix cores (f32 accumulate, bf16 out).  Above 1024 rows
+  the int4 weight is dequantized into a K-contiguous bf16 array per step and multiplied from there; up to 1024
+  rows one kernel dequantizes it slab by slab inside its workgroups (the operator's own choice of path)."""
 
   bound = 'mfma'
   peak_tops = 2500.0   # dense bf16 MFMA peak, TFLOP/s
@@ -363,8 +364,10 @@ class WeightOnlyPrefill(Workload):
     self.dtype = 'bf16 x int4'
     self.metric = 'weight-only int4 g128 prefill TFLOP/s (weight dequantize included)'
     self.unit = 'TFLOP/s'
+    self.fused = M <= 1024
     # 256 x 256 tiles (ping-pong kernel) once they fill most of the chip, 128 x 128 tiles below
-    self.kernel_name = 'qgemm_pp_kernel' if -(-M // 256) * -(-N // 256) >= 192 else 'qgemm_dma_kernel'
+    self.kernel_name = ('wgemm_w4_kernel' if self.fused else
+                        'qgemm_pp_kernel' if -(-M // 256) * -(-N // 256) >= 192 else 'qgemm_dma_kernel')
 
   def setup(self, dev):
     import torch
@@ -384,12 +387,17 @@ class WeightOnlyPrefill(Workload):
 
   def step(self, i=0):
     L = self.L
-    L.call('qwix_hip_dequantize_rm', self.b.data_ptr(), L.INT4, 1, self.K, self.N, self.group, self.s.data_ptr(), None,
-           L.F32, self.w.data_ptr(), L.BF16, self.stream)
+    if not self.fused:
+      L.call('qwix_hip_dequantize_rm', self.b.data_ptr(), L.INT4, 1, self.K, self.N, self.group, self.s.data_ptr(), None,
+             L.F32, self.w.data_ptr(), L.BF16, self.stream)
     self.kernel(i)
 
   def kernel(self, i=0):
     L = self.L
+    if self.fused:
+      L.call('qwix_hip_gemm_bf16_w4', self.x.data_ptr(), self.K, self.b.data_ptr(), self.b.stride(0), self.M, self.N,
+             self.K, self.group, self.s.data_ptr(), L.F32, self.out.data_ptr(), L.BF16, self.N, self.stream)
+      return
     L.call('qwix_hip_gemm_bf16', self.x.data_ptr(), self.K, self.w.data_ptr(), self.K, self.M, self.N, self.K,
            self.out.data_ptr(), L.BF16, self.N, self.stream)
 

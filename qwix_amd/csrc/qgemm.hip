@@ -2009,6 +2009,240 @@ __global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__
   if (lane == 0) out[row] = s;
 }
 
+// ------------------------------------------------------------------------------------------------
+// bf16 activations x int4 weights with K-group scales, beyond the decode batch (prefill): the weights are dequantized
+// inside the workgroup instead of in a pass of their own.  A 256 x 128 tile on 8 wavefronts (64 x 64 each),
+// v_mfma_f32_32x32x16_bf16, K in slabs of 64 elements (128 bytes of a row of activations), 160 KB of LDS.
+//   The packed weights come in whole 128-byte lines: one direct-to-LDS load per 8 rows fetches 256 elements of
+// K per row, four slabs' worth (a superslab), into one of two raw buffers; the next superslab and its four scales
+// (untracked loads) are requested in the first slab of this one.  While slab kt is multiplied, slab kt + 1 of the
+// weight tile is converted: every thread takes 16 nibbles of one row out of the raw buffer, turns them into
+// bf16(q * scale) -- the value the reference's dequantize gives (qarray.py:692-708, computed in f32 and rounded to
+// bf16: exact for bf16 scales, one more rounding for f32 scales, as qwix_hip_dequantize_rm does) -- and writes them
+// where the dense bf16 kernel expects the weight slab (same XOR swizzle), a quarter of the work in front of each of
+// the slab's four k-steps.  The activations go through three LDS stages by direct-to-LDS loads requested two slabs
+// ahead.  One barrier per slab; the wait in front of it is counted (vmcnt), so that the requests of the slab that
+// ends stay in flight: a full wait there costs a memory round trip per slab (87 us instead of 65 at 512 x 14336 x 4096).
+//   LDS is read and written through ext_vector types only (v4i, qwix_v2i).  Through HIP's struct vectors (uint2,
+// uint4) the compiler cannot tell the access from the destinations of the direct-to-LDS loads in flight and puts
+// an s_waitcnt vmcnt(0) in front of it, which turns every counted wait into a full one.
+// Results are bit-identical to qwix_hip_dequantize_rm + qwix_hip_gemm_bf16: the same bf16 weights, the same MFMA,
+// K walked in the same order.
+template <int OUT, bool SBF>
+__global__ void __launch_bounds__(512)
+    wgemm_w4_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ Q, int64_t ldq,
+                    const void* __restrict__ S, int M, int N, int K, int group, uint8_t* __restrict__ out, int64_t ldo) {
+  constexpr int BM = 256, BN = 128, WGN = 2, TM = 2, TN = 2, NWAVES = 8;
+  constexpr int BK = 128, NK = 4;  // bytes of an activation row per slab (64 elements); k-steps of 16 elements
+  constexpr int A_STAGE = BM * BK, C_STAGE = BN * BK, R_STAGE = BN * 128;
+  constexpr int C_BASE = 3 * A_STAGE, R_BASE = C_BASE + 2 * C_STAGE, LDS_BYTES = R_BASE + 2 * R_STAGE;  // 160 KB
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+  int tile_m, tile_n;
+  tile_coords((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  v16f acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // ---- loaders: 8 rows x 128 bytes per instruction; the global 16-byte chunk that lands at position lane & 7
+  const int lr = lane >> 3;
+  uint32_t goffa[4], goffq[2];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = wave * 32 + j * 8 + lr;
+    goffa[j] = static_cast<uint32_t>(min(m0 + row, M - 1)) * static_cast<uint32_t>(lda) + (((lane & 7) ^ swz8(row)) << 4);
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int row = wave * 16 + j * 8 + lr;
+    goffq[j] = static_cast<uint32_t>(min(n0 + row, N - 1)) * static_cast<uint32_t>(ldq) + (((lane & 7) ^ swz8(row)) << 4);
+  }
+  auto issue_a = [&](int kt, int stage) {  // 4 loads
+    const uint8_t* gk = A + kt * BK;
+    uint8_t* dst = smem + stage * A_STAGE + wave * 32 * BK;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) QWIX_GLDS16(gk + goffa[j], dst + j * 1024);
+  };
+  auto issue_raw = [&](int ss) {  // 2 loads: elements 256 ss .. of 16 weight rows
+    const uint8_t* gq = Q + ss * 128;
+    uint8_t* dst = smem + R_BASE + (ss & 1) * R_STAGE + wave * 16 * 128;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) QWIX_GLDS16(gq + goffq[j], dst + j * 1024);
+  };
+
+  // ---- converter: thread -> (weight row, quarter of the slab's 64 elements)
+  const int crow = tid >> 2, cpart = tid & 3;
+  const char* const sptr = static_cast<const char*>(S) + static_cast<int64_t>(min(n0 + crow, N - 1)) * (SBF ? 2 : 4);
+  const int64_t s_group_pitch = static_cast<int64_t>(N) * (SBF ? 2 : 4);
+  // The scales of four slabs are requested at once, a superslab ahead, by untracked loads (valid once a later
+  // end-of-slab wait has covered them); the pointer walks the groups slab by slab.
+  const int slabs_per_group = group >> 6;
+  const char* sc_ptr = sptr;
+  int sc_left = slabs_per_group;
+  auto request_scales = [&](uint32_t (&dst)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if constexpr (SBF)
+        asm volatile("global_load_ushort %0, %1, off" : "=&v"(dst[j]) : "v"(sc_ptr) : "memory");
+      else
+        asm volatile("global_load_dword %0, %1, off" : "=&v"(dst[j]) : "v"(sc_ptr) : "memory");
+      if (--sc_left == 0) {
+        sc_left = slabs_per_group;
+        sc_ptr += s_group_pitch;
+      }
+    }
+  };
+  auto pin_scales = [&](uint32_t (&v)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(v[j]));
+  };
+  qwix_v2i craw;
+  uint32_t cout[8];
+  auto convert_read = [&](int kt) {
+    const int chunk = ((kt & 3) * 2 + (cpart >> 1)) ^ swz8(crow);
+    craw = *reinterpret_cast<const qwix_v2i*>(smem + R_BASE + ((kt >> 2) & 1) * R_STAGE + crow * 128 + (chunk << 4) + (cpart & 1) * 8);
+  };
+  // A nibble n holds q = (n ^ 8) - 8.  With the 8 folded into the multiply-add, q * scale = fma(n ^ 8, scale, -8 scale): every
+  // term is exact in f32 (four bits times the eight of a bf16 scale), so the product is the one of float(q) * scale, and a
+  // byte of the masked word converts in one instruction.
+  auto convert_quarter = [&](int q4, float sc) {  // elements 4 q4 .. 4 q4 + 3 of this thread's 16
+    const uint32_t w = static_cast<uint32_t>((q4 < 2) ? craw[0] : craw[1]) ^ 0x88888888u;
+    const uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
+    const int b0 = (q4 & 1) * 16;
+    const float m8 = -8.f * sc;
+    const float f0 = __builtin_fmaf(static_cast<float>((even >> b0) & 0xFFu), sc, m8);
+    const float f1 = __builtin_fmaf(static_cast<float>((odd >> b0) & 0xFFu), sc, m8);
+    const float f2 = __builtin_fmaf(static_cast<float>((even >> (b0 + 8)) & 0xFFu), sc, m8);
+    const float f3 = __builtin_fmaf(static_cast<float>((odd >> (b0 + 8)) & 0xFFu), sc, m8);
+    cout[2 * q4] = pack_bf16x2(f0, f1);
+    cout[2 * q4 + 1] = pack_bf16x2(f2, f3);
+  };
+  auto convert_write = [&](int kt) {
+    uint8_t* row = smem + C_BASE + (kt & 1) * C_STAGE + crow * 128;
+    *reinterpret_cast<v4i*>(row + (((2 * cpart) ^ swz8(crow)) << 4)) = v4i{(int)cout[0], (int)cout[1], (int)cout[2], (int)cout[3]};
+    *reinterpret_cast<v4i*>(row + (((2 * cpart + 1) ^ swz8(crow)) << 4)) = v4i{(int)cout[4], (int)cout[5], (int)cout[6], (int)cout[7]};
+  };
+  auto scale_value = [&](uint32_t bits) { return __uint_as_float(SBF ? bits << 16 : bits); };
+
+  // ---- fragments
+  const int a_row = (wm * 64 + (lane & 31)) * BK;
+  const int b_row = C_BASE + (wn * 64 + (lane & 31)) * BK;
+  const int hx = lane >> 5, x7 = swz8(lane & 31);
+  v4i fa[2][TM], fb[2][TN];
+  auto read_frags = [&](int sta, int stc, int ks, int buf) {
+    const int off = ((ks * 2 + hx) ^ x7) << 4;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const v4i*>(smem + sta * A_STAGE + a_row + i * 32 * BK + off);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const v4i*>(smem + stc * C_STAGE + b_row + j * 32 * BK + off);
+  };
+  auto mfma_step = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb[buf][j]),
+                                                            __builtin_bit_cast(bf16x8, fa[buf][i]), acc[i][j], 0, 0, 0);
+  };
+  // End of a slab: this wavefront's LDS writes are done and its loads have landed, except the NEWEST `newest` of
+  // them (vmcnt counts in issue order): the requests of the slab that ends are for two slabs ahead and stay in
+  // flight across the barrier.  Then everybody's.
+  auto end_of_slab = [&](auto newest) {
+    constexpr int n = decltype(newest)::value;
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0x0070 | (n & 15) | ((n >> 4) << 14));  // vmcnt(n), lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using std::integral_constant;
+
+  const int KT = K / 64;  // a multiple of 4
+  uint32_t sc_cur[4], sc_next[4] = {0, 0, 0, 0};
+  int sta = 0;  // LDS stage of the activations of the slab being multiplied: kt % 3
+  // One slab, J = kt % 4: requests activations two slabs ahead (and, at J == 0, the packed weights and scales of
+  // the next superslab), converts the weights of slab kt + 1 between the k-steps of slab kt.
+  auto slab = [&](int kt, auto J, auto LAST) {
+    constexpr int j = decltype(J)::value;
+    constexpr bool last = decltype(LAST)::value;  // the last four slabs: nothing further to request after two
+    constexpr bool more = !(last && j == 3);
+    constexpr bool loads_a = !last || j < 2, loads_w = !last && j == 0;
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (loads_a) issue_a(kt + 2, sta == 0 ? 2 : sta - 1);
+    if constexpr (loads_w) {
+      issue_raw((kt >> 2) + 1);
+      request_scales(sc_next);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (j == 2 && !last) pin_scales(sc_next);  // requested at j == 0, covered by the wait that ended j == 1
+    const float sc = scale_value(j == 3 ? sc_next[0] : sc_cur[(j + 1) & 3]);
+    if constexpr (more) convert_read(kt + 1);
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      if (ks + 1 < NK) read_frags(sta, j & 1, ks + 1, (ks + 1) & 1);
+      if constexpr (more) convert_quarter(ks, sc);
+      mfma_step(ks & 1);
+    }
+    if constexpr (more) convert_write(kt + 1);
+    end_of_slab(integral_constant<int, (loads_a ? 4 : 0) + (loads_w ? 6 : 0)>{});
+    sta = sta == 2 ? 0 : sta + 1;
+    if constexpr (more) read_frags(sta, (j + 1) & 1, 0, 0);
+  };
+
+  // ---- prologue: packed weights and scales of slabs 0..3, activations of slabs 0 and 1; slab 0 converted
+  issue_raw(0);
+  request_scales(sc_cur);
+  issue_a(0, 0);
+  issue_a(1, 1);
+  end_of_slab(integral_constant<int, 0>{});
+  pin_scales(sc_cur);
+  convert_read(0);
+#pragma unroll
+  for (int q4 = 0; q4 < 4; ++q4) convert_quarter(q4, scale_value(sc_cur[0]));
+  convert_write(0);
+  end_of_slab(integral_constant<int, 0>{});
+  read_frags(0, 0, 0, 0);
+
+  using I0 = integral_constant<int, 0>;
+  using I1 = integral_constant<int, 1>;
+  using I2 = integral_constant<int, 2>;
+  using I3 = integral_constant<int, 3>;
+  int kt = 0;
+  for (; kt + 4 < KT; kt += 4) {
+    slab(kt, I0{}, std::false_type{});
+    slab(kt + 1, I1{}, std::false_type{});
+    slab(kt + 2, I2{}, std::false_type{});
+    slab(kt + 3, I3{}, std::false_type{});
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sc_cur[e] = sc_next[e];
+  }
+  slab(kt, I0{}, std::true_type{});
+  slab(kt + 1, I1{}, std::true_type{});
+  slab(kt + 2, I2{}, std::true_type{});
+  slab(kt + 3, I3{}, std::true_type{});
+
+  float sav[TM];
+  float sbv[TN][4][4];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) sav[i] = 1.f;
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sbv[j][qd][r] = 1.f;
+  const Epilogue ep{nullptr, nullptr, 0, 0, OUT, 0, 0, 0, nullptr, nullptr};
+  staged_epilogue<OUT, 0, TM, TN, NWAVES, LDS_BYTES, false>(acc, sav, sbv, ep, m0 + wm * 64, n0 + wn * 64, M, N, out, ldo,
+                                                            smem, wave, lane);
+}
+
 }  // namespace
 }  // namespace qwix
 
@@ -2230,6 +2464,47 @@ extern "C" int qwix_hip_gemm_bf16(const void* a, int64_t lda, const void* b, int
   if (big && kb >= 256) return launch_pp<kOpBf16, QWIX_F32, 0>(a, ldab, b, ldbb, M, N, kb, ep, out, ldo, st);
   if (big) return launch_dma<kOpBf16, 256, 256, 2, 4, QWIX_F32, 0>(a, ldab, b, ldbb, M, N, kb, ep, out, ldo, st);
   return launch_dma<kOpBf16, 128, 128, 2, 2, QWIX_F32, 0>(a, ldab, b, ldbb, M, N, kb, ep, out, ldo, st);
+}
+
+extern "C" int qwix_hip_gemm_bf16_w4(const void* a, int64_t lda, const void* q, int64_t ldq_bytes, int64_t M, int64_t N,
+                                     int64_t K, int64_t group, const void* s, int s_dtype, void* out, int out_dtype,
+                                     int64_t ldo, void* stream) {
+  if (!a || !q || !s || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/q/s/out");
+  if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || 2 * K > INT32_MAX)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad GEMM shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
+                (long long)K);
+  if ((out_dtype != QWIX_BF16 && out_dtype != QWIX_F32) || (s_dtype != QWIX_BF16 && s_dtype != QWIX_F32))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "scale and output dtypes must be f32 or bf16");
+  // K in whole 128-byte lines of packed weights (256 elements); a scale group covers whole 64-element slabs
+  if (K % 256 || group <= 0 || group % 64 || K % group)
+    return fail(QWIX_ERR_UNSUPPORTED, "K=%lld must be a multiple of 256 and group=%lld a multiple of 64 that divides K",
+                (long long)K, (long long)group);
+  if (lda % 8 || lda < K || ldq_bytes % 16 || ldq_bytes < K / 2 || !aligned16(a) || !aligned16(q))
+    return fail(QWIX_ERR_UNSUPPORTED, "activation and weight rows must be 16-byte aligned (lda=%lld ldq=%lld)",
+                (long long)lda, (long long)ldq_bytes);
+  if (ldo < N || !aligned16(out) || (N % 4 == 0 && ldo % 4 != 0))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad output leading dimension %lld for N=%lld", (long long)ldo, (long long)N);
+  if (M * lda * 2 >= (int64_t{1} << 31) || N * ldq_bytes >= (int64_t{1} << 31))
+    return fail(QWIX_ERR_UNSUPPORTED, "operands beyond 2 GiB are not supported");
+  constexpr size_t smem = 3 * 256 * 128 + 2 * 128 * 128 + 2 * 128 * 128;  // the whole 160 KB of a CU
+  const dim3 grid(static_cast<unsigned>(((M + 255) / 256) * ((N + 127) / 128)));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define QWIX_W4_LAUNCH(OUTT, SBFF)                                                                                   \
+  do {                                                                                                               \
+    auto kern = wgemm_w4_kernel<OUTT, SBFF>;                                                                         \
+    static LdsGrant granted;                                                                                         \
+    if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;                           \
+    kern<<<grid, 512, smem, st>>>(static_cast<const uint8_t*>(a), 2 * lda, static_cast<const uint8_t*>(q), ldq_bytes, s, \
+                                  static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), static_cast<int>(group), \
+                                  static_cast<uint8_t*>(out), ldo);                                                  \
+  } while (0)
+  if (out_dtype == QWIX_BF16) {
+    if (s_dtype == QWIX_BF16) QWIX_W4_LAUNCH(QWIX_BF16, true); else QWIX_W4_LAUNCH(QWIX_BF16, false);
+  } else {
+    if (s_dtype == QWIX_BF16) QWIX_W4_LAUNCH(QWIX_F32, true); else QWIX_W4_LAUNCH(QWIX_F32, false);
+  }
+#undef QWIX_W4_LAUNCH
+  return check_launch("gemm_bf16_w4");
 }
 
 extern "C" int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M,

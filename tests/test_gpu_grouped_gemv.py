@@ -371,6 +371,40 @@ def test_bf16_gemm_against_float64(M, K, N, out_dtype):
   assert np.all(np.abs(got - want) <= tol + 1e-30), (np.abs(got - want) / (tol + 1e-30)).max()
 
 
+@pytest.mark.parametrize('sdt', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('M,K,N,group', [(300, 256, 136, 128), (512, 1024, 1000, 256), (257, 2048, 520, 64), (2048, 4096, 1536, 128),
+                                         (1, 512, 64, 512)])
+def test_int4_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, out_dtype, sdt):
+  """qwix_hip_gemm_bf16_w4 through the C ABI == qwix_hip_dequantize_rm (to bf16) + qwix_hip_gemm_bf16, bit for bit: the
+  same bf16 weights, the same MFMA, K walked in the same order; edges in M and N, one slab group (64), several."""
+  from qwix_amd import _lib
+  from qwix_amd.core import qarray
+  print('case w4 prefill', M, K, N, group, out_dtype, sdt, flush=True)
+  x_np, x_t = util.make((M, K), O.BF16, seed=M + K + 21)
+  w_np, w_t = util.make((K, N), O.BF16, seed=N + K + 22, scale=0.02)
+  wq = qarray.quantize_api(w_t, 'int4', channelwise_axes=[1], tiled_axes={0: group}, scale_dtype=sdt)
+  from qwix_amd.core import dot_general as dg
+  c = dg._Canon(x_t, wq, DN)
+  b, is4 = c.rhs_values(wq)
+  sb, gb = c.rhs_scale(wq)
+  assert is4 and gb == K // group
+  st = _lib.stream_of(x_t)
+  w = torch.empty(N, K, dtype=torch.bfloat16, device=util.DEV)
+  _lib.call('qwix_hip_dequantize_rm', b.data_ptr(), _lib.INT4, 1, K, N, group, sb.data_ptr(), None, _lib.float_tag(sb.dtype),
+            w.data_ptr(), _lib.BF16, st)
+  want = torch.empty(M, N, dtype=out_dtype, device=util.DEV)
+  _lib.call('qwix_hip_gemm_bf16', x_t.data_ptr(), K, w.data_ptr(), K, M, N, K, want.data_ptr(), _lib.float_tag(out_dtype), N, st)
+  got = torch.full((M, N), float('nan'), dtype=out_dtype, device=util.DEV)
+  _lib.call('qwix_hip_gemm_bf16_w4', x_t.data_ptr(), K, b.data_ptr(), b.stride(0), M, N, K, group, sb.data_ptr(),
+            _lib.float_tag(sb.dtype), got.data_ptr(), _lib.float_tag(out_dtype), N, st)
+  torch.cuda.synchronize()
+  assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
+  # and against float64 on the dequantized weight
+  ref = x_t.double() @ w.double().T
+  assert torch.allclose(got.double(), ref, rtol=1e-2 if out_dtype == torch.bfloat16 else 1e-4, atol=1e-2 * float(ref.abs().mean()))
+
+
 @pytest.mark.parametrize('case', [('int4', 128, False, torch.float32), ('int8', 128, False, torch.bfloat16),
                                   ('int4', 256, True, torch.bfloat16), ('int8', None, True, torch.float32),
                                   ('float8_e4m3fn', None, False, torch.bfloat16)])
