@@ -9,8 +9,8 @@ first).  Arguments are torch tensors / QArrays in HBM; `dimension_numbers` is
 What reaches a hand-written kernel:
   int8 x int8, e4m3 x e4m3 (per-row x per-column scales)          -> qwix_hip_qgemm
   int8 x int8/int4 with K-group scales (tile % 128 == 0)          -> qwix_hip_qgemm_grouped
-  bf16 activations x int4/int8 weight (weight-only, any group)    -> qwix_hip_gemv_wq up to 256 rows,
-      qwix_hip_gemm_bf16_w4 (symmetric int4, 257..1024 rows), qwix_hip_dequantize_rm + qwix_hip_gemm_bf16 above
+  bf16 activations x int4/int8 weight (weight-only, any group)    -> qwix_hip_gemv_wq up to 256 rows (int4: 176),
+      qwix_hip_gemm_bf16_w4 (symmetric int4, 177..1024 rows), qwix_hip_dequantize_rm + qwix_hip_gemm_bf16 above
 Everything else on the slow path is dequantized by the HIP dequantize kernel and contracted by
 the vendor float GEMM.  Unsupported fast-path combinations raise; they never change path silently.
 """
@@ -529,6 +529,11 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   if len(dimension_numbers[1][0]) or len(dimension_numbers[1][1]):
     return _over_batch(_slow_dot_general, lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type)
   c = _weight_only_fit(lhs, rhs, dimension_numbers)
+  if c is not None and fused_w4_min_rows(c.N) < c.M <= WEIGHT_ONLY_MAX_ROWS and isinstance(rhs.qvalue, Int4Tensor):
+    # one row tile of the dequantizing tile GEMM beats the decode kernel from here on
+    out = _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type, fused_only=True)
+    if out is not None:
+      return out
   if c is not None and c.M <= WEIGHT_ONLY_MAX_ROWS:
     sb, gb = c.rhs_scale(rhs)
     x = c.lhs_values(lhs)
@@ -555,12 +560,21 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
 _FUSED_W4_MAX_ROWS = 1024
 
 
-def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type):
+def fused_w4_min_rows(n: int) -> int:
+  """Rows above which one row tile of the dequantizing tile GEMM beats the decode kernel (`qwix_hip_gemv_wq`).  Its
+  time does not depend on the rows (K 4096: 59 us); the decode kernel's grows with them and falls with N
+  (K 4096, 192 / 256 rows: N 14336 66 / 79 us, N 8192 56 / 72 us, N 4096 54 / 67 us)."""
+  return 176 if n >= 12288 else 224
+
+
+def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type, fused_only=False):
   """The dequantize-first path on this library's own kernels, for a bf16 activation against a quantized weight
   of any of the three qtypes, with or without zero point: the weight is dequantized into a K-contiguous bf16
   array (qwix_hip_dequantize_rm, the reference's D(D(q - zp) * scale) in the scale dtype; an f32 result rounded
   once more to bf16) and contracted by the bf16 MFMA GEMM with f32 accumulation (qwix_hip_gemm_bf16).  Returns
-  None when the operands are not of that kind (then: HIP dequantize + the float GEMM of the vendor library)."""
+  None when the operands are not of that kind (then: HIP dequantize + the float GEMM of the vendor library).
+  Symmetric int4 weights of up to `_FUSED_W4_MAX_ROWS` rows skip the dequantized copy (qwix_hip_gemm_bf16_w4);
+  with `fused_only` nothing else is run."""
   if not (_is_float_array(lhs) and lhs.dtype == torch.bfloat16 and isinstance(rhs, QArray)):
     return None
   if _qtype_of(rhs) not in (numerics.INT4, numerics.INT8, numerics.E4M3):
@@ -597,6 +611,8 @@ def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_ty
     _lib.call('qwix_hip_gemm_bf16_w4', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0), c.M, c.N, c.K, c.K // gb,
               sb.data_ptr(), _lib.float_tag(sb.dtype), out.data_ptr(), _lib.float_tag(res_t), c.N, st)
     return out.reshape(c.out_shape)
+  if fused_only:
+    return None
   w = torch.empty(c.N, c.K, dtype=torch.bfloat16, device=dev)
   _lib.call('qwix_hip_dequantize_rm', b.data_ptr(), numerics.qtype_tag(_qtype_of(rhs)), 1, c.K, c.N, c.K // gb,
             sb.data_ptr(), _lib.ptr(zp), _lib.float_tag(sb.dtype), w.data_ptr(), _lib.BF16, st)

@@ -408,7 +408,7 @@ def test_int4_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, out_dtype, 
 @pytest.mark.parametrize('case', [('int4', 128, False, torch.float32), ('int8', 128, False, torch.bfloat16),
                                   ('int4', 256, True, torch.bfloat16), ('int8', None, True, torch.float32),
                                   ('float8_e4m3fn', None, False, torch.bfloat16)])
-@pytest.mark.parametrize('M,K,N', [(64, 512, 384), (512, 1024, 1024), (2048, 4096, 1536)])
+@pytest.mark.parametrize('M,K,N', [(64, 512, 384), (240, 512, 384), (512, 1024, 1024), (2048, 4096, 1536)])
 def test_weight_only_prefill_on_hip_kernels(M, K, N, case):
   """bf16 activations x quantized weight beyond the decode batch: dequantize into a K-contiguous bf16 array, then
   the bf16 MFMA GEMM -- both this library's kernels.  The dequantized operand equals the oracle's dequantize bit
@@ -437,7 +437,9 @@ def test_weight_only_prefill_on_hip_kernels(M, K, N, case):
   want = O.dot_general(O.FArr(x_np, O.BF16), owq, DN, O.BF16)
   got = util.f32np(out)
   assert np.allclose(got, want.v, rtol=1e-2, atol=1e-2 * np.abs(want.v).mean()), np.abs(got - want.v).max()
-  if M > dg.WEIGHT_ONLY_MAX_ROWS or fit is None:
+  # the operator takes this path beyond the decode kernel's rows, for the operand kinds that kernel does not take, and
+  # for symmetric int4 from the row count on at which the dequantizing tile GEMM wins
+  if M > dg.WEIGHT_ONLY_MAX_ROWS or fit is None or (wq_type == 'int4' and M > dg.fused_w4_min_rows(N)):
     assert torch.equal(dg.dot_general(x_t, wq, DN, preferred_element_type=torch.bfloat16), out)
   # the dequantized operand itself, against the oracle's dequantize
   c = dg._Canon(x_t, wq, DN)
