@@ -9,8 +9,8 @@ first).  Arguments are torch tensors / QArrays in HBM; `dimension_numbers` is
 What reaches a hand-written kernel:
   int8 x int8, e4m3 x e4m3 (per-row x per-column scales)          -> qwix_hip_qgemm
   int8 x int8/int4 with K-group scales (tile % 128 == 0)          -> qwix_hip_qgemm_grouped
-  bf16 activations x int4/int8 weight (weight-only, any group)    -> qwix_hip_gemv_wq up to 256 rows (int4: 176),
-      qwix_hip_gemm_bf16_w4 (symmetric int4, 177..1024 rows), qwix_hip_dequantize_rm + qwix_hip_gemm_bf16 above
+  bf16 activations x int4/int8 weight (weight-only, any group)    -> qwix_hip_gemv_wq up to 256 rows (int4: 144),
+      qwix_hip_gemm_bf16_w4 (symmetric int4, 145..1024 rows), qwix_hip_dequantize_rm + qwix_hip_gemm_bf16 above
 Everything else on the slow path is dequantized by the HIP dequantize kernel and contracted by
 the vendor float GEMM.  Unsupported fast-path combinations raise; they never change path silently.
 """
@@ -562,9 +562,9 @@ _FUSED_W4_MAX_ROWS = 1024
 
 def fused_w4_min_rows(n: int) -> int:
   """Rows above which one row tile of the dequantizing tile GEMM beats the decode kernel (`qwix_hip_gemv_wq`).  Its
-  time does not depend on the rows (K 4096: 59 us); the decode kernel's grows with them and falls with N
-  (K 4096, 192 / 256 rows: N 14336 66 / 79 us, N 8192 56 / 72 us, N 4096 54 / 67 us)."""
-  return 176 if n >= 12288 else 224
+  time does not depend on the rows (K 4096: 50 us with the 64-column tiles such calls get); the decode kernel's
+  grows with them and falls with N (K 4096, 128 / 160 / 192 rows: N 14336 50 / 59 / 66 us, N 8192 - / - / 55 us)."""
+  return 144 if n >= 12288 else 200
 
 
 def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type, fused_only=False):

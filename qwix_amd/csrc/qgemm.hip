@@ -2028,14 +2028,22 @@ __global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__
 // an s_waitcnt vmcnt(0) in front of it, which turns every counted wait into a full one.
 // Results are bit-identical to qwix_hip_dequantize_rm + qwix_hip_gemm_bf16: the same bf16 weights, the same MFMA,
 // K walked in the same order.
-template <int OUT, bool SBF>
+// BN = 64 (tiles of 256 x 64, wavefronts of 64 x 32, 128 KB of LDS) is for calls whose 128-column tiles would leave
+// more than half of the CUs without a workgroup: a workgroup's time is mostly its MFMAs and the conversion, which
+// both halve, while its activation traffic stays.
+template <int OUT, bool SBF, int BN>
 __global__ void __launch_bounds__(512)
     wgemm_w4_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ Q, int64_t ldq,
                     const void* __restrict__ S, int M, int N, int K, int group, uint8_t* __restrict__ out, int64_t ldo) {
-  constexpr int BM = 256, BN = 128, WGN = 2, TM = 2, TN = 2, NWAVES = 8;
+  static_assert(BN == 128 || BN == 64, "column tiles of 128 or 64");
+  constexpr int BM = 256, WGN = 2, WN = BN / WGN, TM = 2, TN = WN / 32, NWAVES = 8;
   constexpr int BK = 128, NK = 4;  // bytes of an activation row per slab (64 elements); k-steps of 16 elements
   constexpr int A_STAGE = BM * BK, C_STAGE = BN * BK, R_STAGE = BN * 128;
-  constexpr int C_BASE = 3 * A_STAGE, R_BASE = C_BASE + 2 * C_STAGE, LDS_BYTES = R_BASE + 2 * R_STAGE;  // 160 KB
+  constexpr int C_BASE = 3 * A_STAGE, R_BASE = C_BASE + 2 * C_STAGE, LDS_BYTES = R_BASE + 2 * R_STAGE;  // 160 / 128 KB
+  constexpr int NQ = BN / 64;       // direct-to-LDS loads of packed weights per wavefront and superslab (8 rows each)
+  constexpr int TPR = 512 / BN;     // converter threads per weight row: 4 or 8
+  constexpr int NPT = 64 / TPR;     // nibbles per thread and slab: 16 or 8
+  constexpr int NCQ = NPT / 4;      // conversion steps of four elements: 4 or 2
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -2054,15 +2062,15 @@ __global__ void __launch_bounds__(512)
 
   // ---- loaders: 8 rows x 128 bytes per instruction; the global 16-byte chunk that lands at position lane & 7
   const int lr = lane >> 3;
-  uint32_t goffa[4], goffq[2];
+  uint32_t goffa[4], goffq[NQ];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int row = wave * 32 + j * 8 + lr;
     goffa[j] = static_cast<uint32_t>(min(m0 + row, M - 1)) * static_cast<uint32_t>(lda) + (((lane & 7) ^ swz8(row)) << 4);
   }
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int row = wave * 16 + j * 8 + lr;
+  for (int j = 0; j < NQ; ++j) {
+    const int row = wave * (8 * NQ) + j * 8 + lr;
     goffq[j] = static_cast<uint32_t>(min(n0 + row, N - 1)) * static_cast<uint32_t>(ldq) + (((lane & 7) ^ swz8(row)) << 4);
   }
   auto issue_a = [&](int kt, int stage) {  // 4 loads
@@ -2071,15 +2079,15 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
     for (int j = 0; j < 4; ++j) QWIX_GLDS16(gk + goffa[j], dst + j * 1024);
   };
-  auto issue_raw = [&](int ss) {  // 2 loads: elements 256 ss .. of 16 weight rows
+  auto issue_raw = [&](int ss) {  // NQ loads: elements 256 ss .. of 8 NQ weight rows
     const uint8_t* gq = Q + ss * 128;
-    uint8_t* dst = smem + R_BASE + (ss & 1) * R_STAGE + wave * 16 * 128;
+    uint8_t* dst = smem + R_BASE + (ss & 1) * R_STAGE + wave * (8 * NQ) * 128;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) QWIX_GLDS16(gq + goffq[j], dst + j * 1024);
+    for (int j = 0; j < NQ; ++j) QWIX_GLDS16(gq + goffq[j], dst + j * 1024);
   };
 
-  // ---- converter: thread -> (weight row, quarter of the slab's 64 elements)
-  const int crow = tid >> 2, cpart = tid & 3;
+  // ---- converter: thread -> (weight row, NPT of the slab's 64 elements)
+  const int crow = tid / TPR, cpart = tid % TPR;
   const char* const sptr = static_cast<const char*>(S) + static_cast<int64_t>(min(n0 + crow, N - 1)) * (SBF ? 2 : 4);
   const int64_t s_group_pitch = static_cast<int64_t>(N) * (SBF ? 2 : 4);
   // The scales of four slabs are requested at once, a superslab ahead, by untracked loads (valid once a later
@@ -2104,17 +2112,26 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
     for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(v[j]));
   };
-  qwix_v2i craw;
-  uint32_t cout[8];
+  int craw[NPT / 8];  // NPT / 2 bytes of the row's line: 32 bytes per slab, in two 16-byte chunks
+  uint32_t cout[NPT / 2];
   auto convert_read = [&](int kt) {
-    const int chunk = ((kt & 3) * 2 + (cpart >> 1)) ^ swz8(crow);
-    craw = *reinterpret_cast<const qwix_v2i*>(smem + R_BASE + ((kt >> 2) & 1) * R_STAGE + crow * 128 + (chunk << 4) + (cpart & 1) * 8);
+    const int byte = cpart * (NPT / 2);  // of the slab's 32
+    const int chunk = ((kt & 3) * 2 + (byte >> 4)) ^ swz8(crow);
+    const uint8_t* src = smem + R_BASE + ((kt >> 2) & 1) * R_STAGE + crow * 128 + (chunk << 4) + (byte & 15);
+    if constexpr (NPT == 16) {
+      const qwix_v2i v = *reinterpret_cast<const qwix_v2i*>(src);
+      craw[0] = v[0];
+      craw[1] = v[1];
+    } else {
+      craw[0] = *reinterpret_cast<const int*>(src);
+    }
   };
   // A nibble n holds q = (n ^ 8) - 8.  With the 8 folded into the multiply-add, q * scale = fma(n ^ 8, scale, -8 scale): every
   // term is exact in f32 (four bits times the eight of a bf16 scale), so the product is the one of float(q) * scale, and a
   // byte of the masked word converts in one instruction.
-  auto convert_quarter = [&](int q4, float sc) {  // elements 4 q4 .. 4 q4 + 3 of this thread's 16
-    const uint32_t w = static_cast<uint32_t>((q4 < 2) ? craw[0] : craw[1]) ^ 0x88888888u;
+  auto convert_quarter = [&](int q4, float sc) {  // elements 4 q4 .. 4 q4 + 3 of this thread's NPT
+    if (q4 >= NCQ) return;
+    const uint32_t w = static_cast<uint32_t>(craw[q4 >> 1]) ^ 0x88888888u;
     const uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
     const int b0 = (q4 & 1) * 16;
     const float m8 = -8.f * sc;
@@ -2125,16 +2142,18 @@ __global__ void __launch_bounds__(512)
     cout[2 * q4] = pack_bf16x2(f0, f1);
     cout[2 * q4 + 1] = pack_bf16x2(f2, f3);
   };
-  auto convert_write = [&](int kt) {
+  auto convert_write = [&](int kt) {  // NPT bf16 values: one or two 16-byte chunks of the row's slab
     uint8_t* row = smem + C_BASE + (kt & 1) * C_STAGE + crow * 128;
-    *reinterpret_cast<v4i*>(row + (((2 * cpart) ^ swz8(crow)) << 4)) = v4i{(int)cout[0], (int)cout[1], (int)cout[2], (int)cout[3]};
-    *reinterpret_cast<v4i*>(row + (((2 * cpart + 1) ^ swz8(crow)) << 4)) = v4i{(int)cout[4], (int)cout[5], (int)cout[6], (int)cout[7]};
+#pragma unroll
+    for (int c = 0; c < NPT / 8; ++c)
+      *reinterpret_cast<v4i*>(row + (((cpart * (NPT / 8) + c) ^ swz8(crow)) << 4)) =
+          v4i{(int)cout[4 * c], (int)cout[4 * c + 1], (int)cout[4 * c + 2], (int)cout[4 * c + 3]};
   };
   auto scale_value = [&](uint32_t bits) { return __uint_as_float(SBF ? bits << 16 : bits); };
 
   // ---- fragments
   const int a_row = (wm * 64 + (lane & 31)) * BK;
-  const int b_row = C_BASE + (wn * 64 + (lane & 31)) * BK;
+  const int b_row = C_BASE + (wn * WN + (lane & 31)) * BK;
   const int hx = lane >> 5, x7 = swz8(lane & 31);
   v4i fa[2][TM], fb[2][TN];
   auto read_frags = [&](int sta, int stc, int ks, int buf) {
@@ -2191,7 +2210,7 @@ __global__ void __launch_bounds__(512)
       mfma_step(ks & 1);
     }
     if constexpr (more) convert_write(kt + 1);
-    end_of_slab(integral_constant<int, (loads_a ? 4 : 0) + (loads_w ? 6 : 0)>{});
+    end_of_slab(integral_constant<int, (loads_a ? 4 : 0) + (loads_w ? NQ + 4 : 0)>{});
     sta = sta == 2 ? 0 : sta + 1;
     if constexpr (more) read_frags(sta, (j + 1) & 1, 0, 0);
   };
@@ -2239,7 +2258,7 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
       for (int r = 0; r < 4; ++r) sbv[j][qd][r] = 1.f;
   const Epilogue ep{nullptr, nullptr, 0, 0, OUT, 0, 0, 0, nullptr, nullptr};
-  staged_epilogue<OUT, 0, TM, TN, NWAVES, LDS_BYTES, false>(acc, sav, sbv, ep, m0 + wm * 64, n0 + wn * 64, M, N, out, ldo,
+  staged_epilogue<OUT, 0, TM, TN, NWAVES, LDS_BYTES, false>(acc, sav, sbv, ep, m0 + wm * 64, n0 + wn * WN, M, N, out, ldo,
                                                             smem, wave, lane);
 }
 
@@ -2486,23 +2505,30 @@ extern "C" int qwix_hip_gemm_bf16_w4(const void* a, int64_t lda, const void* q, 
     return fail(QWIX_ERR_INVALID_ARGUMENT, "bad output leading dimension %lld for N=%lld", (long long)ldo, (long long)N);
   if (M * lda * 2 >= (int64_t{1} << 31) || N * ldq_bytes >= (int64_t{1} << 31))
     return fail(QWIX_ERR_UNSUPPORTED, "operands beyond 2 GiB are not supported");
-  constexpr size_t smem = 3 * 256 * 128 + 2 * 128 * 128 + 2 * 128 * 128;  // the whole 160 KB of a CU
-  const dim3 grid(static_cast<unsigned>(((M + 255) / 256) * ((N + 127) / 128)));
+  // 64-column tiles while 128-column ones would occupy at most half of the CUs
+  const bool narrow = ((M + 255) / 256) * ((N + 127) / 128) <= 128;
   hipStream_t st = static_cast<hipStream_t>(stream);
-#define QWIX_W4_LAUNCH(OUTT, SBFF)                                                                                   \
+#define QWIX_W4_LAUNCH(OUTT, SBFF, BNN)                                                                              \
   do {                                                                                                               \
-    auto kern = wgemm_w4_kernel<OUTT, SBFF>;                                                                         \
+    auto kern = wgemm_w4_kernel<OUTT, SBFF, BNN>;                                                                    \
+    constexpr size_t smem = 3 * 256 * 128 + 2 * BNN * 128 + 2 * BNN * 128;  /* 160 KB, all of a CU's, or 128 KB */   \
+    const dim3 grid(static_cast<unsigned>(((M + 255) / 256) * ((N + BNN - 1) / BNN)));                               \
     static LdsGrant granted;                                                                                         \
     if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;                           \
     kern<<<grid, 512, smem, st>>>(static_cast<const uint8_t*>(a), 2 * lda, static_cast<const uint8_t*>(q), ldq_bytes, s, \
                                   static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), static_cast<int>(group), \
                                   static_cast<uint8_t*>(out), ldo);                                                  \
   } while (0)
+#define QWIX_W4_PICK(OUTT, SBFF)                                                                                     \
+  do {                                                                                                               \
+    if (narrow) QWIX_W4_LAUNCH(OUTT, SBFF, 64); else QWIX_W4_LAUNCH(OUTT, SBFF, 128);                                \
+  } while (0)
   if (out_dtype == QWIX_BF16) {
-    if (s_dtype == QWIX_BF16) QWIX_W4_LAUNCH(QWIX_BF16, true); else QWIX_W4_LAUNCH(QWIX_BF16, false);
+    if (s_dtype == QWIX_BF16) QWIX_W4_PICK(QWIX_BF16, true); else QWIX_W4_PICK(QWIX_BF16, false);
   } else {
-    if (s_dtype == QWIX_BF16) QWIX_W4_LAUNCH(QWIX_F32, true); else QWIX_W4_LAUNCH(QWIX_F32, false);
+    if (s_dtype == QWIX_BF16) QWIX_W4_PICK(QWIX_F32, true); else QWIX_W4_PICK(QWIX_F32, false);
   }
+#undef QWIX_W4_PICK
 #undef QWIX_W4_LAUNCH
   return check_launch("gemm_bf16_w4");
 }

@@ -374,10 +374,11 @@ def test_bf16_gemm_against_float64(M, K, N, out_dtype):
 @pytest.mark.parametrize('sdt', [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize('M,K,N,group', [(300, 256, 136, 128), (512, 1024, 1000, 256), (257, 2048, 520, 64), (2048, 4096, 1536, 128),
-                                         (1, 512, 64, 512)])
+                                         (1, 512, 64, 512), (600, 512, 8400, 128), (1100, 256, 4100, 64)])
 def test_int4_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, out_dtype, sdt):
   """qwix_hip_gemm_bf16_w4 through the C ABI == qwix_hip_dequantize_rm (to bf16) + qwix_hip_gemm_bf16, bit for bit: the
-  same bf16 weights, the same MFMA, K walked in the same order; edges in M and N, one slab group (64), several."""
+  same bf16 weights, the same MFMA, K walked in the same order; edges in M and N, one slab group (64), several; the
+  last two shapes have more than 128 tiles of 256 x 128 and run those, the others tiles of 256 x 64."""
   from qwix_amd import _lib
   from qwix_amd.core import qarray
   print('case w4 prefill', M, K, N, group, out_dtype, sdt, flush=True)
@@ -408,7 +409,7 @@ def test_int4_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, out_dtype, 
 @pytest.mark.parametrize('case', [('int4', 128, False, torch.float32), ('int8', 128, False, torch.bfloat16),
                                   ('int4', 256, True, torch.bfloat16), ('int8', None, True, torch.float32),
                                   ('float8_e4m3fn', None, False, torch.bfloat16)])
-@pytest.mark.parametrize('M,K,N', [(64, 512, 384), (240, 512, 384), (512, 1024, 1024), (2048, 4096, 1536)])
+@pytest.mark.parametrize('M,K,N', [(64, 512, 384), (208, 512, 384), (512, 1024, 1024), (2048, 4096, 1536)])
 def test_weight_only_prefill_on_hip_kernels(M, K, N, case):
   """bf16 activations x quantized weight beyond the decode batch: dequantize into a K-contiguous bf16 array, then
   the bf16 MFMA GEMM -- both this library's kernels.  The dequantized operand equals the oracle's dequantize bit
