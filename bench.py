@@ -366,7 +366,7 @@ class WeightOnlyPrefill(Workload):
     self.unit = 'TFLOP/s'
     self.fused = M <= 1024
     # 256 x 256 tiles (ping-pong kernel) once they fill most of the chip, 128 x 128 tiles below
-    self.kernel_name = ('wgemm_w4_kernel' if self.fused else
+    self.kernel_name = ('wgemm_wq_kernel' if self.fused else
                         'qgemm_pp_kernel' if -(-M // 256) * -(-N // 256) >= 192 else 'qgemm_dma_kernel')
 
   def setup(self, dev):
@@ -395,8 +395,8 @@ class WeightOnlyPrefill(Workload):
   def kernel(self, i=0):
     L = self.L
     if self.fused:
-      L.call('qwix_hip_gemm_bf16_w4', self.x.data_ptr(), self.K, self.b.data_ptr(), self.b.stride(0), self.M, self.N,
-             self.K, self.group, self.s.data_ptr(), L.F32, self.out.data_ptr(), L.BF16, self.N, self.stream)
+      L.call('qwix_hip_gemm_bf16_wq', self.x.data_ptr(), self.K, self.b.data_ptr(), self.b.stride(0), L.INT4, self.M,
+             self.N, self.K, self.group, self.s.data_ptr(), L.F32, self.out.data_ptr(), L.BF16, self.N, self.stream)
       return
     L.call('qwix_hip_gemm_bf16', self.x.data_ptr(), self.K, self.w.data_ptr(), self.K, self.M, self.N, self.K,
            self.out.data_ptr(), L.BF16, self.N, self.stream)

@@ -9,8 +9,9 @@ first).  Arguments are torch tensors / QArrays in HBM; `dimension_numbers` is
 What reaches a hand-written kernel:
   int8 x int8, e4m3 x e4m3 (per-row x per-column scales)          -> qwix_hip_qgemm
   int8 x int8/int4 with K-group scales (tile % 128 == 0)          -> qwix_hip_qgemm_grouped
-  bf16 activations x int4/int8 weight (weight-only, any group)    -> qwix_hip_gemv_wq up to 256 rows (int4: 144),
-      qwix_hip_gemm_bf16_w4 (symmetric int4, 145..1024 rows), qwix_hip_dequantize_rm + qwix_hip_gemm_bf16 above
+  bf16 activations x int4/int8 weight (weight-only, any group)    -> qwix_hip_gemv_wq up to 104..200 rows,
+      qwix_hip_gemm_bf16_wq (symmetric int4 up to 1024 rows, int8 up to one round of tiles),
+      qwix_hip_dequantize_rm + qwix_hip_gemm_bf16 above
 Everything else on the slow path is dequantized by the HIP dequantize kernel and contracted by
 the vendor float GEMM.  Unsupported fast-path combinations raise; they never change path silently.
 """
@@ -529,7 +530,7 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   if len(dimension_numbers[1][0]) or len(dimension_numbers[1][1]):
     return _over_batch(_slow_dot_general, lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type)
   c = _weight_only_fit(lhs, rhs, dimension_numbers)
-  if c is not None and fused_w4_min_rows(c.N) < c.M <= WEIGHT_ONLY_MAX_ROWS and isinstance(rhs.qvalue, Int4Tensor):
+  if c is not None and fused_wq_min_rows(c.N, isinstance(rhs.qvalue, Int4Tensor)) < c.M <= WEIGHT_ONLY_MAX_ROWS:
     # one row tile of the dequantizing tile GEMM beats the decode kernel from here on
     out = _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type, fused_only=True)
     if out is not None:
@@ -555,16 +556,30 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   return float_dot_general(lhs, rhs, dimension_numbers, res_t)
 
 
-# Above this many rows the int4 weight is dequantized once into memory instead of once per row tile of the GEMM
-# (K 4096, N 14336, per call: 512 rows 79 us against 114, 1024 rows 154 against 156, 2048 rows 293 against 260).
-_FUSED_W4_MAX_ROWS = 1024
+# The tile GEMM that dequantizes the weight inside its workgroups converts it once per row tile of 256; above these
+# sizes dequantizing it once into memory and running the dense bf16 GEMM is faster.  int4 (K 4096, N 14336, per
+# call): 512 rows 79 us against 114, 1024 rows 154 against 156, 2048 rows 293 against 260.  int8: one round of
+# 256 x 128 tiles (N 14336: 512 rows 82 against 118, 1024 rows 170 against 159; N 4096: 2048 rows 90 against 94).
+_FUSED_WQ_MAX_ROWS = 1024
 
 
-def fused_w4_min_rows(n: int) -> int:
+def _fused_wq_takes(m: int, n: int, int4: bool) -> bool:
+  if int4:
+    return m <= _FUSED_WQ_MAX_ROWS
+  return -(-m // 256) * -(-n // 128) <= _FUSED_W8_MAX_TILES
+
+
+_FUSED_W8_MAX_TILES = 256
+
+
+def fused_wq_min_rows(n: int, int4: bool = True) -> int:
   """Rows above which one row tile of the dequantizing tile GEMM beats the decode kernel (`qwix_hip_gemv_wq`).  Its
   time does not depend on the rows (K 4096: 50 us with the 64-column tiles such calls get); the decode kernel's
-  grows with them and falls with N (K 4096, 128 / 160 / 192 rows: N 14336 50 / 59 / 66 us, N 8192 - / - / 55 us)."""
-  return 144 if n >= 12288 else 200
+  grows with them and falls with N.  K 4096, int4, 128 / 160 / 192 rows: N 14336 50 / 59 / 66 us, N 8192 - / - / 55.
+  int8 (tile GEMM 54 / 47 us at N 14336 / 4096), 96 / 128 / 192 rows: N 14336 54 / 66 / 96 us, N 4096 31 / 39 / 57."""
+  if int4:
+    return 144 if n >= 12288 else 200
+  return 104 if n >= 12288 else 160
 
 
 def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type, fused_only=False):
@@ -573,7 +588,7 @@ def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_ty
   array (qwix_hip_dequantize_rm, the reference's D(D(q - zp) * scale) in the scale dtype; an f32 result rounded
   once more to bf16) and contracted by the bf16 MFMA GEMM with f32 accumulation (qwix_hip_gemm_bf16).  Returns
   None when the operands are not of that kind (then: HIP dequantize + the float GEMM of the vendor library).
-  Symmetric int4 weights of up to `_FUSED_W4_MAX_ROWS` rows skip the dequantized copy (qwix_hip_gemm_bf16_w4);
+  Symmetric int4 / int8 weights skip the dequantized copy while `_fused_wq_takes` (qwix_hip_gemm_bf16_wq);
   with `fused_only` nothing else is run."""
   if not (_is_float_array(lhs) and lhs.dtype == torch.bfloat16 and isinstance(rhs, QArray)):
     return None
@@ -591,7 +606,7 @@ def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_ty
     if len(order) - 1 not in packed:
       return None
   x = c.lhs_values(lhs)
-  b, _ = c.rhs_values(rhs)
+  b, b_is4 = c.rhs_values(rhs)
   sb, _ = c.rhs_scale(rhs)
   zp = None
   if rhs.zero_point is not None:
@@ -603,13 +618,14 @@ def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_ty
   res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.scale.dtype)
   if res_t not in (torch.bfloat16, torch.float32):
     return None
-  if (isinstance(rhs.qvalue, Int4Tensor) and zp is None and c.M <= _FUSED_W4_MAX_ROWS and c.K % 256 == 0
-      and (c.K // gb) % 64 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0):
-    # symmetric int4: dequantized inside the GEMM's workgroups, slab by slab (the same bf16 weights, the same
-    # products in the same order, no dequantized copy of the weight in memory)
+  if (_qtype_of(rhs) in (numerics.INT4, numerics.INT8) and zp is None and _fused_wq_takes(c.M, c.N, b_is4)
+      and c.K % 256 == 0 and (c.K // gb) % 64 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0):
+    # symmetric int4 / int8: dequantized inside the GEMM's workgroups, slab by slab (the same bf16 weights, the
+    # same products in the same order, no dequantized copy of the weight in memory)
     out = torch.empty(c.M, c.N, dtype=res_t, device=dev)
-    _lib.call('qwix_hip_gemm_bf16_w4', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0), c.M, c.N, c.K, c.K // gb,
-              sb.data_ptr(), _lib.float_tag(sb.dtype), out.data_ptr(), _lib.float_tag(res_t), c.N, st)
+    _lib.call('qwix_hip_gemm_bf16_wq', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0),
+              _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
+              out.data_ptr(), _lib.float_tag(res_t), c.N, st)
     return out.reshape(c.out_shape)
   if fused_only:
     return None

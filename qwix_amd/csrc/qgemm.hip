@@ -2031,19 +2031,29 @@ __global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__
 // BN = 64 (tiles of 256 x 64, wavefronts of 64 x 32, 128 KB of LDS) is for calls whose 128-column tiles would leave
 // more than half of the CUs without a workgroup: a workgroup's time is mostly its MFMAs and the conversion, which
 // both halve, while its activation traffic stays.
-template <int OUT, bool SBF, int BN>
+// BITS = 8: int8 weights.  A row's 128-byte line would hold only two slabs, too few to request a buffer ahead, so
+// they come as 64-byte pieces, one slab per request (16 rows per load instruction), into a ring of four buffers:
+// slab kt + 3 is requested in slab kt, behind the activations of slab kt + 2.  With 64-column tiles the upper half of
+// a load instruction's lanes repeats the lower half's rows (every wavefront issues one load per slab, so that all
+// count their requests alike); the repeated rows land in padding.  A byte b holds q = (b ^ 0x80) - 128 and
+// q * scale = fma(b ^ 0x80, scale, -128 scale), exact as for the nibbles.
+template <int OUT, bool SBF, int BN, int BITS>
 __global__ void __launch_bounds__(512)
-    wgemm_w4_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ Q, int64_t ldq,
+    wgemm_wq_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ Q, int64_t ldq,
                     const void* __restrict__ S, int M, int N, int K, int group, uint8_t* __restrict__ out, int64_t ldo) {
   static_assert(BN == 128 || BN == 64, "column tiles of 128 or 64");
   constexpr int BM = 256, WGN = 2, WN = BN / WGN, TM = 2, TN = WN / 32, NWAVES = 8;
   constexpr int BK = 128, NK = 4;  // bytes of an activation row per slab (64 elements); k-steps of 16 elements
-  constexpr int A_STAGE = BM * BK, C_STAGE = BN * BK, R_STAGE = BN * 128;
-  constexpr int C_BASE = 3 * A_STAGE, R_BASE = C_BASE + 2 * C_STAGE, LDS_BYTES = R_BASE + 2 * R_STAGE;  // 160 / 128 KB
-  constexpr int NQ = BN / 64;       // direct-to-LDS loads of packed weights per wavefront and superslab (8 rows each)
+  static_assert(BITS == 4 || BITS == 8, "int4 or int8 weights");
+  constexpr bool W8 = BITS == 8;
+  // raw weights: int4 two buffers of a superslab (BN x 128 bytes), int8 four of a slab (8 x 1 KB, one per wavefront)
+  constexpr int A_STAGE = BM * BK, C_STAGE = BN * BK, R_STAGE = W8 ? 8 * 1024 : BN * 128;
+  constexpr int C_BASE = 3 * A_STAGE, R_BASE = C_BASE + 2 * C_STAGE, LDS_BYTES = R_BASE + (W8 ? 4 : 2) * R_STAGE;  // <= 160 KB
+  constexpr int NQ = W8 ? 1 : BN / 64;  // direct-to-LDS loads of weights per wavefront and request
   constexpr int TPR = 512 / BN;     // converter threads per weight row: 4 or 8
-  constexpr int NPT = 64 / TPR;     // nibbles per thread and slab: 16 or 8
+  constexpr int NPT = 64 / TPR;     // elements per thread and slab: 16 or 8
   constexpr int NCQ = NPT / 4;      // conversion steps of four elements: 4 or 2
+  constexpr int RPW = BN / 8;       // weight rows per wavefront: 16 or 8
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -2070,8 +2080,13 @@ __global__ void __launch_bounds__(512)
   }
 #pragma unroll
   for (int j = 0; j < NQ; ++j) {
-    const int row = wave * (8 * NQ) + j * 8 + lr;
-    goffq[j] = static_cast<uint32_t>(min(n0 + row, N - 1)) * static_cast<uint32_t>(ldq) + (((lane & 7) ^ swz8(row)) << 4);
+    if constexpr (W8) {  // 16 rows x 64 bytes per instruction (64-column tiles: 8 rows, twice)
+      const int row = wave * RPW + ((lane >> 2) & (RPW - 1));
+      goffq[j] = static_cast<uint32_t>(min(n0 + row, N - 1)) * static_cast<uint32_t>(ldq) + ((lane & 3) << 4);
+    } else {
+      const int row = wave * RPW + j * 8 + lr;
+      goffq[j] = static_cast<uint32_t>(min(n0 + row, N - 1)) * static_cast<uint32_t>(ldq) + (((lane & 7) ^ swz8(row)) << 4);
+    }
   }
   auto issue_a = [&](int kt, int stage) {  // 4 loads
     const uint8_t* gk = A + kt * BK;
@@ -2079,11 +2094,15 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
     for (int j = 0; j < 4; ++j) QWIX_GLDS16(gk + goffa[j], dst + j * 1024);
   };
-  auto issue_raw = [&](int ss) {  // NQ loads: elements 256 ss .. of 8 NQ weight rows
-    const uint8_t* gq = Q + ss * 128;
-    uint8_t* dst = smem + R_BASE + (ss & 1) * R_STAGE + wave * (8 * NQ) * 128;
+  auto issue_raw = [&](int ss) {  // int4: superslab ss (elements 256 ss ..), NQ loads; int8: slab ss, one load
+    if constexpr (W8) {
+      QWIX_GLDS16(Q + ss * 64 + goffq[0], smem + R_BASE + (ss & 3) * R_STAGE + wave * 1024);
+    } else {
+      const uint8_t* gq = Q + ss * 128;
+      uint8_t* dst = smem + R_BASE + (ss & 1) * R_STAGE + wave * RPW * 128;
 #pragma unroll
-    for (int j = 0; j < NQ; ++j) QWIX_GLDS16(gq + goffq[j], dst + j * 1024);
+      for (int j = 0; j < NQ; ++j) QWIX_GLDS16(gq + goffq[j], dst + j * 1024);
+    }
   };
 
   // ---- converter: thread -> (weight row, NPT of the slab's 64 elements)
@@ -2112,13 +2131,23 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
     for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(v[j]));
   };
-  int craw[NPT / 8];  // NPT / 2 bytes of the row's line: 32 bytes per slab, in two 16-byte chunks
+  constexpr int NRAW = NPT * BITS / 32;  // dwords of raw weights per thread and slab
+  int craw[NRAW];
   uint32_t cout[NPT / 2];
   auto convert_read = [&](int kt) {
-    const int byte = cpart * (NPT / 2);  // of the slab's 32
-    const int chunk = ((kt & 3) * 2 + (byte >> 4)) ^ swz8(crow);
-    const uint8_t* src = smem + R_BASE + ((kt >> 2) & 1) * R_STAGE + crow * 128 + (chunk << 4) + (byte & 15);
-    if constexpr (NPT == 16) {
+    const uint8_t* src;
+    if constexpr (W8) {  // the row's 64 bytes of this slab, NPT of them
+      src = smem + R_BASE + (kt & 3) * R_STAGE + (crow / RPW) * 1024 + (crow % RPW) * 64 + cpart * NPT;
+    } else {  // NPT / 2 bytes of the row's line: 32 bytes per slab, in two 16-byte chunks
+      const int byte = cpart * (NPT / 2);  // of the slab's 32
+      const int chunk = ((kt & 3) * 2 + (byte >> 4)) ^ swz8(crow);
+      src = smem + R_BASE + ((kt >> 2) & 1) * R_STAGE + crow * 128 + (chunk << 4) + (byte & 15);
+    }
+    if constexpr (NRAW == 4) {
+      const v4i v = *reinterpret_cast<const v4i*>(src);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) craw[e] = v[e];
+    } else if constexpr (NRAW == 2) {
       const qwix_v2i v = *reinterpret_cast<const qwix_v2i*>(src);
       craw[0] = v[0];
       craw[1] = v[1];
@@ -2131,7 +2160,18 @@ __global__ void __launch_bounds__(512)
   // byte of the masked word converts in one instruction.
   auto convert_quarter = [&](int q4, float sc) {  // elements 4 q4 .. 4 q4 + 3 of this thread's NPT
     if (q4 >= NCQ) return;
-    const uint32_t w = static_cast<uint32_t>(craw[q4 >> 1]) ^ 0x88888888u;
+    if constexpr (W8) {
+      const uint32_t u = static_cast<uint32_t>(craw[q4]) ^ 0x80808080u;
+      const float m128 = -128.f * sc;
+      const float f0 = __builtin_fmaf(static_cast<float>(u & 0xFFu), sc, m128);
+      const float f1 = __builtin_fmaf(static_cast<float>((u >> 8) & 0xFFu), sc, m128);
+      const float f2 = __builtin_fmaf(static_cast<float>((u >> 16) & 0xFFu), sc, m128);
+      const float f3 = __builtin_fmaf(static_cast<float>(u >> 24), sc, m128);
+      cout[2 * q4] = pack_bf16x2(f0, f1);
+      cout[2 * q4 + 1] = pack_bf16x2(f2, f3);
+      return;
+    }
+    const uint32_t w = static_cast<uint32_t>(craw[W8 ? 0 : q4 >> 1]) ^ 0x88888888u;
     const uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
     const int b0 = (q4 & 1) * 16;
     const float m8 = -8.f * sc;
@@ -2192,13 +2232,12 @@ __global__ void __launch_bounds__(512)
     constexpr int j = decltype(J)::value;
     constexpr bool last = decltype(LAST)::value;  // the last four slabs: nothing further to request after two
     constexpr bool more = !(last && j == 3);
-    constexpr bool loads_a = !last || j < 2, loads_w = !last && j == 0;
+    constexpr bool loads_a = !last || j < 2, loads_s = !last && j == 0;
+    constexpr bool loads_w = W8 ? (!last || j == 0) : loads_s;  // int8: slab kt + 3; int4: the next superslab
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (loads_a) issue_a(kt + 2, sta == 0 ? 2 : sta - 1);
-    if constexpr (loads_w) {
-      issue_raw((kt >> 2) + 1);
-      request_scales(sc_next);
-    }
+    if constexpr (loads_w) issue_raw(W8 ? kt + 3 : (kt >> 2) + 1);
+    if constexpr (loads_s) request_scales(sc_next);
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (j == 2 && !last) pin_scales(sc_next);  // requested at j == 0, covered by the wait that ended j == 1
     const float sc = scale_value(j == 3 ? sc_next[0] : sc_cur[(j + 1) & 3]);
@@ -2210,13 +2249,17 @@ __global__ void __launch_bounds__(512)
       mfma_step(ks & 1);
     }
     if constexpr (more) convert_write(kt + 1);
-    end_of_slab(integral_constant<int, (loads_a ? 4 : 0) + (loads_w ? NQ + 4 : 0)>{});
+    end_of_slab(integral_constant<int, (loads_a ? 4 : 0) + (loads_w ? NQ : 0) + (loads_s ? 4 : 0)>{});
     sta = sta == 2 ? 0 : sta + 1;
     if constexpr (more) read_frags(sta, (j + 1) & 1, 0, 0);
   };
 
-  // ---- prologue: packed weights and scales of slabs 0..3, activations of slabs 0 and 1; slab 0 converted
+  // ---- prologue: packed weights and scales of slabs 0..3 (int8: 0..2), activations of slabs 0 and 1; slab 0 converted
   issue_raw(0);
+  if constexpr (W8) {
+    issue_raw(1);
+    issue_raw(2);
+  }
   request_scales(sc_cur);
   issue_a(0, 0);
   issue_a(1, 1);
@@ -2485,20 +2528,23 @@ extern "C" int qwix_hip_gemm_bf16(const void* a, int64_t lda, const void* b, int
   return launch_dma<kOpBf16, 128, 128, 2, 2, QWIX_F32, 0>(a, ldab, b, ldbb, M, N, kb, ep, out, ldo, st);
 }
 
-extern "C" int qwix_hip_gemm_bf16_w4(const void* a, int64_t lda, const void* q, int64_t ldq_bytes, int64_t M, int64_t N,
-                                     int64_t K, int64_t group, const void* s, int s_dtype, void* out, int out_dtype,
-                                     int64_t ldo, void* stream) {
+extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, int64_t ldq_bytes, int q_qtype, int64_t M,
+                                     int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, void* out,
+                                     int out_dtype, int64_t ldo, void* stream) {
   if (!a || !q || !s || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/q/s/out");
+  if (q_qtype != QWIX_INT4 && q_qtype != QWIX_INT8)
+    return fail(QWIX_ERR_UNSUPPORTED, "weight qtype %d: int4 or int8", q_qtype);
   if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || 2 * K > INT32_MAX)
     return fail(QWIX_ERR_INVALID_ARGUMENT, "bad GEMM shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
                 (long long)K);
   if ((out_dtype != QWIX_BF16 && out_dtype != QWIX_F32) || (s_dtype != QWIX_BF16 && s_dtype != QWIX_F32))
     return fail(QWIX_ERR_INVALID_ARGUMENT, "scale and output dtypes must be f32 or bf16");
-  // K in whole 128-byte lines of packed weights (256 elements); a scale group covers whole 64-element slabs
+  // K in groups of four 64-element slabs (for int4 a 128-byte line of packed weights); a scale group covers whole slabs
   if (K % 256 || group <= 0 || group % 64 || K % group)
     return fail(QWIX_ERR_UNSUPPORTED, "K=%lld must be a multiple of 256 and group=%lld a multiple of 64 that divides K",
                 (long long)K, (long long)group);
-  if (lda % 8 || lda < K || ldq_bytes % 16 || ldq_bytes < K / 2 || !aligned16(a) || !aligned16(q))
+  const int64_t row_bytes = q_qtype == QWIX_INT4 ? K / 2 : K;
+  if (lda % 8 || lda < K || ldq_bytes % 16 || ldq_bytes < row_bytes || !aligned16(a) || !aligned16(q))
     return fail(QWIX_ERR_UNSUPPORTED, "activation and weight rows must be 16-byte aligned (lda=%lld ldq=%lld)",
                 (long long)lda, (long long)ldq_bytes);
   if (ldo < N || !aligned16(out) || (N % 4 == 0 && ldo % 4 != 0))
@@ -2508,10 +2554,11 @@ extern "C" int qwix_hip_gemm_bf16_w4(const void* a, int64_t lda, const void* q, 
   // 64-column tiles while 128-column ones would occupy at most half of the CUs
   const bool narrow = ((M + 255) / 256) * ((N + 127) / 128) <= 128;
   hipStream_t st = static_cast<hipStream_t>(stream);
-#define QWIX_W4_LAUNCH(OUTT, SBFF, BNN)                                                                              \
+#define QWIX_WQ_LAUNCH(OUTT, SBFF, BNN, BITS)                                                                        \
   do {                                                                                                               \
-    auto kern = wgemm_w4_kernel<OUTT, SBFF, BNN>;                                                                    \
-    constexpr size_t smem = 3 * 256 * 128 + 2 * BNN * 128 + 2 * BNN * 128;  /* 160 KB, all of a CU's, or 128 KB */   \
+    auto kern = wgemm_wq_kernel<OUTT, SBFF, BNN, BITS>;                                                              \
+    /* activations 96 KB, converted weights 2 x BN x 128, raw weights 2 x BN x 128 (int8: 4 x 8 KB): <= 160 KB */    \
+    constexpr size_t smem = 3 * 256 * 128 + 2 * BNN * 128 + (BITS == 8 ? 4 * 8192 : 2 * BNN * 128);                  \
     const dim3 grid(static_cast<unsigned>(((M + 255) / 256) * ((N + BNN - 1) / BNN)));                               \
     static LdsGrant granted;                                                                                         \
     if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;                           \
@@ -2519,18 +2566,23 @@ extern "C" int qwix_hip_gemm_bf16_w4(const void* a, int64_t lda, const void* q, 
                                   static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), static_cast<int>(group), \
                                   static_cast<uint8_t*>(out), ldo);                                                  \
   } while (0)
-#define QWIX_W4_PICK(OUTT, SBFF)                                                                                     \
+#define QWIX_WQ_TILE(OUTT, SBFF, BITS)                                                                               \
   do {                                                                                                               \
-    if (narrow) QWIX_W4_LAUNCH(OUTT, SBFF, 64); else QWIX_W4_LAUNCH(OUTT, SBFF, 128);                                \
+    if (narrow) QWIX_WQ_LAUNCH(OUTT, SBFF, 64, BITS); else QWIX_WQ_LAUNCH(OUTT, SBFF, 128, BITS);                    \
+  } while (0)
+#define QWIX_WQ_BITS(OUTT, SBFF)                                                                                     \
+  do {                                                                                                               \
+    if (q_qtype == QWIX_INT4) QWIX_WQ_TILE(OUTT, SBFF, 4); else QWIX_WQ_TILE(OUTT, SBFF, 8);                         \
   } while (0)
   if (out_dtype == QWIX_BF16) {
-    if (s_dtype == QWIX_BF16) QWIX_W4_PICK(QWIX_BF16, true); else QWIX_W4_PICK(QWIX_BF16, false);
+    if (s_dtype == QWIX_BF16) QWIX_WQ_BITS(QWIX_BF16, true); else QWIX_WQ_BITS(QWIX_BF16, false);
   } else {
-    if (s_dtype == QWIX_BF16) QWIX_W4_PICK(QWIX_F32, true); else QWIX_W4_PICK(QWIX_F32, false);
+    if (s_dtype == QWIX_BF16) QWIX_WQ_BITS(QWIX_F32, true); else QWIX_WQ_BITS(QWIX_F32, false);
   }
-#undef QWIX_W4_PICK
-#undef QWIX_W4_LAUNCH
-  return check_launch("gemm_bf16_w4");
+#undef QWIX_WQ_BITS
+#undef QWIX_WQ_TILE
+#undef QWIX_WQ_LAUNCH
+  return check_launch("gemm_bf16_wq");
 }
 
 extern "C" int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M,

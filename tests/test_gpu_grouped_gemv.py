@@ -373,31 +373,34 @@ def test_bf16_gemm_against_float64(M, K, N, out_dtype):
 
 @pytest.mark.parametrize('sdt', [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
 @pytest.mark.parametrize('M,K,N,group', [(300, 256, 136, 128), (512, 1024, 1000, 256), (257, 2048, 520, 64), (2048, 4096, 1536, 128),
                                          (1, 512, 64, 512), (600, 512, 8400, 128), (1100, 256, 4100, 64)])
-def test_int4_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, out_dtype, sdt):
-  """qwix_hip_gemm_bf16_w4 through the C ABI == qwix_hip_dequantize_rm (to bf16) + qwix_hip_gemm_bf16, bit for bit: the
-  same bf16 weights, the same MFMA, K walked in the same order; edges in M and N, one slab group (64), several; the
-  last two shapes have more than 128 tiles of 256 x 128 and run those, the others tiles of 256 x 64."""
+def test_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, wq_type, out_dtype, sdt):
+  """qwix_hip_gemm_bf16_wq through the C ABI == qwix_hip_dequantize_rm (to bf16) + qwix_hip_gemm_bf16, bit for bit: the
+  same bf16 weights, the same MFMA, K walked in the same order; int4 and int8 weights, edges in M and N, one slab
+  group (64), several; the last two shapes have more than 128 tiles of 256 x 128 and run those, the others tiles of
+  256 x 64."""
   from qwix_amd import _lib
   from qwix_amd.core import qarray
-  print('case w4 prefill', M, K, N, group, out_dtype, sdt, flush=True)
+  print('case wq prefill', M, K, N, group, wq_type, out_dtype, sdt, flush=True)
   x_np, x_t = util.make((M, K), O.BF16, seed=M + K + 21)
   w_np, w_t = util.make((K, N), O.BF16, seed=N + K + 22, scale=0.02)
-  wq = qarray.quantize_api(w_t, 'int4', channelwise_axes=[1], tiled_axes={0: group}, scale_dtype=sdt)
+  wq = qarray.quantize_api(w_t, wq_type, channelwise_axes=[1], tiled_axes={0: group}, scale_dtype=sdt)
   from qwix_amd.core import dot_general as dg
   c = dg._Canon(x_t, wq, DN)
   b, is4 = c.rhs_values(wq)
   sb, gb = c.rhs_scale(wq)
-  assert is4 and gb == K // group
+  assert is4 == (wq_type == 'int4') and gb == K // group
+  tag = _lib.INT4 if is4 else _lib.INT8
   st = _lib.stream_of(x_t)
   w = torch.empty(N, K, dtype=torch.bfloat16, device=util.DEV)
-  _lib.call('qwix_hip_dequantize_rm', b.data_ptr(), _lib.INT4, 1, K, N, group, sb.data_ptr(), None, _lib.float_tag(sb.dtype),
+  _lib.call('qwix_hip_dequantize_rm', b.data_ptr(), tag, 1, K, N, group, sb.data_ptr(), None, _lib.float_tag(sb.dtype),
             w.data_ptr(), _lib.BF16, st)
   want = torch.empty(M, N, dtype=out_dtype, device=util.DEV)
   _lib.call('qwix_hip_gemm_bf16', x_t.data_ptr(), K, w.data_ptr(), K, M, N, K, want.data_ptr(), _lib.float_tag(out_dtype), N, st)
   got = torch.full((M, N), float('nan'), dtype=out_dtype, device=util.DEV)
-  _lib.call('qwix_hip_gemm_bf16_w4', x_t.data_ptr(), K, b.data_ptr(), b.stride(0), M, N, K, group, sb.data_ptr(),
+  _lib.call('qwix_hip_gemm_bf16_wq', x_t.data_ptr(), K, b.data_ptr(), b.stride(0), tag, M, N, K, group, sb.data_ptr(),
             _lib.float_tag(sb.dtype), got.data_ptr(), _lib.float_tag(out_dtype), N, st)
   torch.cuda.synchronize()
   assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
@@ -440,7 +443,7 @@ def test_weight_only_prefill_on_hip_kernels(M, K, N, case):
   assert np.allclose(got, want.v, rtol=1e-2, atol=1e-2 * np.abs(want.v).mean()), np.abs(got - want.v).max()
   # the operator takes this path beyond the decode kernel's rows, for the operand kinds that kernel does not take, and
   # for symmetric int4 from the row count on at which the dequantizing tile GEMM wins
-  if M > dg.WEIGHT_ONLY_MAX_ROWS or fit is None or (wq_type == 'int4' and M > dg.fused_w4_min_rows(N)):
+  if M > dg.WEIGHT_ONLY_MAX_ROWS or fit is None or (wq_type in ('int4', 'int8') and M > dg.fused_wq_min_rows(N, wq_type == 'int4')):
     assert torch.equal(dg.dot_general(x_t, wq, DN, preferred_element_type=torch.bfloat16), out)
   # the dequantized operand itself, against the oracle's dequantize
   c = dg._Canon(x_t, wq, DN)
