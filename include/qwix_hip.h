@@ -267,6 +267,22 @@ QWIX_API int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b, i
                            int sb_dtype, void* out, int out_dtype, int64_t ldo, int exact,
                            int32_t* acc_out, void* stream);
 
+/* Hadamard rotation + activation quantize + sub-channel GEMM in one call: the functional content of
+ * hadamard_quantize_multiply (qwix/contrib/kernels/fused_hadamard_quantized_matmul.py:349-414) with the numerics
+ * of the unfused path (hadamard_rot.py:133-190, quantize, _fast_dot_general with tiled weights):
+ *     xq, sa = quantize_int8( ((x * pre_sign) H_K) * post_sign * out_scale, tile = act_tile along K )
+ *     out    = qwix_hip_qgemm_grouped(xq, b, sa, sb, exact = 0)
+ * x (M, K) of x_dtype, dense rows; act_tile = K (one scale per token) or = group; b, sb, group, out as in
+ * qwix_hip_qgemm_grouped.  workspace: qwix_hip_qgemm_hadamard_act_workspace_bytes(M, K, act_tile, x_dtype) bytes of
+ * device memory, 16-byte aligned (the int8 rows and their scales; nothing is allocated).  Two kernels on the
+ * stream; bit-identical to qwix_hip_fwht_quantize followed by qwix_hip_qgemm_grouped. */
+QWIX_API size_t qwix_hip_qgemm_hadamard_act_workspace_bytes(int64_t M, int64_t K, int64_t act_tile, int x_dtype);
+QWIX_API int qwix_hip_qgemm_hadamard_act(const void* x, int x_dtype, int64_t M, int64_t N, int64_t K, const void* pre_sign,
+                                const void* post_sign, float out_scale, int64_t act_tile, const void* b,
+                                int64_t ldb_bytes, int b_qtype, int64_t group, const void* sb, int sb_dtype,
+                                void* out, int out_dtype, int64_t ldo, void* workspace, size_t workspace_bytes,
+                                void* stream);
+
 /* Sub-channel GEMM with one asymmetric operand.  Replaces the zero-point terms of _fast_dot_general when a
  * contracting axis is tiled (qwix/_src/core/dot_general.py:196-203: the zero point is split with the tiles;
  * :228-253: the correction dot is subtracted from every tile's int32 partial before it is scaled):

@@ -120,3 +120,33 @@ def _inverse_movedim(ndim: int, dim: int) -> tuple[int, ...]:
   order = list(range(ndim - 1))
   order.insert(dim, ndim - 1)
   return tuple(order)
+
+
+def hadamard_quantized_matmul(act: torch.Tensor, weight: qarray.QArray, pre_sign=None, post_sign=None, *,
+                              act_tile: int | None = None, preferred_element_type=None) -> torch.Tensor:
+  """quantize_int8(fwht(act)) @ weight in one library call: the counterpart of `hadamard_quantize_multiply`
+  (qwix/contrib/kernels/fused_hadamard_quantized_matmul.py:349-414) with the numerics of `rotate_and_quantize`
+  followed by the sub-channel quantized dot (dot_general.py:186-203,255-260).
+
+  act: (M, K) bf16 / f32, K a power of two; weight: a symmetric int8 / int4 QArray of logical shape (K, N) with
+  scales per output channel and group of `group` rows (tiles along K only), K-contiguous storage as
+  `quantize(..., reduce-minor)` writes it; act_tile: None = one scale per token, else the weight's group."""
+  from qwix_amd.core import dot_general as dg
+  if act.ndim != 2 or not isinstance(weight, qarray.QArray) or weight.zero_point is not None:
+    raise NotImplementedError('hadamard_quantized_matmul takes a 2-D activation and a symmetric quantized weight')
+  dn = (((1,), (0,)), ((), ()))
+  c = dg._Canon(act, weight, dn)
+  b, b_is4 = c.rhs_values(weight)
+  sb, gb = c.rhs_scale(weight)
+  group = c.K // gb
+  tile = c.K if act_tile is None else int(act_tile)
+  x = act if act.is_contiguous() else act.contiguous()
+  res_t = preferred_element_type or act.dtype
+  need = _lib.load().qwix_hip_qgemm_hadamard_act_workspace_bytes(c.M, c.K, tile, _lib.float_tag(x.dtype))
+  ws = torch.empty(max(int(need), 16), dtype=torch.uint8, device=x.device)
+  out = torch.empty(c.M, c.N, dtype=res_t, device=x.device)
+  _lib.call('qwix_hip_qgemm_hadamard_act', x.data_ptr(), _lib.float_tag(x.dtype), c.M, c.N, c.K, _lib.ptr(pre_sign),
+            _lib.ptr(post_sign), 1.0, tile, b.data_ptr(), b.stride(0), _lib.INT4 if b_is4 else _lib.INT8, group,
+            sb.data_ptr(), _lib.float_tag(sb.dtype), out.data_ptr(), _lib.float_tag(res_t), c.N, ws.data_ptr(), int(need),
+            _lib.stream_of(x))
+  return out

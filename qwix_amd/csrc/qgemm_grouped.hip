@@ -912,3 +912,40 @@ extern "C" int qwix_hip_qgemm_grouped_zp(const void* a, int64_t lda, const void*
   return grouped_impl(a, lda, b, ldb_bytes, b_qtype, M, N, K, group, sa, sa_dtype, ga, sb, sb_dtype, zu, zu_row_stride,
                       zu_group_stride, zv, zv_col_stride, zv_group_stride, out, out_dtype, ldo, exact, acc_out, stream);
 }
+
+// Rotate, quantize, multiply in one call (the functional content of the reference's fused Hadamard kernel,
+// qwix/contrib/kernels/fused_hadamard_quantized_matmul.py:349-414, with the numerics of the unfused path:
+// hadamard_rot.py:133-190, then quantize, then _fast_dot_general): the rotation + per-token or per-group quantize kernel
+// writes int8 rows and their scales into the caller's workspace, the sub-channel GEMM reads them.  Bit-identical to
+// qwix_hip_fwht_quantize followed by qwix_hip_qgemm_grouped.
+static size_t had_align(size_t v) { return (v + 255) & ~size_t{255}; }
+
+extern "C" size_t qwix_hip_qgemm_hadamard_act_workspace_bytes(int64_t M, int64_t K, int64_t act_tile, int x_dtype) {
+  if (M <= 0 || K <= 0 || act_tile <= 0 || K % act_tile) return 0;
+  const size_t es = x_dtype == QWIX_BF16 ? 2 : 4;
+  return had_align(static_cast<size_t>(M) * K) + had_align(static_cast<size_t>(M) * (K / act_tile) * es);
+}
+
+extern "C" int qwix_hip_qgemm_hadamard_act(const void* x, int x_dtype, int64_t M, int64_t N, int64_t K, const void* pre_sign,
+                                           const void* post_sign, float out_scale, int64_t act_tile, const void* b,
+                                           int64_t ldb_bytes, int b_qtype, int64_t group, const void* sb, int sb_dtype,
+                                           void* out, int out_dtype, int64_t ldo, void* workspace, size_t workspace_bytes,
+                                           void* stream) {
+  if (!x || !b || !sb || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null x/b/sb/out");
+  if (M <= 0 || N <= 0 || K <= 0 || group <= 0)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "bad shape M=%lld N=%lld K=%lld group=%lld", (long long)M, (long long)N,
+                (long long)K, (long long)group);
+  // the activations carry one scale per token (act_tile == K) or one per token and weight group
+  if (act_tile != K && act_tile != group)
+    return fail(QWIX_ERR_UNSUPPORTED, "activation tile %lld: K (per token) or the weight's group %lld", (long long)act_tile,
+                (long long)group);
+  const size_t need = qwix_hip_qgemm_hadamard_act_workspace_bytes(M, K, act_tile, x_dtype);
+  if (need == 0 || !workspace || workspace_bytes < need || !aligned16(workspace))
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "workspace of %zu bytes required, got %zu", need, workspace_bytes);
+  uint8_t* q = static_cast<uint8_t*>(workspace);
+  uint8_t* sa = q + had_align(static_cast<size_t>(M) * K);
+  if (int e = qwix_hip_fwht_quantize(x, x_dtype, M, K, pre_sign, post_sign, out_scale, act_tile, QWIX_INT8, q, sa, stream))
+    return e;
+  return qwix_hip_qgemm_grouped(q, K, b, ldb_bytes, b_qtype, M, N, K, group, sa, x_dtype, K / act_tile, sb, sb_dtype, out,
+                                out_dtype, ldo, 0, nullptr, stream);
+}

@@ -109,6 +109,34 @@ def test_weight_side_fused_rotation_feeds_the_grouped_gemm():
   assert np.abs(got - ref).mean() / np.abs(ref).mean() < 0.15
 
 
+@pytest.mark.parametrize('M,K,N,wq_type,group,per_group_act,dtype', [
+    (64, 1024, 256, 'int4', 128, False, torch.bfloat16), (200, 2048, 520, 'int8', 256, False, torch.bfloat16),
+    (33, 512, 136, 'int4', 128, True, torch.bfloat16), (16, 1024, 128, 'int8', 128, False, torch.float32)])
+def test_rotate_quantize_multiply_in_one_call(M, K, N, wq_type, group, per_group_act, dtype):
+  """qwix_hip_qgemm_hadamard_act through the C ABI (hadamard_quantized_matmul) == rotate_and_quantize followed by the
+  sub-channel quantized dot, bit for bit; the latter is held to the oracle by the test above."""
+  from qwix_amd.contrib import hadamard_rot as hr
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  print('case hadamard one call', M, K, N, wq_type, group, per_group_act, dtype, flush=True)
+  x_np, x_t = util.make((M, K), O.BF16 if dtype == torch.bfloat16 else O.F32, seed=M + K)
+  w_np, w_t = util.make((K, N), O.BF16, seed=N + K, scale=0.02)
+  g = util.rng(5)
+  s_t = torch.from_numpy(g.choice([-1.0, 1.0], K).astype(np.float32)).to(dtype).to(util.DEV)
+  wq = hr.rotate_and_quantize(w_t, 0, qarray.HowToQuantize(qtype=wq_type, channelwise_axes=[1], tiled_axes={0: group}),
+                              pre_sign=s_t.to(torch.bfloat16), out_scale=1.0 / K)
+  how_x = qarray.HowToQuantize(qtype='int8', channelwise_axes=[0], tiled_axes={1: group} if per_group_act else {})
+  xq = hr.rotate_and_quantize(x_t, 1, how_x, pre_sign=s_t)
+  want = dg.dot_general(xq, wq, (((1,), (0,)), ((), ())))
+  got = hr.hadamard_quantized_matmul(x_t, wq, pre_sign=s_t, act_tile=group if per_group_act else None,
+                                     preferred_element_type=want.dtype)
+  torch.cuda.synchronize()
+  assert got.dtype == want.dtype and torch.equal(got, want), float((got.float() - want.float()).abs().max())
+  # and the product it stands for
+  ref = x_np.astype(np.float64) @ w_np.astype(np.float64)
+  assert np.abs(util.f32np(got) - ref).mean() / np.abs(ref).mean() < 0.2
+
+
 def test_fwht_errors():
   from qwix_amd.contrib import hadamard_rot as hr
   with pytest.raises(ValueError, match='power of 2'):
