@@ -137,6 +137,31 @@ def test_rotate_quantize_multiply_in_one_call(M, K, N, wq_type, group, per_group
   assert np.abs(util.f32np(got) - ref).mean() / np.abs(ref).mean() < 0.2
 
 
+def test_rotate_quantize_multiply_argument_checks():
+  """The one-call entry point refuses a missing or short scratch buffer and activation tiles that are neither the
+  whole row nor the weight's group."""
+  from qwix_amd import _lib
+  L = _lib.load()
+  M, N, K, G = 32, 128, 512, 128
+  x = torch.zeros(M, K, dtype=torch.bfloat16, device=util.DEV)
+  b = torch.zeros(N, K, dtype=torch.int8, device=util.DEV)
+  sb = torch.ones(K // G, N, dtype=torch.bfloat16, device=util.DEV)
+  out = torch.empty(M, N, dtype=torch.bfloat16, device=util.DEV)
+  need = L.qwix_hip_qgemm_hadamard_act_workspace_bytes(M, K, K, _lib.BF16)
+  assert need >= M * K + 2 * M
+  assert L.qwix_hip_qgemm_hadamard_act_workspace_bytes(M, K, G, _lib.BF16) >= M * K + 2 * M * (K // G)
+  assert L.qwix_hip_qgemm_hadamard_act_workspace_bytes(M, K, 96, _lib.BF16) == 0
+  ws = torch.empty(need, dtype=torch.uint8, device=util.DEV)
+  def call(tile=K, wsp=ws.data_ptr(), nws=need):
+    return L.qwix_hip_qgemm_hadamard_act(x.data_ptr(), _lib.BF16, M, N, K, None, None, 1.0, tile, b.data_ptr(), K, _lib.INT8, G,
+                                         sb.data_ptr(), _lib.BF16, out.data_ptr(), _lib.BF16, N, wsp, nws, None)
+  assert call() == 0
+  assert call(wsp=None, nws=0) != 0 and b'workspace' in L.qwix_hip_last_error()
+  assert call(nws=need - 1) != 0
+  assert call(tile=256) != 0 and b'activation tile' in L.qwix_hip_last_error()
+  torch.cuda.synchronize()
+
+
 def test_fwht_errors():
   from qwix_amd.contrib import hadamard_rot as hr
   with pytest.raises(ValueError, match='power of 2'):

@@ -409,6 +409,31 @@ def test_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, wq_type, out_dty
   assert torch.allclose(got.double(), ref, rtol=1e-2 if out_dtype == torch.bfloat16 else 1e-4, atol=1e-2 * float(ref.abs().mean()))
 
 
+def test_dequantizing_gemm_argument_checks():
+  """qwix_hip_gemm_bf16_wq refuses what its tile loop cannot walk (K not in whole groups of four slabs, groups that
+  are not whole slabs, unaligned rows, other weight types) with an error code and a message instead of launching."""
+  from qwix_amd import _lib
+  L = _lib.load()
+  M, N, K = 64, 128, 512
+  x = torch.zeros(M, K, dtype=torch.bfloat16, device=util.DEV)
+  q = torch.zeros(N, K, dtype=torch.int8, device=util.DEV)
+  s = torch.ones(K // 128, N, dtype=torch.bfloat16, device=util.DEV)
+  out = torch.empty(M, N, dtype=torch.bfloat16, device=util.DEV)
+  def call(lda=K, ldq=K, qt=_lib.INT8, k=K, group=128, sd=_lib.BF16, od=_lib.BF16, ldo=N):
+    return L.qwix_hip_gemm_bf16_wq(x.data_ptr(), lda, q.data_ptr(), ldq, qt, M, N, k, group, s.data_ptr(), sd, out.data_ptr(),
+                                   od, ldo, None)
+  assert call() == 0
+  assert call(qt=_lib.INT4, ldq=K // 2) == 0
+  assert call(qt=_lib.E4M3) != 0 and b'int4 or int8' in L.qwix_hip_last_error()
+  assert call(k=384) != 0 and b'multiple of 256' in L.qwix_hip_last_error()
+  assert call(group=96) != 0 and b'multiple of 64' in L.qwix_hip_last_error()
+  assert call(ldq=K // 2) != 0 and b'aligned' in L.qwix_hip_last_error()       # int8 rows need K bytes
+  assert call(lda=K + 4) != 0
+  assert call(ldo=N - 8) != 0 and b'leading dimension' in L.qwix_hip_last_error()
+  assert call(od=99) != 0 and call(sd=99) != 0
+  torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize('case', [('int4', 128, False, torch.float32), ('int8', 128, False, torch.bfloat16),
                                   ('int4', 256, True, torch.bfloat16), ('int8', None, True, torch.float32),
                                   ('float8_e4m3fn', None, False, torch.bfloat16)])
