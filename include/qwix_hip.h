@@ -343,6 +343,14 @@ QWIX_API int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64_t
                      int64_t M, int64_t N, int64_t K, int64_t group, const void* s,
                      int s_dtype, void* out, int out_dtype, int64_t ldo, void* stream);
 
+/* The same with asymmetric weights (calibration by min/max: dequantize is (q - zero_point) * scale,
+ * qarray.py:692-708): out[m,n] = sum_k x[m,k] * ((q[k,n] - zp[k/group, n]) * s[k/group, n]).  zp: int8,
+ * (K/group, N) row-major like s.  The zero point leaves through the row sums of x per group:
+ * sum_k x (q - zp) = sum_k x q - zp sum_k x, in f32. */
+QWIX_API int qwix_hip_gemv_wq_zp(const void* x, int64_t ldx, const void* q, int64_t ldb_bytes, int b_qtype,
+                        int64_t M, int64_t N, int64_t K, int64_t group, const void* s, int s_dtype,
+                        const int8_t* zp, void* out, int out_dtype, int64_t ldo, void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * Walsh-Hadamard rotation along the last axis (qwix/contrib/hadamard_rot.py:35-117):
  *     y[r, :] = ((x[r, :] * pre_sign) H_n) * post_sign * out_scale

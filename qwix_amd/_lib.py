@@ -56,6 +56,7 @@ SIGNATURES = {
     'qwix_hip_gemm_bf16_wq': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _vp, _int, _i64, _vp]),
     'qwix_hip_dequantize_rm': (_int, [_vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _int, _vp, _int, _vp]),
     'qwix_hip_gemv_wq': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _vp, _int, _i64, _vp]),
+    'qwix_hip_gemv_wq_zp': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _int, _i64, _vp]),
     'qwix_hip_fwht': (_int, [_vp, _int, _i64, _i64, _vp, _vp, _f32, _vp, _vp]),
     'qwix_hip_fwht_quantize': (_int, [_vp, _int, _i64, _i64, _vp, _vp, _f32, _i64, _int, _vp, _vp, _vp]),
 }

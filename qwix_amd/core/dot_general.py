@@ -19,6 +19,7 @@ from __future__ import annotations
 
 import functools
 import math
+import weakref
 from typing import Any, Mapping, Sequence
 
 import torch
@@ -494,15 +495,36 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   return (out, acc.reshape((ngroups,) + c.out_shape)) if return_accumulators else out
 
 
+# The zero points of a weight in the form the weight-only kernels read ((groups, N) int8, contiguous), kept per
+# zero-point tensor and operand order: weights are static, and re-laying them out costs three small launches,
+# more than the decode kernel itself takes.
+_ZP8_CACHE: dict = {}
+
+
+def _rhs_zero_point_i8(c: '_Canon', rhs: QArray) -> tuple[torch.Tensor, int]:
+  z = rhs.zero_point
+  key = (id(z), tuple(c.rca), tuple(c.rfree))
+  hit = _ZP8_CACHE.get(key)
+  if hit is not None and hit[0]() is z and hit[1] == z._version:
+    return hit[2], hit[3]
+  z32, gz = c.rhs_zero_point(rhs)
+  zp = z32.to(torch.int8).contiguous()
+  _ZP8_CACHE[key] = (weakref.ref(z, lambda _, k=key: _ZP8_CACHE.pop(k, None)), z._version, zp, gz)
+  return zp, gz
+
+
 def _weight_only_fit(lhs, rhs, dimension_numbers):
   """The canonical form when the fused weight-only kernels (dequantize in registers, bf16 MFMA) take this pair,
-  else None.  The conditions are the kernels' own: a bf16 activation, a symmetric int4/int8 weight whose
-  scales are tiled along the last contracting axis only, in groups that are multiples of 128."""
+  else None.  The conditions are the kernels' own: a bf16 activation, an int4/int8 weight whose scales (and zero
+  points, if any, in the same groups) are tiled along the last contracting axis only, in groups that are
+  multiples of 128."""
   if not (_is_float_array(lhs) and lhs.dtype == torch.bfloat16 and isinstance(rhs, QArray)):
     return None
-  if rhs.zero_point is not None or _qtype_of(rhs) not in (numerics.INT4, numerics.INT8):
+  if _qtype_of(rhs) not in (numerics.INT4, numerics.INT8):
     return None
   c = _Canon(lhs, rhs, dimension_numbers)
+  if rhs.zero_point is not None and tuple(rhs.zero_point.shape) != tuple(rhs.scale.shape):
+    return None
   if any(rhs.scale.shape[a] != 1 for a in c.rca[:-1]):
     return None
   gb = rhs.scale.shape[c.rca[-1]]
@@ -530,7 +552,8 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   if len(dimension_numbers[1][0]) or len(dimension_numbers[1][1]):
     return _over_batch(_slow_dot_general, lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type)
   c = _weight_only_fit(lhs, rhs, dimension_numbers)
-  if c is not None and fused_wq_min_rows(c.N, isinstance(rhs.qvalue, Int4Tensor)) < c.M <= WEIGHT_ONLY_MAX_ROWS:
+  if (c is not None and rhs.zero_point is None
+      and fused_wq_min_rows(c.N, isinstance(rhs.qvalue, Int4Tensor)) < c.M <= WEIGHT_ONLY_MAX_ROWS):
     # one row tile of the dequantizing tile GEMM beats the decode kernel from here on
     out = _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type, fused_only=True)
     if out is not None:
@@ -541,6 +564,12 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
     b, b_is4 = c.rhs_values(rhs)
     res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.scale.dtype)
     out = torch.empty(c.M, c.N, dtype=res_t, device=x.device)
+    if rhs.zero_point is not None:  # asymmetric weights: (q - zp) * scale, the zero point per group and column
+      zp, _ = _rhs_zero_point_i8(c, rhs)
+      _lib.call('qwix_hip_gemv_wq_zp', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0),
+                _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
+                zp.data_ptr(), out.data_ptr(), _lib.float_tag(res_t), c.N, _lib.stream_of(x))
+      return out.reshape(c.out_shape)
     _lib.call('qwix_hip_gemv_wq', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0),
               _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
               out.data_ptr(), _lib.float_tag(res_t), c.N, _lib.stream_of(x))
@@ -610,10 +639,9 @@ def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_ty
   sb, _ = c.rhs_scale(rhs)
   zp = None
   if rhs.zero_point is not None:
-    z, gz = c.rhs_zero_point(rhs)
+    zp, gz = _rhs_zero_point_i8(c, rhs)
     if gz != gb:
       return None
-    zp = z.to(torch.int8)
   dev, st = x.device, _lib.stream_of(x)
   res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.scale.dtype)
   if res_t not in (torch.bfloat16, torch.float32):

@@ -30,6 +30,7 @@ struct GemvArgs {
   int bpg;         // 128-wide K blocks per scale group
   uint64_t magic;  // ceil(2^32 / bpg): kb / bpg == (kb * magic) >> 32 while kb * bpg < 2^32
   const void* s; int s_dtype;
+  const int8_t* zp;  // zero points (K / group, N) like the scales, or null (symmetric weights)
   void* out; int out_dtype; int64_t ldo;
 };
 
@@ -42,6 +43,7 @@ struct Block {
   v4u xf[RT][4];  // RT tiles of 16 rows of x
   v4u wq[NT][BQT == QWIX_INT4 ? 1 : 2];
   unsigned sraw[NT];  // scale bits as loaded: bf16 in the low half, or f32
+  unsigned zraw[NT];  // zero point as loaded (one byte, zero-extended); only with asymmetric weights
 };
 
 // Every load is a buffer load: a wave-uniform descriptor (the operand's first byte for this workgroup) plus a
@@ -58,6 +60,7 @@ struct LaneOff {
   unsigned f[2];       // bytes from the start of a 16-row tile in the wavefront's LDS panel, per K block
   uint8_t* panel;      // the wavefront's LDS panel: 16 * NT rows of 128 bytes
   const void *bx, *bw, *bs;  // wave-uniform: x from row row0, weights from row n_base, scales from column n_base
+  const void* bz;            // zero points from column n_base (asymmetric weights)
 };
 
 // How the weight bytes are requested decides the speed of this kernel.  The memory side works in 128-byte lines;
@@ -86,7 +89,7 @@ __device__ __forceinline__ void fetch_panel(const GemvArgs& p, const void* bw, u
 }
 
 // Activations and scales of one or two consecutive K blocks, and (WEIGHTS) the weights straight into registers.
-template <int BQT, int NT, bool SBF, int RT, bool TWO, bool WEIGHTS>
+template <int BQT, int NT, bool SBF, int RT, bool TWO, bool WEIGHTS, bool ZP>
 __device__ __forceinline__ void load_blocks(const GemvArgs& p, const LaneOff<NT>& a, const bool (&xrow)[RT], int kb,
                                             Block<BQT, NT, RT>* b0, Block<BQT, NT, RT>* b1) {
   constexpr bool W4 = (BQT == QWIX_INT4);
@@ -121,6 +124,11 @@ __device__ __forceinline__ void load_blocks(const GemvArgs& p, const LaneOff<NT>
       else
         b[h]->sraw[t] = __builtin_amdgcn_raw_buffer_load_b32(rs, a.s[t], s0, 0);
     }
+    if constexpr (ZP) {
+      const auto rz = buffer_from(a.bz);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) b[h]->zraw[t] = __builtin_amdgcn_raw_buffer_load_b8(rz, a.s[t] / (SBF ? 2u : 4u), sg * p.N, 0);
+    }
   }
   if constexpr (WEIGHTS) {
     const int wk = kb * (W4 ? 64 : 128);
@@ -142,8 +150,10 @@ __device__ __forceinline__ void load_blocks(const GemvArgs& p, const LaneOff<NT>
 // the offset times the row sum of x is taken out by four MFMAs against the constant -offset, whose
 // result seeds the accumulator of every column tile.  A widened weight fragment serves all RT row tiles; every
 // output element sees the same operations in the same order whatever RT is.
-template <int BQT, int NT, int RT>
-__device__ __forceinline__ void prepare_x(Block<BQT, NT, RT>& b, v4f (&base)[RT]) {
+// ZP (asymmetric weights): the row sums of x themselves are kept as well (four MFMAs against the constant 1); the
+// zero point of a column and group times that sum is what its partial carries too much.
+template <int BQT, int NT, int RT, bool ZP>
+__device__ __forceinline__ void prepare_x(Block<BQT, NT, RT>& b, v4f (&base)[RT], v4f (&sumx)[RT]) {
   constexpr bool W4 = (BQT == QWIX_INT4);
   constexpr unsigned kNegOff = W4 ? 0xC308C308u : 0xC300C300u;  // bf16 -136 / -128, twice
   const v4u negoff = {kNegOff, kNegOff, kNegOff, kNegOff};
@@ -166,12 +176,19 @@ __device__ __forceinline__ void prepare_x(Block<BQT, NT, RT>& b, v4f (&base)[RT]
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       base[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[rt][j]), as_bf16x8(negoff), base[rt], 0, 0, 0);
+    if constexpr (ZP) {
+      const v4u ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+      sumx[rt] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        sumx[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[rt][j]), as_bf16x8(ones), sumx[rt], 0, 0, 0);
+    }
   }
 }
 
 // Column tile t of one K block, after prepare_x: widen, multiply, scale, add.
-template <int BQT, int NT, bool SBF, int RT>
-__device__ __forceinline__ void compute_tile(const Block<BQT, NT, RT>& b, const v4f (&base)[RT], int t,
+template <int BQT, int NT, bool SBF, int RT, bool ZP>
+__device__ __forceinline__ void compute_tile(const Block<BQT, NT, RT>& b, const v4f (&base)[RT], const v4f (&sumx)[RT], int t,
                                              v4f (&outacc)[RT][NT]) {
   constexpr bool W4 = (BQT == QWIX_INT4);
   v4f acc[RT];
@@ -206,18 +223,25 @@ __device__ __forceinline__ void compute_tile(const Block<BQT, NT, RT>& b, const 
       acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(b.xf[rt][j]), as_bf16x8(w), acc[rt], 0, 0, 0);
   }
   const float sc = __uint_as_float(SBF ? b.sraw[t] << 16 : b.sraw[t]);
+  if constexpr (ZP) {  // sum x (q - z) = sum x q - z sum x
+    const float z = static_cast<float>(static_cast<int>(b.zraw[t] << 24) >> 24);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[rt][r] = fmaf(-z, sumx[rt][r], acc[rt][r]);
+  }
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int r = 0; r < 4; ++r) outacc[rt][t][r] = fmaf(acc[rt][r], sc, outacc[rt][t][r]);
 }
 
-template <int BQT, int NT, bool SBF, int RT>
+template <int BQT, int NT, bool SBF, int RT, bool ZP>
 __device__ __forceinline__ void compute_block(Block<BQT, NT, RT>& b, v4f (&outacc)[RT][NT]) {
-  v4f base[RT];
-  prepare_x<BQT, NT, RT>(b, base);
+  v4f base[RT], sumx[RT];
+  prepare_x<BQT, NT, RT, ZP>(b, base, sumx);
 #pragma unroll
-  for (int t = 0; t < NT; ++t) compute_tile<BQT, NT, SBF, RT>(b, base, t, outacc);
+  for (int t = 0; t < NT; ++t) compute_tile<BQT, NT, SBF, RT, ZP>(b, base, sumx, t, outacc);
 }
 
 // Tiles T .. NT - 1 of a pair of K blocks whose int4 weights come through the LDS panel: the fragments of a tile are
@@ -226,9 +250,10 @@ __device__ __forceinline__ void compute_block(Block<BQT, NT, RT>& b, v4f (&outac
 // stay open), and both blocks' products of that tile follow at once, so that the arithmetic of the early tiles
 // runs while the late ones are still on their way.  Per output element the order of operations is that of
 // compute_block on the first block, then on the second.
-template <int T, int H, int NT, bool SBF, int RT>
+template <int T, int H, int NT, bool SBF, int RT, bool ZP>
 __device__ __forceinline__ void consume_panel(const LaneOff<NT>& a, Block<QWIX_INT4, NT, RT>& b0, Block<QWIX_INT4, NT, RT>& b1,
-                                              const v4f (&base0)[RT], const v4f (&base1)[RT], v4f (&outacc)[RT][NT]) {
+                                              const v4f (&base0)[RT], const v4f (&base1)[RT], const v4f (&sumx0)[RT],
+                                              const v4f (&sumx1)[RT], v4f (&outacc)[RT][NT]) {
   if constexpr (T >= H) {
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * (NT - 1 - T)));
@@ -237,14 +262,14 @@ __device__ __forceinline__ void consume_panel(const LaneOff<NT>& a, Block<QWIX_I
   b0.wq[T][0] = *reinterpret_cast<const v4u*>(a.panel + T * 2048 + a.f[0]);
   b1.wq[T][0] = *reinterpret_cast<const v4u*>(a.panel + T * 2048 + a.f[1]);
   __builtin_amdgcn_sched_barrier(0);
-  compute_tile<QWIX_INT4, NT, SBF, RT>(b0, base0, T, outacc);
-  compute_tile<QWIX_INT4, NT, SBF, RT>(b1, base1, T, outacc);
-  if constexpr (T + 1 < NT) consume_panel<T + 1, H, NT, SBF, RT>(a, b0, b1, base0, base1, outacc);
+  compute_tile<QWIX_INT4, NT, SBF, RT, ZP>(b0, base0, sumx0, T, outacc);
+  compute_tile<QWIX_INT4, NT, SBF, RT, ZP>(b1, base1, sumx1, T, outacc);
+  if constexpr (T + 1 < NT) consume_panel<T + 1, H, NT, SBF, RT, ZP>(a, b0, b1, base0, base1, sumx0, sumx1, outacc);
 }
 
 // NWAVE wavefronts per workgroup, each owning a slice of K; NT tiles of 16 output columns, RT tiles of 16 rows
 // (the weights are read, and widened, once per workgroup whatever RT is).
-template <int BQT, int NWAVE, int NT, bool SBF, int RT = 1>
+template <int BQT, int NWAVE, int NT, bool SBF, int RT = 1, bool ZP = false>
 __global__ void __launch_bounds__(NWAVE * 64) gemv_wq_kernel(GemvArgs p) {
   extern __shared__ float red_raw[];
   float (*red)[RT * NT][4][64] = reinterpret_cast<float (*)[RT * NT][4][64]>(red_raw);  // [NWAVE]
@@ -288,6 +313,7 @@ __global__ void __launch_bounds__(NWAVE * 64) gemv_wq_kernel(GemvArgs p) {
   }
   a.bx = p.x + static_cast<int64_t>(row0) * p.ldx;
   a.bs = static_cast<const char*>(p.s) + static_cast<int64_t>(n_base) * (SBF ? 2 : 4);
+  a.bz = ZP ? p.zp + n_base : nullptr;
   // fragment of K block h: chunk 4 h + kq of panel row col (the key of row 16 t + col does not depend on t)
 #pragma unroll
   for (int h = 0; h < 2; ++h) a.f[h] = col * 128u + static_cast<unsigned>((h * 4 + kq) ^ ((col >> 1) & 7)) * 16u;
@@ -306,29 +332,29 @@ __global__ void __launch_bounds__(NWAVE * 64) gemv_wq_kernel(GemvArgs p) {
   for (; kb + 1 < kb1; kb += 2) {
     Block<BQT, NT, RT> b0, b1;
     if constexpr (BQT == QWIX_INT4) {
-      load_blocks<BQT, NT, SBF, RT, true, false>(p, a, xrow, kb, &b0, &b1);
+      load_blocks<BQT, NT, SBF, RT, true, false, ZP>(p, a, xrow, kb, &b0, &b1);
       __builtin_amdgcn_sched_barrier(0);
       fetch_panel<H, NT>(p, a.bw, a.panel, grow, gchunk, n_base, kb);
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * (NT - H)));  // vmcnt: activations, scales and the first H tiles are here
       __builtin_amdgcn_sched_barrier(0);
-      v4f base0[RT], base1[RT];
-      prepare_x<BQT, NT, RT>(b0, base0);
-      prepare_x<BQT, NT, RT>(b1, base1);
-      consume_panel<0, H, NT, SBF, RT>(a, b0, b1, base0, base1, outacc);
+      v4f base0[RT], base1[RT], sumx0[RT], sumx1[RT];
+      prepare_x<BQT, NT, RT, ZP>(b0, base0, sumx0);
+      prepare_x<BQT, NT, RT, ZP>(b1, base1, sumx1);
+      consume_panel<0, H, NT, SBF, RT, ZP>(a, b0, b1, base0, base1, sumx0, sumx1, outacc);
       __builtin_amdgcn_sched_barrier(0);
       if (kb + 3 < kb1) fetch_panel<0, H>(p, a.bw, a.panel, grow, gchunk, n_base, kb + 2);
       __builtin_amdgcn_sched_barrier(0);
     } else {
-      load_blocks<BQT, NT, SBF, RT, true, true>(p, a, xrow, kb, &b0, &b1);
-      compute_block<BQT, NT, SBF, RT>(b0, outacc);
-      compute_block<BQT, NT, SBF, RT>(b1, outacc);
+      load_blocks<BQT, NT, SBF, RT, true, true, ZP>(p, a, xrow, kb, &b0, &b1);
+      compute_block<BQT, NT, SBF, RT, ZP>(b0, outacc);
+      compute_block<BQT, NT, SBF, RT, ZP>(b1, outacc);
     }
   }
   if (kb < kb1) {  // a last, single block
     Block<BQT, NT, RT> b0;
-    load_blocks<BQT, NT, SBF, RT, false, true>(p, a, xrow, kb, &b0, &b0);
-    compute_block<BQT, NT, SBF, RT>(b0, outacc);
+    load_blocks<BQT, NT, SBF, RT, false, true, ZP>(p, a, xrow, kb, &b0, &b0);
+    compute_block<BQT, NT, SBF, RT, ZP>(b0, outacc);
   }
 
   if constexpr (BQT == QWIX_INT4) __syncthreads();  // the partial sums take the place of the weight panels
@@ -363,9 +389,9 @@ __global__ void __launch_bounds__(NWAVE * 64) gemv_wq_kernel(GemvArgs p) {
 
 using namespace qwix;
 
-extern "C" int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64_t ldb_bytes, int b_qtype, int64_t M,
-                                int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, void* out,
-                                int out_dtype, int64_t ldo, void* stream) {
+static int gemv_wq_impl(const void* x, int64_t ldx, const void* q, int64_t ldb_bytes, int b_qtype, int64_t M, int64_t N,
+                        int64_t K, int64_t group, const void* s, int s_dtype, const int8_t* zp, void* out, int out_dtype,
+                        int64_t ldo, void* stream) {
   if (!x || !q || !s || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null argument");
   if (M <= 0 || N <= 0 || K <= 0 || N > INT32_MAX || K > INT32_MAX || M > 65535 * 16)
     return fail(QWIX_ERR_INVALID_ARGUMENT, "bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
@@ -390,6 +416,7 @@ extern "C" int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64
   p.bpg = static_cast<int>(group / 128);
   p.magic = (0x100000000ull + p.bpg - 1) / p.bpg;
   p.s = s; p.s_dtype = s_dtype;
+  p.zp = zp;
   p.out = out; p.out_dtype = out_dtype; p.ldo = ldo;
   hipStream_t st = static_cast<hipStream_t>(stream);
 #define QWIX_GEMV_KERNEL(KERN, NW, NTT, RTT)                                                                \
@@ -400,18 +427,22 @@ extern "C" int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64
     if (smem >= 65536) if (int e_ = grant_lds(reinterpret_cast<const void*>(KERN), smem, granted)) return e_;\
     KERN<<<grid, NW * 64, smem, st>>>(p);                                                                  \
   } while (0)
-#define QWIX_GEMV_LAUNCH_RT(NW, NTT, RTT)                                                                  \
+#define QWIX_GEMV_LAUNCH_ZP(NW, NTT, RTT, ZPP)                                                             \
   do {                                                                                                     \
     const dim3 grid(static_cast<unsigned>((N + 16 * NTT - 1) / (16 * NTT)),                                \
                     static_cast<unsigned>((M + 16 * RTT - 1) / (16 * RTT)));                               \
     if (b_qtype == QWIX_INT4 && s_dtype == QWIX_BF16)                                                      \
-      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT4, NW, NTT, true, RTT>), NW, NTT, RTT);                     \
+      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT4, NW, NTT, true, RTT, ZPP>), NW, NTT, RTT);                \
     else if (b_qtype == QWIX_INT4)                                                                         \
-      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT4, NW, NTT, false, RTT>), NW, NTT, RTT);                    \
+      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT4, NW, NTT, false, RTT, ZPP>), NW, NTT, RTT);               \
     else if (s_dtype == QWIX_BF16)                                                                         \
-      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT8, NW, NTT, true, RTT>), NW, NTT, RTT);                     \
+      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT8, NW, NTT, true, RTT, ZPP>), NW, NTT, RTT);                \
     else                                                                                                   \
-      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT8, NW, NTT, false, RTT>), NW, NTT, RTT);                    \
+      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT8, NW, NTT, false, RTT, ZPP>), NW, NTT, RTT);               \
+  } while (0)
+#define QWIX_GEMV_LAUNCH_RT(NW, NTT, RTT)                                                                  \
+  do {                                                                                                     \
+    if (zp) QWIX_GEMV_LAUNCH_ZP(NW, NTT, RTT, true); else QWIX_GEMV_LAUNCH_ZP(NW, NTT, RTT, false);        \
   } while (0)
 #define QWIX_GEMV_LAUNCH(NW, NTT)                                                                          \
   do {                                                                                                     \
@@ -429,6 +460,20 @@ extern "C" int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64
     QWIX_GEMV_LAUNCH(16, 1);
 #undef QWIX_GEMV_LAUNCH
 #undef QWIX_GEMV_LAUNCH_RT
+#undef QWIX_GEMV_LAUNCH_ZP
 #undef QWIX_GEMV_KERNEL
   return check_launch("gemv_wq");
+}
+
+extern "C" int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64_t ldb_bytes, int b_qtype, int64_t M,
+                                int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, void* out,
+                                int out_dtype, int64_t ldo, void* stream) {
+  return gemv_wq_impl(x, ldx, q, ldb_bytes, b_qtype, M, N, K, group, s, s_dtype, nullptr, out, out_dtype, ldo, stream);
+}
+
+extern "C" int qwix_hip_gemv_wq_zp(const void* x, int64_t ldx, const void* q, int64_t ldb_bytes, int b_qtype, int64_t M,
+                                   int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, const int8_t* zp,
+                                   void* out, int out_dtype, int64_t ldo, void* stream) {
+  if (!zp) return fail(QWIX_ERR_INVALID_ARGUMENT, "null zero points");
+  return gemv_wq_impl(x, ldx, q, ldb_bytes, b_qtype, M, N, K, group, s, s_dtype, zp, out, out_dtype, ldo, stream);
 }

@@ -156,6 +156,38 @@ def test_weight_only_gemv(M, K, N, group, sdt, wq_type):
 
 
 @pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('M', [1, 16, 40, 100, 250])
+@pytest.mark.parametrize('K,N,group,sdt', [(512, 256, 128, torch.float32), (4224, 1024, 128, torch.bfloat16), (1024, 200, 1024, torch.bfloat16),
+                                           (4096, 14336, 128, torch.float32)])
+def test_weight_only_gemv_asymmetric_weights(M, K, N, group, sdt, wq_type):
+  """bf16 activations x a weight quantized with min/max calibration (zero points per group and column): the decode
+  kernel takes the zero point out through the row sums of x.  Against the oracle's dequantize-first dot on the
+  same quantized weight, at the tolerance of the symmetric case; the kernel is the one that runs (a row count the
+  dequantizing tile GEMM never takes with a zero point)."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  print('case gemv zp', M, K, N, group, wq_type, sdt, flush=True)
+  x_np, x_t = util.make((M, K), O.BF16, seed=M + K + 3)
+  w_np, w_t = util.make((K, N), O.BF16, seed=M + K + 4, scale=0.02)
+  w_np = O.round_to_bf16(w_np + 0.013)   # off-centre, so that the zero points are not all alike
+  w_t = torch.from_numpy(w_np).to(torch.bfloat16).to(util.DEV)
+  tiled = {0: group} if group != K else {}
+  kw = dict(channelwise_axes=[1], tiled_axes=tiled, calibration_method='minmax')
+  wq = qarray.quantize_api(w_t, wq_type, scale_dtype=sdt, **kw)
+  owq = O.quantize_api(O.FArr(w_np, O.BF16), wq_type, scale_dtype=util.ORACLE_DT[sdt], **kw)
+  util.assert_qarray_equal(wq, owq, 'weight')
+  assert wq.zero_point is not None and dg._weight_only_fit(x_t, wq, DN) is not None
+  out = dg.dot_general(x_t, wq, DN, preferred_element_type=torch.float32)
+  torch.cuda.synchronize()
+  want = O.dot_general(O.FArr(x_np, O.BF16), owq, DN, O.F32)
+  got = util.f32np(out)
+  assert np.allclose(got, want.v, rtol=1e-2, atol=1e-2 * np.abs(want.v).mean()), np.abs(got - want.v).max()
+  # the same through the two library kernels that dequantize first (what larger batches run)
+  two = dg._dequantize_then_bf16_gemm(x_t, wq, DN, torch.float32)
+  assert torch.allclose(out, two, rtol=1e-2, atol=1e-2 * float(two.abs().mean()))
+
+
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
 @pytest.mark.parametrize('M', [1, 20, 40])
 @pytest.mark.parametrize('K,N,group', [(384, 72, 128), (4224, 136, 128), (16384, 264, 256), (8192, 2048, 128), (128, 48, 128)])
 def test_weight_only_gemv_k_splits(M, K, N, group, wq_type):
@@ -457,9 +489,9 @@ def test_weight_only_prefill_on_hip_kernels(M, K, N, case):
   wq = qarray.quantize_api(w_t, wq_type, **kw)
   owq = O.quantize_api(O.FArr(w_np, O.BF16), wq_type, **okw)
   util.assert_qarray_equal(wq, owq, 'weight')
-  # the decode kernel is bypassed by its own row limit (M > 256) or by the operand kind (zero point, e4m3)
+  # the decode kernel is bypassed by its own row limit (M > 256) or by the operand kind (e4m3)
   fit = dg._weight_only_fit(x_t, wq, DN)
-  assert (fit is None) == (asym or wq_type == 'float8_e4m3fn')
+  assert (fit is None) == (wq_type == 'float8_e4m3fn')
   out = dg._dequantize_then_bf16_gemm(x_t, wq, DN, torch.bfloat16)
   assert out is not None and out.dtype == torch.bfloat16
   torch.cuda.synchronize()
@@ -468,7 +500,7 @@ def test_weight_only_prefill_on_hip_kernels(M, K, N, case):
   assert np.allclose(got, want.v, rtol=1e-2, atol=1e-2 * np.abs(want.v).mean()), np.abs(got - want.v).max()
   # the operator takes this path beyond the decode kernel's rows, for the operand kinds that kernel does not take, and
   # for symmetric int4 from the row count on at which the dequantizing tile GEMM wins
-  if M > dg.WEIGHT_ONLY_MAX_ROWS or fit is None or (wq_type in ('int4', 'int8') and M > dg.fused_wq_min_rows(N, wq_type == 'int4')):
+  if M > dg.WEIGHT_ONLY_MAX_ROWS or fit is None or (not asym and wq_type in ('int4', 'int8') and M > dg.fused_wq_min_rows(N, wq_type == 'int4')):
     assert torch.equal(dg.dot_general(x_t, wq, DN, preferred_element_type=torch.bfloat16), out)
   # the dequantized operand itself, against the oracle's dequantize
   c = dg._Canon(x_t, wq, DN)
