@@ -543,6 +543,61 @@ def _weight_only_fit(lhs, rhs, dimension_numbers):
 WEIGHT_ONLY_MAX_ROWS = 256
 
 
+# Decode-size calls x (M, K) @ w (K, N) against a static weight spend more time in this module than in the kernel (24 us
+# of host work per call against 8.4 us on the device), most of it on the weight: operand checks, layout views, the
+# zero-point re-layout.  That part is done once per weight object and kept while the weight is alive and unchanged.
+_DECODE_PLANS: dict = {}
+
+
+def _weight_signature(rhs: QArray) -> tuple:
+  z = rhs.zero_point
+  return (id(rhs.qvalue), id(rhs.scale), id(z), None if z is None else z._version)
+
+
+def _decode_plan(lhs, rhs, dimension_numbers):
+  key = id(rhs)
+  hit = _DECODE_PLANS.get(key)
+  if hit is not None and hit[0]() is rhs and hit[1] == _weight_signature(rhs):
+    return hit[2]
+  plan = None
+  c = _weight_only_fit(lhs, rhs, dimension_numbers)
+  if c is not None:
+    b, b_is4 = c.rhs_values(rhs)
+    sb, gb = c.rhs_scale(rhs)
+    zp = _rhs_zero_point_i8(c, rhs)[0] if rhs.zero_point is not None else None
+    plan = (b, _lib.INT4 if b_is4 else _lib.INT8, sb, _lib.float_tag(sb.dtype), zp, c.N, c.K, c.K // gb,
+            fused_wq_min_rows(c.N, b_is4))
+  _DECODE_PLANS[key] = (weakref.ref(rhs, lambda _, k=key: _DECODE_PLANS.pop(k, None)),
+                        _weight_signature(rhs), plan)
+  return plan
+
+
+def _decode_dot(lhs, rhs, dimension_numbers, preferred_element_type):
+  """The decode kernel on a 2-D bf16 activation and a 2-D weight with a kept plan; None when the call is not of that
+  kind (the general code below then decides)."""
+  (lca, rca), _ = dimension_numbers
+  if not (type(lhs) is torch.Tensor and lhs.ndim == 2 and lhs.dtype == torch.bfloat16 and isinstance(rhs, QArray)
+          and len(lca) == 1 and lca[0] == 1 and rca[0] == 0 and lhs.shape[0] <= WEIGHT_ONLY_MAX_ROWS
+          and lhs.stride(1) == 1 and lhs.stride(0) % 8 == 0):
+    return None
+  plan = _decode_plan(lhs, rhs, dimension_numbers)
+  if plan is None:
+    return None
+  b, b_tag, sb, sb_tag, zp, n, k, group, fused_min = plan
+  m = lhs.shape[0]
+  if lhs.shape[1] != k or len(rhs.shape) != 2 or (zp is None and m > fused_min):
+    return None
+  res_t = preferred_element_type or torch.promote_types(lhs.dtype, sb.dtype)
+  out = torch.empty(m, n, dtype=res_t, device=lhs.device)
+  if zp is not None:
+    _lib.call('qwix_hip_gemv_wq_zp', lhs.data_ptr(), lhs.stride(0), b.data_ptr(), b.stride(0), b_tag, m, n, k, group,
+              sb.data_ptr(), sb_tag, zp.data_ptr(), out.data_ptr(), _lib.float_tag(res_t), n, _lib.stream_of(lhs))
+  else:
+    _lib.call('qwix_hip_gemv_wq', lhs.data_ptr(), lhs.stride(0), b.data_ptr(), b.stride(0), b_tag, m, n, k, group,
+              sb.data_ptr(), sb_tag, out.data_ptr(), _lib.float_tag(res_t), n, _lib.stream_of(lhs))
+  return out
+
+
 def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, **kwargs) -> torch.Tensor:
   """Dequantize-first path (dot_general.py:264-275).  A bf16 activation against an int4/int8 weight runs in one
   fused kernel (dequantize in registers, bf16 MFMA) when `_weight_only_fit` says the kernel takes it; every
@@ -551,6 +606,9 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   del kwargs
   if len(dimension_numbers[1][0]) or len(dimension_numbers[1][1]):
     return _over_batch(_slow_dot_general, lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type)
+  out = _decode_dot(lhs, rhs, dimension_numbers, preferred_element_type)
+  if out is not None:
+    return out
   c = _weight_only_fit(lhs, rhs, dimension_numbers)
   if (c is not None and rhs.zero_point is None
       and fused_wq_min_rows(c.N, isinstance(rhs.qvalue, Int4Tensor)) < c.M <= WEIGHT_ONLY_MAX_ROWS):
