@@ -396,7 +396,7 @@ class WeightOnlyPrefill(Workload):
     L = self.L
     if self.fused:
       L.call('qwix_hip_gemm_bf16_wq', self.x.data_ptr(), self.K, self.b.data_ptr(), self.b.stride(0), L.INT4, self.M,
-             self.N, self.K, self.group, self.s.data_ptr(), L.F32, self.out.data_ptr(), L.BF16, self.N, self.stream)
+             self.N, self.K, self.group, self.s.data_ptr(), L.F32, None, self.out.data_ptr(), L.BF16, self.N, self.stream)
       return
     L.call('qwix_hip_gemm_bf16', self.x.data_ptr(), self.K, self.w.data_ptr(), self.K, self.M, self.N, self.K,
            self.out.data_ptr(), L.BF16, self.N, self.stream)

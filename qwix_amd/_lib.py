@@ -53,7 +53,7 @@ SIGNATURES = {
     'qwix_hip_qgemm_grouped_zp': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp, _int, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _int, _i64, _int, _vp, _vp]),
     'qwix_hip_ksum_groups': (_int, [_vp, _int, _i64, _i64, _i64, _i64, _vp, _vp]),
     'qwix_hip_gemm_bf16': (_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
-    'qwix_hip_gemm_bf16_wq': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _vp, _int, _i64, _vp]),
+    'qwix_hip_gemm_bf16_wq': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _int, _i64, _vp]),
     'qwix_hip_dequantize_rm': (_int, [_vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _int, _vp, _int, _vp]),
     'qwix_hip_gemv_wq': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _vp, _int, _i64, _vp]),
     'qwix_hip_gemv_wq_zp': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _int, _i64, _vp]),

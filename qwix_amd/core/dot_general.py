@@ -10,7 +10,7 @@ What reaches a hand-written kernel:
   int8 x int8, e4m3 x e4m3 (per-row x per-column scales)          -> qwix_hip_qgemm
   int8 x int8/int4 with K-group scales (tile % 128 == 0)          -> qwix_hip_qgemm_grouped
   bf16 activations x int4/int8 weight (weight-only, any group)    -> qwix_hip_gemv_wq up to 104..200 rows,
-      qwix_hip_gemm_bf16_wq (symmetric int4 up to 1024 rows, int8 up to one round of tiles),
+      qwix_hip_gemm_bf16_wq (int4 up to 1024 rows, int8 up to one round of tiles),
       qwix_hip_dequantize_rm + qwix_hip_gemm_bf16 above
 Everything else on the slow path is dequantized by the HIP dequantize kernel and contracted by
 the vendor float GEMM.  Unsupported fast-path combinations raise; they never change path silently.
@@ -585,7 +585,7 @@ def _decode_dot(lhs, rhs, dimension_numbers, preferred_element_type):
     return None
   b, b_tag, sb, sb_tag, zp, n, k, group, fused_min = plan
   m = lhs.shape[0]
-  if lhs.shape[1] != k or len(rhs.shape) != 2 or (zp is None and m > fused_min):
+  if lhs.shape[1] != k or len(rhs.shape) != 2 or m > fused_min:
     return None
   res_t = preferred_element_type or torch.promote_types(lhs.dtype, sb.dtype)
   out = torch.empty(m, n, dtype=res_t, device=lhs.device)
@@ -610,8 +610,7 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   if out is not None:
     return out
   c = _weight_only_fit(lhs, rhs, dimension_numbers)
-  if (c is not None and rhs.zero_point is None
-      and fused_wq_min_rows(c.N, isinstance(rhs.qvalue, Int4Tensor)) < c.M <= WEIGHT_ONLY_MAX_ROWS):
+  if c is not None and fused_wq_min_rows(c.N, isinstance(rhs.qvalue, Int4Tensor)) < c.M <= WEIGHT_ONLY_MAX_ROWS:
     # one row tile of the dequantizing tile GEMM beats the decode kernel from here on
     out = _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type, fused_only=True)
     if out is not None:
@@ -675,7 +674,7 @@ def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_ty
   array (qwix_hip_dequantize_rm, the reference's D(D(q - zp) * scale) in the scale dtype; an f32 result rounded
   once more to bf16) and contracted by the bf16 MFMA GEMM with f32 accumulation (qwix_hip_gemm_bf16).  Returns
   None when the operands are not of that kind (then: HIP dequantize + the float GEMM of the vendor library).
-  Symmetric int4 / int8 weights skip the dequantized copy while `_fused_wq_takes` (qwix_hip_gemm_bf16_wq);
+  int4 / int8 weights skip the dequantized copy while `_fused_wq_takes` (qwix_hip_gemm_bf16_wq);
   with `fused_only` nothing else is run."""
   if not (_is_float_array(lhs) and lhs.dtype == torch.bfloat16 and isinstance(rhs, QArray)):
     return None
@@ -704,14 +703,14 @@ def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_ty
   res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.scale.dtype)
   if res_t not in (torch.bfloat16, torch.float32):
     return None
-  if (_qtype_of(rhs) in (numerics.INT4, numerics.INT8) and zp is None and _fused_wq_takes(c.M, c.N, b_is4)
+  if (_qtype_of(rhs) in (numerics.INT4, numerics.INT8) and _fused_wq_takes(c.M, c.N, b_is4)
       and c.K % 256 == 0 and (c.K // gb) % 64 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0):
-    # symmetric int4 / int8: dequantized inside the GEMM's workgroups, slab by slab (the same bf16 weights, the
-    # same products in the same order, no dequantized copy of the weight in memory)
+    # int4 / int8, with or without zero points: dequantized inside the GEMM's workgroups, slab by slab (the same
+    # bf16 weights, the same products in the same order, no dequantized copy of the weight in memory)
     out = torch.empty(c.M, c.N, dtype=res_t, device=dev)
     _lib.call('qwix_hip_gemm_bf16_wq', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0),
               _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
-              out.data_ptr(), _lib.float_tag(res_t), c.N, st)
+              _lib.ptr(zp), out.data_ptr(), _lib.float_tag(res_t), c.N, st)
     return out.reshape(c.out_shape)
   if fused_only:
     return None

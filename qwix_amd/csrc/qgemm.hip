@@ -2037,10 +2037,15 @@ __global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__
 // a load instruction's lanes repeats the lower half's rows (every wavefront issues one load per slab, so that all
 // count their requests alike); the repeated rows land in padding.  A byte b holds q = (b ^ 0x80) - 128 and
 // q * scale = fma(b ^ 0x80, scale, -128 scale), exact as for the nibbles.
-template <int OUT, bool SBF, int BN, int BITS>
+// ZP: asymmetric weights, (q - zero_point) * scale with one int8 zero point per scale.  It is requested with the scale
+// and joins the offset of the storage format: bf16 scales fma(u, scale, -(offset + zp) scale), every term still exact
+// in f32 (nine bits times eight); f32 scales float(u - offset - zp) * scale, the integer difference first, because
+// (offset + zp) * scale would no longer be exact.
+template <int OUT, bool SBF, int BN, int BITS, bool ZP>
 __global__ void __launch_bounds__(512)
     wgemm_wq_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ Q, int64_t ldq,
-                    const void* __restrict__ S, int M, int N, int K, int group, uint8_t* __restrict__ out, int64_t ldo) {
+                    const void* __restrict__ S, const int8_t* __restrict__ Z, int M, int N, int K, int group,
+                    uint8_t* __restrict__ out, int64_t ldo) {
   static_assert(BN == 128 || BN == 64, "column tiles of 128 or 64");
   constexpr int BM = 256, WGN = 2, WN = BN / WGN, TM = 2, TN = WN / 32, NWAVES = 8;
   constexpr int BK = 128, NK = 4;  // bytes of an activation row per slab (64 elements); k-steps of 16 elements
@@ -2113,24 +2118,31 @@ __global__ void __launch_bounds__(512)
   // end-of-slab wait has covered them); the pointer walks the groups slab by slab.
   const int slabs_per_group = group >> 6;
   const char* sc_ptr = sptr;
+  const int8_t* zp_ptr = ZP ? Z + min(n0 + crow, N - 1) : nullptr;
   int sc_left = slabs_per_group;
-  auto request_scales = [&](uint32_t (&dst)[4]) {
+  auto request_scales = [&](uint32_t (&dst)[4], int (&dstz)[4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if constexpr (SBF)
         asm volatile("global_load_ushort %0, %1, off" : "=&v"(dst[j]) : "v"(sc_ptr) : "memory");
       else
         asm volatile("global_load_dword %0, %1, off" : "=&v"(dst[j]) : "v"(sc_ptr) : "memory");
+      if constexpr (ZP) asm volatile("global_load_sbyte %0, %1, off" : "=&v"(dstz[j]) : "v"(zp_ptr) : "memory");
       if (--sc_left == 0) {
         sc_left = slabs_per_group;
         sc_ptr += s_group_pitch;
+        if constexpr (ZP) zp_ptr += N;
       }
     }
   };
-  auto pin_scales = [&](uint32_t (&v)[4]) {
+  auto pin_scales = [&](uint32_t (&v)[4], int (&vz)[4]) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(v[j]));
+    for (int j = 0; j < 4; ++j) {
+      asm volatile("" : "+v"(v[j]));
+      if constexpr (ZP) asm volatile("" : "+v"(vz[j]));
+    }
   };
+  constexpr int kSL = ZP ? 8 : 4;  // loads of one request_scales
   constexpr int NRAW = NPT * BITS / 32;  // dwords of raw weights per thread and slab
   int craw[NRAW];
   uint32_t cout[NPT / 2];
@@ -2158,27 +2170,30 @@ __global__ void __launch_bounds__(512)
   // A nibble n holds q = (n ^ 8) - 8.  With the 8 folded into the multiply-add, q * scale = fma(n ^ 8, scale, -8 scale): every
   // term is exact in f32 (four bits times the eight of a bf16 scale), so the product is the one of float(q) * scale, and a
   // byte of the masked word converts in one instruction.
-  auto convert_quarter = [&](int q4, float sc) {  // elements 4 q4 .. 4 q4 + 3 of this thread's NPT
+  auto convert_quarter = [&](int q4, float sc, int zp) {  // elements 4 q4 .. 4 q4 + 3 of this thread's NPT
     if (q4 >= NCQ) return;
+    const int off = (W8 ? 128 : 8) + (ZP ? zp : 0);          // what the stored byte / nibble carries too much
+    const float moff = -static_cast<float>(off) * sc;        // exact (see above)
+    auto value = [&](uint32_t u) -> float {
+      if constexpr (ZP && !SBF) return static_cast<float>(static_cast<int>(u) - off) * sc;
+      return __builtin_fmaf(static_cast<float>(u), sc, moff);
+    };
+    float f0, f1, f2, f3;
     if constexpr (W8) {
       const uint32_t u = static_cast<uint32_t>(craw[q4]) ^ 0x80808080u;
-      const float m128 = -128.f * sc;
-      const float f0 = __builtin_fmaf(static_cast<float>(u & 0xFFu), sc, m128);
-      const float f1 = __builtin_fmaf(static_cast<float>((u >> 8) & 0xFFu), sc, m128);
-      const float f2 = __builtin_fmaf(static_cast<float>((u >> 16) & 0xFFu), sc, m128);
-      const float f3 = __builtin_fmaf(static_cast<float>(u >> 24), sc, m128);
-      cout[2 * q4] = pack_bf16x2(f0, f1);
-      cout[2 * q4 + 1] = pack_bf16x2(f2, f3);
-      return;
+      f0 = value(u & 0xFFu);
+      f1 = value((u >> 8) & 0xFFu);
+      f2 = value((u >> 16) & 0xFFu);
+      f3 = value(u >> 24);
+    } else {
+      const uint32_t w = static_cast<uint32_t>(craw[q4 >> 1]) ^ 0x88888888u;
+      const uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
+      const int b0 = (q4 & 1) * 16;
+      f0 = value((even >> b0) & 0xFFu);
+      f1 = value((odd >> b0) & 0xFFu);
+      f2 = value((even >> (b0 + 8)) & 0xFFu);
+      f3 = value((odd >> (b0 + 8)) & 0xFFu);
     }
-    const uint32_t w = static_cast<uint32_t>(craw[W8 ? 0 : q4 >> 1]) ^ 0x88888888u;
-    const uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
-    const int b0 = (q4 & 1) * 16;
-    const float m8 = -8.f * sc;
-    const float f0 = __builtin_fmaf(static_cast<float>((even >> b0) & 0xFFu), sc, m8);
-    const float f1 = __builtin_fmaf(static_cast<float>((odd >> b0) & 0xFFu), sc, m8);
-    const float f2 = __builtin_fmaf(static_cast<float>((even >> (b0 + 8)) & 0xFFu), sc, m8);
-    const float f3 = __builtin_fmaf(static_cast<float>((odd >> (b0 + 8)) & 0xFFu), sc, m8);
     cout[2 * q4] = pack_bf16x2(f0, f1);
     cout[2 * q4 + 1] = pack_bf16x2(f2, f3);
   };
@@ -2225,6 +2240,7 @@ __global__ void __launch_bounds__(512)
 
   const int KT = K / 64;  // a multiple of 4
   uint32_t sc_cur[4], sc_next[4] = {0, 0, 0, 0};
+  int zp_cur[4] = {0, 0, 0, 0}, zp_next[4] = {0, 0, 0, 0};
   int sta = 0;  // LDS stage of the activations of the slab being multiplied: kt % 3
   // One slab, J = kt % 4: requests activations two slabs ahead (and, at J == 0, the packed weights and scales of
   // the next superslab), converts the weights of slab kt + 1 between the k-steps of slab kt.
@@ -2237,19 +2253,20 @@ __global__ void __launch_bounds__(512)
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (loads_a) issue_a(kt + 2, sta == 0 ? 2 : sta - 1);
     if constexpr (loads_w) issue_raw(W8 ? kt + 3 : (kt >> 2) + 1);
-    if constexpr (loads_s) request_scales(sc_next);
+    if constexpr (loads_s) request_scales(sc_next, zp_next);
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (j == 2 && !last) pin_scales(sc_next);  // requested at j == 0, covered by the wait that ended j == 1
+    if constexpr (j == 2 && !last) pin_scales(sc_next, zp_next);  // requested at j == 0, covered by the wait that ended j == 1
     const float sc = scale_value(j == 3 ? sc_next[0] : sc_cur[(j + 1) & 3]);
+    const int zc = j == 3 ? zp_next[0] : zp_cur[(j + 1) & 3];
     if constexpr (more) convert_read(kt + 1);
 #pragma unroll
     for (int ks = 0; ks < NK; ++ks) {
       if (ks + 1 < NK) read_frags(sta, j & 1, ks + 1, (ks + 1) & 1);
-      if constexpr (more) convert_quarter(ks, sc);
+      if constexpr (more) convert_quarter(ks, sc, zc);
       mfma_step(ks & 1);
     }
     if constexpr (more) convert_write(kt + 1);
-    end_of_slab(integral_constant<int, (loads_a ? 4 : 0) + (loads_w ? NQ : 0) + (loads_s ? 4 : 0)>{});
+    end_of_slab(integral_constant<int, (loads_a ? 4 : 0) + (loads_w ? NQ : 0) + (loads_s ? kSL : 0)>{});
     sta = sta == 2 ? 0 : sta + 1;
     if constexpr (more) read_frags(sta, (j + 1) & 1, 0, 0);
   };
@@ -2260,14 +2277,14 @@ __global__ void __launch_bounds__(512)
     issue_raw(1);
     issue_raw(2);
   }
-  request_scales(sc_cur);
+  request_scales(sc_cur, zp_cur);
   issue_a(0, 0);
   issue_a(1, 1);
   end_of_slab(integral_constant<int, 0>{});
-  pin_scales(sc_cur);
+  pin_scales(sc_cur, zp_cur);
   convert_read(0);
 #pragma unroll
-  for (int q4 = 0; q4 < 4; ++q4) convert_quarter(q4, scale_value(sc_cur[0]));
+  for (int q4 = 0; q4 < 4; ++q4) convert_quarter(q4, scale_value(sc_cur[0]), zp_cur[0]);
   convert_write(0);
   end_of_slab(integral_constant<int, 0>{});
   read_frags(0, 0, 0, 0);
@@ -2283,7 +2300,10 @@ __global__ void __launch_bounds__(512)
     slab(kt + 2, I2{}, std::false_type{});
     slab(kt + 3, I3{}, std::false_type{});
 #pragma unroll
-    for (int e = 0; e < 4; ++e) sc_cur[e] = sc_next[e];
+    for (int e = 0; e < 4; ++e) {
+      sc_cur[e] = sc_next[e];
+      zp_cur[e] = zp_next[e];
+    }
   }
   slab(kt, I0{}, std::true_type{});
   slab(kt + 1, I1{}, std::true_type{});
@@ -2529,8 +2549,8 @@ extern "C" int qwix_hip_gemm_bf16(const void* a, int64_t lda, const void* b, int
 }
 
 extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, int64_t ldq_bytes, int q_qtype, int64_t M,
-                                     int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, void* out,
-                                     int out_dtype, int64_t ldo, void* stream) {
+                                     int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, const int8_t* zp,
+                                     void* out, int out_dtype, int64_t ldo, void* stream) {
   if (!a || !q || !s || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/q/s/out");
   if (q_qtype != QWIX_INT4 && q_qtype != QWIX_INT8)
     return fail(QWIX_ERR_UNSUPPORTED, "weight qtype %d: int4 or int8", q_qtype);
@@ -2554,17 +2574,21 @@ extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, 
   // 64-column tiles while 128-column ones would occupy at most half of the CUs
   const bool narrow = ((M + 255) / 256) * ((N + 127) / 128) <= 128;
   hipStream_t st = static_cast<hipStream_t>(stream);
-#define QWIX_WQ_LAUNCH(OUTT, SBFF, BNN, BITS)                                                                        \
+#define QWIX_WQ_LAUNCH(OUTT, SBFF, BNN, BITS) \
+  do {                                        \
+    if (zp) QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BNN, BITS, true); else QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BNN, BITS, false); \
+  } while (0)
+#define QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BNN, BITS, ZPP)                                                                 \
   do {                                                                                                               \
-    auto kern = wgemm_wq_kernel<OUTT, SBFF, BNN, BITS>;                                                              \
+    auto kern = wgemm_wq_kernel<OUTT, SBFF, BNN, BITS, ZPP>;                                                         \
     /* activations 96 KB, converted weights 2 x BN x 128, raw weights 2 x BN x 128 (int8: 4 x 8 KB): <= 160 KB */    \
     constexpr size_t smem = 3 * 256 * 128 + 2 * BNN * 128 + (BITS == 8 ? 4 * 8192 : 2 * BNN * 128);                  \
     const dim3 grid(static_cast<unsigned>(((M + 255) / 256) * ((N + BNN - 1) / BNN)));                               \
     static LdsGrant granted;                                                                                         \
     if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;                           \
     kern<<<grid, 512, smem, st>>>(static_cast<const uint8_t*>(a), 2 * lda, static_cast<const uint8_t*>(q), ldq_bytes, s, \
-                                  static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), static_cast<int>(group), \
-                                  static_cast<uint8_t*>(out), ldo);                                                  \
+                                  zp, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K),                 \
+                                  static_cast<int>(group), static_cast<uint8_t*>(out), ldo);                         \
   } while (0)
 #define QWIX_WQ_TILE(OUTT, SBFF, BITS)                                                                               \
   do {                                                                                                               \
@@ -2582,6 +2606,7 @@ extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, 
 #undef QWIX_WQ_BITS
 #undef QWIX_WQ_TILE
 #undef QWIX_WQ_LAUNCH
+#undef QWIX_WQ_LAUNCH_Z
   return check_launch("gemm_bf16_wq");
 }
 

@@ -162,8 +162,8 @@ def test_weight_only_gemv(M, K, N, group, sdt, wq_type):
 def test_weight_only_gemv_asymmetric_weights(M, K, N, group, sdt, wq_type):
   """bf16 activations x a weight quantized with min/max calibration (zero points per group and column): the decode
   kernel takes the zero point out through the row sums of x.  Against the oracle's dequantize-first dot on the
-  same quantized weight, at the tolerance of the symmetric case; the kernel is the one that runs (a row count the
-  dequantizing tile GEMM never takes with a zero point)."""
+  same quantized weight, at the tolerance of the symmetric case (250 rows run the dequantizing tile GEMM, which takes
+  zero points too)."""
   from qwix_amd.core import dot_general as dg
   from qwix_amd.core import qarray
   print('case gemv zp', M, K, N, group, wq_type, sdt, flush=True)
@@ -406,19 +406,23 @@ def test_bf16_gemm_against_float64(M, K, N, out_dtype):
 @pytest.mark.parametrize('sdt', [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('asym', [False, True])
 @pytest.mark.parametrize('M,K,N,group', [(300, 256, 136, 128), (512, 1024, 1000, 256), (257, 2048, 520, 64), (2048, 4096, 1536, 128),
                                          (1, 512, 64, 512), (600, 512, 8400, 128), (1100, 256, 4100, 64)])
-def test_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, wq_type, out_dtype, sdt):
+def test_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, asym, wq_type, out_dtype, sdt):
   """qwix_hip_gemm_bf16_wq through the C ABI == qwix_hip_dequantize_rm (to bf16) + qwix_hip_gemm_bf16, bit for bit: the
-  same bf16 weights, the same MFMA, K walked in the same order; int4 and int8 weights, edges in M and N, one slab
-  group (64), several; the last two shapes have more than 128 tiles of 256 x 128 and run those, the others tiles of
+  same bf16 weights, the same MFMA, K walked in the same order; int4 and int8 weights, with and without zero points,
+  edges in M and N, one slab group (64), several; the last two shapes have more than 128 tiles of 256 x 128 and run those, the others tiles of
   256 x 64."""
   from qwix_amd import _lib
   from qwix_amd.core import qarray
-  print('case wq prefill', M, K, N, group, wq_type, out_dtype, sdt, flush=True)
+  print('case wq prefill', M, K, N, group, asym, wq_type, out_dtype, sdt, flush=True)
   x_np, x_t = util.make((M, K), O.BF16, seed=M + K + 21)
   w_np, w_t = util.make((K, N), O.BF16, seed=N + K + 22, scale=0.02)
-  wq = qarray.quantize_api(w_t, wq_type, channelwise_axes=[1], tiled_axes={0: group}, scale_dtype=sdt)
+  kw = dict(calibration_method='minmax') if asym else {}
+  if asym:
+    w_t = (w_t.float() + 0.013).to(torch.bfloat16)  # off-centre: zero points that differ
+  wq = qarray.quantize_api(w_t, wq_type, channelwise_axes=[1], tiled_axes={0: group}, scale_dtype=sdt, **kw)
   from qwix_amd.core import dot_general as dg
   c = dg._Canon(x_t, wq, DN)
   b, is4 = c.rhs_values(wq)
@@ -426,14 +430,16 @@ def test_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, wq_type, out_dty
   assert is4 == (wq_type == 'int4') and gb == K // group
   tag = _lib.INT4 if is4 else _lib.INT8
   st = _lib.stream_of(x_t)
+  zp = dg._rhs_zero_point_i8(c, wq)[0] if asym else None
+  assert (wq.zero_point is not None) == asym
   w = torch.empty(N, K, dtype=torch.bfloat16, device=util.DEV)
-  _lib.call('qwix_hip_dequantize_rm', b.data_ptr(), tag, 1, K, N, group, sb.data_ptr(), None, _lib.float_tag(sb.dtype),
+  _lib.call('qwix_hip_dequantize_rm', b.data_ptr(), tag, 1, K, N, group, sb.data_ptr(), _lib.ptr(zp), _lib.float_tag(sb.dtype),
             w.data_ptr(), _lib.BF16, st)
   want = torch.empty(M, N, dtype=out_dtype, device=util.DEV)
   _lib.call('qwix_hip_gemm_bf16', x_t.data_ptr(), K, w.data_ptr(), K, M, N, K, want.data_ptr(), _lib.float_tag(out_dtype), N, st)
   got = torch.full((M, N), float('nan'), dtype=out_dtype, device=util.DEV)
   _lib.call('qwix_hip_gemm_bf16_wq', x_t.data_ptr(), K, b.data_ptr(), b.stride(0), tag, M, N, K, group, sb.data_ptr(),
-            _lib.float_tag(sb.dtype), got.data_ptr(), _lib.float_tag(out_dtype), N, st)
+            _lib.float_tag(sb.dtype), _lib.ptr(zp), got.data_ptr(), _lib.float_tag(out_dtype), N, st)
   torch.cuda.synchronize()
   assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
   # and against float64 on the dequantized weight
@@ -452,8 +458,8 @@ def test_dequantizing_gemm_argument_checks():
   s = torch.ones(K // 128, N, dtype=torch.bfloat16, device=util.DEV)
   out = torch.empty(M, N, dtype=torch.bfloat16, device=util.DEV)
   def call(lda=K, ldq=K, qt=_lib.INT8, k=K, group=128, sd=_lib.BF16, od=_lib.BF16, ldo=N):
-    return L.qwix_hip_gemm_bf16_wq(x.data_ptr(), lda, q.data_ptr(), ldq, qt, M, N, k, group, s.data_ptr(), sd, out.data_ptr(),
-                                   od, ldo, None)
+    return L.qwix_hip_gemm_bf16_wq(x.data_ptr(), lda, q.data_ptr(), ldq, qt, M, N, k, group, s.data_ptr(), sd, None,
+                                   out.data_ptr(), od, ldo, None)
   assert call() == 0
   assert call(qt=_lib.INT4, ldq=K // 2) == 0
   assert call(qt=_lib.E4M3) != 0 and b'int4 or int8' in L.qwix_hip_last_error()
@@ -500,7 +506,7 @@ def test_weight_only_prefill_on_hip_kernels(M, K, N, case):
   assert np.allclose(got, want.v, rtol=1e-2, atol=1e-2 * np.abs(want.v).mean()), np.abs(got - want.v).max()
   # the operator takes this path beyond the decode kernel's rows, for the operand kinds that kernel does not take, and
   # for symmetric int4 from the row count on at which the dequantizing tile GEMM wins
-  if M > dg.WEIGHT_ONLY_MAX_ROWS or fit is None or (not asym and wq_type in ('int4', 'int8') and M > dg.fused_wq_min_rows(N, wq_type == 'int4')):
+  if M > dg.WEIGHT_ONLY_MAX_ROWS or fit is None or (wq_type in ('int4', 'int8') and M > dg.fused_wq_min_rows(N, wq_type == 'int4')):
     assert torch.equal(dg.dot_general(x_t, wq, DN, preferred_element_type=torch.bfloat16), out)
   # the dequantized operand itself, against the oracle's dequantize
   c = dg._Canon(x_t, wq, DN)
