@@ -319,9 +319,9 @@ QWIX_API int qwix_hip_gemm_bf16(const void* a, int64_t lda, const void* b, int64
 /* The same contraction with the int4 / int8 weight dequantized inside the GEMM (prefill with weight-only
  * quantization: _slow_dot_general, qwix/_src/core/dot_general.py:264-275, = dequantize, qarray.py:692-708, then a
  * float dot): out[m, n] = sum_k a[m, k] * bf16((q[n, k] - zp[k / group, n]) * s[k / group, n]).  a: (M, K) bf16, row
- * pitch lda elements; q: (N, K) of q_qtype in {INT4 (packed), INT8}, K-contiguous, row pitch ldq_bytes; s:
+ * pitch lda elements; q: (N, K) of q_qtype in {INT4 (packed), INT8, E4M3}, K-contiguous, row pitch ldq_bytes; s:
  * (K / group, N) in s_dtype (the product is formed in f32 and rounded to bf16 once); zp: int8 zero points laid out
- * like s, or NULL for symmetric weights.  K % 256 == 0, group % 64 == 0.  Bit-identical to qwix_hip_dequantize_rm
+ * like s, or NULL for symmetric (and e4m3) weights.  K % 256 == 0, group % 64 == 0.  Bit-identical to qwix_hip_dequantize_rm
  * (to bf16) followed by qwix_hip_gemm_bf16, without the dequantized copy of the weight. */
 QWIX_API int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, int64_t ldq_bytes, int q_qtype, int64_t M,
                           int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, const int8_t* zp,

@@ -703,13 +703,13 @@ def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_ty
   res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.scale.dtype)
   if res_t not in (torch.bfloat16, torch.float32):
     return None
-  if (_qtype_of(rhs) in (numerics.INT4, numerics.INT8) and _fused_wq_takes(c.M, c.N, b_is4)
+  if (_fused_wq_takes(c.M, c.N, b_is4)
       and c.K % 256 == 0 and (c.K // gb) % 64 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0):
-    # int4 / int8, with or without zero points: dequantized inside the GEMM's workgroups, slab by slab (the same
+    # int4 / int8 with or without zero points, e4m3: dequantized inside the GEMM's workgroups, slab by slab (the same
     # bf16 weights, the same products in the same order, no dequantized copy of the weight in memory)
     out = torch.empty(c.M, c.N, dtype=res_t, device=dev)
     _lib.call('qwix_hip_gemm_bf16_wq', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0),
-              _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
+              numerics.qtype_tag(_qtype_of(rhs)), c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
               _lib.ptr(zp), out.data_ptr(), _lib.float_tag(res_t), c.N, st)
     return out.reshape(c.out_shape)
   if fused_only:

@@ -2036,7 +2036,8 @@ __global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__
 // slab kt + 3 is requested in slab kt, behind the activations of slab kt + 2.  With 64-column tiles the upper half of
 // a load instruction's lanes repeats the lower half's rows (every wavefront issues one load per slab, so that all
 // count their requests alike); the repeated rows land in padding.  A byte b holds q = (b ^ 0x80) - 128 and
-// q * scale = fma(b ^ 0x80, scale, -128 scale), exact as for the nibbles.
+// q * scale = fma(b ^ 0x80, scale, -128 scale), exact as for the nibbles.  BITS = 9 stands for e4m3 weights: the same
+// bytes, converted by v_cvt_f32_fp8 and multiplied by the scale.
 // ZP: asymmetric weights, (q - zero_point) * scale with one int8 zero point per scale.  It is requested with the scale
 // and joins the offset of the storage format: bf16 scales fma(u, scale, -(offset + zp) scale), every term still exact
 // in f32 (nine bits times eight); f32 scales float(u - offset - zp) * scale, the integer difference first, because
@@ -2049,8 +2050,10 @@ __global__ void __launch_bounds__(512)
   static_assert(BN == 128 || BN == 64, "column tiles of 128 or 64");
   constexpr int BM = 256, WGN = 2, WN = BN / WGN, TM = 2, TN = WN / 32, NWAVES = 8;
   constexpr int BK = 128, NK = 4;  // bytes of an activation row per slab (64 elements); k-steps of 16 elements
-  static_assert(BITS == 4 || BITS == 8, "int4 or int8 weights");
-  constexpr bool W8 = BITS == 8;
+  static_assert(BITS == 4 || BITS == 8 || BITS == 9, "int4, int8 or (9) e4m3 weights");
+  constexpr bool W8 = BITS >= 8;   // one byte per weight
+  constexpr bool F8 = BITS == 9;   // e4m3: the byte converts to f32 directly; no offset, no zero point
+  static_assert(!(F8 && ZP), "float weights have no zero point");
   // raw weights: int4 two buffers of a superslab (BN x 128 bytes), int8 four of a slab (8 x 1 KB, one per wavefront)
   constexpr int A_STAGE = BM * BK, C_STAGE = BN * BK, R_STAGE = W8 ? 8 * 1024 : BN * 128;
   constexpr int C_BASE = 3 * A_STAGE, R_BASE = C_BASE + 2 * C_STAGE, LDS_BYTES = R_BASE + (W8 ? 4 : 2) * R_STAGE;  // <= 160 KB
@@ -2143,7 +2146,7 @@ __global__ void __launch_bounds__(512)
     }
   };
   constexpr int kSL = ZP ? 8 : 4;  // loads of one request_scales
-  constexpr int NRAW = NPT * BITS / 32;  // dwords of raw weights per thread and slab
+  constexpr int NRAW = NPT * (W8 ? 8 : 4) / 32;  // dwords of raw weights per thread and slab
   int craw[NRAW];
   uint32_t cout[NPT / 2];
   auto convert_read = [&](int kt) {
@@ -2179,7 +2182,12 @@ __global__ void __launch_bounds__(512)
       return __builtin_fmaf(static_cast<float>(u), sc, moff);
     };
     float f0, f1, f2, f3;
-    if constexpr (W8) {
+    if constexpr (F8) {
+      f0 = __builtin_amdgcn_cvt_f32_fp8(craw[q4], 0) * sc;
+      f1 = __builtin_amdgcn_cvt_f32_fp8(craw[q4], 1) * sc;
+      f2 = __builtin_amdgcn_cvt_f32_fp8(craw[q4], 2) * sc;
+      f3 = __builtin_amdgcn_cvt_f32_fp8(craw[q4], 3) * sc;
+    } else if constexpr (W8) {
       const uint32_t u = static_cast<uint32_t>(craw[q4]) ^ 0x80808080u;
       f0 = value(u & 0xFFu);
       f1 = value((u >> 8) & 0xFFu);
@@ -2552,8 +2560,9 @@ extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, 
                                      int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, const int8_t* zp,
                                      void* out, int out_dtype, int64_t ldo, void* stream) {
   if (!a || !q || !s || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/q/s/out");
-  if (q_qtype != QWIX_INT4 && q_qtype != QWIX_INT8)
-    return fail(QWIX_ERR_UNSUPPORTED, "weight qtype %d: int4 or int8", q_qtype);
+  if (q_qtype != QWIX_INT4 && q_qtype != QWIX_INT8 && q_qtype != QWIX_E4M3)
+    return fail(QWIX_ERR_UNSUPPORTED, "weight qtype %d: int4, int8 or e4m3", q_qtype);
+  if (q_qtype == QWIX_E4M3 && zp) return fail(QWIX_ERR_INVALID_ARGUMENT, "e4m3 weights have no zero point");
   if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || 2 * K > INT32_MAX)
     return fail(QWIX_ERR_INVALID_ARGUMENT, "bad GEMM shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
                 (long long)K);
@@ -2576,13 +2585,13 @@ extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, 
   hipStream_t st = static_cast<hipStream_t>(stream);
 #define QWIX_WQ_LAUNCH(OUTT, SBFF, BNN, BITS) \
   do {                                        \
-    if (zp) QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BNN, BITS, true); else QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BNN, BITS, false); \
+    if (zp) QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BNN, BITS, (BITS != 9)); else QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BNN, BITS, false); \
   } while (0)
 #define QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BNN, BITS, ZPP)                                                                 \
   do {                                                                                                               \
     auto kern = wgemm_wq_kernel<OUTT, SBFF, BNN, BITS, ZPP>;                                                         \
     /* activations 96 KB, converted weights 2 x BN x 128, raw weights 2 x BN x 128 (int8: 4 x 8 KB): <= 160 KB */    \
-    constexpr size_t smem = 3 * 256 * 128 + 2 * BNN * 128 + (BITS == 8 ? 4 * 8192 : 2 * BNN * 128);                  \
+    constexpr size_t smem = 3 * 256 * 128 + 2 * BNN * 128 + (BITS >= 8 ? 4 * 8192 : 2 * BNN * 128);                  \
     const dim3 grid(static_cast<unsigned>(((M + 255) / 256) * ((N + BNN - 1) / BNN)));                               \
     static LdsGrant granted;                                                                                         \
     if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;                           \
@@ -2596,7 +2605,9 @@ extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, 
   } while (0)
 #define QWIX_WQ_BITS(OUTT, SBFF)                                                                                     \
   do {                                                                                                               \
-    if (q_qtype == QWIX_INT4) QWIX_WQ_TILE(OUTT, SBFF, 4); else QWIX_WQ_TILE(OUTT, SBFF, 8);                         \
+    if (q_qtype == QWIX_INT4) QWIX_WQ_TILE(OUTT, SBFF, 4);                                                           \
+    else if (q_qtype == QWIX_INT8) QWIX_WQ_TILE(OUTT, SBFF, 8);                                                      \
+    else QWIX_WQ_TILE(OUTT, SBFF, 9); /* e4m3 */                                                                     \
   } while (0)
   if (out_dtype == QWIX_BF16) {
     if (s_dtype == QWIX_BF16) QWIX_WQ_BITS(QWIX_BF16, true); else QWIX_WQ_BITS(QWIX_BF16, false);

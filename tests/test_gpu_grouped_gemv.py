@@ -405,13 +405,13 @@ def test_bf16_gemm_against_float64(M, K, N, out_dtype):
 
 @pytest.mark.parametrize('sdt', [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
-@pytest.mark.parametrize('asym', [False, True])
+@pytest.mark.parametrize('wq_type,asym', [('int4', False), ('int4', True), ('int8', False), ('int8', True),
+                                          ('float8_e4m3fn', False)])
 @pytest.mark.parametrize('M,K,N,group', [(300, 256, 136, 128), (512, 1024, 1000, 256), (257, 2048, 520, 64), (2048, 4096, 1536, 128),
                                          (1, 512, 64, 512), (600, 512, 8400, 128), (1100, 256, 4100, 64)])
 def test_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, asym, wq_type, out_dtype, sdt):
   """qwix_hip_gemm_bf16_wq through the C ABI == qwix_hip_dequantize_rm (to bf16) + qwix_hip_gemm_bf16, bit for bit: the
-  same bf16 weights, the same MFMA, K walked in the same order; int4 and int8 weights, with and without zero points,
+  same bf16 weights, the same MFMA, K walked in the same order; int4, int8 (with and without zero points) and e4m3 weights,
   edges in M and N, one slab group (64), several; the last two shapes have more than 128 tiles of 256 x 128 and run those, the others tiles of
   256 x 64."""
   from qwix_amd import _lib
@@ -428,7 +428,8 @@ def test_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, asym, wq_type, o
   b, is4 = c.rhs_values(wq)
   sb, gb = c.rhs_scale(wq)
   assert is4 == (wq_type == 'int4') and gb == K // group
-  tag = _lib.INT4 if is4 else _lib.INT8
+  from qwix_amd.core import numerics
+  tag = numerics.qtype_tag(wq_type)
   st = _lib.stream_of(x_t)
   zp = dg._rhs_zero_point_i8(c, wq)[0] if asym else None
   assert (wq.zero_point is not None) == asym
@@ -462,7 +463,7 @@ def test_dequantizing_gemm_argument_checks():
                                    out.data_ptr(), od, ldo, None)
   assert call() == 0
   assert call(qt=_lib.INT4, ldq=K // 2) == 0
-  assert call(qt=_lib.E4M3) != 0 and b'int4 or int8' in L.qwix_hip_last_error()
+  assert call(qt=_lib.E4M3) == 0 and call(qt=7) != 0 and b'int4, int8 or e4m3' in L.qwix_hip_last_error()
   assert call(k=384) != 0 and b'multiple of 256' in L.qwix_hip_last_error()
   assert call(group=96) != 0 and b'multiple of 64' in L.qwix_hip_last_error()
   assert call(ldq=K // 2) != 0 and b'aligned' in L.qwix_hip_last_error()       # int8 rows need K bytes
