@@ -9,7 +9,7 @@ first).  Arguments are torch tensors / QArrays in HBM; `dimension_numbers` is
 What reaches a hand-written kernel:
   int8 x int8, e4m3 x e4m3 (per-row x per-column scales)          -> qwix_hip_qgemm
   int8 x int8/int4 with K-group scales (tile % 128 == 0)          -> qwix_hip_qgemm_grouped
-  bf16 activations x int4/int8 weight (weight-only, any group)    -> qwix_hip_gemv_wq up to 104..200 rows,
+  bf16 activations x int4/int8 weight (weight-only, any group)    -> qwix_hip_gemv_wq up to 56..120 rows,
       qwix_hip_gemm_bf16_wq (int4 up to 1024 rows, int8 up to one round of tiles),
       qwix_hip_dequantize_rm + qwix_hip_gemm_bf16 above
 Everything else on the slow path is dequantized by the HIP dequantize kernel and contracted by
@@ -659,13 +659,14 @@ _FUSED_W8_MAX_TILES = 256
 
 
 def fused_wq_min_rows(n: int, int4: bool = True) -> int:
-  """Rows above which one row tile of the dequantizing tile GEMM beats the decode kernel (`qwix_hip_gemv_wq`).  Its
-  time does not depend on the rows (K 4096: 50 us with the 64-column tiles such calls get); the decode kernel's
-  grows with them and falls with N.  K 4096, int4, 128 / 160 / 192 rows: N 14336 50 / 59 / 66 us, N 8192 - / - / 55.
-  int8 (tile GEMM 54 / 47 us at N 14336 / 4096), 96 / 128 / 192 rows: N 14336 54 / 66 / 96 us, N 4096 31 / 39 / 57."""
+  """Rows above which the dequantizing tile GEMM beats the decode kernel (`qwix_hip_gemv_wq`).  The time of one row
+  tile does not depend on the rows (K 4096, up to 128 rows, tiles of 128 x 64: int4 37 / 34 us at N 14336 / 4096, int8
+  33 / 28.5 us; 129-256 rows, tiles of 256 x 64: 50 us); the decode kernel's grows with them and falls with N
+  (K 4096, int4, 64 / 80 / 96 / 128 rows: N 14336 26 / 36 / 40 / 50 us, N 4096 21 / 23 / 28 / 35 us; int8, 48 / 64 / 96
+  rows: N 14336 31 / 35 / 51 us, N 4096 17 / 21 / 30 us)."""
   if int4:
-    return 144 if n >= 12288 else 200
-  return 104 if n >= 12288 else 160
+    return 80 if n >= 12288 else 120
+  return 56 if n >= 12288 else 88
 
 
 def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type, fused_only=False):

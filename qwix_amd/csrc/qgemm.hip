@@ -2042,26 +2042,28 @@ __global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__
 // and joins the offset of the storage format: bf16 scales fma(u, scale, -(offset + zp) scale), every term still exact
 // in f32 (nine bits times eight); f32 scales float(u - offset - zp) * scale, the integer difference first, because
 // (offset + zp) * scale would no longer be exact.
-template <int OUT, bool SBF, int BN, int BITS, bool ZP>
-__global__ void __launch_bounds__(512)
+// BM = 128 (four wavefronts, tiles of 128 x 64) is for calls of at most 128 rows: half the MFMAs and half the
+// activation loads per workgroup of the 256-row tile, whose upper half would multiply padding.
+template <int OUT, bool SBF, int BM, int BN, int BITS, bool ZP>
+__global__ void __launch_bounds__(BM * 2)
     wgemm_wq_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ Q, int64_t ldq,
                     const void* __restrict__ S, const int8_t* __restrict__ Z, int M, int N, int K, int group,
                     uint8_t* __restrict__ out, int64_t ldo) {
-  static_assert(BN == 128 || BN == 64, "column tiles of 128 or 64");
-  constexpr int BM = 256, WGN = 2, WN = BN / WGN, TM = 2, TN = WN / 32, NWAVES = 8;
+  static_assert((BM == 256 && (BN == 128 || BN == 64)) || (BM == 128 && BN == 64), "tiles of 256 x 128, 256 x 64, 128 x 64");
+  constexpr int WGN = 2, WN = BN / WGN, TM = 2, TN = WN / 32, NWAVES = BM / 32, NTHREADS = NWAVES * 64;
   constexpr int BK = 128, NK = 4;  // bytes of an activation row per slab (64 elements); k-steps of 16 elements
   static_assert(BITS == 4 || BITS == 8 || BITS == 9, "int4, int8 or (9) e4m3 weights");
   constexpr bool W8 = BITS >= 8;   // one byte per weight
   constexpr bool F8 = BITS == 9;   // e4m3: the byte converts to f32 directly; no offset, no zero point
   static_assert(!(F8 && ZP), "float weights have no zero point");
-  // raw weights: int4 two buffers of a superslab (BN x 128 bytes), int8 four of a slab (8 x 1 KB, one per wavefront)
-  constexpr int A_STAGE = BM * BK, C_STAGE = BN * BK, R_STAGE = W8 ? 8 * 1024 : BN * 128;
+  // raw weights: int4 two buffers of a superslab (BN x 128 bytes), int8 four of a slab (1 KB per wavefront)
+  constexpr int A_STAGE = BM * BK, C_STAGE = BN * BK, R_STAGE = W8 ? NWAVES * 1024 : BN * 128;
   constexpr int C_BASE = 3 * A_STAGE, R_BASE = C_BASE + 2 * C_STAGE, LDS_BYTES = R_BASE + (W8 ? 4 : 2) * R_STAGE;  // <= 160 KB
-  constexpr int NQ = W8 ? 1 : BN / 64;  // direct-to-LDS loads of weights per wavefront and request
-  constexpr int TPR = 512 / BN;     // converter threads per weight row: 4 or 8
+  constexpr int RPW = BN / NWAVES;  // weight rows per wavefront: 16 or 8
+  constexpr int NQ = W8 ? 1 : RPW / 8;  // direct-to-LDS loads of weights per wavefront and request
+  constexpr int TPR = NTHREADS / BN;    // converter threads per weight row: 4 or 8
   constexpr int NPT = 64 / TPR;     // elements per thread and slab: 16 or 8
   constexpr int NCQ = NPT / 4;      // conversion steps of four elements: 4 or 2
-  constexpr int RPW = BN / 8;       // weight rows per wavefront: 16 or 8
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -2580,28 +2582,31 @@ extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, 
     return fail(QWIX_ERR_INVALID_ARGUMENT, "bad output leading dimension %lld for N=%lld", (long long)ldo, (long long)N);
   if (M * lda * 2 >= (int64_t{1} << 31) || N * ldq_bytes >= (int64_t{1} << 31))
     return fail(QWIX_ERR_UNSUPPORTED, "operands beyond 2 GiB are not supported");
-  // 64-column tiles while 128-column ones would occupy at most half of the CUs
+  // 64-column tiles while 128-column ones would occupy at most half of the CUs; 128-row tiles for up to 128 rows
   const bool narrow = ((M + 255) / 256) * ((N + 127) / 128) <= 128;
+  const bool low = M <= 128;
   hipStream_t st = static_cast<hipStream_t>(stream);
-#define QWIX_WQ_LAUNCH(OUTT, SBFF, BNN, BITS) \
-  do {                                        \
-    if (zp) QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BNN, BITS, (BITS != 9)); else QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BNN, BITS, false); \
+#define QWIX_WQ_LAUNCH(OUTT, SBFF, BMM, BNN, BITS) \
+  do {                                             \
+    if (zp) QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BMM, BNN, BITS, (BITS != 9)); else QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BMM, BNN, BITS, false); \
   } while (0)
-#define QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BNN, BITS, ZPP)                                                                 \
+#define QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BMM, BNN, BITS, ZPP)                                                            \
   do {                                                                                                               \
-    auto kern = wgemm_wq_kernel<OUTT, SBFF, BNN, BITS, ZPP>;                                                         \
+    auto kern = wgemm_wq_kernel<OUTT, SBFF, BMM, BNN, BITS, ZPP>;                                                    \
     /* activations 96 KB, converted weights 2 x BN x 128, raw weights 2 x BN x 128 (int8: 4 x 8 KB): <= 160 KB */    \
-    constexpr size_t smem = 3 * 256 * 128 + 2 * BNN * 128 + (BITS >= 8 ? 4 * 8192 : 2 * BNN * 128);                  \
-    const dim3 grid(static_cast<unsigned>(((M + 255) / 256) * ((N + BNN - 1) / BNN)));                               \
+    constexpr size_t smem = 3 * BMM * 128 + 2 * BNN * 128 + (BITS >= 8 ? 4 * (BMM / 32) * 1024 : 2 * BNN * 128);      \
+    const dim3 grid(static_cast<unsigned>(((M + BMM - 1) / BMM) * ((N + BNN - 1) / BNN)));                           \
     static LdsGrant granted;                                                                                         \
     if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;                           \
-    kern<<<grid, 512, smem, st>>>(static_cast<const uint8_t*>(a), 2 * lda, static_cast<const uint8_t*>(q), ldq_bytes, s, \
+    kern<<<grid, 2 * BMM, smem, st>>>(static_cast<const uint8_t*>(a), 2 * lda, static_cast<const uint8_t*>(q), ldq_bytes, s, \
                                   zp, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K),                 \
                                   static_cast<int>(group), static_cast<uint8_t*>(out), ldo);                         \
   } while (0)
 #define QWIX_WQ_TILE(OUTT, SBFF, BITS)                                                                               \
   do {                                                                                                               \
-    if (narrow) QWIX_WQ_LAUNCH(OUTT, SBFF, 64, BITS); else QWIX_WQ_LAUNCH(OUTT, SBFF, 128, BITS);                    \
+    if (low) QWIX_WQ_LAUNCH(OUTT, SBFF, 128, 64, BITS);                                                              \
+    else if (narrow) QWIX_WQ_LAUNCH(OUTT, SBFF, 256, 64, BITS);                                                      \
+    else QWIX_WQ_LAUNCH(OUTT, SBFF, 256, 128, BITS);                                                                 \
   } while (0)
 #define QWIX_WQ_BITS(OUTT, SBFF)                                                                                     \
   do {                                                                                                               \

@@ -212,12 +212,14 @@ def test_weight_only_gemv_k_splits(M, K, N, group, wq_type):
 
 @pytest.mark.parametrize('wq_type', ['int4', 'int8'])
 @pytest.mark.parametrize('M,K,N', [(30, 1024, 520), (50, 4096, 14336), (130, 512, 6400)])
-def test_weight_only_rows_do_not_depend_on_the_batch(M, K, N, wq_type):
+def test_weight_only_rows_do_not_depend_on_the_batch(M, K, N, wq_type, monkeypatch):
   """More than 16 rows share a pass over the weights (2 tiles of 16 rows per workgroup, fewer wavefronts
   along K): the f32 partial sums meet in another order, nothing else changes, so the result equals the rows
-  computed 16 at a time up to that reordering."""
+  computed 16 at a time up to that reordering.  (The decode kernel for the whole batch: the operator's switch to
+  the dequantizing tile GEMM, which rounds every weight to bf16 first, is held off.)"""
   from qwix_amd.core import dot_general as dg
   from qwix_amd.core import qarray
+  monkeypatch.setattr(dg, 'fused_wq_min_rows', lambda n, int4=True: dg.WEIGHT_ONLY_MAX_ROWS)
   print('case gemv batch', M, K, N, wq_type, flush=True)
   _, x_t = util.make((M, K), O.BF16, seed=M + K)
   _, w_t = util.make((K, N), O.BF16, seed=M + K + 1, scale=0.02)
@@ -408,7 +410,8 @@ def test_bf16_gemm_against_float64(M, K, N, out_dtype):
 @pytest.mark.parametrize('wq_type,asym', [('int4', False), ('int4', True), ('int8', False), ('int8', True),
                                           ('float8_e4m3fn', False)])
 @pytest.mark.parametrize('M,K,N,group', [(300, 256, 136, 128), (512, 1024, 1000, 256), (257, 2048, 520, 64), (2048, 4096, 1536, 128),
-                                         (1, 512, 64, 512), (600, 512, 8400, 128), (1100, 256, 4100, 64)])
+                                         (1, 512, 64, 512), (600, 512, 8400, 128), (1100, 256, 4100, 64), (100, 1024, 520, 128),
+                                         (128, 512, 200, 64)])
 def test_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, asym, wq_type, out_dtype, sdt):
   """qwix_hip_gemm_bf16_wq through the C ABI == qwix_hip_dequantize_rm (to bf16) + qwix_hip_gemm_bf16, bit for bit: the
   same bf16 weights, the same MFMA, K walked in the same order; int4, int8 (with and without zero points) and e4m3 weights,
