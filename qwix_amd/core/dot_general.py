@@ -660,13 +660,13 @@ _FUSED_W8_MAX_TILES = 256
 
 def fused_wq_min_rows(n: int, int4: bool = True) -> int:
   """Rows above which the dequantizing tile GEMM beats the decode kernel (`qwix_hip_gemv_wq`).  The time of one row
-  tile does not depend on the rows (K 4096, up to 128 rows, tiles of 128 x 64: int4 37 / 34 us at N 14336 / 4096, int8
-  33 / 28.5 us; 129-256 rows, tiles of 256 x 64: 50 us); the decode kernel's grows with them and falls with N
-  (K 4096, int4, 64 / 80 / 96 / 128 rows: N 14336 26 / 36 / 40 / 50 us, N 4096 21 / 23 / 28 / 35 us; int8, 48 / 64 / 96
-  rows: N 14336 31 / 35 / 51 us, N 4096 17 / 21 / 30 us)."""
+  tile does not depend on the rows (K 4096, up to 128 rows, tiles of 128 x 64: int4 29 / 26 us at N 14336 / 4096, int8
+  29 / 25 us; 129-256 rows, tiles of 256 x 64: 45 us); the decode kernel's grows with them in steps of 16 rows and
+  falls with N (K 4096, int4, 64 / 80 / 96 / 128 rows: N 14336 26 / 35 / 38 / 48 us, N 4096 21 / 23 / 28 / 35 us; int8,
+  32 / 48 / 64 / 80 rows: N 14336 23 / 31 / 35 / 46 us, N 4096 12 / 17 / 21 / 26 us)."""
   if int4:
-    return 80 if n >= 12288 else 120
-  return 56 if n >= 12288 else 88
+    return 64 if n >= 12288 else 80
+  return 32 if n >= 12288 else 64
 
 
 def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type, fused_only=False):

@@ -2021,7 +2021,7 @@ __global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__
 // bf16: exact for bf16 scales, one more rounding for f32 scales, as qwix_hip_dequantize_rm does) -- and writes them
 // where the dense bf16 kernel expects the weight slab (same XOR swizzle), a quarter of the work in front of each of
 // the slab's four k-steps.  The activations go through three LDS stages by direct-to-LDS loads requested two slabs
-// ahead.  One barrier per slab; the wait in front of it is counted (vmcnt), so that the requests of the slab that
+// ahead (four stages, three slabs in the 128-row tile).  One barrier per slab; the wait in front of it is counted (vmcnt), so that the requests of the slab that
 // ends stay in flight: a full wait there costs a memory round trip per slab (87 us instead of 65 at 512 x 14336 x 4096).
 //   LDS is read and written through ext_vector types only (v4i, qwix_v2i).  Through HIP's struct vectors (uint2,
 // uint4) the compiler cannot tell the access from the destinations of the direct-to-LDS loads in flight and puts
@@ -2042,10 +2042,19 @@ __global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__
 // and joins the offset of the storage format: bf16 scales fma(u, scale, -(offset + zp) scale), every term still exact
 // in f32 (nine bits times eight); f32 scales float(u - offset - zp) * scale, the integer difference first, because
 // (offset + zp) * scale would no longer be exact.
-// BM = 128 (four wavefronts, tiles of 128 x 64) is for calls of at most 128 rows: half the MFMAs and half the
-// activation loads per workgroup of the 256-row tile, whose upper half would multiply padding.
+// BM = 128 (tiles of 128 x 64) is for calls of at most 128 rows: half the MFMAs and half the activation loads per
+// workgroup of the 256-row tile, whose upper half would multiply padding.  Its eight wavefronts split the work: four
+// multiply (64 x 32 each) and load nothing, four only request the operands, three slabs ahead, and wait for them; a
+// wavefront issues in order, so one that requests and multiplies stands at a load instruction while the memory
+// pipeline is full and its SIMD's matrix core idles (requests, conversion and MFMAs added up to the run time: 10 +
+// 4 + 7 us on top of 9.4 us of skeleton at 128 x 4096 x 4096, int8; 34 -> 29 us at 128 x 14336 x 4096).  The
+// requesting wavefronts also dequantize int4 weights (35.6 -> 29.3 us against 32.6 with the conversion between the
+// MFMAs); bytes convert faster between the MFMAs (28.5 against 32.8 us).  The requesting wavefronts end after the last
+// slab: a wavefront that has ended no longer counts at the workgroup's barriers.
+//   In the 256-row tiles every wavefront requests and multiplies; there the four activation loads of a slab are issued
+// one per k-step instead of together (512 x 4096 x 4096: int4 47 -> 42 us, int8 50 -> 45 us).
 template <int OUT, bool SBF, int BM, int BN, int BITS, bool ZP>
-__global__ void __launch_bounds__(BM * 2)
+__global__ void __launch_bounds__(512)
     wgemm_wq_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ Q, int64_t ldq,
                     const void* __restrict__ S, const int8_t* __restrict__ Z, int M, int N, int K, int group,
                     uint8_t* __restrict__ out, int64_t ldo) {
@@ -2058,7 +2067,10 @@ __global__ void __launch_bounds__(BM * 2)
   static_assert(!(F8 && ZP), "float weights have no zero point");
   // raw weights: int4 two buffers of a superslab (BN x 128 bytes), int8 four of a slab (1 KB per wavefront)
   constexpr int A_STAGE = BM * BK, C_STAGE = BN * BK, R_STAGE = W8 ? NWAVES * 1024 : BN * 128;
-  constexpr int C_BASE = 3 * A_STAGE, R_BASE = C_BASE + 2 * C_STAGE, LDS_BYTES = R_BASE + (W8 ? 4 : 2) * R_STAGE;  // <= 160 KB
+  // slabs between the request of activations and their use; the 128-row tile has the LDS for one more
+  constexpr int AL = BM == 128 ? 3 : 2, AST = AL + 1;
+  static_assert(AL == 2 || AL == 3, "the last four slabs are the only special ones");
+  constexpr int C_BASE = AST * A_STAGE, R_BASE = C_BASE + 2 * C_STAGE, LDS_BYTES = R_BASE + (W8 ? 4 : 2) * R_STAGE;  // <= 160 KB
   constexpr int RPW = BN / NWAVES;  // weight rows per wavefront: 16 or 8
   constexpr int NQ = W8 ? 1 : RPW / 8;  // direct-to-LDS loads of weights per wavefront and request
   constexpr int TPR = NTHREADS / BN;    // converter threads per weight row: 4 or 8
@@ -2068,6 +2080,13 @@ __global__ void __launch_bounds__(BM * 2)
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
+  // SPEC: as many wavefronts again that only request the operands (rows and weight rows of wavefront wave - NWAVES)
+  constexpr bool SPEC = BM == 128;
+  const bool loader = SPEC && wave >= NWAVES;
+  // who dequantizes: the requesting wavefronts for int4 (measured 32.6 -> 30.2 us at 128 x 14336 x 4096), the multiplying
+  // ones for bytes (30.4 against 32.8 us)
+  constexpr bool LC = SPEC && !W8;
+  const int ldw = SPEC ? (wave & (NWAVES - 1)) : wave;
   int tile_m, tile_n;
   tile_coords((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
@@ -2085,38 +2104,39 @@ __global__ void __launch_bounds__(BM * 2)
   uint32_t goffa[4], goffq[NQ];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int row = wave * 32 + j * 8 + lr;
+    const int row = ldw * 32 + j * 8 + lr;
     goffa[j] = static_cast<uint32_t>(min(m0 + row, M - 1)) * static_cast<uint32_t>(lda) + (((lane & 7) ^ swz8(row)) << 4);
   }
 #pragma unroll
   for (int j = 0; j < NQ; ++j) {
     if constexpr (W8) {  // 16 rows x 64 bytes per instruction (64-column tiles: 8 rows, twice)
-      const int row = wave * RPW + ((lane >> 2) & (RPW - 1));
+      const int row = ldw * RPW + ((lane >> 2) & (RPW - 1));
       goffq[j] = static_cast<uint32_t>(min(n0 + row, N - 1)) * static_cast<uint32_t>(ldq) + ((lane & 3) << 4);
     } else {
-      const int row = wave * RPW + j * 8 + lr;
+      const int row = ldw * RPW + j * 8 + lr;
       goffq[j] = static_cast<uint32_t>(min(n0 + row, N - 1)) * static_cast<uint32_t>(ldq) + (((lane & 7) ^ swz8(row)) << 4);
     }
   }
   auto issue_a = [&](int kt, int stage) {  // 4 loads
     const uint8_t* gk = A + kt * BK;
-    uint8_t* dst = smem + stage * A_STAGE + wave * 32 * BK;
+    uint8_t* dst = smem + stage * A_STAGE + ldw * 32 * BK;
 #pragma unroll
     for (int j = 0; j < 4; ++j) QWIX_GLDS16(gk + goffa[j], dst + j * 1024);
   };
   auto issue_raw = [&](int ss) {  // int4: superslab ss (elements 256 ss ..), NQ loads; int8: slab ss, one load
     if constexpr (W8) {
-      QWIX_GLDS16(Q + ss * 64 + goffq[0], smem + R_BASE + (ss & 3) * R_STAGE + wave * 1024);
+      QWIX_GLDS16(Q + ss * 64 + goffq[0], smem + R_BASE + (ss & 3) * R_STAGE + ldw * 1024);
     } else {
       const uint8_t* gq = Q + ss * 128;
-      uint8_t* dst = smem + R_BASE + (ss & 1) * R_STAGE + wave * RPW * 128;
+      uint8_t* dst = smem + R_BASE + (ss & 1) * R_STAGE + ldw * RPW * 128;
 #pragma unroll
       for (int j = 0; j < NQ; ++j) QWIX_GLDS16(gq + goffq[j], dst + j * 1024);
     }
   };
 
   // ---- converter: thread -> (weight row, NPT of the slab's 64 elements)
-  const int crow = tid / TPR, cpart = tid % TPR;
+  const int ctid = tid & (NTHREADS - 1);
+  const int crow = ctid / TPR, cpart = ctid % TPR;
   const char* const sptr = static_cast<const char*>(S) + static_cast<int64_t>(min(n0 + crow, N - 1)) * (SBF ? 2 : 4);
   const int64_t s_group_pitch = static_cast<int64_t>(N) * (SBF ? 2 : 4);
   // The scales of four slabs are requested at once, a superslab ahead, by untracked loads (valid once a later
@@ -2254,71 +2274,114 @@ __global__ void __launch_bounds__(BM * 2)
   int sta = 0;  // LDS stage of the activations of the slab being multiplied: kt % 3
   // One slab, J = kt % 4: requests activations two slabs ahead (and, at J == 0, the packed weights and scales of
   // the next superslab), converts the weights of slab kt + 1 between the k-steps of slab kt.
-  auto slab = [&](int kt, auto J, auto LAST) {
-    constexpr int j = decltype(J)::value;
+  // role 0: a wavefront requests and multiplies; 1: multiplies only; 2: requests only
+  constexpr auto requests_of = [](int j, bool last, int role) constexpr {  // load instructions issued in slab j of four
+    const bool converts = role == 0 || (role == 2) == LC;
+    const bool la = role != 1 && (!last || j < 4 - AL), ls = converts && !last && j == 0;
+    const bool lw = role != 1 && (W8 ? (!last || j < 3 - AL) : (!last && j == 0));
+    return (la ? 4 : 0) + (lw ? NQ : 0) + (ls ? kSL : 0);
+  };
+  auto slab = [&](int kt, auto J, auto LAST, auto ROLE) {
+    constexpr int j = decltype(J)::value, role = decltype(ROLE)::value;
     constexpr bool last = decltype(LAST)::value;  // the last four slabs: nothing further to request after two
+    constexpr bool requests = role != 1, multiplies = role != 2, converts = role == 0 || (role == 2) == LC;
     constexpr bool more = !(last && j == 3);
-    constexpr bool loads_a = !last || j < 2, loads_s = !last && j == 0;
-    constexpr bool loads_w = W8 ? (!last || j == 0) : loads_s;  // int8: slab kt + 3; int4: the next superslab
+    constexpr bool loads_a = requests && (!last || j < 4 - AL), loads_s = converts && !last && j == 0;
+    // int8: slab kt + AL + 1; int4: the next superslab
+    constexpr bool loads_w = requests && (W8 ? (!last || j < 3 - AL) : (!last && j == 0));
+    constexpr bool SPREAD = multiplies;  // a wavefront that also multiplies issues one activation load per k-step
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (loads_a) issue_a(kt + 2, sta == 0 ? 2 : sta - 1);
-    if constexpr (loads_w) issue_raw(W8 ? kt + 3 : (kt >> 2) + 1);
+    const int sta_req = sta == 0 ? AST - 1 : sta - 1;
+    if constexpr (loads_a && !SPREAD) issue_a(kt + AL, sta_req);
+    if constexpr (loads_w) issue_raw(W8 ? kt + AL + 1 : (kt >> 2) + 1);
     if constexpr (loads_s) request_scales(sc_next, zp_next);
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (j == 2 && !last) pin_scales(sc_next, zp_next);  // requested at j == 0, covered by the wait that ended j == 1
-    const float sc = scale_value(j == 3 ? sc_next[0] : sc_cur[(j + 1) & 3]);
-    const int zc = j == 3 ? zp_next[0] : zp_cur[(j + 1) & 3];
-    if constexpr (more) convert_read(kt + 1);
-#pragma unroll
-    for (int ks = 0; ks < NK; ++ks) {
-      if (ks + 1 < NK) read_frags(sta, j & 1, ks + 1, (ks + 1) & 1);
-      if constexpr (more) convert_quarter(ks, sc, zc);
-      mfma_step(ks & 1);
+    float sc = 0.f;
+    int zc = 0;
+    if constexpr (converts) {
+      if constexpr (j == AL && !last) pin_scales(sc_next, zp_next);  // requested at j == 0, covered by the wait that ended j == AL - 1
+      sc = scale_value(j == 3 ? sc_next[0] : sc_cur[(j + 1) & 3]);
+      zc = j == 3 ? zp_next[0] : zp_cur[(j + 1) & 3];
+      if constexpr (more) convert_read(kt + 1);
     }
-    if constexpr (more) convert_write(kt + 1);
-    end_of_slab(integral_constant<int, (loads_a ? 4 : 0) + (loads_w ? NQ : 0) + (loads_s ? kSL : 0)>{});
-    sta = sta == 2 ? 0 : sta + 1;
-    if constexpr (more) read_frags(sta, (j + 1) & 1, 0, 0);
-  };
-
-  // ---- prologue: packed weights and scales of slabs 0..3 (int8: 0..2), activations of slabs 0 and 1; slab 0 converted
-  issue_raw(0);
-  if constexpr (W8) {
-    issue_raw(1);
-    issue_raw(2);
-  }
-  request_scales(sc_cur, zp_cur);
-  issue_a(0, 0);
-  issue_a(1, 1);
-  end_of_slab(integral_constant<int, 0>{});
-  pin_scales(sc_cur, zp_cur);
-  convert_read(0);
+    if constexpr (role == 2 && converts && more) {  // the whole conversion while the requests are under way
 #pragma unroll
-  for (int q4 = 0; q4 < 4; ++q4) convert_quarter(q4, scale_value(sc_cur[0]), zp_cur[0]);
-  convert_write(0);
-  end_of_slab(integral_constant<int, 0>{});
-  read_frags(0, 0, 0, 0);
-
+      for (int q4 = 0; q4 < 4; ++q4) convert_quarter(q4, sc, zc);
+    }
+    if constexpr (multiplies) {
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks) {
+        if constexpr (loads_a && SPREAD)  // one of the four activation loads per k-step
+          QWIX_GLDS16(A + (kt + AL) * BK + goffa[ks], smem + sta_req * A_STAGE + ldw * 32 * BK + ks * 1024);
+        if (ks + 1 < NK) read_frags(sta, j & 1, ks + 1, (ks + 1) & 1);
+        if constexpr (converts && more) convert_quarter(ks, sc, zc);
+        mfma_step(ks & 1);
+      }
+    }
+    if constexpr (converts && more) convert_write(kt + 1);
+    // in flight across the barrier: the requests of this slab and of the AL - 2 before it
+    constexpr int before = AL == 3 ? requests_of((j + 3) & 3, last && j > 0, role) : 0;
+    end_of_slab(integral_constant<int, requests_of(j, last, role) + before>{});
+    sta = sta == AST - 1 ? 0 : sta + 1;
+    if constexpr (multiplies && more) read_frags(sta, (j + 1) & 1, 0, 0);
+  };
   using I0 = integral_constant<int, 0>;
   using I1 = integral_constant<int, 1>;
   using I2 = integral_constant<int, 2>;
   using I3 = integral_constant<int, 3>;
-  int kt = 0;
-  for (; kt + 4 < KT; kt += 4) {
-    slab(kt, I0{}, std::false_type{});
-    slab(kt + 1, I1{}, std::false_type{});
-    slab(kt + 2, I2{}, std::false_type{});
-    slab(kt + 3, I3{}, std::false_type{});
+  auto slabs = [&](auto ROLE) {  // every role passes the same K / 64 barriers
+    int kt = 0;
+    for (; kt + 4 < KT; kt += 4) {
+      slab(kt, I0{}, std::false_type{}, ROLE);
+      slab(kt + 1, I1{}, std::false_type{}, ROLE);
+      slab(kt + 2, I2{}, std::false_type{}, ROLE);
+      slab(kt + 3, I3{}, std::false_type{}, ROLE);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      sc_cur[e] = sc_next[e];
-      zp_cur[e] = zp_next[e];
+      for (int e = 0; e < 4; ++e) {
+        sc_cur[e] = sc_next[e];
+        zp_cur[e] = zp_next[e];
+      }
     }
+    slab(kt, I0{}, std::true_type{}, ROLE);
+    slab(kt + 1, I1{}, std::true_type{}, ROLE);
+    slab(kt + 2, I2{}, std::true_type{}, ROLE);
+    slab(kt + 3, I3{}, std::true_type{}, ROLE);
+  };
+
+  // ---- prologue: packed weights of slabs 0..3 (int8: 0..AL), activations of slabs 0..AL - 1, scales; slab 0 converted.
+  // Two barriers for every role.
+  const bool converter = !SPEC || loader == LC;  // wave-uniform
+  if (!SPEC || loader) {
+    issue_raw(0);
+    if constexpr (W8) {
+#pragma unroll
+      for (int i = 1; i <= AL; ++i) issue_raw(i);
+    }
+#pragma unroll
+    for (int i = 0; i < AL; ++i) issue_a(i, i);
   }
-  slab(kt, I0{}, std::true_type{});
-  slab(kt + 1, I1{}, std::true_type{});
-  slab(kt + 2, I2{}, std::true_type{});
-  slab(kt + 3, I3{}, std::true_type{});
+  // every wavefront requests them: registers of loads in flight must not pass the join of a branch
+  request_scales(sc_cur, zp_cur);
+  end_of_slab(integral_constant<int, 0>{});
+  pin_scales(sc_cur, zp_cur);
+  if (converter) {
+    convert_read(0);
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) convert_quarter(q4, scale_value(sc_cur[0]), zp_cur[0]);
+    convert_write(0);
+  }
+  end_of_slab(integral_constant<int, 0>{});
+  if constexpr (SPEC) {
+    if (loader) {
+      slabs(I2{});
+      return;  // a wavefront that has ended no longer counts at the workgroup's barriers
+    }
+    read_frags(0, 0, 0, 0);
+    slabs(I1{});
+  } else {
+    read_frags(0, 0, 0, 0);
+    slabs(I0{});
+  }
 
   float sav[TM];
   float sbv[TN][4][4];
@@ -2594,11 +2657,11 @@ extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, 
   do {                                                                                                               \
     auto kern = wgemm_wq_kernel<OUTT, SBFF, BMM, BNN, BITS, ZPP>;                                                    \
     /* activations 96 KB, converted weights 2 x BN x 128, raw weights 2 x BN x 128 (int8: 4 x 8 KB): <= 160 KB */    \
-    constexpr size_t smem = 3 * BMM * 128 + 2 * BNN * 128 + (BITS >= 8 ? 4 * (BMM / 32) * 1024 : 2 * BNN * 128);      \
+    constexpr size_t smem = (BMM == 128 ? 4 : 3) * BMM * 128 + 2 * BNN * 128 + (BITS >= 8 ? 4 * (BMM / 32) * 1024 : 2 * BNN * 128);      \
     const dim3 grid(static_cast<unsigned>(((M + BMM - 1) / BMM) * ((N + BNN - 1) / BNN)));                           \
     static LdsGrant granted;                                                                                         \
     if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;                           \
-    kern<<<grid, 2 * BMM, smem, st>>>(static_cast<const uint8_t*>(a), 2 * lda, static_cast<const uint8_t*>(q), ldq_bytes, s, \
+    kern<<<grid, 512, smem, st>>>(static_cast<const uint8_t*>(a), 2 * lda, static_cast<const uint8_t*>(q), ldq_bytes, s, \
                                   zp, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K),                 \
                                   static_cast<int>(group), static_cast<uint8_t*>(out), ldo);                         \
   } while (0)
