@@ -877,6 +877,7 @@ WORKLOADS = {
     'c2_gemv_w4_m32': lambda: GemvW4('c2_gemv_w4_m32', 32, 4096, 14336, 128),
     'c2_w4a16_prefill_m2048': lambda: WeightOnlyPrefill('c2_w4a16_prefill_m2048', 2048, 4096, 14336, 128),
     'c2_w4a16_prefill_m512': lambda: WeightOnlyPrefill('c2_w4a16_prefill_m512', 512, 4096, 14336, 128),
+    'c2_w4a16_prefill_m128': lambda: WeightOnlyPrefill('c2_w4a16_prefill_m128', 128, 4096, 14336, 128),
     'c4_quantize_weight_fp8': lambda: QuantizeWeight('c4_quantize_weight_fp8', 8192, 28672, 'float8_e4m3fn'),
     'c5_quantize_weight_int4_g128': lambda: QuantizeWeight('c5_quantize_weight_int4_g128', 8192, 8192, 'int4', 128),
     'c3_quantize_weight_int8': lambda: QuantizeWeight('c3_quantize_weight_int8', 4096, 4096, 'int8'),
@@ -895,7 +896,7 @@ WORKLOADS = {
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
 }
 DEFAULT = 'c3_int8_w8a8_4096'
-EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'c2_w4a16_prefill_m2048', 'c2_w4a16_prefill_m512', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
+EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'c2_w4a16_prefill_m2048', 'c2_w4a16_prefill_m512', 'c2_w4a16_prefill_m128', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
          'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'moe_ragged_int8_8x1024',
          'moe_ragged_int8_64x128', 'moe_decode_int8_64x4', 'quantize_weight_fp8_block128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 
