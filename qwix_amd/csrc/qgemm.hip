@@ -2217,7 +2217,11 @@ __global__ void __launch_bounds__(512)
       f3 = value(u >> 24);
     } else {
       const uint32_t w = static_cast<uint32_t>(craw[q4 >> 1]) ^ 0x88888888u;
-      const uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
+      uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
+      // opaque to the optimizer: it would fold the masks into one bit-field extract per nibble in front of the byte
+      // conversion (v_bfe_u32 + v_cvt_f32_ubyte0) instead of converting the masked words' bytes in place
+      asm("" : "+v"(even));
+      asm("" : "+v"(odd));
       const int b0 = (q4 & 1) * 16;
       f0 = value((even >> b0) & 0xFFu);
       f1 = value((odd >> b0) & 0xFFu);
