@@ -411,7 +411,8 @@ def test_bf16_gemm_against_float64(M, K, N, out_dtype):
                                           ('float8_e4m3fn', False)])
 @pytest.mark.parametrize('M,K,N,group', [(300, 256, 136, 128), (512, 1024, 1000, 256), (257, 2048, 520, 64), (2048, 4096, 1536, 128),
                                          (1, 512, 64, 512), (600, 512, 8400, 128), (1100, 256, 4100, 64), (100, 1024, 520, 128),
-                                         (128, 512, 200, 64), (130, 512, 40, 128), (7, 768, 24, 256)])
+                                         (128, 512, 200, 64), (130, 512, 40, 128), (7, 768, 24, 256),
+                                         (64, 256, 72, 64), (96, 4096, 200, 128), (33, 1280, 64, 128)])
 def test_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, asym, wq_type, out_dtype, sdt):
   """qwix_hip_gemm_bf16_wq through the C ABI == qwix_hip_dequantize_rm (to bf16) + qwix_hip_gemm_bf16, bit for bit: the
   same bf16 weights, the same MFMA, K walked in the same order; int4, int8 (with and without zero points) and e4m3 weights,
