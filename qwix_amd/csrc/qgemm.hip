@@ -2021,8 +2021,9 @@ __global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__
 // bf16: exact for bf16 scales, one more rounding for f32 scales, as qwix_hip_dequantize_rm does) -- and writes them
 // where the dense bf16 kernel expects the weight slab (same XOR swizzle), a quarter of the work in front of each of
 // the slab's four k-steps.  The activations go through three LDS stages by direct-to-LDS loads requested two slabs
-// ahead (four stages, three slabs in the 128-row tile).  One barrier per slab; the wait in front of it is counted (vmcnt), so that the requests of the slab that
-// ends stay in flight: a full wait there costs a memory round trip per slab (87 us instead of 65 at 512 x 14336 x 4096).
+// ahead (four stages, three slabs in the 128-row tile).  One barrier per slab; the wait in front of it is counted
+// (vmcnt), so that the requests of the slab that ends (in the 128-row tile: and of the one before) stay in flight: a
+// full wait there costs a memory round trip per slab (87 us instead of 65 at 512 x 14336 x 4096).
 //   LDS is read and written through ext_vector types only (v4i, qwix_v2i).  Through HIP's struct vectors (uint2,
 // uint4) the compiler cannot tell the access from the destinations of the direct-to-LDS loads in flight and puts
 // an s_waitcnt vmcnt(0) in front of it, which turns every counted wait into a full one.
@@ -2033,11 +2034,12 @@ __global__ void __launch_bounds__(256) ksum_i8_kernel(const int8_t* __restrict__
 // both halve, while its activation traffic stays.
 // BITS = 8: int8 weights.  A row's 128-byte line would hold only two slabs, too few to request a buffer ahead, so
 // they come as 64-byte pieces, one slab per request (16 rows per load instruction), into a ring of four buffers:
-// slab kt + 3 is requested in slab kt, behind the activations of slab kt + 2.  With 64-column tiles the upper half of
+// slab kt + 3 is requested in slab kt, behind the activations of slab kt + 2 (128-row tile: kt + 4 behind kt + 3, into
+// the buffer that was read in slab kt - 1).  With 64-column tiles on eight requesting wavefronts the upper half of
 // a load instruction's lanes repeats the lower half's rows (every wavefront issues one load per slab, so that all
 // count their requests alike); the repeated rows land in padding.  A byte b holds q = (b ^ 0x80) - 128 and
 // q * scale = fma(b ^ 0x80, scale, -128 scale), exact as for the nibbles.  BITS = 9 stands for e4m3 weights: the same
-// bytes, converted by v_cvt_f32_fp8 and multiplied by the scale.
+// bytes, converted by v_cvt_pk_f32_fp8 (two per instruction) and multiplied by the scale.
 // ZP: asymmetric weights, (q - zero_point) * scale with one int8 zero point per scale.  It is requested with the scale
 // and joins the offset of the storage format: bf16 scales fma(u, scale, -(offset + zp) scale), every term still exact
 // in f32 (nine bits times eight); f32 scales float(u - offset - zp) * scale, the integer difference first, because
