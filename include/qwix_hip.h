@@ -337,7 +337,7 @@ QWIX_API int qwix_hip_dequantize_rm(const void* qvalue, int qtype, int64_t outer
 
 /* Weight-only skinny GEMM (the reference's _slow_dot_general, dot_general.py:264-275, with
  * the dequantize fused): out[m,n] = sum_k x[m,k] * (q[k,n] * s[k/group, n]).
- *   x   (M,K) bf16 row-major; q int4/int8 K-contiguous rows (n*ldb_bytes); s (K/group, N)
+ *   x   (M,K) bf16 row-major; q int4/int8/e4m3 K-contiguous rows (n*ldb_bytes); s (K/group, N)
  *   M <= 64 is the intended range (decode); group multiple of 128 or == K.
  */
 QWIX_API int qwix_hip_gemv_wq(const void* x, int64_t ldx, const void* q, int64_t ldb_bytes, int b_qtype,

@@ -9,8 +9,8 @@ first).  Arguments are torch tensors / QArrays in HBM; `dimension_numbers` is
 What reaches a hand-written kernel:
   int8 x int8, e4m3 x e4m3 (per-row x per-column scales)          -> qwix_hip_qgemm
   int8 x int8/int4 with K-group scales (tile % 128 == 0)          -> qwix_hip_qgemm_grouped
-  bf16 activations x int4/int8 weight (weight-only, any group)    -> qwix_hip_gemv_wq up to 56..120 rows,
-      qwix_hip_gemm_bf16_wq (int4 up to 1024 rows, int8 up to one round of tiles),
+  bf16 activations x int4/int8/e4m3 weight (weight-only, any group) -> qwix_hip_gemv_wq up to 32..80 rows,
+      qwix_hip_gemm_bf16_wq (int4 up to 1024 rows, int8 and e4m3 up to one round of tiles),
       qwix_hip_dequantize_rm + qwix_hip_gemm_bf16 above
 Everything else on the slow path is dequantized by the HIP dequantize kernel and contracted by
 the vendor float GEMM.  Unsupported fast-path combinations raise; they never change path silently.
@@ -515,12 +515,14 @@ def _rhs_zero_point_i8(c: '_Canon', rhs: QArray) -> tuple[torch.Tensor, int]:
 
 def _weight_only_fit(lhs, rhs, dimension_numbers):
   """The canonical form when the fused weight-only kernels (dequantize in registers, bf16 MFMA) take this pair,
-  else None.  The conditions are the kernels' own: a bf16 activation, an int4/int8 weight whose scales (and zero
+  else None.  The conditions are the kernels' own: a bf16 activation, an int4 / int8 / e4m3 weight whose scales (and zero
   points, if any, in the same groups) are tiled along the last contracting axis only, in groups that are
   multiples of 128."""
   if not (_is_float_array(lhs) and lhs.dtype == torch.bfloat16 and isinstance(rhs, QArray)):
     return None
-  if _qtype_of(rhs) not in (numerics.INT4, numerics.INT8):
+  if _qtype_of(rhs) not in (numerics.INT4, numerics.INT8, numerics.E4M3):
+    return None
+  if _qtype_of(rhs) == numerics.E4M3 and rhs.zero_point is not None:
     return None
   c = _Canon(lhs, rhs, dimension_numbers)
   if rhs.zero_point is not None and tuple(rhs.zero_point.shape) != tuple(rhs.scale.shape):
@@ -565,7 +567,7 @@ def _decode_plan(lhs, rhs, dimension_numbers):
     b, b_is4 = c.rhs_values(rhs)
     sb, gb = c.rhs_scale(rhs)
     zp = _rhs_zero_point_i8(c, rhs)[0] if rhs.zero_point is not None else None
-    plan = (b, _lib.INT4 if b_is4 else _lib.INT8, sb, _lib.float_tag(sb.dtype), zp, c.N, c.K, c.K // gb,
+    plan = (b, numerics.qtype_tag(_qtype_of(rhs)), sb, _lib.float_tag(sb.dtype), zp, c.N, c.K, c.K // gb,
             fused_wq_min_rows(c.N, b_is4))
   _DECODE_PLANS[key] = (weakref.ref(rhs, lambda _, k=key: _DECODE_PLANS.pop(k, None)),
                         _weight_signature(rhs), plan)
@@ -624,11 +626,11 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
     if rhs.zero_point is not None:  # asymmetric weights: (q - zp) * scale, the zero point per group and column
       zp, _ = _rhs_zero_point_i8(c, rhs)
       _lib.call('qwix_hip_gemv_wq_zp', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0),
-                _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
+                numerics.qtype_tag(_qtype_of(rhs)), c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
                 zp.data_ptr(), out.data_ptr(), _lib.float_tag(res_t), c.N, _lib.stream_of(x))
       return out.reshape(c.out_shape)
     _lib.call('qwix_hip_gemv_wq', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0),
-              _lib.INT4 if b_is4 else _lib.INT8, c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
+              numerics.qtype_tag(_qtype_of(rhs)), c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
               out.data_ptr(), _lib.float_tag(res_t), c.N, _lib.stream_of(x))
     return out.reshape(c.out_shape)
   out = _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type)

@@ -1,4 +1,4 @@
-// Weight-only skinny GEMM (decode): bf16 activations x int4/int8 group-quantized weights.
+// Weight-only skinny GEMM (decode): bf16 activations x int4 / int8 / e4m3 group-quantized weights.
 //
 //   out[m,n] = sum_g s[g,n] * sum_{k in g} x[m,k] * q[n,k]         M small (16 rows per pass)
 //
@@ -7,7 +7,8 @@
 // products run on v_mfma_f32_16x16x32_bf16 with the weights converted to bf16 in registers, in
 // offset binary so that the conversion is one or two bit-ops per pair of weights:
 //   int4: (nibble ^ 8) lands in the mantissa of bf16 128.0, giving 128 + (q + 8) exactly;
-//   int8: (byte ^ 0x80) is converted with v_cvt_f32_ubyte and truncated to bf16 (exact below 256).
+//   int8: (byte ^ 0x80) is converted with v_cvt_f32_ubyte and truncated to bf16 (exact below 256);
+//   e4m3: v_cvt_pk_f32_fp8, truncated to bf16 (exact: four significant bits), no offset.
 // The offset is removed by seeding each accumulator with -offset * rowsum(x), which four MFMAs against
 // a constant operand produce in the accumulator's own layout.
 // A workgroup is 16 wavefronts that split K; each handles NT tiles of 16 output columns with two K
@@ -173,9 +174,11 @@ __device__ __forceinline__ void prepare_x(Block<BQT, NT, RT>& b, v4f (&base)[RT]
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     base[rt] = v4f{0.f, 0.f, 0.f, 0.f};
+    if constexpr (BQT != QWIX_E4M3) {  // float weights carry no offset
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      base[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[rt][j]), as_bf16x8(negoff), base[rt], 0, 0, 0);
+      for (int j = 0; j < 4; ++j)
+        base[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xf[rt][j]), as_bf16x8(negoff), base[rt], 0, 0, 0);
+    }
     if constexpr (ZP) {
       const v4u ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
       sumx[rt] = v4f{0.f, 0.f, 0.f, 0.f};
@@ -205,6 +208,15 @@ __device__ __forceinline__ void compute_tile(const Block<BQT, NT, RT>& b, const 
       w[1] = ((u >> 4) & 0x000F000Fu) ^ 0x43084308u;   // (k1, k5)
       w[2] = ((u >> 8) & 0x000F000Fu) ^ 0x43084308u;   // (k2, k6)
       w[3] = ((u >> 12) & 0x000F000Fu) ^ 0x43084308u;  // (k3, k7)
+    } else if constexpr (BQT == QWIX_E4M3) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        // an e4m3 value has 4 significant bits: the upper half of its f32 is its bf16
+        const int u = static_cast<int>(b.wq[t][j >> 1][2 * (j & 1) + h]);
+        const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(u, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8(u, true);
+        w[2 * h] = __builtin_amdgcn_perm(__float_as_uint(lo[1]), __float_as_uint(lo[0]), 0x07060302);
+        w[2 * h + 1] = __builtin_amdgcn_perm(__float_as_uint(hi[1]), __float_as_uint(hi[0]), 0x07060302);
+      }
     } else {
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
@@ -395,8 +407,9 @@ static int gemv_wq_impl(const void* x, int64_t ldx, const void* q, int64_t ldb_b
   if (!x || !q || !s || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null argument");
   if (M <= 0 || N <= 0 || K <= 0 || N > INT32_MAX || K > INT32_MAX || M > 65535 * 16)
     return fail(QWIX_ERR_INVALID_ARGUMENT, "bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
-  if (b_qtype != QWIX_INT4 && b_qtype != QWIX_INT8)
-    return fail(QWIX_ERR_UNSUPPORTED, "weight-only kernel takes int4 or int8 weights (got qtype %d)", b_qtype);
+  if (b_qtype != QWIX_INT4 && b_qtype != QWIX_INT8 && b_qtype != QWIX_E4M3)
+    return fail(QWIX_ERR_UNSUPPORTED, "weight-only kernel takes int4, int8 or e4m3 weights (got qtype %d)", b_qtype);
+  if (b_qtype == QWIX_E4M3 && zp) return fail(QWIX_ERR_INVALID_ARGUMENT, "float weights have no zero point");
   if (K % 128 || group <= 0 || group % 128 || K % group)
     return fail(QWIX_ERR_UNSUPPORTED, "K=%lld and group=%lld must be multiples of 128 with group | K", (long long)K,
                 (long long)group);
@@ -435,6 +448,10 @@ static int gemv_wq_impl(const void* x, int64_t ldx, const void* q, int64_t ldb_b
       QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT4, NW, NTT, true, RTT, ZPP>), NW, NTT, RTT);                \
     else if (b_qtype == QWIX_INT4)                                                                         \
       QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT4, NW, NTT, false, RTT, ZPP>), NW, NTT, RTT);               \
+    else if (b_qtype == QWIX_E4M3 && s_dtype == QWIX_BF16)                                                 \
+      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_E4M3, NW, NTT, true, RTT, false>), NW, NTT, RTT);              \
+    else if (b_qtype == QWIX_E4M3)                                                                         \
+      QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_E4M3, NW, NTT, false, RTT, false>), NW, NTT, RTT);             \
     else if (s_dtype == QWIX_BF16)                                                                         \
       QWIX_GEMV_KERNEL((gemv_wq_kernel<QWIX_INT8, NW, NTT, true, RTT, ZPP>), NW, NTT, RTT);                \
     else                                                                                                   \

@@ -129,11 +129,12 @@ def test_per_channel_int4_weight_and_tile_mismatch_error():
     dg._fast_dot_general(xq2, wq2, DN)
 
 
-@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('wq_type', ['int4', 'int8', 'float8_e4m3fn'])
 @pytest.mark.parametrize('M', [1, 8, 16, 24, 40, 100])
 @pytest.mark.parametrize('K,N,group,sdt', [(512, 256, 128, torch.float32), (4096, 1024, 128, torch.float32), (1024, 200, 1024, torch.bfloat16)])
 def test_weight_only_gemv(M, K, N, group, sdt, wq_type):
-  """The weight-only int4 benchmark configuration at reduced N: bf16 activations x int4 g128 weight, f32 scales, bf16 out."""
+  """The weight-only int4 benchmark configuration at reduced N: bf16 activations x int4 g128 weight, f32 scales, bf16 out;
+  the same with int8 and e4m3 weights.  The decode kernel is the one that runs: the operator's fit accepts the pair."""
   from qwix_amd.core import dot_general as dg
   from qwix_amd.core import qarray
   print('case gemv', M, K, N, group, wq_type, flush=True)
@@ -143,6 +144,7 @@ def test_weight_only_gemv(M, K, N, group, sdt, wq_type):
   wq = qarray.quantize_api(w_t, wq_type, channelwise_axes=[1], tiled_axes=tiled, scale_dtype=sdt)
   owq = O.quantize_api(O.FArr(w_np, O.BF16), wq_type, channelwise_axes=[1], tiled_axes=tiled, scale_dtype=util.ORACLE_DT[sdt])
   util.assert_qarray_equal(wq, owq, 'weight')
+  assert dg._weight_only_fit(x_t, wq, DN) is not None
   out = dg.dot_general(x_t, wq, DN, preferred_element_type=torch.bfloat16)
   torch.cuda.synchronize()
   want = O.dot_general(O.FArr(x_np, O.BF16), owq, DN, O.BF16)
@@ -187,7 +189,7 @@ def test_weight_only_gemv_asymmetric_weights(M, K, N, group, sdt, wq_type):
   assert torch.allclose(out, two, rtol=1e-2, atol=1e-2 * float(two.abs().mean()))
 
 
-@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('wq_type', ['int4', 'int8', 'float8_e4m3fn'])
 @pytest.mark.parametrize('M', [1, 20, 40])
 @pytest.mark.parametrize('K,N,group', [(384, 72, 128), (4224, 136, 128), (16384, 264, 256), (8192, 2048, 128), (128, 48, 128)])
 def test_weight_only_gemv_k_splits(M, K, N, group, wq_type):
@@ -210,7 +212,7 @@ def test_weight_only_gemv_k_splits(M, K, N, group, wq_type):
   assert np.allclose(got, want.v, rtol=1e-3, atol=1e-3 * np.abs(want.v).mean()), np.abs(got - want.v).max()
 
 
-@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('wq_type', ['int4', 'int8', 'float8_e4m3fn'])
 @pytest.mark.parametrize('M,K,N', [(30, 1024, 520), (50, 4096, 14336), (130, 512, 6400)])
 def test_weight_only_rows_do_not_depend_on_the_batch(M, K, N, wq_type, monkeypatch):
   """More than 16 rows share a pass over the weights (2 tiles of 16 rows per workgroup, fewer wavefronts
@@ -500,18 +502,16 @@ def test_weight_only_prefill_on_hip_kernels(M, K, N, case):
   wq = qarray.quantize_api(w_t, wq_type, **kw)
   owq = O.quantize_api(O.FArr(w_np, O.BF16), wq_type, **okw)
   util.assert_qarray_equal(wq, owq, 'weight')
-  # the decode kernel is bypassed by its own row limit (M > 256) or by the operand kind (e4m3)
-  fit = dg._weight_only_fit(x_t, wq, DN)
-  assert (fit is None) == (wq_type == 'float8_e4m3fn')
+  # every one of these pairs is of the decode kernel's kind; it is bypassed by the row count
+  assert dg._weight_only_fit(x_t, wq, DN) is not None
   out = dg._dequantize_then_bf16_gemm(x_t, wq, DN, torch.bfloat16)
   assert out is not None and out.dtype == torch.bfloat16
   torch.cuda.synchronize()
   want = O.dot_general(O.FArr(x_np, O.BF16), owq, DN, O.BF16)
   got = util.f32np(out)
   assert np.allclose(got, want.v, rtol=1e-2, atol=1e-2 * np.abs(want.v).mean()), np.abs(got - want.v).max()
-  # the operator takes this path beyond the decode kernel's rows, for the operand kinds that kernel does not take, and
-  # for symmetric int4 from the row count on at which the dequantizing tile GEMM wins
-  if M > dg.WEIGHT_ONLY_MAX_ROWS or fit is None or (wq_type in ('int4', 'int8') and M > dg.fused_wq_min_rows(N, wq_type == 'int4')):
+  # the operator takes this path from the row count on at which the dequantizing tile GEMM beats the decode kernel
+  if M > dg.fused_wq_min_rows(N, wq_type == 'int4'):
     assert torch.equal(dg.dot_general(x_t, wq, DN, preferred_element_type=torch.bfloat16), out)
   # the dequantized operand itself, against the oracle's dequantize
   c = dg._Canon(x_t, wq, DN)
