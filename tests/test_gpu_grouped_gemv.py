@@ -479,6 +479,32 @@ def test_dequantizing_gemm_argument_checks():
   torch.cuda.synchronize()
 
 
+def test_decode_kernel_argument_checks():
+  """qwix_hip_gemv_wq / qwix_hip_gemv_wq_zp refuse other weight types, zero points for float weights, K or groups that
+  are not whole 128-wide blocks and unaligned rows, with an error code and a message instead of launching."""
+  from qwix_amd import _lib
+  L = _lib.load()
+  M, N, K = 8, 64, 512
+  x = torch.zeros(M, K, dtype=torch.bfloat16, device=util.DEV)
+  q = torch.zeros(N, K, dtype=torch.int8, device=util.DEV)
+  s = torch.ones(K // 128, N, dtype=torch.bfloat16, device=util.DEV)
+  z = torch.zeros(K // 128, N, dtype=torch.int8, device=util.DEV)
+  out = torch.empty(M, N, dtype=torch.bfloat16, device=util.DEV)
+  def call(qt=_lib.INT8, k=K, group=128, ldb=K, zp=False):
+    if zp:
+      return L.qwix_hip_gemv_wq_zp(x.data_ptr(), K, q.data_ptr(), ldb, qt, M, N, k, group, s.data_ptr(), _lib.BF16,
+                                   z.data_ptr(), out.data_ptr(), _lib.BF16, N, None)
+    return L.qwix_hip_gemv_wq(x.data_ptr(), K, q.data_ptr(), ldb, qt, M, N, k, group, s.data_ptr(), _lib.BF16,
+                              out.data_ptr(), _lib.BF16, N, None)
+  assert call() == 0 and call(qt=_lib.E4M3) == 0 and call(qt=_lib.INT4, ldb=K // 2) == 0 and call(zp=True) == 0
+  assert call(qt=7) != 0 and b'int4, int8 or e4m3' in L.qwix_hip_last_error()
+  assert call(qt=_lib.E4M3, zp=True) != 0 and b'no zero point' in L.qwix_hip_last_error()
+  assert call(k=448) != 0 and b'multiples of 128' in L.qwix_hip_last_error()
+  assert call(group=192) != 0
+  assert call(ldb=K - 16) != 0 and b'aligned' in L.qwix_hip_last_error()
+  torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize('case', [('int4', 128, False, torch.float32), ('int8', 128, False, torch.bfloat16),
                                   ('int4', 256, True, torch.bfloat16), ('int8', None, True, torch.float32),
                                   ('float8_e4m3fn', None, False, torch.bfloat16)])
