@@ -432,10 +432,11 @@ static int gemv_wq_impl(const void* x, int64_t ldx, const void* q, int64_t ldb_b
   p.zp = zp;
   p.out = out; p.out_dtype = out_dtype; p.ldo = ldo;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  // Byte weights of 32 MB and more stream faster through the smaller workgroups of the two-row-tile configuration
-  // (8 wavefronts, two workgroups per CU) even when the second row tile is empty: K 4096, N 14336, 1 / 16 rows,
-  // int8 25.5 / 26.9 -> 16.5 / 18.2 us, e4m3 21.9 / 23.8 -> 15.5 / 17.8; K = N = 8192: 20.0 / 24.4 -> 17.9 / 22.0;
-  // at 16 MB (K = N = 4096) 9.3 against 10.2 us the other way round, and int4 gains nothing at any size.
+  // Byte weights of 32 MB and more stream faster through the smallest workgroups (4 wavefronts, two row tiles, several
+  // workgroups per CU) whatever the rows, even when the second row tile is empty: K 4096, N 14336, int8, 1 / 16 / 32
+  // rows 25.5 / 26.9 / 21.9 -> 16.2 / 17.5 / 21.0 us (8 wavefronts: 16.5 / 18.2), e4m3 21.9 / 23.8 -> 15.5 / 17.8;
+  // K = N = 8192: 20.0 / 24.4 / 29.4 -> 17.8 / 20.0 / 26.9; at 16 MB (K = N = 4096) 9.3 against 10.2 us the other way
+  // round, and int4 gains nothing at any size.
   const bool small_groups = b_qtype != QWIX_INT4 && N * K >= (int64_t{32} << 20);
 #define QWIX_GEMV_KERNEL(KERN, NW, NTT, RTT)                                                                \
   do {                                                                                                     \
@@ -468,8 +469,8 @@ static int gemv_wq_impl(const void* x, int64_t ldx, const void* q, int64_t ldb_b
   } while (0)
 #define QWIX_GEMV_LAUNCH(NW, NTT)                                                                          \
   do {                                                                                                     \
-    if (M <= 16 && !small_groups) QWIX_GEMV_LAUNCH_RT(NW, NTT, 1);        \
-    else if (M <= 32) QWIX_GEMV_LAUNCH_RT(8, NTT, 2);                                                      \
+    if (M <= 16 && !small_groups) QWIX_GEMV_LAUNCH_RT(NW, NTT, 1);                                         \
+    else if (M <= 32 && !small_groups) QWIX_GEMV_LAUNCH_RT(8, NTT, 2);                                     \
     else QWIX_GEMV_LAUNCH_RT(4, NTT, 2); /* several passes side by side: smaller workgroups, two per CU */  \
   } while (0)
   // Wider column tiles reuse each activation fragment more often; narrower ones keep every CU busy
