@@ -306,12 +306,13 @@ class PlainCopy(Workload):
 class GemvW4(Workload):
   bound = 'hbm'
 
-  def __init__(self, name, M, K, N, group):
-    self.name, self.M, self.K, self.N, self.group = name, M, K, N, group
-    self.dtype = 'bf16 x int4'
-    self.metric = 'weight-only int4 g128 GEMV GB/s'
+  def __init__(self, name, M, K, N, group, qtype='int4'):
+    self.name, self.M, self.K, self.N, self.group, self.qtype = name, M, K, N, group, qtype
+    self.dtype = 'bf16 x ' + qtype
+    self.metric = f'weight-only {qtype} g128 GEMV GB/s'
     self.unit = 'GB/s'
     self.kernel_name = 'gemv_wq_kernel'
+    self.wbytes = 0.5 if qtype == 'int4' else 1.0
 
   def setup(self, dev):
     import torch
@@ -320,8 +321,9 @@ class GemvW4(Workload):
     g = torch.Generator(device='cpu').manual_seed(2000)
     self.x = torch.randn(self.M, self.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
     w = (torch.randn(self.K, self.N, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(dev)
-    wq = qarray.quantize_api(w, 'int4', channelwise_axes=[1], tiled_axes={0: self.group}, scale_dtype=torch.float32)
-    b = wq.qvalue.permute(1, 0).data
+    wq = qarray.quantize_api(w, self.qtype, channelwise_axes=[1], tiled_axes={0: self.group}, scale_dtype=torch.float32)
+    b = wq.qvalue.permute(1, 0)
+    b = b.data if self.qtype == 'int4' else b.contiguous()
     assert b.is_contiguous()
     s = wq.scale.contiguous()
     # A decoder walks through a different weight matrix per layer: rotate over enough copies that a
@@ -336,13 +338,14 @@ class GemvW4(Workload):
   def step(self, i=0):
     L = self.L
     c = i % self.copies
-    L.call('qwix_hip_gemv_wq', self.x.data_ptr(), self.K, self.b[c].data_ptr(), self.K // 2, L.INT4, self.M, self.N,
+    L.call('qwix_hip_gemv_wq', self.x.data_ptr(), self.K, self.b[c].data_ptr(), int(self.K * self.wbytes),
+           L.INT4 if self.qtype == 'int4' else L.INT8, self.M, self.N,
            self.K, self.group, self.s[c].data_ptr(), L.F32, self.out.data_ptr(), L.BF16, self.N, self.stream)
 
   kernel = step
 
   def work_per_step(self):
-    return self.K * self.N / 2.0 + (self.K // self.group) * self.N * 4.0 + self.M * self.K * 2.0 + self.M * self.N * 2.0
+    return self.K * self.N * self.wbytes + (self.K // self.group) * self.N * 4.0 + self.M * self.K * 2.0 + self.M * self.N * 2.0
 
   kernel_work = work_per_step
 
@@ -875,6 +878,8 @@ WORKLOADS = {
     'c2_gemv_w4_m1': lambda: GemvW4('c2_gemv_w4_m1', 1, 4096, 14336, 128),
     'c2_gemv_w4_m16': lambda: GemvW4('c2_gemv_w4_m16', 16, 4096, 14336, 128),
     'c2_gemv_w4_m32': lambda: GemvW4('c2_gemv_w4_m32', 32, 4096, 14336, 128),
+    'w8a16_gemv_m1': lambda: GemvW4('w8a16_gemv_m1', 1, 4096, 14336, 128, 'int8'),
+    'w8a16_gemv_m16': lambda: GemvW4('w8a16_gemv_m16', 16, 4096, 14336, 128, 'int8'),
     'c2_w4a16_prefill_m2048': lambda: WeightOnlyPrefill('c2_w4a16_prefill_m2048', 2048, 4096, 14336, 128),
     'c2_w4a16_prefill_m512': lambda: WeightOnlyPrefill('c2_w4a16_prefill_m512', 512, 4096, 14336, 128),
     'c2_w4a16_prefill_m128': lambda: WeightOnlyPrefill('c2_w4a16_prefill_m128', 128, 4096, 14336, 128),
@@ -896,7 +901,7 @@ WORKLOADS = {
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
 }
 DEFAULT = 'c3_int8_w8a8_4096'
-EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'c2_w4a16_prefill_m2048', 'c2_w4a16_prefill_m512', 'c2_w4a16_prefill_m128', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
+EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a16_gemv_m1', 'w8a16_gemv_m16', 'c2_w4a16_prefill_m2048', 'c2_w4a16_prefill_m512', 'c2_w4a16_prefill_m128', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
          'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'moe_ragged_int8_8x1024',
          'moe_ragged_int8_64x128', 'moe_decode_int8_64x4', 'quantize_weight_fp8_block128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 
