@@ -862,12 +862,68 @@ class PtqMlpGraph(Workload):
             'activations': 'int8 per token, quantized on the fly', 'eager_us_per_forward': round(self.eager_us, 1)}
 
 
+class MfmaCeiling(Workload):
+  """What the matrix cores sustain with given operand bytes and no memory traffic: MFMAs back to back on register
+  operands (`qwix_hip_mfma_ceiling`), every launch about 10 ms.  `data`: 'zeros'; 'gauss30' (int8 N(0, 30^2) bytes, the
+  same bytes read as e4m3 for fp8); 'operands' (the quantized activations and weights of the 4096^2 w8a8 workload of
+  that type: per-token / per-channel absmax of bf16 N(0,1) and N(0,0.02))."""
+
+  bound = 'mfma'
+  ITERS = 10000
+
+  def __init__(self, name, qtype, data):
+    self.name, self.qtype, self.data = name, qtype, data
+    self.dtype = 'int8' if qtype == 'int8' else 'f8e4m3'
+    self.metric = ('int8' if qtype == 'int8' else 'fp8') + ' MFMA rate on register operands (no memory traffic): ' + data
+    self.unit = 'TOPS'
+    self.kernel_name = 'mfma_ceiling_kernel'
+
+  def setup(self, dev):
+    import torch
+    from qwix_amd.core import qarray
+    L = _lib()
+    n = 1 << 24
+    g = torch.Generator(device='cpu').manual_seed(77)
+    if self.data == 'zeros':
+      self.a = torch.zeros(n, dtype=torch.uint8, device=dev)
+      self.b = torch.zeros(n, dtype=torch.uint8, device=dev)
+    elif self.data == 'gauss30':
+      mk = lambda: torch.randn(n, generator=g).mul_(30.0).round_().clamp_(-126, 126).to(torch.int8).view(torch.uint8).to(dev)
+      self.a, self.b = mk(), mk()
+    else:
+      x = torch.randn(4096, 4096, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+      w = (torch.randn(4096, 4096, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(dev)
+      xq = qarray.quantize(x, qarray.HowToQuantize(qtype=self.qtype, channelwise_axes=[0]))
+      wq = qarray.quantize(w, qarray.HowToQuantize(qtype=self.qtype, channelwise_axes=[1]))
+      self.a = xq.qvalue.contiguous().view(torch.uint8).reshape(-1)
+      self.b = wq.qvalue.permute(1, 0).contiguous().view(torch.uint8).reshape(-1)
+    self.sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    self.qt = L.INT8 if self.qtype == 'int8' else L.E4M3
+    self.ops = float(L.load().qwix_hip_mfma_ceiling_ops(self.ITERS))
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, i=0):
+    self.L.call('qwix_hip_mfma_ceiling', self.a.data_ptr(), self.a.numel(), self.b.data_ptr(), self.b.numel(), self.qt,
+                self.ITERS, self.sink.data_ptr(), self.stream)
+
+  kernel = step
+
+  def work_per_step(self):
+    return self.ops
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'operand_bytes': self.data, 'iterations': self.ITERS, 'workgroups': 256, 'wavefronts_per_workgroup': 8}
+
+
 WORKLOADS = {
     'quantize_act_8192': lambda: QuantizeRows('quantize_act_8192', 8192, 8192, 'int8'),
     'c3_int8_w8a8_4096': lambda: QdotW8A8('c3_int8_w8a8_4096', 4096, 4096, 4096, 'int8'),
     'c4_fp8_w8a8_ffn': lambda: QdotW8A8('c4_fp8_w8a8_ffn', 8192, 8192, 28672, 'float8_e4m3fn'),
     'c3_fp8_w8a8_4096': lambda: QdotW8A8('c3_fp8_w8a8_4096', 4096, 4096, 4096, 'float8_e4m3fn'),
-    'int8_w8a8_8192': lambda: QdotW8A8('int8_w8a8_8192', 8192, 8192, 8192, 'int8'),
+    'c3_int8_w8a8_8192': lambda: QdotW8A8('c3_int8_w8a8_8192', 8192, 8192, 8192, 'int8'),
     'quantize_act_4096': lambda: QuantizeRows('quantize_act_4096', 4096, 4096, 'int8'),
     'quantize_act_8192_fp8': lambda: QuantizeRows('quantize_act_8192_fp8', 8192, 8192, 'float8_e4m3fn'),
     'w8a8_decode_m16': lambda: QdotDecode('w8a8_decode_m16', 16, 4096, 14336),
@@ -899,9 +955,19 @@ WORKLOADS = {
     'batched_qk_int8_32x2048': lambda: QdotBatched('batched_qk_int8_32x2048', 32, 2048, 2048, 128),
     'c1_ptq_mlp_graph': lambda: PtqMlpGraph('c1_ptq_mlp_graph'),
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
+    'mfma_ceiling_int8_zeros': lambda: MfmaCeiling('mfma_ceiling_int8_zeros', 'int8', 'zeros'),
+    'mfma_ceiling_int8_gauss30': lambda: MfmaCeiling('mfma_ceiling_int8_gauss30', 'int8', 'gauss30'),
+    'mfma_ceiling_int8_operands': lambda: MfmaCeiling('mfma_ceiling_int8_operands', 'int8', 'operands'),
+    'mfma_ceiling_fp8_zeros': lambda: MfmaCeiling('mfma_ceiling_fp8_zeros', 'float8_e4m3fn', 'zeros'),
+    'mfma_ceiling_fp8_gauss30': lambda: MfmaCeiling('mfma_ceiling_fp8_gauss30', 'float8_e4m3fn', 'gauss30'),
+    'mfma_ceiling_fp8_operands': lambda: MfmaCeiling('mfma_ceiling_fp8_operands', 'float8_e4m3fn', 'operands'),
 }
+# The measured matrix-core ceilings: run first, so that every MFMA-bound line can carry `frac_of_ceiling`.
+CEILINGS = {'int8': 'mfma_ceiling_int8_operands', 'f8e4m3': 'mfma_ceiling_fp8_operands'}
+CEILING_EXTRA = ['mfma_ceiling_int8_zeros', 'mfma_ceiling_int8_gauss30', 'mfma_ceiling_int8_operands',
+                 'mfma_ceiling_fp8_zeros', 'mfma_ceiling_fp8_gauss30', 'mfma_ceiling_fp8_operands']
 DEFAULT = 'c3_int8_w8a8_4096'
-EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a16_gemv_m1', 'w8a16_gemv_m16', 'c2_w4a16_prefill_m2048', 'c2_w4a16_prefill_m512', 'c2_w4a16_prefill_m128', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
+EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c3_int8_w8a8_8192', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'w8a16_gemv_m1', 'w8a16_gemv_m16', 'c2_w4a16_prefill_m2048', 'c2_w4a16_prefill_m512', 'c2_w4a16_prefill_m128', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
          'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'moe_ragged_int8_8x1024',
          'moe_ragged_int8_64x128', 'moe_decode_int8_64x4', 'quantize_weight_fp8_block128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 
@@ -968,7 +1034,7 @@ def run(wl: Workload, steps: int, warmup: int, spin_up: float = None, repeats: i
   return med(step_t), med(kern_t), timing
 
 
-def summarize(wl: Workload, step_s: float, kern_s: float) -> dict:
+def summarize(wl: Workload, step_s: float, kern_s: float, ceilings: dict = None) -> dict:
   scale = 1e12 if wl.bound == 'mfma' else 1e9
   value = wl.work_per_step() / step_s / scale
   # the roofline that bounds the dominant kernel need not be the one the metric's unit suggests
@@ -976,12 +1042,36 @@ def summarize(wl: Workload, step_s: float, kern_s: float) -> dict:
   peak = getattr(wl, 'peak_tops', PEAK_MFMA_TOPS) if rb == 'mfma' else PEAK_HBM_GBS
   work = wl.roofline_work() if hasattr(wl, 'roofline_work') else wl.kernel_work()
   achieved = work / kern_s / (1e12 if rb == 'mfma' else 1e9)
-  return {
-      'value': round(value, 2), 'unit': wl.unit, 'ms_per_step': round(step_s * 1e3, 5),
-      'roofline': {'bound': rb, 'kernel': wl.kernel_name, 'achieved': round(achieved, 2), 'peak': peak,
-                   'unit': 'TFLOP/s' if rb == 'mfma' else 'GB/s', 'frac': round(achieved / peak, 4),
-                   'traffic': _traffic(wl.name), **_mfma_util(wl.name)},
-  }
+  roof = {'bound': rb, 'kernel': wl.kernel_name, 'achieved': round(achieved, 2), 'peak': peak,
+          'unit': 'TFLOP/s' if rb == 'mfma' else 'GB/s', 'frac': round(achieved / peak, 4),
+          'traffic': _traffic(wl.name), **_mfma_util(wl.name)}
+  # `frac` stays priced against the nominal peak; `frac_of_ceiling` is the same rate against what the matrix cores
+  # sustained in this very run on register operands of this workload's kind (see MfmaCeiling), no memory traffic.
+  if rb == 'mfma' and peak == PEAK_MFMA_TOPS and not isinstance(wl, MfmaCeiling):
+    c = (ceilings or {}).get(wl.dtype)
+    roof['ceiling'] = c
+    roof['frac_of_ceiling'] = round(achieved / c, 4) if c else None
+  return {'value': round(value, 2), 'unit': wl.unit, 'ms_per_step': round(step_s * 1e3, 5), 'roofline': roof}
+
+
+def measure_ceilings(dtypes, spin_up) -> tuple:
+  """Runs the matrix-core ceiling workloads; returns ({dtype: TOPS on the benchmark's operand bytes}, {name: line})."""
+  import torch
+  ceilings, lines = {}, {}
+  prefixes = tuple(CEILINGS[d].rsplit('_', 1)[0] + '_' for d in dtypes)   # all operand kinds of the wanted types
+  names = [n for n in CEILING_EXTRA if n.startswith(prefixes)]
+  for name in names:
+    w = WORKLOADS[name]()
+    s, km, _ = run(w, 3, 1, min(spin_up, 0.2), 3)
+    r = summarize(w, s, km)
+    lines[name] = {'metric': w.metric, 'value': r['value'], 'unit': r['unit'], 'ms_per_step': r['ms_per_step'],
+                   'roofline': r['roofline']}
+    for d, n in CEILINGS.items():
+      if n == name:
+        ceilings[d] = r['roofline']['achieved']
+    del w
+    torch.cuda.empty_cache()
+  return ceilings, lines
 
 
 def _traffic(name: str):
@@ -1018,6 +1108,8 @@ def main():
                   help='repetitions of the timed region of --steps steps; the median is reported')
   ap.add_argument('--no-extra', action='store_true', help='skip the other workloads of the metric')
   ap.add_argument('--no-cpu-baseline', action='store_true')
+  ap.add_argument('--no-ceiling', action='store_true',
+                  help='skip the matrix-core ceiling measurement that roofline.frac_of_ceiling is priced against')
   ap.add_argument('--spin-up', type=float, default=SPIN_UP_S,
                   help='minimum seconds of untimed warm-up (profiling runs shorten it to keep traces small)')
   args = ap.parse_args()
@@ -1031,8 +1123,14 @@ def main():
     sys.exit(2)
 
   wl = WORKLOADS[args.workload]()
+  extra_on = not args.no_extra and args.workload == DEFAULT
+  ceilings, ceiling_lines = {}, {}
+  if not args.no_ceiling and not isinstance(wl, MfmaCeiling):
+    want = sorted(CEILINGS) if extra_on else [d for d in CEILINGS if d == wl.dtype and getattr(wl, 'roofline_bound', wl.bound) == 'mfma']
+    if want:
+      ceilings, ceiling_lines = measure_ceilings(want, args.spin_up)
   step_s, kmean, timing = run(wl, args.steps, args.warmup, args.spin_up, args.repeats)
-  res = summarize(wl, step_s, kmean)
+  res = summarize(wl, step_s, kmean, ceilings)
   line = {
       'metric': wl.metric, 'value': res['value'], 'unit': res['unit'], 'n_gpus': 1, 'steps': args.steps,
       'warmup': args.warmup, 'ms_per_step': res['ms_per_step'], 'higher_is_better': True, 'scaling': 'weak',
@@ -1043,13 +1141,13 @@ def main():
     line['cpu_baseline'] = wl.cpu_baseline()
   else:
     line['cpu_baseline'] = None
-  if not args.no_extra and args.workload == DEFAULT:
-    extra = {}
+  if extra_on:
+    extra = dict(ceiling_lines)
     for name in EXTRA:
       w = WORKLOADS[name]()
       n = max(5, min(args.steps, 20))
       s, km, _ = run(w, n, 3, args.spin_up, min(args.repeats, 5))
-      r = summarize(w, s, km)
+      r = summarize(w, s, km, ceilings)
       extra[name] = {'metric': w.metric, 'value': r['value'], 'unit': r['unit'], 'ms_per_step': r['ms_per_step'],
                      'roofline': r['roofline']}
       del w

@@ -81,7 +81,9 @@ QWIX_API int qwix_hip_quantize(const void* x, int dtype, int64_t outer, int64_t 
  * runs on holds until the process ends.  Shapes whose qwix_hip_quantize_workspace_bytes(...) exceeds
  * that are refused with QWIX_ERR_UNSUPPORTED.  The call allocates nothing and frees nothing.  All calls
  * on one GPU share that GPU's array: calls that overlap on one GPU (different streams, or threads)
- * race; calls ordered on one stream do not (every call clears what it accumulates into). */
+ * race; calls ordered on one stream do not (every call clears what it accumulates into).  The array used
+ * is the one of the CURRENT device of the calling thread: the caller must have made the stream's device
+ * current (hipSetDevice) before the call, as for any launch on that stream. */
 QWIX_API size_t qwix_hip_quantize_static_max_bytes(void);
 QWIX_API int qwix_hip_quantize_static(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner,
                              int64_t tile, int qtype, int calibration, float calib_factor,
@@ -368,6 +370,17 @@ QWIX_API int qwix_hip_fwht(const void* x, int dtype, int64_t rows, int64_t n, co
 QWIX_API int qwix_hip_fwht_quantize(const void* x, int dtype, int64_t rows, int64_t n,
                            const void* pre_sign, const void* post_sign, float out_scale,
                            int64_t tile, int qtype, void* qvalue, void* scale, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Measurement aid; no counterpart in the reference.  Runs int8 (QWIX_INT8) or OCP e4m3 (QWIX_E4M3) MFMAs back to
+ * back on operands held in registers (no LDS, no memory traffic after the first loads): 256 workgroups of 8
+ * wavefronts, every lane's A / B fragments taken from the caller's arrays `a` / `b` (any bytes; 16-byte aligned),
+ * `iters` rounds of 32 int8 or 16 fp8 MFMAs per wavefront.  The rate it reaches is what the matrix cores of the
+ * board sustain with THOSE operand bytes under its power limit: the ceiling beside the nominal peak for the
+ * quantized GEMMs.  qwix_hip_mfma_ceiling_ops(iters) = operations of one launch.  `sink`: 4 writable bytes. */
+QWIX_API double qwix_hip_mfma_ceiling_ops(int64_t iters);
+QWIX_API int qwix_hip_mfma_ceiling(const void* a, size_t a_bytes, const void* b, size_t b_bytes, int qtype,
+                          int64_t iters, int32_t* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -59,6 +59,8 @@ SIGNATURES = {
     'qwix_hip_gemv_wq_zp': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _int, _i64, _vp]),
     'qwix_hip_fwht': (_int, [_vp, _int, _i64, _i64, _vp, _vp, _f32, _vp, _vp]),
     'qwix_hip_fwht_quantize': (_int, [_vp, _int, _i64, _i64, _vp, _vp, _f32, _i64, _int, _vp, _vp, _vp]),
+    'qwix_hip_mfma_ceiling_ops': (_c.c_double, [_i64]),
+    'qwix_hip_mfma_ceiling': (_int, [_vp, _sz, _vp, _sz, _int, _i64, _vp, _vp]),
 }
 
 _lib = None

@@ -118,6 +118,8 @@ class _Canon:
       v = v.unpack()  # int4 activations are widened to int8 (exact); the MFMA kernels take int8 rows
     v = v.permute(*(self.lfree + self.lca))  # contracting axes last (a no-op view in the usual layout)
     v = v if v.is_contiguous() else v.contiguous()
+    if v.data_ptr() % 16:  # a contiguous view that starts inside a 16-byte unit: the kernels load 16 bytes per lane
+      v = v.clone()
     return v.reshape(self.M, self.K)
 
   def rhs_values(self, rhs) -> tuple[torch.Tensor, bool]:
@@ -341,12 +343,12 @@ def fused_act_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=No
   return out.reshape(c.out_shape)
 
 
-@functools.lru_cache(maxsize=None)
+@functools.lru_cache(maxsize=4096)
 def _dynamic_act_bytes(M: int, N: int, K: int, x_tag: int) -> int:
   return int(_lib.load().qwix_hip_qgemm_dynamic_act_workspace_bytes(M, N, K, x_tag))
 
 
-@functools.lru_cache(maxsize=None)
+@functools.lru_cache(maxsize=4096)
 def _splitk_bytes(M: int, N: int, K: int) -> int:
   """Scratch bytes with which the GEMM may split K for this shape (0: it would not)."""
   return int(_lib.load().qwix_hip_qgemm_workspace_bytes(M, N, K))
@@ -540,6 +542,29 @@ def _weight_only_fit(lhs, rhs, dimension_numbers):
   return c
 
 
+_I31 = (1 << 31) - 1
+
+
+def _decode_kernel_limits_ok(ldx: int, ldb_bytes: int, n: int, k: int, group: int, int4: bool, scale_bytes: int) -> bool:
+  """The address arithmetic of `qwix_hip_gemv_wq`: 31-bit lane offsets over 32 activation rows, 64 weight rows and the
+  whole scale array.  Calls beyond it take the dequantize-first route."""
+  brow = k // 2 if int4 else k
+  return 32 * ldx * 2 + 2 * k <= _I31 and 64 * ldb_bytes + brow <= _I31 and (k // group) * n * scale_bytes <= _I31
+
+
+def _bf16_gemm_limits_ok(m: int, lda: int, n: int, ldb_bytes: int) -> bool:
+  """`qwix_hip_gemm_bf16` / `qwix_hip_gemm_bf16_wq` address each operand with 31-bit byte offsets."""
+  return m * lda * 2 <= _I31 and n * ldb_bytes <= _I31
+
+
+def _aligned_rows(x: torch.Tensor) -> torch.Tensor:
+  """The activation as the kernels want it: unit stride along K, row pitch a multiple of 8 elements, 16-byte aligned
+  base.  A view that is not (a slice that starts inside a row) is copied."""
+  if x.stride(-1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0:
+    return x
+  return x.contiguous()
+
+
 # Rows up to which the fused weight-only kernel (one pass over the weight per 16 or 32 rows) is used; above
 # it the weight is dequantized once (HIP kernel) and contracted by the float GEMM.
 WEIGHT_ONLY_MAX_ROWS = 256
@@ -552,8 +577,14 @@ _DECODE_PLANS: dict = {}
 
 
 def _weight_signature(rhs: QArray) -> tuple:
-  z = rhs.zero_point
-  return (id(rhs.qvalue), id(rhs.scale), id(z), None if z is None else z._version)
+  """Identity and torch version counter of every tensor a kept plan may hold a re-laid-out COPY of: an in-place update
+  (`copy_`, a state reload into existing tensors) keeps the object and bumps the counter."""
+  def sig(t):
+    if t is None:
+      return None
+    store = t.data if isinstance(t, Int4Tensor) else t
+    return (id(t), id(store), store._version)
+  return (sig(rhs.qvalue), sig(rhs.scale), sig(rhs.zero_point))
 
 
 def _decode_plan(lhs, rhs, dimension_numbers):
@@ -579,8 +610,7 @@ def _decode_dot(lhs, rhs, dimension_numbers, preferred_element_type):
   kind (the general code below then decides)."""
   (lca, rca), _ = dimension_numbers
   if not (type(lhs) is torch.Tensor and lhs.ndim == 2 and lhs.dtype == torch.bfloat16 and isinstance(rhs, QArray)
-          and len(lca) == 1 and lca[0] == 1 and rca[0] == 0 and lhs.shape[0] <= WEIGHT_ONLY_MAX_ROWS
-          and lhs.stride(1) == 1 and lhs.stride(0) % 8 == 0):
+          and len(lca) == 1 and lca[0] == 1 and rca[0] == 0 and lhs.shape[0] <= WEIGHT_ONLY_MAX_ROWS):
     return None
   plan = _decode_plan(lhs, rhs, dimension_numbers)
   if plan is None:
@@ -588,6 +618,9 @@ def _decode_dot(lhs, rhs, dimension_numbers, preferred_element_type):
   b, b_tag, sb, sb_tag, zp, n, k, group, fused_min = plan
   m = lhs.shape[0]
   if lhs.shape[1] != k or len(rhs.shape) != 2 or m > fused_min:
+    return None
+  lhs = _aligned_rows(lhs)
+  if not _decode_kernel_limits_ok(lhs.stride(0), b.stride(0), n, k, group, b_tag == _lib.INT4, sb.element_size()):
     return None
   res_t = preferred_element_type or torch.promote_types(lhs.dtype, sb.dtype)
   out = torch.empty(m, n, dtype=res_t, device=lhs.device)
@@ -617,7 +650,7 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
     out = _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type, fused_only=True)
     if out is not None:
       return out
-  if c is not None and c.M <= WEIGHT_ONLY_MAX_ROWS:
+  if c is not None and c.M <= WEIGHT_ONLY_MAX_ROWS and _decode_fits_limits(c, rhs):
     sb, gb = c.rhs_scale(rhs)
     x = c.lhs_values(lhs)
     b, b_is4 = c.rhs_values(rhs)
@@ -642,6 +675,13 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
     rhs = qarray.dequantize(rhs)
   res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs.dtype)
   return float_dot_general(lhs, rhs, dimension_numbers, res_t)
+
+
+def _decode_fits_limits(c, rhs: QArray) -> bool:
+  """`_decode_kernel_limits_ok` from the shapes alone (K-contiguous weight rows, contiguous activation rows)."""
+  int4 = isinstance(rhs.qvalue, Int4Tensor)
+  gb = rhs.scale.shape[c.rca[-1]]
+  return _decode_kernel_limits_ok(c.K, c.K // 2 if int4 else c.K, c.N, c.K, c.K // gb, int4, rhs.scale.element_size())
 
 
 # The tile GEMM that dequantizes the weight inside its workgroups converts it once per row tile of 256; above these
@@ -694,6 +734,8 @@ def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_ty
     packed = (rhs.qvalue.permute(*order).packed_axis, rhs.qvalue.permute(*(c.rca + c.rfree)).packed_axis)
     if len(order) - 1 not in packed:
       return None
+  if not _bf16_gemm_limits_ok(c.M, c.K, c.N, 2 * c.K):  # beyond the kernels' 31-bit offsets: HIP dequantize + float GEMM
+    return None
   x = c.lhs_values(lhs)
   b, b_is4 = c.rhs_values(rhs)
   sb, _ = c.rhs_scale(rhs)

@@ -157,6 +157,76 @@ def test_weight_only_gemv(M, K, N, group, sdt, wq_type):
   assert out2.dtype == sdt
 
 
+@pytest.mark.parametrize('sdt', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('wq_type', ['int8', 'float8_e4m3fn'])
+@pytest.mark.parametrize('K,N', [(4096, 14336), (8192, 8192)])
+def test_weight_only_gemv_large_byte_weights(K, N, wq_type, sdt):
+  """Byte weights of 32 MB and more take the decode kernel's four-wavefront configuration with two row tiles (the second
+  one empty up to 16 rows): symmetric int8 and e4m3, both scale dtypes, 1 to 32 rows, each against the oracle's
+  dequantize-first dot on the same quantized weight.  The weight is quantized once per case; the rows vary inside."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  print('case gemv large', K, N, wq_type, sdt, flush=True)
+  w_np, w_t = util.make((K, N), O.BF16, seed=K + N + 11, scale=0.02)
+  wq = qarray.quantize_api(w_t, wq_type, channelwise_axes=[1], tiled_axes={0: 128}, scale_dtype=sdt)
+  owq = O.quantize_api(O.FArr(w_np, O.BF16), wq_type, channelwise_axes=[1], tiled_axes={0: 128}, scale_dtype=util.ORACLE_DT[sdt])
+  util.assert_qarray_equal(wq, owq, 'weight')
+  del w_t
+  x_np, x_t = util.make((32, K), O.BF16, seed=K + 12)
+  want_all = O.dot_general(O.FArr(x_np, O.BF16), owq, DN, O.F32).v
+  for M in (1, 8, 16, 32):
+    print('  rows', M, flush=True)
+    xm = x_t[:M].contiguous()
+    assert dg._weight_only_fit(xm, wq, DN) is not None
+    out = dg.dot_general(xm, wq, DN, preferred_element_type=torch.float32)
+    torch.cuda.synchronize()
+    got, want = util.f32np(out), want_all[:M]
+    assert got.shape == (M, N)
+    # f32 partial sums in another order than the oracle's
+    assert np.allclose(got, want, rtol=1e-3, atol=1e-3 * np.abs(want).mean()), np.abs(got - want).max()
+    outb = dg.dot_general(xm, wq, DN, preferred_element_type=torch.bfloat16)
+    assert np.allclose(util.f32np(outb), want, rtol=1e-2, atol=1e-2 * np.abs(want).mean())
+
+
+def test_decode_plan_follows_in_place_weight_updates():
+  """A natural-layout weight reaches the decode kernel through a re-laid-out copy that is kept per weight object.
+  Updating qvalue, scale or zero point in place (same tensors, new contents) must not serve the old copy."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  M, K, N = 8, 512, 384
+  x_np, x_t = util.make((M, K), O.BF16, seed=71)
+  for wq_type, asym in (('int8', False), ('int4', False), ('int8', True)):
+    kw = dict(channelwise_axes=[1], tiled_axes={0: 128})
+    if asym:
+      kw['calibration_method'] = 'minmax'
+    w1_np, w1_t = util.make((K, N), O.BF16, seed=72, scale=0.02)
+    w2_np, w2_t = util.make((K, N), O.BF16, seed=73, scale=0.05)
+    if asym:
+      w2_np = O.round_to_bf16(w2_np + 0.02)
+      w2_t = torch.from_numpy(w2_np).to(torch.bfloat16).to(util.DEV)
+    wq = qarray.quantize_api(w1_t, wq_type, scale_dtype=torch.float32, layout='natural', **kw)
+    wq2 = qarray.quantize_api(w2_t, wq_type, scale_dtype=torch.float32, layout='natural', **kw)
+    owq2 = O.quantize_api(O.FArr(w2_np, O.BF16), wq_type, scale_dtype=O.F32, **kw)
+    first = dg.dot_general(x_t, wq, DN, preferred_element_type=torch.float32)   # builds and keeps the plan
+    assert dg._DECODE_PLANS.get(id(wq)) is not None and dg._DECODE_PLANS[id(wq)][2] is not None
+    store = lambda q: q.data if isinstance(q, qarray.Int4Tensor) else q
+    store(wq.qvalue).copy_(store(wq2.qvalue))
+    wq.scale.copy_(wq2.scale)
+    if asym:
+      wq.zero_point.copy_(wq2.zero_point)
+    out = dg.dot_general(x_t, wq, DN, preferred_element_type=torch.float32)
+    torch.cuda.synchronize()
+    want = O.dot_general(O.FArr(x_np, O.BF16), owq2, DN, O.F32).v
+    got = util.f32np(out)
+    assert np.allclose(got, want, rtol=1e-3, atol=1e-3 * np.abs(want).mean()), (wq_type, asym, np.abs(got - want).max())
+    assert not torch.allclose(out, first, rtol=1e-2, atol=1e-4)
+    # each part on its own: scale only
+    wq.scale.mul_(2.0)
+    out2 = dg.dot_general(x_t, wq, DN, preferred_element_type=torch.float32)
+    torch.cuda.synchronize()
+    assert np.allclose(util.f32np(out2), 2.0 * want, rtol=1e-3, atol=2e-3 * np.abs(want).mean()), (wq_type, asym)
+
+
 @pytest.mark.parametrize('wq_type', ['int4', 'int8'])
 @pytest.mark.parametrize('M', [1, 16, 40, 100, 250])
 @pytest.mark.parametrize('K,N,group,sdt', [(512, 256, 128, torch.float32), (4224, 1024, 128, torch.bfloat16), (1024, 200, 1024, torch.bfloat16),

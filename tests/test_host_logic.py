@@ -270,3 +270,49 @@ def test_provider_pass_through_honours_batch_axes():
   assert torch.allclose(out, torch.einsum('cbkl,lknbc->bcn', a, b), atol=1e-5)
   with pytest.raises(TypeError, match='differ'):
     dg.float_dot_general(torch.zeros(2, 3), torch.zeros(4, 3), (((0,), (0,)), ((), ())))
+
+
+def test_own_kernel_size_limits_are_decided_in_python():
+  """The routes onto this library's kernels are chosen from the kernels' own address limits, so that a call beyond
+  them takes the dequantize + float GEMM route instead of raising from the C layer."""
+  from qwix_amd.core import dot_general as dg
+  # decode kernel: 31-bit lane offsets over 32 activation rows, 64 weight rows and all scales
+  assert dg._decode_kernel_limits_ok(4096, 4096, 14336, 4096, 128, False, 4)
+  assert dg._decode_kernel_limits_ok(4096, 2048, 14336, 4096, 128, True, 4)
+  assert not dg._decode_kernel_limits_ok(1 << 25, 4096, 14336, 4096, 128, False, 4)        # activation pitch
+  assert not dg._decode_kernel_limits_ok(1 << 25, 1 << 25, 64, 1 << 25, 128, False, 4)     # weight rows
+  assert not dg._decode_kernel_limits_ok(8192, 8192, 1 << 24, 8192, 128, False, 4)         # scale array
+  # bf16 tile GEMMs: each operand inside 2 GiB (a language-model head: vocabulary 131072 x K 8192 bf16 is exactly 2 GiB)
+  assert dg._bf16_gemm_limits_ok(2048, 4096, 14336, 8192)
+  assert not dg._bf16_gemm_limits_ok(512, 8192, 131072, 2 * 8192)
+  assert not dg._bf16_gemm_limits_ok(1 << 20, 4096, 4096, 8192)
+  # an activation view that starts inside a 16-byte unit or has a ragged pitch is copied, others pass through
+  x = torch.zeros(4, 264, dtype=torch.bfloat16)
+  assert dg._aligned_rows(x) is x
+  assert dg._aligned_rows(x[:, 8:]) is not None and dg._aligned_rows(x[:, 8:]).data_ptr() == x[:, 8:].data_ptr()
+  y = dg._aligned_rows(x[:, 3:259])
+  assert y.data_ptr() % 16 == 0 and y.is_contiguous() and y.shape == (4, 256)
+
+
+def test_weight_signature_sees_in_place_updates():
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  q = torch.zeros(8, 4, dtype=torch.int8)
+  s = torch.ones(1, 4)
+  z = torch.zeros(1, 4, dtype=torch.int8)
+  w = qarray.QArray(q, s, z, 'int8')
+  a = dg._weight_signature(w)
+  assert a == dg._weight_signature(w)
+  q.add_(1)
+  b = dg._weight_signature(w)
+  assert b != a
+  s.mul_(2.0)
+  c = dg._weight_signature(w)
+  assert c != b
+  z.add_(1)
+  assert dg._weight_signature(w) != c
+  p = qarray.Int4Tensor(torch.zeros(8, 2, dtype=torch.uint8), (8, 4), 1)
+  w4 = qarray.QArray(p, s, None, 'int4')
+  a4 = dg._weight_signature(w4)
+  p.data.add_(1)
+  assert dg._weight_signature(w4) != a4

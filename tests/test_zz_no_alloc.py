@@ -82,3 +82,24 @@ def test_static_scratch_limit_is_enforced_on_the_host():
   with pytest.raises(NotImplementedError, match='static buffer holds'):
     _lib.call('qwix_hip_quantize_static', x.data_ptr(), _lib.BF16, 1, 256, inner, 256, _lib.INT8, _lib.ABSMAX, 0.0,
               _lib.LAYOUT_NATURAL, x.data_ptr(), x.data_ptr(), None, _lib.stream_of(x))
+
+
+def test_static_scratch_quantize_allocates_no_device_memory():
+  """What the entry point exists for: free device memory, as the driver reports it, is the same before and after a
+  series of calls (after one warm-up call, which may load the code object and resolve the array's address)."""
+  outer, reduce, inner, tile = 1, 2048, 1024, 2048
+  x = torch.randn(outer * reduce * inner, dtype=torch.float32).to(torch.bfloat16).to(DEV)
+  q = torch.empty(outer * reduce * inner, dtype=torch.uint8, device=DEV)
+  scale = torch.empty(inner, dtype=torch.bfloat16, device=DEV)
+  st = _lib.stream_of(x)
+  args = (x.data_ptr(), _lib.BF16, outer, reduce, inner, tile, _lib.INT8, _lib.ABSMAX, 0.0, _lib.LAYOUT_REDUCE_MINOR,
+          q.data_ptr(), scale.data_ptr(), None, st)
+  _lib.call('qwix_hip_quantize_static', *args)
+  torch.cuda.synchronize()
+  free_before = torch.cuda.mem_get_info()[0]
+  reserved_before = torch.cuda.memory_reserved()
+  for _ in range(8):
+    _lib.call('qwix_hip_quantize_static', *args)
+  torch.cuda.synchronize()
+  assert torch.cuda.mem_get_info()[0] == free_before
+  assert torch.cuda.memory_reserved() == reserved_before
