@@ -182,8 +182,10 @@ def test_weight_only_gemv_large_byte_weights(K, N, wq_type, sdt):
     torch.cuda.synchronize()
     got, want = util.f32np(out), want_all[:M]
     assert got.shape == (M, N)
-    # f32 partial sums in another order than the oracle's
-    assert np.allclose(got, want, rtol=1e-3, atol=1e-3 * np.abs(want).mean()), np.abs(got - want).max()
+    # f32 scales: f32 partial sums in another order than the oracle's.  bf16 scales: the oracle rounds every dequantized
+    # weight to bf16 (2^-9 relative each) where the kernel keeps q * scale in f32: the tolerance of a bf16 result.
+    tol = 1e-3 if sdt == torch.float32 else 1e-2
+    assert np.allclose(got, want, rtol=tol, atol=tol * np.abs(want).mean()), np.abs(got - want).max()
     outb = dg.dot_general(xm, wq, DN, preferred_element_type=torch.bfloat16)
     assert np.allclose(util.f32np(outb), want, rtol=1e-2, atol=1e-2 * np.abs(want).mean())
 
