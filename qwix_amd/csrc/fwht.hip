@@ -8,6 +8,8 @@
 // f32; the result is rounded once to the array dtype, exactly where the reference rounds the
 // output of its dense x @ H.  In the fused variant the rounded row is then quantized in place:
 // absmax per row or per group, scale, divide, round, pack -- only qvalues and scales reach HBM.
+#include <algorithm>
+
 #include "common.h"
 
 namespace qwix {
@@ -375,6 +377,420 @@ __global__ void __launch_bounds__(RegFwht<B>::kThreads)
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// bf16 rows of 8192 elements: seven of the thirteen butterfly levels on the matrix cores.
+//
+// H_8192 is a Kronecker product over the 13 index bits and the factors commute, so any seven bits may be transformed
+// first, as one multiplication by H_128 = [(-1)^popcount(k & n)], and the other six by butterflies.  The first
+// factor sees the bf16 inputs themselves: the products with +-1 are exact and v_mfma_f32_32x32x16_bf16 adds them in
+// f32, which is what a butterfly network in f32 does too (sums of small integers stay exact either way).  One
+// WAVEFRONT owns a row, 128 elements per lane, and nothing goes through LDS but the constant matrix:
+//
+//   element index bits   i[12:10] = j    i[9] = mb    i[8] = h    i[7:3] = ml    i[2:0] = e
+//   load (mb, j)         lane l = 32 h + ml reads the 16 bytes at (j, mb, l): 1 KB contiguous per instruction
+//   MFMA operand A       rows m = ml (two blocks mb), k = j + 8 h + 16 kk: the eight loads of a lane, transposed in
+//                        registers (16-bit interleaves), give for each e the eight j of one k-step kk(e)
+//   MFMA operand B       H_128 fragments (k-step, column block nb) from a table in LDS
+//   MFMA result          lane l holds column n = (l & 31) + 32 nb of H_128's output, i.e. index bits
+//                        i[12:10] = l[2:0], i[8] = l[3], i[2] = l[4], i[1:0] = nb, and rows m = 8 (r / 4) + 4 h + r % 4:
+//                        i[4:3] = r[1:0], i[5] = h, i[7:6] = r[3:2], i[9] = mb
+//   butterflies          over the six m bits: r[0..3] and mb inside the lane, h by one v_permlane32_swap per pair of
+//                        registers (mb = 0, mb = 1), after which the lane half stands for i[9] and the pair for i[5]
+//   finish               a lane ends with runs of four consecutive elements (i[1:0]); two rounds of v_permlane16_swap
+//                        on the packed results (over i[3], then i[4]) turn them into runs of sixteen
+//
+// The sign vector in front of the transform is applied as an XOR of sign bits on the packed inputs.
+struct HFragTable {
+  uint32_t w[8 * 4 * 64 * 4];  // [k-step][column block][lane][4 dwords = 8 bf16]
+};
+constexpr HFragTable make_hfrag_table() {
+  HFragTable t{};
+  for (int kk = 0; kk < 8; ++kk)
+    for (int nb = 0; nb < 4; ++nb)
+      for (int l = 0; l < 64; ++l)
+        for (int d = 0; d < 4; ++d) {
+          uint32_t word = 0;
+          for (int half = 0; half < 2; ++half) {
+            const int k = 16 * kk + 8 * (l >> 5) + 2 * d + half, n = 32 * nb + (l & 31);
+            int par = 0;
+            for (int b = 0; b < 7; ++b) par ^= ((k & n) >> b) & 1;
+            word |= static_cast<uint32_t>(par ? 0xBF80u : 0x3F80u) << (16 * half);
+          }
+          t.w[((kk * 4 + nb) * 64 + l) * 4 + d] = word;
+        }
+  return t;
+}
+__device__ const HFragTable kHFrag = make_hfrag_table();
+
+typedef __bf16 fw_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float fw_v16f __attribute__((ext_vector_type(16)));
+typedef int fw_v4i __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t dword_of(const uint4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+
+// Swaps A's lanes 16-31 / 48-63 with B's lanes 0-15 / 32-47.
+__device__ __forceinline__ void swap_rows16(uint32_t& a, uint32_t& b) {
+  const auto r = __builtin_amdgcn_permlane16_swap(a, b, false, false);
+  a = r[0];
+  b = r[1];
+}
+
+// MODE 0: write y (bf16).  MODE 1: quantize to QT, one absmax scale per 2^ltile elements (ltile == 13: per row).
+template <int MODE, int QT, bool PRE, bool POST>
+__global__ void __launch_bounds__(512)
+    fwht_mfma_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ pre, const uint16_t* __restrict__ post,
+                     float out_scale, int ltile, int rows, void* __restrict__ y, void* __restrict__ scale) {
+  constexpr int B = 13, n = 1 << B;
+  constexpr int EB = (MODE == 0) ? 16 : (QT == QWIX_INT4 ? 4 : 8);  // bits per stored element
+  constexpr int ROW_BYTES = n * EB / 8;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t fw_smem[];
+  uint32_t* htab = reinterpret_cast<uint32_t*>(fw_smem);                  // 32 KB: the H_128 fragments
+  uint8_t* stage = fw_smem + 32768 + (threadIdx.x >> 6) * ROW_BYTES;      // this wavefront's finished row
+  const int tid = threadIdx.x;
+  const int nwaves = gridDim.x * 8;
+
+  uint4 raw[2][8];
+  // loads of a row: (mb, j) -> 16 bytes at element (j << 10) | (mb << 9) | (lane << 3)
+  auto load_row = [&](int row) {
+    int ln = tid & 63;
+    asm volatile("" : "+v"(ln));  // opaque: the addresses are rebuilt here instead of living (spilled) across the loop
+    const uint16_t* src = x + static_cast<int64_t>(row) * n + (ln << 3);
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) raw[mb][j] = nt_load16(reinterpret_cast<const uint4*>(src + ((j << 10) | (mb << 9))));
+  };
+  int row = blockIdx.x * 8 + (tid >> 6);
+  if (row < rows) load_row(row);
+  // the constant matrix, under the latency of the first row
+  for (int i = tid; i < 8 * 4 * 64; i += 512)
+    reinterpret_cast<uint4*>(htab)[i] = reinterpret_cast<const uint4*>(kHFrag.w)[i];
+  __syncthreads();
+  for (; row < rows; row += nwaves) {
+    const int64_t base = static_cast<int64_t>(row) * n;
+    // Opaque per row: the per-lane addresses below are rebuilt for every row instead of being kept (and spilled)
+    // across the whole loop.
+    int lane = tid & 63;
+    asm volatile("" : "+v"(lane));
+    const int l4 = (lane >> 4) & 1, hh = lane >> 5;
+    // after all exchanges: element index of this lane's (pair p, register r) run, without the run's own low bits
+    const int lane_bits = (((lane >> 3) & 1) << 8) | (hh << 9) | ((lane & 7) << 10);
+    if constexpr (PRE) {
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const uint4 sg = *reinterpret_cast<const uint4*>(pre + ((j << 10) | (mb << 9) | (lane << 3)));
+          raw[mb][j].x ^= sg.x & 0x80008000u;
+          raw[mb][j].y ^= sg.y & 0x80008000u;
+          raw[mb][j].z ^= sg.z & 0x80008000u;
+          raw[mb][j].w ^= sg.w & 0x80008000u;
+        }
+    }
+    // ---- H_128 on the matrix cores: all four column blocks (nb = i[1:0]) of both row blocks
+    auto run_index = [&](int p, int r) { return (l4 << 2) | ((r & 3) << 3) | (p << 5) | ((r >> 2) << 6) | lane_bits; };
+    uint32_t pk[2][2][16];  // [pair p][half][r]: the finished elements i[1:0] = 2 half, 2 half + 1 as packed bf16
+    fw_v16f acc[2][4];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+      // k-step kk multiplies element e of every 16-byte load: k[4] = i[2], k[5] = i[0], k[6] = i[1]
+      constexpr int kSel[2] = {0x05040100, 0x07060302};  // low halves / high halves of two dwords
+      const int e = ((kk & 1) << 2) | (((kk >> 2) & 1) << 1) | ((kk >> 1) & 1);
+      fw_v4i a[2];
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const uint32_t lo = dword_of(raw[mb][2 * d], e >> 1), hi = dword_of(raw[mb][2 * d + 1], e >> 1);
+          a[mb][d] = static_cast<int>(__builtin_amdgcn_perm(hi, lo, kSel[e & 1]));
+        }
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb) {
+        const fw_v4i b = *reinterpret_cast<const fw_v4i*>(htab + ((kk * 4 + nb) * 64 + lane) * 4);
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+          acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(fw_bf16x8, a[mb]),
+                                                                __builtin_bit_cast(fw_bf16x8, b), acc[mb][nb], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // The inputs are used up: request the next row of this wavefront now, under the butterflies and the finish.
+    if (row + nwaves < rows) load_row(row + nwaves);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- the rest in two halves (nb = 0, 1 and nb = 2, 3): less is alive at a time
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      // ---- butterflies over the register bits r[0..3] and mb
+      float v[2][2][16];
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int nl = 0; nl < 2; ++nl)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) v[mb][nl][r] = acc[mb][2 * half + nl][r];
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+          for (int nl = 0; nl < 2; ++nl)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              if ((r & (1 << s)) == 0) {
+                const float a0 = v[mb][nl][r], c0 = v[mb][nl][r | (1 << s)];
+                v[mb][nl][r] = a0 + c0;
+                v[mb][nl][r | (1 << s)] = a0 - c0;
+              }
+      // mb inside the lane, then the bit held by the lane half (h = i[5]): trade it for i[9].  After the swap the lower
+      // half of the wavefront holds both h of mb = 0 and the upper half both h of mb = 1; index 0 / 1 of the pair is i[5].
+#pragma unroll
+      for (int nl = 0; nl < 2; ++nl)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float m0 = v[0][nl][r] + v[1][nl][r], m1 = v[0][nl][r] - v[1][nl][r];
+          const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(m0), __float_as_uint(m1), false, false);
+          const float a0 = __uint_as_float(sw[0]), c0 = __uint_as_float(sw[1]);
+          v[0][nl][r] = a0 + c0;
+          v[1][nl][r] = a0 - c0;
+        }
+      // v[p][nl][r] is element i = nl | half << 1 | l4 << 2 | r[1:0] << 3 | p << 5 | r[3:2] << 6 | lane_bits
+      // ---- sign behind the transform, rounding to bf16, scale
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float t0 = v[p][0][r], t1 = v[p][1][r];
+          if constexpr (POST) {
+            const uint32_t w = *reinterpret_cast<const uint32_t*>(post + run_index(p, r) + 2 * half);
+            t0 *= __uint_as_float(w << 16);
+            t1 *= __uint_as_float(w & 0xFFFF0000u);
+          }
+          uint32_t w2 = pack_bf16x2(t0, t1);
+          if (out_scale != 1.0f) w2 = pack_bf16x2(__uint_as_float(w2 << 16) * out_scale, __uint_as_float(w2 & 0xFFFF0000u) * out_scale);
+          pk[p][half][r] = w2;
+        }
+      __builtin_amdgcn_sched_barrier(0);  // the halves one after the other: together they do not fit the register file
+    }
+    // ---- pack every run of four, then make runs of sixteen: word[p][r][..] -> out[p][r >> 2][..]
+    constexpr int W = (MODE == 0) ? 2 : 1;          // dwords per run of four (int4: 16 bits in one dword)
+    uint32_t word[2][16][W];
+    if constexpr (MODE == 0) {
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          word[p][r][0] = pk[p][0][r];
+          word[p][r][1] = pk[p][1][r];
+        }
+    } else {
+      // |x| of bf16 orders like its low 15 bits
+      typedef unsigned short fw_u16x2 __attribute__((ext_vector_type(2)));
+      // quantizes the run (p, r) with scale s1 (r1 = its reciprocal) into word[p][r]
+      auto quantize_run4 = [&](int p, int r, float s1, float r1) {
+        Divider<BF16, false, false> div(1.f);  // zero quotients come out as +0; e4m3 takes its signs from the dividends
+        div.s = s1;
+        div.r = r1;
+        float t[4];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          t[2 * hf] = __uint_as_float(pk[p][hf][r] << 16);
+          t[2 * hf + 1] = __uint_as_float(pk[p][hf][r] & 0xFFFF0000u);
+          div.pair_unsigned(t[2 * hf], t[2 * hf + 1]);
+        }
+        if constexpr (QT == QWIX_INT8) {
+          word[p][r][0] = pack4_low_bytes(rne_bits_clamped(t[0], -128.f, 127.f), rne_bits_clamped(t[1], -128.f, 127.f),
+                                          rne_bits_clamped(t[2], -128.f, 127.f), rne_bits_clamped(t[3], -128.f, 127.f));
+        } else if constexpr (QT == QWIX_INT4) {
+          word[p][r][0] = (rne_bits_clamped(t[0], -8.f, 7.f) & 0xFu) | ((rne_bits_clamped(t[1], -8.f, 7.f) & 0xFu) << 4) |
+                          ((rne_bits_clamped(t[2], -8.f, 7.f) & 0xFu) << 8) | ((rne_bits_clamped(t[3], -8.f, 7.f) & 0xFu) << 12);
+        } else {
+          // a quotient carries the sign of its dividend, zero quotients included: the four sign bits come from there
+          const uint32_t w = to_e4m3x2_bounded(t[0], t[1]) | (to_e4m3x2_bounded(t[2], t[3]) << 16);
+          word[p][r][0] = (__builtin_amdgcn_perm(pk[p][1][r], pk[p][0][r], 0x07050301u) & 0x80808080u) | (w & 0x7F7F7F7Fu);
+        }
+      };
+      __builtin_amdgcn_sched_barrier(0);
+      if (ltile == B) {
+        fw_u16x2 m = {0, 0};
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+          for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) m = __builtin_elementwise_max(m, __builtin_bit_cast(fw_u16x2, pk[p][hf][r] & 0x7FFF7FFFu));
+        const float am = wave_xor_max(bf16_bits_to_f32(m[0] > m[1] ? m[0] : m[1]), 64);
+        const float s1 = sym_scale<BF16, QT>(am), r1 = __builtin_amdgcn_rcpf(s1);
+        if (lane == 0) store1<BF16>(scale, row, s1);
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            quantize_run4(p, r, s1, r1);
+            if (r & 1) __builtin_amdgcn_sched_barrier(0);  // two runs at a time: all 32 at once do not fit the registers
+          }
+      } else {
+        float gm[2][16];
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const fw_u16x2 m = __builtin_elementwise_max(__builtin_bit_cast(fw_u16x2, pk[p][0][r] & 0x7FFF7FFFu),
+                                                         __builtin_bit_cast(fw_u16x2, pk[p][1][r] & 0x7FFF7FFFu));
+            gm[p][r] = bf16_bits_to_f32(m[0] > m[1] ? m[0] : m[1]);
+          }
+        // index bits below ltile, in the order they sit: i[2] = lane bit 4, i[3], i[4] = r[0], r[1], i[5] = p,
+        // i[6], i[7] = r[2], r[3], i[8] = lane bit 3
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) gm[p][r] = fmaxf(gm[p][r], __shfl_xor(gm[p][r], 16, 64));
+        auto over_r = [&](int bit) {
+#pragma unroll
+          for (int p = 0; p < 2; ++p)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              if ((r & bit) == 0) {
+                const float m = fmaxf(gm[p][r], gm[p][r | bit]);
+                gm[p][r] = m;
+                gm[p][r | bit] = m;
+              }
+        };
+        if (ltile > 3) over_r(1);
+        if (ltile > 4) over_r(2);
+        if (ltile > 5) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float m = fmaxf(gm[0][r], gm[1][r]);
+            gm[0][r] = m;
+            gm[1][r] = m;
+          }
+        }
+        if (ltile > 6) over_r(4);
+        if (ltile > 7) over_r(8);
+        if (ltile > 8) {
+#pragma unroll
+          for (int p = 0; p < 2; ++p)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) gm[p][r] = fmaxf(gm[p][r], __shfl_xor(gm[p][r], 8, 64));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float s1 = sym_scale<BF16, QT>(gm[p][r]);
+            const int i0 = run_index(p, r);
+            if ((i0 & ((1 << ltile) - 1)) == 0) store1<BF16>(scale, (base + i0) >> ltile, s1);
+            quantize_run4(p, r, s1, __builtin_amdgcn_rcpf(s1));
+            if (r & 1) __builtin_amdgcn_sched_barrier(0);
+          }
+      }
+    }
+    // round 1 over r[0] (i[3]): afterwards lane bit 4 stands for i[3] and the word order for i[2];
+    // round 2 over r[1] (i[4]): afterwards lane bit 4 stands for i[4].
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if ((r & 1) == 0)
+#pragma unroll
+          for (int w = 0; w < W; ++w) swap_rows16(word[p][r][w], word[p][r | 1][w]);
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if ((r & 2) == 0)
+#pragma unroll
+          for (int w = 0; w < W; ++w) swap_rows16(word[p][r][w], word[p][r | 2][w]);
+    // out run (p, r >> 2): words in the order r = 4 q, 4 q + 1, 4 q + 2, 4 q + 3: sixteen consecutive elements at
+    // i = l4 << 4 | p << 5 | q << 6 | lane_bits.  A lane's runs lie 32 bytes (int8) apart from its neighbour's and far
+    // from everybody else's, so the row is put together in this wavefront's piece of LDS and leaves with whole
+    // kilobytes per store instruction.  Inside every 256-byte block of the staged row the 16-byte chunks are XOR-ed
+    // with a key taken from the block number, so that the sixteen lanes that write at the same time (same chunk
+    // number, different blocks) hit different banks.
+    const int l3 = (lane >> 3) & 1, l210 = lane & 7;
+    const int wkey = (EB == 4) ? l210 : (l3 | (l210 << 1));
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int i = (l4 << 4) | (p << 5) | (q << 6) | lane_bits;
+        const int o = i * EB / 8;                                  // byte offset in the row
+        const int blk = o >> 8, c = (o >> 4) & 15;
+        uint8_t* dst = stage + (blk << 8) + ((c ^ wkey) << 4) + (o & 15);
+        if constexpr (MODE == 0) {
+          *reinterpret_cast<uint4*>(dst) = make_uint4(word[p][4 * q][0], word[p][4 * q][1], word[p][4 * q + 1][0], word[p][4 * q + 1][1]);
+          uint8_t* dst2 = stage + (blk << 8) + (((c + 1) ^ wkey) << 4);
+          *reinterpret_cast<uint4*>(dst2) =
+              make_uint4(word[p][4 * q + 2][0], word[p][4 * q + 2][1], word[p][4 * q + 3][0], word[p][4 * q + 3][1]);
+        } else if constexpr (QT == QWIX_INT4) {
+          *reinterpret_cast<uint2*>(dst) = make_uint2(word[p][4 * q][0] | (word[p][4 * q + 1][0] << 16),
+                                                      word[p][4 * q + 2][0] | (word[p][4 * q + 3][0] << 16));
+        } else {
+          *reinterpret_cast<uint4*>(dst) = make_uint4(word[p][4 * q][0], word[p][4 * q + 1][0], word[p][4 * q + 2][0], word[p][4 * q + 3][0]);
+        }
+      }
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("" ::: "memory");  // the reads below are of other lanes' writes: LDS serves one wavefront in order
+    uint8_t* out = static_cast<uint8_t*>(y) + base * EB / 8;
+#pragma unroll
+    for (int k = 0; k < ROW_BYTES / 1024; ++k) {
+      const int L = k * 1024 + lane * 16;
+      const int blk = L >> 8, c = (L >> 4) & 15;
+      // the key the writers of this block used: EB 8: blk = l3 + 2 hh + 4 l210; EB 16: blk = q[1] + 2 l3 + 4 hh + 8 l210;
+      // EB 4: blk = hh + 2 l210 (there l3 is part of the chunk number)
+      const int rkey = (EB == 8) ? ((blk & 1) | ((blk >> 2) << 1)) : (EB == 16) ? (((blk >> 1) & 1) | ((blk >> 3) << 1)) : (blk >> 1);
+      const uint4 v16 = *reinterpret_cast<const uint4*>(stage + (blk << 8) + ((c ^ rkey) << 4));
+      nt_store16(reinterpret_cast<uint4*>(out + L), v16);
+    }
+    asm volatile("" ::: "memory");
+  }
+}
+
+template <int MODE, int QT, bool PRE, bool POST>
+int launch_fwht_mfma2(const void* x, int64_t rows, const void* pre, const void* post, float out_scale, int ltile, void* y,
+                      void* scale, hipStream_t st) {
+  // eight wavefronts per workgroup (two per SIMD: one multiplies while the other adds), a row per wavefront and trip;
+  // one workgroup per CU is all that fits, so the grid is at most that and the wavefronts walk the rows
+  int cus = 0, dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  const int64_t groups = std::min<int64_t>((rows + 7) / 8, cus);
+  constexpr size_t smem = 32768 + 8 * (size_t{8192} * ((MODE == 0) ? 16 : (QT == QWIX_INT4 ? 4 : 8)) / 8);
+  auto kern = fwht_mfma_kernel<MODE, QT, PRE, POST>;
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
+  kern<<<dim3(static_cast<unsigned>(groups)), 512, smem, st>>>(
+      static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(pre), static_cast<const uint16_t*>(post), out_scale,
+      ltile, static_cast<int>(rows), y, scale);
+  return check_launch("fwht (matrix cores)");
+}
+
+template <int MODE, int QT>
+int launch_fwht_mfma(const void* x, int64_t rows, const void* pre, const void* post, float out_scale, int ltile, void* y,
+                     void* scale, hipStream_t st) {
+  if (pre != nullptr) {
+    if (post != nullptr) return launch_fwht_mfma2<MODE, QT, true, true>(x, rows, pre, post, out_scale, ltile, y, scale, st);
+    return launch_fwht_mfma2<MODE, QT, true, false>(x, rows, pre, post, out_scale, ltile, y, scale, st);
+  }
+  if (post != nullptr) return launch_fwht_mfma2<MODE, QT, false, true>(x, rows, pre, post, out_scale, ltile, y, scale, st);
+  return launch_fwht_mfma2<MODE, QT, false, false>(x, rows, pre, post, out_scale, ltile, y, scale, st);
+}
+
+// bf16 rows of 8192 with 16-byte aligned operands; scale groups of 8 to 512 elements or the whole row.
+inline bool mfma_path_ok(int dtype, int logn, const void* x, const void* pre, const void* post, const void* y) {
+  return dtype == QWIX_BF16 && logn == 13 && aligned16(x) && aligned16(y) && (pre == nullptr || aligned16(pre)) &&
+         (post == nullptr || (reinterpret_cast<uintptr_t>(post) & 7) == 0);
+}
+
 template <typename D, int MODE, int QT, int B>
 int launch_fwht_reg(const void* x, int64_t rows, const void* pre, const void* post, float out_scale, int ltile,
                     void* y, void* scale, hipStream_t st) {
@@ -433,6 +849,8 @@ extern "C" int qwix_hip_fwht(const void* x, int dtype, int64_t rows, int64_t n, 
   if (!y) return fail(QWIX_ERR_INVALID_ARGUMENT, "null output");
   const size_t smem = static_cast<size_t>(n + n / 8 + 8) * sizeof(float);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (mfma_path_ok(dtype, logn, x, pre_sign, post_sign, y))
+    return launch_fwht_mfma<0, QWIX_INT8>(x, rows, pre_sign, post_sign, out_scale, logn, y, nullptr, st);
   if (reg_path_ok(logn, x, pre_sign, y) && (dtype == QWIX_BF16 || dtype == QWIX_F32)) {
     if (dtype == QWIX_BF16)
       return dispatch_fwht_reg<BF16, 0, QWIX_INT8>(logn, x, rows, pre_sign, post_sign, out_scale, logn, y, nullptr, st);
@@ -466,6 +884,11 @@ extern "C" int qwix_hip_fwht_quantize(const void* x, int dtype, int64_t rows, in
   hipStream_t st = static_cast<hipStream_t>(stream);
   int ltile = 0;
   while ((int64_t{1} << ltile) < tile) ++ltile;
+  if (mfma_path_ok(dtype, logn, x, pre_sign, post_sign, qvalue) && (qtype == QWIX_INT8 || qtype == QWIX_INT4 || qtype == QWIX_E4M3)) {
+    if (qtype == QWIX_INT8) return launch_fwht_mfma<1, QWIX_INT8>(x, rows, pre_sign, post_sign, out_scale, ltile, qvalue, scale, st);
+    if (qtype == QWIX_INT4) return launch_fwht_mfma<1, QWIX_INT4>(x, rows, pre_sign, post_sign, out_scale, ltile, qvalue, scale, st);
+    return launch_fwht_mfma<1, QWIX_E4M3>(x, rows, pre_sign, post_sign, out_scale, ltile, qvalue, scale, st);
+  }
   if (reg_path_ok(logn, x, pre_sign, qvalue) && (dtype == QWIX_BF16 || dtype == QWIX_F32) &&
       (qtype == QWIX_INT8 || qtype == QWIX_INT4 || qtype == QWIX_E4M3)) {
 #define QWIX_FWHT_R(DT, QT) return dispatch_fwht_reg<DT, 1, QT>(logn, x, rows, pre_sign, post_sign, out_scale, ltile, qvalue, scale, st)

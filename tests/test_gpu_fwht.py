@@ -29,6 +29,59 @@ def test_fwht_exact_on_small_integers(n):
     assert np.array_equal(util.f32np(yb), want.astype(np.float32))
 
 
+@pytest.mark.parametrize('rows', [3, 8, 37, 8200])
+def test_matrix_core_rotation_exact_on_small_integers(rows):
+  """bf16 rows of 8192 take seven of the thirteen butterfly levels on the matrix cores (products with +-1 and f32 sums:
+  exact on small integers like the butterflies), one wavefront per row.  Every partial sum of integers in [-4, 4] is an
+  integer below 2^24, so the result is the exact transform rounded once to bf16, for any number of rows per wavefront,
+  with and without the sign vectors in front of and behind the transform and the output factor."""
+  from qwix_amd.contrib import hadamard_rot as hr
+  n, p = 8192, 13
+  g = util.rng(rows)
+  x = g.integers(-4, 5, (rows, n)).astype(np.float32)
+  xt = torch.from_numpy(x).to(torch.bfloat16).to(util.DEV)
+  H = O.hadamard_matrix(p).astype(np.float32)
+  want = x @ H                                   # integers below 2^24: exact in f32 whatever the order
+  y = hr.fwht(xt, 1)
+  assert y.dtype == torch.bfloat16
+  assert np.array_equal(util.f32np(y), O.round_to_bf16(want))
+  pre = g.choice([-1.0, 1.0], n).astype(np.float32)
+  post = g.choice([-1.0, 1.0], n).astype(np.float32)
+  dev = lambda a: torch.from_numpy(a).to(torch.bfloat16).to(util.DEV)
+  y2 = hr.fwht(xt, 1, pre_sign=dev(pre), post_sign=dev(post), out_scale=1.0 / n)
+  want2 = O.round_to_bf16(O.round_to_bf16(((x * pre) @ H) * post) * np.float32(1.0 / n))
+  assert np.array_equal(util.f32np(y2), want2)
+  # an impulse in every position of one row picks out one row of H: every index bit is where it belongs
+  if rows == 8:
+    for pos in (1, 4, 8, 32, 256, 512, 1024, 4096, 8191, 2730):
+      e = np.zeros((1, n), np.float32)
+      e[0, pos] = 3.0
+      ye = hr.fwht(torch.from_numpy(e).to(torch.bfloat16).to(util.DEV), 1)
+      assert np.array_equal(util.f32np(ye)[0], 3.0 * H[pos]), pos
+
+
+@pytest.mark.parametrize('qtype,tile', [('int8', None), ('int8', 8), ('int4', 16), ('float8_e4m3fn', 32), ('int8', 64), ('int4', 128),
+                                        ('int8', 256), ('float8_e4m3fn', 512), ('int4', None)])
+def test_matrix_core_rotation_fused_quantize_group_sizes(qtype, tile):
+  """Every scale-group size the fused kernel takes at n = 8192 (the group's index bits sit partly in registers and
+  partly across lanes): fused == rotate, then the oracle's quantize of the rotated array, bit for bit."""
+  from qwix_amd.contrib import hadamard_rot as hr
+  from qwix_amd.core import qarray
+  n, rows = 8192, 19
+  x_np, x_t = util.make((rows, n), O.BF16, seed=tile or 1)
+  x_np[3] = 0
+  x_np[5, 100:300] *= 50                          # outliers inside a few groups
+  x_t = util.to_gpu(O.round_to_bf16(x_np), O.BF16)
+  signs = torch.from_numpy(util.rng(6).choice([-1.0, 1.0], n).astype(np.float32)).to(torch.bfloat16).to(util.DEV)
+  kw = dict(qtype=qtype, channelwise_axes=[0])
+  if tile:
+    kw['tiled_axes'] = {1: tile}
+  fused = hr.rotate_and_quantize(x_t, 1, qarray.HowToQuantize(**kw), pre_sign=signs)
+  rot = hr.fwht(x_t, 1, pre_sign=signs)
+  want = O.quantize(util.farr(rot), O.HowToQuantize(**kw))
+  util.assert_qarray_equal(fused, want, f'fused {qtype} {tile}')
+
+
 @pytest.mark.parametrize('dtype', [O.BF16, O.F32])
 @pytest.mark.parametrize('n', [64, 512, 8192])
 def test_rotate_inputs_matches_oracle_and_preserves_product(n, dtype):
