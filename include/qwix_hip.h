@@ -114,6 +114,14 @@ QWIX_API int qwix_hip_quantize_with_scale(const void* x, int dtype, int64_t oute
                                  const void* zero_point, int q_layout, void* qvalue,
                                  void* stream);
 
+/* The same with stochastic rounding (numerics.convert_to with a noise_fn, numerics.py:191-195; reached through
+ * quantize_with_scale_zero_point(..., noise_fn), qarray.py:594-635): int8 / int4 only; the quotient (plus zero point)
+ * is formed in the array dtype, widened to f32, noise[i] (f32, shaped and ordered like x) is added, and the sum is
+ * rounded half to even and saturated.  Natural layout (int4: pairs along the contiguous axis). */
+QWIX_API int qwix_hip_quantize_with_scale_noise(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner,
+                                       int64_t tile, int qtype, const void* scale, const void* zero_point,
+                                       const float* noise, void* qvalue, void* stream);
+
 /* Generic fallback for shapes the 3-D view cannot express (two tiled/reduced axes):
  * x is the row-major 5-D view (d0, r1, d2, r3, d4); tiles t1 | r1 and t3 | r3 are reduced;
  * scale is (d0, r1/t1, d2, r3/t3, d4).  Natural layout only.  Slow but complete. */

@@ -220,8 +220,9 @@ def get_symmetric_bound(qtype) -> float:
   return {INT8: 127.5, INT4: 7.5, E4M3: 448.0}[q]
 
 
-def convert_to(x: np.ndarray, qtype) -> np.ndarray:
-  """numerics.py:139-196 for int8 / int4 / e4m3 (no stochastic rounding).
+def convert_to(x: np.ndarray, qtype, noise: np.ndarray | None = None) -> np.ndarray:
+  """numerics.py:139-196 for int8 / int4 / e4m3.  `noise` (what the reference's noise_fn(x.shape) returned): added in
+  float32 before the rounding to an integer type (numerics.py:191-195); float types ignore it, as the reference does.
 
   ints: round-half-even then a saturating cast (XLA convert semantics:
   out-of-range and +-inf clamp to the bounds; NaN -> 0, unpinned).
@@ -235,6 +236,8 @@ def convert_to(x: np.ndarray, qtype) -> np.ndarray:
     c = np.where(np.isnan(x), x, np.clip(x, -448.0, 448.0))
     return f32_to_e4m3_bits(c)
   qmin, qmax = get_asymmetric_bound(q)
+  if noise is not None:
+    x = (x + np.asarray(noise, dtype=np.float32)).astype(np.float32)
   r = np.rint(x)
   r = np.where(np.isnan(r), 0.0, np.clip(r, qmin, qmax))
   return r.astype(np.int8)
@@ -414,9 +417,9 @@ def compute_scale_zero_point(calibration: Mapping[str, FArr], qtype):
 
 
 def quantize_with_scale_zero_point(
-    array: FArr, qtype, scale: FArr, zero_point: np.ndarray | None
+    array: FArr, qtype, scale: FArr, zero_point: np.ndarray | None, noise: np.ndarray | None = None
 ) -> QArray:
-  """qarray.py:594-635 (true division, no reciprocal, no noise)."""
+  """qarray.py:594-635 (true division, no reciprocal); `noise` as in convert_to."""
   if array.dtype not in _FLOAT_DTYPES:
     raise ValueError(f'Refuse to quantize: {array.dtype}')
   if zero_point is not None and zero_point.shape != scale.shape:
@@ -430,14 +433,14 @@ def quantize_with_scale_zero_point(
     if zero_point is not None:
       zpf = rnd(zero_point.astype(np.float32), d)
       q = rnd(generic_broadcast(np.add, q, zpf), d)
-  return QArray(convert_to(q, qtype), scale, zero_point, canonical_qtype(qtype))
+  return QArray(convert_to(q, qtype, noise), scale, zero_point, canonical_qtype(qtype))
 
 
-def quantize(array: FArr, how: HowToQuantize) -> QArray:
+def quantize(array: FArr, how: HowToQuantize, noise: np.ndarray | None = None) -> QArray:
   """qarray.py:638-644."""
   cal = calibrate(array, how)
   scale, zp = compute_scale_zero_point(cal, how.qtype)
-  return quantize_with_scale_zero_point(array, how.qtype, scale, zp)
+  return quantize_with_scale_zero_point(array, how.qtype, scale, zp, noise)
 
 
 def quantize_api(

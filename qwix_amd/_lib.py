@@ -33,6 +33,7 @@ SIGNATURES = {
     'qwix_hip_calibrate_rms': (_int, [_vp, _int, _c.POINTER(_i64), _i64, _i64, _f32, _vp, _vp]),
     'qwix_hip_compute_scale_zero_point': (_int, [_vp, _vp, _int, _i64, _int, _int, _vp, _vp, _vp]),
     'qwix_hip_quantize_with_scale': (_int, [_vp, _int, _i64, _i64, _i64, _i64, _int, _vp, _vp, _int, _vp, _vp]),
+    'qwix_hip_quantize_with_scale_noise': (_int, [_vp, _int, _i64, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp, _vp]),
     'qwix_hip_quantize_generic': (_int, [_vp, _int, _c.POINTER(_i64), _i64, _i64, _int, _int, _f32, _vp, _vp, _vp, _vp]),
     'qwix_hip_dequantize': (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64, _vp, _vp, _int, _vp, _vp]),
     'qwix_hip_dequantize_generic': (_int, [_vp, _int, _c.POINTER(_i64), _i64, _i64, _vp, _vp, _int, _vp, _vp]),

@@ -207,8 +207,14 @@ class _Canon:
 def _index_batch(x, axes: Sequence[int], idx: Sequence[int]):
   """x[..., idx_k at axes_k, ...] for a tensor or a QArray (scale / zero point axes of size 1 broadcast)."""
   def take(t):
-    if isinstance(t, Int4Tensor):
-      raise NotImplementedError('batch dimensions with int4 operands are not supported')
+    if isinstance(t, Int4Tensor):  # index the packed bytes; the pairs must not run along a batch axis
+      if t.packed_axis in axes:
+        raise NotImplementedError('int4 values packed along a batch axis are not supported')
+      sel = [slice(None)] * t.ndim
+      for a, i in zip(axes, idx):
+        sel[a] = i
+      kept = [a for a in range(t.ndim) if a not in axes]
+      return Int4Tensor(t.data[tuple(sel)], tuple(t.shape[a] for a in kept), kept.index(t.packed_axis))
     sel = [slice(None)] * t.ndim
     for a, i in zip(axes, idx):
       sel[a] = i if t.shape[a] != 1 else 0

@@ -582,9 +582,9 @@ def compute_scale_zero_point(calibration: Mapping[str, torch.Tensor], qtype) -> 
 
 def quantize_with_scale_zero_point(array: torch.Tensor, qtype, scale: torch.Tensor, zero_point: torch.Tensor | None,
                                    noise_fn=None, *, layout: str | None = None) -> QArray:
-  """Quantizes with a given (static) scale; the scale is first cast to the array dtype."""
-  if noise_fn is not None:
-    raise NotImplementedError('stochastic rounding is not part of the HIP path')
+  """Quantizes with a given (static) scale; the scale is first cast to the array dtype.  `noise_fn(shape)` returns the
+  noise of stochastic rounding (numerics.py:191-195): added in f32 before the rounding to an integer type; float
+  qtypes ignore it, as the reference does."""
   array = _check_float_input(array)
   if zero_point is not None and tuple(zero_point.shape) != tuple(scale.shape):
     raise ValueError(f'Expect zero_point shape {tuple(scale.shape)} but got {tuple(zero_point.shape)}')
@@ -598,6 +598,17 @@ def quantize_with_scale_zero_point(array: torch.Tensor, qtype, scale: torch.Tens
   plan = _plan(shape, tuple(d // s for d, s in zip(shape, scale.shape)))
   if plan.kind != '3d':
     raise NotImplementedError('static-scale quantization supports a single reduced axis group')
+  if noise_fn is not None and q in (numerics.INT8, numerics.INT4):
+    noise = noise_fn(shape)
+    if not isinstance(noise, torch.Tensor) or tuple(noise.shape) != shape:
+      raise ValueError(f'noise_fn must return a tensor of shape {shape}')
+    noise = noise.to(device=array.device, dtype=torch.float32).contiguous()
+    data, view = _alloc_q(shape, q, plan, _lib.LAYOUT_NATURAL, array.device)
+    zp = None if zero_point is None else zero_point.contiguous()
+    _lib.call('qwix_hip_quantize_with_scale_noise', array.data_ptr(), _lib.float_tag(array.dtype), *plan.dims,
+              plan.tiles[0], numerics.qtype_tag(q), scale.data_ptr(), _lib.ptr(zp), noise.data_ptr(), data.data_ptr(),
+              _lib.stream_of(array))
+    return QArray(view, scale, zero_point, q)
   lay = _default_layout(plan, layout)
   data, view = _alloc_q(shape, q, plan, lay, array.device)
   zp = None if zero_point is None else zero_point.contiguous()
@@ -607,9 +618,11 @@ def quantize_with_scale_zero_point(array: torch.Tensor, qtype, scale: torch.Tens
 
 
 def quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = None) -> QArray:
-  """Dynamic-range quantization: calibrate, derive scale (and zero point), quantize -- one fused pass."""
-  if how.noise_fn is not None:
-    raise NotImplementedError('stochastic rounding is not part of the HIP path')
+  """Dynamic-range quantization: calibrate, derive scale (and zero point), quantize -- one fused pass.  With a
+  `noise_fn` (stochastic rounding) the three steps run one after the other, as the reference's do (qarray.py:638-644)."""
+  if how.noise_fn is not None and numerics.canonical_qtype(how.qtype) in (numerics.INT8, numerics.INT4) and array.numel():
+    scale, zp = compute_scale_zero_point(calibrate(array, how), how.qtype)
+    return quantize_with_scale_zero_point(array, how.qtype, scale, zp, how.noise_fn, layout='natural')
   if not isinstance(array, torch.Tensor) or not numerics.should_quantize(array.dtype):
     raise ValueError(f'Refuse to quantize: {getattr(array, "dtype", type(array))}')
   shape = tuple(array.shape)

@@ -10,6 +10,7 @@
 //           and merges panels with a 32-bit atomic max into a caller-provided workspace; pass 2
 //           re-reads each panel, quantizes it, and writes either the natural layout or the
 //           reduce-minor (transposed) layout the GEMM kernels consume.
+#include <algorithm>
 #include <cstdlib>
 #include <mutex>
 
@@ -968,6 +969,37 @@ __global__ void __launch_bounds__(256)
 }
 
 // ------------------------------------------------------------------------------------ misc
+// Quantize with a given scale and noise before the rounding (stochastic rounding, numerics.py:191-195): integer
+// qtypes only; the quotient (and the zero point added to it) is formed in the array dtype as always, then widened to
+// f32, the caller's f32 noise added, and the sum rounded half to even and saturated.  Natural layout, one thread per
+// pair of consecutive elements; a training-time path, not tuned.
+template <typename D, int QT, bool ASYM>
+__global__ void __launch_bounds__(256)
+    noise_quantize_kernel(const void* __restrict__ x, int64_t pairs, int64_t reduce, int64_t inner, int64_t tile,
+                          const void* __restrict__ scale, const int8_t* __restrict__ zp, const float* __restrict__ noise,
+                          uint8_t* __restrict__ q) {
+  const int64_t ntile = reduce / tile;
+  for (int64_t pr = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; pr < pairs; pr += static_cast<int64_t>(gridDim.x) * 256) {
+    int v[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int64_t i = 2 * pr + h;
+      const int64_t c = i % inner, r = (i / inner) % reduce, o = i / (inner * reduce);
+      const int64_t si = (o * ntile + r / tile) * inner + c;
+      const Divider<D, true, true> div(load1<D>(scale, si));
+      float t = div(load1<D>(x, i));
+      if constexpr (ASYM) t = rnd<D>(t + static_cast<float>(zp[si]));
+      v[h] = to_int_q<QT>(t + noise[i]);
+    }
+    if constexpr (QT == QWIX_INT4) {
+      q[pr] = static_cast<uint8_t>(pack2_i4(v[0], v[1]));
+    } else {
+      q[2 * pr] = static_cast<uint8_t>(v[0] & 0xFF);
+      q[2 * pr + 1] = static_cast<uint8_t>(v[1] & 0xFF);
+    }
+  }
+}
+
 template <typename D, int QT, int CAL>
 __global__ void scale_zp_kernel(const void* __restrict__ c0, const void* __restrict__ c1, int64_t n,
                                 void* __restrict__ scale, int8_t* __restrict__ zp) {
@@ -1590,6 +1622,36 @@ int qwix_hip_quantize_with_scale(const void* x, int dtype, int64_t outer, int64_
   const ColGeom g = make_col_geom(outer, reduce, inner, tile, dtype == QWIX_BF16 ? 8 : 4);
   return run_cols_quantize<1>(x, dtype, g, qtype, cal, q_layout, nullptr, 0.f, qvalue, const_cast<void*>(scale),
                               const_cast<void*>(zero_point), st);
+}
+
+int qwix_hip_quantize_with_scale_noise(const void* x, int dtype, int64_t outer, int64_t reduce, int64_t inner,
+                                       int64_t tile, int qtype, const void* scale, const void* zero_point,
+                                       const float* noise, void* qvalue, void* stream) {
+  if (int e = check_geom(outer, reduce, inner, tile)) return e;
+  if (!x || !qvalue || !scale || !noise) return fail(QWIX_ERR_INVALID_ARGUMENT, "null x/qvalue/scale/noise");
+  if (qtype != QWIX_INT8 && qtype != QWIX_INT4)
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "noise is added before the rounding to an integer type only (qtype %d)", qtype);
+  const int64_t n = outer * reduce * inner;
+  if (n & 1) return fail(QWIX_ERR_UNSUPPORTED, "an even element count is needed");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t pairs = n / 2;
+  const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((pairs + 255) / 256, 65536));
+  uint8_t* qb = static_cast<uint8_t*>(qvalue);
+  const int8_t* zb = static_cast<const int8_t*>(zero_point);
+#define QWIX_NOISE(DT, QT)                                                                                          \
+  do {                                                                                                              \
+    if (zb) noise_quantize_kernel<DT, QT, true><<<blocks, 256, 0, st>>>(x, pairs, reduce, inner, tile, scale, zb, noise, qb); \
+    else noise_quantize_kernel<DT, QT, false><<<blocks, 256, 0, st>>>(x, pairs, reduce, inner, tile, scale, zb, noise, qb);  \
+  } while (0)
+  if (dtype == QWIX_BF16) {
+    if (qtype == QWIX_INT8) QWIX_NOISE(BF16, QWIX_INT8); else QWIX_NOISE(BF16, QWIX_INT4);
+  } else if (dtype == QWIX_F32) {
+    if (qtype == QWIX_INT8) QWIX_NOISE(F32, QWIX_INT8); else QWIX_NOISE(F32, QWIX_INT4);
+  } else {
+    return fail(QWIX_ERR_INVALID_ARGUMENT, "dtype %d is not f32/bf16", dtype);
+  }
+#undef QWIX_NOISE
+  return check_launch("quantize_with_scale_noise");
 }
 
 int qwix_hip_quantize_generic(const void* x, int dtype, const int64_t dims[5], int64_t t1, int64_t t3, int qtype,

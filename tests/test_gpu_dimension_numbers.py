@@ -279,3 +279,35 @@ def test_einsum_mixed_operands_scalar_and_incompatible_shapes():
   assert tuple(out.shape) == (128, 128) and ((out - 2 * lhs).abs().mean() / (2 * lhs).abs().mean()).item() < 0.02
   with pytest.raises(ValueError, match='Cannot broadcast'):
     es.einsum('BTNH,BSNH->BTNS', torch.ones(1, 2, 3, 8, device=util.DEV), torch.ones(1, 3, 4, 8, device=util.DEV))
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('group', [None, 128])
+def test_int4_weights_with_a_batch_axis(group, dtype):
+  """Batched contraction 'bmk,bkn->bmn' against int4 weights (one weight matrix per batch element, with and without
+  sub-channel scales): the packed bytes are sliced per element, each element runs the 2-D kernels; int8 activations
+  give the oracle's int32 sums and outputs bit for bit, bf16 activations (weight-only) meet the 1e-2 bar."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  B, M, K, N = 3, 24, 256, 72
+  x_np, x_t = util.make((B, M, K), dtype, seed=61)
+  w_np, w_t = util.make((B, K, N), dtype, seed=62, scale=0.05)
+  rkw = dict(qtype='int4', channelwise_axes=[0, 2])
+  if group:
+    rkw['tiled_axes'] = {1: group}
+  lkw = dict(qtype='int8', channelwise_axes=[0, 1])
+  wq = qarray.quantize(w_t, qarray.HowToQuantize(**rkw))
+  owq = O.quantize(O.FArr(w_np, dtype), O.HowToQuantize(**rkw))
+  util.assert_qarray_equal(wq, owq, 'int4 weights')
+  xq = qarray.quantize(x_t, qarray.HowToQuantize(**lkw))
+  oxq = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(**lkw))
+  dn = (((2,), (1,)), ((0,), (0,)))
+  out = dg._fast_dot_general(xq, wq, dn, exact=True)   # the mode whose roundings are the reference's, step by step
+  torch.cuda.synchronize()
+  want = O.dot_general(oxq, owq, dn)
+  assert tuple(out.shape) == (B, M, N)
+  assert np.array_equal(util.f32np(out), want.v)
+  # weight-only: a float activation against the batched int4 weight
+  out2 = dg.dot_general(x_t, wq, dn)
+  want2 = O.dot_general(O.FArr(x_np, dtype), owq, dn)
+  np.testing.assert_allclose(util.f32np(out2), want2.v, rtol=1e-2, atol=1e-2 * float(np.abs(want2.v).mean()))

@@ -340,3 +340,33 @@ def test_array_methods_commute_with_dequantize():
   assert torch.equal(qarray.dequantize(q[..., 1]), full[..., 1])
   assert torch.equal(qarray.dequantize(q[1]), full[1])
   assert torch.equal(qarray.dequantize(q.transpose(1, 2, 0)), full.permute(1, 2, 0))
+
+
+@pytest.mark.parametrize('qtype', ['int8', 'int4'])
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('shape,kw', [((64, 512), dict(channelwise_axes=[0])), ((256, 96), dict(channelwise_axes=[1])),
+                                      ((128, 256), dict(channelwise_axes=[1], tiled_axes={0: 64})),
+                                      ((6, 40, 64), dict(channelwise_axes=[0, 1], calibration_method='minmax')),
+                                      ((32, 128), dict(calibration_method='fixed,-3,3'))])
+def test_stochastic_rounding_with_caller_noise(shape, kw, dtype, qtype):
+  """`noise_fn` (numerics.py:191-195): the noise is added in f32 before the rounding.  The same noise array through the
+  HIP kernel and through the oracle: qvalues, scales and zero points bit for bit; float qtypes ignore the noise."""
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make(shape, dtype, seed=sum(shape))
+  noise_np = util.rng(17).uniform(-0.5, 0.5, shape).astype(np.float32)
+  noise_t = torch.from_numpy(noise_np).to(util.DEV)
+  calls = []
+  def noise_fn(s):
+    calls.append(tuple(s))
+    return noise_t
+  how = qarray.HowToQuantize(qtype=qtype, noise_fn=noise_fn, **kw)
+  got = qarray.quantize(x_t, how)
+  torch.cuda.synchronize()
+  assert calls == [shape]
+  want = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(qtype=qtype, **kw), noise_np)
+  util.assert_qarray_equal(got, want, f'noise {qtype}')
+  plain = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(qtype=qtype, **kw))
+  assert (want.qvalue != plain.qvalue).mean() > 0.1        # the noise did move roundings
+  if 'calibration_method' not in kw:
+    f8 = qarray.quantize(x_t, qarray.HowToQuantize(qtype='float8_e4m3fn', noise_fn=noise_fn, **kw))
+    util.assert_qarray_equal(f8, O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(qtype='float8_e4m3fn', **kw)), 'f8 ignores noise')

@@ -329,3 +329,34 @@ def test_rms_calibration_closed_forms():
   assert cal['absmax'].v.shape == (3, 4) and np.all(cal['absmax'].v == 1.0)
   with pytest.raises(ValueError, match='scale factor'):
     O.calibrate(x, O.HowToQuantize(qtype='int8', calibration_method='rms'))
+
+
+def test_stochastic_rounding_noise_is_added_in_float32():
+  """numerics.py:191-195: the noise meets the scaled value in float32, not in the array dtype.  The reference's own
+  example: bf16(41) - 0.4 rounds to 41 (40.6), where bf16 arithmetic would give round(40.5) = 40.  Brute force on a
+  small grid: the rounding is floor(v + noise + 0.5) away from ties for every value and noise."""
+  x = O.FArr(np.array([[41.0, -41.0, 3.0, 0.0]], np.float32), O.BF16)
+  one = O.FArr(np.ones((1, 1), np.float32), O.BF16)
+  noise = np.array([[-0.4, 0.4, 0.49, -0.49]], np.float32)
+  q = O.quantize_with_scale_zero_point(x, 'int8', one, None, noise)
+  assert q.qvalue.tolist() == [[41, -41, 3, 0]]
+  assert O.round_to_bf16(np.float32(41.0) - np.float32(0.4)) == 40.5   # what the bf16 sum would have been
+  # zero noise is the plain rounding; float qtypes ignore the noise
+  g = np.random.Generator(np.random.PCG64(5))
+  v = O.round_to_bf16((g.standard_normal((8, 64)) * 40).astype(np.float32))
+  for qtype in ('int8', 'int4'):
+    assert np.array_equal(O.convert_to(v, qtype, np.zeros_like(v)), O.convert_to(v, qtype))
+  assert np.array_equal(O.convert_to(v, 'float8_e4m3fn', np.full_like(v, 0.3)), O.convert_to(v, 'float8_e4m3fn'))
+  # brute force, element by element, in Python floats restricted to float32 steps
+  nz = g.uniform(-0.5, 0.5, v.shape).astype(np.float32)
+  got = O.convert_to(v, 'int8', nz)
+  for a, b, c in zip(v.ravel(), nz.ravel(), got.ravel()):
+    s = float(np.float32(a) + np.float32(b))
+    lo = np.floor(s)
+    want = lo if s - lo < 0.5 else lo + 1 if s - lo > 0.5 else (lo if lo % 2 == 0 else lo + 1)
+    assert c == int(min(max(want, -128), 127))
+  # saturation and the zero point still apply: the zero point is added in the array dtype, before the noise
+  xs = O.FArr(np.array([[300.0, -300.0, 10.0]], np.float32), O.F32)
+  qz = O.quantize_with_scale_zero_point(xs, 'int8', O.FArr(np.ones((1, 1), np.float32), O.F32),
+                                        np.array([[5]], np.int8), np.array([[0.3, -0.3, 0.4]], np.float32))
+  assert qz.qvalue.tolist() == [[127, -128, 15]]
