@@ -526,6 +526,33 @@ def test_prefill_gemm_dequantizes_in_the_kernel(M, K, N, group, asym, wq_type, o
   assert torch.allclose(got.double(), ref, rtol=1e-2 if out_dtype == torch.bfloat16 else 1e-4, atol=1e-2 * float(ref.abs().mean()))
 
 
+@pytest.mark.parametrize('wq_type', ['int4', 'int8', 'float8_e4m3fn'])
+@pytest.mark.parametrize('M', [512, 2048])
+def test_prefill_with_f32_scales_stays_within_a_bf16_rounding_of_the_f32_contraction(M, wq_type):
+  """bf16 activations x weight with f32 scales, f32 result, above the decode batch: the reference contracts the
+  dequantized weight in f32 (dot_general.py:264-275); here the dequantized weight is rounded to bf16 for the bf16
+  matrix cores (512 rows: inside the GEMM; 2048 rows: dequantize + GEMM).  One rounding of 2^-9 relative per weight, K
+  = 4096 of them per output with independent signs: the mean deviation must stay below 2^-9 of the mean magnitude
+  and every element inside the 1e-2 of a bf16 result."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  K, N = 4096, 1024
+  print('case prefill f32 scales', M, wq_type, flush=True)
+  x_np, x_t = util.make((M, K), O.BF16, seed=M + 31)
+  w_np, w_t = util.make((K, N), O.BF16, seed=M + 32, scale=0.02)
+  wq = qarray.quantize_api(w_t, wq_type, channelwise_axes=[1], tiled_axes={0: 128}, scale_dtype=torch.float32)
+  owq = O.quantize_api(O.FArr(w_np, O.BF16), wq_type, channelwise_axes=[1], tiled_axes={0: 128}, scale_dtype=O.F32)
+  util.assert_qarray_equal(wq, owq, 'weight')
+  out = dg.dot_general(x_t, wq, DN, preferred_element_type=torch.float32)
+  torch.cuda.synchronize()
+  assert out.dtype == torch.float32
+  want = O.dot_general(O.FArr(x_np, O.BF16), owq, DN, O.F32).v
+  got = util.f32np(out)
+  mag = np.abs(want).mean()
+  assert np.abs(got - want).mean() < 2.0 ** -9 * mag, np.abs(got - want).mean() / mag
+  assert np.allclose(got, want, rtol=1e-2, atol=1e-2 * mag), np.abs(got - want).max() / mag
+
+
 def test_dequantizing_gemm_argument_checks():
   """qwix_hip_gemm_bf16_wq refuses what its tile loop cannot walk (K not in whole groups of four slabs, groups that
   are not whole slabs, unaligned rows, other weight types) with an error code and a message instead of launching."""
