@@ -374,9 +374,69 @@ def _qtype_of(x) -> str:
   return numerics.canonical_qtype(x.dtype)
 
 
+def _narrow_tiles(x, tiles: Mapping[int, tuple[int, int]]):
+  """The operand restricted to tile `i` of `n` elements along every axis of `tiles` ({axis: (i, n)}): values are
+  narrowed, scale and zero point keep the one entry of that tile (or their single entry when this operand is not
+  tiled along the axis).  Packed int4 values are narrowed in bytes and copied (the kernels need rows that start at
+  a byte)."""
+  def values(v):
+    if isinstance(v, Int4Tensor):
+      data, shape = v.data, list(v.shape)
+      for a, (i, n) in tiles.items():
+        if a == v.packed_axis:
+          if n % 2:
+            raise NotImplementedError('int4 values tiled by an odd tile size along their packed axis')
+          data = data.narrow(a, i * n // 2, n // 2)
+        else:
+          data = data.narrow(a, i * n, n)
+        shape[a] = n
+      return Int4Tensor(data.contiguous(), tuple(shape), v.packed_axis)
+    for a, (i, n) in tiles.items():
+      v = v.narrow(a, i * n, n)
+    return v
+
+  def per_tile(t):
+    for a, (i, _) in tiles.items():
+      if t.shape[a] != 1:
+        t = t.narrow(a, i, 1)
+    return t
+
+  if isinstance(x, QArray):
+    return QArray(values(x.qvalue), per_tile(x.scale), None if x.zero_point is None else per_tile(x.zero_point), x.qtype)
+  return values(x)
+
+
+def _tile_by_tile(lhs, rhs, dimension_numbers, tiled, preferred_element_type, exact) -> torch.Tensor:
+  """The tiled contraction of dot_general.py:186-226, 255-260 as the reference writes it, for the operand kinds
+  that the sub-channel MFMA kernel does not take (several contracting axes, e4m3 values, tile sizes that are not
+  multiples of 128): every tile combination is an untiled contraction of its own (one launch each), scaled by that
+  tile's scales with the roundings of the untiled path; the partials are summed in f32 in row-major order of the
+  tile axes (the order of the contracting axes) and rounded once to the type the scaled partials have, then cast
+  to the result type.  `tiled` lists (lhs axis, rhs axis, tile size)."""
+  import itertools
+  acc_t, res_t = qarray.get_accumulator_and_result_type(lhs, rhs, preferred_element_type=preferred_element_type)
+  cur = acc_t  # dtype of a scaled partial: the accumulator's, promoted by every scale it meets
+  for operand in (lhs, rhs):
+    if isinstance(operand, QArray):
+      sd = operand.scale.dtype
+      cur = sd if cur == torch.int32 else torch.promote_types(cur, sd)
+  counts = [lhs.shape[l] // n for l, _, n in tiled]
+  total = None
+  for combo in itertools.product(*[range(c) for c in counts]):
+    lsel = {l: (i, n) for (l, _, n), i in zip(tiled, combo)}
+    rsel = {r: (i, n) for (_, r, n), i in zip(tiled, combo)}
+    part = _fast_dot_general(_narrow_tiles(lhs, lsel), _narrow_tiles(rhs, rsel), dimension_numbers,
+                             preferred_element_type=preferred_element_type, exact=exact, _partial_dtype=cur)
+    part = part.to(torch.float32) if cur != torch.int32 else part
+    total = part if total is None else total + part
+  return total.to(cur).to(res_t)
+
+
 def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, *, exact: bool = False,
-                      return_accumulators: bool = False, **kwargs) -> torch.Tensor:
-  """Contract the quantized values on the matrix cores, then scale: out = ((acc * sx) * sy)."""
+                      return_accumulators: bool = False, _partial_dtype=None, **kwargs) -> torch.Tensor:
+  """Contract the quantized values on the matrix cores, then scale: out = ((acc * sx) * sy).
+  `_partial_dtype` (internal, set by the tile-by-tile route): the dtype the result is delivered in, in place of the
+  result type, while the accumulator type still follows `preferred_element_type`."""
   del kwargs
   if _is_float_array(lhs) or _is_float_array(rhs):
     # The reference contracts a raw float operand with the other side's quantized values and scales the
@@ -404,9 +464,18 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
     if lt.get(l) and rt.get(r) and lt[l] != rt[r]:
       raise ValueError(f'Contracting axes must be tiled with the same tile size. lhs_tiled_axes={lt} rhs_tiled_axes={rt} {dimension_numbers=}')
   acc_t, res_t = qarray.get_accumulator_and_result_type(lhs, rhs, preferred_element_type=preferred_element_type)
+  if _partial_dtype is not None:
+    res_t = _partial_dtype
   lq, rq = _qtype_of(lhs), _qtype_of(rhs)
   if lq == numerics.INT4:
     lq = numerics.INT8  # lhs_values widens int4 rows
+  tiled = [(l, r, lt.get(l) or rt.get(r)) for l, r in zip(c.lca, c.rca) if lt.get(l) or rt.get(r)]
+  if tiled and (len(c.lca) > 1 or lq != numerics.INT8 or rq not in (numerics.INT8, numerics.INT4)
+                or any(n % 128 for _, _, n in tiled)):
+    # what the sub-channel MFMA kernel does not take runs tile by tile on the untiled kernels
+    if return_accumulators:
+      raise NotImplementedError('raw accumulators are returned for one tiled contracting axis of int8 x int8/int4 only')
+    return _tile_by_tile(lhs, rhs, dimension_numbers, tiled, preferred_element_type, exact)
   a = c.lhs_values(lhs)
   b, b_is4 = c.rhs_values(rhs)
   sa, ga = c.lhs_scale(lhs) if isinstance(lhs, QArray) else (None, 1)

@@ -311,3 +311,97 @@ def test_int4_weights_with_a_batch_axis(group, dtype):
   out2 = dg.dot_general(x_t, wq, dn)
   want2 = O.dot_general(O.FArr(x_np, dtype), owq, dn)
   np.testing.assert_allclose(util.f32np(out2), want2.v, rtol=1e-2, atol=1e-2 * float(np.abs(want2.v).mean()))
+
+
+def _pair(lshape, rshape, lhow, rhow, dtype, seed):
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make(lshape, dtype, seed=seed)
+  w_np, w_t = util.make(rshape, dtype, seed=seed + 1, scale=0.05)
+  xq, wq = qarray.quantize(x_t, qarray.HowToQuantize(**lhow)), qarray.quantize(w_t, qarray.HowToQuantize(**rhow))
+  oxq, owq = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(**lhow)), O.quantize(O.FArr(w_np, dtype), O.HowToQuantize(**rhow))
+  util.assert_qarray_equal(xq, oxq, 'lhs')
+  util.assert_qarray_equal(wq, owq, 'rhs')
+  return xq, wq, oxq, owq
+
+
+# lhs (T, N, H) x rhs (N, H, D), contracting (N, H): the output projection of attention
+TILED_DN = (((1, 2), (0, 1)), ((), ()))
+TILED_CASES = [
+    # both contracting axes tiled on both sides (2 x 2 tile combinations)
+    ('both axes, both sides', (24, 256, 256), (256, 256, 40), {1: 128, 2: 128}, {0: 128, 1: 128}),
+    # last axis tiled on the weight only, heads untiled: groups that are not contiguous in the flattened K
+    ('last axis, weight only', (24, 4, 256), (4, 256, 40), {}, {1: 128}),
+    # first contracting axis tiled only
+    ('first axis only', (24, 256, 8), (256, 8, 40), {1: 128}, {0: 128}),
+    # activation tiled, weight per channel
+    ('lhs only', (10, 2, 384), (2, 384, 24), {2: 128}, {}),
+]
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('name,lshape,rshape,ltiles,rtiles', TILED_CASES)
+def test_tiled_scales_over_several_contracting_axes_bit_exact(name, lshape, rshape, ltiles, rtiles, dtype):
+  """dot_general.py:93-122, 186-226, 255-260: every tiled contracting axis becomes a tile axis of the product, the
+  partials are scaled tile by tile and summed.  int8 x int8: exact partials, the oracle's roundings, the oracle's
+  order of the sum over tiles: equal bits."""
+  from qwix_amd.core import dot_general as dg
+  print('case tiled multi-axis', name, dtype, flush=True)
+  xq, wq, oxq, owq = _pair(lshape, rshape, dict(qtype='int8', channelwise_axes=[0], tiled_axes=ltiles),
+                           dict(qtype='int8', channelwise_axes=[2], tiled_axes=rtiles), dtype, seed=sum(lshape))
+  assert dg._use_fast_path(xq, wq, TILED_DN)
+  for pet, opet in ((None, None), (torch.float32, O.F32)):
+    out = dg.dot_general(xq, wq, TILED_DN, preferred_element_type=pet)
+    torch.cuda.synchronize()
+    want = O.dot_general(oxq, owq, TILED_DN, opet)
+    assert tuple(out.shape) == tuple(want.v.shape) and out.dtype == util.TORCH_DT[want.dtype]
+    got = util.f32np(out)
+    bad = np.flatnonzero(got.ravel() != want.v.ravel())
+    assert bad.size == 0, f'{bad.size} outputs differ: {got.ravel()[bad[:5]]} vs {want.v.ravel()[bad[:5]]}'
+
+
+def test_tiled_zero_points_over_several_contracting_axes_bit_exact():
+  """An asymmetric activation tiled along the last of two contracting axes: the zero point is split with the tiles
+  (dot_general.py:196-203) and every tile's partial corrected before it is scaled."""
+  from qwix_amd.core import dot_general as dg
+  xq, wq, oxq, owq = _pair((12, 3, 256), (3, 256, 20),
+                           dict(qtype='int8', channelwise_axes=[0], tiled_axes={2: 128}, calibration_method='minmax'),
+                           dict(qtype='int8', channelwise_axes=[2], tiled_axes={1: 128}), O.BF16, seed=77)
+  assert xq.zero_point is not None
+  out = dg.dot_general(xq, wq, TILED_DN)
+  torch.cuda.synchronize()
+  want = O.dot_general(oxq, owq, TILED_DN)
+  assert np.array_equal(util.f32np(out), want.v)
+
+
+@pytest.mark.parametrize('tile', [128, 192])
+def test_tiled_scales_that_the_sub_channel_kernel_does_not_take(tile):
+  """One contracting axis, tiles of 192 (not a multiple of the kernel's 128-wide slabs): int8 bit-exact; e4m3
+  operands with sub-channel scales (no sub-channel fp8 kernel): the fp8 tolerance."""
+  from qwix_amd.core import dot_general as dg
+  dn = (((1,), (0,)), ((), ()))
+  K = 3 * tile
+  for qtype in ('int8', O.E4M3):
+    if qtype == 'int8' and tile == 128:
+      continue  # the sub-channel kernel's own case
+    print('case tile-by-tile', tile, qtype, flush=True)
+    xq, wq, oxq, owq = _pair((40, K), (K, 72), dict(qtype=qtype, channelwise_axes=[0], tiled_axes={1: tile}),
+                             dict(qtype=qtype, channelwise_axes=[1], tiled_axes={0: tile}), O.BF16, seed=tile)
+    out = dg.dot_general(xq, wq, dn, preferred_element_type=torch.float32)
+    torch.cuda.synchronize()
+    want = O.dot_general(oxq, owq, dn, O.F32).v
+    got = util.f32np(out)
+    if qtype == 'int8':
+      assert np.array_equal(got, want)
+    else:
+      assert np.allclose(got, want, rtol=1e-2, atol=1e-2 * np.abs(want).mean()), np.abs(got - want).max()
+
+
+def test_int4_weights_tiled_under_two_contracting_axes():
+  """int4 weights (N, H, D) packed along D, tiled along H: tiles are cut out of the packed bytes."""
+  from qwix_amd.core import dot_general as dg
+  xq, wq, oxq, owq = _pair((16, 2, 256), (2, 256, 48), dict(qtype='int8', channelwise_axes=[0]),
+                           dict(qtype='int4', channelwise_axes=[2], tiled_axes={1: 128}), O.BF16, seed=91)
+  out = dg._fast_dot_general(xq, wq, TILED_DN, exact=True)
+  torch.cuda.synchronize()
+  want = O.dot_general(oxq, owq, TILED_DN)
+  assert np.array_equal(util.f32np(out), want.v)
