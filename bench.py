@@ -548,6 +548,60 @@ class HadamardQdot(Workload):
     return {'workload': self.name, 'M': self.M, 'K': self.K, 'N': self.N, 'group': 128}
 
 
+class QdotSubChannel(Workload):
+  """Sub-channel w8a8: per-token, per-group activation quantize each step (groups of `group` along K), then the
+  sub-channel GEMM against a weight with one scale per group and output channel; qtype int8 or e4m3."""
+
+  bound = 'mfma'
+
+  def __init__(self, name, M, K, N, group, qtype):
+    self.name, self.M, self.K, self.N, self.group, self.qtype = name, M, K, N, group, qtype
+    self.dtype = 'int8' if qtype == 'int8' else 'f8e4m3'
+    self.metric = self.dtype + ' sub-channel qdot TOPS (group %d on both operands, activation quantize included)' % group
+    self.unit = 'TOPS'
+    self.kernel_name = 'qgemm_grouped_dma_kernel' if qtype == 'int8' else 'qgemm_grouped_kernel'
+
+  def setup(self, dev):
+    import torch
+    from qwix_amd.core import qarray
+    L = _lib()
+    g = torch.Generator(device='cpu').manual_seed(3100 + self.M)
+    self.x = torch.randn(self.M, self.K, generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+    w = (torch.randn(self.K, self.N, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(dev)
+    wq = qarray.quantize(w, qarray.HowToQuantize(qtype=self.qtype, channelwise_axes=[1], tiled_axes={0: self.group}))
+    del w
+    self.b = wq.qvalue.permute(1, 0)
+    assert self.b.is_contiguous()
+    self.sb = wq.scale.contiguous()           # (K / group, N)
+    self.ga = self.K // self.group
+    self.xq = torch.empty(self.M, self.K, dtype=wq.qvalue.dtype, device=dev)
+    self.sa = torch.empty(self.M, self.ga, dtype=torch.bfloat16, device=dev)
+    self.out = torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev)
+    self.qt = L.INT8 if self.qtype == 'int8' else L.E4M3
+    self.stream = torch.cuda.current_stream().cuda_stream
+    self.L = L
+
+  def step(self, i=0):
+    L = self.L
+    L.call('qwix_hip_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, 1, self.group, self.qt, L.ABSMAX, 0.0,
+           L.LAYOUT_NATURAL, self.xq.data_ptr(), self.sa.data_ptr(), None, None, 0, self.stream)
+    self.kernel(i)
+
+  def kernel(self, i=0):
+    L = self.L
+    L.call('qwix_hip_qgemm_grouped', self.xq.data_ptr(), self.K, self.b.data_ptr(), self.K, self.qt, self.M, self.N,
+           self.K, self.group, self.sa.data_ptr(), L.BF16, self.ga, self.sb.data_ptr(), L.BF16, self.out.data_ptr(),
+           L.BF16, self.N, 0, None, self.stream)
+
+  def work_per_step(self):
+    return 2.0 * self.M * self.N * self.K
+
+  kernel_work = work_per_step
+
+  def describe(self):
+    return {'workload': self.name, 'M': self.M, 'K': self.K, 'N': self.N, 'group': self.group, 'qtype': self.qtype}
+
+
 class RaggedQdot(Workload):
   """Mixture-of-experts matmul: the tokens are sorted by expert (uneven groups, sizes in device memory);
   per-token int8 activation quantize + one ragged MFMA GEMM against G per-channel int8 expert weights."""
@@ -955,6 +1009,8 @@ WORKLOADS = {
     'batched_qk_int8_32x2048': lambda: QdotBatched('batched_qk_int8_32x2048', 32, 2048, 2048, 128),
     'c1_ptq_mlp_graph': lambda: PtqMlpGraph('c1_ptq_mlp_graph'),
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
+    'int8_subchannel_g128_4096': lambda: QdotSubChannel('int8_subchannel_g128_4096', 4096, 4096, 4096, 128, 'int8'),
+    'fp8_subchannel_g128_4096': lambda: QdotSubChannel('fp8_subchannel_g128_4096', 4096, 4096, 4096, 128, 'float8_e4m3fn'),
     'mfma_ceiling_int8_zeros': lambda: MfmaCeiling('mfma_ceiling_int8_zeros', 'int8', 'zeros'),
     'mfma_ceiling_int8_gauss30': lambda: MfmaCeiling('mfma_ceiling_int8_gauss30', 'int8', 'gauss30'),
     'mfma_ceiling_int8_operands': lambda: MfmaCeiling('mfma_ceiling_int8_operands', 'int8', 'operands'),
@@ -1048,10 +1104,16 @@ def summarize(wl: Workload, step_s: float, kern_s: float, ceilings: dict = None)
   # `frac` stays priced against the nominal peak; `frac_of_ceiling` is the same rate against what the matrix cores
   # sustained in this very run on register operands of this workload's kind (see MfmaCeiling), no memory traffic.
   if rb == 'mfma' and peak == PEAK_MFMA_TOPS and not isinstance(wl, MfmaCeiling):
-    c = (ceilings or {}).get(wl.dtype)
+    c = (ceilings or {}).get(_ceiling_dtype(wl))
     roof['ceiling'] = c
     roof['frac_of_ceiling'] = round(achieved / c, 4) if c else None
   return {'value': round(value, 2), 'unit': wl.unit, 'ms_per_step': round(step_s * 1e3, 5), 'roofline': roof}
+
+
+def _ceiling_dtype(wl) -> str:
+  """The operand type whose matrix-core ceiling prices this workload: int4 weights are widened to int8 in registers
+  and multiplied by the int8 instruction."""
+  return 'int8' if wl.dtype.startswith('int8') else wl.dtype
 
 
 def measure_ceilings(dtypes, spin_up) -> tuple:
@@ -1126,7 +1188,7 @@ def main():
   extra_on = not args.no_extra and args.workload == DEFAULT
   ceilings, ceiling_lines = {}, {}
   if not args.no_ceiling and not isinstance(wl, MfmaCeiling):
-    want = sorted(CEILINGS) if extra_on else [d for d in CEILINGS if d == wl.dtype and getattr(wl, 'roofline_bound', wl.bound) == 'mfma']
+    want = sorted(CEILINGS) if extra_on else [d for d in CEILINGS if d == _ceiling_dtype(wl) and getattr(wl, 'roofline_bound', wl.bound) == 'mfma']
     if want:
       ceilings, ceiling_lines = measure_ceilings(want, args.spin_up)
   step_s, kmean, timing = run(wl, args.steps, args.warmup, args.spin_up, args.repeats)

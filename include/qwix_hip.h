@@ -270,6 +270,10 @@ QWIX_API int qwix_hip_ksum_i8(const void* q, int64_t ld, int64_t rows, int64_t K
  *   exact    1: every intermediate is rounded exactly as the reference does (bit-exact with
  *               the CPU oracle, slower); 0: f32 throughout (within rtol 1e-2)
  *   acc_out  optional (K/group, M, N) int32 raw partials for parity tests, else NULL
+ * b_qtype QWIX_E4M3: a and b are both OCP e4m3 bytes; every group's dot is summed in f32 on the
+ * matrix cores, delivered in out_dtype (float operands accumulate in the result type,
+ * qarray.py:781-821), then scaled lhs first with one rounding per step and summed over the groups
+ * in f32, always with the reference's roundings (`exact` is ignored; acc_out must be NULL).
  */
 QWIX_API int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b, int64_t ldb_bytes,
                            int b_qtype, int64_t M, int64_t N, int64_t K, int64_t group,

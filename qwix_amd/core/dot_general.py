@@ -470,8 +470,9 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   if lq == numerics.INT4:
     lq = numerics.INT8  # lhs_values widens int4 rows
   tiled = [(l, r, lt.get(l) or rt.get(r)) for l, r in zip(c.lca, c.rca) if lt.get(l) or rt.get(r)]
-  if tiled and (len(c.lca) > 1 or lq != numerics.INT8 or rq not in (numerics.INT8, numerics.INT4)
-                or any(n % 128 for _, _, n in tiled)):
+  int_pair = lq == numerics.INT8 and rq in (numerics.INT8, numerics.INT4)
+  f8_pair = lq == numerics.E4M3 and rq == numerics.E4M3
+  if tiled and (len(c.lca) > 1 or not (int_pair or f8_pair) or any(n % 128 for _, _, n in tiled)):
     # what the sub-channel MFMA kernel does not take runs tile by tile on the untiled kernels
     if return_accumulators:
       raise NotImplementedError('raw accumulators are returned for one tiled contracting axis of int8 x int8/int4 only')
@@ -531,8 +532,10 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
     out = out.reshape(c.out_shape)
     return (out, acc.reshape(c.out_shape)) if return_accumulators else out
   # sub-channel / int4 weights
-  if lq != numerics.INT8 or rq not in (numerics.INT8, numerics.INT4):
-    raise NotImplementedError(f'sub-channel MFMA kernel needs int8 x int8/int4 operands, got {lq} x {rq}')
+  if not (int_pair or f8_pair):
+    raise NotImplementedError(f'sub-channel MFMA kernel needs int8 x int8/int4 or e4m3 x e4m3 operands, got {lq} x {rq}')
+  if f8_pair and return_accumulators:
+    raise NotImplementedError('raw accumulators are int32 partials; e4m3 operands have none')
   ngroups = max(ga, gb)
   if c.K % ngroups or (c.K // ngroups) % 128:
     raise NotImplementedError(f'K-group size {c.K / ngroups} must be a multiple of 128')
@@ -542,7 +545,7 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   if gb != ngroups:  # rhs per-channel, lhs tiled: repeat the rhs scale per group
     sb = sb.expand(ngroups, c.N).contiguous()
   acc = torch.empty(ngroups, c.M, c.N, dtype=torch.int32, device=dev) if return_accumulators else None
-  bq = _lib.INT4 if b_is4 else _lib.INT8
+  bq = _lib.E4M3 if f8_pair else _lib.INT4 if b_is4 else _lib.INT8
   if lzp is not None or rzp is not None:
     # dot_general.py:196-203, 228-253: the zero point is split with the tiles and every tile's partial is
     # corrected by zero_point x (K-sum of the other operand over that tile) before it is scaled.

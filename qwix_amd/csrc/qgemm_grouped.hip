@@ -22,7 +22,9 @@ namespace qwix {
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 128, BN = 128, BK = 128, TM = 2, TN = 2, kPad = 16;
 
@@ -32,7 +34,8 @@ struct GroupedArgs {
   int M, N, K, group;
   const void* sa; int sa_dtype; int ga;
   const void* sb; int sb_dtype;
-  int t_dtype;      // dtype of the scaled partials (promotion of the scale dtypes)
+  int t_dtype;      // dtype of the scaled partials (promotion of the scale dtypes, and of acc_dtype for e4m3)
+  int acc_dtype;    // e4m3 operands: the dtype each group's f32 dot is rounded to before it is scaled
   uint8_t* out; int out_dtype; int64_t ldo;
   int32_t* acc_out;
   // Zero-point correction of an asymmetric operand, per group: acc_g[m,n] -= zu[m,g] * zv[g,n].  One array
@@ -50,6 +53,8 @@ __device__ __forceinline__ float ld_scale(const void* p, int dtype, int64_t i) {
 template <int BQT, bool EXACT>
 __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
   constexpr bool W4 = (BQT == QWIX_INT4);
+  constexpr bool F8 = (BQT == QWIX_E4M3);  // both operands e4m3, f32 partial per group (v_mfma_f32_32x32x64_f8f6f4)
+  using AccV = typename std::conditional<F8, v16f, v16i>::type;
   constexpr int A_STRIDE = BK + kPad;
   constexpr int B_ROW = W4 ? BK / 2 : BK;
   constexpr int B_STRIDE = B_ROW + kPad;
@@ -65,7 +70,7 @@ __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
   if ((gridDim.x & 7) == 0) pid = (pid & 7) * (gridDim.x >> 3) + (pid >> 3);  // one XCD, one run of tiles
   const int m0 = (pid / tiles_n) * BM, n0 = (pid % tiles_n) * BN;
 
-  v16i acc[TM][TN];
+  AccV acc[TM][TN];
   float accf[TM][TN][16];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -111,6 +116,31 @@ __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
   auto compute = [&](int s) {
     const uint8_t* pa = smem + s * STAGE + (wm * (BM / 2) + (lane & 31)) * A_STRIDE;
     const uint8_t* pb = smem + s * STAGE + BM * A_STRIDE + (wn * (BN / 2) + (lane & 31)) * B_STRIDE;
+    if constexpr (F8) {
+      // a lane holds 32 consecutive bytes of its row per k-step of 64
+#pragma unroll
+      for (int ks = 0; ks < BK / 64; ++ks) {
+        v8i fa[TM], fb[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const uint8_t* q = pa + i * 32 * A_STRIDE + ks * 64 + (lane >> 5) * 32;
+          const v4i lo = *reinterpret_cast<const v4i*>(q), hi = *reinterpret_cast<const v4i*>(q + 16);
+          fa[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const uint8_t* q = pb + j * 32 * B_STRIDE + ks * 64 + (lane >> 5) * 32;
+          const v4i lo = *reinterpret_cast<const v4i*>(q), hi = *reinterpret_cast<const v4i*>(q + 16);
+          fb[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+      }
+      return;
+    } else {
 #pragma unroll
     for (int ks = 0; ks < BK / 32; ++ks) {
       v4i fa[TM], fb[TN];
@@ -144,6 +174,7 @@ __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
     }
+    }
   };
 
   // acc[i][j][r]: m = m0 + wm*64 + i*32 + 8*(r/4) + 4*(lane/32) + r%4,  n = n0 + wn*(BN/2) + j*32 + lane%32.
@@ -165,11 +196,29 @@ __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
       for (int r = 0; r < 16; ++r) {
         const int m = row_of(i, r);
         float sav = 1.f;
-        if (p.sa != nullptr && (EXACT || p.ga > 1) && m < p.M)
+        if (p.sa != nullptr && (EXACT || F8 || p.ga > 1) && m < p.M)
           sav = ld_scale(p.sa, p.sa_dtype, static_cast<int64_t>(m) * p.ga + (p.ga > 1 ? g : 0));
         const int zuv = (p.zu != nullptr && m < p.M) ? p.zu[m * p.zu_sm + g * p.zu_sg] : 0;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
+          if constexpr (F8) {
+            // dot_general.py:214-260 for float operands: the group's dot is delivered in the accumulator dtype, then
+            // scaled lhs first, every step in the promotion of the types met so far, one rounding per step
+            float v = acc[i][j][r];
+            bool bf = (p.acc_dtype == QWIX_BF16);
+            if (bf) v = round_bf16(v);
+            if (p.sa != nullptr) {
+              bf = bf && p.sa_dtype == QWIX_BF16;
+              v *= sav;
+              if (bf) v = round_bf16(v);
+            }
+            bf = bf && p.sb_dtype == QWIX_BF16;
+            v *= sbv[j];
+            if (bf) v = round_bf16(v);
+            accf[i][j][r] += v;
+            acc[i][j][r] = 0;
+            continue;
+          } else {
           // int4 weights were widened to 16 x value: the partial is an exact multiple of 16
           const int raw = (W4 ? (acc[i][j][r] >> 4) : acc[i][j][r]) - zuv * zvv[j];
           if (p.acc_out != nullptr && m < p.M && col_of(j) < p.N)
@@ -187,6 +236,7 @@ __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
             accf[i][j][r] = __builtin_fmaf(v, (p.ga > 1 ? sav : 1.f) * sbv[j], accf[i][j][r]);
           }
           acc[i][j][r] = 0;
+          }
         }
       }
   };
@@ -218,7 +268,7 @@ __global__ void __launch_bounds__(256) qgemm_grouped_kernel(GroupedArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         float v = accf[i][j][r];
-        if (!EXACT && p.sa != nullptr && p.ga == 1) {
+        if (!EXACT && !F8 && p.sa != nullptr && p.ga == 1) {
           const int m = row_of(i, r);
           v *= (m < p.M) ? ld_scale(p.sa, p.sa_dtype, m) : 0.f;
         }
@@ -849,8 +899,10 @@ static int grouped_impl(const void* a, int64_t lda, const void* b, int64_t ldb_b
   if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX)
     return fail(QWIX_ERR_INVALID_ARGUMENT, "bad GEMM shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
                 (long long)K);
-  if (b_qtype != QWIX_INT8 && b_qtype != QWIX_INT4)
-    return fail(QWIX_ERR_UNSUPPORTED, "grouped GEMM takes int8 or int4 weights (got qtype %d)", b_qtype);
+  if (b_qtype != QWIX_INT8 && b_qtype != QWIX_INT4 && b_qtype != QWIX_E4M3)
+    return fail(QWIX_ERR_UNSUPPORTED, "grouped GEMM takes int8, int4 or e4m3 weights (got qtype %d)", b_qtype);
+  if (b_qtype == QWIX_E4M3 && (zu || acc_out))
+    return fail(QWIX_ERR_UNSUPPORTED, "e4m3 operands have neither zero points nor int32 partials");
   if (group <= 0 || group % 128 || K % group)
     return fail(QWIX_ERR_UNSUPPORTED, "group %lld must be a multiple of 128 that divides K=%lld", (long long)group,
                 (long long)K);
@@ -866,18 +918,25 @@ static int grouped_impl(const void* a, int64_t lda, const void* b, int64_t ldb_b
     return fail(QWIX_ERR_INVALID_ARGUMENT, "zu and zv come together (zero points and the other operand's K-sums)");
   if (zu && (zu_row_stride < 0 || zu_group_stride < 0 || zv_col_stride < 0 || zv_group_stride < 0))
     return fail(QWIX_ERR_INVALID_ARGUMENT, "negative zero-point stride");
-  GroupedArgs p;
+  GroupedArgs p{};
   p.A = static_cast<const uint8_t*>(a); p.lda = lda;
   p.B = static_cast<const uint8_t*>(b); p.ldb = ldb_bytes;
   p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(K); p.group = static_cast<int>(group);
   p.sa = sa; p.sa_dtype = sa_dtype; p.ga = static_cast<int>(ga);
   p.sb = sb; p.sb_dtype = sb_dtype;
   p.t_dtype = (sb_dtype == QWIX_F32 || (sa && sa_dtype == QWIX_F32)) ? QWIX_F32 : QWIX_BF16;
+  p.acc_dtype = QWIX_F32;
+  if (b_qtype == QWIX_E4M3) {
+    // float operands accumulate in the result type (qarray.py:781-821): the caller's out dtype
+    p.acc_dtype = out_dtype;
+    if (out_dtype == QWIX_F32) p.t_dtype = QWIX_F32;
+  }
   p.out = static_cast<uint8_t*>(out); p.out_dtype = out_dtype; p.ldo = ldo;
   p.acc_out = acc_out;
   p.zu = zu; p.zu_sm = zu_row_stride; p.zu_sg = zu_group_stride;
   p.zv = zv; p.zv_sn = zv_col_stride; p.zv_sg = zv_group_stride;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (b_qtype == QWIX_E4M3) return launch_grouped<QWIX_E4M3, true>(p, st);
   const bool row_strides_fit = 128 * lda < (int64_t{1} << 31) && 256 * ldb_bytes < (int64_t{1} << 31);
   if (!exact && row_strides_fit) {
     // per-group activation scales ride along in LDS: the tile's scales must fit behind the slab stages

@@ -405,3 +405,46 @@ def test_int4_weights_tiled_under_two_contracting_axes():
   torch.cuda.synchronize()
   want = O.dot_general(oxq, owq, TILED_DN)
   assert np.array_equal(util.f32np(out), want.v)
+
+
+@pytest.mark.parametrize('sdt', [O.BF16, O.F32])
+@pytest.mark.parametrize('ltile,rtile', [(128, 128), (None, 128), (256, None), (128, 256)])
+def test_e4m3_operands_with_sub_channel_scales(ltile, rtile, sdt):
+  """e4m3 x e4m3 with scales tiled along the contracting axis: one launch of the sub-channel kernel (f32 partial per
+  group on the fp8 matrix-core instruction, the oracle's roundings per group, f32 sum over groups).  The order in
+  which the hardware adds inside a group is not the oracle's: the fp8 tolerance."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  dn = (((1,), (0,)), ((), ()))
+  M, K, N = 200, 1024, 136
+  if ltile and rtile and ltile != rtile:
+    with pytest.raises(ValueError):
+      xq, wq, _, _ = _pair((M, K), (K, N), dict(qtype=O.E4M3, channelwise_axes=[0], tiled_axes={1: ltile}),
+                           dict(qtype=O.E4M3, channelwise_axes=[1], tiled_axes={0: rtile}), O.BF16, seed=5)
+      dg.dot_general(xq, wq, dn)
+    return
+  print('case e4m3 sub-channel', ltile, rtile, sdt, flush=True)
+  x_np, x_t = util.make((M, K), O.BF16, seed=41)
+  w_np, w_t = util.make((K, N), O.BF16, seed=42, scale=0.05)
+  lkw = dict(qtype=O.E4M3, channelwise_axes=[0], tiled_axes={1: ltile} if ltile else {})
+  rkw = dict(qtype=O.E4M3, channelwise_axes=[1], tiled_axes={0: rtile} if rtile else {})
+  tsdt = util.TORCH_DT[sdt]
+  xq = qarray.quantize_api(x_t, scale_dtype=tsdt, **lkw)
+  wq = qarray.quantize_api(w_t, scale_dtype=tsdt, **rkw)
+  oxq = O.quantize_api(O.FArr(x_np, O.BF16), scale_dtype=sdt, **lkw)
+  owq = O.quantize_api(O.FArr(w_np, O.BF16), scale_dtype=sdt, **rkw)
+  util.assert_qarray_equal(xq, oxq, 'lhs')
+  util.assert_qarray_equal(wq, owq, 'rhs')
+  for pet, opet in ((None, None), (torch.float32, O.F32), (torch.bfloat16, O.BF16)):
+    out = dg.dot_general(xq, wq, dn, preferred_element_type=pet)
+    torch.cuda.synchronize()
+    want = O.dot_general(oxq, owq, dn, opet)
+    assert out.dtype == util.TORCH_DT[want.dtype] and tuple(out.shape) == (M, N)
+    got = util.f32np(out)
+    assert np.allclose(got, want.v, rtol=1e-2, atol=1e-2 * np.abs(want.v).mean()), np.abs(got - want.v).max()
+  # and the same numbers as the tile-by-tile route on the untiled kernels, up to the order of the f32 additions
+  tiled = [(1, 0, ltile or rtile)]
+  ref = dg._tile_by_tile(xq, wq, dn, tiled, torch.float32, False)
+  out = dg.dot_general(xq, wq, dn, preferred_element_type=torch.float32)
+  torch.cuda.synchronize()
+  assert torch.allclose(out, ref, rtol=1e-4, atol=1e-4 * ref.abs().mean().item())
