@@ -559,7 +559,7 @@ class QdotSubChannel(Workload):
     self.dtype = 'int8' if qtype == 'int8' else 'f8e4m3'
     self.metric = self.dtype + ' sub-channel qdot TOPS (group %d on both operands, activation quantize included)' % group
     self.unit = 'TOPS'
-    self.kernel_name = 'qgemm_grouped_dma_kernel' if qtype == 'int8' else 'qgemm_grouped_kernel'
+    self.kernel_name = 'qgemm_grouped_dma_kernel'
 
   def setup(self, dev):
     import torch

@@ -273,7 +273,8 @@ QWIX_API int qwix_hip_ksum_i8(const void* q, int64_t ld, int64_t rows, int64_t K
  * b_qtype QWIX_E4M3: a and b are both OCP e4m3 bytes; every group's dot is summed in f32 on the
  * matrix cores, delivered in out_dtype (float operands accumulate in the result type,
  * qarray.py:781-821), then scaled lhs first with one rounding per step and summed over the groups
- * in f32, always with the reference's roundings (`exact` is ignored; acc_out must be NULL).
+ * in f32 (exact = 1: with the reference's roundings; 0: f32 throughout, one rounding of the sum;
+ * acc_out must be NULL).
  */
 QWIX_API int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b, int64_t ldb_bytes,
                            int b_qtype, int64_t M, int64_t N, int64_t K, int64_t group,

@@ -367,6 +367,12 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
   constexpr int BM = Fast::kBM, BN = Fast::kBN, BK = Fast::kBK, NW = Fast::kNW, TM = Fast::kTM;
   constexpr int WR = 1;  // every wavefront owns all rows of its 32 columns
   constexpr bool W4 = (BQT == QWIX_INT4);
+  // e4m3 x e4m3: bytes travel like int8; two 16-byte fragments of consecutive k-steps make one operand of
+  // v_mfma_f32_32x32x64_f8f6f4 (both operands take the same 32 of the 64 k per lane half, so the dot is complete),
+  // the group's partial is f32 already.  Never MAGIC, never AUX.
+  constexpr bool F8 = (BQT == QWIX_E4M3);
+  static_assert(!F8 || (!MAGIC && !AUX), "e4m3 operands have neither int32 partials nor zero points");
+  using AccV = typename std::conditional<F8, v16f, v16i>::type;
   constexpr int B_ROWB = W4 ? 64 : 128;          // bytes of one B row in a slab
   constexpr int A_BYTES = BM * BK, B_BYTES = BN * B_ROWB, STAGE = A_BYTES + B_BYTES;
   constexpr int A_LOADS = A_BYTES / 1024 / NW;   // KiB pieces per wavefront and slab
@@ -451,6 +457,29 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
   const int b_row = (wc * 32 + frow) * B_ROWB, b_sw = W4 ? ((frow >> 2) & 3) : swz128(wc * 32 + frow);
   v4i fa[2][TM];
   v4i fbr[2];  // int4: one chunk = two k-steps; int8: one chunk = one k-step
+  // e4m3: an operand of the 64-wide MFMA is two such 16-byte pieces (k-steps 2 kp and 2 kp + 1 of pair kp), read
+  // straight into the halves of an 8-register operand; buffer kp holds pair kp
+  v8i fa8[2][TM];
+  v8i fb8[2];
+  auto read_pair_a = [&](int s, int kp, int i) __attribute__((always_inline)) {
+    const int c0 = 4 * kp + hx, c1 = c0 + 2;
+    const uint8_t* ab = smem + s * STAGE + a_row + i * 32 * BK;
+    const v4i lo = *reinterpret_cast<const v4i*>(ab + ((c0 ^ a_sw) << 4));
+    const v4i hi = *reinterpret_cast<const v4i*>(ab + ((c1 ^ a_sw) << 4));
+    fa8[kp][i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+  auto read_pair_b = [&](int s, int kp) __attribute__((always_inline)) {
+    const int c0 = 4 * kp + hx, c1 = c0 + 2;
+    const uint8_t* bb = smem + s * STAGE + A_BYTES + b_row;
+    const v4i lo = *reinterpret_cast<const v4i*>(bb + ((c0 ^ b_sw) << 4));
+    const v4i hi = *reinterpret_cast<const v4i*>(bb + ((c1 ^ b_sw) << 4));
+    fb8[kp] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+  auto read_pair = [&](int s, int kp) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) read_pair_a(s, kp, i);
+    read_pair_b(s, kp);
+  };
   auto read_a = [&](int s, int ks, int buf) __attribute__((always_inline)) {
     const int chunk = W4 ? (4 * (ks >> 1) + 2 * hx + (ks & 1)) : (2 * ks + hx);
     const uint8_t* base = smem + s * STAGE + a_row + ((chunk ^ a_sw) << 4);
@@ -478,7 +507,7 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
     }
   };
 
-  v16i acc[TM];
+  AccV acc[TM];
   float accf[TM][16];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -527,8 +556,12 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
   issue_loads(0, 0);
   if (ST == 3 && KT > 1) issue_loads(1, 1);
   __syncthreads();
-  read_a(0, 0, 0);
-  read_b(0, 0, 0);
+  if constexpr (F8) {
+    read_pair(0, 0);
+  } else {
+    read_a(0, 0, 0);
+    read_b(0, 0, 0);
+  }
 
   int cs = 0;  // stage that holds the current slab
   auto next_stage = [&](int s, int by) __attribute__((always_inline)) { return s + by >= ST ? s + by - ST : s + by; };
@@ -546,8 +579,12 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
     }
     cs = next_stage(cs, 1);
     if (kt + 1 < KT) {
-      read_a(cs, 0, 0);
-      read_b(cs, 0, 0);
+      if constexpr (F8) {
+        read_pair(cs, 0);
+      } else {
+        read_a(cs, 0, 0);
+        read_b(cs, 0, 0);
+      }
     }
   };
 
@@ -591,6 +628,34 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
     constexpr bool LAST = decltype(last_tag)::value && !AUX;
     const int cur = cs;
     if (kt + ST - 1 < KT) issue_loads(next_stage(cs, ST - 1), kt + ST - 1);
+    if constexpr (F8) {
+      // pair 0 was read at the end of the slab before; pair 1 is read under the MFMAs of pair 0; when the slab closes
+      // a group, the fold of tile i - 1 sits behind the last MFMA of tile i, as in the integer kernel
+      // (a tile's half of pair 1 is requested behind that tile's MFMA of pair 0: its registers can be the ones that MFMA
+      // has just read, and three MFMAs run before it is needed)
+      read_pair_b(cur, 1);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        if constexpr (FIRST) {
+          const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+          acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa8[0][i], fb8[0], zero, 0, 0, 0, 0, 0, 0);
+        } else {
+          acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa8[0][i], fb8[0], acc[i], 0, 0, 0, 0, 0, 0);
+        }
+        read_pair_a(cur, 1, i);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa8[1][i], fb8[1], acc[i], 0, 0, 0, 0, 0, 0);
+        if constexpr (LAST) {
+          if (i > 0) fold_tile(i - 1, g, sbg, recentre);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      if constexpr (LAST) fold_tile(TM - 1, g, sbg, recentre);
+      return;
+    } else {
     auto read_next = [&](int ks) __attribute__((always_inline)) {  // fragments of k-step ks + 1
       if (ks + 1 < NK) {
         read_a(cur, ks + 1, (ks + 1) & 1);
@@ -632,6 +697,7 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
         __builtin_amdgcn_sched_barrier(0);
       }
       fold_tile(TM - 1, g, sbg, recentre);
+    }
     }
   };
 
@@ -816,6 +882,23 @@ int dispatch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
              : launch_grouped_dma<BQT, false, SAG, false, false, 2, false>(p, st);
 }
 
+// The instantiations for e4m3 x e4m3 (no zero points, no int32 partials).
+template <bool SAG>
+int dispatch_grouped_f8(const GroupedArgs& p, hipStream_t st) {
+  constexpr int Q = QWIX_E4M3;
+  const bool sbf = p.sb_dtype == QWIX_BF16;
+  if (grouped_dma_lds<Q>(SAG, p.K, p.group, 2) > kLdsMax) return -1;
+  if (p.group == Fast::kBK) {
+    if (grouped_dma_lds<Q>(SAG, p.K, p.group, 3) <= kLdsMax)
+      return sbf ? launch_grouped_dma<Q, true, SAG, false, false, 3, true>(p, st)
+                 : launch_grouped_dma<Q, false, SAG, false, false, 3, true>(p, st);
+    return sbf ? launch_grouped_dma<Q, true, SAG, false, false, 2, true>(p, st)
+               : launch_grouped_dma<Q, false, SAG, false, false, 2, true>(p, st);
+  }
+  return sbf ? launch_grouped_dma<Q, true, SAG, false, false, 2, false>(p, st)
+             : launch_grouped_dma<Q, false, SAG, false, false, 2, false>(p, st);
+}
+
 // Per-group K-sums of quantized rows: out[row, g] = sum over the g-th group of `group` values of row `row`
 // (int8, or packed int4).  One 16-byte chunk per thread; the chunks of a group that sit in `seg` adjacent
 // lanes (a power of two that divides the chunks per group) are added by shuffles, the rest by integer
@@ -936,8 +1019,14 @@ static int grouped_impl(const void* a, int64_t lda, const void* b, int64_t ldb_b
   p.zu = zu; p.zu_sm = zu_row_stride; p.zu_sg = zu_group_stride;
   p.zv = zv; p.zv_sn = zv_col_stride; p.zv_sg = zv_group_stride;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (b_qtype == QWIX_E4M3) return launch_grouped<QWIX_E4M3, true>(p, st);
   const bool row_strides_fit = 128 * lda < (int64_t{1} << 31) && 256 * ldb_bytes < (int64_t{1} << 31);
+  if (b_qtype == QWIX_E4M3) {
+    if (!exact && row_strides_fit) {
+      const int rc = (sa != nullptr && ga > 1) ? dispatch_grouped_f8<true>(p, st) : dispatch_grouped_f8<false>(p, st);
+      if (rc >= 0) return rc;
+    }
+    return launch_grouped<QWIX_E4M3, true>(p, st);
+  }
   if (!exact && row_strides_fit) {
     // per-group activation scales ride along in LDS: the tile's scales must fit behind the slab stages
     const bool sag = sa != nullptr && ga > 1;

@@ -441,7 +441,16 @@ def test_e4m3_operands_with_sub_channel_scales(ltile, rtile, sdt):
     want = O.dot_general(oxq, owq, dn, opet)
     assert out.dtype == util.TORCH_DT[want.dtype] and tuple(out.shape) == (M, N)
     got = util.f32np(out)
-    assert np.allclose(got, want.v, rtol=1e-2, atol=1e-2 * np.abs(want.v).mean()), np.abs(got - want.v).max()
+    mag = np.abs(want.v).mean()
+    # The default kernel keeps every scaled partial in f32 where the reference rounds it to the scale dtype three
+    # times per group (more accurate than the reference, inside its rounding envelope): the mean error is held to
+    # about a bf16 step (2^-8), single elements to a few steps.
+    assert np.abs(got - want.v).mean() < 5e-3 * mag, np.abs(got - want.v).mean() / mag
+    assert np.allclose(got, want.v, rtol=2e-2, atol=2e-2 * mag), np.abs(got - want.v).max()
+    # with the reference's roundings per group: only the order of the f32 additions inside a group is left
+    ex = dg._fast_dot_general(xq, wq, dn, preferred_element_type=pet, exact=True)
+    torch.cuda.synchronize()
+    assert np.allclose(util.f32np(ex), want.v, rtol=1e-2, atol=1e-2 * mag), np.abs(util.f32np(ex) - want.v).max()
   # and the same numbers as the tile-by-tile route on the untiled kernels, up to the order of the f32 additions
   tiled = [(1, 0, ltile or rtile)]
   ref = dg._tile_by_tile(xq, wq, dn, tiled, torch.float32, False)
