@@ -65,7 +65,8 @@ def _lib():
 
 
 class QdotW8A8(Workload):
-  """activation quantize (per token) + MFMA GEMM with fused scale epilogue; qtype int8 or e4m3."""
+  """activation quantize (per token) + MFMA GEMM with fused scale epilogue, one library call per step
+  (qwix_hip_qgemm_dynamic_act: the quantize kernel and the GEMM back to back on a caller workspace); qtype int8 or e4m3."""
 
   bound = 'mfma'
 
@@ -96,12 +97,18 @@ class QdotW8A8(Workload):
     self.qt = L.INT8 if self.qtype == 'int8' else L.E4M3
     self.stream = torch.cuda.current_stream().cuda_stream
     self.L = L
+    # the step is one library call (quantize + GEMM on a caller workspace); the GEMM alone, for the roofline figure,
+    # runs on activations quantized once here
+    nws = int(L.load().qwix_hip_qgemm_dynamic_act_workspace_bytes(self.M, self.N, self.K, L.BF16))
+    self.ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dev)
+    L.call('qwix_hip_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, 1, self.K, self.qt, L.ABSMAX, 0.0,
+           L.LAYOUT_NATURAL, self.xq.data_ptr(), self.sa.data_ptr(), None, None, 0, self.stream)
 
   def step(self, i=0):
     L = self.L
-    L.call('qwix_hip_quantize', self.x.data_ptr(), L.BF16, self.M, self.K, 1, self.K, self.qt, L.ABSMAX, 0.0,
-           L.LAYOUT_NATURAL, self.xq.data_ptr(), self.sa.data_ptr(), None, None, 0, self.stream)
-    self.kernel(i)
+    L.call('qwix_hip_qgemm_dynamic_act', self.x.data_ptr(), L.BF16, self.K, self.b.data_ptr(), self.K, self.qt, self.M,
+           self.N, self.K, self.sb.data_ptr(), L.BF16, L.BF16, self.out.data_ptr(), L.BF16, self.N, self.ws.data_ptr(),
+           self.ws.numel(), self.stream)
 
   def kernel(self, i=0):
     L = self.L
