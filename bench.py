@@ -249,7 +249,7 @@ class FwhtQuantize(Workload):
     self.dtype = 'bf16->int8'
     self.metric = 'Hadamard rotate + quantize GB/s (per-token absmax, bf16 -> int8)'
     self.unit = 'GB/s'
-    self.kernel_name = 'fwht_reg_kernel'
+    self.kernel_name = 'fwht_mfma_kernel' if K == 8192 else 'fwht_reg_kernel'
 
   def setup(self, dev):
     import torch

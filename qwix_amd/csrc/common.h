@@ -212,10 +212,12 @@ __device__ __forceinline__ float apply_factor(float v, float factor) {
   return factor > 0.f ? rnd<D>(v * rnd<D>(factor)) : v;
 }
 
-// x / s rounded to D.  f32: IEEE division.  bf16: both operands have 8-bit significands, so
-// the exact quotient is never closer than 2^-18 (relative) to a bf16 rounding boundary unless
-// it lies exactly on one, in which case it is representable in f32 and the residual step below
-// reproduces it exactly.  Hence one reciprocal + one Newton step gives RNE_bf16(RNE_f32(x/s)).
+// x / s rounded to D.  f32: IEEE division.  bf16: both operands have 8-bit significands X and S (128 .. 255).  The
+// quotient cannot lie on a bf16 rounding boundary (a boundary has an odd 9-bit significand Q >= 257, and
+// X * 2^m = Q * S would make Q divide X), and its distance from the nearest one is at least 1 / (512 S) > 2^-17
+// relative.  x * rcp(s) is within 2^-22 of the quotient (v_rcp_f32: 1 ulp, the product: half an ulp), so it rounds
+// to the same bf16 as RNE_bf16(RNE_f32(x / s)) does: one multiply per element.  (Quotients in the bf16 subnormal range
+// round to zero in every target type.)
 // kSafe=false is for quotients known to be bounded (dynamic range: |x| <= absmax).
 // kSignedZero keeps the sign of a zero quotient (matters for e4m3's -0 only).
 template <typename D, bool kSafe = true, bool kSignedZero = true>
@@ -227,11 +229,9 @@ struct Divider {
   // The quotient before its rounding to D (f32: the quotient itself).
   __device__ __forceinline__ float raw(float x) const {
     if constexpr (D::kTag == QWIX_BF16) {
-      float q0 = x * r;
-      float e = __builtin_fmaf(-q0, s, x);
-      float q1 = __builtin_fmaf(e, r, q0);
+      float q1 = x * r;
       if constexpr (kSafe) {
-        const bool odd = !(__builtin_fabsf(q0) < 0x1p100f);
+        const bool odd = !(__builtin_fabsf(q1) < 0x1p100f);
         if (__builtin_amdgcn_ballot_w64(odd) != 0) {
           if (odd) q1 = x / s;
         }
@@ -257,19 +257,17 @@ struct Divider {
   }
   __device__ __forceinline__ float operator()(float x) const {
     if constexpr (D::kTag == QWIX_BF16) {
-      float q0 = x * r;
-      float e = __builtin_fmaf(-q0, s, x);
-      float q1 = __builtin_fmaf(e, r, q0);
+      float q1 = x * r;
       // Overflowing or non-finite quotients (static scales only): take the IEEE path.  The test is made
       // wave-uniform first, so that the division sequence is branched over instead of being computed
       // for every element and selected away.
       if constexpr (kSafe) {
-        const bool odd = !(__builtin_fabsf(q0) < 0x1p100f);
+        const bool odd = !(__builtin_fabsf(q1) < 0x1p100f);
         if (__builtin_amdgcn_ballot_w64(odd) != 0) {
           if (odd) q1 = x / s;
         }
       }
-      // The residual step turns -0 into +0; the quotient always carries the sign of x (s > 0).
+      // The quotient always carries the sign of x (s > 0).
       if constexpr (kSignedZero) return __builtin_copysignf(round_bf16(q1), x);
       return round_bf16(q1);
     } else {

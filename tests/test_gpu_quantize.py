@@ -312,6 +312,30 @@ def test_long_contiguous_groups_calibrate_and_static(dtype):
     util.assert_qarray_equal(qa, O.quantize(O.FArr(x_np, dtype), ohow), f'static per-tensor {cal}')
 
 
+@pytest.mark.parametrize('qtype', ['int8', 'int4', 'float8_e4m3fn'])
+def test_bf16_division_for_every_pair_of_significands(qtype):
+  """The kernels divide bf16 by bf16 as x * rcp(s).  Every scale significand (128 of them, two exponents) against
+  every finite bf16 value: each (significand of x, significand of s) pair occurs at every exponent difference, in
+  particular where the quotient lies in [64, 128) and a bf16 step is 0.5, so that a quotient rounded to the wrong
+  bf16 neighbour changes the int8 that comes out.  Given scales (the static-range kernel) and the oracle's true
+  division."""
+  from qwix_amd.core import qarray
+  bits = torch.arange(0, 1 << 16, dtype=torch.int32).to(torch.uint16)
+  xb = bits.view(torch.bfloat16)
+  xb = xb[torch.isfinite(xb)]
+  n = (xb.numel() // 64) * 64
+  row = xb[:n].to(torch.float32).numpy()
+  for e in (-2, 9):
+    sig = (np.arange(128, 256, dtype=np.float32) / 128.0) * np.float32(2.0 ** e)
+    x_np = np.broadcast_to(row, (128, n)).copy()
+    scale_np = sig.reshape(128, 1)
+    assert np.array_equal(O.round_to_bf16(scale_np), scale_np)
+    x_t = util.to_gpu(x_np, O.BF16)
+    qa = qarray.quantize_with_scale_zero_point(x_t, qtype, util.to_gpu(scale_np, O.BF16), None)
+    want = O.quantize_with_scale_zero_point(O.FArr(x_np, O.BF16), qtype, O.FArr(scale_np, O.BF16), None)
+    util.assert_qarray_equal(qa, want, f'all significand pairs, scale exponent {e}')
+
+
 @pytest.mark.parametrize('qtype', ['int8', 'float8_e4m3fn'])
 def test_static_scale_with_overflowing_quotients(qtype):
   """A given scale need not come from the data: quotients that overflow or are infinite must still follow
