@@ -25,6 +25,10 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+// LDS reads inside the main loops go through these, never through HIP's struct vectors (float4, int4): behind a
+// struct-typed LDS access the compiler waits for every direct-to-LDS load in flight (vmcnt 0), the slabs requested
+// ahead included.
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 128, BN = 128, BK = 128, TM = 2, TN = 2, kPad = 16;
 
@@ -445,10 +449,21 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
     const uint8_t* ga = a_base + kt * BK;
     const uint8_t* gb = b_base + kt * B_ROWB;
     uint8_t* ls = smem + s * STAGE;
+    // The 32-bit lane offsets are made opaque here, inside the slab: widened to 64 bits once, ahead of the loop, each
+    // would occupy two registers for the whole kernel and every load would need a 64-bit vector add; seen next to the
+    // load, base + offset is a scalar base register plus a 32-bit vector offset.
 #pragma unroll
-    for (int j = 0; j < A_LOADS; ++j) QWIX_GLDS16(ga + a_off[j], ls + (j * NW + wave) * 1024);
+    for (int j = 0; j < A_LOADS; ++j) {
+      uint32_t o = a_off[j];
+      asm volatile("" : "+v"(o));
+      QWIX_GLDS16(ga + o, ls + (j * NW + wave) * 1024);
+    }
 #pragma unroll
-    for (int j = 0; j < B_LOADS; ++j) QWIX_GLDS16(gb + b_off[j], ls + A_BYTES + (j * NW + wave) * 1024);
+    for (int j = 0; j < B_LOADS; ++j) {
+      uint32_t o = b_off[j];
+      asm volatile("" : "+v"(o));
+      QWIX_GLDS16(gb + o, ls + A_BYTES + (j * NW + wave) * 1024);
+    }
   };
 
   // ---- fragments
@@ -596,8 +611,8 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
       const float* sg = sa_lds + g * BM + wr * WROWS + 4 * hx;
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
-        const float4 sa4 = *reinterpret_cast<const float4*>(sg + i * 32 + 8 * qd);
-        const float sv[4] = {sa4.x, sa4.y, sa4.z, sa4.w};
+        const v4f sa4 = *reinterpret_cast<const v4f*>(sg + i * 32 + 8 * qd);
+        const float sv[4] = {sa4[0], sa4[1], sa4[2], sa4[3]};
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           accf[i][4 * qd + j] = __builtin_fmaf(static_cast<float>(acc[i][4 * qd + j]) * sv[j], sbg, accf[i][4 * qd + j]);
@@ -615,6 +630,16 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
 #pragma unroll
       for (int r = 0; r < 16; ++r) accf[i][r] = __builtin_fmaf(static_cast<float>(acc[i][r]), sbg, accf[i][r]);
     }
+  };
+
+  // A use of a tile's sums right behind its fold: without one the compiler moves the whole fold into the block
+  // where the sums are next read (behind the slab's barrier), all scale reads of the four tiles are then in flight at
+  // once and their registers push loop invariants into scratch memory.
+  auto pin_sums = [&](int i) __attribute__((always_inline)) {
+    asm volatile("" : "+v"(accf[i][0]), "+v"(accf[i][1]), "+v"(accf[i][2]), "+v"(accf[i][3]), "+v"(accf[i][4]),
+                 "+v"(accf[i][5]), "+v"(accf[i][6]), "+v"(accf[i][7]), "+v"(accf[i][8]), "+v"(accf[i][9]),
+                 "+v"(accf[i][10]), "+v"(accf[i][11]), "+v"(accf[i][12]), "+v"(accf[i][13]), "+v"(accf[i][14]),
+                 "+v"(accf[i][15]));
   };
 
   // One slab.  FIRST: it opens a group (the accumulators restart from zero, or from the magic constant).
@@ -649,11 +674,17 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
       for (int i = 0; i < TM; ++i) {
         acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa8[1][i], fb8[1], acc[i], 0, 0, 0, 0, 0, 0);
         if constexpr (LAST) {
-          if (i > 0) fold_tile(i - 1, g, sbg, recentre);
+          if (i > 0) {
+            fold_tile(i - 1, g, sbg, recentre);
+            pin_sums(i - 1);
+          }
           __builtin_amdgcn_sched_barrier(0);
         }
       }
-      if constexpr (LAST) fold_tile(TM - 1, g, sbg, recentre);
+      if constexpr (LAST) {
+        fold_tile(TM - 1, g, sbg, recentre);
+        pin_sums(TM - 1);
+      }
       return;
     } else {
     auto read_next = [&](int ks) __attribute__((always_inline)) {  // fragments of k-step ks + 1
@@ -745,13 +776,13 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int qd = 0; qd < 4; ++qd) {
-            int4 z4 = make_int4(0, 0, 0, 0);
-            if (zp) z4 = *reinterpret_cast<const int4*>(zrow + i * 32 + 8 * qd);  // a broadcast per wavefront half
-            const int zz[4] = {z4.x, z4.y, z4.z, z4.w};
+            v4i z4 = {0, 0, 0, 0};
+            if (zp) z4 = *reinterpret_cast<const v4i*>(zrow + i * 32 + 8 * qd);  // a broadcast per wavefront half
+            const int zz[4] = {z4[0], z4[1], z4[2], z4[3]};
             float sv[4] = {1.f, 1.f, 1.f, 1.f};
             if constexpr (SAG) {
-              const float4 s4 = *reinterpret_cast<const float4*>(sa_lds + g * BM + wr * WROWS + 4 * hx + i * 32 + 8 * qd);
-              sv[0] = s4.x; sv[1] = s4.y; sv[2] = s4.z; sv[3] = s4.w;
+              const v4f s4 = *reinterpret_cast<const v4f*>(sa_lds + g * BM + wr * WROWS + 4 * hx + i * 32 + 8 * qd);
+              sv[0] = s4[0]; sv[1] = s4[1]; sv[2] = s4[2]; sv[3] = s4[3];
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
