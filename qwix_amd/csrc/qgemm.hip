@@ -342,6 +342,15 @@ __global__ void __launch_bounds__(256)
 #define QWIX_GLDS16(gptr, lptr)                                                                       \
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),             \
                                    (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
+// The same load from a wave-uniform base pointer plus a per-lane 32-bit byte offset.  The offset is made opaque next to
+// the load: the address is then a scalar base register plus a 32-bit vector offset, where an offset that the compiler
+// widens to 64 bits ahead of the loop occupies two registers for the whole kernel and costs a 64-bit vector add per load.
+#define QWIX_GLDS16_AT(gbase, off32, lptr)                                                            \
+  do {                                                                                                \
+    uint32_t qwix_off_ = (off32);                                                                     \
+    asm volatile("" : "+v"(qwix_off_));                                                               \
+    QWIX_GLDS16((gbase) + qwix_off_, lptr);                                                           \
+  } while (0)
 
 // The per-row and per-column scales of one wavefront's part of the tile, in the accumulator layout
 // (acc[i][j][r]: m = m_base + i*32 + lane%32, n = n_base + j*32 + 8*(r/4) + 4*(lane/32) + r%4).
@@ -534,7 +543,7 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
   auto issue_loads = [&](int s, int k0) {
     const uint8_t* gk = gbase + k0;
 #pragma unroll
-    for (int j = 0; j < LOADS; ++j) QWIX_GLDS16(gk + goff[j], smem + s * STAGE + (wave * LOADS + j) * 1024);
+    for (int j = 0; j < LOADS; ++j) QWIX_GLDS16_AT(gk, goff[j], smem + s * STAGE + (wave * LOADS + j) * 1024);
   };
 
   // ---- fragment addresses: row r, k-chunk c lives at r*128 + ((c ^ swz8(r)) << 4); wave tiles start at multiples of 32
@@ -747,7 +756,7 @@ __device__ __forceinline__ void qgemm_mid_tile(const uint8_t* __restrict__ A, in
     if (kt >= KT) kt -= KT;
     const uint8_t* ga = A + kt * BK;
 #pragma unroll
-    for (int j = 0; j < PW; ++j) QWIX_GLDS16(ga + aoff[j], smem + st * ASTAGE + (wave * PW + j) * 1024);
+    for (int j = 0; j < PW; ++j) QWIX_GLDS16_AT(ga, aoff[j], smem + st * ASTAGE + (wave * PW + j) * 1024);
     // Issued as asm so that the compiler does not track them: its own waits for these registers, merged over
     // the loop's back edge, come out as vmcnt(0) once per trip and would drain every load in flight.  The
     // explicit waits below are what guarantees that a register set has landed before it is multiplied.
@@ -1118,13 +1127,13 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
     const uint8_t* gk = A + kt * BK;
     uint8_t* dst = smem + (kt & 1) * A_STAGE + lrow0 * BK;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) QWIX_GLDS16(gk + goffa[j], dst + j * 1024);
+    for (int j = 0; j < 4; ++j) QWIX_GLDS16_AT(gk, goffa[j], dst + j * 1024);
   };
   auto load_b = [&](int kt, int stage) {  // own half of the B rows of slab kt
     const uint8_t* gk = B + kt * BK;
     uint8_t* dst = smem + B_BASE + stage * B_STAGE + lrow0 * BK;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) QWIX_GLDS16(gk + goffb[j], dst + j * 1024);
+    for (int j = 0; j < 4; ++j) QWIX_GLDS16_AT(gk, goffb[j], dst + j * 1024);
   };
 
   // ---- fragments of a whole slab
@@ -1233,7 +1242,7 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
         }
       if (more_b) {
 #pragma unroll
-        for (int j = ks * (4 / NK); j < (ks + 1) * (4 / NK); ++j) QWIX_GLDS16(gkb + goffb[j], dstb + j * 1024);
+        for (int j = ks * (4 / NK); j < (ks + 1) * (4 / NK); ++j) QWIX_GLDS16_AT(gkb, goffb[j], dstb + j * 1024);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
