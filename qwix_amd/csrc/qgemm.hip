@@ -345,11 +345,11 @@ __global__ void __launch_bounds__(256)
 // The same load from a wave-uniform base pointer plus a per-lane 32-bit byte offset.  The offset is made opaque next to
 // the load: the address is then a scalar base register plus a 32-bit vector offset, where an offset that the compiler
 // widens to 64 bits ahead of the loop occupies two registers for the whole kernel and costs a 64-bit vector add per load.
+// (`off32` is a variable, made opaque in its own register: no copy.)
 #define QWIX_GLDS16_AT(gbase, off32, lptr)                                                            \
   do {                                                                                                \
-    uint32_t qwix_off_ = (off32);                                                                     \
-    asm volatile("" : "+v"(qwix_off_));                                                               \
-    QWIX_GLDS16((gbase) + qwix_off_, lptr);                                                           \
+    asm volatile("" : "+v"(off32));                                                                   \
+    QWIX_GLDS16((gbase) + (off32), lptr);                                                             \
   } while (0)
 
 // The per-row and per-column scales of one wavefront's part of the tile, in the accumulator layout

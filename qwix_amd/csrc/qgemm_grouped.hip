@@ -454,15 +454,13 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
     // load, base + offset is a scalar base register plus a 32-bit vector offset.
 #pragma unroll
     for (int j = 0; j < A_LOADS; ++j) {
-      uint32_t o = a_off[j];
-      asm volatile("" : "+v"(o));
-      QWIX_GLDS16(ga + o, ls + (j * NW + wave) * 1024);
+      asm volatile("" : "+v"(a_off[j]));
+      QWIX_GLDS16(ga + a_off[j], ls + (j * NW + wave) * 1024);
     }
 #pragma unroll
     for (int j = 0; j < B_LOADS; ++j) {
-      uint32_t o = b_off[j];
-      asm volatile("" : "+v"(o));
-      QWIX_GLDS16(gb + o, ls + A_BYTES + (j * NW + wave) * 1024);
+      asm volatile("" : "+v"(b_off[j]));
+      QWIX_GLDS16(gb + b_off[j], ls + A_BYTES + (j * NW + wave) * 1024);
     }
   };
 
