@@ -1213,13 +1213,20 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
   // loads have three phases to land); A one slab ahead, in the memory phase.  The waits before the
   // barriers leave the four loads just issued in flight and cover the four issued one phase earlier.
   int bst = 0;  // B stage of slab kt = kt % 3
-  for (int kt = 0; kt < KT; ++kt) {
+  // One slab; whether A of the next slab and B of the one after it are still to be requested is known at compile time,
+  // so that the steady state is one basic block (a branch would end the scheduling regions that the fences below
+  // delimit): the loop runs the slabs that request both, the last two slabs follow it.
+  auto slab = [&](int kt, auto more_a_tag, auto more_b_tag) __attribute__((always_inline)) {
+    constexpr bool more_a = decltype(more_a_tag)::value, more_b = decltype(more_b_tag)::value;
     // memory phase
     read_slab(kt & 1, bst);
     __builtin_amdgcn_sched_barrier(0);  // fragment reads first: the loads below may not slip in front of them
-    const bool more_a = kt + 1 < KT, more_b = kt + 2 < KT;
-    if (more_a) load_a(kt + 1);
-    if (more_a) wait_loads(4); else wait_loads(0);
+    if constexpr (more_a) {
+      load_a(kt + 1);
+      wait_loads(4);
+    } else {
+      wait_loads(0);
+    }
     barrier();
     // compute phase
     const int bst2 = bst == 0 ? 2 : bst - 1;  // (kt + 2) % 3
@@ -1240,17 +1247,26 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
           else
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0, 0, 0, 0);
         }
-      if (more_b) {
+      if constexpr (more_b) {
 #pragma unroll
         for (int j = ks * (4 / NK); j < (ks + 1) * (4 / NK); ++j) QWIX_GLDS16_AT(gkb, goffb[j], dstb + j * 1024);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     __builtin_amdgcn_s_setprio(0);
-    if (more_b) wait_loads(4); else wait_loads(0);
+    if constexpr (more_b) wait_loads(4); else wait_loads(0);
     barrier();
     bst = bst == 2 ? 0 : bst + 1;
+  };
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+  int kt = 0;
+  for (; kt + 2 < KT; ++kt) slab(kt, T_{}, T_{});
+  if (kt + 1 < KT) {
+    slab(kt, T_{}, F_{});
+    ++kt;
   }
+  slab(kt, F_{}, F_{});
   if (wm == 0) barrier();
 
   const int m_base = m0 + wm * 128, n_base = n0 + wn * 64;
