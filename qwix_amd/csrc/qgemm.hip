@@ -345,8 +345,15 @@ __global__ void __launch_bounds__(256)
 // The same load from a wave-uniform base pointer plus a per-lane 32-bit byte offset.  The offset is made opaque next to
 // the load: the address is then a scalar base register plus a 32-bit vector offset, where an offset that the compiler
 // widens to 64 bits ahead of the loop occupies two registers for the whole kernel and costs a 64-bit vector add per load.
-// (`off32` is a variable, made opaque in its own register: no copy.)
 #define QWIX_GLDS16_AT(gbase, off32, lptr)                                                            \
+  do {                                                                                                \
+    uint32_t qwix_off_ = (off32);                                                                     \
+    asm volatile("" : "+v"(qwix_off_));                                                               \
+    QWIX_GLDS16((gbase) + qwix_off_, lptr);                                                           \
+  } while (0)
+// The same with the offset variable made opaque in its own register (no copy per load): measured 1 % faster in the
+// ping-pong kernel's slab loop, and 20 % slower in the one-slab batched kernel, which therefore takes the form above.
+#define QWIX_GLDS16_AT_INPLACE(gbase, off32, lptr)                                                    \
   do {                                                                                                \
     asm volatile("" : "+v"(off32));                                                                   \
     QWIX_GLDS16((gbase) + (off32), lptr);                                                             \
@@ -1127,13 +1134,13 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
     const uint8_t* gk = A + kt * BK;
     uint8_t* dst = smem + (kt & 1) * A_STAGE + lrow0 * BK;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) QWIX_GLDS16_AT(gk, goffa[j], dst + j * 1024);
+    for (int j = 0; j < 4; ++j) QWIX_GLDS16_AT_INPLACE(gk, goffa[j], dst + j * 1024);
   };
   auto load_b = [&](int kt, int stage) {  // own half of the B rows of slab kt
     const uint8_t* gk = B + kt * BK;
     uint8_t* dst = smem + B_BASE + stage * B_STAGE + lrow0 * BK;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) QWIX_GLDS16_AT(gk, goffb[j], dst + j * 1024);
+    for (int j = 0; j < 4; ++j) QWIX_GLDS16_AT_INPLACE(gk, goffb[j], dst + j * 1024);
   };
 
   // ---- fragments of a whole slab
@@ -1249,7 +1256,7 @@ __device__ __forceinline__ void qgemm_pp_tile(const uint8_t* __restrict__ A, int
         }
       if constexpr (more_b) {
 #pragma unroll
-        for (int j = ks * (4 / NK); j < (ks + 1) * (4 / NK); ++j) QWIX_GLDS16_AT(gkb, goffb[j], dstb + j * 1024);
+        for (int j = ks * (4 / NK); j < (ks + 1) * (4 / NK); ++j) QWIX_GLDS16_AT_INPLACE(gkb, goffb[j], dstb + j * 1024);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
