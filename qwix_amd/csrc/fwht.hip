@@ -693,8 +693,8 @@ __global__ void __launch_bounds__(512)
           }
       }
     }
-    // round 1 over r[0] (i[3]): afterwards lane bit 4 stands for i[3] and the word order for i[2];
-    // round 2 over r[1] (i[4]): afterwards lane bit 4 stands for i[4].
+    // first exchange, over r[0] (i[3]): afterwards lane bit 4 stands for i[3] and the word order for i[2];
+    // second exchange, over r[1] (i[4]): afterwards lane bit 4 stands for i[4].
 #pragma unroll
     for (int p = 0; p < 2; ++p)
 #pragma unroll
