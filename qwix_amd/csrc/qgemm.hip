@@ -1426,7 +1426,7 @@ inline unsigned ragged_grid(int64_t M, int64_t N, int64_t G, int BM, int BN) {
   return static_cast<unsigned>((tiles + unit - 1) / unit * unit);
 }
 
-template <int QT, int OUT>
+template <int QT, int OUT, int EPI>
 __global__ void __launch_bounds__(512)
     qgemm_ragged_pp_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
                            Ragged rg, int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
@@ -1439,20 +1439,30 @@ __global__ void __launch_bounds__(512)
     return;
   }
   const Epilogue e = group_epilogue(ep, rg, g);
-  qgemm_pp_tile<QT, OUT, 2>(A, lda, B + g * rg.b_group_stride, ldb, m0, n0, m_lim, N, K, e, out, ldo);
+  qgemm_pp_tile<QT, OUT, EPI>(A, lda, B + g * rg.b_group_stride, ldb, m0, n0, m_lim, N, K, e, out, ldo);
 }
 
-template <int QT, int OUT>
-int launch_ragged_pp(const void* a, int64_t lda, const void* b, int64_t ldb, const Ragged& rg, int64_t M, int64_t N,
-                     int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+template <int QT, int OUT, int EPI>
+int launch_ragged_pp_epi(const void* a, int64_t lda, const void* b, int64_t ldb, const Ragged& rg, int64_t M, int64_t N,
+                         int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   constexpr size_t smem = 5 * 256 * 128;
-  auto kern = qgemm_ragged_pp_kernel<QT, OUT>;
+  auto kern = qgemm_ragged_pp_kernel<QT, OUT, EPI>;
   static LdsGrant granted;
   if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   kern<<<dim3(ragged_grid(M, N, rg.G, 256, 256)), 512, smem, st>>>(
       static_cast<const uint8_t*>(a), lda, static_cast<const uint8_t*>(b), ldb, rg, static_cast<int>(M),
       static_cast<int>(N), static_cast<int>(K), ep, static_cast<uint8_t*>(out), ldo);
   return check_launch("ragged qgemm (ping-pong)");
+}
+// The epilogue's rounding flags at compile time when every step rounds to bf16 (bf16 scales, bf16 result) or none
+// does (f32 throughout), as the dense dispatch does; at run time otherwise.
+template <int QT, int OUT>
+int launch_ragged_pp(const void* a, int64_t lda, const void* b, int64_t ldb, const Ragged& rg, int64_t M, int64_t N,
+                     int64_t K, const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
+  const bool all = ep.r0 && ep.r1 && ep.r2, none = !ep.r0 && !ep.r1 && !ep.r2;
+  if (OUT == QWIX_BF16 && all) return launch_ragged_pp_epi<QT, OUT, 1>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+  if (OUT == QWIX_F32 && none) return launch_ragged_pp_epi<QT, OUT, 0>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
+  return launch_ragged_pp_epi<QT, OUT, 2>(a, lda, b, ldb, rg, M, N, K, ep, out, ldo, st);
 }
 
 template <int QT, int BM, int BN, int BK>
