@@ -3039,10 +3039,14 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
         if (out_dtype == QWIX_BF16) return launch_mid<QWIX_INT8, QWIX_BF16, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
         return launch_mid<QWIX_INT8, QWIX_F32, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       }
+      // (the epilogue's rounding flags at compile time in the common case: bf16 scales, bf16 result)
+      const bool all_round = ep.r0 && ep.r1 && ep.r2;
       if (qtype == QWIX_INT8) {
+        if (out_dtype == QWIX_BF16 && all_round) return launch_mid<QWIX_INT8, QWIX_BF16, 1>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
         if (out_dtype == QWIX_BF16) return launch_mid<QWIX_INT8, QWIX_BF16>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
         return launch_mid<QWIX_INT8, QWIX_F32>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       }
+      if (out_dtype == QWIX_BF16 && all_round) return launch_mid<QWIX_E4M3, QWIX_BF16, 1>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       if (out_dtype == QWIX_BF16) return launch_mid<QWIX_E4M3, QWIX_BF16>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       return launch_mid<QWIX_E4M3, QWIX_F32>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     }
