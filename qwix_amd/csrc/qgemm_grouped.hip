@@ -674,14 +674,14 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
         if constexpr (LAST) {
           if (i > 0) {
             fold_tile(i - 1, g, sbg, recentre);
-            pin_sums(i - 1);
+            if constexpr (SAG) pin_sums(i - 1);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
       }
       if constexpr (LAST) {
         fold_tile(TM - 1, g, sbg, recentre);
-        pin_sums(TM - 1);
+        if constexpr (SAG) pin_sums(TM - 1);
       }
       return;
     } else {
