@@ -338,7 +338,7 @@ __global__ void __launch_bounds__(256)
 // The workgroup is WGM x WGN wavefronts; with 8 wavefronts (two per SIMD) the issue time of one
 // wavefront's loads and fragment reads hides behind the other's MFMAs.
 // EPI: 0 = no bf16 rounding in the epilogue, 1 = every step rounds to bf16, 2 = flags at run time,
-// 3 = flags at run time and zero-point correction.
+// 3 = flags at run time and zero-point correction, 4 = every step rounds to bf16 and zero-point correction.
 #define QWIX_GLDS16(gptr, lptr)                                                                       \
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),             \
                                    (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
@@ -416,9 +416,9 @@ __device__ __forceinline__ void staged_epilogue(const AccT (&acc)[TM][TN], const
   constexpr int CPR = WTN * ES / 16;             // 16-byte chunks per staged row
   constexpr int EPC = 16 / ES;                   // elements per chunk
   static_assert(NWAVES * 32 * ROWB <= LDS_BYTES, "epilogue staging does not fit in LDS");
-  constexpr bool ZP = (EPI == 3);  // run-time rounding flags plus zero-point correction
-  const bool r0 = EPI >= 2 ? ep.r0 != 0 : EPI == 1, r1 = EPI >= 2 ? ep.r1 != 0 : EPI == 1,
-             r2 = EPI >= 2 ? ep.r2 != 0 : EPI == 1;
+  constexpr bool ZP = (EPI == 3 || EPI == 4);  // zero-point correction
+  constexpr bool ALL = (EPI == 1 || EPI == 4), RUNTIME = (EPI == 2 || EPI == 3);
+  const bool r0 = RUNTIME ? ep.r0 != 0 : ALL, r1 = RUNTIME ? ep.r1 != 0 : ALL, r2 = RUNTIME ? ep.r2 != 0 : ALL;
   int zuv[TM];
   if constexpr (ZP) {
 #pragma unroll
@@ -439,14 +439,25 @@ __device__ __forceinline__ void staged_epilogue(const AccT (&acc)[TM][TN], const
         if constexpr (OUT == QWIX_I32) {
           *reinterpret_cast<int4*>(dst) = make_int4(static_cast<int>(acc[i][j][4 * qd]), static_cast<int>(acc[i][j][4 * qd + 1]),
                                                     static_cast<int>(acc[i][j][4 * qd + 2]), static_cast<int>(acc[i][j][4 * qd + 3]));
-        } else if constexpr (EPI == 1 && OUT == QWIX_BF16) {
+        } else if constexpr (ALL && OUT == QWIX_BF16) {
           // Every step rounds to bf16 and the result is bf16: round two values per v_cvt_pk_bf16_f32,
           // and let the last rounding produce the packed output directly.
           uint32_t w[2];
+          int zvv[4] = {0, 0, 0, 0};
+          if constexpr (ZP) {
+            const int n = n_base + j * 32 + 8 * qd + 4 * (lane >> 5);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) zvv[r] = ep.zv[min(n + r, N - 1)];
+          }
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
-            uint32_t pk = pack_bf16x2(static_cast<float>(acc[i][j][4 * qd + 2 * h]),
-                                      static_cast<float>(acc[i][j][4 * qd + 2 * h + 1]));
+            uint32_t pk;
+            if constexpr (ZP)
+              pk = pack_bf16x2(static_cast<float>(static_cast<int>(acc[i][j][4 * qd + 2 * h]) - zuv[i] * zvv[2 * h]),
+                               static_cast<float>(static_cast<int>(acc[i][j][4 * qd + 2 * h + 1]) - zuv[i] * zvv[2 * h + 1]));
+            else
+              pk = pack_bf16x2(static_cast<float>(acc[i][j][4 * qd + 2 * h]),
+                               static_cast<float>(acc[i][j][4 * qd + 2 * h + 1]));
             pk = pack_bf16x2(__uint_as_float(pk << 16) * sa, __uint_as_float(pk & 0xFFFF0000u) * sa);
             w[h] = pack_bf16x2(__uint_as_float(pk << 16) * sbv[j][qd][2 * h],
                                __uint_as_float(pk & 0xFFFF0000u) * sbv[j][qd][2 * h + 1]);
@@ -1312,6 +1323,7 @@ int dispatch_pp(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t 
   const bool all = ep.r0 && ep.r1 && ep.r2, none = !ep.r0 && !ep.r1 && !ep.r2;
   if (ep.zu != nullptr) {
     if constexpr (QT == QWIX_INT8) {
+      if (ep.out_dtype == QWIX_BF16 && all) return launch_pp<QT, QWIX_BF16, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       if (ep.out_dtype == QWIX_BF16) return launch_pp<QT, QWIX_BF16, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       return launch_pp<QT, QWIX_F32, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     }
