@@ -481,6 +481,10 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   b, b_is4 = c.rhs_values(rhs)
   sa, ga = c.lhs_scale(lhs) if isinstance(lhs, QArray) else (None, 1)
   sb, gb = c.rhs_scale(rhs) if isinstance(rhs, QArray) else (None, 1)
+  if b_is4 and ga == 1 and gb == 1 and c.K % 128:
+    # per-channel int4 weights whose K the sub-channel kernel does not take: widened to int8 (the same integers)
+    b = rhs.qvalue.unpack().permute(*(c.rfree + c.rca)).contiguous().reshape(c.N, c.K)
+    b_is4, rq = False, numerics.INT8
   dev = a.device
   st = _lib.stream_of(a)
   out = torch.empty(c.M, c.N, dtype=res_t, device=dev)

@@ -60,6 +60,15 @@ class Int4Tensor:
     out = torch.stack([lo, hi], dim=-1).reshape(*d.shape[:-1], d.shape[-1] * 2)
     return out.movedim(-1, self.packed_axis)
 
+  @staticmethod
+  def pack(values: torch.Tensor, packed_axis: int = -1) -> 'Int4Tensor':
+    """The reverse of unpack(): int8 values in [-8, 7] to nibble pairs along `packed_axis` (a host-side convenience
+    for re-laying out values that exist already; quantization itself writes packed nibbles)."""
+    packed_axis = packed_axis % values.ndim
+    v = values.movedim(packed_axis, -1).to(torch.uint8) & 0xF
+    data = (v[..., 0::2] | (v[..., 1::2] << 4)).contiguous()
+    return Int4Tensor(data.movedim(-1, packed_axis), tuple(values.shape), packed_axis)
+
   def permute(self, *axes) -> 'Int4Tensor':
     axes = tuple(axes[0]) if len(axes) == 1 and not isinstance(axes[0], int) else tuple(axes)
     return Int4Tensor(self.data.permute(*axes), tuple(self.shape[a] for a in axes), axes.index(self.packed_axis))
@@ -414,6 +423,39 @@ def _plan_cached(shape: tuple[int, ...], tiles: tuple[int, ...]) -> _Plan:
   )
 
 
+def _regrouped(shape, sshape):
+  """Any tiling as a 2-D problem: every axis split into (tile count, tile), the counts in front.  Returns the split
+  shape, the permutation that brings the counts to the front, and (rows, cols) = (scales, elements per scale)."""
+  tiles = [d // s for d, s in zip(shape, sshape)]
+  split = [v for st in zip(sshape, tiles) for v in st]
+  n = len(shape)
+  perm = [2 * a for a in range(n)] + [2 * a + 1 for a in range(n)]
+  return tiles, split, perm, math.prod(sshape), math.prod(tiles)
+
+
+def _ungroup(values2d: torch.Tensor, shape, sshape) -> torch.Tensor:
+  tiles, _, perm, _, _ = _regrouped(shape, sshape)
+  inv = [perm.index(a) for a in range(len(perm))]
+  return values2d.reshape(*sshape, *tiles).permute(*inv).reshape(shape)
+
+
+def _quantize_regrouped(array: torch.Tensor, how: HowToQuantize, q: str, sshape) -> 'QArray':
+  """Patterns with more than two separate groups of reduced axes (say 2-D blocks and a whole axis besides): the
+  elements of a scale are gathered into a row (one copy), the rows are quantized with one scale each, and the values
+  return to their places (one copy).  The same maxima over the same elements: identical results."""
+  shape = tuple(array.shape)
+  _, split, perm, rows, cols = _regrouped(shape, sshape)
+  x2 = array.reshape(split).permute(*perm).reshape(rows, cols).contiguous()
+  q2 = quantize(x2, HowToQuantize(qtype=q, channelwise_axes=(0,), calibration_method=how.calibration_method),
+                layout='natural')
+  vals = q2.qvalue.unpack() if isinstance(q2.qvalue, Int4Tensor) else q2.qvalue
+  vals = _ungroup(vals, shape, sshape).contiguous()
+  if q == numerics.INT4:
+    vals = Int4Tensor.pack(vals)
+  zp = None if q2.zero_point is None else q2.zero_point.reshape(sshape)
+  return QArray(vals, q2.scale.reshape(sshape), zp, q)
+
+
 def _tiles_from_how(shape, how: HowToQuantize) -> tuple[int, ...]:
   ss = get_scale_shape(shape, how)
   return tuple(d // s for d, s in zip(shape, ss))
@@ -483,6 +525,12 @@ def _workspace(plan: _Plan, cal: int, device) -> tuple[torch.Tensor | None, int]
   return torch.empty(n, dtype=torch.uint8, device=device), n
 
 
+def _reduce_minor_order(shape, plan: _Plan) -> tuple[int, ...]:
+  red = tuple(plan.reduce_axes)
+  return (tuple(plan.outer_axes) + tuple(plan.inner_axes) + tuple(a for a in red if shape[a] == 1) +
+          tuple(a for a in red if shape[a] != 1))
+
+
 def _alloc_q(shape, qtype: str, plan: _Plan, layout: int, device):
   """Allocates the qvalue buffer; returns (flat storage tensor, logical view)."""
   is4 = qtype == numerics.INT4
@@ -494,11 +542,14 @@ def _alloc_q(shape, qtype: str, plan: _Plan, layout: int, device):
       return data, Int4Tensor(data, shape, len(shape) - 1)
     data = torch.empty(tuple(shape), dtype=numerics.storage_dtype(qtype), device=device)
     return data, data
-  # reduce-minor: physical order (outer axes, inner axes, reduce axes).
-  order = plan.outer_axes + plan.inner_axes + plan.reduce_axes
+  # reduce-minor: physical order (outer axes, inner axes, reduce axes); reduce axes of size 1 lead the others
+  # (the memory is the same) so that the last axis, which int4 pairs run along, is a real one.
+  order = _reduce_minor_order(shape, plan)
   phys_shape = [shape[a] for a in order]
   inv = [order.index(a) for a in range(len(shape))]
   if is4:
+    if phys_shape[-1] % 2:
+      raise NotImplementedError(f'int4 in the reduce-minor layout needs an even last reduced axis, got {tuple(shape)}')
     phys_shape[-1] //= 2
     data = torch.empty(phys_shape, dtype=torch.uint8, device=device)
     return data, Int4Tensor(data.permute(*inv), shape, order[-1])
@@ -522,9 +573,14 @@ def _check_empty_reduction(sshape) -> None:
     raise ValueError('zero-size array to reduction operation max which has no identity')
 
 
-def _default_layout(plan: _Plan, layout: str | None) -> int:
+def _default_layout(plan: _Plan, layout: str | None, shape=None, qtype: str | None = None) -> int:
   if layout is None:
     layout = 'reduce_minor' if (plan.kind == '3d' and plan.dims[2] > 1 and plan.dims[1] % 8 == 0 and plan.tiles[0] % 8 == 0) else 'natural'
+    if layout == 'reduce_minor' and qtype == numerics.INT4:
+      # int4 pairs run along the last reduce axis that is not of size 1: it has to be even
+      real = [shape[a] for a in plan.reduce_axes if shape[a] != 1]
+      if not real or real[-1] % 2:
+        layout = 'natural'
   if layout not in ('natural', 'reduce_minor'):
     raise ValueError(f'unknown layout {layout!r}')
   return _lib.LAYOUT_NATURAL if layout == 'natural' else _lib.LAYOUT_REDUCE_MINOR
@@ -609,7 +665,7 @@ def quantize_with_scale_zero_point(array: torch.Tensor, qtype, scale: torch.Tens
               plan.tiles[0], numerics.qtype_tag(q), scale.data_ptr(), _lib.ptr(zp), noise.data_ptr(), data.data_ptr(),
               _lib.stream_of(array))
     return QArray(view, scale, zero_point, q)
-  lay = _default_layout(plan, layout)
+  lay = _default_layout(plan, layout, shape, q)
   data, view = _alloc_q(shape, q, plan, lay, array.device)
   zp = None if zero_point is None else zero_point.contiguous()
   _lib.call('qwix_hip_quantize_with_scale', array.data_ptr(), _lib.float_tag(array.dtype), *plan.dims, plan.tiles[0],
@@ -641,7 +697,12 @@ def quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = No
     _check_empty_reduction(sshape)
     zp = torch.empty(sshape, dtype=torch.int8, device=array.device) if cal == _lib.MINMAX else None
     return QArray(_empty_qvalue(shape, q, array.device), torch.empty(sshape, dtype=array.dtype, device=array.device), zp, q)
-  plan = _plan(shape, tuple(d // s for d, s in zip(shape, sshape)))
+  try:
+    plan = _plan(shape, tuple(d // s for d, s in zip(shape, sshape)))
+  except NotImplementedError:
+    if layout not in (None, 'natural'):
+      raise
+    return _quantize_regrouped(_check_float_input(array), how, q, sshape)
   if not array.is_contiguous() and plan.kind == '3d' and plan.dims[2] > 1 and layout in (None, 'reduce_minor'):
     # A strided view whose reduced axes are already the contiguous ones (e.g. a rotated weight kept
     # K-contiguous): quantize its physical rows and hand back views with the logical shape.
@@ -671,10 +732,12 @@ def quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = No
               numerics.qtype_tag(q), cal, factor, data.data_ptr(), scale.data_ptr(), _lib.ptr(zp),
               _lib.stream_of(array))
     return QArray(view, scale, zp, q)
-  lay = _default_layout(plan, layout)
+  lay = _default_layout(plan, layout, shape, q)
   outer, reduce, inner = plan.dims
-  if inner > 1 and (inner % (8 if array.dtype == torch.bfloat16 else 4) != 0):
-    # ragged strided reduce: the complete-but-slow kernel handles it (natural layout).
+  if (inner > 1 and (inner % (8 if array.dtype == torch.bfloat16 else 4) != 0)) or (
+      q == numerics.INT4 and inner == 1 and plan.tiles[0] % 2):
+    # ragged strided reduce, or int4 groups of odd length (a nibble pair straddles two groups): the
+    # complete-but-slow kernel handles it (natural layout).
     data, view = _alloc_q(shape, q, plan, _lib.LAYOUT_NATURAL, array.device)
     import ctypes
     dims = (ctypes.c_int64 * 5)(outer, reduce, inner, 1, 1)
@@ -715,7 +778,7 @@ def physical_layout(qa: QArray) -> tuple[_Plan, int, torch.Tensor]:
   if data.is_contiguous() and (not is4 or qa.qvalue.packed_axis == len(shape) - 1):
     return plan, _lib.LAYOUT_NATURAL, data
   if plan.kind == '3d':
-    order = plan.outer_axes + plan.inner_axes + plan.reduce_axes
+    order = _reduce_minor_order(shape, plan)
     phys = data.permute(*order)
     if phys.is_contiguous() and (not is4 or qa.qvalue.packed_axis == order[-1]):
       return plan, _lib.LAYOUT_REDUCE_MINOR, phys
@@ -732,7 +795,20 @@ def dequantize(array: QArray) -> torch.Tensor:
   validate_qarray(array)
   if math.prod(array.shape) == 0:
     return torch.empty(array.shape, dtype=array.scale.dtype, device=array.scale.device)
-  plan, lay, data = physical_layout(array)
+  try:
+    plan, lay, data = physical_layout(array)
+  except NotImplementedError as e:
+    if 'separate reduced axis groups' not in str(e):
+      raise
+    # more than two separate groups of reduced axes: gather the elements of a scale into a row, dequantize the rows,
+    # put the values back (a copy each way)
+    shape, sshape = tuple(array.shape), tuple(array.scale.shape)
+    _, split, perm, rows, cols = _regrouped(shape, sshape)
+    vals = array.qvalue.unpack() if isinstance(array.qvalue, Int4Tensor) else array.qvalue
+    v2 = vals.reshape(split).permute(*perm).reshape(rows, cols).contiguous()
+    q2 = QArray(v2, array.scale.reshape(rows, 1), None if array.zero_point is None else array.zero_point.reshape(rows, 1),
+                numerics.INT8 if array.qtype == numerics.INT4 else array.qtype)
+    return _ungroup(dequantize(q2), shape, sshape).contiguous()
   out = torch.empty(array.shape, dtype=array.scale.dtype, device=array.scale.device)
   scale = array.scale.contiguous()
   zp = None if array.zero_point is None else array.zero_point.contiguous()

@@ -47,6 +47,9 @@ struct GroupedArgs {
   // group axis for an array that is the same for all groups.  Both null: symmetric operands.
   const int32_t* zu; int64_t zu_sm, zu_sg;
   const int32_t* zv; int64_t zv_sn, zv_sg;
+  // One group spans all of K (int4 weights with per-channel scales): the fast kernel then scales like the untiled
+  // contraction, ((T(acc) * sx) * sy) with a rounding per step (dot_general.py:255-261), not like a sum of partials.
+  int single;
 };
 
 __device__ __forceinline__ float ld_scale(const void* p, int dtype, int64_t i) {
@@ -733,6 +736,7 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
   // The scale of the next group is fetched at the start of a group, together with the slab loads:
   // a load issued just before the barrier would make the barrier's wait for the slab wait for it too.
   auto to_scale = [&](unsigned raw) __attribute__((always_inline)) {
+    if (p.single) return AUX ? 1.0f : kUnscale;  // the sums hold the plain integer; the epilogue scales it
     return __uint_as_float(SBF ? raw << 16 : raw) * (AUX ? 1.0f : kUnscale);
   };
   unsigned sb_cur = sb_raw, sb_next = 0;
@@ -826,12 +830,31 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
       const int c = lane + 64 * q, row = c >> 3, cc = c & 7;
       const float4 v4 = *reinterpret_cast<const float4*>(stg + row * ROW_F + cc * 4);
       float v[4] = {v4.x, v4.y, v4.z, v4.w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        v[e] *= sav[i][q];
-        if (t_bf16) v[e] = round_bf16(v[e]);
-      }
       const int m = m0 + wr * WROWS + i * 32 + row, n = n0 + wc * 32 + cc * 4;
+      if (p.single) {
+        // the untiled chain: the integer takes the first scale's dtype, every product the promotion of its factors
+        const bool a_bf = p.sa == nullptr || p.sa_dtype == QWIX_BF16;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float t = v[e];
+          if (p.sa != nullptr) {
+            if (a_bf) t = round_bf16(t);
+            t *= sav[i][q];
+            if (a_bf) t = round_bf16(t);
+          } else if (t_bf16) {
+            t = round_bf16(t);
+          }
+          t *= (n + e < p.N) ? ld_scale(p.sb, p.sb_dtype, n + e) : 0.f;
+          if (t_bf16) t = round_bf16(t);
+          v[e] = t;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] *= sav[i][q];
+          if (t_bf16) v[e] = round_bf16(v[e]);
+        }
+      }
       if (m >= p.M || n >= p.N) continue;
       if (p.out_dtype == QWIX_BF16) {
         uint16_t* o = reinterpret_cast<uint16_t*>(p.out) + static_cast<int64_t>(m) * p.ldo + n;
@@ -1049,6 +1072,9 @@ static int grouped_impl(const void* a, int64_t lda, const void* b, int64_t ldb_b
   p.zv = zv; p.zv_sn = zv_col_stride; p.zv_sg = zv_group_stride;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool row_strides_fit = 128 * lda < (int64_t{1} << 31) && 256 * ldb_bytes < (int64_t{1} << 31);
+  // One group: there is no sum of partials to keep in f32, so both modes give the reference's roundings.
+  p.single = (b_qtype != QWIX_E4M3 && group == K) ? 1 : 0;
+  if (p.single) exact = 1;
   if (b_qtype == QWIX_E4M3) {
     if (!exact && row_strides_fit) {
       const int rc = (sa != nullptr && ga > 1) ? dispatch_grouped_f8<true>(p, st) : dispatch_grouped_f8<false>(p, st);
@@ -1056,7 +1082,7 @@ static int grouped_impl(const void* a, int64_t lda, const void* b, int64_t ldb_b
     }
     return launch_grouped<QWIX_E4M3, true>(p, st);
   }
-  if (!exact && row_strides_fit) {
+  if ((!exact || p.single) && row_strides_fit) {
     // per-group activation scales ride along in LDS: the tile's scales must fit behind the slab stages
     const bool sag = sa != nullptr && ga > 1;
     int rc;

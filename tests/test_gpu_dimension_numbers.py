@@ -457,3 +457,32 @@ def test_e4m3_operands_with_sub_channel_scales(ltile, rtile, sdt):
   out = dg.dot_general(xq, wq, dn, preferred_element_type=torch.float32)
   torch.cuda.synchronize()
   assert torch.allclose(out, ref, rtol=1e-4, atol=1e-4 * ref.abs().mean().item())
+
+
+@pytest.mark.parametrize('act_calibration', ['absmax', 'minmax'])
+@pytest.mark.parametrize('M,K,N,dtype', [
+    (64, 2048, 264, O.BF16), (513, 256, 264, O.BF16), (128, 1152, 128, O.F32), (8, 768, 72, O.BF16),
+    (256, 64, 1024, O.BF16), (17, 192, 1024, O.BF16), (3, 144, 64, O.F32),  # K the sub-channel kernel does not take
+])
+def test_int4_weights_with_per_channel_scales_bit_exact(M, K, N, dtype, act_calibration):
+  """int8 x int4 with one scale per row / column is the untiled contraction of dot_general.py:205-226,255-261:
+  exact integers, then (T(acc) * sx) * sy with a rounding per step, whatever kernel multiplies."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  print('case int4 per-channel', M, K, N, dtype, act_calibration, flush=True)
+  x_np, x_t = util.make((M, K), dtype, seed=M + K)
+  if act_calibration == 'minmax':
+    x_np = O.rnd(x_np + 0.7, dtype)
+    x_t = util.to_gpu(x_np, dtype)
+  w_np, w_t = util.make((K, N), dtype, seed=N + K, scale=0.05)
+  ha = dict(qtype='int8', channelwise_axes=[0], calibration_method=act_calibration)
+  hw = dict(qtype='int4', channelwise_axes=[1])
+  xq, wq = qarray.quantize(x_t, qarray.HowToQuantize(**ha)), qarray.quantize(w_t, qarray.HowToQuantize(**hw))
+  oxq, owq = O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(**ha)), O.quantize(O.FArr(w_np, dtype), O.HowToQuantize(**hw))
+  util.assert_qarray_equal(xq, oxq, 'lhs')
+  util.assert_qarray_equal(wq, owq, 'rhs')
+  dn = (((1,), (0,)), ((), ()))
+  got = util.f32np(dg.dot_general(xq, wq, dn))
+  want = O.dot_general(oxq, owq, dn).v
+  bad = np.flatnonzero(got.ravel() != want.ravel())
+  assert bad.size == 0, f'{bad.size} of {got.size} outputs differ: {got.ravel()[bad[:4]]} vs {want.ravel()[bad[:4]]}'

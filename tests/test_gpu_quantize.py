@@ -394,3 +394,29 @@ def test_stochastic_rounding_with_caller_noise(shape, kw, dtype, qtype):
   if 'calibration_method' not in kw:
     f8 = qarray.quantize(x_t, qarray.HowToQuantize(qtype='float8_e4m3fn', noise_fn=noise_fn, **kw))
     util.assert_qarray_equal(f8, O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(qtype='float8_e4m3fn', **kw)), 'f8 ignores noise')
+
+
+@pytest.mark.parametrize('qtype,calibration', [('int8', 'absmax'), ('int4', 'minmax'), (O.E4M3, 'absmax')])
+def test_three_separate_groups_of_reduced_axes(qtype, calibration):
+  """Blocks on the first two axes and the whole last axis under one scale, a kept axis between them: more groups
+  of reduced axes than the kernels take in place; the elements of a scale are gathered into rows first."""
+  from qwix_amd.core import qarray
+  shape, how = (48, 16, 40, 2), dict(qtype=qtype, channelwise_axes=[2], tiled_axes={0: 2, 1: 8}, calibration_method=calibration)
+  x_np, x_t = util.make(shape, O.BF16, seed=77)
+  q = qarray.quantize(x_t, qarray.HowToQuantize(**how))
+  oq = O.quantize(O.FArr(x_np, O.BF16), O.HowToQuantize(**how))
+  assert tuple(q.scale.shape) == (24, 2, 40, 1)
+  util.assert_qarray_equal(q, oq, 'regrouped')
+  assert np.array_equal(util.f32np(qarray.dequantize(q)), O.dequantize(oq).v)
+
+
+def test_int4_with_a_scale_per_element_and_unit_reduced_axes():
+  """Groups of one element (every axis channelwise) and reduced axes of size 1 next to real ones."""
+  from qwix_amd.core import qarray
+  for shape, how in [((64, 16), dict(qtype='int4', channelwise_axes=[0, 1])),
+                     ((16, 256, 1, 24), dict(qtype='int4', channelwise_axes=[0, 3], tiled_axes={2: 1}, calibration_method='minmax'))]:
+    x_np, x_t = util.make(shape, O.BF16, seed=5)
+    q = qarray.quantize(x_t, qarray.HowToQuantize(**how))
+    oq = O.quantize(O.FArr(x_np, O.BF16), O.HowToQuantize(**how))
+    util.assert_qarray_equal(q, oq, str(shape))
+    assert np.array_equal(util.f32np(qarray.dequantize(q)), O.dequantize(oq).v)
