@@ -868,6 +868,8 @@ def float_dot_general(lhs: torch.Tensor, rhs: torch.Tensor, dimension_numbers, p
   out = ([lsub[a] for a in lba] + [lsub[a] for a in range(lhs.ndim) if a not in lca and a not in lba] +
          [rsub[a] for a in range(rhs.ndim) if a not in rca and a not in rba])
   ct = torch.promote_types(lhs.dtype, rhs.dtype)
+  if preferred_element_type == torch.float32:
+    ct = torch.float32  # bf16 operands with an f32 result: f32 sums delivered as they are, not rounded to bf16 on the way
   res = torch.einsum(f"{''.join(lsub)},{''.join(rsub)}->{''.join(out)}", lhs.to(ct), rhs.to(ct))
   return res if preferred_element_type is None else res.to(preferred_element_type)
 

@@ -486,3 +486,23 @@ def test_int4_weights_with_per_channel_scales_bit_exact(M, K, N, dtype, act_cali
   want = O.dot_general(oxq, owq, dn).v
   bad = np.flatnonzero(got.ravel() != want.ravel())
   assert bad.size == 0, f'{bad.size} of {got.size} outputs differ: {got.ravel()[bad[:4]]} vs {want.ravel()[bad[:4]]}'
+
+
+def test_f32_result_of_the_dequantize_first_path_is_not_rounded_to_bf16():
+  """Tiles finer than 128 send both operands through dequantize + float dot (dot_general.py:407-491, 264-275); with
+  preferred_element_type f32 the bf16 x bf16 products are summed and delivered in f32.  Compared at 1e-5 of the
+  largest output (the order of the f32 additions is free); a result rounded to bf16 on the way is off by 2e-3."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make((33, 128), O.BF16, seed=34)
+  w_np, w_t = util.make((128, 16), O.BF16, seed=35, scale=0.05)
+  ha = dict(qtype='int8', channelwise_axes=[0], tiled_axes={1: 32})
+  hw = dict(qtype='int8', channelwise_axes=[1], tiled_axes={0: 32})
+  xq, wq = qarray.quantize(x_t, qarray.HowToQuantize(**ha)), qarray.quantize(w_t, qarray.HowToQuantize(**hw))
+  oxq, owq = O.quantize(O.FArr(x_np, O.BF16), O.HowToQuantize(**ha)), O.quantize(O.FArr(w_np, O.BF16), O.HowToQuantize(**hw))
+  dn = (((1,), (0,)), ((), ()))
+  assert not O.use_fast_path(oxq, owq, dn)
+  out = dg.dot_general(xq, wq, dn, preferred_element_type=torch.float32)
+  want = O.dot_general(oxq, owq, dn, preferred_element_type=O.F32)
+  assert out.dtype == torch.float32 and want.dtype == O.F32
+  np.testing.assert_allclose(util.f32np(out), want.v, rtol=0, atol=1e-5 * float(np.abs(want.v).max()))
