@@ -97,6 +97,9 @@ def rotate_and_quantize(x: torch.Tensor, dim: int, how: qarray.HowToQuantize, pr
     raise NotImplementedError('rotate_and_quantize supports plain absmax calibration')
   tile = tiles[dim]
   q = numerics.canonical_qtype(how.qtype)
+  if n < 8 or (tile != n and tile > 512) or tile & (tile - 1):
+    # outside the fused kernel's shapes (rows of fewer than 8, tiles of more than 512 short of the row): two launches
+    return qarray.quantize(fwht(x, dim, pre_sign, post_sign, out_scale).contiguous(), how)
   rows = _rows_view(x, dim)
   nrows = rows.numel() // n
   lead = tuple(rows.shape[:-1])

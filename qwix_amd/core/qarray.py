@@ -607,9 +607,17 @@ def calibrate(array: torch.Tensor, how: HowToQuantize) -> dict[str, torch.Tensor
     _check_empty_reduction(sshape)
     outs = [torch.empty(sshape, dtype=array.dtype, device=array.device) for _ in range(2 if cal == _lib.MINMAX else 1)]
     return {'min': outs[0], 'max': outs[1]} if cal == _lib.MINMAX else {'absmax': outs[0]}
-  plan = _plan(shape, _tiles_from_how(shape, how))
-  if plan.kind != '3d':
-    raise NotImplementedError('calibrate() alone supports a single reduced axis group')
+  try:
+    plan = _plan(shape, _tiles_from_how(shape, how))
+  except NotImplementedError:
+    plan = None
+  ev = 8 if array.dtype == torch.bfloat16 else 4
+  if plan is None or plan.kind != '3d' or (plan.dims[2] > 1 and plan.dims[2] % ev):
+    # more than one group of reduced axes: the elements of a scale gathered into a row, one statistic per row
+    _, split, perm, rows, cols = _regrouped(shape, sshape)
+    x2 = array.reshape(split).permute(*perm).reshape(rows, cols).contiguous()
+    got = calibrate(x2, HowToQuantize(qtype=how.qtype, channelwise_axes=(0,), calibration_method=how.calibration_method))
+    return {k: v.reshape(sshape) for k, v in got.items()}
   outs = [torch.empty(sshape, dtype=array.dtype, device=array.device) for _ in range(2 if cal == _lib.MINMAX else 1)]
   ws, nws = _workspace(plan, cal, array.device)
   _lib.call('qwix_hip_calibrate', array.data_ptr(), _lib.float_tag(array.dtype), *plan.dims, plan.tiles[0], cal,
@@ -651,9 +659,37 @@ def quantize_with_scale_zero_point(array: torch.Tensor, qtype, scale: torch.Tens
   scale = scale.to(array.dtype).contiguous()
   if array.numel() == 0:
     return QArray(_empty_qvalue(shape, q, array.device), scale, zero_point, q)
-  plan = _plan(shape, tuple(d // s for d, s in zip(shape, scale.shape)))
-  if plan.kind != '3d':
-    raise NotImplementedError('static-scale quantization supports a single reduced axis group')
+  try:
+    plan = _plan(shape, tuple(d // s for d, s in zip(shape, scale.shape)))
+  except NotImplementedError:
+    plan = None
+  ev = 8 if array.dtype == torch.bfloat16 else 4
+  if (plan is None or plan.kind != '3d' or (plan.dims[2] > 1 and plan.dims[2] % ev)
+      or (q == numerics.INT4 and plan.dims[2] == 1 and plan.tiles[0] % 2)):
+    # The static-scale kernels take one group of reduced axes (and whole 16-byte pieces of kept inner axes): any
+    # other pattern gathers the elements of a scale into a row first and puts the values back afterwards.
+    if layout not in (None, 'natural'):
+      raise NotImplementedError(f'static-scale quantization of shape {shape} with scales {tuple(scale.shape)} is '
+                                'delivered in the natural layout only')
+    sshape = tuple(scale.shape)
+    _, split, perm, rows, cols = _regrouped(shape, sshape)
+    if q == numerics.INT4 and cols % 2:
+      raise NotImplementedError(f'static-scale int4 quantization needs an even number of elements per scale, got {cols}')
+    regroup = lambda t: t.reshape(split).permute(*perm).reshape(rows, cols).contiguous()
+    noise2 = None
+    if noise_fn is not None and q in (numerics.INT8, numerics.INT4):
+      noise = noise_fn(shape)
+      if not isinstance(noise, torch.Tensor) or tuple(noise.shape) != shape:
+        raise ValueError(f'noise_fn must return a tensor of shape {shape}')
+      noise2 = lambda _shape, n=regroup(noise.to(array.device)): n
+    q2 = quantize_with_scale_zero_point(regroup(array), q, scale.reshape(rows, 1),
+                                        None if zero_point is None else zero_point.reshape(rows, 1), noise2,
+                                        layout='natural')
+    vals = q2.qvalue.unpack() if isinstance(q2.qvalue, Int4Tensor) else q2.qvalue
+    vals = _ungroup(vals, shape, sshape).contiguous()
+    if q == numerics.INT4:
+      vals = Int4Tensor.pack(vals)
+    return QArray(vals, scale, zero_point, q)
   if noise_fn is not None and q in (numerics.INT8, numerics.INT4):
     noise = noise_fn(shape)
     if not isinstance(noise, torch.Tensor) or tuple(noise.shape) != shape:

@@ -420,3 +420,28 @@ def test_int4_with_a_scale_per_element_and_unit_reduced_axes():
     oq = O.quantize(O.FArr(x_np, O.BF16), O.HowToQuantize(**how))
     util.assert_qarray_equal(q, oq, str(shape))
     assert np.array_equal(util.f32np(qarray.dequantize(q)), O.dequantize(oq).v)
+
+
+@pytest.mark.parametrize('shape,sshape,qtype,asym', [
+    ((64, 2, 128), (4, 2, 1), 'int4', True),       # two groups of reduced axes around a kept one
+    ((8, 64), (2, 4), 'int8', False),              # 2-D blocks
+    ((16, 2), (4, 2), 'int8', False),              # a kept inner axis shorter than a 16-byte piece
+    ((256, 128, 8), (2, 2, 4), O.E4M3, False),     # three groups of reduced axes
+])
+def test_static_scales_of_any_tiling(shape, sshape, qtype, asym):
+  """quantize_with_scale_zero_point (qarray.py:594-635) broadcasts a scale of any tiling; so does calibrate."""
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make(shape, O.BF16, seed=sum(shape))
+  s_np = O.round_to_bf16(np.abs(util.make_np(sshape, O.BF16, seed=9)) * 0.02 + 0.005)
+  z_np = util.rng(4).integers(-20, 20, sshape).astype(np.int8) if asym else None
+  z_t = None if z_np is None else torch.from_numpy(z_np).to(util.DEV)
+  q = qarray.quantize_with_scale_zero_point(x_t, qtype, util.to_gpu(s_np, O.BF16), z_t)
+  oq = O.quantize_with_scale_zero_point(O.FArr(x_np, O.BF16), qtype, O.FArr(s_np, O.BF16), z_np)
+  util.assert_qarray_equal(q, oq, 'static')
+  assert np.array_equal(util.f32np(qarray.dequantize(q)), O.dequantize(oq).v)
+  how = dict(qtype=qtype, channelwise_axes=[a for a in range(len(shape)) if sshape[a] == shape[a]],
+             tiled_axes={a: shape[a] // sshape[a] for a in range(len(shape)) if 1 < sshape[a] < shape[a]},
+             calibration_method='minmax' if asym else 'absmax')
+  got, want = qarray.calibrate(x_t, qarray.HowToQuantize(**how)), O.calibrate(O.FArr(x_np, O.BF16), O.HowToQuantize(**how))
+  for k in want:
+    assert np.array_equal(util.f32np(got[k]), want[k].v), k
