@@ -85,12 +85,13 @@ _INT_QTYPES = (INT8, INT4)
 
 def round_to_bf16(x) -> np.ndarray:
   """RNE f32 -> bf16, returned as f32 holding bf16-representable values."""
+  shape = np.shape(x)  # ascontiguousarray turns a 0-d array into one of shape (1,)
   x = np.ascontiguousarray(x, dtype=np.float32)
   u = x.view(np.uint32).astype(np.uint64)
   bias = ((u >> 16) & 1) + 0x7FFF
   r = ((u + bias) & 0xFFFF0000).astype(np.uint32)
   r = np.where(np.isnan(x), np.uint32(0x7FC00000), r).astype(np.uint32)
-  return r.view(np.float32).reshape(x.shape)
+  return r.view(np.float32).reshape(shape)
 
 
 def rnd(x, dtype: str) -> np.ndarray:
@@ -560,7 +561,7 @@ def _dot_general_f64(lhs, rhs, dimension_numbers) -> np.ndarray:
   l2 = l.reshape(b, -1, k)
   r2 = r.reshape(b, k, -1)
   out = np.matmul(l2, r2)
-  return out.reshape(*bshape, *lfree, *rfree)
+  return out.reshape(tuple(bshape) + tuple(lfree) + tuple(rfree))
 
 
 def _transpose_array(a: np.ndarray, transpose) -> np.ndarray:

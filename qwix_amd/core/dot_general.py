@@ -136,7 +136,7 @@ class _Canon:
         _lib.call('qwix_hip_transpose_q', nat.data.data_ptr(), _lib.INT4, self.K, self.N, dst.data_ptr(),
                   _lib.stream_of(dst))
         return dst, True
-      raise NotImplementedError(f'int4 weight layout {v} cannot be brought to K-contiguous form')
+      raise qarray.Int4LayoutError(f'int4 weight layout {v} cannot be brought to K-contiguous form')
     p = v.permute(*order)
     if p.is_contiguous():
       return p.reshape(self.N, self.K), False
@@ -209,7 +209,7 @@ def _index_batch(x, axes: Sequence[int], idx: Sequence[int]):
   def take(t):
     if isinstance(t, Int4Tensor):  # index the packed bytes; the pairs must not run along a batch axis
       if t.packed_axis in axes:
-        raise NotImplementedError('int4 values packed along a batch axis are not supported')
+        raise qarray.Int4LayoutError('int4 values packed along a batch axis are not supported')
       sel = [slice(None)] * t.ndim
       for a, i in zip(axes, idx):
         sel[a] = i
@@ -902,9 +902,22 @@ def dot_general(lhs: MaybeQ, rhs: MaybeQ, dimension_numbers: DotDimensionNumbers
   empty = _degenerate(lhs, rhs, dimension_numbers, preferred_element_type)
   if empty is not None:
     return empty
-  if _use_fast_path(lhs, rhs, dimension_numbers):
-    return _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type, **kwargs)
-  return _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type, **kwargs)
+  fn = _fast_dot_general if _use_fast_path(lhs, rhs, dimension_numbers) else _slow_dot_general
+  try:
+    return fn(lhs, rhs, dimension_numbers, preferred_element_type=preferred_element_type, **kwargs)
+  except qarray.Int4LayoutError:
+    # packed int4 values that no kernel reads where they lie (pairs along a batch axis, or along an axis that is
+    # neither the last contracting one nor the last free one): the same integers as int8, one byte each
+    wl, wr = _widen_int4(lhs), _widen_int4(rhs)
+    if wl is lhs and wr is rhs:
+      raise
+    return fn(wl, wr, dimension_numbers, preferred_element_type=preferred_element_type, **kwargs)
+
+
+def _widen_int4(x):
+  if isinstance(x, QArray) and isinstance(x.qvalue, Int4Tensor):
+    return QArray(x.qvalue.unpack().contiguous(), x.scale, x.zero_point, numerics.INT8)
+  return x
 
 
 MaybeQ = Any

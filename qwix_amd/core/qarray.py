@@ -31,6 +31,10 @@ from qwix_amd.core import numerics
 # ------------------------------------------------------------------------------------------
 
 
+class Int4LayoutError(NotImplementedError):
+  """Packed int4 values in a layout that a kernel cannot read in place; callers may widen them to int8 and go on."""
+
+
 class Int4Tensor:
   """Packed int4 values: `data` (uint8) has the logical shape with `packed_axis` halved.
 
@@ -820,7 +824,7 @@ def physical_layout(qa: QArray) -> tuple[_Plan, int, torch.Tensor]:
       return plan, _lib.LAYOUT_REDUCE_MINOR, phys
   if not is4:  # any other strided view (a slice of a batch, a transposed copy): one compaction
     return plan, _lib.LAYOUT_NATURAL, data.contiguous()
-  raise NotImplementedError(
+  raise Int4LayoutError(
       f'int4 values of shape {shape} with strides {tuple(data.stride())} are neither row-major nor '
       'reduce-minor; make them contiguous first.'
   )

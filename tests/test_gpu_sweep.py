@@ -269,6 +269,73 @@ def test_sweep_dot_general_types_and_tiles(seed):
 
 
 # ---------------------------------------------------------------------------------------------------------------
+# general dimension numbers: batch axes, several contracting axes, any axis order (dot_general.py:79-132)
+# ---------------------------------------------------------------------------------------------------------------
+
+
+def _dimension_number_cases(seed, count):
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  r = util.rng(seed)
+  for c in range(count):
+    nb, nc = int(r.choice([0, 0, 1, 2])), int(r.choice([1, 1, 2]))
+    nlf, nrf = int(r.choice([0, 1, 1, 2])), int(r.choice([0, 1, 1, 2]))
+    bs = [int(r.choice([1, 2, 3])) for _ in range(nb)]
+    cs = [int(r.choice([16, 32, 64, 128, 256])) for _ in range(nc)]
+    lf = [int(r.choice([1, 5, 16, 40])) for _ in range(nlf)]
+    rf = [int(r.choice([2, 8, 24, 64])) for _ in range(nrf)]
+    l_axes = [('b', i) for i in range(nb)] + [('c', i) for i in range(nc)] + [('f', i) for i in range(nlf)]
+    r_axes = [('b', i) for i in range(nb)] + [('c', i) for i in range(nc)] + [('f', i) for i in range(nrf)]
+    l_axes = [l_axes[i] for i in r.permutation(len(l_axes))]
+    r_axes = [r_axes[i] for i in r.permutation(len(r_axes))]
+    size = lambda kind, i, free: {'b': bs, 'c': cs, 'f': free}[kind][i]
+    lshape = tuple(size(k, i, lf) for k, i in l_axes)
+    rshape = tuple(size(k, i, rf) for k, i in r_axes)
+    dn = ((tuple(l_axes.index(('c', i)) for i in range(nc)), tuple(r_axes.index(('c', i)) for i in range(nc))),
+          (tuple(l_axes.index(('b', i)) for i in range(nb)), tuple(r_axes.index(('b', i)) for i in range(nb))))
+    dt = O.BF16 if r.random() < 0.7 else O.F32
+    lq = str(r.choice(['int8', 'int8', 'int4', O.E4M3]))
+    rq = lq if lq == O.E4M3 else str(r.choice(['int8', 'int8', 'int4']))
+    tile = int(r.choice([0, 0, 16, 64, 128]))
+    if tile and cs[-1] % tile:
+      tile = 0
+    asym = lq != O.E4M3 and r.random() < 0.2
+    if (lq == 'int4' and lshape[-1] % 2) or (rq == 'int4' and rshape[-1] % 2):
+      continue  # packed int4 storage pairs elements of the last axis
+
+    def thunk(lshape=lshape, rshape=rshape, dn=dn, dt=dt, lq=lq, rq=rq, tile=tile, asym=asym, last_k=cs[-1], c=c):
+      x_np, x_t = util.make(lshape, dt, seed=c)
+      w_np, w_t = util.make(rshape, dt, seed=c + 999, scale=0.05)
+      if asym:
+        x_np = O.rnd(x_np + 0.5, dt)
+        x_t = util.to_gpu(x_np, dt)
+      kw = dict(dimension_numbers=dn, ndims=(len(lshape), len(rshape)), tile_size=tile or None)
+      cm = 'minmax' if asym else 'absmax'
+      xq = qarray.quantize(x_t, dg.get_how_to_quantize(for_lhs=True, qtype=lq, calibration_method=cm, **kw))
+      wq = qarray.quantize(w_t, dg.get_how_to_quantize(for_lhs=False, qtype=rq, **kw))
+      oxq = O.quantize(O.FArr(x_np, dt), O.dg_get_how_to_quantize(for_lhs=True, qtype=lq, calibration_method=cm, **kw))
+      owq = O.quantize(O.FArr(w_np, dt), O.dg_get_how_to_quantize(for_lhs=False, qtype=rq, **kw))
+      util.assert_qarray_equal(xq, oxq, 'lhs')
+      util.assert_qarray_equal(wq, owq, 'rhs')
+      got, want = util.f32np(dg.dot_general(xq, wq, dn, exact=True)), O.dot_general(oxq, owq, dn).v
+      assert got.shape == want.shape, (got.shape, want.shape)
+      groups = last_k // tile if tile else 1
+      if lq == O.E4M3 or (tile and tile < 128 and groups > 1):
+        assert _rel(got, want) < (2e-2 if dt == O.BF16 else 2e-3)
+      elif groups > 1 and dt == O.F32:
+        assert _rel(got, want) < 1e-5
+      else:
+        _exact(got, want)
+
+    yield f'dimension numbers {lshape} x {rshape} {dn} {dt} {lq}x{rq} tile={tile} asym={asym}', thunk
+
+
+@pytest.mark.parametrize('seed', [3, 17])
+def test_sweep_dimension_numbers(seed):
+  _run(_dimension_number_cases(seed, 250))
+
+
+# ---------------------------------------------------------------------------------------------------------------
 # einsum, ragged_dot
 # ---------------------------------------------------------------------------------------------------------------
 
