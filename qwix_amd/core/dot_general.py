@@ -120,7 +120,10 @@ class _Canon:
     v = v if v.is_contiguous() else v.contiguous()
     if v.data_ptr() % 16:  # a contiguous view that starts inside a 16-byte unit: the kernels load 16 bytes per lane
       v = v.clone()
-    return v.reshape(self.M, self.K)
+    v = v.reshape(self.M, self.K)
+    if self.M == 1 and v.stride(0) != self.K:  # a single row keeps whatever pitch its parent had
+      v = v.as_strided((1, self.K), (self.K, 1))
+    return v
 
   def rhs_values(self, rhs) -> tuple[torch.Tensor, bool]:
     """(N, K) K-contiguous storage (for int4: (N, K/2) bytes), is_int4."""
@@ -642,9 +645,15 @@ def _bf16_gemm_limits_ok(m: int, lda: int, n: int, ldb_bytes: int) -> bool:
 def _aligned_rows(x: torch.Tensor) -> torch.Tensor:
   """The activation as the kernels want it: unit stride along K, row pitch a multiple of 8 elements, 16-byte aligned
   base.  A view that is not (a slice that starts inside a row) is copied."""
-  if x.stride(-1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0:
-    return x
-  return x.contiguous()
+  if x.stride(-1) == 1 and x.data_ptr() % 16 == 0:
+    if x.stride(0) % 8 == 0:
+      return x
+    if x.shape[0] == 1:  # the pitch of a single row means nothing: state a valid one
+      return x.as_strided(tuple(x.shape), (x.shape[1], 1))
+  # (`contiguous()` would hand a single row back as it is, whatever its pitch and base)
+  y = torch.empty(tuple(x.shape), dtype=x.dtype, device=x.device)
+  y.copy_(x)
+  return y
 
 
 # Rows up to which the fused weight-only kernel (one pass over the weight per 16 or 32 rows) is used; above

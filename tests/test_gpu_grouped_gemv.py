@@ -650,3 +650,20 @@ def test_weight_only_prefill_on_hip_kernels(M, K, N, case):
   deq = O.dequantize(owq)
   want_w = O.round_to_bf16(deq.v) if sdt == torch.float32 else deq.v
   assert np.array_equal(util.f32np(w).T, want_w)
+
+
+@pytest.mark.parametrize('col0', [0, 8, 1])
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+def test_decode_call_on_one_row_of_a_wider_matrix(wq_type, col0):
+  """A single-row view keeps the pitch and the base of its parent (torch calls it contiguous whatever they are): the
+  decode kernel gets a 16-byte aligned row with a valid pitch, by restating the pitch or by one copy."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  g = torch.Generator().manual_seed(5)
+  big = torch.randn(7, 1100, generator=g).to(torch.bfloat16).to(util.DEV)   # rows 2200 bytes apart
+  w = (torch.randn(1024, 520, generator=g) * 0.05).to(torch.bfloat16).to(util.DEV)
+  wq = qarray.quantize(w, qarray.HowToQuantize(qtype=wq_type, channelwise_axes=[1], tiled_axes={0: 128}))
+  dn = (((1,), (0,)), ((), ()))
+  row = big[3:4, col0:col0 + 1024]
+  assert row.is_contiguous() and row.stride(0) == 1100
+  assert torch.equal(dg.dot_general(row, wq, dn), dg.dot_general(row.clone(), wq, dn))
