@@ -863,6 +863,78 @@ def ragged_dot(lhs, rhs, group_sizes, preferred_element_type=None):
   return fn(lhs, rhs, group_sizes, preferred_element_type)
 
 
+def _take(x, axis: int, index):
+  """x[..., index, ...] along `axis` for an array, FArr or QArray (index: a slice keeps the axis, an int
+  drops it); scales and zero points with one entry along the axis are kept whole."""
+  def cut(a, n):
+    if a is None:
+      return None
+    if a.shape[axis] == 1:
+      idx = slice(None) if isinstance(index, slice) else 0
+    else:
+      assert a.shape[axis] == n, 'scales tiled along a ragged / group axis are not restated'
+      idx = index
+    return a[(slice(None),) * axis + (idx,)]
+
+  n = x.shape[axis]
+  if isinstance(x, QArray):
+    zp = cut(x.zero_point, n)
+    return QArray(cut(x.qvalue, n), FArr(cut(x.scale.v, n), x.scale.dtype), zp, x.qtype)
+  if isinstance(x, FArr):
+    return FArr(cut(x.v, n), x.dtype)
+  return cut(x, n)
+
+
+def ragged_dot_general(lhs, rhs, group_sizes, dot_dimension_numbers, lhs_ragged_dimension: int,
+                       rhs_group_dimension: int, preferred_element_type=None):
+  """ragged_dot.py:123-313 for dimension numbers whose ragged axis is the only free axis of the lhs (batch
+  axes, several contracting axes, any axis order; the reference's own non-basic case is
+  tests/_src/core/ragged_dot_test.py:255-275).
+
+  The reference scales the group-wise accumulator of lax.ragged_dot_general by the lhs scale and then by the
+  rhs scale that a ragged dot of ones has expanded over the rows (:32-57, 196-220), and sums the tile axes
+  last (:222-224).  Row by row that is the arithmetic of dot_general on the row's group: restated here as one
+  dot_general per group on slices (rows of the group along the ragged axis, the group's slice of the rhs with
+  the group axis dropped), written to those rows of a zero result of shape (batch, ragged, rhs free).  For the
+  dimension numbers of ragged_dot it equals fast_ragged_dot / slow_ragged_dot bit for bit (tests)."""
+  (lca, rca), (lba, rba) = dot_dimension_numbers
+  r, g_ax = lhs_ragged_dimension, rhs_group_dimension
+  lfree = [a for a in range(len(lhs.shape)) if a not in lca and a not in lba]
+  assert lfree == [r], 'the ragged axis has to be the only free axis of the lhs'
+  drop = lambda a: a - (a > g_ax)
+  dn = ((tuple(lca), tuple(drop(a) for a in rca)), (tuple(lba), tuple(drop(a) for a in rba)))
+  fast = True
+  for operand in (lhs, rhs):
+    if isinstance(operand, QArray):
+      if operand.zero_point is not None:
+        fast = False
+    elif isinstance(operand, FArr):
+      fast = False
+  fn = fast_dot_general if fast else slow_dot_general
+  m = lhs.shape[r]
+  out, out_t = None, None
+  start = 0
+  parts = []
+  for g, size in enumerate(group_sizes):
+    stop = min(start + max(int(size), 0), m)
+    if stop > start:
+      part = fn(_take(lhs, r, slice(start, stop)), _take(rhs, g_ax, g), dn, preferred_element_type)
+      parts.append((start, stop, part))
+    start = stop
+  _, res_t = get_accumulator_and_result_type(lhs, rhs, preferred_element_type=preferred_element_type)
+  if not fast:
+    lt = lhs.scale.dtype if isinstance(lhs, QArray) else lhs.dtype
+    rt = rhs.scale.dtype if isinstance(rhs, QArray) else rhs.dtype
+    res_t = preferred_element_type or promote(lt, rt)
+  rfree = [d for a, d in enumerate(rhs.shape) if a != g_ax and a not in rca and a not in rba]
+  shape = tuple(lhs.shape[a] for a in lba) + (m,) + tuple(rfree)
+  out = np.zeros(shape, np.int32 if res_t == INT32 else np.float32)
+  for start, stop, part in parts:
+    v = part if isinstance(part, np.ndarray) else part.v
+    out[(slice(None),) * len(lba) + (slice(start, stop),)] = v
+  return out if res_t == INT32 else FArr(out, res_t)
+
+
 # ----------------------------------------------------------------------------
 # einsum_info.py / einsum.py (binary einsum)
 # ----------------------------------------------------------------------------

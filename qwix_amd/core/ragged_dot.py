@@ -8,8 +8,9 @@ lhs is (M, K), rhs is (G, K, N); the rows of lhs form G consecutive groups of `g
 and group g is multiplied with rhs[g].  `group_sizes` stays in device memory: the kernel reads it,
 so the quantized path never synchronises with the host.  Rows past the last group come out as
 zeros.  int4 expert weights and the dequantize-first path run the dense kernels of dot_general group by
-group (these need the group boundaries on the host).  Only the dimension numbers of `ragged_dot` are
-supported; others raise.
+group (these need the group boundaries on the host).  Other dimension numbers with the ragged axis as the only
+free axis of the lhs and one group axis on the rhs (batch axes, several contracting axes, any axis order) run one
+dense contraction per group (`_general_ragged`); a ragged contracting or batch axis raises.
 """
 from __future__ import annotations
 
@@ -120,11 +121,125 @@ def _group_by_group(fn, lhs, rhs, group_sizes, res_t, **kwargs) -> torch.Tensor:
   return out
 
 
+def _is_basic(dn: RaggedDotDimensionNumbers) -> bool:
+  (lca, rca), (lba, rba) = dn.dot_dimension_numbers
+  return (tuple(lca), tuple(rca), tuple(lba), tuple(rba), tuple(dn.lhs_ragged_dimensions),
+          tuple(dn.rhs_group_dimensions)) == ((1,), (1,), (), (), (0,), (0,))
+
+
+def _narrow(x, axis: int, start: int, stop: int):
+  """Positions start .. stop - 1 along `axis` of a tensor or QArray: views; scales and zero points are cut where they
+  have one entry per position and kept where they have one in all."""
+  full = x.shape[axis]
+
+  def cut(t):
+    if t is None or t.shape[axis] == 1:
+      return t
+    if t.shape[axis] != full:
+      raise NotImplementedError('scales tiled along the ragged axis cannot be sliced by groups')
+    return t.narrow(axis, start, stop - start)
+
+  def values(q):
+    if isinstance(q, Int4Tensor):
+      if q.packed_axis == axis:
+        raise NotImplementedError('int4 values packed along the ragged axis cannot be sliced by groups')
+      shape = tuple(stop - start if a == axis else d for a, d in enumerate(q.shape))
+      return Int4Tensor(q.data.narrow(axis, start, stop - start), shape, q.packed_axis)
+    return q.narrow(axis, start, stop - start)
+
+  if isinstance(x, QArray):
+    return QArray(qvalue=values(x.qvalue), scale=cut(x.scale), zero_point=cut(x.zero_point), qtype=x.qtype)
+  return values(x)
+
+
+def _select(w, axis: int, g: int):
+  """Entry g along `axis` of a tensor or QArray, the axis removed: views."""
+  full = w.shape[axis]
+
+  def pick(t):
+    if t is None:
+      return None
+    if t.shape[axis] not in (1, full):
+      raise NotImplementedError('scales tiled along the group axis cannot be sliced by groups')
+    return t.select(axis, g if t.shape[axis] > 1 else 0)
+
+  def values(q):
+    if isinstance(q, Int4Tensor):
+      if q.packed_axis == axis:
+        raise NotImplementedError('int4 weights packed along the group axis cannot be sliced by groups')
+      shape = tuple(d for a, d in enumerate(q.shape) if a != axis)
+      return Int4Tensor(q.data.select(axis, g), shape, q.packed_axis - (q.packed_axis > axis))
+    return q.select(axis, g)
+
+  if isinstance(w, QArray):
+    return QArray(qvalue=values(w.qvalue), scale=pick(w.scale), zero_point=pick(w.zero_point), qtype=w.qtype)
+  return values(w)
+
+
+def _check_general(dn: RaggedDotDimensionNumbers, lhs, rhs, group_sizes, group_offset):
+  """The ragged axis is a free axis of the lhs (its rows form the groups) and the rhs has one group axis: the first of
+  the three modes of lax.ragged_dot_general, with batch axes, several contracting axes and any axis order.  Returns
+  (ragged axis, group axis, dimension numbers of one group's dense contraction)."""
+  (lca, rca), (lba, rba) = dn.dot_dimension_numbers
+  lca, rca, lba, rba = ([int(a) for a in x] for x in (lca, rca, lba, rba))
+  if group_offset is not None:
+    raise NotImplementedError('group_offset is not supported')
+  if len(dn.lhs_ragged_dimensions) != 1 or len(dn.rhs_group_dimensions) != 1:
+    raise NotImplementedError(f'one ragged axis on the lhs and one group axis on the rhs are supported, got {dn}')
+  ragged, group = int(dn.lhs_ragged_dimensions[0]), int(dn.rhs_group_dimensions[0])
+  if ragged in lca or ragged in lba:
+    raise NotImplementedError('a ragged contracting or batch axis (the modes without an rhs group axis) is not supported')
+  if group in rca or group in rba:
+    raise ValueError(f'the rhs group axis {group} cannot be a contracting or batch axis')
+  lfree = [a for a in range(len(lhs.shape)) if a not in lca and a not in lba]
+  if lfree != [ragged]:
+    raise NotImplementedError(f'the ragged axis has to be the only free axis of the lhs, got free axes {lfree}')
+  if len(lca) != len(rca) or len(lba) != len(rba):
+    raise ValueError(f'contracting / batch axes differ in number: {dn}')
+  for l, r in list(zip(lca, rca)) + list(zip(lba, rba)):
+    if lhs.shape[l] != rhs.shape[r]:
+      raise ValueError(f'sizes of lhs axis {l} and rhs axis {r} differ: {tuple(lhs.shape)} and {tuple(rhs.shape)}')
+  if group_sizes.ndim != 1 or group_sizes.shape[0] != rhs.shape[group]:
+    raise ValueError(f'group_sizes must have one entry per group: {tuple(group_sizes.shape)} vs G={rhs.shape[group]}')
+  if group_sizes.dtype not in (torch.int32, torch.int64):
+    raise TypeError(f'group_sizes must be an integer tensor, got {group_sizes.dtype}')
+  drop = lambda a: a - (a > group)
+  return ragged, group, ((tuple(lca), tuple(drop(a) for a in rca)), (tuple(lba), tuple(drop(a) for a in rba)))
+
+
+def _general_ragged(fn, lhs, rhs, group_sizes, dimension_numbers, res_t, group_offset, **kwargs) -> torch.Tensor:
+  """Dimension numbers other than ragged_dot's (ragged_dot.py:123-226 hands any to lax.ragged_dot_general): one dense
+  contraction per non-empty group on views of the operands -- the rows of the group along the ragged axis against
+  that group's slice of the rhs -- written to the group's rows of the result (batch axes, the ragged axis, the free
+  axes of the rhs).  Per element the same arithmetic as the reference's: the group's accumulator scaled by the row's
+  lhs scale, then by the group's rhs scale, tile partials summed last.  The group boundaries are needed on the host."""
+  ragged, group, dn = _check_general(dimension_numbers, lhs, rhs, group_sizes, group_offset)
+  (_, _), (lba, rba) = dn
+  M = lhs.shape[ragged]
+  rfree = [d for a, d in enumerate(rhs.shape) if a != group and (a - (a > group)) not in dn[0][1] and (a - (a > group)) not in rba]
+  dev = (lhs.scale if isinstance(lhs, QArray) else lhs).device
+  out = torch.zeros([lhs.shape[a] for a in lba] + [M] + rfree, dtype=res_t, device=dev)
+  start = 0
+  for g, size in enumerate(group_sizes.tolist()):
+    stop = min(start + max(int(size), 0), M)
+    if stop > start:
+      part = fn(_narrow(lhs, ragged, start, stop), _select(rhs, group, g), dn, preferred_element_type=res_t, **kwargs)
+      out.narrow(len(lba), start, stop - start).copy_(part)
+    start = stop
+  return out
+
+
 def _fast_ragged_dot_general(lhs, rhs, group_sizes, dimension_numbers=_BASIC_RAGGED_DOT_DIMENSION_NUMBERS,
                              precision=None, preferred_element_type=None, group_offset=None) -> torch.Tensor:
   """Contract the quantized values group by group on the matrix cores, then scale:
   out = ((acc * lhs_scale) * rhs_scale[group of the row]), tile partials summed last."""
   del precision
+  if not _is_basic(dimension_numbers):
+    for x in (lhs, rhs):
+      if isinstance(x, QArray) and x.zero_point is not None:
+        raise NotImplementedError('zero-point operands take the dequantize-first ragged dot')
+    _, res_t = qarray.get_accumulator_and_result_type(lhs, rhs, preferred_element_type=preferred_element_type)
+    return _general_ragged(_dot_general._fast_dot_general, lhs, rhs, group_sizes, dimension_numbers, res_t, group_offset)
   _check_basic(dimension_numbers, lhs, rhs, group_sizes, group_offset)
   for x in (lhs, rhs):
     if isinstance(x, QArray) and x.zero_point is not None:
@@ -203,11 +318,17 @@ def _slow_ragged_dot_general(lhs, rhs, group_sizes, dimension_numbers=_BASIC_RAG
   dequantize + bf16 MFMA kernel up to 256 rows, dequantize + the bf16 MFMA GEMM beyond), every other combination
   is dequantized by the HIP kernel and contracted by the float GEMM."""
   del precision
-  _check_basic(dimension_numbers, lhs, rhs, group_sizes, group_offset)
+  basic = _is_basic(dimension_numbers)
+  if basic:
+    _check_basic(dimension_numbers, lhs, rhs, group_sizes, group_offset)
+  else:
+    _check_general(dimension_numbers, lhs, rhs, group_sizes, group_offset)
   if isinstance(lhs, QArray):
     lhs = qarray.dequantize(lhs)
   rhs_t = rhs.scale.dtype if isinstance(rhs, QArray) else rhs.dtype
   res_t = preferred_element_type or torch.promote_types(lhs.dtype, rhs_t)
+  if not basic:
+    return _general_ragged(_dot_general._slow_dot_general, lhs, rhs, group_sizes, dimension_numbers, res_t, group_offset)
   return _group_by_group(_dot_general._slow_dot_general, lhs, rhs, group_sizes, res_t)
 
 
@@ -216,10 +337,15 @@ def ragged_dot_general(lhs, rhs, group_sizes: torch.Tensor, dimension_numbers: R
   """Drop-in for lax.ragged_dot_general that accepts QArray operands."""
   if math.prod(lhs.shape) == 0 or math.prod(rhs.shape) == 0:
     # nothing to launch: no rows or no columns give an empty result, an empty contraction gives zeros
-    _check_basic(dimension_numbers, lhs, rhs, group_sizes, group_offset)
     _, res_t = qarray.get_accumulator_and_result_type(lhs, rhs, preferred_element_type=preferred_element_type)
     dev = (lhs.scale if isinstance(lhs, QArray) else lhs).device
-    return torch.zeros(lhs.shape[0], rhs.shape[2], dtype=res_t, device=dev)
+    if _is_basic(dimension_numbers):
+      _check_basic(dimension_numbers, lhs, rhs, group_sizes, group_offset)
+      return torch.zeros(lhs.shape[0], rhs.shape[2], dtype=res_t, device=dev)
+    ragged, group, dn = _check_general(dimension_numbers, lhs, rhs, group_sizes, group_offset)
+    rfree = [d for a, d in enumerate(rhs.shape)
+             if a != group and (a - (a > group)) not in dn[0][1] and (a - (a > group)) not in dn[1][1]]
+    return torch.zeros([lhs.shape[a] for a in dn[1][0]] + [lhs.shape[ragged]] + rfree, dtype=res_t, device=dev)
   use_fast_path = True
   for operand in (lhs, rhs):
     if isinstance(operand, QArray):

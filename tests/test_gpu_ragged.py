@@ -211,6 +211,77 @@ def test_ragged_dot_errors():
     qwix_amd.ragged_dot(xq, wq, _sizes((64, 64)))
   with pytest.raises(NotImplementedError, match='group_offset'):
     qwix_amd.ragged_dot(xq, wq, _sizes((64, 64, 0, 0)), group_offset=_sizes((0,)))
-  dn = rd.RaggedDotDimensionNumbers((((0,), (1,)), ((), ())), (1,), (0,))
-  with pytest.raises(NotImplementedError, match='dimension numbers'):
+  dn = rd.RaggedDotDimensionNumbers((((0,), (1,)), ((), ())), (1,), (0,))   # contracts 128 rows with K = 256
+  with pytest.raises(ValueError, match='differ'):
     qwix_amd.ragged_dot_general(xq, wq, _sizes((64, 64, 0, 0)), dn)
+  dn = rd.RaggedDotDimensionNumbers((((1,), (1,)), ((), ())), (0,), ())     # no group axis: another ragged mode
+  with pytest.raises(NotImplementedError, match='one group axis'):
+    qwix_amd.ragged_dot_general(xq, wq, _sizes((64, 64, 0, 0)), dn)
+
+
+def _rdn(dn, ragged, group):
+  from qwix_amd.core.ragged_dot import RaggedDotDimensionNumbers
+  return RaggedDotDimensionNumbers(dot_dimension_numbers=dn, lhs_ragged_dimensions=(ragged,), rhs_group_dimensions=(group,))
+
+
+GENERAL_CASES = [
+    # name, lhs shape, rhs shape, dot dimension numbers, ragged axis, group axis, sizes, lhs how, rhs how
+    ("the reference's non-basic case: a batch axis, K in tiles of 64, no free axis on the rhs", (8, 620, 256), (8, 4, 256),
+     (((2,), (2,)), ((0,), (0,))), 1, 1, (60, 120, 190, 250), dict(tiled_axes={2: 64}), dict(tiled_axes={2: 64})),
+    ('weights stored (G, N, K)', (200, 128), (3, 72, 128), (((1,), (2,)), ((), ())), 0, 0, (60, 0, 100),
+     dict(channelwise_axes=[0]), dict(channelwise_axes=[0, 1])),
+    ('rows last on the lhs, group axis in the middle of the rhs', (128, 300), (128, 5, 40), (((0,), (0,)), ((), ())), 1, 1,
+     (10, 0, 130, 1, 70), dict(channelwise_axes=[1]), dict(channelwise_axes=[1, 2])),
+    ('two contracting axes', (96, 4, 64), (3, 4, 64, 24), (((1, 2), (1, 2)), ((), ())), 0, 0, (30, 50, 16),
+     dict(channelwise_axes=[0]), dict(channelwise_axes=[0, 3])),
+    ('batch axis and K in tiles of 128', (2, 150, 256), (2, 4, 256, 136), (((2,), (2,)), ((0,), (0,))), 1, 1, (40, 0, 100, 10),
+     dict(channelwise_axes=[0, 1], tiled_axes={2: 128}), dict(channelwise_axes=[0, 1, 3], tiled_axes={2: 128})),
+]
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('name,lshape,rshape,dn,ragged,group,sizes,lhow,rhow', GENERAL_CASES)
+def test_ragged_dot_general_dimension_numbers(name, lshape, rshape, dn, ragged, group, sizes, lhow, rhow, dtype):
+  """Dimension numbers other than ragged_dot's (ragged_dot.py:123-226 passes any to lax.ragged_dot_general): the ragged
+  axis as the only free axis of the lhs, with batch axes, several contracting axes and any axis order.  int8: exact
+  sums and an elementwise epilogue, so bit for bit wherever a single K tile is scaled; f32 sums of tile partials at
+  1e-5."""
+  import qwix_amd
+  from qwix_amd.core import qarray
+  print('case ragged general', name, dtype, flush=True)
+  x_np, x_t = util.make(lshape, dtype, seed=len(name))
+  w_np, w_t = util.make(rshape, dtype, seed=len(name) + 1, scale=0.05)
+  xq, oxq = qarray.quantize(x_t, qarray.HowToQuantize(qtype='int8', **lhow)), O.quantize(O.FArr(x_np, dtype), O.HowToQuantize(qtype='int8', **lhow))
+  wq, owq = qarray.quantize(w_t, qarray.HowToQuantize(qtype='int8', **rhow)), O.quantize(O.FArr(w_np, dtype), O.HowToQuantize(qtype='int8', **rhow))
+  util.assert_qarray_equal(xq, oxq, 'lhs')
+  util.assert_qarray_equal(wq, owq, 'rhs')
+  out = qwix_amd.ragged_dot_general(xq, wq, _sizes(sizes), _rdn(dn, ragged, group))
+  want = O.ragged_dot_general(oxq, owq, sizes, dn, ragged, group)
+  assert out.dtype == util.TORCH_DT[want.dtype]
+  tiled = 'tiled_axes' in lhow or 'tiled_axes' in rhow
+  if tiled and dtype == O.F32:
+    np.testing.assert_allclose(util.f32np(out), want.v, rtol=0, atol=1e-5 * float(np.abs(want.v).max()))
+  elif tiled:
+    # bf16 partials: the reference rounds each three times before the f32 sum; the default mode keeps them in f32
+    np.testing.assert_allclose(util.f32np(out), want.v, rtol=0, atol=2e-2 * float(np.abs(want.v).max()))
+  else:
+    _check_exact(out, want)
+
+
+def test_ragged_dot_general_weight_only_and_errors():
+  import qwix_amd
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make((200, 128), O.BF16, seed=3)
+  w_np, w_t = util.make((3, 72, 128), O.BF16, seed=4, scale=0.05)
+  how = dict(qtype='int8', channelwise_axes=[0, 1])
+  wq, owq = qarray.quantize(w_t, qarray.HowToQuantize(**how)), O.quantize(O.FArr(w_np, O.BF16), O.HowToQuantize(**how))
+  dn = (((1,), (2,)), ((), ()))
+  out = qwix_amd.ragged_dot_general(x_t, wq, _sizes((60, 0, 100)), _rdn(dn, 0, 0))     # float lhs: dequantize first
+  want = O.ragged_dot_general(O.FArr(x_np, O.BF16), owq, (60, 0, 100), dn, 0, 0)
+  np.testing.assert_allclose(util.f32np(out), want.v, rtol=1e-2, atol=1e-2 * float(np.abs(want.v).max()))
+  assert np.all(util.f32np(out)[160:] == 0)
+  with pytest.raises(NotImplementedError, match='ragged contracting or batch axis'):
+    qwix_amd.ragged_dot_general(x_t, wq, _sizes((60, 0, 100)), _rdn(dn, 1, 0))
+  x3 = torch.zeros(4, 200, 128, dtype=torch.bfloat16, device=util.DEV)
+  with pytest.raises(NotImplementedError, match='only free axis'):
+    qwix_amd.ragged_dot_general(x3, wq, _sizes((60, 0, 100)), _rdn((((2,), (2,)), ((), ())), 1, 0))

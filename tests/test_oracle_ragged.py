@@ -114,3 +114,38 @@ def test_dispatch_and_slow_path_agree_with_fast():
   xz = O.quantize(x, O.HowToQuantize(qtype='int8', calibration_method='minmax'))
   assert np.array_equal(O.ragged_dot(xz, wq, (64, 64, 0, 0)).v, O.slow_ragged_dot(xz, wq, (64, 64, 0, 0)).v)
   assert np.array_equal(O.ragged_dot(x, wq, (64, 64, 0, 0)).v, O.slow_ragged_dot(x, wq, (64, 64, 0, 0)).v)
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('name,lhs_how,rhs_how', HOWS[:4])
+@pytest.mark.parametrize('sizes', [(128, 100, 0, 28), (10, 20, 30, 68), (5, 0, 7, 3)])
+def test_general_dimension_numbers_reduce_to_ragged_dot(name, lhs_how, rhs_how, sizes, dtype):
+  """ragged_dot_general on the dimension numbers of ragged_dot is fast_ragged_dot, bit for bit (the two are written
+  independently: a masked sum with expanded scales against one dot_general per group)."""
+  xq, wq = _operands(dtype, 11, lhs_how, rhs_how)
+  want = O.ragged_dot(xq, wq, sizes)
+  got = O.ragged_dot_general(xq, wq, sizes, (((1,), (1,)), ((), ())), 0, 0)
+  assert got.dtype == want.dtype and np.array_equal(got.v, want.v)
+
+
+def test_general_dimension_numbers_with_a_batch_axis_and_tiles():
+  """The reference's non-basic case (tests/_src/core/ragged_dot_test.py:255-275): lhs (32, 620, 256) and rhs (32, 4, 256)
+  int8 in tiles of 64 along K, batch axis 0, ragged axis 1, group axis 1, groups (60, 120, 190, 250).  Its inputs
+  come from jax.random, so the reference's bound is what is checked: relative mean absolute error against the float
+  result below 0.04 (a smaller batch keeps the CPU run short); and batch element by batch element the result is the
+  basic ragged dot of that element."""
+  dn, sizes = (((2,), (2,)), ((0,), (0,))), (60, 120, 190, 250)
+  x = util.make_np((4, 620, 256), O.F32, 5)
+  w = util.make_np((4, 4, 256), O.F32, 6)
+  how = O.HowToQuantize(qtype='int8', tiled_axes={2: 64})
+  xq, wq = O.quantize(O.FArr(x, O.F32), how), O.quantize(O.FArr(w, O.F32), how)
+  got = O.ragged_dot_general(xq, wq, sizes, dn, 1, 1)
+  assert got.v.shape == (4, 620)
+  rows_group = np.repeat(np.arange(4), sizes)
+  want_fp = np.einsum('bmk,bmk->bm', x.astype(np.float64), w.astype(np.float64)[:, rows_group, :])
+  assert np.abs(got.v - want_fp).mean() / np.abs(want_fp).mean() < 0.04
+  for b in range(4):
+    assert xq.scale.v.shape == (1, 1, 4) and wq.scale.v.shape == (1, 1, 4)      # one scale per K tile
+    xb = O.QArray(xq.qvalue[b], O.FArr(xq.scale.v[0], O.F32), None, 'int8')
+    wb = O.QArray(wq.qvalue[b][:, :, None], O.FArr(wq.scale.v[0][:, :, None], O.F32), None, 'int8')   # (G, K, N=1)
+    assert np.array_equal(O.ragged_dot(xb, wb, sizes).v[:, 0], got.v[b])
