@@ -435,6 +435,25 @@ def _tile_by_tile(lhs, rhs, dimension_numbers, tiled, preferred_element_type, ex
   return total.to(cur).to(res_t)
 
 
+# K-sums of a weight's quantized values (the zero-point correction of an asymmetric activation, dot_general.py:228-253,
+# multiplies them with the activation's zero points): weights are static, so the sums are kept per values tensor while it
+# is alive and unchanged (identity + torch version counter; entries leave with their tensor).
+_KSUM_CACHE: dict = {}
+
+
+def _weight_ksums(values_owner, b: torch.Tensor, key_extra: tuple, compute) -> torch.Tensor:
+  """`values_owner`: the tensor object the weight's QArray holds (its identity and version key the entry; `b` may be a
+  re-laid-out copy of it); `compute()` launches the sum kernel and returns the result."""
+  store = values_owner.data if isinstance(values_owner, Int4Tensor) else values_owner
+  key = (id(store),) + key_extra
+  hit = _KSUM_CACHE.get(key)
+  if hit is not None and hit[0]() is store and hit[1] == store._version:
+    return hit[2]
+  out = compute()
+  _KSUM_CACHE[key] = (weakref.ref(store, lambda _, k=key: _KSUM_CACHE.pop(k, None)), store._version, out)
+  return out
+
+
 def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, *, exact: bool = False,
                       return_accumulators: bool = False, _partial_dtype=None, **kwargs) -> torch.Tensor:
   """Contract the quantized values on the matrix cores, then scale: out = ((acc * sx) * sy).
@@ -515,8 +534,12 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
         raise NotImplementedError('raw accumulators are not returned for zero-point operands')
       if lzp is not None:
         zu = c.lhs_zero_point(lhs)[0].reshape(c.M)
-        zv = torch.empty(c.N, dtype=torch.int32, device=dev)
-        _lib.call('qwix_hip_ksum_i8', b.data_ptr(), b.stride(0), c.N, K, zv.data_ptr(), st)
+
+        def ksum():
+          zv = torch.empty(c.N, dtype=torch.int32, device=dev)
+          _lib.call('qwix_hip_ksum_i8', b.data_ptr(), b.stride(0), c.N, K, zv.data_ptr(), st)
+          return zv
+        zv = _weight_ksums(rhs.qvalue, b, (tuple(c.rca), tuple(c.rfree), K), ksum)
       else:
         zv = c.rhs_zero_point(rhs)[0].reshape(c.N)
         zu = torch.empty(c.M, dtype=torch.int32, device=dev)
@@ -559,8 +582,12 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
     if lzp is not None:
       zu, gz = c.lhs_zero_point(lhs)                       # (M, gz)
       zu_strides = (gz, 1 if gz > 1 else 0)
-      zv = torch.empty(c.N, ngroups, dtype=torch.int32, device=dev)
-      _lib.call('qwix_hip_ksum_groups', b.data_ptr(), bq, b.stride(0), c.N, c.K, group, zv.data_ptr(), st)
+
+      def ksum():
+        zv = torch.empty(c.N, ngroups, dtype=torch.int32, device=dev)
+        _lib.call('qwix_hip_ksum_groups', b.data_ptr(), bq, b.stride(0), c.N, c.K, group, zv.data_ptr(), st)
+        return zv
+      zv = _weight_ksums(rhs.qvalue, b, (tuple(c.rca), tuple(c.rfree), group), ksum)
       zv_strides = (ngroups, 1)
     else:
       zv, gz = c.rhs_zero_point(rhs)                       # (gz, N)

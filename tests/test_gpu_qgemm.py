@@ -146,6 +146,41 @@ def test_int8_gemm_with_zero_point_operand_bit_exact(M, K, N, side, dtype):
     assert np.abs(got - ref).mean() / np.abs(ref).mean() < 0.05
 
 
+@pytest.mark.parametrize('tile', [None, 128])
+def test_weight_k_sums_are_kept_per_weight_and_follow_in_place_updates(tile):
+  """The K-sums of a static weight (the other factor of an asymmetric activation's correction term) are computed once
+  per weight tensor; a weight changed in place (same tensor object, new contents) gets new sums."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make((64, 256), O.BF16, seed=71)
+  x_t = x_t + 0.75
+  x_np = util.f32np(x_t)
+  w_np, w_t = util.make((256, 136), O.BF16, seed=72, scale=0.02)
+  lkw = dict(qtype='int8', channelwise_axes=[0], tiled_axes={1: tile} if tile else {}, calibration_method='minmax')
+  rkw = dict(qtype='int8', channelwise_axes=[1], tiled_axes={0: tile} if tile else {})
+  xq, oxq = qarray.quantize(x_t, qarray.HowToQuantize(**lkw)), O.quantize(O.FArr(x_np, O.BF16), O.HowToQuantize(**lkw))
+  wq, owq = qarray.quantize(w_t, qarray.HowToQuantize(**rkw)), O.quantize(O.FArr(w_np, O.BF16), O.HowToQuantize(**rkw))
+  calls = []
+  real = dg._lib.call
+  def counting(name, *a):
+    calls.append(name)
+    return real(name, *a)
+  dg._lib.call = counting
+  try:
+    first = util.f32np(dg.dot_general(xq, wq, DN, exact=True))
+    again = util.f32np(dg.dot_general(xq, wq, DN, exact=True))
+    n_sums = sum(c.startswith('qwix_hip_ksum') for c in calls)
+    wq.qvalue.neg_()                                          # in place: same tensor, other values
+    owq2 = O.QArray(-owq.qvalue, owq.scale, None, owq.qtype)
+    third = util.f32np(dg.dot_general(xq, wq, DN, exact=True))
+  finally:
+    dg._lib.call = real
+  assert n_sums == 1, calls
+  assert sum(c.startswith('qwix_hip_ksum') for c in calls) == 2
+  assert np.array_equal(first, O.dot_general(oxq, owq, DN).v) and np.array_equal(again, first)
+  assert np.array_equal(third, O.dot_general(oxq, owq2, DN).v)
+
+
 def test_both_operands_asymmetric_is_an_error():
   from qwix_amd.core import dot_general as dg
   from qwix_amd.core import qarray
