@@ -716,6 +716,30 @@ def quantize_with_scale_zero_point(array: torch.Tensor, qtype, scale: torch.Tens
 def quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = None) -> QArray:
   """Dynamic-range quantization: calibrate, derive scale (and zero point), quantize -- one fused pass.  With a
   `noise_fn` (stochastic rounding) the three steps run one after the other, as the reference's do (qarray.py:638-644)."""
+  try:
+    return _quantize(array, how, layout=layout)
+  except NotImplementedError as e:
+    # Packed int4 pairs run along one axis of even length; the natural layout takes the last one.  With an odd last
+    # axis the array is quantized with an even axis moved to the end (one copy) and the packed values are handed back
+    # as a view in the caller's axis order.
+    if 'even last dimension' not in str(e) or layout is not None or how.noise_fn is not None:
+      raise
+    shape, nd = tuple(array.shape), array.ndim
+    even = [a for a in range(nd - 1) if shape[a] % 2 == 0]
+    if not even:
+      raise
+    a = even[-1]
+    order = [d for d in range(nd) if d != a] + [a]        # new axis i is old axis order[i]
+    new_of = {old: new for new, old in enumerate(order)}
+    how2 = dataclasses.replace(how, channelwise_axes=tuple(new_of[c % nd] for c in how.channelwise_axes),
+                               tiled_axes={new_of[k % nd]: v for k, v in how.tiled_axes.items()})
+    q2 = _quantize(array.permute(*order).contiguous(), how2, layout='natural')
+    inv = [new_of[d] for d in range(nd)]
+    back = lambda t: None if t is None else t.permute(*inv).contiguous()
+    return QArray(q2.qvalue.permute(*inv), back(q2.scale), back(q2.zero_point), q2.qtype)
+
+
+def _quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = None) -> QArray:
   if how.noise_fn is not None and numerics.canonical_qtype(how.qtype) in (numerics.INT8, numerics.INT4) and array.numel():
     scale, zp = compute_scale_zero_point(calibrate(array, how), how.qtype)
     return quantize_with_scale_zero_point(array, how.qtype, scale, zp, how.noise_fn, layout='natural')
@@ -723,6 +747,146 @@ def quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = No
     raise ValueError(f'Refuse to quantize: {getattr(array, "dtype", type(array))}')
   shape = tuple(array.shape)
   q = numerics.canonical_qtype(how.qtype)
+  sshape = get_scale_shape(shape, how)
+  fixed = _fixed_calibration(how.calibration_method, array)
+  if fixed is not None:
+    return fixed
+  rms = _rms_calibration(how.calibration_method, array, sshape, _tiles_from_how(shape, how) if array.numel() else ())
+  if rms is not None:
+    return rms
+  cal, factor = _parse_calibration(how.calibration_method)
+  if array.numel() == 0:
+    _check_empty_reduction(sshape)
+    outs = [torch.empty(sshape, dtype=array.dtype, device=array.device) for _ in range(2 if cal == _lib.MINMAX else 1)]
+    return {'min': outs[0], 'max': outs[1]} if cal == _lib.MINMAX else {'absmax': outs[0]}
+  try:
+    plan = _plan(shape, _tiles_from_how(shape, how))
+  except NotImplementedError:
+    plan = None
+  ev = 8 if array.dtype == torch.bfloat16 else 4
+  if plan is None or plan.kind != '3d' or (plan.dims[2] > 1 and plan.dims[2] % ev):
+    # more than one group of reduced axes: the elements of a scale gathered into a row, one statistic per row
+    _, split, perm, rows, cols = _regrouped(shape, sshape)
+    x2 = array.reshape(split).permute(*perm).reshape(rows, cols).contiguous()
+    got = calibrate(x2, HowToQuantize(qtype=how.qtype, channelwise_axes=(0,), calibration_method=how.calibration_method))
+    return {k: v.reshape(sshape) for k, v in got.items()}
+  outs = [torch.empty(sshape, dtype=array.dtype, device=array.device) for _ in range(2 if cal == _lib.MINMAX else 1)]
+  ws, nws = _workspace(plan, cal, array.device)
+  _lib.call('qwix_hip_calibrate', array.data_ptr(), _lib.float_tag(array.dtype), *plan.dims, plan.tiles[0], cal,
+            factor, outs[0].data_ptr(), _lib.ptr(outs[1] if len(outs) > 1 else None), _lib.ptr(ws), nws,
+            _lib.stream_of(array))
+  if cal == _lib.MINMAX:
+    return {'min': outs[0], 'max': outs[1]}
+  return {'absmax': outs[0]}
+
+
+def compute_scale_zero_point(calibration: Mapping[str, torch.Tensor], qtype) -> tuple[torch.Tensor, torch.Tensor | None]:
+  """scale (and zero_point for min/max calibrations) from calibration statistics."""
+  if 'min' in calibration and 'max' in calibration:
+    c0, c1, cal = calibration['min'].contiguous(), calibration['max'].contiguous(), _lib.MINMAX
+    numerics.get_asymmetric_bound(qtype)  # raises for fp8
+  elif 'absmax' in calibration:
+    c0, c1, cal = calibration['absmax'].contiguous(), None, _lib.ABSMAX
+  else:
+    raise ValueError(f'Unsupported calibration: {calibration}')
+  scale = torch.empty_like(c0)
+  zp = torch.empty(c0.shape, dtype=torch.int8, device=c0.device) if cal == _lib.MINMAX else None
+  _lib.call('qwix_hip_compute_scale_zero_point', c0.data_ptr(), _lib.ptr(c1), _lib.float_tag(c0.dtype), c0.numel(),
+            numerics.qtype_tag(qtype), cal, scale.data_ptr(), _lib.ptr(zp), _lib.stream_of(c0))
+  return scale, zp
+
+
+def quantize_with_scale_zero_point(array: torch.Tensor, qtype, scale: torch.Tensor, zero_point: torch.Tensor | None,
+                                   noise_fn=None, *, layout: str | None = None) -> QArray:
+  """Quantizes with a given (static) scale; the scale is first cast to the array dtype.  `noise_fn(shape)` returns the
+  noise of stochastic rounding (numerics.py:191-195): added in f32 before the rounding to an integer type; float
+  qtypes ignore it, as the reference does."""
+  array = _check_float_input(array)
+  if zero_point is not None and tuple(zero_point.shape) != tuple(scale.shape):
+    raise ValueError(f'Expect zero_point shape {tuple(scale.shape)} but got {tuple(zero_point.shape)}')
+  shape = tuple(array.shape)
+  if len(shape) != scale.ndim or any((d % s) if s else d for d, s in zip(shape, scale.shape)):
+    raise ValueError(f'Cannot broadcast between {shape} {tuple(scale.shape)}')
+  q = numerics.canonical_qtype(qtype)
+  scale = scale.to(array.dtype).contiguous()
+  if array.numel() == 0:
+    return QArray(_empty_qvalue(shape, q, array.device), scale, zero_point, q)
+  try:
+    plan = _plan(shape, tuple(d // s for d, s in zip(shape, scale.shape)))
+  except NotImplementedError:
+    plan = None
+  ev = 8 if array.dtype == torch.bfloat16 else 4
+  if (plan is None or plan.kind != '3d' or (plan.dims[2] > 1 and plan.dims[2] % ev)
+      or (q == numerics.INT4 and plan.dims[2] == 1 and plan.tiles[0] % 2)):
+    # The static-scale kernels take one group of reduced axes (and whole 16-byte pieces of kept inner axes): any
+    # other pattern gathers the elements of a scale into a row first and puts the values back afterwards.
+    if layout not in (None, 'natural'):
+      raise NotImplementedError(f'static-scale quantization of shape {shape} with scales {tuple(scale.shape)} is '
+                                'delivered in the natural layout only')
+    sshape = tuple(scale.shape)
+    _, split, perm, rows, cols = _regrouped(shape, sshape)
+    if q == numerics.INT4 and cols % 2:
+      raise NotImplementedError(f'static-scale int4 quantization needs an even number of elements per scale, got {cols}')
+    regroup = lambda t: t.reshape(split).permute(*perm).reshape(rows, cols).contiguous()
+    noise2 = None
+    if noise_fn is not None and q in (numerics.INT8, numerics.INT4):
+      noise = noise_fn(shape)
+      if not isinstance(noise, torch.Tensor) or tuple(noise.shape) != shape:
+        raise ValueError(f'noise_fn must return a tensor of shape {shape}')
+      noise2 = lambda _shape, n=regroup(noise.to(array.device)): n
+    q2 = quantize_with_scale_zero_point(regroup(array), q, scale.reshape(rows, 1),
+                                        None if zero_point is None else zero_point.reshape(rows, 1), noise2,
+                                        layout='natural')
+    vals = q2.qvalue.unpack() if isinstance(q2.qvalue, Int4Tensor) else q2.qvalue
+    vals = _ungroup(vals, shape, sshape).contiguous()
+    if q == numerics.INT4:
+      vals = Int4Tensor.pack(vals)
+    return QArray(vals, scale, zero_point, q)
+  if noise_fn is not None and q in (numerics.INT8, numerics.INT4):
+    noise = noise_fn(shape)
+    if not isinstance(noise, torch.Tensor) or tuple(noise.shape) != shape:
+      raise ValueError(f'noise_fn must return a tensor of shape {shape}')
+    noise = noise.to(device=array.device, dtype=torch.float32).contiguous()
+    data, view = _alloc_q(shape, q, plan, _lib.LAYOUT_NATURAL, array.device)
+    zp = None if zero_point is None else zero_point.contiguous()
+    _lib.call('qwix_hip_quantize_with_scale_noise', array.data_ptr(), _lib.float_tag(array.dtype), *plan.dims,
+              plan.tiles[0], numerics.qtype_tag(q), scale.data_ptr(), _lib.ptr(zp), noise.data_ptr(), data.data_ptr(),
+              _lib.stream_of(array))
+    return QArray(view, scale, zero_point, q)
+  lay = _default_layout(plan, layout, shape, q)
+  data, view = _alloc_q(shape, q, plan, lay, array.device)
+  zp = None if zero_point is None else zero_point.contiguous()
+  _lib.call('qwix_hip_quantize_with_scale', array.data_ptr(), _lib.float_tag(array.dtype), *plan.dims, plan.tiles[0],
+            numerics.qtype_tag(q), scale.data_ptr(), _lib.ptr(zp), lay, data.data_ptr(), _lib.stream_of(array))
+  return QArray(view, scale, zero_point, q)
+
+
+def quantize(array: torch.Tensor, how: HowToQuantize, *, layout: str | None = None) -> QArray:
+  """Dynamic-range quantization: calibrate, derive scale (and zero point), quantize -- one fused pass.  With a
+  `noise_fn` (stochastic rounding) the three steps run one after the other, as the reference's do (qarray.py:638-644)."""
+  if how.noise_fn is not None and numerics.canonical_qtype(how.qtype) in (numerics.INT8, numerics.INT4) and array.numel():
+    scale, zp = compute_scale_zero_point(calibrate(array, how), how.qtype)
+    return quantize_with_scale_zero_point(array, how.qtype, scale, zp, how.noise_fn, layout='natural')
+  if not isinstance(array, torch.Tensor) or not numerics.should_quantize(array.dtype):
+    raise ValueError(f'Refuse to quantize: {getattr(array, "dtype", type(array))}')
+  shape = tuple(array.shape)
+  q = numerics.canonical_qtype(how.qtype)
+  if q == numerics.INT4 and array.ndim > 1 and shape[-1] % 2 and layout is None and math.prod(shape):
+    # Packed int4 pairs run along one axis of even length; the natural layout takes the last one.  With an odd last
+    # axis the array is quantized with an even axis moved to the end (one copy) and the packed values are handed back
+    # as a view in the caller's axis order.
+    even = [a for a in range(array.ndim - 1) if shape[a] % 2 == 0]
+    if even:
+      a = even[-1]
+      order = [d for d in range(array.ndim) if d != a] + [a]        # new axis i is old axis order[i]
+      new_of = {old: new for new, old in enumerate(order)}
+      how2 = dataclasses.replace(
+          how, channelwise_axes=tuple(new_of[c % array.ndim] for c in how.channelwise_axes),
+          tiled_axes={new_of[k % array.ndim]: v for k, v in how.tiled_axes.items()})
+      q2 = quantize(array.permute(*order).contiguous(), how2, layout='natural')
+      inv = [new_of[d] for d in range(array.ndim)]
+      back = lambda t: None if t is None else t.permute(*inv).contiguous()
+      return QArray(q2.qvalue.permute(*inv), back(q2.scale), back(q2.zero_point), q)
   sshape = get_scale_shape(shape, how)
   fixed = _fixed_calibration(how.calibration_method, array)
   if fixed is None:  # rms: its own reduction kernel, then the static-scale kernel
@@ -837,6 +1001,9 @@ def dequantize(array: QArray) -> torch.Tensor:
     return torch.empty(array.shape, dtype=array.scale.dtype, device=array.scale.device)
   try:
     plan, lay, data = physical_layout(array)
+  except Int4LayoutError:
+    # packed pairs along an axis that is neither the last nor the reduced one: the same integers, one byte each
+    return dequantize(QArray(array.qvalue.unpack().contiguous(), array.scale, array.zero_point, numerics.INT8))
   except NotImplementedError as e:
     if 'separate reduced axis groups' not in str(e):
       raise

@@ -445,3 +445,26 @@ def test_static_scales_of_any_tiling(shape, sshape, qtype, asym):
   got, want = qarray.calibrate(x_t, qarray.HowToQuantize(**how)), O.calibrate(O.FArr(x_np, O.BF16), O.HowToQuantize(**how))
   for k in want:
     assert np.array_equal(util.f32np(got[k]), want[k].v), k
+
+
+@pytest.mark.parametrize('shape,how', [
+    ((2, 1024, 3), dict(channelwise_axes=[0, 2], tiled_axes={1: 128})),
+    ((16, 5), dict(channelwise_axes=[1])),
+    ((6, 4, 7), dict(channelwise_axes=[0], calibration_method='minmax')),
+])
+def test_int4_with_an_odd_last_axis(shape, how):
+  """Packed int4 pairs need an axis of even length; when the last axis is odd another one carries them."""
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  x_np, x_t = util.make(shape, O.BF16, seed=sum(shape))
+  q = qarray.quantize(x_t, qarray.HowToQuantize(qtype='int4', **how))
+  oq = O.quantize(O.FArr(x_np, O.BF16), O.HowToQuantize(qtype='int4', **how))
+  assert q.qvalue.packed_axis != len(shape) - 1
+  util.assert_qarray_equal(q, oq, 'int4')
+  assert np.array_equal(util.f32np(qarray.dequantize(q)), O.dequantize(oq).v)
+  if len(shape) == 2:  # and it multiplies: contracted over the first axis against an int8 activation
+    a_np, a_t = util.make((8, shape[0]), O.BF16, seed=3)
+    aq = qarray.quantize(a_t, qarray.HowToQuantize(qtype='int8', channelwise_axes=[0]))
+    oaq = O.quantize(O.FArr(a_np, O.BF16), O.HowToQuantize(qtype='int8', channelwise_axes=[0]))
+    dn = (((1,), (0,)), ((), ()))
+    assert np.array_equal(util.f32np(dg.dot_general(aq, q, dn)), O.dot_general(oaq, oq, dn).v)

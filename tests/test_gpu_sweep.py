@@ -78,8 +78,8 @@ def _quantize_cases(seed, count):
       if a not in cw and r.random() < 0.3:
         tiled[a] = int(r.choice([d for d in (1, 2, 4, 8, 16, 32, 64, 128) if shape[a] % d == 0]))
     calib = str(r.choice(['absmax', 'absmax', 'minmax', 'absmax,0.9'])) if qt != O.E4M3 else 'absmax'
-    if np.prod(shape) > 4_000_000 or (qt == 'int4' and shape[-1] % 2):
-      continue  # packed int4 storage pairs elements of the last axis
+    if np.prod(shape) > 4_000_000 or (qt == 'int4' and all(d % 2 for d in shape)):
+      continue  # packed int4 storage pairs the elements of an axis of even length
 
     def thunk(shape=shape, dt=dt, qt=qt, cw=cw, tiled=tiled, calib=calib, c=c):
       x_np, x_t = util.make(shape, dt, seed=100 + c)
@@ -300,8 +300,8 @@ def _dimension_number_cases(seed, count):
     if tile and cs[-1] % tile:
       tile = 0
     asym = lq != O.E4M3 and r.random() < 0.2
-    if (lq == 'int4' and lshape[-1] % 2) or (rq == 'int4' and rshape[-1] % 2):
-      continue  # packed int4 storage pairs elements of the last axis
+    if (lq == 'int4' and all(d % 2 for d in lshape)) or (rq == 'int4' and all(d % 2 for d in rshape)):
+      continue  # packed int4 storage pairs the elements of an axis of even length
 
     def thunk(lshape=lshape, rshape=rshape, dn=dn, dt=dt, lq=lq, rq=rq, tile=tile, asym=asym, last_k=cs[-1], c=c):
       x_np, x_t = util.make(lshape, dt, seed=c)
