@@ -320,3 +320,36 @@ def test_weight_only_int4_prefill_at_the_gemv_weight_shape():
   assert np.array_equal(out[rows].cpu().to(torch.float64).numpy() * 2, want.astype(np.float64))
   total = out.to(torch.float64).sum().item() * 2
   assert total == float(x_i.to(torch.float64).sum(0).cpu().numpy() @ w2.to(torch.float64).sum(0).cpu().numpy())
+
+
+def test_quantize_of_more_than_2_31_elements():
+  """70000 x 32768 bf16 (2.29e9 elements, 4.6 GB): element indices pass 2^31 in every quantize layout.  Sampled rows
+  and columns are compared with the oracle bit for bit (the oracle on the whole array would take minutes)."""
+  from qwix_amd.core import qarray
+  M, K = 70000, 32768
+  x = torch.randn(M, K, device=util.DEV, dtype=torch.bfloat16)
+  rows = [0, 1, 12345, 65535, 65536, M - 1]
+  xs = x[rows].float().cpu().numpy()
+  for qt in ('int8', 'int4', O.E4M3):
+    print('case big per-token', qt, flush=True)
+    q = qarray.quantize(x, qarray.HowToQuantize(qtype=qt, channelwise_axes=[0]))
+    oq = O.quantize(O.FArr(xs, O.BF16), O.HowToQuantize(qtype=qt, channelwise_axes=[0]))
+    vals = q.qvalue.unpack()[rows] if qt == 'int4' else q.qvalue[rows]
+    got = vals.view(torch.uint8).cpu().numpy() if qt == O.E4M3 else vals.cpu().numpy()
+    assert np.array_equal(got, oq.qvalue), qt
+    assert np.array_equal(util.f32np(q.scale[rows]), oq.scale.v), qt
+    del q, vals
+  print('case big groups of 128', flush=True)
+  how = dict(qtype='int8', channelwise_axes=[0], tiled_axes={1: 128})
+  q = qarray.quantize(x, qarray.HowToQuantize(**how))
+  oq = O.quantize(O.FArr(xs, O.BF16), O.HowToQuantize(**how))
+  assert np.array_equal(q.qvalue[rows].cpu().numpy(), oq.qvalue) and np.array_equal(util.f32np(q.scale[rows]), oq.scale.v)
+  del q
+  print('case big per-channel', flush=True)
+  cols = [0, 7, 8, 1000, K - 1]
+  q = qarray.quantize(x, qarray.HowToQuantize(qtype='int8', channelwise_axes=[1]))
+  oq = O.quantize(O.FArr(x[:, cols].float().cpu().numpy(), O.BF16), O.HowToQuantize(qtype='int8', channelwise_axes=[1]))
+  assert np.array_equal(util.f32np(q.scale[:, cols]), oq.scale.v)
+  assert np.array_equal(q.qvalue[:, cols].cpu().numpy(), oq.qvalue)
+  d = qarray.dequantize(q)
+  assert np.array_equal(util.f32np(d[:, cols]), O.dequantize(oq).v)
