@@ -353,3 +353,29 @@ def test_quantize_of_more_than_2_31_elements():
   assert np.array_equal(q.qvalue[:, cols].cpu().numpy(), oq.qvalue)
   d = qarray.dequantize(q)
   assert np.array_equal(util.f32np(d[:, cols]), O.dequantize(oq).v)
+
+
+@pytest.mark.parametrize('M,K,N', [(50000, 49152, 256), (300, 98304, 50000)])
+def test_int8_gemm_with_an_operand_of_more_than_2_31_bytes(M, K, N):
+  """Byte offsets into one operand pass 2^31 (2.46 GB of activations / 4.9 GB of weights): sampled outputs against the
+  exact integer product and the bf16 epilogue chain."""
+  from qwix_amd import _lib
+  print('case big gemm', M, K, N, flush=True)
+  a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device=util.DEV)
+  b = torch.randint(-128, 128, (N, K), dtype=torch.int8, device=util.DEV)
+  acc = torch.empty(M, N, dtype=torch.int32, device=util.DEV)
+  st = _lib.stream_of(a)
+  _lib.call('qwix_hip_qgemm', a.data_ptr(), K, b.data_ptr(), K, _lib.INT8, M, N, K, None, 0, None, 0, 0, acc.data_ptr(),
+            _lib.I32, N, st)
+  rows, cols = [0, 1, M // 2 + 3, M - 1], [0, 5, N // 2, N - 1]
+  want = a[rows].double() @ b[cols].double().T            # |sums| < 2^53: exact
+  assert torch.equal(acc[rows][:, cols].double(), want)
+  sa = (torch.rand(M, device=util.DEV) * 0.01 + 0.001).to(torch.bfloat16)
+  sb = (torch.rand(N, device=util.DEV) * 0.01 + 0.001).to(torch.bfloat16)
+  out = torch.empty(M, N, dtype=torch.bfloat16, device=util.DEV)
+  _lib.call('qwix_hip_qgemm', a.data_ptr(), K, b.data_ptr(), K, _lib.INT8, M, N, K, sa.data_ptr(), _lib.BF16,
+            sb.data_ptr(), _lib.BF16, 0, out.data_ptr(), _lib.BF16, N, st)
+  w = acc[rows][:, cols].float().bfloat16()
+  w = (w.float() * sa[rows].float()[:, None]).bfloat16()
+  w = (w.float() * sb[cols].float()[None, :]).bfloat16()
+  assert torch.equal(out[rows][:, cols], w)
