@@ -2478,6 +2478,27 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
                       const int32_t* zv, void* out, int out_dtype, int64_t ldo, void* stream, void* workspace = nullptr,
                       size_t workspace_bytes = 0);
 static int splitk_plan(int64_t M, int64_t N, int64_t K, double other_us);
+// Problems of up to this many 128 x 128 tiles take 64 x 64 tiles (four times the workgroups).  Measured, int8 and
+// e4m3, bf16 result, weights in the second-level cache / from HBM: 256 x 4096 over K 1024 9.5 -> 5.6 / 12.1 -> 8.4 us,
+// 1024^3 9.3 -> 5.4 / 11.7 -> 8.2, 512 x 4096 over K 4096 23.5 -> 16.2 / 34.9 -> 26.8, 1536 x 2048 over K 2048 (192
+// tiles) 16.0 -> 12.6 / 18.3 -> 14.6; level from 256 tiles on (2048 x 2048 over K 1024: 10.6 / 10.4 us), behind at 512
+// (4096 x 2048 over K 1024: 13.0 / 17.1 us).
+#ifndef QWIX_SMALL_TILES
+#define QWIX_SMALL_TILES 200
+#endif
+constexpr int64_t kSmallTiles = QWIX_SMALL_TILES;
+
+// What the unsplit tiled kernel takes, in us (the figure a split of K has to beat), with weights that come from HBM
+// as a model's do (copies in rotation, 600 MB): 64 x 64 tiles on small problems 3.5 us + 0.58 us per 128 of K (256 x 1024
+// over K 4096 21.7 us, 512 x 512 over K 8192 40.4 us; with the weights in the second-level cache it is 0.24 us per
+// slab), 128 x 128 tiles beyond.
+static double tiled_model_us(int64_t M, int64_t N, int64_t K) {
+  const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+  const double slabs = static_cast<double>(K / 128);
+  if (tiles128 <= kSmallTiles) return 3.5 + 0.58 * slabs;
+  return 5.0 + 0.55 * slabs;
+}
+
 static bool streams_weights(int64_t M, int64_t N, int64_t K, bool one_tile_row = false);
 
 // Dtype chain of the reference epilogue: int32 adopts the first scale's dtype (through f32); a
@@ -2761,7 +2782,7 @@ extern "C" int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t
 extern "C" size_t qwix_hip_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   // the split count qwix_hip_qgemm_ws would pick: the plan against the unsplit tiled kernel's model
-  const int splits = streams_weights(M, N, K) ? 0 : splitk_plan(M, N, K, 5.0 + 0.55 * static_cast<double>(K / 128));
+  const int splits = streams_weights(M, N, K) ? 0 : splitk_plan(M, N, K, tiled_model_us(M, N, K));
   return splits > 0 ? static_cast<size_t>(splits) * M * N * 4 : 0;
 }
 
@@ -3007,7 +3028,7 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
   // model favours it (streams_weights): the skinny kernel makes one pass over the weights per 16 rows (about
   // 0.5 us + 5.2 bytes/ns each) after a 4 us start; the tiled kernels walk K in 128-wide slabs after 5 us,
   // however few of the chip's CUs their 128 x 128 tiles occupy.
-  const double tiled_us = 5.0 + 0.55 * static_cast<double>(K / 128);
+  const double tiled_us = tiled_model_us(M, N, K);
   // what the one-tile-row kernel (launch_mid) needs
   // (65 to 128 rows: one workgroup per CU for its 96 or 128 KB of LDS stages, so only while one round of
   // workgroups covers N: 64-column ones up to N 16384, 128-column ones up to N 32768.  Measured against the
@@ -3062,11 +3083,16 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
       if (out_dtype == QWIX_BF16) return launch_mid<QWIX_E4M3, QWIX_BF16>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       return launch_mid<QWIX_E4M3, QWIX_F32>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     }
+    // 128 x 128 tiles that would occupy less than a third of the chip: 64 x 64 tiles, four times as many workgroups
+    // (a layer of 256 tokens x 4096 features over K 1024 is 64 tiles of 128 x 128)
+    const bool small = ((M + 127) / 128) * ((N + 127) / 128) <= kSmallTiles;
     if (qtype == QWIX_INT8) {
       if (big) return dispatch_dma<QWIX_INT8, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      if (small) return dispatch_dma<QWIX_INT8, 64, 64, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       return dispatch_dma<QWIX_INT8, 128, 128, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     }
     if (big) return dispatch_dma<QWIX_E4M3, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    if (small) return dispatch_dma<QWIX_E4M3, 64, 64, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     return dispatch_dma<QWIX_E4M3, 128, 128, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
   }
   // register-staged kernel: any K that is a multiple of 16

@@ -325,6 +325,7 @@ def test_weight_only_int4_prefill_at_the_gemv_weight_shape():
 def test_quantize_of_more_than_2_31_elements():
   """70000 x 32768 bf16 (2.29e9 elements, 4.6 GB): element indices pass 2^31 in every quantize layout.  Sampled rows
   and columns are compared with the oracle bit for bit (the oracle on the whole array would take minutes)."""
+  from oracle import qwix_oracle as O
   from qwix_amd.core import qarray
   M, K = 70000, 32768
   x = torch.randn(M, K, device=util.DEV, dtype=torch.bfloat16)
