@@ -512,7 +512,10 @@ __device__ __forceinline__ void staged_epilogue(const AccT (&acc)[TM][TN], const
   }
 }
 
-template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI>
+// NST: slab stages of the direct-to-LDS tile body.  Two by default; four for the 64 x 64 tile of small problems while
+// its workgroups are at most two per CU: they have nothing else to cover the latency of weights that come from HBM
+// (three slabs in flight instead of one; with more workgroups per CU the LDS the stages take costs more than it gives).
+template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI, int NST = 2>
 __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, int64_t lda,
                                                const uint8_t* __restrict__ B, int64_t ldb, int m0, int n0, int M,
                                                int N, int K, const Epilogue& ep, uint8_t* __restrict__ out,
@@ -626,6 +629,44 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
   float sav[TM];
   fetch_scales<OUT, TM, TN>(ep, m_base, n_base, M, N, lane, sav, sbv);
   const int KT = K / BK;
+  if constexpr (NST > 2) {
+    // Slabs kt + 1 .. kt + NST - 1 are in flight while slab kt is multiplied.  At the end of slab kt: wait until only
+    // the loads of the slabs after kt + 1 are outstanding, barrier (everyone's part of slab kt + 1 has landed, everyone
+    // is done reading slab kt), and the stage of slab kt is requested again at the start of slab kt + 1.
+    auto wait_for = [&](int newer) __attribute__((always_inline)) {  // `newer`: slabs requested after the awaited one
+      static_assert(NST == 4 && 2 * LOADS < 16, "wait counts are written out for four stages");
+      if (newer >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * LOADS));
+      else if (newer == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | LOADS);
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
+    };
+#pragma unroll
+    for (int s = 0; s < NST - 1; ++s)
+      if (s < KT) issue_loads(s, s * BK);
+    wait_for(min(KT - 1, NST - 2));
+    __builtin_amdgcn_s_barrier();
+    read_frags(0, 0, 0);
+    int cur = 0;
+    for (int kt = 0; kt < KT; ++kt) {
+      const int nxt = cur + 1 == NST ? 0 : cur + 1;
+      if (kt + NST - 1 < KT) issue_loads(cur == 0 ? NST - 1 : cur - 1, (kt + NST - 1) * BK);  // the stage of slab kt - 1
+#pragma unroll
+      for (int ks = 0; ks + 1 < NK; ++ks) {
+        read_frags(cur, ks + 1, (ks + 1) & 1);
+        mfma_step(ks & 1);
+        hint_kstep(ks == 0 ? LOADS : 0);
+      }
+      mfma_step((NK - 1) & 1);
+      if (kt + 1 < KT) {
+        wait_for(min(KT - 1, kt + NST - 1) - (kt + 1));
+        __builtin_amdgcn_s_barrier();
+        read_frags(nxt, 0, 0);
+      }
+      cur = nxt;
+    }
+    staged_epilogue<OUT, EPI, TM, TN, NWAVES, NST * STAGE>(acc, sav, sbv, ep, m_base, n_base, M, N, out, ldo, smem, wave,
+                                                             lane);
+    return;
+  }
   issue_loads(0, 0);
   __syncthreads();
   read_frags(0, 0, 0);
@@ -657,20 +698,20 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
                                                          lane);
 }
 
-template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI>
+template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI, int NST = 2>
 __global__ void __launch_bounds__(WGM * WGN * 64)
     qgemm_dma_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
                      int M, int N, int K, Epilogue ep, uint8_t* __restrict__ out, int64_t ldo) {
   int tile_m, tile_n;
   tile_coords((M + BM - 1) / BM, (N + BN - 1) / BN, &tile_m, &tile_n);
-  qgemm_dma_tile<QT, BM, BN, WGM, WGN, OUT, EPI>(A, lda, B, ldb, tile_m * BM, tile_n * BN, M, N, K, ep, out, ldo);
+  qgemm_dma_tile<QT, BM, BN, WGM, WGN, OUT, EPI, NST>(A, lda, B, ldb, tile_m * BM, tile_n * BN, M, N, K, ep, out, ldo);
 }
 
-template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI>
+template <int QT, int BM, int BN, int WGM, int WGN, int OUT, int EPI, int NST = 2>
 int launch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
                const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
-  constexpr size_t smem = 2 * (BM + BN) * 128;
-  auto kern = qgemm_dma_kernel<QT, BM, BN, WGM, WGN, OUT, EPI>;
+  constexpr size_t smem = NST * (BM + BN) * 128;
+  auto kern = qgemm_dma_kernel<QT, BM, BN, WGM, WGN, OUT, EPI, NST>;
   static LdsGrant granted;
   if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
@@ -682,27 +723,27 @@ int launch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M
 
 // Picks the epilogue specialisation: (bf16 out, all-bf16 rounding), (f32 out, no rounding), raw int32,
 // or the run-time-flag version for mixed scale dtypes.
-template <int QT, int BM, int BN, int WGM, int WGN>
+template <int QT, int BM, int BN, int WGM, int WGN, int NST = 2>
 int dispatch_dma(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
                  const Epilogue& ep, void* out, int64_t ldo, hipStream_t st) {
   const bool all = ep.r0 && ep.r1 && ep.r2, none = !ep.r0 && !ep.r1 && !ep.r2;
   if (ep.out_dtype == QWIX_I32) {
-    if constexpr (QT == QWIX_INT8) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_I32, 0>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    if constexpr (QT == QWIX_INT8) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_I32, 0, NST>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     return fail(QWIX_ERR_INVALID_ARGUMENT, "int32 output needs int8 operands");
   }
   if (ep.zu != nullptr) {
     if constexpr (QT == QWIX_INT8) {
-      if (ep.out_dtype == QWIX_BF16) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_BF16, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
-      return launch_dma<QT, BM, BN, WGM, WGN, QWIX_F32, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      if (ep.out_dtype == QWIX_BF16) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_BF16, 3, NST>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      return launch_dma<QT, BM, BN, WGM, WGN, QWIX_F32, 3, NST>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     }
     return fail(QWIX_ERR_UNSUPPORTED, "zero-point correction needs int8 operands");
   }
   if (ep.out_dtype == QWIX_BF16) {
-    if (all) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_BF16, 1>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
-    return launch_dma<QT, BM, BN, WGM, WGN, QWIX_BF16, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    if (all) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_BF16, 1, NST>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    return launch_dma<QT, BM, BN, WGM, WGN, QWIX_BF16, 2, NST>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
   }
-  if (none) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_F32, 0>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
-  return launch_dma<QT, BM, BN, WGM, WGN, QWIX_F32, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+  if (none) return launch_dma<QT, BM, BN, WGM, WGN, QWIX_F32, 0, NST>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+  return launch_dma<QT, BM, BN, WGM, WGN, QWIX_F32, 2, NST>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -2489,12 +2530,14 @@ static int splitk_plan(int64_t M, int64_t N, int64_t K, double other_us);
 constexpr int64_t kSmallTiles = QWIX_SMALL_TILES;
 
 // What the unsplit tiled kernel takes, in us (the figure a split of K has to beat), with weights that come from HBM
-// as a model's do (copies in rotation, 600 MB): 64 x 64 tiles on small problems 3.5 us + 0.58 us per 128 of K (256 x 1024
-// over K 4096 21.7 us, 512 x 512 over K 8192 40.4 us; with the weights in the second-level cache it is 0.24 us per
-// slab), 128 x 128 tiles beyond.
+// as a model's do (copies in rotation, 600 MB): 64 x 64 tiles with four stages 3.5 us + 0.29 us per 128 of K and round
+// of 256 workgroups (256 x 1024 over K 4096 12.7 us, 512 x 512 over K 8192 21.8 us, 512 x 4096 over K 4096 21.0 us),
+// 0.58 us per slab with two stages, 128 x 128 tiles beyond.
 static double tiled_model_us(int64_t M, int64_t N, int64_t K) {
-  const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+  const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128), tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
   const double slabs = static_cast<double>(K / 128);
+  if (M < 64 && N * K >= (int64_t{8} << 20)) return 5.0 + 0.55 * slabs;  // the one-tile-row kernel's range
+  if (tiles128 <= kSmallTiles && tiles64 <= 512) return 3.5 + 0.29 * slabs * (tiles64 <= 256 ? 1.0 : tiles64 / 256.0);
   if (tiles128 <= kSmallTiles) return 3.5 + 0.58 * slabs;
   return 5.0 + 0.55 * slabs;
 }
@@ -2970,8 +3013,9 @@ static bool streams_weights(int64_t M, int64_t N, int64_t K, bool one_tile_row) 
     return skinny_us < 5.8 + (slabs_us > bytes_us ? slabs_us : bytes_us);
   }
   if (M <= 32) return skinny_us < tiled_us;
-  // more rows: the comparison that was tuned with weights that stay in the last-level cache between calls
-  return M <= 256 && tiles128 <= 256 && skinny_us < 5.0 + 0.55 * static_cast<double>(K / 128);
+  // more rows: against the tiled kernel this shape would get (64 x 64 tiles with four stages on small problems:
+  // 256 rows over K 8192 against 1024 columns take 22 us there, 30.6 us in sixteen passes of the weight-streaming kernel)
+  return M <= 256 && tiles128 <= 256 && skinny_us < tiled_model_us(M, N, K);
 }
 
 // Number of K ranges worth cutting the problem into (0: do not split).  Model, in microseconds, fitted to
@@ -3065,7 +3109,14 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
       if (qtype == QWIX_INT8) return dispatch_pp<QWIX_INT8>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       return dispatch_pp<QWIX_E4M3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     }
-    if (mid_ok) {
+    // 64 x 64 tiles with four slab stages, at most two per CU
+    const bool small_deep = ((M + 127) / 128) * ((N + 127) / 128) <= kSmallTiles && ((M + 63) / 64) * ((N + 63) / 64) <= 512;
+    // From 64 rows on those tiles take the shapes of the one-tile-row kernel faster (weights from HBM, 100 rows: K 4096,
+    // N 4096 23.5 -> 12.9 us, K 14336, N 4096 68.3 -> 36.2, K 8192, N 8192 41.8 -> 23.5; 64 rows: 14.6 -> 13.2, 41.0 ->
+    // 37.9, 25.5 -> 24.3; 256 rows, K 4096, N 4096: 22.5 -> 13.4; level at 48 rows, behind below).  Where they do not
+    // apply (N 28672: 224 tiles of 128 x 128) the one-tile-row kernel stays ahead of 128 x 128 tiles (28.6 against 39.3 us
+    // at 64 rows).
+    if (mid_ok && !(small_deep && M >= 64)) {
       // up to 64 rows against a weight of megabytes (and too many rows, or too large a weight, for the
       // weight-streaming kernel): the tile that keeps three slabs of weights in flight per wavefront
       if (qtype == QWIX_INT8 && zu != nullptr) {  // zero-point correction in the epilogue
@@ -3086,12 +3137,18 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
     // 128 x 128 tiles that would occupy less than a third of the chip: 64 x 64 tiles, four times as many workgroups
     // (a layer of 256 tokens x 4096 features over K 1024 is 64 tiles of 128 x 128)
     const bool small = ((M + 127) / 128) * ((N + 127) / 128) <= kSmallTiles;
+    // four slab stages (64 KB) while the 64 x 64 tiles are at most two per CU: weights from HBM, 256 x 1024 over
+    // K 4096 21.8 -> 12.7 us, 512 x 512 over K 8192 40.7 -> 21.8, 512 x 4096 over K 4096 26.8 -> 21.0; with 768 tiles
+    // (1536 x 2048 over K 2048) 14.6 -> 17.1 us, so those keep two stages
+    const bool deep = ((M + 63) / 64) * ((N + 63) / 64) <= 512;
     if (qtype == QWIX_INT8) {
       if (big) return dispatch_dma<QWIX_INT8, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      if (small && deep) return dispatch_dma<QWIX_INT8, 64, 64, 2, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       if (small) return dispatch_dma<QWIX_INT8, 64, 64, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       return dispatch_dma<QWIX_INT8, 128, 128, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     }
     if (big) return dispatch_dma<QWIX_E4M3, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    if (small && deep) return dispatch_dma<QWIX_E4M3, 64, 64, 2, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     if (small) return dispatch_dma<QWIX_E4M3, 64, 64, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     return dispatch_dma<QWIX_E4M3, 128, 128, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
   }
