@@ -988,7 +988,7 @@ WORKLOADS = {
     'quantize_act_4096': lambda: QuantizeRows('quantize_act_4096', 4096, 4096, 'int8'),
     'quantize_act_8192_fp8': lambda: QuantizeRows('quantize_act_8192_fp8', 8192, 8192, 'float8_e4m3fn'),
     'w8a8_decode_m16': lambda: QdotDecode('w8a8_decode_m16', 16, 4096, 14336),
-    'w8a8_decode_m64': lambda: QdotDecode('w8a8_decode_m64', 64, 4096, 14336, 'qgemm_mid_kernel'),
+    'w8a8_decode_m64': lambda: QdotDecode('w8a8_decode_m64', 64, 4096, 14336, 'qgemm_dma_kernel'),
     'w8a8_decode_m64_k8192': lambda: QdotDecode('w8a8_decode_m64_k8192', 64, 8192, 28672, 'qgemm_mid_kernel'),
     'w8a8_decode_m16_k2048': lambda: QdotDecode('w8a8_decode_m16_k2048', 16, 2048, 8192),
     'w8a8_decode_m16_k2048_fused': lambda: QdotDecodeFused('w8a8_decode_m16_k2048_fused', 16, 2048, 8192),
