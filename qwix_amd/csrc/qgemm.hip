@@ -634,9 +634,12 @@ __device__ __forceinline__ void qgemm_dma_tile(const uint8_t* __restrict__ A, in
     // the loads of the slabs after kt + 1 are outstanding, barrier (everyone's part of slab kt + 1 has landed, everyone
     // is done reading slab kt), and the stage of slab kt is requested again at the start of slab kt + 1.
     auto wait_for = [&](int newer) __attribute__((always_inline)) {  // `newer`: slabs requested after the awaited one
-      static_assert(NST == 4 && 2 * LOADS < 16, "wait counts are written out for four stages");
-      if (newer >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * LOADS));
-      else if (newer == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | LOADS);
+      static_assert((NST == 3 || NST == 4) && 2 * LOADS < 64, "wait counts are written out for three or four stages");
+      // vmcnt is a six-bit field in two pieces: bits 3:0 and 15:14
+      constexpr int W2 = 0x0F70 | ((2 * LOADS) & 0xF) | (((2 * LOADS) >> 4) << 14);
+      constexpr int W1 = 0x0F70 | (LOADS & 0xF) | ((LOADS >> 4) << 14);
+      if (newer >= 2) __builtin_amdgcn_s_waitcnt(W2);
+      else if (newer == 1) __builtin_amdgcn_s_waitcnt(W1);
       else __builtin_amdgcn_s_waitcnt(0x0F70);
     };
 #pragma unroll
@@ -3141,15 +3144,21 @@ static int qgemm_impl(const void* a, int64_t lda, const void* b, int64_t ldb, in
     // K 4096 21.8 -> 12.7 us, 512 x 512 over K 8192 40.7 -> 21.8, 512 x 4096 over K 4096 26.8 -> 21.0; with 768 tiles
     // (1536 x 2048 over K 2048) 14.6 -> 17.1 us, so those keep two stages
     const bool deep = ((M + 63) / 64) * ((N + 63) / 64) <= 512;
+    // 128 x 128 tiles that are at most one per CU: three slab stages (96 KB).  Weights from HBM, 256 tiles: 1024 x 4096
+    // over K 4096 34.8 -> 25.3 us, 2048 x 2048 over K 4096 31.8 -> 26.4, over K 1024 12.5 -> 11.3; with two tiles per CU
+    // (512 tiles) the second workgroup hides more than the third stage does (4096 x 2048 over K 1024: 14.2 against 20.0 us)
+    const bool one_round = ((M + 127) / 128) * ((N + 127) / 128) <= 256;
     if (qtype == QWIX_INT8) {
       if (big) return dispatch_dma<QWIX_INT8, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       if (small && deep) return dispatch_dma<QWIX_INT8, 64, 64, 2, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       if (small) return dispatch_dma<QWIX_INT8, 64, 64, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+      if (one_round) return dispatch_dma<QWIX_INT8, 128, 128, 2, 2, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
       return dispatch_dma<QWIX_INT8, 128, 128, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     }
     if (big) return dispatch_dma<QWIX_E4M3, 256, 256, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     if (small && deep) return dispatch_dma<QWIX_E4M3, 64, 64, 2, 2, 4>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     if (small) return dispatch_dma<QWIX_E4M3, 64, 64, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
+    if (one_round) return dispatch_dma<QWIX_E4M3, 128, 128, 2, 2, 3>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
     return dispatch_dma<QWIX_E4M3, 128, 128, 2, 2>(a, lda, b, ldb, M, N, K, ep, out, ldo, st);
   }
   // register-staged kernel: any K that is a multiple of 16
