@@ -4,7 +4,8 @@
 //
 // Tile bodies (device functions of a tile origin and a row limit, shared by all entry points):
 //   qgemm_tile      register-staged 128 x 128 tile, any K that is a multiple of 16
-//   qgemm_dma_tile  K % 128 == 0: 128-byte K slabs go global -> LDS directly, two stages
+//   qgemm_dma_tile  K % 128 == 0: 128-byte K slabs go global -> LDS directly, two stages (three or four where a
+//                   problem's tiles are so few per CU that nothing else covers the latency of the loads)
 //   qgemm_pp_tile   256 x 256, long K: two wavefront groups half a slab out of phase (ping-pong)
 // Kernels around them: dense (one tile per workgroup, XCD-aware tile order), batched (blockIdx.y
 // selects the problem), ragged (rows in groups whose sizes live in device memory, one weight panel
