@@ -349,6 +349,20 @@ int launch_grouped(const GroupedArgs& p, hipStream_t st) {
 struct Fast {
   static constexpr int kBM = 128, kBN = 256, kBK = 128, kNW = 8, kTM = 4;
 };
+// The same kernel with two wavefronts and 64 columns per workgroup: four times the workgroups, for problems whose
+// 128 x 256 tiles would leave most of the chip idle (a few hundred rows, or decode batches, against a weight of a few
+// thousand columns).
+struct Narrow {
+  static constexpr int kBM = 128, kBN = 64, kBK = 128, kNW = 2, kTM = 4;
+};
+// ... and with 64 or 32 rows for decode batches: a quarter of the MFMAs and folds per slab where the other rows of a
+// 128-row tile would be padding.
+struct Narrow64 {
+  static constexpr int kBM = 64, kBN = 64, kBK = 128, kNW = 2, kTM = 2;
+};
+struct Narrow32 {
+  static constexpr int kBM = 32, kBN = 64, kBK = 128, kNW = 2, kTM = 1;
+};
 
 // SAG: the activations carry one scale per row and group as well (both operands tiled along K): the
 // tile's (groups x 128 rows) scales are converted to f32 and parked in LDS behind the slab stages; folding a
@@ -368,10 +382,11 @@ struct Fast {
 // time to land; the wait before the barrier that ends slab k leaves them in flight (vmcnt counts oldest first).
 // ONE: every group is one slab (group == 128): the main loop then has a single straight-line body.
 // DUMP (with AUX): the corrected partials are also written to acc_out (parity runs).
-template <int BQT, bool SBF, bool SAG, bool AUX, bool MAGIC = false, int ST = 2, bool ONE = false, bool DUMP = false>
-__global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <int BQT, bool SBF, bool SAG, bool AUX, bool MAGIC = false, int ST = 2, bool ONE = false, bool DUMP = false,
+          typename G = Fast>
+__global__ void __launch_bounds__(G::kNW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     qgemm_grouped_dma_kernel(GroupedArgs p) {
-  constexpr int BM = Fast::kBM, BN = Fast::kBN, BK = Fast::kBK, NW = Fast::kNW, TM = Fast::kTM;
+  constexpr int BM = G::kBM, BN = G::kBN, BK = G::kBK, NW = G::kNW, TM = G::kTM;
   constexpr int WR = 1;  // every wavefront owns all rows of its 32 columns
   constexpr bool W4 = (BQT == QWIX_INT4);
   // e4m3 x e4m3: bytes travel like int8; two 16-byte fragments of consecutive k-steps make one operand of
@@ -883,22 +898,25 @@ __global__ void __launch_bounds__(Fast::kNW * 64) __attribute__((amdgpu_waves_pe
 }
 
 // LDS of the fast kernel: `st` slab stages, plus the f32 activation scales of the tile when they are per group.
-template <int BQT>
+template <int BQT, typename G = Fast>
 size_t grouped_dma_lds(bool sag, int64_t K, int64_t group, int st, int64_t zu_groups = 0) {
-  const size_t stages = st * (Fast::kBM * Fast::kBK + Fast::kBN * (BQT == QWIX_INT4 ? 64 : 128));
-  return stages + (sag ? static_cast<size_t>(K / group) * Fast::kBM * sizeof(float) : 0) +
-         static_cast<size_t>(zu_groups) * Fast::kBM * sizeof(int);
+  const size_t stages = st * (G::kBM * G::kBK + G::kBN * (BQT == QWIX_INT4 ? 64 : 128));
+  return stages + (sag ? static_cast<size_t>(K / group) * G::kBM * sizeof(float) : 0) +
+         static_cast<size_t>(zu_groups) * G::kBM * sizeof(int);
 }
 // rows of zero-point side values that ride along in LDS: one per group, one in all, or none
 inline int64_t zu_groups_of(const GroupedArgs& p) { return p.zu == nullptr ? 0 : (p.zu_sg != 0 ? p.K / p.group : 1); }
 constexpr size_t kLdsMax = 160 * 1024;
+// Up to this many 128 x 256 tiles the narrow geometries run instead (from about 128 tiles on the wide tile's reuse of
+// a weight fragment over four MFMAs wins: 512 x 14336 over K 4096, 224 tiles, 42.6 against 71.5 us).
+constexpr int64_t kNarrowTiles = 80;
 
-template <int BQT, bool SBF, bool SAG, bool AUX, bool MAGIC, int ST, bool ONE, bool DUMP = false>
+template <int BQT, bool SBF, bool SAG, bool AUX, bool MAGIC, int ST, bool ONE, bool DUMP = false, typename G = Fast>
 int launch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
-  constexpr int BM = Fast::kBM, BN = Fast::kBN, NW = Fast::kNW;
-  const size_t smem = grouped_dma_lds<BQT>(SAG, p.K, p.group, ST, zu_groups_of(p));
-  static_assert(ST * (Fast::kBM * Fast::kBK + BN * 64) >= NW * 32 * 36 * sizeof(float), "epilogue staging must fit");
-  auto kern = qgemm_grouped_dma_kernel<BQT, SBF, SAG, AUX, MAGIC, ST, ONE, DUMP>;
+  constexpr int BM = G::kBM, BN = G::kBN, NW = G::kNW;
+  const size_t smem = grouped_dma_lds<BQT, G>(SAG, p.K, p.group, ST, zu_groups_of(p));
+  static_assert(ST * (G::kBM * G::kBK + BN * 64) >= NW * 32 * 36 * sizeof(float), "epilogue staging must fit");
+  auto kern = qgemm_grouped_dma_kernel<BQT, SBF, SAG, AUX, MAGIC, ST, ONE, DUMP, G>;
   static LdsGrant granted;
   if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   const int64_t tiles = static_cast<int64_t>((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
@@ -919,6 +937,30 @@ int dispatch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
   if (p.zu != nullptr)  // an asymmetric operand
     return sbf ? launch_grouped_dma<BQT, true, SAG, true, false, 2, false>(p, st)
                : launch_grouped_dma<BQT, false, SAG, true, false, 2, false>(p, st);
+  if constexpr (!SAG) {
+    // Few 128 x 256 tiles (under a third of the CUs), or a decode batch: 128 x 64 tiles of two wavefronts, four times
+    // the workgroups; 32 or 64 rows per tile up to 64 rows.  int8 x int4 in groups of 128, weights from HBM, K 4096,
+    // N 4096, 16 / 64 / 128 / 512 rows: 35.7 / 36.5 / 38.4 / 39.0 us with the wide tile, 15.5 / 19.6 / 28.3 / 29.5 us now
+    // (K 8192, N 8192: 64.1 / 65.0 / 67.7 / 69.9 -> 27.2 / 34.7 / 49.1 / 70.0 us).
+    const int64_t wide = static_cast<int64_t>((p.M + Fast::kBM - 1) / Fast::kBM) * ((p.N + Fast::kBN - 1) / Fast::kBN);
+    if (wide <= kNarrowTiles || p.M <= 64) {
+      if (p.group == Fast::kBK && p.M <= 64) {  // decode batches: tiles of 32 or 64 rows
+        if (sbf && p.t_dtype == QWIX_BF16)
+          return p.M <= 32 ? launch_grouped_dma<BQT, true, false, false, true, 3, true, false, Narrow32>(p, st)
+                           : launch_grouped_dma<BQT, true, false, false, true, 3, true, false, Narrow64>(p, st);
+        if (!sbf)
+          return p.M <= 32 ? launch_grouped_dma<BQT, false, false, false, false, 3, true, false, Narrow32>(p, st)
+                           : launch_grouped_dma<BQT, false, false, false, false, 3, true, false, Narrow64>(p, st);
+      }
+      if (p.group == Fast::kBK) {
+        if (sbf && p.t_dtype == QWIX_BF16) return launch_grouped_dma<BQT, true, false, false, true, 3, true, false, Narrow>(p, st);
+        return sbf ? launch_grouped_dma<BQT, true, false, false, false, 3, true, false, Narrow>(p, st)
+                   : launch_grouped_dma<BQT, false, false, false, false, 3, true, false, Narrow>(p, st);
+      }
+      return sbf ? launch_grouped_dma<BQT, true, false, false, false, 2, false, false, Narrow>(p, st)
+                 : launch_grouped_dma<BQT, false, false, false, false, 2, false, false, Narrow>(p, st);
+    }
+  }
   if (p.group == Fast::kBK) {  // one slab per group
     if constexpr (!SAG) {
       // scaled partials that the reference keeps in bf16: the conversion-free fold
