@@ -924,6 +924,170 @@ int launch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
   return check_launch("qgemm_grouped (dma)");
 }
 
+// Decode batches (at most 32 rows) of the sub-channel GEMM with groups of 128 and one scale per token: the four
+// wavefronts of a workgroup share one 32 x 32 output tile and split K by groups (wavefront w takes groups w, w + 4,
+// ...).  Each wavefront streams its own slabs through a private three-stage ring in LDS (direct-to-LDS loads, its own
+// vmcnt waits, no barrier in the loop), multiplies a group with four MFMAs, folds it into f32 sums with the group's
+// weight scale (parked in LDS at the start), and the four partial sums meet in LDS once, at the end.  Against the
+// tile kernels that is four slabs in flight per workgroup and N / 32 workgroups of four independent wavefronts where
+// a decode batch left the tile kernel one 16-MFMA chain per slab: the arithmetic per output element is the same
+// (exact int32 partial per group, f32 fold, per-token scale and rounding at the end), the groups are added in another
+// order.
+template <int BQT, bool SBF>
+__global__ void __launch_bounds__(256) qgemm_grouped_decode_kernel(GroupedArgs p) {
+  constexpr bool W4 = (BQT == QWIX_INT4);
+  constexpr int BK = 128, NWV = 4, ST = 3;
+  constexpr int B_ROWB = W4 ? 64 : 128;
+  constexpr int A_BYTES = 32 * BK, B_BYTES = 32 * B_ROWB, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_LOADS = A_BYTES / 1024, B_LOADS = B_BYTES / 1024, L = A_LOADS + B_LOADS;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int KT = p.K / BK;
+  const int nw_max = (KT + NWV - 1) / NWV;              // groups of wavefront 0 (the most any wavefront has)
+  const int nw = (KT - wave + NWV - 1) / NWV;           // groups of this wavefront: wave, wave + 4, ...
+  const int tiles_n = (p.N + 31) / 32;
+  const int m0 = (static_cast<int>(blockIdx.x) / tiles_n) * 32, n0 = (static_cast<int>(blockIdx.x) % tiles_n) * 32;
+  uint8_t* wsm = smem + wave * (ST * STAGE + nw_max * 32 * static_cast<int>(sizeof(float)));
+  float* scl = reinterpret_cast<float*>(wsm + ST * STAGE);  // [group of this wavefront][column of the tile]
+
+  const uint8_t* a_base = p.A + static_cast<int64_t>(m0) * p.lda;
+  const uint8_t* b_base = p.B + static_cast<int64_t>(n0) * p.ldb;
+  uint32_t a_off[A_LOADS], b_off[B_LOADS];
+#pragma unroll
+  for (int j = 0; j < A_LOADS; ++j) {
+    const int row = j * 8 + (lane >> 3);
+    a_off[j] = static_cast<uint32_t>(min(row, p.M - 1 - m0)) * static_cast<uint32_t>(p.lda) + (((lane & 7) ^ swz128(row)) << 4);
+  }
+#pragma unroll
+  for (int j = 0; j < B_LOADS; ++j) {
+    int row, chunk;
+    if constexpr (W4) {
+      row = j * 16 + (lane >> 2);
+      chunk = (lane & 3) ^ ((lane >> 4) & 3);
+    } else {
+      row = j * 8 + (lane >> 3);
+      chunk = (lane & 7) ^ swz128(row);
+    }
+    b_off[j] = static_cast<uint32_t>(min(row, p.N - 1 - n0)) * static_cast<uint32_t>(p.ldb) + (chunk << 4);
+  }
+  auto issue_loads = [&](int s, int kt) __attribute__((always_inline)) {
+    const uint8_t* ga = a_base + static_cast<int64_t>(kt) * BK;
+    const uint8_t* gb = b_base + static_cast<int64_t>(kt) * B_ROWB;
+    uint8_t* ls = wsm + s * STAGE;
+#pragma unroll
+    for (int j = 0; j < A_LOADS; ++j) QWIX_GLDS16(ga + a_off[j], ls + j * 1024);
+#pragma unroll
+    for (int j = 0; j < B_LOADS; ++j) QWIX_GLDS16(gb + b_off[j], ls + A_BYTES + j * 1024);
+  };
+  if (nw > 0) issue_loads(0, wave);
+  if (nw > 1) issue_loads(1, wave + NWV);
+
+  // the weight scales of this wavefront's groups, one column per lane: lanes 0-31 take the even, lanes 32-63 the odd ones
+  const int frow = lane & 31, hx = lane >> 5;
+  const int ncl = min(n0 + frow, p.N - 1);
+  for (int i = hx; i < nw; i += 2) {
+    const int64_t at = static_cast<int64_t>(wave + i * NWV) * p.N + ncl;
+    float s;
+    if constexpr (SBF) s = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.sb)[at]);
+    else s = reinterpret_cast<const float*>(p.sb)[at];
+    scl[i * 32 + frow] = s * (W4 ? 0.0625f : 1.0f);  // the widened int4 weights carry a factor 16, exactly
+  }
+  // (the compiler's wait for these loads covers the two slabs requested above as well: they are needed next anyway)
+
+  const int a_row = frow * BK, a_sw = swz128(frow);
+  const int b_row = frow * B_ROWB, b_sw = W4 ? ((frow >> 2) & 3) : swz128(frow);
+  float accf[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) accf[r] = 0.f;
+  constexpr int W2 = 0x0F70 | ((2 * L) & 0xF) | (((2 * L) >> 4) << 14), W1 = 0x0F70 | (L & 0xF) | ((L >> 4) << 14);
+
+  int cur = 0;
+  for (int i = 0; i < nw; ++i) {
+    if (i + 2 < nw) issue_loads(cur == 0 ? 2 : cur - 1, wave + (i + 2) * NWV);  // the stage of slab i - 1
+    // this wavefront's slab i has landed once at most the slabs requested after it are outstanding
+    const int newer = min(nw - 1, i + 2) - i;
+    if (newer >= 2) __builtin_amdgcn_s_waitcnt(W2);
+    else if (newer == 1) __builtin_amdgcn_s_waitcnt(W1);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    __builtin_amdgcn_sched_barrier(0);
+    const uint8_t* sa_ = wsm + cur * STAGE + a_row;
+    const uint8_t* sb_ = wsm + cur * STAGE + A_BYTES + b_row;
+    v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (W4) {
+      v4i raw[2];
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) raw[pr] = *reinterpret_cast<const v4i*>(sb_ + (((2 * pr + hx) ^ b_sw) << 4));
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int chunk = 4 * (ks >> 1) + 2 * hx + (ks & 1);
+        const v4i fa = *reinterpret_cast<const v4i*>(sa_ + ((chunk ^ a_sw) << 4));
+        v4i fb;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const unsigned w = static_cast<unsigned>(raw[ks >> 1][2 * (ks & 1) + h]);
+          const unsigned ev = (w << 4) & 0xF0F0F0F0u, od = w & 0xF0F0F0F0u;  // nibbles 0,2,4,6 and 1,3,5,7, x 16
+          fb[2 * h] = static_cast<int>(__builtin_amdgcn_perm(od, ev, 0x05010400));
+          fb[2 * h + 1] = static_cast<int>(__builtin_amdgcn_perm(od, ev, 0x07030602));
+        }
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, acc, 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int chunk = 2 * ks + hx;
+        const v4i fa = *reinterpret_cast<const v4i*>(sa_ + ((chunk ^ a_sw) << 4));
+        const v4i fb = *reinterpret_cast<const v4i*>(sb_ + ((chunk ^ b_sw) << 4));
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, acc, 0, 0, 0);
+      }
+    }
+    const float sbg = scl[i * 32 + frow];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) accf[r] = __builtin_fmaf(static_cast<float>(acc[r]), sbg, accf[r]);
+    cur = cur == 2 ? 0 : cur + 1;
+  }
+
+  // the four partial sums meet in LDS (each wavefront writes into its own ring, then wavefront 0 adds them up)
+  float* red = reinterpret_cast<float*>(wsm);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) red[r * 64 + lane] = accf[r];
+  __syncthreads();
+  if (wave != 0) return;
+  const int wstride = (ST * STAGE + nw_max * 32 * static_cast<int>(sizeof(float))) / static_cast<int>(sizeof(float));
+#pragma unroll
+  for (int w = 1; w < NWV; ++w)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) accf[r] += red[w * wstride + r * 64 + lane];
+  const bool t_bf16 = (p.t_dtype == QWIX_BF16);
+  const int n = n0 + frow;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int m = m0 + 8 * (r >> 2) + 4 * hx + (r & 3);
+    if (m >= p.M || n >= p.N) continue;
+    float v = accf[r];
+    if (p.sa != nullptr) v *= ld_scale(p.sa, p.sa_dtype, m);
+    if (t_bf16) v = round_bf16(v);
+    if (p.out_dtype == QWIX_BF16)
+      reinterpret_cast<uint16_t*>(p.out)[static_cast<int64_t>(m) * p.ldo + n] = f32_to_bf16_bits(v);
+    else
+      reinterpret_cast<float*>(p.out)[static_cast<int64_t>(m) * p.ldo + n] = v;
+  }
+}
+
+template <int BQT, bool SBF>
+int launch_grouped_decode(const GroupedArgs& p, hipStream_t st) {
+  constexpr int STAGE = 32 * 128 + 32 * (BQT == QWIX_INT4 ? 64 : 128);
+  const int KT = p.K / 128, nw_max = (KT + 3) / 4;
+  const size_t smem = 4 * (3 * static_cast<size_t>(STAGE) + static_cast<size_t>(nw_max) * 32 * sizeof(float));
+  if (smem > kLdsMax) return -1;
+  auto kern = qgemm_grouped_decode_kernel<BQT, SBF>;
+  static LdsGrant granted;
+  if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
+  const int64_t tiles = static_cast<int64_t>((p.M + 31) / 32) * ((p.N + 31) / 32);
+  kern<<<dim3(static_cast<unsigned>(tiles)), 256, smem, st>>>(p);
+  return check_launch("qgemm_grouped (decode)");
+}
+
 // Picks the instantiation.  Returns -1 when the tile's per-group activation scales do not fit in LDS (the caller
 // then takes the register-staged kernel).
 template <int BQT, bool SAG>
@@ -938,6 +1102,15 @@ int dispatch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
     return sbf ? launch_grouped_dma<BQT, true, SAG, true, false, 2, false>(p, st)
                : launch_grouped_dma<BQT, false, SAG, true, false, 2, false>(p, st);
   if constexpr (!SAG) {
+    // A decode batch against groups of 128 with one scale per token: the kernel that splits K over wavefronts, while
+    // its N / 32 workgroups (each reads all the activation rows) are a few hundred.  int8 x int4, weights from HBM,
+    // 16 rows: K 4096, N 4096 15.5 -> 8.6 us, N 14336 16.0 -> 12.3, K 14336, N 4096 76.6 -> 19.9, K 8192, N 8192
+    // 27.2 -> 13.8; at N 28672 the narrow tiles are ahead (19.9 against 23.6 us), with int8 weights from N 14336 on.
+    if (p.M <= 32 && p.group == Fast::kBK && !p.single && p.ga == 1 && (p.K / Fast::kBK) >= 4 &&
+        p.N * (BQT == QWIX_INT4 ? 1 : 2) <= 16384 && 32 * p.lda < (int64_t{1} << 31) && 32 * p.ldb < (int64_t{1} << 31)) {
+      const int rc = sbf ? launch_grouped_decode<BQT, true>(p, st) : launch_grouped_decode<BQT, false>(p, st);
+      if (rc >= 0) return rc;
+    }
     // Few 128 x 256 tiles (under a third of the CUs), or a decode batch: 128 x 64 tiles of two wavefronts, four times
     // the workgroups; 32 or 64 rows per tile up to 64 rows.  int8 x int4 in groups of 128, weights from HBM, K 4096,
     // N 4096, 16 / 64 / 128 / 512 rows: 35.7 / 36.5 / 38.4 / 39.0 us with the wide tile, 15.5 / 19.6 / 28.3 / 29.5 us now

@@ -667,3 +667,36 @@ def test_decode_call_on_one_row_of_a_wider_matrix(wq_type, col0):
   row = big[3:4, col0:col0 + 1024]
   assert row.is_contiguous() and row.stride(0) == 1100
   assert torch.equal(dg.dot_general(row, wq, dn), dg.dot_general(row.clone(), wq, dn))
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('M,K,N', [(1, 512, 40), (5, 1024, 72), (16, 4096, 264), (32, 4224, 520), (17, 640, 32), (31, 896, 1000)])
+def test_grouped_gemm_decode_batches(M, K, N, wq_type, dtype):
+  """At most 32 rows against groups of 128 with one scale per token: the kernel whose four wavefronts split K by
+  groups (K / 128 = 4, 5, 7, 8, 32, 33 groups: every remainder of the split; column tiles that end inside the last
+  32).  Its outputs are the exact integer partials combined in f32: compared with their float64 combination."""
+  from qwix_amd.core import dot_general as dg
+  print('case grouped decode', M, K, N, wq_type, dtype, flush=True)
+  group = 128
+  xq, wq, oxq, owq, x_np, w_np = _pair(M, K, N, dtype, wq_type, group, seed=7 + M + N)
+  out = dg.dot_general(xq, wq, DN)
+  torch.cuda.synchronize()
+  want, wacc = O.fast_dot_general(oxq, owq, DN, return_acc=True)
+  got = util.f32np(out)
+  assert got.shape == (M, N)
+  assert np.all(np.abs(got - want.v) <= 1e-2 * np.abs(want.v) + util.partials_envelope(wacc, oxq, owq)), np.abs(got - want.v).max()
+  sa = np.asarray(oxq.scale.v, np.float64).reshape(M, 1)
+  sb = np.asarray(owq.scale.v, np.float64).reshape(K // group, 1, N)
+  parts = np.asarray(wacc, np.float64).reshape(K // group, M, N) * sb
+  exact, scale = parts.sum(0) * sa, np.abs(parts).sum(0) * sa
+  tol = 2.0 ** -7 if dtype is O.BF16 else 1e-5
+  assert np.all(np.abs(got - exact) <= tol * scale + 1e-30), (np.abs(got - exact) / (scale + 1e-30)).max()
+  # the same rows inside a larger batch go through the tile kernel: equal up to the order of the f32 additions
+  big_x = torch.cat([xq.qvalue, xq.qvalue.flip(0), xq.qvalue, xq.qvalue], 0)[:max(40, M)]
+  if big_x.shape[0] >= 40:
+    from qwix_amd.core.qarray import QArray
+    big_s = torch.cat([xq.scale, xq.scale.flip(0), xq.scale, xq.scale], 0)[:big_x.shape[0]]
+    if big_x.shape[0] == 40 and 4 * M >= 40:
+      tiled = util.f32np(dg.dot_general(QArray(big_x.contiguous(), big_s.contiguous(), None, 'int8'), wq, DN))[:M]
+      assert np.all(np.abs(tiled - got) <= tol * scale + 1e-30)
