@@ -555,6 +555,28 @@ class HadamardQdot(Workload):
     return {'workload': self.name, 'M': self.M, 'K': self.K, 'N': self.N, 'group': 128}
 
 
+class HadamardQdotDecode(HadamardQdot):
+  """C5 at a decode batch: the weight (int4 values + group scales) is streamed once per step, so the step is HBM-bound;
+  the figure is bytes of weights, scales, activations and outputs per second."""
+
+  bound = 'hbm'
+
+  def __init__(self, name, M, K, N):
+    super().__init__(name, M, K, N)
+    self.metric = 'Hadamard-rotated a8w4 g128 decode GB/s (FWHT + activation quantize included)'
+    self.unit = 'GB/s'
+    self.kernel_name = 'qgemm_grouped_decode_kernel'
+
+  def work_per_step(self):
+    return self.K * self.N / 2 + (self.K // 128) * self.N * 2 + self.M * self.K * 2 + self.M * self.N * 2
+
+  def kernel_work(self):
+    return self.K * self.N / 2 + (self.K // 128) * self.N * 2 + self.M * self.K + self.M * self.N * 2
+
+  def cpu_baseline(self, *a, **k):
+    return None
+
+
 class QdotSubChannel(Workload):
   """Sub-channel w8a8: per-token, per-group activation quantize each step (groups of `group` along K), then the
   sub-channel GEMM against a weight with one scale per group and output channel; qtype int8 or e4m3."""
@@ -1016,6 +1038,7 @@ WORKLOADS = {
     'batched_qk_int8_32x2048': lambda: QdotBatched('batched_qk_int8_32x2048', 32, 2048, 2048, 128),
     'c1_ptq_mlp_graph': lambda: PtqMlpGraph('c1_ptq_mlp_graph'),
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
+    'c5_hadamard_a8w4_decode_m16': lambda: HadamardQdotDecode('c5_hadamard_a8w4_decode_m16', 16, 8192, 8192),
     'int8_subchannel_g128_4096': lambda: QdotSubChannel('int8_subchannel_g128_4096', 4096, 4096, 4096, 128, 'int8'),
     'fp8_subchannel_g128_4096': lambda: QdotSubChannel('fp8_subchannel_g128_4096', 4096, 4096, 4096, 128, 'float8_e4m3fn'),
     'mfma_ceiling_int8_zeros': lambda: MfmaCeiling('mfma_ceiling_int8_zeros', 'int8', 'zeros'),
@@ -1031,7 +1054,7 @@ CEILING_EXTRA = ['mfma_ceiling_int8_zeros', 'mfma_ceiling_int8_gauss30', 'mfma_c
                  'mfma_ceiling_fp8_zeros', 'mfma_ceiling_fp8_gauss30', 'mfma_ceiling_fp8_operands']
 DEFAULT = 'c3_int8_w8a8_4096'
 EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c3_int8_w8a8_8192', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'c2_gemv_w4_m32', 'w8a16_gemv_m1', 'w8a16_gemv_m16', 'c2_w4a16_prefill_m2048', 'c2_w4a16_prefill_m512', 'c2_w4a16_prefill_m128', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
-         'c5_hadamard_a8w4', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'int8_subchannel_g128_4096', 'fp8_subchannel_g128_4096', 'moe_ragged_int8_8x1024',
+         'c5_hadamard_a8w4', 'c5_hadamard_a8w4_decode_m16', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'int8_subchannel_g128_4096', 'fp8_subchannel_g128_4096', 'moe_ragged_int8_8x1024',
          'moe_ragged_int8_64x128', 'moe_decode_int8_64x4', 'quantize_weight_fp8_block128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 
 

@@ -791,6 +791,15 @@ inline bool mfma_path_ok(int dtype, int logn, const void* x, const void* pre, co
          (post == nullptr || (reinterpret_cast<uintptr_t>(post) & 7) == 0);
 }
 
+// The matrix-core kernel runs a row per wavefront, 2048 rows per trip of the chip; the register kernel runs a row per
+// workgroup of four wavefronts.  Measured (rotate + quantize to int8): 16 / 256 / 1024 rows 12.9 / 13.3 / 15.4 us against
+// 5.8 / 6.0 / 9.8 us, 2048 rows 16.5 against 18.7, 3072 rows (two trips, the second half empty) 26.9 against 24.8, 8192
+// rows 51.8 against 57.2: the matrix-core kernel where whole trips of 2048 rows make it cheaper by this model.
+inline bool mfma_rows_pay(int64_t rows) {
+  const double trips = static_cast<double>((rows + 2047) / 2048);
+  return 4.5 + 11.8 * trips < 5.0 + 0.0065 * static_cast<double>(rows);
+}
+
 template <typename D, int MODE, int QT, int B>
 int launch_fwht_reg(const void* x, int64_t rows, const void* pre, const void* post, float out_scale, int ltile,
                     void* y, void* scale, hipStream_t st) {
@@ -849,7 +858,7 @@ extern "C" int qwix_hip_fwht(const void* x, int dtype, int64_t rows, int64_t n, 
   if (!y) return fail(QWIX_ERR_INVALID_ARGUMENT, "null output");
   const size_t smem = static_cast<size_t>(n + n / 8 + 8) * sizeof(float);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (mfma_path_ok(dtype, logn, x, pre_sign, post_sign, y))
+  if (mfma_rows_pay(rows) && mfma_path_ok(dtype, logn, x, pre_sign, post_sign, y))
     return launch_fwht_mfma<0, QWIX_INT8>(x, rows, pre_sign, post_sign, out_scale, logn, y, nullptr, st);
   if (reg_path_ok(logn, x, pre_sign, y) && (dtype == QWIX_BF16 || dtype == QWIX_F32)) {
     if (dtype == QWIX_BF16)
@@ -884,7 +893,7 @@ extern "C" int qwix_hip_fwht_quantize(const void* x, int dtype, int64_t rows, in
   hipStream_t st = static_cast<hipStream_t>(stream);
   int ltile = 0;
   while ((int64_t{1} << ltile) < tile) ++ltile;
-  if (mfma_path_ok(dtype, logn, x, pre_sign, post_sign, qvalue) && (qtype == QWIX_INT8 || qtype == QWIX_INT4 || qtype == QWIX_E4M3)) {
+  if (mfma_rows_pay(rows) && mfma_path_ok(dtype, logn, x, pre_sign, post_sign, qvalue) && (qtype == QWIX_INT8 || qtype == QWIX_INT4 || qtype == QWIX_E4M3)) {
     if (qtype == QWIX_INT8) return launch_fwht_mfma<1, QWIX_INT8>(x, rows, pre_sign, post_sign, out_scale, ltile, qvalue, scale, st);
     if (qtype == QWIX_INT4) return launch_fwht_mfma<1, QWIX_INT4>(x, rows, pre_sign, post_sign, out_scale, ltile, qvalue, scale, st);
     return launch_fwht_mfma<1, QWIX_E4M3>(x, rows, pre_sign, post_sign, out_scale, ltile, qvalue, scale, st);

@@ -29,9 +29,10 @@ def test_fwht_exact_on_small_integers(n):
     assert np.array_equal(util.f32np(yb), want.astype(np.float32))
 
 
-@pytest.mark.parametrize('rows', [3, 8, 37, 8200])
+@pytest.mark.parametrize('rows', [3, 8, 37, 2048, 4096])
 def test_matrix_core_rotation_exact_on_small_integers(rows):
-  """bf16 rows of 8192 take seven of the thirteen butterfly levels on the matrix cores (products with +-1 and f32 sums:
+  """bf16 rows of 8192 in whole trips of 2048 rows (2048, 4096: the matrix-core kernel; fewer rows: the register
+  kernel) take seven of the thirteen butterfly levels on the matrix cores (products with +-1 and f32 sums:
   exact on small integers like the butterflies), one wavefront per row.  Every partial sum of integers in [-4, 4] is an
   integer below 2^24, so the result is the exact transform rounded once to bf16, for any number of rows per wavefront,
   with and without the sign vectors in front of and behind the transform and the output factor."""
@@ -51,13 +52,16 @@ def test_matrix_core_rotation_exact_on_small_integers(rows):
   y2 = hr.fwht(xt, 1, pre_sign=dev(pre), post_sign=dev(post), out_scale=1.0 / n)
   want2 = O.round_to_bf16(O.round_to_bf16(((x * pre) @ H) * post) * np.float32(1.0 / n))
   assert np.array_equal(util.f32np(y2), want2)
-  # an impulse in every position of one row picks out one row of H: every index bit is where it belongs
-  if rows == 8:
-    for pos in (1, 4, 8, 32, 256, 512, 1024, 4096, 8191, 2730):
-      e = np.zeros((1, n), np.float32)
-      e[0, pos] = 3.0
-      ye = hr.fwht(torch.from_numpy(e).to(torch.bfloat16).to(util.DEV), 1)
-      assert np.array_equal(util.f32np(ye)[0], 3.0 * H[pos]), pos
+  # an impulse in one position of a row picks out one row of H: every index bit is where it belongs
+  # (8 rows: the register kernel; 2048 rows: one whole trip of the matrix-core kernel, which is what runs there)
+  if rows in (8, 2048):
+    places = (1, 4, 8, 32, 256, 512, 1024, 4096, 8191, 2730)
+    e = np.zeros((rows, n), np.float32)
+    for i in range(rows):
+      e[i, places[i % len(places)]] = 3.0
+    ye = util.f32np(hr.fwht(torch.from_numpy(e).to(torch.bfloat16).to(util.DEV), 1))
+    for i in list(range(min(rows, 20))) + [rows - 1]:
+      assert np.array_equal(ye[i], 3.0 * H[places[i % len(places)]]), i
 
 
 @pytest.mark.parametrize('qtype,tile', [('int8', None), ('int8', 8), ('int4', 16), ('float8_e4m3fn', 32), ('int8', 64), ('int4', 128),
