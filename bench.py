@@ -394,6 +394,9 @@ class WeightOnlyPrefill(Workload):
     self.out = torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev)
     self.stream = torch.cuda.current_stream().cuda_stream
     self.L = L
+    # few tiles (the down projection's N 4096): K in ranges, f32 partials in a workspace, as the operator calls it
+    self.nws = int(L.load().qwix_hip_gemm_bf16_wq_workspace_bytes(self.M, self.N, self.K, self.group)) if self.fused else 0
+    self.ws = torch.empty(max(self.nws, 16), dtype=torch.uint8, device=dev)
 
   def step(self, i=0):
     L = self.L
@@ -405,8 +408,9 @@ class WeightOnlyPrefill(Workload):
   def kernel(self, i=0):
     L = self.L
     if self.fused:
-      L.call('qwix_hip_gemm_bf16_wq', self.x.data_ptr(), self.K, self.b.data_ptr(), self.b.stride(0), L.INT4, self.M,
-             self.N, self.K, self.group, self.s.data_ptr(), L.F32, None, self.out.data_ptr(), L.BF16, self.N, self.stream)
+      L.call('qwix_hip_gemm_bf16_wq_ws', self.x.data_ptr(), self.K, self.b.data_ptr(), self.b.stride(0), L.INT4, self.M,
+             self.N, self.K, self.group, self.s.data_ptr(), L.F32, None, self.out.data_ptr(), L.BF16, self.N,
+             self.ws.data_ptr() if self.nws else None, self.nws, self.stream)
       return
     L.call('qwix_hip_gemm_bf16', self.x.data_ptr(), self.K, self.w.data_ptr(), self.K, self.M, self.N, self.K,
            self.out.data_ptr(), L.BF16, self.N, self.stream)
@@ -1022,6 +1026,7 @@ WORKLOADS = {
     'c2_w4a16_prefill_m2048': lambda: WeightOnlyPrefill('c2_w4a16_prefill_m2048', 2048, 4096, 14336, 128),
     'c2_w4a16_prefill_m512': lambda: WeightOnlyPrefill('c2_w4a16_prefill_m512', 512, 4096, 14336, 128),
     'c2_w4a16_prefill_m128': lambda: WeightOnlyPrefill('c2_w4a16_prefill_m128', 128, 4096, 14336, 128),
+    'c2_w4a16_prefill_m128_down': lambda: WeightOnlyPrefill('c2_w4a16_prefill_m128_down', 128, 14336, 4096, 128),
     'c4_quantize_weight_fp8': lambda: QuantizeWeight('c4_quantize_weight_fp8', 8192, 28672, 'float8_e4m3fn'),
     'c5_quantize_weight_int4_g128': lambda: QuantizeWeight('c5_quantize_weight_int4_g128', 8192, 8192, 'int4', 128),
     'c3_quantize_weight_int8': lambda: QuantizeWeight('c3_quantize_weight_int8', 4096, 4096, 'int8'),
@@ -1053,7 +1058,7 @@ CEILINGS = {'int8': 'mfma_ceiling_int8_operands', 'f8e4m3': 'mfma_ceiling_fp8_op
 CEILING_EXTRA = ['mfma_ceiling_int8_zeros', 'mfma_ceiling_int8_gauss30', 'mfma_ceiling_int8_operands',
                  'mfma_ceiling_fp8_zeros', 'mfma_ceiling_fp8_gauss30', 'mfma_ceiling_fp8_operands']
 DEFAULT = 'c3_int8_w8a8_4096'
-EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c3_int8_w8a8_8192', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'c2_gemv_w4_m32', 'w8a16_gemv_m1', 'w8a16_gemv_m16', 'c2_w4a16_prefill_m2048', 'c2_w4a16_prefill_m512', 'c2_w4a16_prefill_m128', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
+EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c3_int8_w8a8_8192', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'c2_gemv_w4_m32', 'w8a16_gemv_m1', 'w8a16_gemv_m16', 'c2_w4a16_prefill_m2048', 'c2_w4a16_prefill_m512', 'c2_w4a16_prefill_m128', 'c2_w4a16_prefill_m128_down', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
          'c5_hadamard_a8w4', 'c5_hadamard_a8w4_decode_m16', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'int8_subchannel_g128_4096', 'fp8_subchannel_g128_4096', 'moe_ragged_int8_8x1024',
          'moe_ragged_int8_64x128', 'moe_decode_int8_64x4', 'quantize_weight_fp8_block128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 

@@ -342,6 +342,18 @@ QWIX_API int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, in
                           int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, const int8_t* zp,
                           void* out, int out_dtype, int64_t ldo, void* stream);
 
+/* qwix_hip_gemm_bf16_wq with K cut into ranges while its tiles would cover at most half of the CUs (the same call in
+ * the reference: _slow_dot_general, qwix/_src/core/dot_general.py:264-275): every range's workgroups write f32
+ * partials into `workspace` (qwix_hip_gemm_bf16_wq_workspace_bytes(M, N, K, group) bytes, 16-byte aligned; 0 = this
+ * shape is not split) and a second kernel adds them in range order and rounds once to out_dtype.  The f32 sums are
+ * then formed in another order than the unsplit kernel's, so results agree with qwix_hip_gemm_bf16_wq to f32
+ * rounding of the accumulation, not bit for bit.  With workspace NULL or too small: exactly qwix_hip_gemm_bf16_wq. */
+QWIX_API size_t qwix_hip_gemm_bf16_wq_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group);
+QWIX_API int qwix_hip_gemm_bf16_wq_ws(const void* a, int64_t lda, const void* q, int64_t ldq_bytes, int q_qtype, int64_t M,
+                             int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, const int8_t* zp,
+                             void* out, int out_dtype, int64_t ldo, void* workspace, size_t workspace_bytes,
+                             void* stream);
+
 /* dequantize (qarray.py:692-708) of a REDUCE_MINOR qvalue that keeps that layout: out[(o, i, r)] =
  * D(D(q - zp) * scale[o, r / tile, i]) as a row-major (outer, inner, reduce) array, the K-contiguous operand
  * qwix_hip_gemm_bf16 reads.  D = `dtype` = the scale dtype; out_dtype is `dtype`, or QWIX_BF16 for f32 scales

@@ -55,6 +55,8 @@ SIGNATURES = {
     'qwix_hip_ksum_groups': (_int, [_vp, _int, _i64, _i64, _i64, _i64, _vp, _vp]),
     'qwix_hip_gemm_bf16': (_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
     'qwix_hip_gemm_bf16_wq': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _int, _i64, _vp]),
+    'qwix_hip_gemm_bf16_wq_workspace_bytes': (_sz, [_i64, _i64, _i64, _i64]),
+    'qwix_hip_gemm_bf16_wq_ws': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _int, _i64, _vp, _sz, _vp]),
     'qwix_hip_dequantize_rm': (_int, [_vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _int, _vp, _int, _vp]),
     'qwix_hip_gemv_wq': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _vp, _int, _i64, _vp]),
     'qwix_hip_gemv_wq_zp': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _int, _i64, _vp]),

@@ -717,7 +717,7 @@ def _decode_plan(lhs, rhs, dimension_numbers):
     sb, gb = c.rhs_scale(rhs)
     zp = _rhs_zero_point_i8(c, rhs)[0] if rhs.zero_point is not None else None
     plan = (b, numerics.qtype_tag(_qtype_of(rhs)), sb, _lib.float_tag(sb.dtype), zp, c.N, c.K, c.K // gb,
-            fused_wq_min_rows(c.N, b_is4))
+            fused_wq_min_rows(c.N, b_is4, c.K, c.K // gb))
   _DECODE_PLANS[key] = (weakref.ref(rhs, lambda _, k=key: _DECODE_PLANS.pop(k, None)),
                         _weight_signature(rhs), plan)
   return plan
@@ -763,7 +763,8 @@ def _slow_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
   if out is not None:
     return out
   c = _weight_only_fit(lhs, rhs, dimension_numbers)
-  if c is not None and fused_wq_min_rows(c.N, isinstance(rhs.qvalue, Int4Tensor)) < c.M <= WEIGHT_ONLY_MAX_ROWS:
+  if c is not None and (fused_wq_min_rows(c.N, isinstance(rhs.qvalue, Int4Tensor), c.K, c.K // rhs.scale.shape[c.rca[-1]])
+                        < c.M <= WEIGHT_ONLY_MAX_ROWS):
     # one row tile of the dequantizing tile GEMM beats the decode kernel from here on
     out = _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_type, fused_only=True)
     if out is not None:
@@ -818,12 +819,18 @@ def _fused_wq_takes(m: int, n: int, int4: bool) -> bool:
 _FUSED_W8_MAX_TILES = 256
 
 
-def fused_wq_min_rows(n: int, int4: bool = True) -> int:
+def fused_wq_min_rows(n: int, int4: bool = True, k: int = 0, group: int = 0) -> int:
   """Rows above which the dequantizing tile GEMM beats the decode kernel (`qwix_hip_gemv_wq`).  The time of one row
   tile does not depend on the rows (K 4096, up to 128 rows, tiles of 128 x 64: int4 29 / 26 us at N 14336 / 4096, int8
   29 / 25 us; 129-256 rows, tiles of 256 x 64: 45 us); the decode kernel's grows with them in steps of 16 rows and
   falls with N (K 4096, int4, 64 / 80 / 96 / 128 rows: N 14336 26 / 35 / 38 / 48 us, N 4096 21 / 23 / 28 / 35 us; int8,
-  32 / 48 / 64 / 80 rows: N 14336 23 / 31 / 35 / 46 us, N 4096 12 / 17 / 21 / 26 us)."""
+  32 / 48 / 64 / 80 rows: N 14336 23 / 31 / 35 / 46 us, N 4096 12 / 17 / 21 / 26 us).
+  Where the tile GEMM cuts K into ranges (given `k` and `group`: few tiles, `qwix_hip_gemm_bf16_wq_ws`) it wins earlier.
+  Weights from HBM, decode kernel at 32 / 48 / 64 rows against the tile GEMM's one time up to 128 rows: int4 K 4096,
+  N 4096 12 / 15 / 21 against 15 us; K 8192, N 8192 23 / 29 / 40 against 33; K 14336, N 4096 34 / 45 / 64 against 31;
+  int8 13 / 17 / 21 against 15; 25 / 40 / 48 against 34; 35 / 55 / 67 against 32."""
+  if k and group and _lib.load().qwix_hip_gemm_bf16_wq_workspace_bytes(64, n, k, group):
+    return 48 if int4 else 32
   if int4:
     return 64 if n >= 12288 else 80
   return 32 if n >= 12288 else 64
@@ -871,9 +878,12 @@ def _dequantize_then_bf16_gemm(lhs, rhs, dimension_numbers, preferred_element_ty
     # int4 / int8 with or without zero points, e4m3: dequantized inside the GEMM's workgroups, slab by slab (the same
     # bf16 weights, the same products in the same order, no dequantized copy of the weight in memory)
     out = torch.empty(c.M, c.N, dtype=res_t, device=dev)
-    _lib.call('qwix_hip_gemm_bf16_wq', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0),
+    # few tiles: K in ranges over more workgroups, f32 partials in a workspace (0 bytes = not split)
+    nws = int(_lib.load().qwix_hip_gemm_bf16_wq_workspace_bytes(c.M, c.N, c.K, c.K // gb))
+    ws = torch.empty(nws, dtype=torch.uint8, device=dev) if nws else None
+    _lib.call('qwix_hip_gemm_bf16_wq_ws', x.data_ptr(), x.stride(0), b.data_ptr(), b.stride(0),
               numerics.qtype_tag(_qtype_of(rhs)), c.M, c.N, c.K, c.K // gb, sb.data_ptr(), _lib.float_tag(sb.dtype),
-              _lib.ptr(zp), out.data_ptr(), _lib.float_tag(res_t), c.N, st)
+              _lib.ptr(zp), out.data_ptr(), _lib.float_tag(res_t), c.N, _lib.ptr(ws), nws, st)
     return out.reshape(c.out_shape)
   if fused_only:
     return None

@@ -2158,8 +2158,20 @@ template <int OUT, bool SBF, int BM, int BN, int BITS, bool ZP>
 __global__ void __launch_bounds__(512)
     wgemm_wq_kernel(const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ Q, int64_t ldq,
                     const void* __restrict__ S, const int8_t* __restrict__ Z, int M, int N, int K, int group,
-                    uint8_t* __restrict__ out, int64_t ldo) {
+                    uint8_t* __restrict__ out, int64_t ldo, int ksplit) {
   static_assert((BM == 256 && (BN == 128 || BN == 64)) || (BM == 128 && BN == 64), "tiles of 256 x 128, 256 x 64, 128 x 64");
+  if (ksplit > 0) {
+    // K split over blockIdx.y: this workgroup contracts elements [y ksplit, (y + 1) ksplit) -- ksplit a multiple of 256
+    // and of the group that divides K -- and writes its tile of the y-th M x N partial (the host passes OUT = f32 and
+    // ldo = N); every operand pointer moves to the range's first element.
+    const int k0 = static_cast<int>(blockIdx.y) * ksplit;
+    A += static_cast<int64_t>(k0) * 2;
+    Q += (BITS >= 8) ? k0 : k0 / 2;
+    S = static_cast<const char*>(S) + static_cast<int64_t>(k0 / group) * N * (SBF ? 2 : 4);
+    if constexpr (ZP) Z += static_cast<int64_t>(k0 / group) * N;
+    out += static_cast<int64_t>(blockIdx.y) * M * N * 4;
+    K = ksplit;
+  }
   constexpr int WGN = 2, WN = BN / WGN, TM = 2, TN = WN / 32, NWAVES = BM / 32, NTHREADS = NWAVES * 64;
   constexpr int BK = 128, NK = 4;  // bytes of an activation row per slab (64 elements); k-steps of 16 elements
   static_assert(BITS == 4 || BITS == 8 || BITS == 9, "int4, int8 or (9) e4m3 weights");
@@ -2751,9 +2763,32 @@ extern "C" int qwix_hip_gemm_bf16(const void* a, int64_t lda, const void* b, int
   return launch_dma<kOpBf16, 128, 128, 2, 2, QWIX_F32, 0>(a, ldab, b, ldbb, M, N, kb, ep, out, ldo, st);
 }
 
-extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, int64_t ldq_bytes, int q_qtype, int64_t M,
-                                     int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, const int8_t* zp,
-                                     void* out, int out_dtype, int64_t ldo, void* stream) {
+template <bool IS_INT>
+__global__ void __launch_bounds__(256)
+    splitk_reduce_kernel(const uint8_t* __restrict__ ws, int splits, int M, int N, Epilogue ep, uint8_t* __restrict__ out,
+                         int64_t ldo);  // defined with the split-K kernels of the quantized GEMM below
+
+// The K split of qwix_hip_gemm_bf16_wq_ws: 0 = none.  The tile kernel walks K in 64-element slabs of about 0.37 us
+// each, however few workgroups there are; while they cover at most half of the CUs, K is cut into equal ranges (whole
+// 256-element superslabs and scale groups, at least 1024 elements) for up to one workgroup per CU.
+static int wq_splits(int64_t M, int64_t N, int64_t K, int64_t group) {
+  if (M <= 0 || N <= 0 || K <= 0 || group <= 0 || K % 256 || group % 64 || K % group) return 0;
+  const bool low = M <= 128;
+  const bool narrow = ((M + 255) / 256) * ((N + 127) / 128) <= 128;
+  const int64_t tiles = ((M + (low ? 127 : 255)) / (low ? 128 : 256)) * ((N + (low || narrow ? 63 : 127)) / (low || narrow ? 64 : 128));
+  if (tiles > 128) return 0;
+  int64_t unit = 256;  // a range is a multiple of 256 and of the group: of lcm(256, group)
+  while (unit % group) unit += 256;
+  int best = 0;
+  for (int64_t sp = 2; sp * tiles <= 256 && sp * 1024 <= K; ++sp)
+    if (K % (sp * unit) == 0) best = static_cast<int>(sp);
+  return best;
+}
+
+static int gemm_bf16_wq_impl(const void* a, int64_t lda, const void* q, int64_t ldq_bytes, int q_qtype, int64_t M,
+                             int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, const int8_t* zp,
+                             void* out, int out_dtype, int64_t ldo, void* stream, void* workspace,
+                             size_t workspace_bytes) {
   if (!a || !q || !s || !out) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/q/s/out");
   if (q_qtype != QWIX_INT4 && q_qtype != QWIX_INT8 && q_qtype != QWIX_E4M3)
     return fail(QWIX_ERR_UNSUPPORTED, "weight qtype %d: int4, int8 or e4m3", q_qtype);
@@ -2779,6 +2814,13 @@ extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, 
   const bool narrow = ((M + 255) / 256) * ((N + 127) / 128) <= 128;
   const bool low = M <= 128;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  // with a workspace that holds them: f32 partials of `splits` K ranges, added up (in range order) by a second kernel
+  int splits = workspace ? wq_splits(M, N, K, group) : 0;
+  if (splits > 0 && (workspace_bytes < static_cast<size_t>(splits) * M * N * 4 || !aligned16(workspace))) splits = 0;
+  const int ksplit = splits > 0 ? static_cast<int>(K / splits) : 0;
+  const int kern_out = splits > 0 ? QWIX_F32 : out_dtype;
+  uint8_t* const kern_dst = static_cast<uint8_t*>(splits > 0 ? workspace : out);
+  const int64_t kern_ldo = splits > 0 ? N : ldo;
 #define QWIX_WQ_LAUNCH(OUTT, SBFF, BMM, BNN, BITS) \
   do {                                             \
     if (zp) QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BMM, BNN, BITS, (BITS != 9)); else QWIX_WQ_LAUNCH_Z(OUTT, SBFF, BMM, BNN, BITS, false); \
@@ -2788,12 +2830,13 @@ extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, 
     auto kern = wgemm_wq_kernel<OUTT, SBFF, BMM, BNN, BITS, ZPP>;                                                    \
     /* activations 96 KB, converted weights 2 x BN x 128, raw weights 2 x BN x 128 (int8: 4 x 8 KB): <= 160 KB */    \
     constexpr size_t smem = (BMM == 128 ? 4 : 3) * BMM * 128 + 2 * BNN * 128 + (BITS >= 8 ? 4 * (BMM / 32) * 1024 : 2 * BNN * 128);      \
-    const dim3 grid(static_cast<unsigned>(((M + BMM - 1) / BMM) * ((N + BNN - 1) / BNN)));                           \
+    const dim3 grid(static_cast<unsigned>(((M + BMM - 1) / BMM) * ((N + BNN - 1) / BNN)),                            \
+                    static_cast<unsigned>(splits > 0 ? splits : 1));                                                 \
     static LdsGrant granted;                                                                                         \
     if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;                           \
     kern<<<grid, 512, smem, st>>>(static_cast<const uint8_t*>(a), 2 * lda, static_cast<const uint8_t*>(q), ldq_bytes, s, \
                                   zp, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K),                 \
-                                  static_cast<int>(group), static_cast<uint8_t*>(out), ldo);                         \
+                                  static_cast<int>(group), kern_dst, kern_ldo, ksplit);                              \
   } while (0)
 #define QWIX_WQ_TILE(OUTT, SBFF, BITS)                                                                               \
   do {                                                                                                               \
@@ -2807,7 +2850,7 @@ extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, 
     else if (q_qtype == QWIX_INT8) QWIX_WQ_TILE(OUTT, SBFF, 8);                                                      \
     else QWIX_WQ_TILE(OUTT, SBFF, 9); /* e4m3 */                                                                     \
   } while (0)
-  if (out_dtype == QWIX_BF16) {
+  if (kern_out == QWIX_BF16) {
     if (s_dtype == QWIX_BF16) QWIX_WQ_BITS(QWIX_BF16, true); else QWIX_WQ_BITS(QWIX_BF16, false);
   } else {
     if (s_dtype == QWIX_BF16) QWIX_WQ_BITS(QWIX_F32, true); else QWIX_WQ_BITS(QWIX_F32, false);
@@ -2816,7 +2859,35 @@ extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, 
 #undef QWIX_WQ_TILE
 #undef QWIX_WQ_LAUNCH
 #undef QWIX_WQ_LAUNCH_Z
-  return check_launch("gemm_bf16_wq");
+  if (int e = check_launch("gemm_bf16_wq")) return e;
+  if (splits > 0) {
+    const Epilogue ep{nullptr, nullptr, 0, 0, out_dtype, 0, 0, 0, nullptr, nullptr};
+    const int64_t threads = (M * N + 3) / 4;
+    splitk_reduce_kernel<false><<<dim3(static_cast<unsigned>((threads + 255) / 256)), 256, 0, st>>>(
+        static_cast<const uint8_t*>(workspace), splits, static_cast<int>(M), static_cast<int>(N), ep,
+        static_cast<uint8_t*>(out), ldo);
+    return check_launch("gemm_bf16_wq (split K)");
+  }
+  return 0;
+}
+
+extern "C" int qwix_hip_gemm_bf16_wq(const void* a, int64_t lda, const void* q, int64_t ldq_bytes, int q_qtype, int64_t M,
+                                     int64_t N, int64_t K, int64_t group, const void* s, int s_dtype, const int8_t* zp,
+                                     void* out, int out_dtype, int64_t ldo, void* stream) {
+  return gemm_bf16_wq_impl(a, lda, q, ldq_bytes, q_qtype, M, N, K, group, s, s_dtype, zp, out, out_dtype, ldo, stream,
+                           nullptr, 0);
+}
+
+extern "C" size_t qwix_hip_gemm_bf16_wq_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group) {
+  return static_cast<size_t>(wq_splits(M, N, K, group)) * static_cast<size_t>(M > 0 ? M : 0) * static_cast<size_t>(N > 0 ? N : 0) * 4;
+}
+
+extern "C" int qwix_hip_gemm_bf16_wq_ws(const void* a, int64_t lda, const void* q, int64_t ldq_bytes, int q_qtype,
+                                        int64_t M, int64_t N, int64_t K, int64_t group, const void* s, int s_dtype,
+                                        const int8_t* zp, void* out, int out_dtype, int64_t ldo, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
+  return gemm_bf16_wq_impl(a, lda, q, ldq_bytes, q_qtype, M, N, K, group, s, s_dtype, zp, out, out_dtype, ldo, stream,
+                           workspace, workspace_bytes);
 }
 
 extern "C" int qwix_hip_qgemm(const void* a, int64_t lda, const void* b, int64_t ldb, int qtype, int64_t M,

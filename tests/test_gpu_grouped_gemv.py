@@ -264,12 +264,14 @@ def test_weight_only_gemv_asymmetric_weights(M, K, N, group, sdt, wq_type):
 @pytest.mark.parametrize('wq_type', ['int4', 'int8', 'float8_e4m3fn'])
 @pytest.mark.parametrize('M', [1, 20, 40])
 @pytest.mark.parametrize('K,N,group', [(384, 72, 128), (4224, 136, 128), (16384, 264, 256), (8192, 2048, 128), (128, 48, 128)])
-def test_weight_only_gemv_k_splits(M, K, N, group, wq_type):
+def test_weight_only_gemv_k_splits(M, K, N, group, wq_type, monkeypatch):
   """How the wavefronts of the weight-only kernel share K: an odd number of 128-wide blocks (a last, single block
   after the pairs), one block in all, and so many blocks that a wavefront makes several trips (the next pair's
-  weights are requested while this pair is multiplied); N that ends inside a column tile."""
+  weights are requested while this pair is multiplied); N that ends inside a column tile.  (The decode kernel at every
+  row count: the operator's switch to the dequantizing tile GEMM is held off.)"""
   from qwix_amd.core import dot_general as dg
   from qwix_amd.core import qarray
+  monkeypatch.setattr(dg, 'fused_wq_min_rows', lambda *args: dg.WEIGHT_ONLY_MAX_ROWS)
   print('case gemv k-split', M, K, N, group, wq_type, flush=True)
   x_np, x_t = util.make((M, K), O.BF16, seed=M + K + 5)
   w_np, w_t = util.make((K, N), O.BF16, seed=N + K + 6, scale=0.02)
@@ -293,7 +295,7 @@ def test_weight_only_rows_do_not_depend_on_the_batch(M, K, N, wq_type, monkeypat
   the dequantizing tile GEMM, which rounds every weight to bf16 first, is held off.)"""
   from qwix_amd.core import dot_general as dg
   from qwix_amd.core import qarray
-  monkeypatch.setattr(dg, 'fused_wq_min_rows', lambda n, int4=True: dg.WEIGHT_ONLY_MAX_ROWS)
+  monkeypatch.setattr(dg, 'fused_wq_min_rows', lambda *args: dg.WEIGHT_ONLY_MAX_ROWS)
   print('case gemv batch', M, K, N, wq_type, flush=True)
   _, x_t = util.make((M, K), O.BF16, seed=M + K)
   _, w_t = util.make((K, N), O.BF16, seed=M + K + 1, scale=0.02)
@@ -553,6 +555,65 @@ def test_prefill_with_f32_scales_stays_within_a_bf16_rounding_of_the_f32_contrac
   assert np.allclose(got, want, rtol=1e-2, atol=1e-2 * mag), np.abs(got - want).max() / mag
 
 
+@pytest.mark.parametrize('sdt', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('wq_type,asym', [('int4', False), ('int4', True), ('int8', False), ('int8', True),
+                                          ('float8_e4m3fn', False)])
+@pytest.mark.parametrize('M,K,N,group,splits', [(128, 4096, 1024, 128, 4), (96, 14336, 520, 128, 14), (300, 2048, 136, 64, 2),
+                                                (512, 4096, 1000, 256, 4), (64, 8192, 264, 512, 8), (130, 3072, 72, 1024, 3),
+                                                (2048, 4096, 1536, 128, 0), (64, 1024, 64, 128, 0)])
+def test_prefill_gemm_k_ranges(M, K, N, group, splits, asym, wq_type, out_dtype, sdt):
+  """qwix_hip_gemm_bf16_wq_ws: K in `splits` ranges with f32 partials in a workspace while the tiles are few (edges in
+  M and N, groups of 64 to 1024, ranges of 1024 elements and more).  Against the unsplit kernel: another order of the
+  f32 sums, so equal to 2^-18 of the mean magnitude (plus one bf16 step, 2^-7 relative, for bf16 results); with no workspace, and
+  for shapes that are not split (workspace size 0), the very same bits."""
+  from qwix_amd import _lib
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import numerics
+  from qwix_amd.core import qarray
+  print('case wq k ranges', M, K, N, group, splits, asym, wq_type, out_dtype, sdt, flush=True)
+  x_np, x_t = util.make((M, K), O.BF16, seed=M + K + 41)
+  w_np, w_t = util.make((K, N), O.BF16, seed=N + K + 42, scale=0.02)
+  kw = dict(calibration_method='minmax') if asym else {}
+  if asym:
+    w_t = (w_t.float() + 0.013).to(torch.bfloat16)
+  wq = qarray.quantize_api(w_t, wq_type, channelwise_axes=[1], tiled_axes={0: group}, scale_dtype=sdt, **kw)
+  c = dg._Canon(x_t, wq, DN)
+  b, _ = c.rhs_values(wq)
+  sb, gb = c.rhs_scale(wq)
+  assert gb == K // group
+  tag = numerics.qtype_tag(wq_type)
+  st = _lib.stream_of(x_t)
+  zp = dg._rhs_zero_point_i8(c, wq)[0] if asym else None
+  nws = int(_lib.load().qwix_hip_gemm_bf16_wq_workspace_bytes(M, N, K, group))
+  assert nws == splits * M * N * 4
+  want = torch.empty(M, N, dtype=out_dtype, device=util.DEV)
+  _lib.call('qwix_hip_gemm_bf16_wq', x_t.data_ptr(), K, b.data_ptr(), b.stride(0), tag, M, N, K, group, sb.data_ptr(),
+            _lib.float_tag(sb.dtype), _lib.ptr(zp), want.data_ptr(), _lib.float_tag(out_dtype), N, st)
+
+  def run(ws, n):
+    got = torch.full((M, N), float('nan'), dtype=out_dtype, device=util.DEV)
+    _lib.call('qwix_hip_gemm_bf16_wq_ws', x_t.data_ptr(), K, b.data_ptr(), b.stride(0), tag, M, N, K, group,
+              sb.data_ptr(), _lib.float_tag(sb.dtype), _lib.ptr(zp), got.data_ptr(), _lib.float_tag(out_dtype), N,
+              _lib.ptr(ws), n, st)
+    torch.cuda.synchronize()
+    return got
+
+  assert torch.equal(run(None, 0), want)
+  if not splits:
+    return
+  ws = torch.full((nws,), 0xFF, dtype=torch.uint8, device=util.DEV)  # NaN patterns: every partial must be written
+  assert torch.equal(run(ws, nws - 1), want)  # too small a workspace: not split
+  got = util.f32np(run(ws, nws))
+  ref = util.f32np(want)
+  mag = np.abs(ref).mean()
+  tol = 2.0 ** -18 * mag * np.sqrt(K / 1024) + (2.0 ** -7 * np.abs(ref) if out_dtype == torch.bfloat16 else 0)
+  assert np.all(np.abs(got - ref) <= tol + 1e-30), (np.abs(got - ref) / (tol + 1e-30)).max()
+  # and through the operator, which passes the workspace
+  res = dg._dequantize_then_bf16_gemm(x_t, wq, DN, out_dtype, fused_only=True)
+  assert res is not None and np.array_equal(util.f32np(res), got)
+
+
 def test_dequantizing_gemm_argument_checks():
   """qwix_hip_gemm_bf16_wq refuses what its tile loop cannot walk (K not in whole groups of four slabs, groups that
   are not whole slabs, unaligned rows, other weight types) with an error code and a message instead of launching."""
@@ -636,7 +697,7 @@ def test_weight_only_prefill_on_hip_kernels(M, K, N, case):
   got = util.f32np(out)
   assert np.allclose(got, want.v, rtol=1e-2, atol=1e-2 * np.abs(want.v).mean()), np.abs(got - want.v).max()
   # the operator takes this path from the row count on at which the dequantizing tile GEMM beats the decode kernel
-  if M > dg.fused_wq_min_rows(N, wq_type == 'int4'):
+  if M > dg.fused_wq_min_rows(N, wq_type == 'int4', K, group or K):
     assert torch.equal(dg.dot_general(x_t, wq, DN, preferred_element_type=torch.bfloat16), out)
   # the dequantized operand itself, against the oracle's dequantize
   c = dg._Canon(x_t, wq, DN)
