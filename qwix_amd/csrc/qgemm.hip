@@ -2161,9 +2161,10 @@ __global__ void __launch_bounds__(512)
                     uint8_t* __restrict__ out, int64_t ldo, int ksplit) {
   static_assert((BM == 256 && (BN == 128 || BN == 64)) || (BM == 128 && BN == 64), "tiles of 256 x 128, 256 x 64, 128 x 64");
   if (ksplit > 0) {
-    // K split over blockIdx.y: this workgroup contracts elements [y ksplit, (y + 1) ksplit) -- ksplit a multiple of 256
-    // and of the group that divides K -- and writes its tile of the y-th M x N partial (the host passes OUT = f32 and
-    // ldo = N); every operand pointer moves to the range's first element.
+    // K split over blockIdx.y: this workgroup contracts elements [y ksplit, (y + 1) ksplit) -- ksplit a multiple of 256,
+    // and a multiple or a divisor of the group, so that a range starts a group or lies inside one -- and writes its tile
+    // of the y-th M x N partial (the host passes OUT = f32 and ldo = N); every operand pointer moves to the range's
+    // first element (the scales': to the group that holds it).
     const int k0 = static_cast<int>(blockIdx.y) * ksplit;
     A += static_cast<int64_t>(k0) * 2;
     Q += (BITS >= 8) ? k0 : k0 / 2;
@@ -2770,18 +2771,21 @@ __global__ void __launch_bounds__(256)
 
 // The K split of qwix_hip_gemm_bf16_wq_ws: 0 = none.  The tile kernel walks K in 64-element slabs of about 0.37 us
 // each, however few workgroups there are; while they cover at most half of the CUs, K is cut into equal ranges (whole
-// 256-element superslabs and scale groups, at least 1024 elements) for up to one workgroup per CU.
+// 256-element superslabs; whole scale groups, or equal parts of one; at least 1024 elements) for up to one workgroup
+// per CU.
 static int wq_splits(int64_t M, int64_t N, int64_t K, int64_t group) {
   if (M <= 0 || N <= 0 || K <= 0 || group <= 0 || K % 256 || group % 64 || K % group) return 0;
   const bool low = M <= 128;
   const bool narrow = ((M + 255) / 256) * ((N + 127) / 128) <= 128;
   const int64_t tiles = ((M + (low ? 127 : 255)) / (low ? 128 : 256)) * ((N + (low || narrow ? 63 : 127)) / (low || narrow ? 64 : 128));
   if (tiles > 128) return 0;
-  int64_t unit = 256;  // a range is a multiple of 256 and of the group: of lcm(256, group)
-  while (unit % group) unit += 256;
+  // a range is whole superslabs, and whole scale groups or a whole part of one (never across a group's end)
   int best = 0;
-  for (int64_t sp = 2; sp * tiles <= 256 && sp * 1024 <= K; ++sp)
-    if (K % (sp * unit) == 0) best = static_cast<int>(sp);
+  for (int64_t sp = 2; sp * tiles <= 256 && sp * 1024 <= K; ++sp) {
+    if (K % (sp * 256)) continue;
+    const int64_t len = K / sp;
+    if (len % group == 0 || group % len == 0) best = static_cast<int>(sp);
+  }
   return best;
 }
 

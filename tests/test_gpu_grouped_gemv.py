@@ -561,10 +561,12 @@ def test_prefill_with_f32_scales_stays_within_a_bf16_rounding_of_the_f32_contrac
                                           ('float8_e4m3fn', False)])
 @pytest.mark.parametrize('M,K,N,group,splits', [(128, 4096, 1024, 128, 4), (96, 14336, 520, 128, 14), (300, 2048, 136, 64, 2),
                                                 (512, 4096, 1000, 256, 4), (64, 8192, 264, 512, 8), (130, 3072, 72, 1024, 3),
+                                                (128, 4096, 1024, 4096, 4), (64, 4096, 520, 2048, 4), (200, 6144, 136, 3072, 6),
                                                 (2048, 4096, 1536, 128, 0), (64, 1024, 64, 128, 0)])
 def test_prefill_gemm_k_ranges(M, K, N, group, splits, asym, wq_type, out_dtype, sdt):
   """qwix_hip_gemm_bf16_wq_ws: K in `splits` ranges with f32 partials in a workspace while the tiles are few (edges in
-  M and N, groups of 64 to 1024, ranges of 1024 elements and more).  Against the unsplit kernel: another order of the
+  M and N, groups of 64 to 1024 in whole numbers per range, groups of 2048 to K (one scale per column) that hold several
+  ranges, ranges of 1024 elements and more).  Against the unsplit kernel: another order of the
   f32 sums, so equal to 2^-18 of the mean magnitude (plus one bf16 step, 2^-7 relative, for bf16 results); with no workspace, and
   for shapes that are not split (workspace size 0), the very same bits."""
   from qwix_amd import _lib
