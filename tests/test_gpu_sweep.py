@@ -269,6 +269,61 @@ def test_sweep_dot_general_types_and_tiles(seed):
 
 
 # ---------------------------------------------------------------------------------------------------------------
+# weight-only: float activations against a quantized weight, the dequantize-first path (dot_general.py:264-275)
+# ---------------------------------------------------------------------------------------------------------------
+
+
+def _weight_only_cases(seed, count):
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import qarray
+  r = util.rng(seed)
+  for c in range(count):
+    dt = O.BF16 if r.random() < 0.85 else O.F32
+    lead = [int(r.choice([1, 2, 3, 5, 8, 17, 33, 40, 50, 64, 100, 130, 300])) for _ in range(int(r.choice([1, 1, 2])))]
+    if int(np.prod(lead)) > 700:
+      lead = lead[:1]
+    K = int(r.choice([256, 512, 1024, 2048, 3072, 4096, 6144]))
+    N = int(r.choice([48, 64, 136, 520, 1024, 2048]))
+    wt = str(r.choice(['int4', 'int8', O.E4M3]))
+    g = int(r.choice([0, 64, 128, 256, 512, 1024]))
+    g = 0 if g and K % g else g
+    asym = wt != O.E4M3 and r.random() < 0.3
+    sdt, pet = r.choice([None, O.F32, O.BF16]), r.choice([None, O.F32, O.BF16])
+
+    def thunk(lead=lead, K=K, N=N, wt=wt, g=g, asym=asym, dt=dt, sdt=sdt, pet=pet, c=c):
+      x_np, x_t = util.make(tuple(lead) + (K,), dt, seed=c)
+      w_np, w_t = util.make((K, N), dt, seed=c + 999, scale=0.05)
+      if asym:
+        w_np = O.rnd(w_np + 0.02, dt)
+        w_t = util.to_gpu(w_np, dt)
+      dn = (((len(lead),), (0,)), ((), ()))
+      kw = dict(channelwise_axes=[1], tiled_axes={0: g} if g else {})
+      if asym:
+        kw['calibration_method'] = 'minmax'
+      wq = qarray.quantize_api(w_t, wt, scale_dtype=None if sdt is None else TD[sdt], **kw)
+      owq = O.quantize_api(O.FArr(w_np, dt), wt, scale_dtype=sdt, **kw)
+      util.assert_qarray_equal(wq, owq, 'weight')
+      out = dg.dot_general(x_t, wq, dn, preferred_element_type=None if pet is None else TD[pet])
+      want = O.dot_general(O.FArr(x_np, dt), owq, dn, preferred_element_type=pet)
+      assert out.dtype == TD[want.dtype], (out.dtype, want.dtype)
+      got = util.f32np(out)
+      assert got.shape == want.v.shape, (got.shape, want.v.shape)
+      # the decode kernel, the dequantizing tile GEMM (with and without K ranges) or dequantize + GEMM, by the shape:
+      # bf16 operands on the matrix cores with f32 sums in the kernel's order.  A weight with f32 scales is rounded to
+      # bf16 once more there (2^-9 relative; with one scale per column the same few roundings all along K, so the
+      # deviations add up in step: up to 1.2e-2 of the mean magnitude at 300 x 512 x 1024 by construction)
+      mag = np.abs(want.v).mean()
+      assert np.allclose(got, want.v, rtol=1e-2, atol=2e-2 * mag), np.abs(got - want.v).max() / mag
+
+    yield f'weight-only {lead} K={K} N={N} {wt} group={g} asym={asym} {dt} scale={sdt} result={pet}', thunk
+
+
+@pytest.mark.parametrize('seed', [11, 12])
+def test_sweep_weight_only(seed):
+  _run(_weight_only_cases(seed, 80))
+
+
+# ---------------------------------------------------------------------------------------------------------------
 # general dimension numbers: batch axes, several contracting axes, any axis order (dot_general.py:79-132)
 # ---------------------------------------------------------------------------------------------------------------
 
