@@ -298,6 +298,21 @@ QWIX_API int qwix_hip_qgemm_hadamard_act(const void* x, int x_dtype, int64_t M, 
                                 void* out, int out_dtype, int64_t ldo, void* workspace, size_t workspace_bytes,
                                 void* stream);
 
+/* qwix_hip_qgemm_grouped with K cut into ranges where its tiles are few (the same call of the reference:
+ * _fast_dot_general with tiled scales, qwix/_src/core/dot_general.py:160-262): symmetric int8 x int8 / int4 operands, one
+ * activation scale per row (ga == 1), more than 32 rows, exact == 0.  Every range's workgroups write the f32 sums of
+ * their groups' scaled partials into `workspace` (qwix_hip_qgemm_grouped_workspace_bytes(M, N, K, group, b_qtype)
+ * bytes, 16-byte aligned; 0 = this shape is not split); a second kernel adds them in range order, applies the
+ * activation scale and rounds as the unsplit kernel's epilogue does.  The groups' f32 partials are then added in
+ * another order than in qwix_hip_qgemm_grouped with exact == 0 (which itself is free in that order).  With workspace
+ * NULL or too small, with exact != 0, zero points, per-group activation scales or acc_out: exactly
+ * qwix_hip_qgemm_grouped. */
+QWIX_API size_t qwix_hip_qgemm_grouped_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group, int b_qtype);
+QWIX_API int qwix_hip_qgemm_grouped_ws(const void* a, int64_t lda, const void* b, int64_t ldb_bytes, int b_qtype, int64_t M,
+                              int64_t N, int64_t K, int64_t group, const void* sa, int sa_dtype, int64_t ga,
+                              const void* sb, int sb_dtype, void* out, int out_dtype, int64_t ldo, int exact,
+                              int32_t* acc_out, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Sub-channel GEMM with one asymmetric operand.  Replaces the zero-point terms of _fast_dot_general when a
  * contracting axis is tiled (qwix/_src/core/dot_general.py:196-203: the zero point is split with the tiles;
  * :228-253: the correction dot is subtracted from every tile's int32 partial before it is scaled):

@@ -51,6 +51,8 @@ SIGNATURES = {
     'qwix_hip_qgemm_hadamard_act': (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _f32, _i64, _vp, _i64, _int, _i64, _vp, _int, _vp, _int, _i64, _vp, _sz, _vp]),
     'qwix_hip_ksum_i8': (_int, [_vp, _i64, _i64, _i64, _vp, _vp]),
     'qwix_hip_qgemm_grouped': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp, _int, _vp, _int, _i64, _int, _vp, _vp]),
+    'qwix_hip_qgemm_grouped_workspace_bytes': (_sz, [_i64, _i64, _i64, _i64, _int]),
+    'qwix_hip_qgemm_grouped_ws': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp, _int, _vp, _int, _i64, _int, _vp, _vp, _sz, _vp]),
     'qwix_hip_qgemm_grouped_zp': (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp, _int, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _int, _i64, _int, _vp, _vp]),
     'qwix_hip_ksum_groups': (_int, [_vp, _int, _i64, _i64, _i64, _i64, _vp, _vp]),
     'qwix_hip_gemm_bf16': (_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp]),

@@ -602,9 +602,12 @@ def _fast_dot_general(lhs, rhs, dimension_numbers, preferred_element_type=None, 
               _lib.float_tag(sb.dtype), zu.data_ptr(), zu_strides[0], zu_strides[1], zv.data_ptr(), zv_strides[0],
               zv_strides[1], out.data_ptr(), _tag_of(res_t), c.N, int(exact), _lib.ptr(acc), st)
   else:
-    _lib.call('qwix_hip_qgemm_grouped', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), bq, c.M, c.N, c.K, group,
+    # few tiles: K in ranges with f32 partial sums in a workspace (0 bytes: not split; never with `exact`)
+    nws = 0 if exact or acc is not None else int(_lib.load().qwix_hip_qgemm_grouped_workspace_bytes(c.M, c.N, c.K, group, bq))
+    ws = torch.empty(nws, dtype=torch.uint8, device=dev) if nws else None
+    _lib.call('qwix_hip_qgemm_grouped_ws', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), bq, c.M, c.N, c.K, group,
               _lib.ptr(sa), 0 if sa is None else _lib.float_tag(sa.dtype), ga, sb.data_ptr(), _lib.float_tag(sb.dtype),
-              out.data_ptr(), _tag_of(res_t), c.N, int(exact), _lib.ptr(acc), st)
+              out.data_ptr(), _tag_of(res_t), c.N, int(exact), _lib.ptr(acc), _lib.ptr(ws), nws, st)
   out = out.reshape(c.out_shape)
   return (out, acc.reshape((ngroups,) + c.out_shape)) if return_accumulators else out
 

@@ -50,6 +50,10 @@ struct GroupedArgs {
   // One group spans all of K (int4 weights with per-channel scales): the fast kernel then scales like the untiled
   // contraction, ((T(acc) * sx) * sy) with a rounding per step (dot_general.py:255-261), not like a sum of partials.
   int single;
+  // K in ranges (0: none): workgroups with blockIdx.y = y contract elements [y ksplit, (y + 1) ksplit) -- whole groups --
+  // and write the f32 sums of their scaled partials, without the activation scale and the final rounding, as the y-th
+  // M x N array at `out` (the host passes f32, ldo = N, sa = null); grouped_reduce_kernel finishes.
+  int ksplit;
 };
 
 __device__ __forceinline__ float ld_scale(const void* p, int dtype, int64_t i) {
@@ -389,6 +393,14 @@ __global__ void __launch_bounds__(G::kNW * 64) __attribute__((amdgpu_waves_per_e
   constexpr int BM = G::kBM, BN = G::kBN, BK = G::kBK, NW = G::kNW, TM = G::kTM;
   constexpr int WR = 1;  // every wavefront owns all rows of its 32 columns
   constexpr bool W4 = (BQT == QWIX_INT4);
+  if (p.ksplit > 0) {  // this workgroup's range of K: every operand moves to its first element
+    const int y = blockIdx.y, k0 = y * p.ksplit;
+    p.A += k0;
+    p.B += W4 ? k0 / 2 : k0;
+    p.sb = static_cast<const uint8_t*>(p.sb) + static_cast<int64_t>(k0 / p.group) * p.N * (SBF ? 2 : 4);
+    p.out += static_cast<int64_t>(y) * p.M * p.N * 4;
+    p.K = p.ksplit;
+  }
   // e4m3 x e4m3: bytes travel like int8; two 16-byte fragments of consecutive k-steps make one operand of
   // v_mfma_f32_32x32x64_f8f6f4 (both operands take the same 32 of the 64 k per lane half, so the dot is complete),
   // the group's partial is f32 already.  Never MAGIC, never AUX.
@@ -825,7 +837,7 @@ __global__ void __launch_bounds__(G::kNW * 64) __attribute__((amdgpu_waves_per_e
   // ---- epilogue: 32 rows x 32 columns of f32 per wavefront and pass through LDS
   constexpr int ROW_F = 36;  // floats per staged row (32 + padding)
   float* stg = reinterpret_cast<float*>(smem) + wave * (32 * ROW_F);
-  const bool t_bf16 = (p.t_dtype == QWIX_BF16);
+  const bool t_bf16 = (p.t_dtype == QWIX_BF16) && p.ksplit == 0;  // a range's sums stay f32: the reduction rounds
   const bool vec_ok = (p.ldo % 8 == 0) && (p.N % 4 == 0);
   // chunk c = lane + 64*q of the 32 x 8 grid of 16-byte pieces: row c/8, columns 4*(c%8) .. +3
   float sav[TM][4];
@@ -920,7 +932,8 @@ int launch_grouped_dma(const GroupedArgs& p, hipStream_t st) {
   static LdsGrant granted;
   if (int e_ = grant_lds(reinterpret_cast<const void*>(kern), smem, granted)) return e_;
   const int64_t tiles = static_cast<int64_t>((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-  kern<<<dim3(static_cast<unsigned>(tiles)), NW * 64, smem, st>>>(p);
+  const unsigned ranges = p.ksplit > 0 ? static_cast<unsigned>(p.K / p.ksplit) : 1u;
+  kern<<<dim3(static_cast<unsigned>(tiles), ranges), NW * 64, smem, st>>>(p);
   return check_launch("qgemm_grouped (dma)");
 }
 
@@ -1166,6 +1179,72 @@ int dispatch_grouped_f8(const GroupedArgs& p, hipStream_t st) {
              : launch_grouped_dma<Q, false, SAG, false, false, 2, false>(p, st);
 }
 
+// out[m, n] = cast(T(sa[m] * sum over ranges of ws[r][m][n])): what the tile kernel's epilogue does with its f32 sums,
+// after the K ranges' partial sums are added in range order.  Four consecutive elements of (m, n) per thread.
+__global__ void __launch_bounds__(256)
+    grouped_reduce_kernel(const float* __restrict__ ws, int ranges, int M, int N, const void* __restrict__ sa,
+                          int sa_dtype, int t_bf16, uint8_t* __restrict__ out, int out_dtype, int64_t ldo) {
+  const int64_t total = static_cast<int64_t>(M) * N;
+  const int64_t i0 = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  if (i0 >= total) return;
+  const bool vec = (N & 3) == 0;  // then the four share a row and the loads are 16-byte aligned
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  if (vec) {
+    float4 w[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      w[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (j < ranges) w[j] = *reinterpret_cast<const float4*>(ws + j * total + i0);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < ranges) { v[0] += w[j].x; v[1] += w[j].y; v[2] += w[j].z; v[3] += w[j].w; }
+  } else {
+    for (int r = 0; r < ranges; ++r)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (i0 + e < total) v[e] += ws[r * total + i0 + e];
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int64_t i = i0 + e;
+    if (i >= total) break;
+    const int m = static_cast<int>(i / N), n = static_cast<int>(i % N);
+    float t = v[e];
+    if (sa != nullptr) t *= ld_scale(sa, sa_dtype, m);
+    if (t_bf16) t = round_bf16(t);
+    if (out_dtype == QWIX_BF16)
+      reinterpret_cast<uint16_t*>(out)[static_cast<int64_t>(m) * ldo + n] = f32_to_bf16_bits(t);
+    else
+      reinterpret_cast<float*>(out)[static_cast<int64_t>(m) * ldo + n] = t;
+  }
+}
+constexpr int kMaxRanges = 8;  // what grouped_reduce_kernel reads in one batch
+
+// The K ranges of qwix_hip_qgemm_grouped_ws (0: none): for the narrow tiles (128 x 64, two workgroups per CU) of the
+// fast kernel with one activation scale per row and symmetric operands, above the decode kernel's 32 rows.  A tile
+// walks its slabs at about 0.78 us each (0.51 us up to 64 rows) after 3 us, however few tiles there are (weights from
+// HBM); the ranges cost a second launch and their partial arrays written and read.
+static int grouped_ranges(int64_t M, int64_t N, int64_t K, int64_t group, int b_qtype) {
+  if (b_qtype == QWIX_E4M3 || M <= 32 || group <= 0 || group % 128 || K % group || group == K) return 0;
+  const int64_t wide = ((M + Fast::kBM - 1) / Fast::kBM) * ((N + Fast::kBN - 1) / Fast::kBN);
+  if (!(wide <= kNarrowTiles || M <= 64)) return 0;
+  const int64_t tiles = ((M + 127) / 128) * ((N + 63) / 64);
+  auto model = [&](int64_t sp) {
+    const double rounds = static_cast<double>((sp * tiles + 511) / 512);
+    const double walk = 3.0 + static_cast<double>(K / 128 / sp) * (M <= 64 ? 0.51 : 0.78) * rounds;
+    return sp == 1 ? walk : walk + 3.5 + static_cast<double>(sp * M * N) * 8.0 / 4.0e6;
+  };
+  int best = 1;
+  double best_us = model(1);
+  for (int64_t sp = 2; sp <= kMaxRanges && sp * 1024 <= K; ++sp) {
+    if (K % (sp * group)) continue;
+    const double us = model(sp);
+    if (us < 0.85 * best_us) { best = static_cast<int>(sp); best_us = us; }
+  }
+  return best > 1 ? best : 0;
+}
+
 // Per-group K-sums of quantized rows: out[row, g] = sum over the g-th group of `group` values of row `row`
 // (int8, or packed int4).  One 16-byte chunk per thread; the chunks of a group that sit in `seg` adjacent
 // lanes (a power of two that divides the chunks per group) are added by shuffles, the rest by integer
@@ -1244,7 +1323,8 @@ static int grouped_impl(const void* a, int64_t lda, const void* b, int64_t ldb_b
                         int64_t K, int64_t group, const void* sa, int sa_dtype, int64_t ga, const void* sb, int sb_dtype,
                         const int32_t* zu, int64_t zu_row_stride, int64_t zu_group_stride, const int32_t* zv,
                         int64_t zv_col_stride, int64_t zv_group_stride, void* out, int out_dtype, int64_t ldo,
-                        int exact, int32_t* acc_out, void* stream) {
+                        int exact, int32_t* acc_out, void* stream, void* workspace = nullptr,
+                        size_t workspace_bytes = 0) {
   if (!a || !b || !out || !sb) return fail(QWIX_ERR_INVALID_ARGUMENT, "null a/b/out/sb");
   if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX)
     return fail(QWIX_ERR_INVALID_ARGUMENT, "bad GEMM shape M=%lld N=%lld K=%lld", (long long)M, (long long)N,
@@ -1300,6 +1380,25 @@ static int grouped_impl(const void* a, int64_t lda, const void* b, int64_t ldb_b
   if ((!exact || p.single) && row_strides_fit) {
     // per-group activation scales ride along in LDS: the tile's scales must fit behind the slab stages
     const bool sag = sa != nullptr && ga > 1;
+    // K in ranges with f32 partial sums in the caller's workspace, where the narrow tiles are few
+    const int ranges = (workspace && !exact && !sag && !zu && !acc_out && aligned16(workspace))
+                           ? grouped_ranges(M, N, K, group, b_qtype) : 0;
+    if (ranges > 0 && workspace_bytes >= static_cast<size_t>(ranges) * M * N * 4) {
+      GroupedArgs q = p;
+      q.ksplit = static_cast<int>(K / ranges);
+      q.sa = nullptr;
+      q.out = static_cast<uint8_t*>(workspace); q.out_dtype = QWIX_F32; q.ldo = N;
+      const int rc = b_qtype == QWIX_INT4 ? dispatch_grouped_dma<QWIX_INT4, false>(q, st)
+                                          : dispatch_grouped_dma<QWIX_INT8, false>(q, st);
+      if (rc > 0) return rc;
+      if (rc == 0) {
+        const int64_t threads = (M * N + 3) / 4;
+        grouped_reduce_kernel<<<dim3(static_cast<unsigned>((threads + 255) / 256)), 256, 0, st>>>(
+            static_cast<const float*>(workspace), ranges, p.M, p.N, sa, sa_dtype, p.t_dtype == QWIX_BF16 ? 1 : 0,
+            static_cast<uint8_t*>(out), out_dtype, ldo);
+        return check_launch("qgemm_grouped (K ranges)");
+      }
+    }
     int rc;
     if (b_qtype == QWIX_INT4)
       rc = sag ? dispatch_grouped_dma<QWIX_INT4, true>(p, st) : dispatch_grouped_dma<QWIX_INT4, false>(p, st);
@@ -1318,6 +1417,20 @@ extern "C" int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b,
                                       int exact, int32_t* acc_out, void* stream) {
   return grouped_impl(a, lda, b, ldb_bytes, b_qtype, M, N, K, group, sa, sa_dtype, ga, sb, sb_dtype, nullptr, 0, 0,
                       nullptr, 0, 0, out, out_dtype, ldo, exact, acc_out, stream);
+}
+
+extern "C" size_t qwix_hip_qgemm_grouped_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group, int b_qtype) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  return static_cast<size_t>(grouped_ranges(M, N, K, group, b_qtype)) * M * N * 4;
+}
+
+extern "C" int qwix_hip_qgemm_grouped_ws(const void* a, int64_t lda, const void* b, int64_t ldb_bytes, int b_qtype,
+                                         int64_t M, int64_t N, int64_t K, int64_t group, const void* sa, int sa_dtype,
+                                         int64_t ga, const void* sb, int sb_dtype, void* out, int out_dtype, int64_t ldo,
+                                         int exact, int32_t* acc_out, void* workspace, size_t workspace_bytes,
+                                         void* stream) {
+  return grouped_impl(a, lda, b, ldb_bytes, b_qtype, M, N, K, group, sa, sa_dtype, ga, sb, sb_dtype, nullptr, 0, 0,
+                      nullptr, 0, 0, out, out_dtype, ldo, exact, acc_out, stream, workspace, workspace_bytes);
 }
 
 extern "C" int qwix_hip_qgemm_grouped_zp(const void* a, int64_t lda, const void* b, int64_t ldb_bytes, int b_qtype,

@@ -763,3 +763,66 @@ def test_grouped_gemm_decode_batches(M, K, N, wq_type, dtype):
     if big_x.shape[0] == 40 and 4 * M >= 40:
       tiled = util.f32np(dg.dot_general(QArray(big_x.contiguous(), big_s.contiguous(), None, 'int8'), wq, DN))[:M]
       assert np.all(np.abs(tiled - got) <= tol * scale + 1e-30)
+
+
+@pytest.mark.parametrize('dtype', [O.BF16, O.F32])
+@pytest.mark.parametrize('wq_type', ['int4', 'int8'])
+@pytest.mark.parametrize('M,K,N,group,split', [(128, 4096, 1024, 128, True), (64, 8192, 520, 128, True), (200, 4096, 264, 256, True),
+                                               (40, 3072, 72, 1024, True), (512, 8192, 1024, 128, True), (33, 4096, 64, 128, True),
+                                               (16, 4096, 1024, 128, False), (2048, 4096, 4096, 128, False),
+                                               (128, 1024, 1024, 128, False)])
+def test_grouped_gemm_k_ranges(M, K, N, group, split, wq_type, dtype):
+  """The sub-channel GEMM with K in ranges (qwix_hip_qgemm_grouped_ws, what the operator calls without `exact`): above
+  the decode kernel's 32 rows, where the narrow tiles are few, every range's f32 sums go through a workspace and a
+  second kernel adds them, applies the token scale and rounds.  The outputs are the exact integer partials combined in
+  f32 in another order: compared with their float64 combination, and with the unsplit kernel through the C ABI (same
+  bound); shapes that are not split report a workspace of 0 bytes and give the unsplit kernel's bits."""
+  from qwix_amd import _lib
+  from qwix_amd.core import dot_general as dg
+  from qwix_amd.core import numerics
+  print('case grouped k ranges', M, K, N, group, split, wq_type, dtype, flush=True)
+  xq, wq, oxq, owq, x_np, w_np = _pair(M, K, N, dtype, wq_type, group, seed=11 + M + N)
+  bq = numerics.qtype_tag(wq_type)
+  nws = int(_lib.load().qwix_hip_qgemm_grouped_workspace_bytes(M, N, K, group, bq))
+  assert (nws > 0) == split and nws % (M * N * 4) == 0
+  out = dg.dot_general(xq, wq, DN)
+  torch.cuda.synchronize()
+  got = util.f32np(out)
+  assert got.shape == (M, N)
+  want, wacc = O.fast_dot_general(oxq, owq, DN, return_acc=True)
+  sa = np.asarray(oxq.scale.v, np.float64).reshape(M, 1)
+  sb = np.asarray(owq.scale.v, np.float64).reshape(K // group, 1, N)
+  parts = np.asarray(wacc, np.float64).reshape(K // group, M, N) * sb
+  exact, scale = parts.sum(0) * sa, np.abs(parts).sum(0) * sa
+  tol = 2.0 ** -7 if dtype is O.BF16 else 1e-5
+  assert np.all(np.abs(got - exact) <= tol * scale + 1e-30), (np.abs(got - exact) / (scale + 1e-30)).max()
+  # through the C ABI: without a workspace the unsplit kernel runs; with one the result stays inside the same bound
+  c = dg._Canon(xq, wq, DN)
+  a = c.lhs_values(xq)
+  b, _ = c.rhs_values(wq)
+  sa_t, _ = c.lhs_scale(xq)
+  sb_t, _ = c.rhs_scale(wq)
+  st = _lib.stream_of(a)
+  res_t = out.dtype
+
+  def run(ws, n):
+    o = torch.full((M, N), float('nan'), dtype=res_t, device=util.DEV)
+    _lib.call('qwix_hip_qgemm_grouped_ws', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), bq, M, N, K, group,
+              sa_t.data_ptr(), _lib.float_tag(sa_t.dtype), 1, sb_t.data_ptr(), _lib.float_tag(sb_t.dtype), o.data_ptr(),
+              _lib.float_tag(res_t), N, 0, None, _lib.ptr(ws), n, st)
+    torch.cuda.synchronize()
+    return o
+
+  plain = torch.empty(M, N, dtype=res_t, device=util.DEV)
+  _lib.call('qwix_hip_qgemm_grouped', a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), bq, M, N, K, group,
+            sa_t.data_ptr(), _lib.float_tag(sa_t.dtype), 1, sb_t.data_ptr(), _lib.float_tag(sb_t.dtype), plain.data_ptr(),
+            _lib.float_tag(res_t), N, 0, None, st)
+  torch.cuda.synchronize()
+  assert torch.equal(run(None, 0), plain)
+  if not split:
+    assert torch.equal(out, plain)
+    return
+  ws = torch.full((nws,), 0xFF, dtype=torch.uint8, device=util.DEV)  # NaN patterns: every partial sum must be written
+  assert torch.equal(run(ws, nws - 1), plain)   # too small a workspace: not split
+  assert torch.equal(run(ws, nws), out)         # what the operator ran
+  assert np.all(np.abs(util.f32np(plain) - exact) <= tol * scale + 1e-30)
