@@ -537,6 +537,9 @@ class HadamardQdot(Workload):
     self.out = torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev)
     self.stream = torch.cuda.current_stream().cuda_stream
     self.L = L
+    # few tiles: K in ranges with f32 partial sums in a workspace, as the operator calls it (0 bytes: not split)
+    self.nws = int(L.load().qwix_hip_qgemm_grouped_workspace_bytes(self.M, self.N, self.K, 128, L.INT4))
+    self.ws = torch.empty(max(self.nws, 16), dtype=torch.uint8, device=dev)
 
   def step(self, i=0):
     L = self.L
@@ -546,9 +549,9 @@ class HadamardQdot(Workload):
 
   def kernel(self, i=0):
     L = self.L
-    L.call('qwix_hip_qgemm_grouped', self.xq.data_ptr(), self.K, self.b.data_ptr(), self.K // 2, L.INT4, self.M, self.N,
+    L.call('qwix_hip_qgemm_grouped_ws', self.xq.data_ptr(), self.K, self.b.data_ptr(), self.K // 2, L.INT4, self.M, self.N,
            self.K, 128, self.sa.data_ptr(), L.BF16, 1, self.sb.data_ptr(), L.BF16, self.out.data_ptr(), L.BF16, self.N, 0,
-           None, self.stream)
+           None, self.ws.data_ptr() if self.nws else None, self.nws, self.stream)
 
   def work_per_step(self):
     return 2.0 * self.M * self.N * self.K
@@ -1043,6 +1046,7 @@ WORKLOADS = {
     'batched_qk_int8_32x2048': lambda: QdotBatched('batched_qk_int8_32x2048', 32, 2048, 2048, 128),
     'c1_ptq_mlp_graph': lambda: PtqMlpGraph('c1_ptq_mlp_graph'),
     'c5_hadamard_a8w4': lambda: HadamardQdot('c5_hadamard_a8w4', 2048, 8192, 8192),
+    'c5_hadamard_a8w4_m128': lambda: HadamardQdot('c5_hadamard_a8w4_m128', 128, 8192, 8192),
     'c5_hadamard_a8w4_decode_m16': lambda: HadamardQdotDecode('c5_hadamard_a8w4_decode_m16', 16, 8192, 8192),
     'int8_subchannel_g128_4096': lambda: QdotSubChannel('int8_subchannel_g128_4096', 4096, 4096, 4096, 128, 'int8'),
     'fp8_subchannel_g128_4096': lambda: QdotSubChannel('fp8_subchannel_g128_4096', 4096, 4096, 4096, 128, 'float8_e4m3fn'),
@@ -1059,7 +1063,7 @@ CEILING_EXTRA = ['mfma_ceiling_int8_zeros', 'mfma_ceiling_int8_gauss30', 'mfma_c
                  'mfma_ceiling_fp8_zeros', 'mfma_ceiling_fp8_gauss30', 'mfma_ceiling_fp8_operands']
 DEFAULT = 'c3_int8_w8a8_4096'
 EXTRA = ['quantize_act_4096', 'quantize_act_8192', 'quantize_act_8192_fp8', 'c4_quantize_weight_fp8', 'c5_quantize_weight_int4_g128', 'c3_int8_w8a8_8192', 'c4_fp8_w8a8_ffn', 'c2_gemv_w4_m1', 'c2_gemv_w4_m16', 'c2_gemv_w4_m32', 'w8a16_gemv_m1', 'w8a16_gemv_m16', 'c2_w4a16_prefill_m2048', 'c2_w4a16_prefill_m512', 'c2_w4a16_prefill_m128', 'c2_w4a16_prefill_m128_down', 'w8a8_decode_m16', 'w8a8_decode_m64', 'w8a8_decode_m64_k8192', 'w8a8_decode_m16_k2048', 'w8a8_decode_m16_k2048_fused',
-         'c5_hadamard_a8w4', 'c5_hadamard_a8w4_decode_m16', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'int8_subchannel_g128_4096', 'fp8_subchannel_g128_4096', 'moe_ragged_int8_8x1024',
+         'c5_hadamard_a8w4', 'c5_hadamard_a8w4_m128', 'c5_hadamard_a8w4_decode_m16', 'c5_fwht_quantize_act', 'fwht_quantize_8192x8192', 'int8_subchannel_g128_4096', 'fp8_subchannel_g128_4096', 'moe_ragged_int8_8x1024',
          'moe_ragged_int8_64x128', 'moe_decode_int8_64x4', 'quantize_weight_fp8_block128', 'srq_quantize_act_4096', 'zp_int8_w8a8_4096', 'batched_qk_int8_32x2048', 'c1_ptq_mlp_graph']
 
 
