@@ -290,7 +290,9 @@ QWIX_API int qwix_hip_qgemm_grouped(const void* a, int64_t lda, const void* b, i
  * x (M, K) of x_dtype, dense rows; act_tile = K (one scale per token) or = group; b, sb, group, out as in
  * qwix_hip_qgemm_grouped.  workspace: qwix_hip_qgemm_hadamard_act_workspace_bytes(M, K, act_tile, x_dtype) bytes of
  * device memory, 16-byte aligned (the int8 rows and their scales; nothing is allocated).  Two kernels on the
- * stream; bit-identical to qwix_hip_fwht_quantize followed by qwix_hip_qgemm_grouped. */
+ * stream; bit-identical to qwix_hip_fwht_quantize followed by qwix_hip_qgemm_grouped.  A workspace that is larger by
+ * qwix_hip_qgemm_grouped_workspace_bytes(M, N, K, group, b_qtype) lets the GEMM cut K into ranges where that pays
+ * (then: followed by qwix_hip_qgemm_grouped_ws on the surplus, three kernels). */
 QWIX_API size_t qwix_hip_qgemm_hadamard_act_workspace_bytes(int64_t M, int64_t K, int64_t act_tile, int x_dtype);
 QWIX_API int qwix_hip_qgemm_hadamard_act(const void* x, int x_dtype, int64_t M, int64_t N, int64_t K, const void* pre_sign,
                                 const void* post_sign, float out_scale, int64_t act_tile, const void* b,

@@ -145,11 +145,14 @@ def hadamard_quantized_matmul(act: torch.Tensor, weight: qarray.QArray, pre_sign
   tile = c.K if act_tile is None else int(act_tile)
   x = act if act.is_contiguous() else act.contiguous()
   res_t = preferred_element_type or act.dtype
-  need = _lib.load().qwix_hip_qgemm_hadamard_act_workspace_bytes(c.M, c.K, tile, _lib.float_tag(x.dtype))
+  bq = _lib.INT4 if b_is4 else _lib.INT8
+  need = int(_lib.load().qwix_hip_qgemm_hadamard_act_workspace_bytes(c.M, c.K, tile, _lib.float_tag(x.dtype)))
+  # room behind it for the GEMM's K ranges (few tiles, one scale per token; 0 bytes otherwise)
+  need += int(_lib.load().qwix_hip_qgemm_grouped_workspace_bytes(c.M, c.N, c.K, group, bq)) if tile == c.K else 0
   ws = torch.empty(max(int(need), 16), dtype=torch.uint8, device=x.device)
   out = torch.empty(c.M, c.N, dtype=res_t, device=x.device)
   _lib.call('qwix_hip_qgemm_hadamard_act', x.data_ptr(), _lib.float_tag(x.dtype), c.M, c.N, c.K, _lib.ptr(pre_sign),
-            _lib.ptr(post_sign), 1.0, tile, b.data_ptr(), b.stride(0), _lib.INT4 if b_is4 else _lib.INT8, group,
+            _lib.ptr(post_sign), 1.0, tile, b.data_ptr(), b.stride(0), bq, group,
             sb.data_ptr(), _lib.float_tag(sb.dtype), out.data_ptr(), _lib.float_tag(res_t), c.N, ws.data_ptr(), int(need),
             _lib.stream_of(x))
   return out

@@ -1448,7 +1448,8 @@ extern "C" int qwix_hip_qgemm_grouped_zp(const void* a, int64_t lda, const void*
 // qwix/contrib/kernels/fused_hadamard_quantized_matmul.py:349-414, with the numerics of the unfused path:
 // hadamard_rot.py:133-190, then quantize, then _fast_dot_general): the rotation + per-token or per-group quantize kernel
 // writes int8 rows and their scales into the caller's workspace, the sub-channel GEMM reads them.  Bit-identical to
-// qwix_hip_fwht_quantize followed by qwix_hip_qgemm_grouped.
+// qwix_hip_fwht_quantize followed by qwix_hip_qgemm_grouped -- or, when the workspace is larger than required by at
+// least qwix_hip_qgemm_grouped_workspace_bytes, by qwix_hip_qgemm_grouped_ws on that surplus (K in ranges).
 static size_t had_align(size_t v) { return (v + 255) & ~size_t{255}; }
 
 extern "C" size_t qwix_hip_qgemm_hadamard_act_workspace_bytes(int64_t M, int64_t K, int64_t act_tile, int x_dtype) {
@@ -1477,6 +1478,9 @@ extern "C" int qwix_hip_qgemm_hadamard_act(const void* x, int x_dtype, int64_t M
   uint8_t* sa = q + had_align(static_cast<size_t>(M) * K);
   if (int e = qwix_hip_fwht_quantize(x, x_dtype, M, K, pre_sign, post_sign, out_scale, act_tile, QWIX_INT8, q, sa, stream))
     return e;
-  return qwix_hip_qgemm_grouped(q, K, b, ldb_bytes, b_qtype, M, N, K, group, sa, x_dtype, K / act_tile, sb, sb_dtype, out,
-                                out_dtype, ldo, 0, nullptr, stream);
+  // what the caller provides beyond `need` serves the GEMM's K ranges (qwix_hip_qgemm_grouped_workspace_bytes; `need`
+  // is a multiple of 256, so the rest is aligned like the workspace)
+  const size_t rest = workspace_bytes - need;
+  return grouped_impl(q, K, b, ldb_bytes, b_qtype, M, N, K, group, sa, x_dtype, K / act_tile, sb, sb_dtype, nullptr, 0, 0,
+                      nullptr, 0, 0, out, out_dtype, ldo, 0, nullptr, stream, rest ? q + need : nullptr, rest);
 }

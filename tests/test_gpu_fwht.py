@@ -168,11 +168,16 @@ def test_weight_side_fused_rotation_feeds_the_grouped_gemm():
 
 @pytest.mark.parametrize('M,K,N,wq_type,group,per_group_act,dtype', [
     (64, 1024, 256, 'int4', 128, False, torch.bfloat16), (200, 2048, 520, 'int8', 256, False, torch.bfloat16),
-    (33, 512, 136, 'int4', 128, True, torch.bfloat16), (16, 1024, 128, 'int8', 128, False, torch.float32)])
+    (33, 512, 136, 'int4', 128, True, torch.bfloat16), (16, 1024, 128, 'int8', 128, False, torch.float32),
+    (128, 4096, 1024, 'int4', 128, False, torch.bfloat16)])
 def test_rotate_quantize_multiply_in_one_call(M, K, N, wq_type, group, per_group_act, dtype):
   """qwix_hip_qgemm_hadamard_act through the C ABI (hadamard_quantized_matmul) == rotate_and_quantize followed by the
-  sub-channel quantized dot, bit for bit; the latter is held to the oracle by the test above."""
+  sub-channel quantized dot, bit for bit; the latter is held to the oracle by the test above.  (The last shape is one
+  whose GEMM cuts K into ranges, in both: the one call takes them from the surplus of its workspace.)"""
+  from qwix_amd import _lib
   from qwix_amd.contrib import hadamard_rot as hr
+  if M == 128:
+    assert _lib.load().qwix_hip_qgemm_grouped_workspace_bytes(M, N, K, group, _lib.INT4) > 0
   from qwix_amd.core import dot_general as dg
   from qwix_amd.core import qarray
   print('case hadamard one call', M, K, N, wq_type, group, per_group_act, dtype, flush=True)
